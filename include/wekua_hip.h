@@ -1,0 +1,171 @@
+/*
+ * wekua_hip.h -- C ABI of libwekua_hip: wekua's BLAS hot path (gemm, axpy) and the
+ * device/tensor plumbing it needs, on one AMD Instinct MI355X (gfx950) through HIP.
+ *
+ * The reference (kython28/wekua) has no FFI boundary of its own for this path: its Zig
+ * modules call OpenCL through the zig-opencl binding.  Each entry point below names
+ * the reference interface it replaces, so that a wekua maintainer can swap
+ * `cl.buffer.*` / `cl.kernel.enqueueNdRange` call sites for one `extern fn` each.
+ *
+ * Conventions
+ *   - every function returns 0 (WK_OK) or a WK_E_* code; nothing throws or aborts;
+ *   - pointers are DEVICE pointers unless the name starts with host_;
+ *   - pitches / leading dimensions are in ELEMENTS of `dtype`;
+ *   - host_alpha / host_beta point at ONE element of `dtype` in host memory and are
+ *     read before the call returns; NULL means "absent" (Zig `null`), which selects
+ *     the reference's option semantics, not the value 0 or 1;
+ *   - all work is enqueued on the wk_stream (in order, like the reference's in-order
+ *     cl_command_queue, src/core/command_queue.zig:130) and is complete after
+ *     wk_stream_sync();
+ *   - dtype = src/core/types.zig:60-86 getTypeIndex: 0 i8, 1 u8, 2 i16, 3 u16, 4 i32,
+ *     5 u32, 6 i64, 7 u64, 8 f32, 9 f64, 10..19 the complex {real, imag} struct of each.
+ *   - one thread per wk_stream at a time (the reference's queues have no locking either).
+ */
+#ifndef WEKUA_HIP_H
+#define WEKUA_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define WK_ABI_VERSION 1
+
+/* ---- error codes: src/tensor/main.zig:25-33 `Errors`, plus allocator / device errors --- */
+enum {
+    WK_OK = 0,
+    WK_E_INVALID_VALUE = 1,            /* Errors.InvalidValue            */
+    WK_E_INVALID_COORDINATES = 2,      /* Errors.InvalidCoordinates      */
+    WK_E_INVALID_BUFFER = 3,           /* Errors.InvalidBuffer           */
+    WK_E_UNQUAL_TENSORS_ATTRIBUTE = 4, /* Errors.UnqualTensorsAttribute  */
+    WK_E_UNQUAL_TENSORS_SHAPE = 5,     /* Errors.UnqualTensorsShape      */
+    WK_E_UNQUAL_TENSORS_DIMENSION = 6, /* Errors.UnqualTensorsDimension  */
+    WK_E_UNQUAL_TENSORS_CONTEXT = 7,   /* Errors.UnqualTensorsContext    */
+    WK_E_OUT_OF_MEMORY = 8,            /* std.mem.Allocator.Error.OutOfMemory / hipErrorOutOfMemory */
+    WK_E_TYPE_NOT_SUPPORTED = 9,       /* core.KernelsSet.Errors.TypeNotSupported (src/core/kernel.zig:151) */
+    WK_E_NO_DEVICE = 10,               /* Context.init: DevicesArrayEmpty (src/core/context.zig:18) */
+    WK_E_HIP_BASE = 1000               /* WK_E_HIP_BASE + hipError_t: replaces cl.errors.OpenCLError */
+};
+
+enum {
+    WK_I8 = 0, WK_U8, WK_I16, WK_U16, WK_I32, WK_U32, WK_I64, WK_U64, WK_F32, WK_F64,
+    WK_COMPLEX = 10, /* WK_COMPLEX + real id */
+    WK_DTYPE_COUNT = 20
+};
+
+/* src/blas/gemm.zig:25-29 `Operation` */
+enum { WK_OP_NO_TRANSPOSE = 0, WK_OP_TRANSPOSE = 1 };
+
+typedef struct wk_device wk_device;
+typedef struct wk_stream wk_stream;
+
+/* What src/core/command_queue.zig:10-229 caches per queue from clGetDeviceInfo. */
+typedef struct wk_props {
+    char     name[64];
+    char     arch[32];               /* "gfx950..." */
+    int      ordinal;
+    int      compute_units;          /* CommandQueue.compute_units */
+    int      wavefront_size;
+    int      max_work_group_size;    /* CommandQueue.max_work_group_size */
+    uint64_t local_mem_bytes;        /* CommandQueue.local_mem_size (LDS per work-group) */
+    uint64_t global_mem_bytes;
+    int      cache_line_size;        /* CommandQueue.cache_line_size */
+    int      clock_mhz;
+} wk_props;
+
+const char *wk_strerror(int code);
+int         wk_abi_version(void);
+size_t      wk_dtype_size(int dtype);
+
+/* ---- device / stream: src/core/context.zig:13-196, command_queue.zig:100-160 ---------- */
+int  wk_device_count(int *out_count);                     /* cl.platform/device enumeration   */
+int  wk_device_open(int ordinal, wk_device **out);        /* Context.init / initFromBestDevice */
+void wk_device_close(wk_device *dev);                     /* Context.deinit                    */
+int  wk_device_props(wk_device *dev, wk_props *out);      /* CommandQueue.init device queries  */
+int  wk_stream_create(wk_device *dev, wk_stream **out);   /* cl.command_queue.create           */
+void wk_stream_destroy(wk_stream *s);                     /* cl.command_queue.release          */
+int  wk_stream_sync(wk_stream *s);                        /* Pipeline.waitAndCleanup, src/core/pipeline.zig:47-61 */
+void *wk_stream_native(wk_stream *s);                     /* the hipStream_t, for event timing by the caller */
+
+/* ---- memory: cl.buffer.create/release (src/tensor/main.zig:229-234,253-263) ----------- */
+int  wk_malloc(wk_device *dev, size_t bytes, void **out_dptr);
+int  wk_free(wk_device *dev, void *dptr);
+int  wk_mem_info(wk_device *dev, size_t *free_bytes, size_t *total_bytes);
+/* cl.buffer.fill of the whole buffer: fill.zeroes, src/tensor/fill.zig:70-95 */
+int  wk_memset_async(wk_stream *s, void *dptr, int byte, size_t bytes);
+/* cl.buffer.writeRect: memory.readFromBuffer (HOST -> DEVICE), src/tensor/memory/read_from_buffer.zig:13-63.
+ * Copies `slices` x `rows` runs of width_bytes; pitches in BYTES.  The host buffer must
+ * stay valid until wk_stream_sync(). */
+int  wk_copy_h2d_rect_async(wk_stream *s, void *dst, size_t dst_row_pitch_bytes, size_t dst_slice_pitch_bytes,
+                            const void *host_src, size_t src_row_pitch_bytes, size_t src_slice_pitch_bytes,
+                            size_t width_bytes, size_t rows, size_t slices);
+/* cl.buffer.readRect: memory.writeToBuffer (DEVICE -> HOST), src/tensor/memory/write_to_buffer.zig:13-63 */
+int  wk_copy_d2h_rect_async(wk_stream *s, void *host_dst, size_t dst_row_pitch_bytes, size_t dst_slice_pitch_bytes,
+                            const void *src, size_t src_row_pitch_bytes, size_t src_slice_pitch_bytes,
+                            size_t width_bytes, size_t rows, size_t slices);
+/* cl.buffer.copyRect: memory.copy, src/tensor/memory/copy.zig */
+int  wk_copy_d2d_rect_async(wk_stream *s, void *dst, size_t dst_row_pitch_bytes, size_t dst_slice_pitch_bytes,
+                            const void *src, size_t src_row_pitch_bytes, size_t src_slice_pitch_bytes,
+                            size_t width_bytes, size_t rows, size_t slices);
+
+/* ---- support kernels used by the reference's gemm/axpy tests -------------------------- */
+/* fill.constant / fill.one: `fill` kernel over the logical {depth, rows, cols} region,
+ * src/tensor/fill.zig:16-57, kernels/fill.cl */
+int  wk_fill(wk_stream *s, int dtype, void *dptr, const uint64_t shape3[3],
+             uint64_t row_pitch, uint64_t slice_pitch, const void *host_scalar);
+/* identity: ones at index i*sum(pitches) for i < size, src/tensor/identity.zig:16-70,
+ * kernels/identity.cl.  The caller zeroes the buffer first (as identity.zig:27 does). */
+int  wk_identity(wk_stream *s, int dtype, void *dptr, uint64_t size, uint64_t pitch_sum);
+
+/* ---- the hot path ----------------------------------------------------------------------- */
+/* blas.axpy: y = alpha*x + y over the logical {depth, rows, cols} region
+ * (src/blas/axpy.zig:93-169, kernels/axpy.cl:3-72).
+ *   host_alpha == NULL      -> y += x
+ *   alpha == -1 (floats: |alpha+1| < eps; signed ints exactly; axpy.zig:66-91) -> y -= x
+ *   otherwise               -> y[i] = fma(alpha, x[i], y[i]) for floats, wrapping for ints,
+ *                              the 3-multiply product of wekua_cl_lib.cl:648-653 for complex.
+ * x and y must not overlap.  A region whose rows are contiguous in both operands
+ * (row_pitch == cols, slice_pitch == rows*cols) runs the vectorised streaming kernel. */
+int  wk_axpy(wk_stream *s, int dtype, const uint64_t shape3[3],
+             const void *x, uint64_t x_row_pitch, uint64_t x_slice_pitch,
+             void *y, uint64_t y_row_pitch, uint64_t y_slice_pitch,
+             const void *host_alpha);
+
+/* blas.gemm: C = alpha*op(A)*op(B) + beta*C  (src/blas/gemm.zig:834-874; kernels
+ * gemm_nxn_gpu.cl, gemm_nxn.cl, gemm_2x2.cl and their packed twins).
+ *   op(A) is M x K, op(B) is K x N, C is M x N, all row-major; A is stored M x K
+ *   (op_a = N) or K x M (op_a = T) with leading dimension lda, likewise B.
+ *   Option semantics (gemm.zig:500-501,591-602):
+ *     alpha NULL, beta NULL -> C = op(A)op(B)                 (C is not read)
+ *     alpha set,  beta NULL -> C = alpha*op(A)op(B)           (C is not read)
+ *     beta set              -> C = (alpha or 1)*op(A)op(B) + beta*C_old; C_old is read and
+ *                              multiplied even when beta == 0 (NaN/Inf propagate).
+ *   Integers wrap modulo 2^width; f32/f64 accumulate in their own precision.
+ *   The reference's PackedTensors pass (gemm.zig:60-359) has no counterpart: tiles are
+ *   staged through LDS straight from the row-major operands.
+ *   workspace may be NULL when wk_gemm_workspace_bytes() returns 0 (it currently
+ *   always does); it is reserved for split-K variants. */
+int    wk_gemm(wk_stream *s, int dtype, int op_a, int op_b, uint64_t M, uint64_t N, uint64_t K,
+               const void *host_alpha, const void *A, uint64_t lda, const void *B, uint64_t ldb,
+               const void *host_beta, void *C, uint64_t ldc, void *workspace, size_t workspace_bytes);
+size_t wk_gemm_workspace_bytes(int dtype, int op_a, int op_b, uint64_t M, uint64_t N, uint64_t K);
+
+/* Name of the kernel variant wk_gemm() would launch for these arguments ("mfma_f32_256x128",
+ * "tile64", ...).  For benchmarks and profiles; not part of the reference's surface. */
+const char *wk_gemm_variant(int dtype, int op_a, int op_b, uint64_t M, uint64_t N, uint64_t K,
+                            uint64_t lda, uint64_t ldb, uint64_t ldc, const void *A, const void *B, const void *C);
+
+/* Test/benchmark knob: force a gemm variant by name ("auto" restores selection).
+ * Returns WK_E_INVALID_VALUE for an unknown name. */
+int wk_gemm_force_variant(const char *name);
+
+/* A plain device-to-device streaming copy kernel of known size, used only to calibrate
+ * profiler byte counters against a known amount of traffic. */
+int wk_copy_kernel(wk_stream *s, void *dst, const void *src, size_t bytes);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* WEKUA_HIP_H */

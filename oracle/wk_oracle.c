@@ -1,0 +1,389 @@
+/*
+ * wk_oracle.c -- CPU restatement of wekua's gemm / axpy.  TEST INFRASTRUCTURE ONLY:
+ * the checker for the HIP path and the timed "port" CPU baseline; never part of the
+ * shipped GPU path.  File-by-file map to the reference: see wk_oracle.h.
+ *
+ * The reference itself cannot be built in this image: its host is Zig (no zig
+ * toolchain; the zig-opencl v0.8.1 binding is a URL dependency) and its kernels are
+ * OpenCL C that need an OpenCL CPU runtime (none installed).  The oracle is therefore
+ * pinned without executing reference code:
+ *
+ *   wko_axpy            pinned  -- the reference's own known answers (axpy.zig:178-972:
+ *                                  2*[1..5]+[10..50], null alpha, alpha=-1, 2-D, 3-D,
+ *                                  zero alpha, complex (2+i)) + per-element closed form
+ *                                  against exact integer / float64 arithmetic.
+ *   wko_gemm            pinned  -- the reference's identity-product known answers
+ *                                  (gemm.zig:945-1307, test_helpers.zig:88-247) for every
+ *                                  block size, packed and unpacked, alpha/beta options,
+ *                                  transposes; integers by the ring identity (exact product
+ *                                  mod 2^w, order independent, vs Python big-int brute force);
+ *                                  floats vs float64/longdouble brute force within
+ *                                  1e-5*sqrt(K) / 1e-12*sqrt(K), rank-1 and all-ones closed
+ *                                  forms, integer-valued floats (exact).  Its float rounding
+ *                                  ORDER (k-pair association, per-tile partial sums) follows
+ *                                  the .cl files by reading only: parity unpinned at the
+ *                                  last-bit level, which the reference does not fix either
+ *                                  (fast-relaxed-math, device-dependent vector width).
+ *   wko_pack            pinned  -- the layout formula the reference's pack tests assert
+ *                                  (gemm.zig:1309-1951), restated independently in the tests.
+ *   wko_tensor_layout,
+ *   wko_default_block_cpu,
+ *   wko_get_algorithm   pinned  -- hand-computed cases from tensor/main.zig:142-199,
+ *                                  work_configuration.zig:110-193, gemm.zig:42-58.
+ *
+ * Build: see oracle/Makefile (-ffp-contract=off so that the unfused float path is unfused).
+ */
+#include "wk_oracle.h"
+
+#include <float.h>
+#include <math.h>
+#include <omp.h>
+#include <stdlib.h>
+#include <string.h>
+
+#define CAT_(a, b) a##b
+#define CAT(a, b) CAT_(a, b)
+
+/* ---- 10 real + 10 complex instantiations ---------------------------------------- */
+#define EPS 0
+#define FMA(a, b, c) ((a) * (b) + (c))
+#define IS_FLOAT 0
+
+#define S uint8_t
+#define W uint32_t
+#define SS int8_t
+#define IS_SIGNED 1
+#define CPLX 0
+#define NAME(x) CAT(x, _i8)
+#include "wk_oracle_impl.inc"
+#undef NAME
+#undef CPLX
+#define CPLX 1
+#define NAME(x) CAT(x, _ci8)
+#include "wk_oracle_impl.inc"
+#undef NAME
+#undef CPLX
+#undef IS_SIGNED
+#define IS_SIGNED 0
+#define CPLX 0
+#define NAME(x) CAT(x, _u8)
+#include "wk_oracle_impl.inc"
+#undef NAME
+#undef CPLX
+#define CPLX 1
+#define NAME(x) CAT(x, _cu8)
+#include "wk_oracle_impl.inc"
+#undef NAME
+#undef CPLX
+#undef IS_SIGNED
+#undef S
+#undef SS
+
+#define S uint16_t
+#define SS int16_t
+#define IS_SIGNED 1
+#define CPLX 0
+#define NAME(x) CAT(x, _i16)
+#include "wk_oracle_impl.inc"
+#undef NAME
+#undef CPLX
+#define CPLX 1
+#define NAME(x) CAT(x, _ci16)
+#include "wk_oracle_impl.inc"
+#undef NAME
+#undef CPLX
+#undef IS_SIGNED
+#define IS_SIGNED 0
+#define CPLX 0
+#define NAME(x) CAT(x, _u16)
+#include "wk_oracle_impl.inc"
+#undef NAME
+#undef CPLX
+#define CPLX 1
+#define NAME(x) CAT(x, _cu16)
+#include "wk_oracle_impl.inc"
+#undef NAME
+#undef CPLX
+#undef IS_SIGNED
+#undef S
+#undef SS
+
+#define S uint32_t
+#define SS int32_t
+#define IS_SIGNED 1
+#define CPLX 0
+#define NAME(x) CAT(x, _i32)
+#include "wk_oracle_impl.inc"
+#undef NAME
+#undef CPLX
+#define CPLX 1
+#define NAME(x) CAT(x, _ci32)
+#include "wk_oracle_impl.inc"
+#undef NAME
+#undef CPLX
+#undef IS_SIGNED
+#define IS_SIGNED 0
+#define CPLX 0
+#define NAME(x) CAT(x, _u32)
+#include "wk_oracle_impl.inc"
+#undef NAME
+#undef CPLX
+#define CPLX 1
+#define NAME(x) CAT(x, _cu32)
+#include "wk_oracle_impl.inc"
+#undef NAME
+#undef CPLX
+#undef IS_SIGNED
+#undef S
+#undef SS
+#undef W
+
+#define S uint64_t
+#define W uint64_t
+#define SS int64_t
+#define IS_SIGNED 1
+#define CPLX 0
+#define NAME(x) CAT(x, _i64)
+#include "wk_oracle_impl.inc"
+#undef NAME
+#undef CPLX
+#define CPLX 1
+#define NAME(x) CAT(x, _ci64)
+#include "wk_oracle_impl.inc"
+#undef NAME
+#undef CPLX
+#undef IS_SIGNED
+#define IS_SIGNED 0
+#define CPLX 0
+#define NAME(x) CAT(x, _u64)
+#include "wk_oracle_impl.inc"
+#undef NAME
+#undef CPLX
+#define CPLX 1
+#define NAME(x) CAT(x, _cu64)
+#include "wk_oracle_impl.inc"
+#undef NAME
+#undef CPLX
+#undef IS_SIGNED
+#undef S
+#undef SS
+#undef W
+
+#undef IS_FLOAT
+#undef EPS
+#undef FMA
+#define IS_FLOAT 1
+#define IS_SIGNED 1
+
+#define S float
+#define W float
+#define SS float
+#define EPS FLT_EPSILON
+#define FMA(a, b, c) fmaf((a), (b), (c))
+#define CPLX 0
+#define NAME(x) CAT(x, _f32)
+#include "wk_oracle_impl.inc"
+#undef NAME
+#undef CPLX
+#define CPLX 1
+#define NAME(x) CAT(x, _cf32)
+#include "wk_oracle_impl.inc"
+#undef NAME
+#undef CPLX
+#undef S
+#undef W
+#undef SS
+#undef EPS
+#undef FMA
+
+#define S double
+#define W double
+#define SS double
+#define EPS DBL_EPSILON
+#define FMA(a, b, c) fma((a), (b), (c))
+#define CPLX 0
+#define NAME(x) CAT(x, _f64)
+#include "wk_oracle_impl.inc"
+#undef NAME
+#undef CPLX
+#define CPLX 1
+#define NAME(x) CAT(x, _cf64)
+#include "wk_oracle_impl.inc"
+#undef NAME
+#undef CPLX
+#undef S
+#undef W
+#undef SS
+#undef EPS
+#undef FMA
+
+/* ---- dtype helpers ------------------------------------------------------------- */
+
+static const size_t k_real_size[10] = {1, 1, 2, 2, 4, 4, 8, 8, 4, 8};
+
+size_t wko_dtype_size(int dtype) {
+    if (dtype < 0 || dtype >= 20) return 0;
+    return dtype >= 10 ? 2 * k_real_size[dtype - 10] : k_real_size[dtype];
+}
+
+/* Dispatch helper: real tags in dtype order, complex tags prefixed with c */
+#define DISPATCH(dtype, CALL)                                   \
+    switch (dtype) {                                            \
+    case 0:  CALL(_i8);   break; case 1:  CALL(_u8);   break;   \
+    case 2:  CALL(_i16);  break; case 3:  CALL(_u16);  break;   \
+    case 4:  CALL(_i32);  break; case 5:  CALL(_u32);  break;   \
+    case 6:  CALL(_i64);  break; case 7:  CALL(_u64);  break;   \
+    case 8:  CALL(_f32);  break; case 9:  CALL(_f64);  break;   \
+    case 10: CALL(_ci8);  break; case 11: CALL(_cu8);  break;   \
+    case 12: CALL(_ci16); break; case 13: CALL(_cu16); break;   \
+    case 14: CALL(_ci32); break; case 15: CALL(_cu32); break;   \
+    case 16: CALL(_ci64); break; case 17: CALL(_cu64); break;   \
+    case 18: CALL(_cf32); break; case 19: CALL(_cf64); break;   \
+    default: return -1;                                         \
+    }
+
+/* ---- layout / block choice ----------------------------------------------------- */
+
+int wko_tensor_layout(const uint64_t *shape, int ndim, int dtype, uint64_t vector_width,
+                      int vectors_enabled, wko_layout *out) {
+    if (ndim <= 0 || !shape || !out || dtype < 0 || dtype >= 20) return -1;
+    for (int d = 0; d < ndim; ++d) if (shape[d] == 0) return -1;
+    const int is_complex = dtype >= 10;
+    uint64_t vw = 1;
+    if (!is_complex && vectors_enabled && vector_width > 1) vw = vector_width;
+
+    const int last = ndim - 1, pen = last > 0 ? last - 1 : 0;
+    uint64_t depth = 1;
+    for (int d = 0; d < pen; ++d) depth *= shape[d];
+    const uint64_t rows = ndim >= 2 ? shape[pen] : 1, cols = shape[last];
+    const uint64_t padded_rows = rows + (rows % 2);
+
+    uint64_t row_pitch = cols;
+    if (vw > 1 && row_pitch % vw) row_pitch += vw - row_pitch % vw;
+    uint64_t rpv = row_pitch / vw;
+    const uint64_t rem = rpv % 2;
+    rpv += rem;
+    row_pitch += vw * rem;
+
+    out->depth = depth; out->rows = rows; out->cols = cols; out->padded_rows = padded_rows;
+    out->row_pitch = row_pitch; out->row_pitch_for_vectors = rpv;
+    out->slice_pitch = row_pitch * padded_rows;
+    out->number_of_elements = out->slice_pitch * depth;
+    out->number_of_elements_without_padding = depth * rows * cols;
+    out->number_of_vectors = out->number_of_elements / vw;
+    return 0;
+}
+
+int wko_default_block_cpu(uint64_t padded_rows, uint64_t row_pitch, uint64_t vector_width, size_t elem_size) {
+    int max_block = 0, algorithm = 2;
+    for (int bl = 2; bl < 128; bl *= 2)
+        if (padded_rows % bl == 0 && row_pitch % bl == 0) max_block = bl;
+    for (int bl = 2; bl < 128; bl *= 2) {
+        const uint64_t block_size = vector_width * (uint64_t)bl * elem_size;
+        if (bl <= max_block && block_size * bl <= 16 * 1024) algorithm = bl;
+    }
+    return algorithm;
+}
+
+int wko_get_algorithm(int default_block, uint64_t k_size) {
+    for (int bs = 64; bs >= 2; bs /= 2)
+        if (k_size % bs == 0 && default_block >= bs) return bs;
+    return -1; /* the reference panics */
+}
+
+/* ---- axpy ------------------------------------------------------------------------ */
+
+int wko_axpy(int dtype, const uint64_t shape3[3],
+             const void *x, uint64_t xrp, uint64_t xsp,
+             void *y, uint64_t yrp, uint64_t ysp, const void *alpha, int contract) {
+#define CALL(tag) CAT(axpy, tag)(shape3, (const CAT(elem, tag) *)x, xrp, xsp, (CAT(elem, tag) *)y, yrp, ysp, \
+                                 (const CAT(elem, tag) *)alpha, contract)
+    DISPATCH(dtype, CALL)
+#undef CALL
+    return 0;
+}
+
+/* ---- pack ------------------------------------------------------------------------ */
+
+int wko_pack(int dtype, const void *src, uint64_t src_rows, uint64_t src_cols, uint64_t src_pitch,
+             void *dst, uint64_t tiles, uint64_t ktiles, int block, uint64_t vw, int transpose) {
+    if (dtype >= 10) vw = 1;
+#define CALL(tag) CAT(pack, tag)((const CAT(elem, tag) *)src, src_rows, src_cols, src_pitch, \
+                                 (CAT(elem, tag) *)dst, tiles, ktiles, (uint64_t)block, vw, transpose)
+    DISPATCH(dtype, CALL)
+#undef CALL
+    return 0;
+}
+
+/* ---- gemm ------------------------------------------------------------------------ */
+
+typedef struct { uint64_t vw, kv, grid_rows_elems, grid_cols_elems; int block; } gemm_plan;
+
+static int plan_gemm(int dtype, int op_a, int op_b, uint64_t M, uint64_t N, uint64_t K,
+                     uint64_t device_vw, int packed, int force_block, gemm_plan *p) {
+    if (dtype < 0 || dtype >= 20 || !M || !N || !K) return -1;
+    const int is_complex = dtype >= 10;
+    if (device_vw == 0) device_vw = 1;
+    if (device_vw > 16 || (device_vw & (device_vw - 1))) return -1;
+
+    /* C's own layout and default block (tensor/main.zig:142-199, work_configuration.zig:110-193) */
+    uint64_t cshape[2] = {M, N};
+    wko_layout cl;
+    wko_tensor_layout(cshape, 2, dtype, device_vw, 1, &cl);
+    const int def_block = wko_default_block_cpu(cl.padded_rows, cl.row_pitch,
+                                                is_complex ? 1 : device_vw, wko_dtype_size(dtype));
+
+    /* lanes in use: packed path always (gemm.zig:129-137,181); unpacked only for N/T (gemm.zig:503-508) */
+    uint64_t vw = 1;
+    if (!is_complex && device_vw > 1 && (packed || (op_a == 0 && op_b == 1))) vw = device_vw;
+
+    uint64_t kv;
+    if (vw > 1) { kv = (K + vw - 1) / vw; kv += kv % 2; }   /* row_pitch_for_vectors / padded_k_size */
+    else        { kv = K + K % 2; }                          /* gemm.zig:514-515 */
+
+    int block = force_block > 0 ? force_block : wko_get_algorithm(def_block, kv);
+    if (block < 2 || block > 64 || (block & (block - 1))) return -1;
+    if (cl.padded_rows % block || cl.row_pitch % block || kv % block) return -1;
+
+    p->vw = vw; p->kv = kv; p->block = block;
+    p->grid_rows_elems = cl.padded_rows; p->grid_cols_elems = cl.row_pitch;
+    return 0;
+}
+
+int wko_gemm_block(int dtype, int op_a, int op_b, uint64_t M, uint64_t N, uint64_t K,
+                   uint64_t vector_width, int packed) {
+    gemm_plan p;
+    if (plan_gemm(dtype, op_a, op_b, M, N, K, vector_width, packed, 0, &p)) return -1;
+    return p.block;
+}
+
+int wko_gemm(int dtype, int op_a, int op_b, uint64_t M, uint64_t N, uint64_t K,
+             const void *alpha, const void *A, uint64_t lda, const void *B, uint64_t ldb,
+             const void *beta, void *C, uint64_t ldc,
+             uint64_t vector_width, int packed, int block, int contract, int threads) {
+    gemm_plan p;
+    if (plan_gemm(dtype, op_a, op_b, M, N, K, vector_width, packed, block, &p)) return -1;
+    const uint64_t grid_rows = p.grid_rows_elems / p.block, grid_cols = p.grid_cols_elems / p.block;
+
+    /* has_alpha = alpha or beta given; alpha defaults to one when only beta is (gemm.zig:500-501,592-596) */
+    union { uint8_t b[16]; float f[2]; double d[2]; uint64_t q[2]; } one;
+    memset(&one, 0, sizeof one);
+    const int rid = dtype % 10;
+    if (rid == 8) one.f[0] = 1.0f; else if (rid == 9) one.d[0] = 1.0; else one.b[0] = 1; /* little endian */
+    const void *alpha_eff = alpha ? alpha : (beta ? (const void *)&one : NULL);
+
+    int rc = 0;
+#define CALL(tag) do {                                                                     \
+        CAT(gargs, tag) g;                                                                 \
+        memset(&g, 0, sizeof g);                                                           \
+        g.A = (const CAT(elem, tag) *)A; g.B = (const CAT(elem, tag) *)B;                  \
+        g.C = (CAT(elem, tag) *)C; g.lda = lda; g.ldb = ldb; g.ldc = ldc;                  \
+        g.M = M; g.N = N; g.K = K; g.ta = op_a; g.tb = op_b;                               \
+        g.alpha = (const CAT(elem, tag) *)alpha_eff; g.beta = (const CAT(elem, tag) *)beta; \
+        g.BS = (uint64_t)p.block; g.vw = p.vw; g.kv = p.kv; g.contract = contract;         \
+        rc = CAT(gemm, tag)(&g, grid_rows, grid_cols, packed, threads);                    \
+    } while (0)
+    DISPATCH(dtype, CALL)
+#undef CALL
+    return rc;
+}

@@ -1,0 +1,136 @@
+"""GPU parity: wk_axpy (through the C ABI) against the oracle on the same seeded inputs."""
+import numpy as np
+import pytest
+
+import oracle
+from helpers import make_operand
+
+pytestmark = pytest.mark.gpu
+
+ALL_DTYPES = oracle.DTYPE_NAMES
+
+
+def run_axpy(dev, dtype, x, alpha, y, pitched=False):
+    cx = oracle.is_complex(dtype)
+    shape = x.shape[:-1] if cx else x.shape
+    cols = shape[-1]
+    rows = shape[-2] if len(shape) >= 2 else 1
+    depth = int(np.prod(shape[:-2])) if len(shape) >= 3 else 1
+    tail = (2,) if cx else ()
+    x3 = x.reshape((depth, rows, cols) + tail)
+    y3 = y.reshape((depth, rows, cols) + tail)
+    if pitched:
+        xrp, yrp = cols + 3, cols + 5
+        xs = np.full((depth, rows + 1, xrp) + tail, 55, dtype=x.dtype)
+        ys = np.full((depth, rows + 2, yrp) + tail, 66, dtype=y.dtype)
+        xs[:, :rows, :cols] = x3
+        ys[:, :rows, :cols] = y3
+        xsp, ysp = (rows + 1) * xrp, (rows + 2) * yrp
+    else:
+        xs, ys = x3, y3
+        xrp = yrp = cols
+        xsp = ysp = rows * cols
+    dx, dy = dev.upload(xs), dev.upload(ys)
+    dev.axpy(dtype, (depth, rows, cols), dx, xrp, xsp, alpha, dy, yrp, ysp)
+    dev.sync()
+    out = dy.download(ys.dtype, ys.shape)
+    dx.free(); dy.free()
+    if pitched:
+        mask = np.ones(out.shape, dtype=bool)
+        mask[:, :rows, :cols] = False
+        assert (out[mask] == 66).all(), "axpy wrote outside the logical region"
+        out = np.ascontiguousarray(out[:, :rows, :cols])
+    return out.reshape(y.shape)
+
+
+def expect(dtype, x, alpha, y):
+    """Integers: the exact result mod 2^w.  Floats: the fused form fma(alpha, x, y), which is
+    what the HIP kernel computes and one of the two roundings the reference permits."""
+    if oracle.is_float(dtype):
+        return oracle.axpy(dtype, x, alpha, y, contract=True)
+    return oracle.semantic_axpy(dtype, x, alpha, y)
+
+
+@pytest.mark.parametrize("dtype", ALL_DTYPES)
+def test_axpy_all_dtypes_shapes_alphas(dev, dtype):
+    signed = oracle.real_np_dtype(dtype).kind != "u"
+    cx = oracle.is_complex(dtype)
+    alphas = [None, 2, 0, 3]
+    if signed:
+        alphas.append(-1)
+    if oracle.is_float(dtype):
+        alphas += [0.75, -1.0 + 1e-9 if dtype.endswith("f64") else -1.0]
+    if cx:
+        alphas = [None, (2, 0), (2, 1), (0, 0)] + ([(-1, 0), (-1, -1)] if signed else [])
+    for shape in [(1,), (5,), (4,), (2, 3), (2, 2, 2), (3, 5, 7), (1000,), (4099,), (65536 + 3,), (2, 3, 4, 5)]:
+        for alpha in alphas:
+            x = make_operand(dtype, shape, 7)
+            y = make_operand(dtype, shape, 8)
+            got = run_axpy(dev, dtype, x, alpha, y)
+            want = expect(dtype, x, alpha, y)
+            if oracle.is_float(dtype) and cx:
+                np.testing.assert_allclose(got, want, rtol=1e-5 if dtype.endswith("f32") else 1e-13,
+                                           atol=1e-6 if dtype.endswith("f32") else 1e-14)
+            else:
+                assert np.array_equal(got, want), f"{dtype} shape={shape} alpha={alpha}"
+
+
+@pytest.mark.parametrize("dtype", ["f32", "f64", "i32", "u8", "cf32", "ci16"])
+def test_axpy_pitched_regions(dev, dtype):
+    for shape in [(5,), (2, 3), (3, 5, 7), (4, 33, 65)]:
+        x = make_operand(dtype, shape, 9)
+        y = make_operand(dtype, shape, 10)
+        alpha = (2, 1) if oracle.is_complex(dtype) else 3
+        got = run_axpy(dev, dtype, x, alpha, y, pitched=True)
+        want = expect(dtype, x, alpha, y)
+        if dtype == "cf32":
+            np.testing.assert_allclose(got, want, rtol=1e-5, atol=1e-6)
+        else:
+            assert np.array_equal(got, want)
+
+
+@pytest.mark.parametrize("dtype", ["f32", "f64"])
+@pytest.mark.parametrize("n", [2 ** 20, 2 ** 24])
+def test_axpy_config_sizes(dev, dtype, n):
+    """BASELINE config 2 at the sizes the oracle finishes in seconds (2^28: see the property test)."""
+    x = make_operand(dtype, (n,), 0x5EED0020)
+    y = make_operand(dtype, (n,), 0x5EED0021)
+    got = run_axpy(dev, dtype, x, 0.75, y)
+    want = oracle.axpy(dtype, x, 0.75, y, contract=True)
+    assert np.array_equal(got, want)
+    # and within one rounding of the unfused form the reference may equally produce
+    unfused = oracle.axpy(dtype, x, 0.75, y, contract=False)
+    eps = np.finfo(oracle.real_np_dtype(dtype)).eps
+    assert np.all(np.abs(got.astype(np.float64) - unfused) <= eps * (np.abs(0.75 * x.astype(np.float64)) + np.abs(got)))
+
+
+@pytest.mark.parametrize("dtype", ["f32", "f64"])
+def test_axpy_full_size_roundtrip(dev, dtype):
+    """n = 2^28 (config 2): y + a*x - a*x restores y exactly when a*x is exactly representable
+    (x, y small integers, a = 0.75 -> 3x/4 exact for multiples of 4), a size-independent property."""
+    n = 2 ** 28
+    rd = oracle.real_np_dtype(dtype)
+    rng = np.random.default_rng(3)
+    x = (rng.integers(-64, 64, size=n) * 4).astype(rd)
+    y = rng.integers(-1000, 1000, size=n).astype(rd)
+    dx, dy = dev.upload(x), dev.upload(y)
+    dev.axpy(dtype, (1, 1, n), dx, n, n, 0.75, dy, n, n)
+    mid = dy.download(rd, (n,))
+    assert np.array_equal(mid, y + rd.type(0.75) * x)
+    dev.axpy(dtype, (1, 1, n), dx, n, n, -0.75, dy, n, n)
+    back = dy.download(rd, (n,))
+    assert np.array_equal(back, y)
+    dx.free(); dy.free()
+
+
+def test_axpy_invalid_arguments(dev):
+    import ctypes
+    buf = dev.malloc(1024)
+    s3 = (ctypes.c_uint64 * 3)(1, 2, 8)
+    z3 = (ctypes.c_uint64 * 3)(1, 0, 8)
+    lib, p = dev.lib, buf.ptr
+    assert lib.wk_axpy(dev.stream, 8, z3, p, 8, 16, p, 8, 16, None) == 1      # zero dim
+    assert lib.wk_axpy(dev.stream, 8, s3, p, 4, 16, p, 8, 16, None) == 1      # pitch < cols
+    assert lib.wk_axpy(dev.stream, 25, s3, p, 8, 16, p, 8, 16, None) == 9     # bad dtype
+    assert lib.wk_axpy(dev.stream, 8, s3, None, 8, 16, p, 8, 16, None) == 1   # null
+    buf.free()

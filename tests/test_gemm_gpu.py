@@ -1,0 +1,151 @@
+"""GPU parity: wk_gemm (through the C ABI) against the oracle on the same seeded inputs."""
+import itertools
+
+import numpy as np
+import pytest
+
+import oracle
+from helpers import assert_gemm_close, gemm_operands
+
+pytestmark = pytest.mark.gpu
+
+OPS = list(itertools.product((0, 1), (0, 1)))
+
+
+def run_gemm(dev, dtype, alpha, a, op_a, b, op_b, beta, c, lda=None, ldb=None, ldc=None):
+    """Uploads dense operands (optionally re-pitched), runs wk_gemm, returns C as dense numpy."""
+    cx = oracle.is_complex(dtype)
+
+    def dims(m):
+        return m.shape[:2]
+
+    def pitched(m, ld):
+        r, cc = dims(m)
+        if ld is None or ld == cc:
+            return m, cc
+        shape = (r, ld) + ((2,) if cx else ())
+        out = np.full(shape, 77, dtype=m.dtype)    # poison in the gaps
+        out[:, :cc] = m
+        return out, ld
+
+    (M, N) = dims(c)
+    K = dims(a)[0] if op_a else dims(a)[1]
+    ap, lda = pitched(a, lda)
+    bp, ldb = pitched(b, ldb)
+    cp, ldc = pitched(c, ldc)
+    dA, dB, dC = dev.upload(ap), dev.upload(bp), dev.upload(cp)
+    dev.gemm(dtype, op_a, op_b, M, N, K, alpha, dA, lda, dB, ldb, beta, dC, ldc)
+    dev.sync()
+    out = dC.download(cp.dtype, cp.shape)
+    for d in (dA, dB, dC):
+        d.free()
+    if out.shape[1] != N:
+        gaps = out[:, N:]
+        assert (gaps == 77).all(), "gemm wrote outside the logical region of C"
+        out = np.ascontiguousarray(out[:, :N])
+    return out
+
+
+def check(dev, dtype, M, N, K, op_a, op_b, alpha, beta, seed=1, int_range=None, **ld):
+    a, b, c = gemm_operands(dtype, M, N, K, op_a, op_b, seed, int_range)
+    got = run_gemm(dev, dtype, alpha, a, op_a, b, op_b, beta, c, **ld)
+    if M * N * K <= 64 ** 3 * 8:
+        want = oracle.semantic_gemm(dtype, alpha, a, op_a, b, op_b, beta, c)
+    else:
+        want = oracle.gemm(dtype, alpha, a, op_a, b, op_b, beta, c)
+    assert_gemm_close(dtype, got, want, alpha, a, op_a, b, op_b, beta, c, K,
+                      what=f"{dtype} {M}x{N}x{K} op=({op_a},{op_b}) alpha={alpha} beta={beta}")
+
+
+SMALL_SHAPES = [(1, 1, 1), (5, 7, 3), (6, 10, 10), (33, 17, 65), (64, 64, 16), (64, 128, 96), (127, 129, 31),
+                (130, 70, 200)]
+
+
+@pytest.mark.parametrize("dtype", ["f32", "f64"])
+@pytest.mark.parametrize("op_a,op_b", OPS)
+@pytest.mark.parametrize("alpha,beta", [(None, None), (2.0, None), (1.5, 0.5), (None, -0.25)])
+def test_float_small_shapes(dev, dtype, op_a, op_b, alpha, beta):
+    for (M, N, K) in SMALL_SHAPES:
+        check(dev, dtype, M, N, K, op_a, op_b, alpha, beta)
+
+
+@pytest.mark.parametrize("variant", ["tile64", "mfma_f32_64x64", "mfma_f32_128x128", "mfma_f32_256x128"])
+@pytest.mark.parametrize("op_a,op_b", OPS)
+def test_f32_every_variant(dev, variant, op_a, op_b):
+    import ctypes
+    assert dev.lib.wk_gemm_force_variant(variant.encode()) == 0
+    try:
+        for (M, N, K) in [(256, 256, 64), (300, 200, 100), (512, 384, 256), (257, 129, 17)]:
+            check(dev, "f32", M, N, K, op_a, op_b, 1.5, 0.5, seed=11)
+    finally:
+        dev.lib.wk_gemm_force_variant(b"auto")
+
+
+@pytest.mark.parametrize("variant", ["tile64", "mfma_f64_64x64", "mfma_f64_128x128"])
+@pytest.mark.parametrize("op_a,op_b", OPS)
+def test_f64_every_variant(dev, variant, op_a, op_b):
+    assert dev.lib.wk_gemm_force_variant(variant.encode()) == 0
+    try:
+        for (M, N, K) in [(256, 256, 64), (300, 200, 100), (257, 129, 17)]:
+            check(dev, "f64", M, N, K, op_a, op_b, 1.0, 1.0, seed=12)
+    finally:
+        dev.lib.wk_gemm_force_variant(b"auto")
+
+
+@pytest.mark.parametrize("dtype", ["i8", "u8", "i16", "u16", "i32", "u32", "i64", "u64"])
+@pytest.mark.parametrize("op_a,op_b", OPS)
+def test_integer_wraparound_bit_exact(dev, dtype, op_a, op_b):
+    signed = dtype.startswith("i")
+    for (M, N, K) in [(5, 7, 3), (33, 17, 65), (64, 128, 96), (130, 70, 200)]:
+        for alpha, beta in [(None, None), (3, None), (3, -2 if signed else 250), (None, 7)]:
+            check(dev, dtype, M, N, K, op_a, op_b, alpha, beta, seed=21)   # full-range entries: overflow is the norm
+
+
+@pytest.mark.parametrize("dtype", ["cf32", "cf64", "ci32", "cu16", "ci8", "ci64"])
+def test_complex(dev, dtype):
+    for op_a, op_b in OPS:
+        for (M, N, K) in [(5, 7, 3), (33, 17, 65), (64, 96, 48)]:
+            for alpha, beta in [(None, None), ((2, 1), None), ((2, 1), (1, -1))]:
+                check(dev, dtype, M, N, K, op_a, op_b, alpha, beta, seed=31)
+
+
+@pytest.mark.parametrize("dtype", ["f32", "f64", "i32"])
+def test_leading_dimensions_and_untouched_gaps(dev, dtype):
+    for op_a, op_b in OPS:
+        M, N, K = 70, 45, 33
+        a_cols = M if op_a else K
+        b_cols = K if op_b else N
+        check(dev, dtype, M, N, K, op_a, op_b, 2, 3, seed=41, int_range=(-100, 100) if dtype == "i32" else None,
+              lda=a_cols + 3, ldb=b_cols + 5, ldc=N + 7)
+        check(dev, dtype, M, N, K, op_a, op_b, 2, 3, seed=42, int_range=(-100, 100) if dtype == "i32" else None,
+              lda=a_cols + 4, ldb=b_cols + 8, ldc=N + 4)
+
+
+def test_beta_zero_still_reads_c(dev):
+    """gemm.zig:598-602 / gemm_nxn_gpu.cl:280-298: with beta given, C_old is multiplied even if
+    beta == 0, so NaN in C propagates; with beta absent C is overwritten."""
+    a, b, c = gemm_operands("f32", 64, 64, 64, 0, 0, 5)
+    c[:] = np.nan
+    out = run_gemm(dev, "f32", 1.0, a, 0, b, 0, 0.0, c)
+    assert np.isnan(out).all()
+    out = run_gemm(dev, "f32", 1.0, a, 0, b, 0, None, c)
+    assert np.isfinite(out).all()
+
+
+def test_invalid_arguments(dev):
+    import ctypes
+    from wekua_amd import _capi
+    buf = dev.malloc(1024)
+    one = ctypes.c_float(1.0)
+    lib = dev.lib
+    p = buf.ptr
+    # zero dimension, bad op, leading dimension too small, bad dtype, null pointer
+    assert lib.wk_gemm(dev.stream, 8, 0, 0, 0, 4, 4, None, p, 4, p, 4, None, p, 4, None, 0) == 1
+    assert lib.wk_gemm(dev.stream, 8, 2, 0, 4, 4, 4, None, p, 4, p, 4, None, p, 4, None, 0) == 1
+    assert lib.wk_gemm(dev.stream, 8, 0, 0, 4, 4, 4, None, p, 3, p, 4, None, p, 4, None, 0) == 1
+    assert lib.wk_gemm(dev.stream, 8, 1, 0, 4, 4, 8, None, p, 3, p, 4, None, p, 4, None, 0) == 1
+    assert lib.wk_gemm(dev.stream, 8, 0, 0, 4, 4, 4, None, p, 4, p, 4, None, p, 3, None, 0) == 1
+    assert lib.wk_gemm(dev.stream, 20, 0, 0, 4, 4, 4, None, p, 4, p, 4, None, p, 4, None, 0) == 9
+    assert lib.wk_gemm(dev.stream, 8, 0, 0, 4, 4, 4, None, None, 4, p, 4, None, p, 4, None, 0) == 1
+    assert lib.wk_gemm(None, 8, 0, 0, 4, 4, 4, None, p, 4, p, 4, None, p, 4, None, 0) == 1
+    buf.free()

@@ -1,0 +1,96 @@
+"""ctypes binding of the C ABI declared in include/wekua_hip.h (libwekua_hip.so).
+
+The library is loaded from the package directory (built in-tree by wekua_amd/build.py).
+There is no CPU fallback: if the library is missing, loading raises.
+"""
+from __future__ import annotations
+
+import ctypes
+import os
+
+_PKG = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_PKG, "libwekua_hip.so")
+
+u64 = ctypes.c_uint64
+vp = ctypes.c_void_p
+ci = ctypes.c_int
+sz = ctypes.c_size_t
+u64p = ctypes.POINTER(u64)
+
+
+class WkProps(ctypes.Structure):
+    _fields_ = [
+        ("name", ctypes.c_char * 64),
+        ("arch", ctypes.c_char * 32),
+        ("ordinal", ci),
+        ("compute_units", ci),
+        ("wavefront_size", ci),
+        ("max_work_group_size", ci),
+        ("local_mem_bytes", u64),
+        ("global_mem_bytes", u64),
+        ("cache_line_size", ci),
+        ("clock_mhz", ci),
+    ]
+
+
+# name -> (restype, argtypes); one entry per declaration in include/wekua_hip.h
+SIGNATURES = {
+    "wk_strerror": (ctypes.c_char_p, [ci]),
+    "wk_abi_version": (ci, []),
+    "wk_dtype_size": (sz, [ci]),
+    "wk_device_count": (ci, [ctypes.POINTER(ci)]),
+    "wk_device_open": (ci, [ci, ctypes.POINTER(vp)]),
+    "wk_device_close": (None, [vp]),
+    "wk_device_props": (ci, [vp, ctypes.POINTER(WkProps)]),
+    "wk_stream_create": (ci, [vp, ctypes.POINTER(vp)]),
+    "wk_stream_destroy": (None, [vp]),
+    "wk_stream_sync": (ci, [vp]),
+    "wk_stream_native": (vp, [vp]),
+    "wk_malloc": (ci, [vp, sz, ctypes.POINTER(vp)]),
+    "wk_free": (ci, [vp, vp]),
+    "wk_mem_info": (ci, [vp, ctypes.POINTER(sz), ctypes.POINTER(sz)]),
+    "wk_memset_async": (ci, [vp, vp, ci, sz]),
+    "wk_copy_h2d_rect_async": (ci, [vp, vp, sz, sz, vp, sz, sz, sz, sz, sz]),
+    "wk_copy_d2h_rect_async": (ci, [vp, vp, sz, sz, vp, sz, sz, sz, sz, sz]),
+    "wk_copy_d2d_rect_async": (ci, [vp, vp, sz, sz, vp, sz, sz, sz, sz, sz]),
+    "wk_fill": (ci, [vp, ci, vp, u64p, u64, u64, vp]),
+    "wk_identity": (ci, [vp, ci, vp, u64, u64]),
+    "wk_axpy": (ci, [vp, ci, u64p, vp, u64, u64, vp, u64, u64, vp]),
+    "wk_gemm": (ci, [vp, ci, ci, ci, u64, u64, u64, vp, vp, u64, vp, u64, vp, vp, u64, vp, sz]),
+    "wk_gemm_workspace_bytes": (sz, [ci, ci, ci, u64, u64, u64]),
+    "wk_gemm_variant": (ctypes.c_char_p, [ci, ci, ci, u64, u64, u64, u64, u64, u64, vp, vp, vp]),
+    "wk_gemm_force_variant": (ci, [ctypes.c_char_p]),
+    "wk_copy_kernel": (ci, [vp, vp, vp, sz]),
+}
+
+_lib = None
+
+
+def load() -> ctypes.CDLL:
+    """Loads libwekua_hip.so; raises if it has not been built."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise ImportError(
+                f"{LIB_PATH} is missing: build it with `python -m wekua_amd.build` "
+                "(there is no CPU fallback for the GPU path)")
+        lib = ctypes.CDLL(LIB_PATH, mode=ctypes.RTLD_GLOBAL)
+        for name, (res, args) in SIGNATURES.items():
+            fn = getattr(lib, name)
+            fn.restype = res
+            fn.argtypes = args
+        _lib = lib
+    return _lib
+
+
+class WkError(RuntimeError):
+    def __init__(self, code: int, where: str = ""):
+        self.code = code
+        msg = load().wk_strerror(code).decode()
+        super().__init__(f"{where}: {msg} ({code})" if where else f"{msg} ({code})")
+        self.name = msg
+
+
+def check(code: int, where: str = "") -> None:
+    if code != 0:
+        raise WkError(code, where)

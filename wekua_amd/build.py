@@ -1,0 +1,77 @@
+"""Builds libwekua_hip.so (HIP kernels + C ABI) and libwekua_host.so (the host-side mirror
+of wekua's Zig API, used by the Python binding) in-tree with hipcc for gfx950."""
+from __future__ import annotations
+
+import concurrent.futures
+import os
+import subprocess
+import sys
+
+PKG = os.path.dirname(os.path.abspath(__file__))
+ROOT = os.path.dirname(PKG)
+CSRC = os.path.join(PKG, "csrc")
+HOST = os.path.join(PKG, "host")
+INCLUDE = os.path.join(ROOT, "include")
+OBJ = os.path.join(PKG, "build")
+
+LIB_HIP = os.path.join(PKG, "libwekua_hip.so")
+LIB_HOST = os.path.join(PKG, "libwekua_host.so")
+
+HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
+
+# -packed-fp32-ops off: the compiler must not form v_pk_*_f32 from scalar float code.
+HIP_FLAGS = [
+    "--offload-arch=gfx950", "-O3", "-std=c++20", "-fPIC", "-fno-gpu-rdc",
+    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    "-Wall", "-Wno-unused-function", "-Wno-unknown-warning-option",
+    "-I" + INCLUDE, "-I" + CSRC,
+]
+
+HIP_SOURCES = ["wk_runtime.hip", "wk_axpy.hip", "wk_gemm.hip", "wk_gemm_generic.hip", "wk_gemm_mfma.hip"]
+
+
+def _run(cmd):
+    res = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    if res.returncode != 0:
+        raise RuntimeError("command failed: %s\n%s" % (" ".join(cmd), res.stdout))
+    return res.stdout
+
+
+def build_hip(verbose: bool = False, extra_flags=()) -> str:
+    os.makedirs(OBJ, exist_ok=True)
+    objs = []
+    jobs = []
+    with concurrent.futures.ThreadPoolExecutor(max_workers=min(8, len(HIP_SOURCES))) as pool:
+        for src in HIP_SOURCES:
+            obj = os.path.join(OBJ, src.replace(".hip", ".o"))
+            objs.append(obj)
+            cmd = [HIPCC] + HIP_FLAGS + list(extra_flags) + ["-c", os.path.join(CSRC, src), "-o", obj]
+            jobs.append(pool.submit(_run, cmd))
+        for j in jobs:
+            out = j.result()
+            if verbose and out.strip():
+                print(out)
+    _run([HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB_HIP] + objs)
+    return LIB_HIP
+
+
+def build_host(verbose: bool = False) -> str:
+    src = os.path.join(HOST, "wekua_c.cpp")
+    if not os.path.exists(src):
+        return ""
+    cmd = ["g++", "-O2", "-std=c++17", "-fPIC", "-shared", "-Wall", "-Wextra", "-I" + INCLUDE, "-I" + HOST,
+           src, "-o", LIB_HOST, "-L" + PKG, "-lwekua_hip", "-Wl,-rpath,$ORIGIN"]
+    out = _run(cmd)
+    if verbose and out.strip():
+        print(out)
+    return LIB_HOST
+
+
+def build_all(verbose: bool = False):
+    build_hip(verbose)
+    build_host(verbose)
+
+
+if __name__ == "__main__":
+    build_all(verbose=True)
+    print("built", LIB_HIP, LIB_HOST if os.path.exists(LIB_HOST) else "")

@@ -1,0 +1,101 @@
+// blas.gemm entry point: argument validation, option semantics of alpha/beta, and the choice
+// of kernel variant (what src/blas/gemm.zig:361-440,487-617 does with JIT flags and
+// per-tensor work-item tables).
+#include "wk_internal.hpp"
+
+#include <atomic>
+#include <cstring>
+
+using namespace wk;
+
+namespace {
+
+// -2: automatic; -1: generic tile kernel; >= 0: index into the MFMA variant table
+std::atomic<int> g_forced{-2};
+
+const char *k_generic_name = "tile64";
+
+int build_problem(GemmProblem &p, int dtype, int op_a, int op_b, uint64_t M, uint64_t N, uint64_t K,
+                  const void *host_alpha, const void *A, uint64_t lda, const void *B, uint64_t ldb,
+                  const void *host_beta, void *C, uint64_t ldc) {
+    const size_t es = wk_dtype_size(dtype);
+    if (es == 0) return WK_E_TYPE_NOT_SUPPORTED;
+    if ((op_a != WK_OP_NO_TRANSPOSE && op_a != WK_OP_TRANSPOSE) || (op_b != WK_OP_NO_TRANSPOSE && op_b != WK_OP_TRANSPOSE))
+        return WK_E_INVALID_VALUE;
+    if (!M || !N || !K || !A || !B || !C) return WK_E_INVALID_VALUE;
+    // stored shapes: A is M x K (N) or K x M (T); B is K x N (N) or N x K (T)
+    const uint64_t a_cols = op_a ? M : K, b_cols = op_b ? K : N;
+    if (lda < a_cols || ldb < b_cols || ldc < N) return WK_E_INVALID_VALUE;
+
+    p.dtype = dtype; p.op_a = op_a; p.op_b = op_b;
+    p.M = M; p.N = N; p.K = K; p.lda = lda; p.ldb = ldb; p.ldc = ldc;
+    p.A = A; p.B = B; p.C = C;
+    std::memset(p.alpha, 0, sizeof p.alpha);
+    std::memset(p.beta, 0, sizeof p.beta);
+    // has_alpha = alpha or beta given; alpha defaults to one (src/blas/gemm.zig:500-501,592-596)
+    if (!host_alpha && !host_beta) {
+        p.epi = EPI_STORE;
+    } else {
+        p.epi = host_beta ? EPI_ALPHA_BETA : EPI_ALPHA;
+        if (host_alpha) {
+            std::memcpy(p.alpha, host_alpha, es);
+        } else {
+            const int r = dtype % 10;
+            if (r == WK_F32) { const float one = 1.f; std::memcpy(p.alpha, &one, 4); }
+            else if (r == WK_F64) { const double one = 1.; std::memcpy(p.alpha, &one, 8); }
+            else p.alpha[0] = 1; // little-endian integer one; the imaginary part stays zero
+        }
+        if (host_beta) std::memcpy(p.beta, host_beta, es);
+    }
+    return WK_OK;
+}
+
+int choose(const GemmProblem &p) {
+    const int forced = g_forced.load(std::memory_order_relaxed);
+    if (forced == -1) return -1;
+    if (forced >= 0) return gemm_mfma_variant_dtype(forced) == p.dtype ? forced : gemm_mfma_pick(p);
+    return gemm_mfma_pick(p);
+}
+
+} // namespace
+
+extern "C" {
+
+size_t wk_gemm_workspace_bytes(int, int, int, uint64_t, uint64_t, uint64_t) { return 0; }
+
+int wk_gemm(wk_stream *s, int dtype, int op_a, int op_b, uint64_t M, uint64_t N, uint64_t K, const void *host_alpha,
+            const void *A, uint64_t lda, const void *B, uint64_t ldb, const void *host_beta, void *C, uint64_t ldc,
+            void *workspace, size_t workspace_bytes) {
+    (void)workspace;
+    (void)workspace_bytes;
+    int rc = bind(s);
+    if (rc) return rc;
+    GemmProblem p;
+    rc = build_problem(p, dtype, op_a, op_b, M, N, K, host_alpha, A, lda, B, ldb, host_beta, C, ldc);
+    if (rc) return rc;
+    const int v = choose(p);
+    if (v >= 0) return gemm_mfma_launch(s->stream, p, v);
+    return gemm_generic_launch(s->stream, p);
+}
+
+const char *wk_gemm_variant(int dtype, int op_a, int op_b, uint64_t M, uint64_t N, uint64_t K, uint64_t lda, uint64_t ldb,
+                            uint64_t ldc, const void *A, const void *B, const void *C) {
+    GemmProblem p;
+    // non-null stand-ins keep the alignment test meaningful when the caller passes no pointers
+    alignas(16) static unsigned char dummy[16];
+    if (build_problem(p, dtype, op_a, op_b, M, N, K, nullptr, A ? A : dummy, lda, B ? B : dummy, ldb, nullptr,
+                      C ? const_cast<void *>(C) : dummy, ldc))
+        return "invalid";
+    const int v = choose(p);
+    return v >= 0 ? gemm_mfma_variant_name(v) : k_generic_name;
+}
+
+int wk_gemm_force_variant(const char *name) {
+    if (!name || !std::strcmp(name, "auto")) { g_forced.store(-2); return WK_OK; }
+    if (!std::strcmp(name, k_generic_name)) { g_forced.store(-1); return WK_OK; }
+    for (int v = 0; gemm_mfma_variant_name(v); ++v)
+        if (!std::strcmp(name, gemm_mfma_variant_name(v))) { g_forced.store(v); return WK_OK; }
+    return WK_E_INVALID_VALUE;
+}
+
+} // extern "C"

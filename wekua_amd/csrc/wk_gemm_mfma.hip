@@ -1,0 +1,571 @@
+// f32 / f64 GEMM on the CDNA4 matrix cores (gfx950).
+//
+//   f32: v_mfma_f32_32x32x2_f32   -- one wavefront computes a 32x32 block per instruction,
+//   f64: v_mfma_f64_16x16x4_f64   -- one wavefront computes a 16x16 block per instruction.
+//
+// Structure (both precisions):
+//   * work-group = WAVES_M x WAVES_N wavefronts (64 lanes each), macro tile BM x BN of C,
+//     k advanced in steps of BK through two LDS buffers (one barrier per step);
+//   * the next k-slab is fetched from global memory into registers (16-byte loads along
+//     whichever index is contiguous for the transpose flag) while the matrix cores work on
+//     the current LDS buffer, then written to the other buffer;
+//   * LDS layouts are chosen per operand so that both the 16-byte stores and the fragment
+//     reads are bank-conflict free:
+//        k-contiguous operand (A for op_a=N, B for op_b=T): [row][BK + pad], fragments are
+//        one 16-byte read per lane (4 consecutive k of one row);
+//        m/n-contiguous operand (A for op_a=T, B for op_b=N): [k][rows + pad], fragments
+//        are 4-byte reads, 32 consecutive lanes on consecutive addresses;
+//     both give lane l the k values k0 + KL*(l / ROWS) + t for t = 0..KL-1, so the two
+//     operands of one instruction always agree on k;
+//   * work-groups are renumbered so that the 8 XCDs (each with its own L2) get contiguous
+//     runs of tiles, and tiles are walked in groups of GROUP_M rows for L2 reuse;
+//   * the epilogue applies the reference's option semantics (src/blas/gemm.zig:500-501,
+//     591-602): store / alpha*acc / alpha*acc + beta*C_old.
+//
+// The EDGE instantiation bounds-checks every global access (ragged M, N, K, unaligned
+// leading dimensions); the interior instantiation assumes M % BM == N % BN == K % BK == 0
+// and 16-byte aligned rows.
+#include "wk_internal.hpp"
+
+#include <cstring>
+
+using namespace wk;
+
+namespace {
+
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef double f64x2 __attribute__((ext_vector_type(2)));
+typedef double f64x4 __attribute__((ext_vector_type(4)));
+
+constexpr int GROUP_M = 8;
+constexpr int NUM_XCD = 8;
+
+template <typename T> struct MArgs {
+    const T *A, *B;
+    T *C;
+    uint32_t M, N, K;
+    uint32_t lda, ldb, ldc;
+    uint32_t tiles_m, tiles_n;
+    int epi;
+    T alpha, beta;
+};
+
+// blockIdx.x -> (tile_m, tile_n): XCD-contiguous renumbering, then grouped row-major walk.
+__device__ __forceinline__ void tile_coords(uint32_t tiles_m, uint32_t tiles_n, uint32_t &tm, uint32_t &tn) {
+    const uint32_t nb = gridDim.x;
+    uint32_t pid = blockIdx.x;
+    if ((nb % NUM_XCD) == 0) pid = (pid % NUM_XCD) * (nb / NUM_XCD) + pid / NUM_XCD;
+    const uint32_t group_size = GROUP_M * tiles_n;
+    const uint32_t group = pid / group_size;
+    const uint32_t first_m = group * GROUP_M;
+    const uint32_t gsz = min(tiles_m - first_m, (uint32_t)GROUP_M);
+    const uint32_t in_group = pid - group * group_size;
+    tm = first_m + in_group % gsz;
+    tn = in_group / gsz;
+}
+
+// ------------------------------------------------------------------------------------ f32 ---
+
+// LDS geometry of one operand slab (ROWS rows of the m or n index, BK values of k)
+template <int ROWS, int BK, bool KCONTIG> struct Slab {
+    static constexpr int LD = KCONTIG ? BK + 4 : ROWS + 8; // floats per LDS row
+    static constexpr int SIZE = KCONTIG ? ROWS * LD : BK * LD;
+};
+
+template <int BM, int BN, int BK, int WAVES_M, int WAVES_N, bool A_K, bool B_K, bool EDGE>
+__global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void gemm_f32_mfma_kernel(MArgs<float> g) {
+    constexpr int NT = WAVES_M * WAVES_N * 64;
+    constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N;
+    constexpr int FM = WM / 32, FN = WN / 32;
+    static_assert(WM % 32 == 0 && WN % 32 == 0 && BK % 8 == 0, "tile shape");
+    using SA = Slab<BM, BK, A_K>;
+    using SB = Slab<BN, BK, B_K>;
+    constexpr int A_V4 = BM * BK / 4 / NT, B_V4 = BN * BK / 4 / NT; // 16-byte loads per thread per slab
+    static_assert(A_V4 * NT * 4 == BM * BK && B_V4 * NT * 4 == BN * BK, "slab must divide over the threads");
+
+    extern __shared__ __align__(16) float lds[];
+    float *As = lds;                     // [2][SA::SIZE]
+    float *Bs = lds + 2 * SA::SIZE;      // [2][SB::SIZE]
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63, wave = tid >> 6;
+    const int wm = wave / WAVES_N, wn = wave % WAVES_N;
+    const int l32 = lane & 31, lhi = lane >> 5;
+
+    uint32_t tile_m, tile_n;
+    tile_coords(g.tiles_m, g.tiles_n, tile_m, tile_n);
+    const uint32_t m0 = tile_m * BM, n0 = tile_n * BN;
+
+    f32x16 acc[FM][FN];
+#pragma unroll
+    for (int i = 0; i < FM; ++i)
+#pragma unroll
+        for (int j = 0; j < FN; ++j)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+
+    f32x4 ra[A_V4], rb[B_V4];
+
+    // ---- global -> registers -----------------------------------------------------------
+    // KCONTIG: slab is ROWS x BK, q -> (row = q / (BK/4), c4 = q % (BK/4)), address row*ld + k0 + 4*c4
+    // else   : slab is BK x ROWS, q -> (k = q / (ROWS/4), c4 = q % (ROWS/4)), address (k0+k)*ld + 4*c4
+    auto gload = [&](f32x4 *dst, const float *__restrict__ base, uint32_t ld, uint32_t row0, uint32_t row_lim,
+                     uint32_t k0, auto kc_tag, auto rows_tag, auto nv_tag) {
+        constexpr bool KC = decltype(kc_tag)::value;
+        constexpr int ROWS = decltype(rows_tag)::value;
+        constexpr int NV = decltype(nv_tag)::value;
+#pragma unroll
+        for (int i = 0; i < NV; ++i) {
+            const int q = tid + i * NT;
+            uint32_t r, c;     // r: index along the row-of-storage direction, c: first of 4 contiguous
+            uint32_t r_lim, c_lim;
+            if constexpr (KC) {
+                r = row0 + q / (BK / 4); c = k0 + 4 * (q % (BK / 4));
+                r_lim = row_lim; c_lim = g.K;
+            } else {
+                r = k0 + q / (ROWS / 4); c = row0 + 4 * (q % (ROWS / 4));
+                r_lim = g.K; c_lim = row_lim;
+            }
+            const float *p = base + (size_t)r * ld + c;
+            if constexpr (!EDGE) {
+                dst[i] = *reinterpret_cast<const f32x4 *>(p);
+            } else {
+                f32x4 v = {0.f, 0.f, 0.f, 0.f};
+                if (r < r_lim) {
+                    if (c + 3 < c_lim && ((reinterpret_cast<uintptr_t>(p) & 15u) == 0)) {
+                        v = *reinterpret_cast<const f32x4 *>(p);
+                    } else {
+                        if (c + 0 < c_lim) v[0] = p[0];
+                        if (c + 1 < c_lim) v[1] = p[1];
+                        if (c + 2 < c_lim) v[2] = p[2];
+                        if (c + 3 < c_lim) v[3] = p[3];
+                    }
+                }
+                dst[i] = v;
+            }
+        }
+    };
+    // ---- registers -> LDS ------------------------------------------------------------------
+    auto sstore = [&](float *slab, const f32x4 *src, auto kc_tag, auto rows_tag, auto nv_tag) {
+        constexpr bool KC = decltype(kc_tag)::value;
+        constexpr int ROWS = decltype(rows_tag)::value;
+        constexpr int NV = decltype(nv_tag)::value;
+        constexpr int LD = Slab<ROWS, BK, KC>::LD;
+#pragma unroll
+        for (int i = 0; i < NV; ++i) {
+            const int q = tid + i * NT;
+            int off;
+            if constexpr (KC) off = (q / (BK / 4)) * LD + 4 * (q % (BK / 4));
+            else off = (q / (ROWS / 4)) * LD + 4 * (q % (ROWS / 4));
+            *reinterpret_cast<f32x4 *>(slab + off) = src[i];
+        }
+    };
+
+    using std::integral_constant;
+    auto load_a = [&](uint32_t k0) {
+        gload(ra, g.A, g.lda, m0, g.M, k0, integral_constant<bool, A_K>{}, integral_constant<int, BM>{},
+              integral_constant<int, A_V4>{});
+    };
+    auto load_b = [&](uint32_t k0) {
+        gload(rb, g.B, g.ldb, n0, g.N, k0, integral_constant<bool, B_K>{}, integral_constant<int, BN>{},
+              integral_constant<int, B_V4>{});
+    };
+    auto store_ab = [&](int buf) {
+        sstore(As + buf * SA::SIZE, ra, integral_constant<bool, A_K>{}, integral_constant<int, BM>{},
+               integral_constant<int, A_V4>{});
+        sstore(Bs + buf * SB::SIZE, rb, integral_constant<bool, B_K>{}, integral_constant<int, BN>{},
+               integral_constant<int, B_V4>{});
+    };
+
+    const uint32_t ktiles = (g.K + BK - 1) / BK;
+
+    load_a(0);
+    load_b(0);
+    store_ab(0);
+    __syncthreads();
+
+    for (uint32_t kt = 0; kt < ktiles; ++kt) {
+        const int cur = kt & 1;
+        const bool more = kt + 1 < ktiles;
+        if (more) {
+            load_a((kt + 1) * BK);
+            load_b((kt + 1) * BK);
+        }
+        const float *as = As + cur * SA::SIZE + (A_K ? (wm * WM + l32) * SA::LD : wm * WM + l32);
+        const float *bs = Bs + cur * SB::SIZE + (B_K ? (wn * WN + l32) * SB::LD : wn * WN + l32);
+#pragma unroll
+        for (int s = 0; s < BK / 8; ++s) {
+            // lane holds k = 8*s + 4*lhi + t, t = 0..3
+            f32x4 af[FM], bf[FN];
+#pragma unroll
+            for (int i = 0; i < FM; ++i) {
+                if constexpr (A_K) {
+                    af[i] = *reinterpret_cast<const f32x4 *>(as + i * 32 * SA::LD + 8 * s + 4 * lhi);
+                } else {
+#pragma unroll
+                    for (int t = 0; t < 4; ++t) af[i][t] = as[(8 * s + 4 * lhi + t) * SA::LD + i * 32];
+                }
+            }
+#pragma unroll
+            for (int j = 0; j < FN; ++j) {
+                if constexpr (B_K) {
+                    bf[j] = *reinterpret_cast<const f32x4 *>(bs + j * 32 * SB::LD + 8 * s + 4 * lhi);
+                } else {
+#pragma unroll
+                    for (int t = 0; t < 4; ++t) bf[j][t] = bs[(8 * s + 4 * lhi + t) * SB::LD + j * 32];
+                }
+            }
+#pragma unroll
+            for (int t = 0; t < 4; ++t)
+#pragma unroll
+                for (int i = 0; i < FM; ++i)
+#pragma unroll
+                    for (int j = 0; j < FN; ++j)
+                        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(af[i][t], bf[j][t], acc[i][j], 0, 0, 0);
+        }
+        if (more) store_ab(cur ^ 1);
+        __syncthreads();
+    }
+
+    // ---- epilogue: acc register r of lane l is C[8*(r/4) + 4*(l/32) + r%4][l%32] of its 32x32 block
+    const float alpha = g.alpha, beta = g.beta;
+#pragma unroll
+    for (int i = 0; i < FM; ++i)
+#pragma unroll
+        for (int j = 0; j < FN; ++j) {
+            const uint32_t col = n0 + wn * WN + j * 32 + l32;
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const uint32_t row = m0 + wm * WM + i * 32 + 8 * (r / 4) + 4 * lhi + (r % 4);
+                if (EDGE && (row >= g.M || col >= g.N)) continue;
+                float *p = g.C + (size_t)row * g.ldc + col;
+                float v = acc[i][j][r];
+                if (g.epi == EPI_ALPHA) v = alpha * v;
+                else if (g.epi == EPI_ALPHA_BETA) v = alpha * v + beta * (*p);
+                *p = v;
+            }
+        }
+}
+
+// ------------------------------------------------------------------------------------ f64 ---
+// Same structure with v_mfma_f64_16x16x4_f64: lane l supplies A[l%16][l/16] and B[l/16][l%16];
+// result register r of lane l is C[4*(l/16) + r][l%16] of the 16x16 block.
+// LDS element = double, "vectors" are 2 doubles (16 bytes).
+
+template <int ROWS, int BK, bool KCONTIG> struct SlabD {
+    static constexpr int LD = KCONTIG ? BK + 2 : ROWS + 4; // doubles per LDS row
+    static constexpr int SIZE = KCONTIG ? ROWS * LD : BK * LD;
+};
+
+template <int BM, int BN, int BK, int WAVES_M, int WAVES_N, bool A_K, bool B_K, bool EDGE>
+__global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void gemm_f64_mfma_kernel(MArgs<double> g) {
+    constexpr int NT = WAVES_M * WAVES_N * 64;
+    constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N;
+    constexpr int FM = WM / 16, FN = WN / 16;
+    static_assert(WM % 16 == 0 && WN % 16 == 0 && BK % 8 == 0, "tile shape");
+    using SA = SlabD<BM, BK, A_K>;
+    using SB = SlabD<BN, BK, B_K>;
+    constexpr int A_V2 = BM * BK / 2 / NT, B_V2 = BN * BK / 2 / NT;
+    static_assert(A_V2 * NT * 2 == BM * BK && B_V2 * NT * 2 == BN * BK, "slab must divide over the threads");
+
+    extern __shared__ __align__(16) float lds[];
+    double *As = reinterpret_cast<double *>(lds);
+    double *Bs = As + 2 * SA::SIZE;
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63, wave = tid >> 6;
+    const int wm = wave / WAVES_N, wn = wave % WAVES_N;
+    const int l16 = lane & 15, lq = lane >> 4; // lq = 0..3
+
+    uint32_t tile_m, tile_n;
+    tile_coords(g.tiles_m, g.tiles_n, tile_m, tile_n);
+    const uint32_t m0 = tile_m * BM, n0 = tile_n * BN;
+
+    f64x4 acc[FM][FN];
+#pragma unroll
+    for (int i = 0; i < FM; ++i)
+#pragma unroll
+        for (int j = 0; j < FN; ++j)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) acc[i][j][r] = 0.0;
+
+    f64x2 ra[A_V2], rb[B_V2];
+
+    auto gload = [&](f64x2 *dst, const double *__restrict__ base, uint32_t ld, uint32_t row0, uint32_t row_lim,
+                     uint32_t k0, auto kc_tag, auto rows_tag, auto nv_tag) {
+        constexpr bool KC = decltype(kc_tag)::value;
+        constexpr int ROWS = decltype(rows_tag)::value;
+        constexpr int NV = decltype(nv_tag)::value;
+#pragma unroll
+        for (int i = 0; i < NV; ++i) {
+            const int q = tid + i * NT;
+            uint32_t r, c, r_lim, c_lim;
+            if constexpr (KC) {
+                r = row0 + q / (BK / 2); c = k0 + 2 * (q % (BK / 2));
+                r_lim = row_lim; c_lim = g.K;
+            } else {
+                r = k0 + q / (ROWS / 2); c = row0 + 2 * (q % (ROWS / 2));
+                r_lim = g.K; c_lim = row_lim;
+            }
+            const double *p = base + (size_t)r * ld + c;
+            if constexpr (!EDGE) {
+                dst[i] = *reinterpret_cast<const f64x2 *>(p);
+            } else {
+                f64x2 v = {0.0, 0.0};
+                if (r < r_lim) {
+                    if (c + 1 < c_lim && ((reinterpret_cast<uintptr_t>(p) & 15u) == 0)) {
+                        v = *reinterpret_cast<const f64x2 *>(p);
+                    } else {
+                        if (c + 0 < c_lim) v[0] = p[0];
+                        if (c + 1 < c_lim) v[1] = p[1];
+                    }
+                }
+                dst[i] = v;
+            }
+        }
+    };
+    auto sstore = [&](double *slab, const f64x2 *src, auto kc_tag, auto rows_tag, auto nv_tag) {
+        constexpr bool KC = decltype(kc_tag)::value;
+        constexpr int ROWS = decltype(rows_tag)::value;
+        constexpr int NV = decltype(nv_tag)::value;
+        constexpr int LD = SlabD<ROWS, BK, KC>::LD;
+#pragma unroll
+        for (int i = 0; i < NV; ++i) {
+            const int q = tid + i * NT;
+            int off;
+            if constexpr (KC) off = (q / (BK / 2)) * LD + 2 * (q % (BK / 2));
+            else off = (q / (ROWS / 2)) * LD + 2 * (q % (ROWS / 2));
+            *reinterpret_cast<f64x2 *>(slab + off) = src[i];
+        }
+    };
+
+    using std::integral_constant;
+    auto load_a = [&](uint32_t k0) {
+        gload(ra, g.A, g.lda, m0, g.M, k0, integral_constant<bool, A_K>{}, integral_constant<int, BM>{},
+              integral_constant<int, A_V2>{});
+    };
+    auto load_b = [&](uint32_t k0) {
+        gload(rb, g.B, g.ldb, n0, g.N, k0, integral_constant<bool, B_K>{}, integral_constant<int, BN>{},
+              integral_constant<int, B_V2>{});
+    };
+    auto store_ab = [&](int buf) {
+        sstore(As + buf * SA::SIZE, ra, integral_constant<bool, A_K>{}, integral_constant<int, BM>{},
+               integral_constant<int, A_V2>{});
+        sstore(Bs + buf * SB::SIZE, rb, integral_constant<bool, B_K>{}, integral_constant<int, BN>{},
+               integral_constant<int, B_V2>{});
+    };
+
+    const uint32_t ktiles = (g.K + BK - 1) / BK;
+    load_a(0);
+    load_b(0);
+    store_ab(0);
+    __syncthreads();
+
+    for (uint32_t kt = 0; kt < ktiles; ++kt) {
+        const int cur = kt & 1;
+        const bool more = kt + 1 < ktiles;
+        if (more) {
+            load_a((kt + 1) * BK);
+            load_b((kt + 1) * BK);
+        }
+        const double *as = As + cur * SA::SIZE + (A_K ? (wm * WM + l16) * SA::LD : wm * WM + l16);
+        const double *bs = Bs + cur * SB::SIZE + (B_K ? (wn * WN + l16) * SB::LD : wn * WN + l16);
+#pragma unroll
+        for (int s = 0; s < BK / 8; ++s) {
+            // lane holds k = 8*s + 2*lq + t, t = 0..1  (two instructions per 8 k)
+            f64x2 af[FM], bf[FN];
+#pragma unroll
+            for (int i = 0; i < FM; ++i) {
+                if constexpr (A_K) {
+                    af[i] = *reinterpret_cast<const f64x2 *>(as + i * 16 * SA::LD + 8 * s + 2 * lq);
+                } else {
+#pragma unroll
+                    for (int t = 0; t < 2; ++t) af[i][t] = as[(8 * s + 2 * lq + t) * SA::LD + i * 16];
+                }
+            }
+#pragma unroll
+            for (int j = 0; j < FN; ++j) {
+                if constexpr (B_K) {
+                    bf[j] = *reinterpret_cast<const f64x2 *>(bs + j * 16 * SB::LD + 8 * s + 2 * lq);
+                } else {
+#pragma unroll
+                    for (int t = 0; t < 2; ++t) bf[j][t] = bs[(8 * s + 2 * lq + t) * SB::LD + j * 16];
+                }
+            }
+#pragma unroll
+            for (int t = 0; t < 2; ++t)
+#pragma unroll
+                for (int i = 0; i < FM; ++i)
+#pragma unroll
+                    for (int j = 0; j < FN; ++j)
+                        acc[i][j] = __builtin_amdgcn_mfma_f64_16x16x4f64(af[i][t], bf[j][t], acc[i][j], 0, 0, 0);
+        }
+        if (more) store_ab(cur ^ 1);
+        __syncthreads();
+    }
+
+    const double alpha = g.alpha, beta = g.beta;
+#pragma unroll
+    for (int i = 0; i < FM; ++i)
+#pragma unroll
+        for (int j = 0; j < FN; ++j) {
+            const uint32_t col = n0 + wn * WN + j * 16 + l16;
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const uint32_t row = m0 + wm * WM + i * 16 + 4 * lq + r;
+                if (EDGE && (row >= g.M || col >= g.N)) continue;
+                double *p = g.C + (size_t)row * g.ldc + col;
+                double v = acc[i][j][r];
+                if (g.epi == EPI_ALPHA) v = alpha * v;
+                else if (g.epi == EPI_ALPHA_BETA) v = alpha * v + beta * (*p);
+                *p = v;
+            }
+        }
+}
+
+// ------------------------------------------------------------------------------ dispatch ---
+
+struct Variant {
+    const char *name;
+    int dtype;
+    int bm, bn, bk;
+    size_t lds_bytes[4]; // per (op_a, op_b)
+    int (*launch)(hipStream_t, const GemmProblem &, bool edge);
+};
+
+template <typename T> MArgs<T> make_args(const GemmProblem &p, int bm, int bn) {
+    MArgs<T> g;
+    g.A = static_cast<const T *>(p.A);
+    g.B = static_cast<const T *>(p.B);
+    g.C = static_cast<T *>(p.C);
+    g.M = (uint32_t)p.M; g.N = (uint32_t)p.N; g.K = (uint32_t)p.K;
+    g.lda = (uint32_t)p.lda; g.ldb = (uint32_t)p.ldb; g.ldc = (uint32_t)p.ldc;
+    g.tiles_m = (uint32_t)((p.M + bm - 1) / bm);
+    g.tiles_n = (uint32_t)((p.N + bn - 1) / bn);
+    g.epi = p.epi;
+    std::memcpy(&g.alpha, p.alpha, sizeof(T));
+    std::memcpy(&g.beta, p.beta, sizeof(T));
+    return g;
+}
+
+template <typename K> int set_lds(K kernel, size_t bytes) {
+    if (bytes > 48 * 1024) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes);
+        if (e != hipSuccess) { (void)hipGetLastError(); return hip_code(e); }
+    }
+    return WK_OK;
+}
+
+template <int BM, int BN, int BK, int WMS, int WNS, bool AK, bool BKC, bool EDGE>
+int launch_f32_one(hipStream_t st, const GemmProblem &p) {
+    constexpr size_t lds = 2 * (Slab<BM, BK, AK>::SIZE + Slab<BN, BK, BKC>::SIZE) * sizeof(float);
+    auto kern = gemm_f32_mfma_kernel<BM, BN, BK, WMS, WNS, AK, BKC, EDGE>;
+    static int attr_rc = set_lds(kern, lds);
+    if (attr_rc) return attr_rc;
+    MArgs<float> g = make_args<float>(p, BM, BN);
+    hipLaunchKernelGGL(kern, dim3(g.tiles_m * g.tiles_n), dim3(WMS * WNS * 64), lds, st, g);
+    return launch_status();
+}
+
+template <int BM, int BN, int BK, int WMS, int WNS>
+int launch_f32(hipStream_t st, const GemmProblem &p, bool edge) {
+    const int sel = (p.op_a ? 0 : 2) | (p.op_b ? 1 : 0); // bit1: A k-contiguous, bit0: B k-contiguous
+#define WK_CASE(AK, BKC)                                                                                   \
+    return edge ? launch_f32_one<BM, BN, BK, WMS, WNS, AK, BKC, true>(st, p)                               \
+                : launch_f32_one<BM, BN, BK, WMS, WNS, AK, BKC, false>(st, p)
+    switch (sel) {
+    case 0: WK_CASE(false, false);
+    case 1: WK_CASE(false, true);
+    case 2: WK_CASE(true, false);
+    default: WK_CASE(true, true);
+    }
+#undef WK_CASE
+}
+
+template <int BM, int BN, int BK, int WMS, int WNS, bool AK, bool BKC, bool EDGE>
+int launch_f64_one(hipStream_t st, const GemmProblem &p) {
+    constexpr size_t lds = 2 * (SlabD<BM, BK, AK>::SIZE + SlabD<BN, BK, BKC>::SIZE) * sizeof(double);
+    auto kern = gemm_f64_mfma_kernel<BM, BN, BK, WMS, WNS, AK, BKC, EDGE>;
+    static int attr_rc = set_lds(kern, lds);
+    if (attr_rc) return attr_rc;
+    MArgs<double> g = make_args<double>(p, BM, BN);
+    hipLaunchKernelGGL(kern, dim3(g.tiles_m * g.tiles_n), dim3(WMS * WNS * 64), lds, st, g);
+    return launch_status();
+}
+
+template <int BM, int BN, int BK, int WMS, int WNS>
+int launch_f64(hipStream_t st, const GemmProblem &p, bool edge) {
+    const int sel = (p.op_a ? 0 : 2) | (p.op_b ? 1 : 0);
+#define WK_CASE(AK, BKC)                                                                                   \
+    return edge ? launch_f64_one<BM, BN, BK, WMS, WNS, AK, BKC, true>(st, p)                               \
+                : launch_f64_one<BM, BN, BK, WMS, WNS, AK, BKC, false>(st, p)
+    switch (sel) {
+    case 0: WK_CASE(false, false);
+    case 1: WK_CASE(false, true);
+    case 2: WK_CASE(true, false);
+    default: WK_CASE(true, true);
+    }
+#undef WK_CASE
+}
+
+struct VariantDesc {
+    const char *name;
+    int dtype, bm, bn, bk;
+    int (*launch)(hipStream_t, const GemmProblem &, bool);
+};
+
+const VariantDesc k_variants[] = {
+    {"mfma_f32_256x128", WK_F32, 256, 128, 16, &launch_f32<256, 128, 16, 2, 2>},
+    {"mfma_f32_128x128", WK_F32, 128, 128, 16, &launch_f32<128, 128, 16, 2, 2>},
+    {"mfma_f32_64x64", WK_F32, 64, 64, 16, &launch_f32<64, 64, 16, 2, 2>},
+    {"mfma_f64_128x128", WK_F64, 128, 128, 16, &launch_f64<128, 128, 16, 2, 2>},
+    {"mfma_f64_64x64", WK_F64, 64, 64, 16, &launch_f64<64, 64, 16, 2, 2>},
+};
+constexpr int k_num_variants = sizeof(k_variants) / sizeof(k_variants[0]);
+
+bool needs_edge(const GemmProblem &p, const VariantDesc &v) {
+    const size_t es = p.dtype == WK_F32 ? 4 : 8;
+    const uint64_t vec = 16 / es;
+    if (p.M % v.bm || p.N % v.bn || p.K % v.bk) return true;
+    if (p.lda % vec || p.ldb % vec) return true;
+    if ((reinterpret_cast<uintptr_t>(p.A) | reinterpret_cast<uintptr_t>(p.B)) & 15u) return true;
+    return false;
+}
+
+} // namespace
+
+const char *wk::gemm_mfma_variant_name(int variant) {
+    return (variant >= 0 && variant < k_num_variants) ? k_variants[variant].name : nullptr;
+}
+
+int wk::gemm_mfma_variant_dtype(int variant) {
+    return (variant >= 0 && variant < k_num_variants) ? k_variants[variant].dtype : -1;
+}
+
+// Largest macro tile that still yields at least ~2 work-groups per CU; small problems take
+// smaller tiles so that the 256 CUs are not left idle.
+int wk::gemm_mfma_pick(const GemmProblem &p) {
+    if (p.dtype != WK_F32 && p.dtype != WK_F64) return -1;
+    if (p.M > 0x7fffffffull || p.N > 0x7fffffffull || p.K > 0x7fffffffull || p.lda > 0x7fffffffull ||
+        p.ldb > 0x7fffffffull || p.ldc > 0x7fffffffull)
+        return -1;
+    int best = -1;
+    for (int v = 0; v < k_num_variants; ++v) {
+        if (k_variants[v].dtype != p.dtype) continue;
+        const uint64_t tiles = ((p.M + k_variants[v].bm - 1) / k_variants[v].bm) *
+                               ((p.N + k_variants[v].bn - 1) / k_variants[v].bn);
+        best = v;
+        if (tiles >= 512) break;
+    }
+    return best;
+}
+
+int wk::gemm_mfma_launch(hipStream_t st, const GemmProblem &p, int variant) {
+    if (variant < 0 || variant >= k_num_variants || k_variants[variant].dtype != p.dtype) return WK_E_INVALID_VALUE;
+    const VariantDesc &v = k_variants[variant];
+    const uint64_t tiles = ((p.M + v.bm - 1) / v.bm) * ((p.N + v.bn - 1) / v.bn);
+    if (tiles > 0x7fffffffull) return WK_E_INVALID_VALUE;
+    return v.launch(st, p, needs_edge(p, v));
+}

@@ -1,0 +1,160 @@
+// Internal declarations shared by the HIP translation units of libwekua_hip.
+#pragma once
+
+#include <hip/hip_runtime.h>
+
+#include <cstddef>
+#include <cstdint>
+
+#include "wekua_hip.h"
+
+struct wk_device {
+    int ordinal;
+    hipDeviceProp_t props;
+};
+
+struct wk_stream {
+    wk_device *dev;
+    hipStream_t stream;
+};
+
+namespace wk {
+
+inline int hip_code(hipError_t e) {
+    if (e == hipSuccess) return WK_OK;
+    if (e == hipErrorOutOfMemory) return WK_E_OUT_OF_MEMORY;
+    return WK_E_HIP_BASE + static_cast<int>(e);
+}
+
+#define WK_HIP_TRY(expr)                                  \
+    do {                                                  \
+        hipError_t wk_e_ = (expr);                        \
+        if (wk_e_ != hipSuccess) {                        \
+            (void)hipGetLastError();                      \
+            return ::wk::hip_code(wk_e_);                 \
+        }                                                 \
+    } while (0)
+
+// Every launch is followed by this: a bad launch configuration surfaces here, not later.
+inline int launch_status() { return hip_code(hipGetLastError()); }
+
+inline int bind(wk_stream *s) {
+    if (!s || !s->dev) return WK_E_INVALID_VALUE;
+    WK_HIP_TRY(hipSetDevice(s->dev->ordinal));
+    return WK_OK;
+}
+
+// ---- element types -------------------------------------------------------------------
+// Integer dtypes are computed in the unsigned type of the same width: +, -, * modulo 2^w
+// do not depend on signedness, and unsigned overflow is defined.  This is the wraparound
+// of the reference's OpenCL kernels (i8/i16 promote to int there and truncate on store:
+// the same low bits).
+template <typename R>
+struct cplx {
+    R re, im;
+};
+
+template <typename T> struct elem_traits;
+#define WK_REAL_TRAITS(T_, ACC_, ISF_)                                               \
+    template <> struct elem_traits<T_> {                                             \
+        using real = T_;                                                             \
+        using acc = ACC_; /* accumulator: 32-bit for narrow ints, else same type */  \
+        static constexpr bool is_complex = false;                                    \
+        static constexpr bool is_float = ISF_;                                       \
+    };
+WK_REAL_TRAITS(uint8_t, uint32_t, false)
+WK_REAL_TRAITS(uint16_t, uint32_t, false)
+WK_REAL_TRAITS(uint32_t, uint32_t, false)
+WK_REAL_TRAITS(uint64_t, uint64_t, false)
+WK_REAL_TRAITS(float, float, true)
+WK_REAL_TRAITS(double, double, true)
+#undef WK_REAL_TRAITS
+template <typename R> struct elem_traits<cplx<R>> {
+    using real = R;
+    using acc = cplx<typename elem_traits<R>::acc>;
+    static constexpr bool is_complex = true;
+    static constexpr bool is_float = elem_traits<R>::is_float;
+};
+
+template <typename A> __host__ __device__ inline A zero_of() { return A(0); }
+template <> __host__ __device__ inline cplx<uint32_t> zero_of<cplx<uint32_t>>() { return {0u, 0u}; }
+template <> __host__ __device__ inline cplx<uint64_t> zero_of<cplx<uint64_t>>() { return {0ull, 0ull}; }
+template <> __host__ __device__ inline cplx<float> zero_of<cplx<float>>() { return {0.f, 0.f}; }
+template <> __host__ __device__ inline cplx<double> zero_of<cplx<double>>() { return {0., 0.}; }
+
+// widen / narrow between storage and accumulator types
+template <typename A, typename T> __host__ __device__ inline A widen(T v) { return static_cast<A>(v); }
+template <typename A, typename R> __host__ __device__ inline A widen(cplx<R> v) {
+    return A{static_cast<decltype(A::re)>(v.re), static_cast<decltype(A::im)>(v.im)};
+}
+template <typename T, typename A> __host__ __device__ inline T narrow(A v) { return static_cast<T>(v); }
+template <typename T, typename R> __host__ __device__ inline T narrow(cplx<R> v) {
+    return T{static_cast<decltype(T::re)>(v.re), static_cast<decltype(T::im)>(v.im)};
+}
+
+template <typename A> __host__ __device__ inline A add(A a, A b) { return a + b; }
+template <typename R> __host__ __device__ inline cplx<R> add(cplx<R> a, cplx<R> b) { return {a.re + b.re, a.im + b.im}; }
+template <typename A> __host__ __device__ inline A sub(A a, A b) { return a - b; }
+template <typename R> __host__ __device__ inline cplx<R> sub(cplx<R> a, cplx<R> b) { return {a.re - b.re, a.im - b.im}; }
+template <typename A> __host__ __device__ inline A mul(A a, A b) { return a * b; }
+// The reference's complex product (src/core/wekua_cl_lib.cl:648-653): three multiplies.
+// Kept in this form so float rounding stays close to the reference's; for integers it is
+// the ordinary product modulo 2^w.
+template <typename R> __host__ __device__ inline cplx<R> mul(cplx<R> a, cplx<R> b) {
+    const R k1 = b.re * (a.re + a.im);
+    const R k2 = a.re * (b.im - b.re);
+    const R k3 = a.im * (b.re + b.im);
+    return {k1 - k3, k1 + k2};
+}
+// acc += a*b
+template <typename A> __host__ __device__ inline A mad(A a, A b, A c) { return a * b + c; }
+template <> __host__ __device__ inline float mad<float>(float a, float b, float c) { return __builtin_fmaf(a, b, c); }
+template <> __host__ __device__ inline double mad<double>(double a, double b, double c) { return __builtin_fma(a, b, c); }
+template <typename R> __host__ __device__ inline cplx<R> mad(cplx<R> a, cplx<R> b, cplx<R> c) { return add(c, mul(a, b)); }
+
+// dtype id -> run F.template operator()<T>() with the computational element type.
+template <typename F> inline int dispatch_dtype(int dtype, F &&f) {
+    switch (dtype) {
+    case WK_I8: case WK_U8:   return f.template operator()<uint8_t>();
+    case WK_I16: case WK_U16: return f.template operator()<uint16_t>();
+    case WK_I32: case WK_U32: return f.template operator()<uint32_t>();
+    case WK_I64: case WK_U64: return f.template operator()<uint64_t>();
+    case WK_F32:              return f.template operator()<float>();
+    case WK_F64:              return f.template operator()<double>();
+    case WK_COMPLEX + WK_I8: case WK_COMPLEX + WK_U8:   return f.template operator()<cplx<uint8_t>>();
+    case WK_COMPLEX + WK_I16: case WK_COMPLEX + WK_U16: return f.template operator()<cplx<uint16_t>>();
+    case WK_COMPLEX + WK_I32: case WK_COMPLEX + WK_U32: return f.template operator()<cplx<uint32_t>>();
+    case WK_COMPLEX + WK_I64: case WK_COMPLEX + WK_U64: return f.template operator()<cplx<uint64_t>>();
+    case WK_COMPLEX + WK_F32: return f.template operator()<cplx<float>>();
+    case WK_COMPLEX + WK_F64: return f.template operator()<cplx<double>>();
+    default: return WK_E_TYPE_NOT_SUPPORTED;
+    }
+}
+
+inline bool dtype_is_signed(int dtype) {
+    const int r = dtype % 10;
+    return r == WK_I8 || r == WK_I16 || r == WK_I32 || r == WK_I64 || r == WK_F32 || r == WK_F64;
+}
+
+// ---- gemm plumbing shared between wk_gemm.hip and the kernel files ------------------------
+enum : int { EPI_STORE = 0, EPI_ALPHA = 1, EPI_ALPHA_BETA = 2 };
+
+struct GemmProblem {
+    int dtype, op_a, op_b;
+    uint64_t M, N, K, lda, ldb, ldc;
+    const void *A, *B;
+    void *C;
+    int epi;                          // EPI_*
+    alignas(16) unsigned char alpha[16];  // one element of dtype (valid when epi != EPI_STORE)
+    alignas(16) unsigned char beta[16];   // one element of dtype (valid when epi == EPI_ALPHA_BETA)
+};
+
+// generic LDS-tiled VALU kernel, every dtype and shape (wk_gemm_generic.hip)
+int gemm_generic_launch(hipStream_t st, const GemmProblem &p);
+// MFMA kernels for f32 / f64 (wk_gemm_mfma.hip); `variant` indexes mfma_variant_name()
+int gemm_mfma_launch(hipStream_t st, const GemmProblem &p, int variant);
+int gemm_mfma_pick(const GemmProblem &p);        // -1: not applicable
+const char *gemm_mfma_variant_name(int variant); // nullptr past the end
+int gemm_mfma_variant_dtype(int variant);
+
+} // namespace wk

@@ -1,0 +1,286 @@
+// Device, stream, memory and the small support kernels (fill, identity, calibration copy).
+// Replaces what src/core/{context,command_queue,pipeline}.zig and src/tensor/{fill,identity,
+// memory/*}.zig obtain from OpenCL.
+#include "wk_internal.hpp"
+
+#include <cstdio>
+#include <cstring>
+#include <new>
+
+using namespace wk;
+
+extern "C" {
+
+const char *wk_strerror(int code) {
+    switch (code) {
+    case WK_OK: return "ok";
+    case WK_E_INVALID_VALUE: return "InvalidValue";
+    case WK_E_INVALID_COORDINATES: return "InvalidCoordinates";
+    case WK_E_INVALID_BUFFER: return "InvalidBuffer";
+    case WK_E_UNQUAL_TENSORS_ATTRIBUTE: return "UnqualTensorsAttribute";
+    case WK_E_UNQUAL_TENSORS_SHAPE: return "UnqualTensorsShape";
+    case WK_E_UNQUAL_TENSORS_DIMENSION: return "UnqualTensorsDimension";
+    case WK_E_UNQUAL_TENSORS_CONTEXT: return "UnqualTensorsContext";
+    case WK_E_OUT_OF_MEMORY: return "OutOfMemory";
+    case WK_E_TYPE_NOT_SUPPORTED: return "TypeNotSupported";
+    case WK_E_NO_DEVICE: return "DevicesArrayEmpty";
+    default: break;
+    }
+    if (code >= WK_E_HIP_BASE) return hipGetErrorString(static_cast<hipError_t>(code - WK_E_HIP_BASE));
+    return "unknown wekua_hip error";
+}
+
+int wk_abi_version(void) { return WK_ABI_VERSION; }
+
+size_t wk_dtype_size(int dtype) {
+    static const size_t real_size[10] = {1, 1, 2, 2, 4, 4, 8, 8, 4, 8};
+    if (dtype < 0 || dtype >= WK_DTYPE_COUNT) return 0;
+    return dtype >= WK_COMPLEX ? 2 * real_size[dtype - WK_COMPLEX] : real_size[dtype];
+}
+
+int wk_device_count(int *out_count) {
+    if (!out_count) return WK_E_INVALID_VALUE;
+    int n = 0;
+    hipError_t e = hipGetDeviceCount(&n);
+    if (e != hipSuccess) {
+        (void)hipGetLastError();
+        *out_count = 0;
+        return e == hipErrorNoDevice ? WK_OK : hip_code(e);
+    }
+    *out_count = n;
+    return WK_OK;
+}
+
+int wk_device_open(int ordinal, wk_device **out) {
+    if (!out) return WK_E_INVALID_VALUE;
+    *out = nullptr;
+    int n = 0;
+    int rc = wk_device_count(&n);
+    if (rc) return rc;
+    if (n == 0) return WK_E_NO_DEVICE;
+    if (ordinal < 0 || ordinal >= n) return WK_E_INVALID_VALUE;
+    wk_device *d = new (std::nothrow) wk_device;
+    if (!d) return WK_E_OUT_OF_MEMORY;
+    d->ordinal = ordinal;
+    hipError_t e = hipGetDeviceProperties(&d->props, ordinal);
+    if (e == hipSuccess) e = hipSetDevice(ordinal);
+    if (e != hipSuccess) {
+        (void)hipGetLastError();
+        delete d;
+        return hip_code(e);
+    }
+    *out = d;
+    return WK_OK;
+}
+
+void wk_device_close(wk_device *dev) { delete dev; }
+
+int wk_device_props(wk_device *dev, wk_props *out) {
+    if (!dev || !out) return WK_E_INVALID_VALUE;
+    std::memset(out, 0, sizeof *out);
+    std::snprintf(out->name, sizeof out->name, "%s", dev->props.name);
+    std::snprintf(out->arch, sizeof out->arch, "%s", dev->props.gcnArchName);
+    out->ordinal = dev->ordinal;
+    out->compute_units = dev->props.multiProcessorCount;
+    out->wavefront_size = dev->props.warpSize;
+    out->max_work_group_size = dev->props.maxThreadsPerBlock;
+    out->local_mem_bytes = dev->props.sharedMemPerBlock;
+    out->global_mem_bytes = dev->props.totalGlobalMem;
+    out->cache_line_size = 128;
+    out->clock_mhz = dev->props.clockRate / 1000;
+    return WK_OK;
+}
+
+int wk_stream_create(wk_device *dev, wk_stream **out) {
+    if (!dev || !out) return WK_E_INVALID_VALUE;
+    *out = nullptr;
+    WK_HIP_TRY(hipSetDevice(dev->ordinal));
+    wk_stream *s = new (std::nothrow) wk_stream;
+    if (!s) return WK_E_OUT_OF_MEMORY;
+    s->dev = dev;
+    hipError_t e = hipStreamCreateWithFlags(&s->stream, hipStreamNonBlocking);
+    if (e != hipSuccess) {
+        (void)hipGetLastError();
+        delete s;
+        return hip_code(e);
+    }
+    *out = s;
+    return WK_OK;
+}
+
+void wk_stream_destroy(wk_stream *s) {
+    if (!s) return;
+    if (hipSetDevice(s->dev->ordinal) == hipSuccess) {
+        (void)hipStreamSynchronize(s->stream);
+        (void)hipStreamDestroy(s->stream);
+    }
+    (void)hipGetLastError();
+    delete s;
+}
+
+int wk_stream_sync(wk_stream *s) {
+    int rc = bind(s);
+    if (rc) return rc;
+    WK_HIP_TRY(hipStreamSynchronize(s->stream));
+    return WK_OK;
+}
+
+void *wk_stream_native(wk_stream *s) { return s ? static_cast<void *>(s->stream) : nullptr; }
+
+int wk_malloc(wk_device *dev, size_t bytes, void **out_dptr) {
+    if (!dev || !out_dptr || bytes == 0) return WK_E_INVALID_VALUE;
+    *out_dptr = nullptr;
+    WK_HIP_TRY(hipSetDevice(dev->ordinal));
+    WK_HIP_TRY(hipMalloc(out_dptr, bytes));
+    return WK_OK;
+}
+
+int wk_free(wk_device *dev, void *dptr) {
+    if (!dev) return WK_E_INVALID_VALUE;
+    if (!dptr) return WK_OK;
+    WK_HIP_TRY(hipSetDevice(dev->ordinal));
+    WK_HIP_TRY(hipFree(dptr));
+    return WK_OK;
+}
+
+int wk_mem_info(wk_device *dev, size_t *free_bytes, size_t *total_bytes) {
+    if (!dev || !free_bytes || !total_bytes) return WK_E_INVALID_VALUE;
+    WK_HIP_TRY(hipSetDevice(dev->ordinal));
+    WK_HIP_TRY(hipMemGetInfo(free_bytes, total_bytes));
+    return WK_OK;
+}
+
+int wk_memset_async(wk_stream *s, void *dptr, int byte, size_t bytes) {
+    int rc = bind(s);
+    if (rc) return rc;
+    if (!dptr) return WK_E_INVALID_VALUE;
+    if (bytes == 0) return WK_OK;
+    WK_HIP_TRY(hipMemsetAsync(dptr, byte, bytes, s->stream));
+    return WK_OK;
+}
+
+static int rect_copy(wk_stream *s, void *dst, size_t drp, size_t dsp, const void *src, size_t srp, size_t ssp,
+                     size_t width, size_t rows, size_t slices, hipMemcpyKind kind) {
+    int rc = bind(s);
+    if (rc) return rc;
+    if (!dst || !src) return WK_E_INVALID_VALUE;
+    if (width == 0 || rows == 0 || slices == 0) return WK_OK;
+    if (drp < width || srp < width) return WK_E_INVALID_VALUE;
+    if (slices > 1 && (dsp < drp * rows || ssp < srp * rows)) return WK_E_INVALID_VALUE;
+    // fully contiguous on both sides: one linear copy
+    if (drp == width && srp == width && (slices == 1 || (dsp == width * rows && ssp == width * rows))) {
+        WK_HIP_TRY(hipMemcpyAsync(dst, src, width * rows * slices, kind, s->stream));
+        return WK_OK;
+    }
+    for (size_t z = 0; z < slices; ++z) {
+        WK_HIP_TRY(hipMemcpy2DAsync(static_cast<char *>(dst) + z * dsp, drp, static_cast<const char *>(src) + z * ssp,
+                                    srp, width, rows, kind, s->stream));
+    }
+    return WK_OK;
+}
+
+int wk_copy_h2d_rect_async(wk_stream *s, void *dst, size_t drp, size_t dsp, const void *host_src, size_t srp,
+                           size_t ssp, size_t width_bytes, size_t rows, size_t slices) {
+    return rect_copy(s, dst, drp, dsp, host_src, srp, ssp, width_bytes, rows, slices, hipMemcpyHostToDevice);
+}
+
+int wk_copy_d2h_rect_async(wk_stream *s, void *host_dst, size_t drp, size_t dsp, const void *src, size_t srp,
+                           size_t ssp, size_t width_bytes, size_t rows, size_t slices) {
+    return rect_copy(s, host_dst, drp, dsp, src, srp, ssp, width_bytes, rows, slices, hipMemcpyDeviceToHost);
+}
+
+int wk_copy_d2d_rect_async(wk_stream *s, void *dst, size_t drp, size_t dsp, const void *src, size_t srp, size_t ssp,
+                           size_t width_bytes, size_t rows, size_t slices) {
+    return rect_copy(s, dst, drp, dsp, src, srp, ssp, width_bytes, rows, slices, hipMemcpyDeviceToDevice);
+}
+
+} // extern "C"
+
+// ---- fill / identity -------------------------------------------------------------------
+
+template <typename T>
+__global__ __launch_bounds__(256) void fill_kernel(T *__restrict__ buf, uint64_t depth, uint64_t rows, uint64_t cols,
+                                                   uint64_t row_pitch, uint64_t slice_pitch, T value) {
+    const uint64_t total = depth * rows * cols;
+    for (uint64_t idx = blockIdx.x * (uint64_t)blockDim.x + threadIdx.x; idx < total;
+         idx += (uint64_t)gridDim.x * blockDim.x) {
+        const uint64_t k = idx % cols;
+        const uint64_t ij = idx / cols;
+        const uint64_t j = ij % rows, i = ij / rows;
+        buf[i * slice_pitch + j * row_pitch + k] = value;
+    }
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void identity_kernel(T *__restrict__ buf, uint64_t size, uint64_t pitch_sum, T one) {
+    const uint64_t i = blockIdx.x * (uint64_t)blockDim.x + threadIdx.x;
+    if (i < size) buf[i * pitch_sum] = one;
+}
+
+template <typename T> static T load_scalar(const void *host) {
+    T v;
+    std::memcpy(&v, host, sizeof(T));
+    return v;
+}
+
+template <typename T> static T one_of() {
+    if constexpr (elem_traits<T>::is_complex) {
+        using R = typename elem_traits<T>::real;
+        return T{R(1), R(0)};
+    } else {
+        return T(1);
+    }
+}
+
+static unsigned grid_for(uint64_t total, unsigned block) {
+    uint64_t g = (total + block - 1) / block;
+    const uint64_t cap = 256ull * 64;
+    return static_cast<unsigned>(g < cap ? (g ? g : 1) : cap);
+}
+
+extern "C" int wk_fill(wk_stream *s, int dtype, void *dptr, const uint64_t shape3[3], uint64_t row_pitch,
+                       uint64_t slice_pitch, const void *host_scalar) {
+    int rc = bind(s);
+    if (rc) return rc;
+    if (!dptr || !shape3 || !host_scalar) return WK_E_INVALID_VALUE;
+    const uint64_t d = shape3[0], r = shape3[1], c = shape3[2];
+    if (!d || !r || !c || row_pitch < c || (d > 1 && slice_pitch < row_pitch * r)) return WK_E_INVALID_VALUE;
+    return dispatch_dtype(dtype, [&]<typename T>() -> int {
+        const T v = load_scalar<T>(host_scalar);
+        hipLaunchKernelGGL(fill_kernel<T>, dim3(grid_for(d * r * c, 256)), dim3(256), 0, s->stream,
+                           static_cast<T *>(dptr), d, r, c, row_pitch, slice_pitch, v);
+        return launch_status();
+    });
+}
+
+extern "C" int wk_identity(wk_stream *s, int dtype, void *dptr, uint64_t size, uint64_t pitch_sum) {
+    int rc = bind(s);
+    if (rc) return rc;
+    if (!dptr || !size || !pitch_sum) return WK_E_INVALID_VALUE;
+    return dispatch_dtype(dtype, [&]<typename T>() -> int {
+        hipLaunchKernelGGL(identity_kernel<T>, dim3((unsigned)((size + 255) / 256)), dim3(256), 0, s->stream,
+                           static_cast<T *>(dptr), size, pitch_sum, one_of<T>());
+        return launch_status();
+    });
+}
+
+// ---- calibration copy ----------------------------------------------------------------------
+
+__global__ __launch_bounds__(256) void copy16_kernel(uint4 *__restrict__ dst, const uint4 *__restrict__ src, size_t n16) {
+    for (size_t i = blockIdx.x * (size_t)blockDim.x + threadIdx.x; i < n16; i += (size_t)gridDim.x * blockDim.x)
+        dst[i] = src[i];
+}
+
+extern "C" int wk_copy_kernel(wk_stream *s, void *dst, const void *src, size_t bytes) {
+    int rc = bind(s);
+    if (rc) return rc;
+    if (!dst || !src || bytes % 16 || (reinterpret_cast<uintptr_t>(dst) | reinterpret_cast<uintptr_t>(src)) % 16)
+        return WK_E_INVALID_VALUE;
+    if (!bytes) return WK_OK;
+    const size_t n16 = bytes / 16;
+    const size_t want = (n16 + 255) / 256;
+    const unsigned grid = static_cast<unsigned>(want < 256ull * 32 ? want : 256ull * 32);
+    hipLaunchKernelGGL(copy16_kernel, dim3(grid), dim3(256), 0, s->stream, static_cast<uint4 *>(dst),
+                       static_cast<const uint4 *>(src), n16);
+    return launch_status();
+}
