@@ -250,7 +250,7 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void gemm_f32_mfma_kernel(MA
 
 // ------------------------------------------------------------------------------------ f64 ---
 // Same structure with v_mfma_f64_16x16x4_f64: lane l supplies A[l%16][l/16] and B[l/16][l%16];
-// result register r of lane l is C[4*(l/16) + r][l%16] of the 16x16 block.
+// result register r of lane l is C[4*r + l/16][l%16] of the 16x16 block.
 // LDS element = double, "vectors" are 2 doubles (16 bytes).
 
 template <int ROWS, int BK, bool KCONTIG> struct SlabD {
@@ -413,7 +413,7 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void gemm_f64_mfma_kernel(MA
             const uint32_t col = n0 + wn * WN + j * 16 + l16;
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
-                const uint32_t row = m0 + wm * WM + i * 16 + 4 * lq + r;
+                const uint32_t row = m0 + wm * WM + i * 16 + 4 * r + lq;
                 if (EDGE && (row >= g.M || col >= g.N)) continue;
                 double *p = g.C + (size_t)row * g.ldc + col;
                 double v = acc[i][j][r];
