@@ -89,6 +89,16 @@ void wk_stream_destroy(wk_stream *s);                     /* cl.command_queue.re
 int  wk_stream_sync(wk_stream *s);                        /* Pipeline.waitAndCleanup, src/core/pipeline.zig:47-61 */
 void *wk_stream_native(wk_stream *s);                     /* the hipStream_t, for event timing by the caller */
 
+/* ---- events: cl.event.* as used by src/core/pipeline.zig:35-61 (ordering itself comes from the
+ * in-order stream; events are for waiting on a point of the stream and for timing, which the
+ * reference's queue cannot do: it is created without CL_QUEUE_PROFILING_ENABLE) ------------ */
+typedef struct wk_event wk_event;
+int  wk_event_create(wk_device *dev, wk_event **out);
+void wk_event_destroy(wk_event *e);                       /* cl.event.release */
+int  wk_event_record(wk_event *e, wk_stream *s);          /* the event a cl enqueue call returns */
+int  wk_event_sync(wk_event *e);                          /* cl.event.wait */
+int  wk_event_elapsed_ms(wk_event *start, wk_event *stop, float *out_ms);
+
 /* ---- memory: cl.buffer.create/release (src/tensor/main.zig:229-234,253-263) ----------- */
 int  wk_malloc(wk_device *dev, size_t bytes, void **out_dptr);
 int  wk_free(wk_device *dev, void *dptr);

@@ -46,6 +46,11 @@ SIGNATURES = {
     "wk_stream_destroy": (None, [vp]),
     "wk_stream_sync": (ci, [vp]),
     "wk_stream_native": (vp, [vp]),
+    "wk_event_create": (ci, [vp, ctypes.POINTER(vp)]),
+    "wk_event_destroy": (None, [vp]),
+    "wk_event_record": (ci, [vp, vp]),
+    "wk_event_sync": (ci, [vp]),
+    "wk_event_elapsed_ms": (ci, [vp, vp, ctypes.POINTER(ctypes.c_float)]),
     "wk_malloc": (ci, [vp, sz, ctypes.POINTER(vp)]),
     "wk_free": (ci, [vp, vp]),
     "wk_mem_info": (ci, [vp, ctypes.POINTER(sz), ctypes.POINTER(sz)]),

@@ -18,6 +18,11 @@ struct wk_stream {
     hipStream_t stream;
 };
 
+struct wk_event {
+    wk_device *dev;
+    hipEvent_t event;
+};
+
 namespace wk {
 
 inline int hip_code(hipError_t e) {

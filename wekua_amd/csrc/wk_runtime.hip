@@ -127,6 +127,52 @@ int wk_stream_sync(wk_stream *s) {
 
 void *wk_stream_native(wk_stream *s) { return s ? static_cast<void *>(s->stream) : nullptr; }
 
+int wk_event_create(wk_device *dev, wk_event **out) {
+    if (!dev || !out) return WK_E_INVALID_VALUE;
+    *out = nullptr;
+    WK_HIP_TRY(hipSetDevice(dev->ordinal));
+    wk_event *e = new (std::nothrow) wk_event;
+    if (!e) return WK_E_OUT_OF_MEMORY;
+    e->dev = dev;
+    hipError_t rc = hipEventCreate(&e->event);
+    if (rc != hipSuccess) {
+        (void)hipGetLastError();
+        delete e;
+        return hip_code(rc);
+    }
+    *out = e;
+    return WK_OK;
+}
+
+void wk_event_destroy(wk_event *e) {
+    if (!e) return;
+    if (hipSetDevice(e->dev->ordinal) == hipSuccess) (void)hipEventDestroy(e->event);
+    (void)hipGetLastError();
+    delete e;
+}
+
+int wk_event_record(wk_event *e, wk_stream *s) {
+    int rc = bind(s);
+    if (rc) return rc;
+    if (!e) return WK_E_INVALID_VALUE;
+    WK_HIP_TRY(hipEventRecord(e->event, s->stream));
+    return WK_OK;
+}
+
+int wk_event_sync(wk_event *e) {
+    if (!e) return WK_E_INVALID_VALUE;
+    WK_HIP_TRY(hipSetDevice(e->dev->ordinal));
+    WK_HIP_TRY(hipEventSynchronize(e->event));
+    return WK_OK;
+}
+
+int wk_event_elapsed_ms(wk_event *start, wk_event *stop, float *out_ms) {
+    if (!start || !stop || !out_ms) return WK_E_INVALID_VALUE;
+    WK_HIP_TRY(hipSetDevice(start->dev->ordinal));
+    WK_HIP_TRY(hipEventElapsedTime(out_ms, start->event, stop->event));
+    return WK_OK;
+}
+
 int wk_malloc(wk_device *dev, size_t bytes, void **out_dptr) {
     if (!dev || !out_dptr || bytes == 0) return WK_E_INVALID_VALUE;
     *out_dptr = nullptr;

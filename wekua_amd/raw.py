@@ -92,6 +92,25 @@ class Device:
             self.lib.wk_device_close(self.dev)
             self.dev = None
 
+    def time_stream_ms(self, enqueue, iters: int) -> float:
+        """Average duration in ms of `iters` calls of enqueue() measured with events recorded on
+        this device's stream (the stream the kernels are launched on)."""
+        e0, e1 = ctypes.c_void_p(), ctypes.c_void_p()
+        check(self.lib.wk_event_create(self.dev, ctypes.byref(e0)), "wk_event_create")
+        check(self.lib.wk_event_create(self.dev, ctypes.byref(e1)), "wk_event_create")
+        try:
+            check(self.lib.wk_event_record(e0, self.stream), "wk_event_record")
+            for _ in range(iters):
+                enqueue()
+            check(self.lib.wk_event_record(e1, self.stream), "wk_event_record")
+            check(self.lib.wk_event_sync(e1), "wk_event_sync")
+            ms = ctypes.c_float()
+            check(self.lib.wk_event_elapsed_ms(e0, e1, ctypes.byref(ms)), "wk_event_elapsed_ms")
+        finally:
+            self.lib.wk_event_destroy(e0)
+            self.lib.wk_event_destroy(e1)
+        return ms.value / iters
+
     # -- the hot path ---------------------------------------------------------------------
     def gemm(self, dtype: str, op_a: int, op_b: int, M: int, N: int, K: int, alpha, A: "DeviceBuffer", lda: int,
              B: "DeviceBuffer", ldb: int, beta, C: "DeviceBuffer", ldc: int) -> None:
