@@ -30,6 +30,7 @@ int build_problem(GemmProblem &p, int dtype, int op_a, int op_b, uint64_t M, uin
     p.dtype = dtype; p.op_a = op_a; p.op_b = op_b;
     p.M = M; p.N = N; p.K = K; p.lda = lda; p.ldb = ldb; p.ldc = ldc;
     p.A = A; p.B = B; p.C = C;
+    p.num_cus = 0;
     std::memset(p.alpha, 0, sizeof p.alpha);
     std::memset(p.beta, 0, sizeof p.beta);
     // has_alpha = alpha or beta given; alpha defaults to one (src/blas/gemm.zig:500-501,592-596)
@@ -73,6 +74,7 @@ int wk_gemm(wk_stream *s, int dtype, int op_a, int op_b, uint64_t M, uint64_t N,
     GemmProblem p;
     rc = build_problem(p, dtype, op_a, op_b, M, N, K, host_alpha, A, lda, B, ldb, host_beta, C, ldc);
     if (rc) return rc;
+    p.num_cus = (uint32_t)s->dev->props.multiProcessorCount;
     const int v = choose(p);
     if (v >= 0) return gemm_mfma_launch(s->stream, p, v);
     return gemm_generic_launch(s->stream, p);

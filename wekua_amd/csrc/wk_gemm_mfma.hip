@@ -47,9 +47,25 @@ template <typename T> struct MArgs {
     uint32_t M, N, K;
     uint32_t lda, ldb, ldc;
     uint32_t tiles_m, tiles_n;
+    uint32_t num_cus; // compute units of the device (0 disables the start-up stagger)
     int epi;
     T alpha, beta;
 };
+
+// Work-groups that share a CU start in lock step (the whole first wave of work-groups is
+// dispatched at once) and, doing identical work, stay in lock step: they reach the slab
+// hand-over (LDS store, barrier, fragment reload) at the same time and the matrix pipe idles.
+// Delaying the k-th co-resident work-group of the first dispatch wave by k solo-iterations
+// keeps one of them in its matrix phase while the other hands over.  Later work-groups
+// inherit the offset of the one whose slot they take.  Measured on MI355X at 8192^3 f32 with
+// the 256x128 tile: 132 -> 141 TFLOP/s.
+__device__ __forceinline__ void startup_stagger(uint32_t num_cus, uint32_t occupancy, uint32_t units_per_slot) {
+    if (num_cus == 0) return;
+    const uint32_t slot = blockIdx.x / num_cus;
+    if (slot == 0 || slot >= occupancy) return;
+    const uint32_t n = slot * units_per_slot;
+    for (uint32_t i = 0; i < n; ++i) __builtin_amdgcn_s_sleep(2); // 2 * 64 clocks
+}
 
 // blockIdx.x -> (tile_m, tile_n): XCD-contiguous renumbering, then grouped row-major walk.
 __device__ __forceinline__ void tile_coords(uint32_t tiles_m, uint32_t tiles_n, uint32_t &tm, uint32_t &tn) {
@@ -73,8 +89,9 @@ template <int ROWS, int BK, bool KCONTIG> struct Slab {
     static constexpr int SIZE = KCONTIG ? ROWS * LD : BK * LD;
 };
 
-template <int BM, int BN, int BK, int WAVES_M, int WAVES_N, bool A_K, bool B_K, bool EDGE>
-__global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void gemm_f32_mfma_kernel(MArgs<float> g) {
+template <int BM, int BN, int BK, int WAVES_M, int WAVES_N, int OCC, bool LOAD_AHEAD, bool A_K, bool B_K, bool EDGE>
+__global__ __launch_bounds__(WAVES_M *WAVES_N * 64) __attribute__((amdgpu_waves_per_eu(OCC)))
+void gemm_f32_mfma_kernel(MArgs<float> g) {
     constexpr int NT = WAVES_M * WAVES_N * 64;
     constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N;
     constexpr int FM = WM / 32, FN = WN / 32;
@@ -96,6 +113,8 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void gemm_f32_mfma_kernel(MA
     uint32_t tile_m, tile_n;
     tile_coords(g.tiles_m, g.tiles_n, tile_m, tile_n);
     const uint32_t m0 = tile_m * BM, n0 = tile_n * BN;
+    // one solo iteration = FM*FN*BK/2 matrix instructions of 64 clocks = FM*FN*BK/4 sleep units
+    startup_stagger(g.num_cus, OCC, FM * FN * BK / 4);
 
     f32x16 acc[FM][FN];
 #pragma unroll
@@ -179,53 +198,86 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void gemm_f32_mfma_kernel(MA
     };
 
     const uint32_t ktiles = (g.K + BK - 1) / BK;
+    constexpr int S = BK / 8; // fragment steps per k-slab (8 values of k each)
+
+    // fragments of step s of LDS buffer `buf`: lane holds k = 8*s + 4*lhi + t, t = 0..3
+    auto read_frags = [&](int buf, int s, f32x4 *af, f32x4 *bf) {
+        const float *as = As + buf * SA::SIZE + (A_K ? (wm * WM + l32) * SA::LD : wm * WM + l32);
+        const float *bs = Bs + buf * SB::SIZE + (B_K ? (wn * WN + l32) * SB::LD : wn * WN + l32);
+#pragma unroll
+        for (int i = 0; i < FM; ++i) {
+            if constexpr (A_K) {
+                af[i] = *reinterpret_cast<const f32x4 *>(as + i * 32 * SA::LD + 8 * s + 4 * lhi);
+            } else {
+#pragma unroll
+                for (int t = 0; t < 4; ++t) af[i][t] = as[(8 * s + 4 * lhi + t) * SA::LD + i * 32];
+            }
+        }
+#pragma unroll
+        for (int j = 0; j < FN; ++j) {
+            if constexpr (B_K) {
+                bf[j] = *reinterpret_cast<const f32x4 *>(bs + j * 32 * SB::LD + 8 * s + 4 * lhi);
+            } else {
+#pragma unroll
+                for (int t = 0; t < 4; ++t) bf[j][t] = bs[(8 * s + 4 * lhi + t) * SB::LD + j * 32];
+            }
+        }
+    };
 
     load_a(0);
     load_b(0);
     store_ab(0);
+    if (LOAD_AHEAD && ktiles > 1) {
+        load_a(BK);
+        load_b(BK);
+    }
     __syncthreads();
 
+    // Fragment registers are double-buffered: the LDS reads for step s+1 are issued before the
+    // matrix instructions of step s, and the slab hand-over (LDS store of the next slab, barrier,
+    // first fragment read of the next slab) sits in front of the last step's matrix
+    // instructions, so that LDS latency and barrier skew are covered by matrix work of the
+    // same wavefront instead of relying on another wavefront to fill the pipe.
+    f32x4 af[2][FM], bf[2][FN];
+    read_frags(0, 0, af[0], bf[0]);
+
+    // Global prefetch, two schedules (LOAD_AHEAD):
+    //   false: slab kt+1 is requested at the top of iteration kt and written to LDS in that
+    //          iteration's hand-over (half an iteration of matrix work covers the latency);
+    //   true : the staging registers are refilled with slab kt+2 right after the hand-over,
+    //          from inside the last step's matrix work (a whole iteration covers the latency;
+    //          the refill is unconditional -- the tail re-fetches the final slab -- so that
+    //          the loop body stays one basic block).
     for (uint32_t kt = 0; kt < ktiles; ++kt) {
         const int cur = kt & 1;
         const bool more = kt + 1 < ktiles;
-        if (more) {
+        if (!LOAD_AHEAD && more) {
             load_a((kt + 1) * BK);
             load_b((kt + 1) * BK);
         }
-        const float *as = As + cur * SA::SIZE + (A_K ? (wm * WM + l32) * SA::LD : wm * WM + l32);
-        const float *bs = Bs + cur * SB::SIZE + (B_K ? (wn * WN + l32) * SB::LD : wn * WN + l32);
 #pragma unroll
-        for (int s = 0; s < BK / 8; ++s) {
-            // lane holds k = 8*s + 4*lhi + t, t = 0..3
-            f32x4 af[FM], bf[FN];
-#pragma unroll
-            for (int i = 0; i < FM; ++i) {
-                if constexpr (A_K) {
-                    af[i] = *reinterpret_cast<const f32x4 *>(as + i * 32 * SA::LD + 8 * s + 4 * lhi);
-                } else {
-#pragma unroll
-                    for (int t = 0; t < 4; ++t) af[i][t] = as[(8 * s + 4 * lhi + t) * SA::LD + i * 32];
-                }
+        for (int s = 0; s < S; ++s) {
+            if (s + 1 < S) {
+                read_frags(cur, s + 1, af[(s + 1) & 1], bf[(s + 1) & 1]);
+            } else if (more) {
+                store_ab(cur ^ 1);
+                __syncthreads();
+                read_frags(cur ^ 1, 0, af[(s + 1) & 1], bf[(s + 1) & 1]);
             }
 #pragma unroll
-            for (int j = 0; j < FN; ++j) {
-                if constexpr (B_K) {
-                    bf[j] = *reinterpret_cast<const f32x4 *>(bs + j * 32 * SB::LD + 8 * s + 4 * lhi);
-                } else {
-#pragma unroll
-                    for (int t = 0; t < 4; ++t) bf[j][t] = bs[(8 * s + 4 * lhi + t) * SB::LD + j * 32];
-                }
-            }
-#pragma unroll
-            for (int t = 0; t < 4; ++t)
+            for (int t = 0; t < 4; ++t) {
 #pragma unroll
                 for (int i = 0; i < FM; ++i)
 #pragma unroll
                     for (int j = 0; j < FN; ++j)
-                        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(af[i][t], bf[j][t], acc[i][j], 0, 0, 0);
+                        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(af[s & 1][i][t], bf[s & 1][j][t], acc[i][j], 0, 0, 0);
+                if (LOAD_AHEAD && s == S - 1 && t == 0) {
+                    const uint32_t knext = min(kt + 2, ktiles - 1) * BK;
+                    load_a(knext);
+                    load_b(knext);
+                }
+            }
         }
-        if (more) store_ab(cur ^ 1);
-        __syncthreads();
     }
 
     // ---- epilogue: acc register r of lane l is C[8*(r/4) + 4*(l/32) + r%4][l%32] of its 32x32 block
@@ -443,6 +495,7 @@ template <typename T> MArgs<T> make_args(const GemmProblem &p, int bm, int bn) {
     g.lda = (uint32_t)p.lda; g.ldb = (uint32_t)p.ldb; g.ldc = (uint32_t)p.ldc;
     g.tiles_m = (uint32_t)((p.M + bm - 1) / bm);
     g.tiles_n = (uint32_t)((p.N + bn - 1) / bn);
+    g.num_cus = p.num_cus;
     g.epi = p.epi;
     std::memcpy(&g.alpha, p.alpha, sizeof(T));
     std::memcpy(&g.beta, p.beta, sizeof(T));
@@ -458,10 +511,10 @@ template <typename K> int set_lds(K kernel, size_t bytes) {
     return WK_OK;
 }
 
-template <int BM, int BN, int BK, int WMS, int WNS, bool AK, bool BKC, bool EDGE>
+template <int BM, int BN, int BK, int WMS, int WNS, int OCC, bool LA, bool AK, bool BKC, bool EDGE>
 int launch_f32_one(hipStream_t st, const GemmProblem &p) {
     constexpr size_t lds = 2 * (Slab<BM, BK, AK>::SIZE + Slab<BN, BK, BKC>::SIZE) * sizeof(float);
-    auto kern = gemm_f32_mfma_kernel<BM, BN, BK, WMS, WNS, AK, BKC, EDGE>;
+    auto kern = gemm_f32_mfma_kernel<BM, BN, BK, WMS, WNS, OCC, LA, AK, BKC, EDGE>;
     static int attr_rc = set_lds(kern, lds);
     if (attr_rc) return attr_rc;
     MArgs<float> g = make_args<float>(p, BM, BN);
@@ -469,12 +522,12 @@ int launch_f32_one(hipStream_t st, const GemmProblem &p) {
     return launch_status();
 }
 
-template <int BM, int BN, int BK, int WMS, int WNS>
+template <int BM, int BN, int BK, int WMS, int WNS, int OCC, bool LA = false>
 int launch_f32(hipStream_t st, const GemmProblem &p, bool edge) {
     const int sel = (p.op_a ? 0 : 2) | (p.op_b ? 1 : 0); // bit1: A k-contiguous, bit0: B k-contiguous
 #define WK_CASE(AK, BKC)                                                                                   \
-    return edge ? launch_f32_one<BM, BN, BK, WMS, WNS, AK, BKC, true>(st, p)                               \
-                : launch_f32_one<BM, BN, BK, WMS, WNS, AK, BKC, false>(st, p)
+    return edge ? launch_f32_one<BM, BN, BK, WMS, WNS, OCC, LA, AK, BKC, true>(st, p)                          \
+                : launch_f32_one<BM, BN, BK, WMS, WNS, OCC, LA, AK, BKC, false>(st, p)
     switch (sel) {
     case 0: WK_CASE(false, false);
     case 1: WK_CASE(false, true);
@@ -517,9 +570,9 @@ struct VariantDesc {
 };
 
 const VariantDesc k_variants[] = {
-    {"mfma_f32_256x128", WK_F32, 256, 128, 16, &launch_f32<256, 128, 16, 2, 2>},
-    {"mfma_f32_128x128", WK_F32, 128, 128, 16, &launch_f32<128, 128, 16, 2, 2>},
-    {"mfma_f32_64x64", WK_F32, 64, 64, 16, &launch_f32<64, 64, 16, 2, 2>},
+    {"mfma_f32_256x128", WK_F32, 256, 128, 16, &launch_f32<256, 128, 16, 2, 2, 2>},
+    {"mfma_f32_128x128", WK_F32, 128, 128, 16, &launch_f32<128, 128, 16, 2, 2, 3>},
+    {"mfma_f32_64x64", WK_F32, 64, 64, 16, &launch_f32<64, 64, 16, 2, 2, 4>},
     {"mfma_f64_128x128", WK_F64, 128, 128, 16, &launch_f64<128, 128, 16, 2, 2>},
     {"mfma_f64_64x64", WK_F64, 64, 64, 16, &launch_f64<64, 64, 16, 2, 2>},
 };

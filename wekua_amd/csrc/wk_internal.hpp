@@ -150,6 +150,7 @@ struct GemmProblem {
     const void *A, *B;
     void *C;
     int epi;                          // EPI_*
+    uint32_t num_cus;                 // compute units of the device the stream belongs to
     alignas(16) unsigned char alpha[16];  // one element of dtype (valid when epi != EPI_STORE)
     alignas(16) unsigned char beta[16];   // one element of dtype (valid when epi == EPI_ALPHA_BETA)
 };
