@@ -1,0 +1,108 @@
+"""CPU: the C-ABI library loads and exports every symbol include/wekua_hip.h declares; the
+Python binding declares a signature for each; host-only entry points behave; and without a GPU
+the product path fails loudly instead of falling back to anything."""
+import ctypes
+import os
+import re
+import subprocess
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = os.path.join(ROOT, "include", "wekua_hip.h")
+
+
+def declared_functions():
+    text = open(HEADER).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(wk_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_header_declares_the_hot_path():
+    names = declared_functions()
+    for must in ("wk_gemm", "wk_axpy", "wk_device_open", "wk_stream_create", "wk_malloc", "wk_copy_h2d_rect_async",
+                 "wk_copy_d2h_rect_async", "wk_fill", "wk_identity", "wk_stream_sync", "wk_strerror"):
+        assert must in names
+
+
+def test_library_exports_every_declared_symbol():
+    from wekua_amd import _capi
+    lib = _capi.load()
+    missing = [n for n in declared_functions() if not hasattr(lib, n)]
+    assert not missing, f"declared in wekua_hip.h but not exported: {missing}"
+
+
+def test_binding_covers_every_declared_symbol():
+    from wekua_amd import _capi
+    declared = set(declared_functions())
+    bound = set(_capi.SIGNATURES)
+    assert declared == bound, f"unbound: {declared - bound}; undeclared: {bound - declared}"
+
+
+def test_header_compiles_as_plain_c():
+    """The boundary is a C ABI: the header must be valid C, not only C++."""
+    src = '#include "wekua_hip.h"\nint main(void){ return wk_gemm == 0; }\n'
+    res = subprocess.run(["gcc", "-std=c99", "-Wall", "-Werror", "-fsyntax-only", "-I", os.path.join(ROOT, "include"),
+                          "-x", "c", "-"], input=src, text=True, capture_output=True)
+    assert res.returncode == 0, res.stderr
+
+
+def test_host_only_entry_points():
+    from wekua_amd import _capi
+    lib = _capi.load()
+    assert lib.wk_abi_version() == 1
+    sizes = [lib.wk_dtype_size(i) for i in range(20)]
+    assert sizes == [1, 1, 2, 2, 4, 4, 8, 8, 4, 8, 2, 2, 4, 4, 8, 8, 16, 16, 8, 16]
+    assert lib.wk_dtype_size(20) == 0 and lib.wk_dtype_size(-1) == 0
+    # error names are the reference's Zig error names (src/tensor/main.zig:25-33)
+    names = {1: "InvalidValue", 2: "InvalidCoordinates", 3: "InvalidBuffer", 4: "UnqualTensorsAttribute",
+             5: "UnqualTensorsShape", 6: "UnqualTensorsDimension", 7: "UnqualTensorsContext", 8: "OutOfMemory",
+             9: "TypeNotSupported", 10: "DevicesArrayEmpty"}
+    for code, name in names.items():
+        assert lib.wk_strerror(code).decode() == name
+    assert lib.wk_gemm_workspace_bytes(8, 0, 0, 8192, 8192, 8192) == 0
+    assert lib.wk_gemm_force_variant(b"no-such-kernel") == 1
+    assert lib.wk_gemm_force_variant(b"auto") == 0
+    # kernel selection is host logic: f32/f64 go to the matrix cores, everything else to the tile kernel
+    v = lambda dt, n: lib.wk_gemm_variant(dt, 0, 0, n, n, n, n, n, n, None, None, None).decode()
+    assert v(8, 8192).startswith("mfma_f32")
+    assert v(9, 4096).startswith("mfma_f64")
+    assert v(4, 2048) == "tile64"
+    assert v(18, 512) == "tile64"
+    assert lib.wk_gemm_variant(8, 0, 0, 0, 4, 4, 4, 4, 4, None, None, None).decode() == "invalid"
+
+
+def _gpu_present():
+    from wekua_amd import _capi
+    n = ctypes.c_int(-1)
+    assert _capi.load().wk_device_count(ctypes.byref(n)) == 0
+    return n.value > 0
+
+
+def test_no_gpu_means_loud_failure_not_fallback():
+    """Without a device the product path raises DevicesArrayEmpty (src/core/context.zig:18); it
+    never computes on the host."""
+    if _gpu_present():
+        pytest.skip("a GPU is present")
+    import wekua_amd
+    with pytest.raises(wekua_amd.WekuaError) as e:
+        wekua_amd.Context.initFromDeviceType(wekua_amd.DeviceType.all)
+    assert e.value.name == "DevicesArrayEmpty"
+    from wekua_amd import raw
+    with pytest.raises(wekua_amd.WekuaError):
+        raw.Device(0)
+
+
+def test_product_package_never_touches_the_oracle():
+    """The GPU package must not import, load or link anything under oracle/."""
+    pkg = os.path.join(ROOT, "wekua_amd")
+    for dirpath, _dirs, files in os.walk(pkg):
+        if os.path.basename(dirpath) in ("build", "__pycache__"):
+            continue
+        for f in files:
+            if f.endswith((".py", ".hip", ".hpp", ".cpp", ".h")):
+                text = open(os.path.join(dirpath, f)).read()
+                assert "wk_oracle" not in text and "import oracle" not in text and "from oracle" not in text, f
+    for so in ("libwekua_hip.so", "libwekua_host.so"):
+        out = subprocess.run(["ldd", os.path.join(pkg, so)], capture_output=True, text=True).stdout
+        assert "oracle" not in out

@@ -1,0 +1,340 @@
+"""wekua_amd -- wekua's BLAS hot path (blas.gemm, blas.axpy) on AMD Instinct MI355X.
+
+Layers, bottom up:
+
+* ``libwekua_hip.so``  -- hand-written HIP kernels for gfx950 behind the C ABI of
+  ``include/wekua_hip.h`` (``wekua_amd/csrc``).
+* ``libwekua_host.so`` -- the host side of the reference's API (Context, Pipeline, Tensor,
+  blas.gemm / blas.axpy / GemmPackedTensors, memory, fill, identity) as C++ templates
+  (``wekua_amd/host/wekua.hpp``) with flat C entry points for this binding.
+* this module -- a thin Python binding of those entry points that keeps the reference's names
+  and argument order, so that tests read like the reference's own Zig tests:
+
+      ctx = Context.initFromDeviceType(DeviceType.all)
+      pipeline = Pipeline.init(ctx.command_queues[0])
+      a = Tensor.alloc("f32", ctx, pipeline, (m, k))
+      memory.readFromBuffer(pipeline, a, host_array)
+      blas.gemm(pipeline, alpha, a, blas.Operation.no_transpose, b, blas.Operation.transpose, beta, c, None)
+      memory.writeToBuffer(pipeline, c, out); pipeline.waitAndCleanup()
+
+Zig errors surface as ``WekuaError`` whose ``.name`` is the Zig error name
+(``InvalidValue``, ``UnqualTensorsShape``, ...).  There is no CPU fallback anywhere: a
+missing native library raises at import of the symbol that needs it.
+"""
+from __future__ import annotations
+
+import ctypes
+import enum
+import os
+
+import numpy as np
+
+from . import _capi
+from ._capi import WkError as WekuaError  # noqa: F401  (re-export)
+from .raw import DTYPE_NAMES, dtype_id, elem_size, is_complex, real_np_dtype, scalar_bytes
+
+_PKG = os.path.dirname(os.path.abspath(__file__))
+HOST_LIB_PATH = os.path.join(_PKG, "libwekua_host.so")
+
+u64, vp, ci = ctypes.c_uint64, ctypes.c_void_p, ctypes.c_int
+u64p = ctypes.POINTER(u64)
+
+
+class _TensorInfo(ctypes.Structure):
+    _fields_ = [
+        ("dtype", ci), ("ndim", ci), ("shape", u64 * 8), ("pitches", u64 * 8),
+        ("number_of_elements", u64), ("number_of_elements_without_padding", u64),
+        ("row_pitch", u64), ("row_pitch_for_vectors", u64), ("slice_pitch", u64),
+        ("slice_pitch_for_vectors", u64), ("number_of_vectors", u64), ("size", u64),
+        ("vectors_enabled", ci), ("gemm_algorithm", ci), ("buffer", vp),
+    ]
+
+
+HOST_SIGNATURES = {
+    "wkz_context_init_from_device_type": (ci, [ci, ctypes.POINTER(vp)]),
+    "wkz_context_init_from_best_device": (ci, [ci, ctypes.POINTER(vp)]),
+    "wkz_context_init": (ci, [ci, ctypes.POINTER(vp)]),
+    "wkz_context_deinit": (None, [vp]),
+    "wkz_context_num_queues": (ci, [vp]),
+    "wkz_context_stream": (vp, [vp, ci]),
+    "wkz_context_device": (vp, [vp]),
+    "wkz_pipeline_init": (ci, [vp, ci, ctypes.POINTER(vp)]),
+    "wkz_pipeline_deinit": (None, [vp]),
+    "wkz_pipeline_prealloc": (ci, [vp, u64]),
+    "wkz_pipeline_wait_and_cleanup": (ci, [vp]),
+    "wkz_pipeline_pending": (u64, [vp]),
+    "wkz_pipeline_prev_events": (u64, [vp]),
+    "wkz_pipeline_clear": (None, [vp]),
+    "wkz_tensor_alloc": (ci, [vp, vp, ci, u64p, ci, ci, ctypes.POINTER(vp)]),
+    "wkz_tensor_empty": (ci, [vp, vp, ci, u64p, ci, ci, ctypes.POINTER(vp)]),
+    "wkz_tensor_release": (ci, [vp, vp]),
+    "wkz_tensor_get_info": (ci, [vp, ctypes.POINTER(_TensorInfo)]),
+    "wkz_read_from_buffer": (ci, [vp, vp, vp, u64]),
+    "wkz_write_to_buffer": (ci, [vp, vp, vp, u64]),
+    "wkz_fill_zeroes": (ci, [vp, vp]),
+    "wkz_fill_one": (ci, [vp, vp]),
+    "wkz_fill_constant": (ci, [vp, vp, vp]),
+    "wkz_identity": (ci, [vp, vp]),
+    "wkz_axpy": (ci, [vp, vp, vp, vp]),
+    "wkz_packed_init": (ci, [vp, vp, u64, ci, ctypes.POINTER(vp)]),
+    "wkz_packed_init_with_dimensions": (ci, [vp, ci, u64, u64, u64, ci, ci, ctypes.POINTER(vp)]),
+    "wkz_packed_deinit": (ci, [vp, vp]),
+    "wkz_packed_pack": (ci, [vp, vp, vp, ci, vp, ci]),
+    "wkz_gemm": (ci, [vp, vp, vp, ci, vp, ci, vp, vp, vp]),
+}
+
+_host = None
+
+
+def _lib():
+    global _host
+    if _host is None:
+        _capi.load()  # libwekua_hip.so first (RTLD_GLOBAL): the host library links against it
+        if not os.path.exists(HOST_LIB_PATH):
+            raise ImportError(f"{HOST_LIB_PATH} is missing: build it with `python -m wekua_amd.build`")
+        lib = ctypes.CDLL(HOST_LIB_PATH)
+        for name, (res, args) in HOST_SIGNATURES.items():
+            fn = getattr(lib, name)
+            fn.restype = res
+            fn.argtypes = args
+        _host = lib
+    return _host
+
+
+def _check(code: int, where: str) -> None:
+    if code != 0:
+        raise WekuaError(code, where)
+
+
+def _scalar_ptr(dtype: str, value):
+    buf = scalar_bytes(dtype, value)
+    return buf, (ctypes.cast(buf, vp) if buf is not None else None)
+
+
+class DeviceType(enum.IntEnum):
+    cpu = 0
+    gpu = 1
+    all = 2
+
+
+class CommandQueue:
+    def __init__(self, context: "Context", index: int):
+        self.context = context
+        self.wekua_id = index
+
+    def isTypeSupported(self, dtype: str) -> bool:
+        return dtype in DTYPE_NAMES
+
+
+class Context:
+    """core.Context (src/core/context.zig): one HIP device, one in-order queue."""
+
+    def __init__(self, handle):
+        self._h = handle
+        n = _lib().wkz_context_num_queues(handle)
+        self.command_queues = [CommandQueue(self, i) for i in range(n)]
+
+    @classmethod
+    def initFromDeviceType(cls, device_type: DeviceType = DeviceType.all) -> "Context":
+        h = vp()
+        _check(_lib().wkz_context_init_from_device_type(int(device_type), ctypes.byref(h)), "Context.initFromDeviceType")
+        return cls(h)
+
+    @classmethod
+    def initFromBestDevice(cls, device_type: DeviceType = DeviceType.gpu) -> "Context":
+        h = vp()
+        _check(_lib().wkz_context_init_from_best_device(int(device_type), ctypes.byref(h)), "Context.initFromBestDevice")
+        return cls(h)
+
+    @classmethod
+    def init(cls, ordinal: int = 0) -> "Context":
+        h = vp()
+        _check(_lib().wkz_context_init(ordinal, ctypes.byref(h)), "Context.init")
+        return cls(h)
+
+    def deinit(self) -> None:
+        if self._h:
+            _lib().wkz_context_deinit(self._h)
+            self._h = None
+
+
+class Pipeline:
+    """core.Pipeline (src/core/pipeline.zig)."""
+
+    def __init__(self, handle, command_queue: CommandQueue):
+        self._h = handle
+        self.command_queue = command_queue
+
+    @classmethod
+    def init(cls, command_queue: CommandQueue) -> "Pipeline":
+        h = vp()
+        _check(_lib().wkz_pipeline_init(command_queue.context._h, command_queue.wekua_id, ctypes.byref(h)), "Pipeline.init")
+        return cls(h, command_queue)
+
+    def deinit(self) -> None:
+        if self._h:
+            _lib().wkz_pipeline_deinit(self._h)
+            self._h = None
+
+    def prealloc(self, capacity: int) -> None:
+        _check(_lib().wkz_pipeline_prealloc(self._h, capacity), "Pipeline.prealloc")
+
+    def waitAndCleanup(self) -> None:
+        _check(_lib().wkz_pipeline_wait_and_cleanup(self._h), "Pipeline.waitAndCleanup")
+        self._keepalive = []
+
+    def pending(self) -> int:
+        return int(_lib().wkz_pipeline_pending(self._h))
+
+    def prevEvents(self) -> int:
+        """Number of events in the last appended batch (0 when nothing is pending)."""
+        return int(_lib().wkz_pipeline_prev_events(self._h))
+
+    def clear(self) -> None:
+        _lib().wkz_pipeline_clear(self._h)
+
+
+class Tensor:
+    """Tensor(T) (src/tensor/main.zig): `dtype` plays the role of the comptime type."""
+
+    def __init__(self, handle, dtype: str, context: Context):
+        self._h = handle
+        self.dtype = dtype
+        self.context = context
+        info = _TensorInfo()
+        _check(_lib().wkz_tensor_get_info(handle, ctypes.byref(info)), "Tensor info")
+        nd = info.ndim
+        self.shape = tuple(int(info.shape[i]) for i in range(nd))
+        self.pitches = tuple(int(info.pitches[i]) for i in range(nd))
+        self.number_of_elements = int(info.number_of_elements)
+        self.number_of_elements_without_padding = int(info.number_of_elements_without_padding)
+        self.row_pitch = int(info.row_pitch)
+        self.row_pitch_for_vectors = int(info.row_pitch_for_vectors)
+        self.slice_pitch = int(info.slice_pitch)
+        self.slice_pitch_for_vectors = int(info.slice_pitch_for_vectors)
+        self.number_of_vectors = int(info.number_of_vectors)
+        self.size = int(info.size)
+        self.vectors_enabled = bool(info.vectors_enabled)
+        self.gemm_algorithm = int(info.gemm_algorithm)
+        self.buffer = info.buffer
+
+    @classmethod
+    def _create(cls, fn, dtype, context, pipeline, shape, vectors_enabled):
+        arr = (u64 * max(len(shape), 1))(*shape)
+        h = vp()
+        _check(fn(context._h, pipeline._h, dtype_id(dtype), arr, len(shape), int(vectors_enabled), ctypes.byref(h)),
+               "Tensor.alloc")
+        return cls(h, dtype, context)
+
+    @classmethod
+    def alloc(cls, dtype: str, context: Context, pipeline: Pipeline, shape, vectors_enabled: bool = True) -> "Tensor":
+        return cls._create(_lib().wkz_tensor_alloc, dtype, context, pipeline, tuple(shape), vectors_enabled)
+
+    @classmethod
+    def empty(cls, dtype: str, context: Context, pipeline: Pipeline, shape, vectors_enabled: bool = True) -> "Tensor":
+        return cls._create(_lib().wkz_tensor_empty, dtype, context, pipeline, tuple(shape), vectors_enabled)
+
+    def release(self, pipeline: Pipeline) -> None:
+        if self._h:
+            _check(_lib().wkz_tensor_release(self._h, pipeline._h), "Tensor.release")
+            self._h = None
+
+    def host_shape(self):
+        return self.shape + ((2,) if is_complex(self.dtype) else ())
+
+
+class memory:
+    @staticmethod
+    def readFromBuffer(pipeline: Pipeline, tensor: Tensor, buffer: np.ndarray) -> None:
+        """HOST -> DEVICE; `buffer` holds exactly the logical elements (complex: trailing (re, im) axis)."""
+        buffer = np.ascontiguousarray(buffer, dtype=real_np_dtype(tensor.dtype))
+        n = buffer.size // (2 if is_complex(tensor.dtype) else 1)
+        _check(_lib().wkz_read_from_buffer(pipeline._h, tensor._h, buffer.ctypes.data, n), "memory.readFromBuffer")
+        pipeline._keepalive = getattr(pipeline, "_keepalive", []) + [buffer]
+
+    @staticmethod
+    def writeToBuffer(pipeline: Pipeline, tensor: Tensor, buffer: np.ndarray) -> None:
+        """DEVICE -> HOST into a C-contiguous array of the tensor's dtype."""
+        if buffer.dtype != real_np_dtype(tensor.dtype) or not buffer.flags.c_contiguous:
+            raise TypeError("writeToBuffer needs a C-contiguous array of the tensor's dtype")
+        n = buffer.size // (2 if is_complex(tensor.dtype) else 1)
+        _check(_lib().wkz_write_to_buffer(pipeline._h, tensor._h, buffer.ctypes.data, n), "memory.writeToBuffer")
+
+
+class fill:
+    @staticmethod
+    def zeroes(pipeline: Pipeline, tensor: Tensor) -> None:
+        _check(_lib().wkz_fill_zeroes(pipeline._h, tensor._h), "fill.zeroes")
+
+    @staticmethod
+    def one(pipeline: Pipeline, tensor: Tensor) -> None:
+        _check(_lib().wkz_fill_one(pipeline._h, tensor._h), "fill.one")
+
+    @staticmethod
+    def constant(pipeline: Pipeline, tensor: Tensor, value) -> None:
+        _keep, p = _scalar_ptr(tensor.dtype, value)
+        _check(_lib().wkz_fill_constant(pipeline._h, tensor._h, p), "fill.constant")
+
+
+def identity(pipeline: Pipeline, tensor: Tensor) -> None:
+    _check(_lib().wkz_identity(pipeline._h, tensor._h), "identity")
+
+
+class GemmPackedTensors:
+    """blas.GemmPackedTensors (src/blas/gemm.zig:60-359).  Holds no device memory here."""
+
+    def __init__(self, handle, dtype):
+        self._h = handle
+        self.dtype = dtype
+
+    @classmethod
+    def init(cls, pipeline: Pipeline, result_tensor: Tensor, k_size: int, vectors_enabled: bool) -> "GemmPackedTensors":
+        h = vp()
+        _check(_lib().wkz_packed_init(pipeline._h, result_tensor._h, k_size, int(vectors_enabled), ctypes.byref(h)),
+               "GemmPackedTensors.init")
+        return cls(h, result_tensor.dtype)
+
+    @classmethod
+    def initWithDimensions(cls, pipeline: Pipeline, dtype: str, n_size: int, m_size: int, k_size: int,
+                           recommended_algorithm: int, vectors_enabled: bool) -> "GemmPackedTensors":
+        h = vp()
+        _check(_lib().wkz_packed_init_with_dimensions(pipeline._h, dtype_id(dtype), n_size, m_size, k_size,
+                                                      recommended_algorithm, int(vectors_enabled), ctypes.byref(h)),
+               "GemmPackedTensors.initWithDimensions")
+        return cls(h, dtype)
+
+    def deinit(self, pipeline: Pipeline) -> None:
+        if self._h:
+            _check(_lib().wkz_packed_deinit(self._h, pipeline._h), "GemmPackedTensors.deinit")
+            self._h = None
+
+    def pack(self, pipeline: Pipeline, a: Tensor, op_a: int, b: Tensor, op_b: int) -> None:
+        _check(_lib().wkz_packed_pack(self._h, pipeline._h, a._h, int(op_a), b._h, int(op_b)), "GemmPackedTensors.pack")
+
+
+class blas:
+    class Operation(enum.IntEnum):
+        no_transpose = 0
+        transpose = 1
+
+    GemmOperation = Operation
+    GemmPackedTensors = GemmPackedTensors
+
+    @staticmethod
+    def axpy(pipeline: Pipeline, x: Tensor, alpha, y: Tensor) -> None:
+        """blas.axpy(T, pipeline, x, alpha, y): y = alpha*x + y (alpha None: y += x)."""
+        _keep, p = _scalar_ptr(x.dtype, alpha)
+        _check(_lib().wkz_axpy(pipeline._h, x._h, p, y._h), "blas.axpy")
+
+    @staticmethod
+    def gemm(pipeline: Pipeline, alpha, a: Tensor, op_a: int, b: Tensor, op_b: int, beta, c: Tensor,
+             packed_tensors: "GemmPackedTensors | None" = None) -> None:
+        """blas.gemm(T, pipeline, alpha, a, op_a, b, op_b, beta, c, packed_tensors)."""
+        _ka, pa = _scalar_ptr(c.dtype, alpha)
+        _kb, pb = _scalar_ptr(c.dtype, beta)
+        _check(_lib().wkz_gemm(pipeline._h, pa, a._h, int(op_a), b._h, int(op_b), pb, c._h,
+                               packed_tensors._h if packed_tensors is not None else None), "blas.gemm")
+
+
+__all__ = ["Context", "Pipeline", "Tensor", "CommandQueue", "DeviceType", "memory", "fill", "identity", "blas",
+           "GemmPackedTensors", "WekuaError", "DTYPE_NAMES", "dtype_id", "elem_size", "is_complex", "real_np_dtype"]

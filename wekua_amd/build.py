@@ -59,7 +59,7 @@ def build_host(verbose: bool = False) -> str:
     src = os.path.join(HOST, "wekua_c.cpp")
     if not os.path.exists(src):
         return ""
-    cmd = ["g++", "-O2", "-std=c++17", "-fPIC", "-shared", "-Wall", "-Wextra", "-I" + INCLUDE, "-I" + HOST,
+    cmd = ["g++", "-O2", "-std=c++20", "-fPIC", "-shared", "-Wall", "-Wextra", "-I" + INCLUDE, "-I" + HOST,
            src, "-o", LIB_HOST, "-L" + PKG, "-lwekua_hip", "-Wl,-rpath,$ORIGIN"]
     out = _run(cmd)
     if verbose and out.strip():

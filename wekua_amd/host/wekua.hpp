@@ -1,0 +1,496 @@
+// wekua.hpp -- host-side mirror of wekua's public API for the BLAS hot path, on top of the
+// C ABI of libwekua_hip (include/wekua_hip.h).
+//
+// The reference's host layer is Zig generics over OpenCL.  No Zig toolchain is available to
+// this build, so the same surface is written as C++ templates with the reference's names,
+// parameter order and error behaviour, one for one:
+//
+//   wekua::core::Context        src/core/context.zig:13-196
+//   wekua::core::CommandQueue   src/core/command_queue.zig:10-229
+//   wekua::core::Pipeline       src/core/pipeline.zig:6-66
+//   wekua::core::types          src/core/types.zig:1-115
+//   wekua::Tensor<T>            src/tensor/main.zig:62-279
+//   wekua::memory::*            src/tensor/memory/{read_from_buffer,write_to_buffer}.zig
+//   wekua::fill::*, identity    src/tensor/fill.zig:16-95, identity.zig:16-70
+//   wekua::blas::axpy           src/blas/axpy.zig:93-169
+//   wekua::blas::gemm           src/blas/gemm.zig:834-874 (validateTensors :442-485)
+//   wekua::blas::PackedTensors  src/blas/gemm.zig:60-359
+//
+// Zig error unions become exceptions of type wekua::Error carrying the WK_E_* code whose
+// name is the Zig error name; Zig optionals (`?T`) become std::optional<T>.
+//
+// What differs on purpose (MI355X-first):
+//   * a Context owns one HIP device; its single CommandQueue is an in-order HIP stream;
+//   * a Pipeline orders work by the stream, so its "events" are tickets kept only for the
+//     prevEvents()/append() bookkeeping callers rely on; waitAndCleanup() syncs the stream;
+//   * Tensor rows are padded to 16 bytes (the per-lane load width of gfx950), not to an
+//     even vector count, and row counts are not padded at all;
+//   * PackedTensors allocates nothing: the HIP kernels tile straight from the row-major
+//     operands through LDS, so pack() only validates.
+#pragma once
+
+#include <cstdint>
+#include <cstring>
+#include <exception>
+#include <optional>
+#include <string>
+#include <type_traits>
+#include <vector>
+
+#include "wekua_hip.h"
+
+namespace wekua {
+
+struct Error : std::exception {
+    int code;
+    explicit Error(int c) : code(c) {}
+    const char *what() const noexcept override { return wk_strerror(code); }
+};
+
+inline void check(int code) {
+    if (code != WK_OK) throw Error(code);
+}
+
+namespace core {
+
+// ---- types (src/core/types.zig) ----------------------------------------------------------
+template <typename R> struct Complex {
+    R real, imag;
+};
+
+template <typename T> struct is_complex : std::false_type {};
+template <typename R> struct is_complex<Complex<R>> : std::true_type {};
+template <typename T> struct scalar_of { using type = T; };
+template <typename R> struct scalar_of<Complex<R>> { using type = R; };
+
+template <typename T> constexpr bool isComplex() { return is_complex<T>::value; }
+
+// getTypeId: 0..9 over the scalar type (types.zig:88-104)
+template <typename T> constexpr int getTypeId() {
+    using R = typename scalar_of<T>::type;
+    if constexpr (std::is_same_v<R, int8_t>) return 0;
+    else if constexpr (std::is_same_v<R, uint8_t>) return 1;
+    else if constexpr (std::is_same_v<R, int16_t>) return 2;
+    else if constexpr (std::is_same_v<R, uint16_t>) return 3;
+    else if constexpr (std::is_same_v<R, int32_t>) return 4;
+    else if constexpr (std::is_same_v<R, uint32_t>) return 5;
+    else if constexpr (std::is_same_v<R, int64_t>) return 6;
+    else if constexpr (std::is_same_v<R, uint64_t>) return 7;
+    else if constexpr (std::is_same_v<R, float>) return 8;
+    else if constexpr (std::is_same_v<R, double>) return 9;
+    else static_assert(sizeof(R) == 0, "Type not supported");
+}
+// getTypeIndex: 0..19 (types.zig:60-86); also the dtype id of the C ABI
+template <typename T> constexpr int getTypeIndex() { return getTypeId<T>() + (isComplex<T>() ? 10 : 0); }
+
+template <typename T> constexpr T getOne() {
+    if constexpr (isComplex<T>()) return T{1, 0};
+    else return T(1);
+}
+
+// ---- CommandQueue / Context ------------------------------------------------------------------
+struct Context;
+
+enum class DeviceType { cpu, gpu, all };
+enum class LocalMemType { local, global };
+
+struct CommandQueue {
+    const Context *context = nullptr;
+    wk_stream *stream = nullptr;
+    uint32_t wekua_id = 0;
+    std::string device_name;
+    LocalMemType local_mem_type = LocalMemType::local;
+    uint64_t local_mem_size = 0;
+    uint32_t compute_units = 0;
+    uint64_t max_work_group_size = 0;
+    uint32_t cache_line_size = 0;
+    // elements per 16-byte lane access for the 10 scalar types (command_queue.zig:81-98 keeps the
+    // OpenCL native widths here)
+    uint32_t vector_widths[10] = {16, 16, 8, 8, 4, 4, 2, 2, 4, 2};
+
+    template <typename T> bool isTypeSupported() const { return true; }
+};
+
+struct Context {
+    wk_device *device = nullptr;
+    std::vector<CommandQueue> command_queues;
+
+    // Context.init with an explicit device ordinal
+    static Context *init(int ordinal) {
+        Context *ctx = new Context;
+        int rc = wk_device_open(ordinal, &ctx->device);
+        if (rc) {
+            delete ctx;
+            throw Error(rc);
+        }
+        ctx->command_queues.resize(1);
+        CommandQueue &q = ctx->command_queues[0];
+        q.context = ctx;
+        rc = wk_stream_create(ctx->device, &q.stream);
+        if (rc) {
+            wk_device_close(ctx->device);
+            delete ctx;
+            throw Error(rc);
+        }
+        wk_props props;
+        wk_device_props(ctx->device, &props);
+        q.device_name = std::string(props.name) + " " + props.arch;
+        q.local_mem_size = props.local_mem_bytes;
+        q.compute_units = (uint32_t)props.compute_units;
+        q.max_work_group_size = (uint64_t)props.max_work_group_size;
+        q.cache_line_size = (uint32_t)props.cache_line_size;
+        return ctx;
+    }
+
+    // Context.initFromDeviceType (context.zig:36-65): this build only has GPU devices
+    static Context *initFromDeviceType(DeviceType type) {
+        if (type == DeviceType::cpu) throw Error(WK_E_NO_DEVICE);
+        return init(0);
+    }
+
+    // Context.initFromBestDevice (context.zig:67-93): the reference scores devices by work-group
+    // size x sub-device count; with identical GPUs that is ordinal 0
+    static Context *initFromBestDevice(DeviceType type) { return initFromDeviceType(type); }
+
+    void deinit() {
+        for (CommandQueue &q : command_queues) wk_stream_destroy(q.stream);
+        wk_device_close(device);
+        delete this;
+    }
+};
+
+// ---- Pipeline ------------------------------------------------------------------------------
+// The reference chains cl_events: each enqueue waits on prevEvents() (the last appended batch)
+// and appends its own event.  On an in-order HIP stream the chain is implicit; the ticket list
+// only preserves the observable bookkeeping (pipeline.zig:35-61).
+struct Pipeline {
+    CommandQueue *command_queue = nullptr;
+    std::vector<uint64_t> events;
+    size_t prev_batch_start = 0;
+    uint64_t next_ticket = 1;
+
+    static Pipeline *init(CommandQueue *cq) {
+        Pipeline *p = new Pipeline;
+        p->command_queue = cq;
+        return p;
+    }
+    void deinit() { delete this; }
+    void prealloc(size_t capacity) { events.reserve(capacity); }
+
+    // last appended batch, empty when nothing is pending
+    std::pair<const uint64_t *, size_t> prevEvents() const {
+        if (events.empty()) return {nullptr, 0};
+        return {events.data() + prev_batch_start, events.size() - prev_batch_start};
+    }
+    void append(size_t count) {
+        prev_batch_start = events.size();
+        for (size_t i = 0; i < count; ++i) events.push_back(next_ticket++);
+    }
+    void waitAndCleanup() {
+        if (events.empty()) return;
+        check(wk_stream_sync(command_queue->stream));
+        events.clear();
+        prev_batch_start = 0;
+    }
+    void clear() {
+        events.clear();
+        events.shrink_to_fit();
+        prev_batch_start = 0;
+    }
+};
+
+} // namespace core
+
+using core::Context;
+using core::Pipeline;
+
+// src/tensor/work_configuration.zig:9-16
+enum class GemmAlgorithm : uint8_t { a2x2 = 0, a4x4 = 1, a8x8 = 2, a16x16 = 3, a32x32 = 4, a64x64 = 5 };
+
+struct CreateConfig {
+    bool vectors_enabled = true; // src/tensor/main.zig:35-39 (cl_mem_flags / host_ptr have no HIP meaning)
+};
+
+template <typename T> struct Tensor {
+    struct Dimensions {
+        std::vector<uint64_t> shape, vl_shape, pitches;
+        uint64_t number_of_elements = 0;
+        uint64_t number_of_elements_without_padding = 0;
+    };
+    struct MemoryLayout {
+        uint64_t row_pitch = 0, row_pitch_for_vectors = 0;
+        uint64_t slice_pitch = 0, slice_pitch_for_vectors = 0;
+        uint64_t number_of_vectors = 0;
+        size_t size = 0;
+    };
+    struct Flags {
+        bool vectors_enabled = false;
+    };
+    struct WorkConfiguration {
+        std::vector<GemmAlgorithm> gemm_algorithm_per_device;
+    };
+
+    const Context *context = nullptr;
+    void *buffer = nullptr; // device memory (hipMalloc)
+    Dimensions dimensions;
+    MemoryLayout memory_layout;
+    Flags flags;
+    WorkConfiguration work_configuration;
+
+    // logical {depth, rows, cols} view used by every kernel launch
+    uint64_t depth() const {
+        uint64_t d = 1;
+        const size_t n = dimensions.shape.size();
+        for (size_t i = 0; i + 2 < n; ++i) d *= dimensions.shape[i];
+        return d;
+    }
+    uint64_t rows() const {
+        const size_t n = dimensions.shape.size();
+        return n >= 2 ? dimensions.shape[n - 2] : 1;
+    }
+    uint64_t cols() const { return dimensions.shape.back(); }
+
+    // Tensor.empty, src/tensor/main.zig:112-251.  Layout differences are listed at the top of
+    // this file; the fields keep their meaning.
+    static Tensor *empty(const Context *context, Pipeline *pipeline, const std::vector<uint64_t> &shape,
+                         CreateConfig config = {}) {
+        (void)pipeline;
+        if (shape.empty()) throw Error(WK_E_INVALID_VALUE);
+        for (uint64_t s : shape)
+            if (s == 0) throw Error(WK_E_INVALID_VALUE);
+
+        Tensor *t = new Tensor;
+        t->context = context;
+        t->dimensions.shape = shape;
+        t->dimensions.vl_shape = shape;
+
+        constexpr bool cplx = core::isComplex<T>();
+        const bool vectors_enabled = !cplx && config.vectors_enabled;
+        const uint64_t vw = vectors_enabled ? context->command_queues[0].vector_widths[core::getTypeId<T>()] : 1;
+        t->flags.vectors_enabled = vectors_enabled && vw > 1;
+
+        const uint64_t cols = shape.back();
+        const uint64_t rows = shape.size() >= 2 ? shape[shape.size() - 2] : 1;
+        uint64_t depth = 1;
+        for (size_t i = 0; i + 2 < shape.size(); ++i) depth *= shape[i];
+
+        uint64_t row_pitch = cols;
+        if (vw > 1 && row_pitch % vw) row_pitch += vw - row_pitch % vw;
+
+        t->dimensions.number_of_elements_without_padding = depth * rows * cols;
+        t->memory_layout.row_pitch = row_pitch;
+        t->memory_layout.row_pitch_for_vectors = row_pitch / vw;
+        t->dimensions.vl_shape.back() = row_pitch / vw;
+        t->memory_layout.slice_pitch = row_pitch * rows;
+        t->memory_layout.slice_pitch_for_vectors = t->memory_layout.slice_pitch / vw;
+        t->dimensions.number_of_elements = t->memory_layout.slice_pitch * depth;
+        t->memory_layout.number_of_vectors = t->dimensions.number_of_elements / vw;
+        t->memory_layout.size = (size_t)t->dimensions.number_of_elements * sizeof(T);
+
+        // pitches per dimension (main.zig:198-220): element strides of the padded layout
+        const size_t nd = shape.size();
+        t->dimensions.pitches.assign(nd, 1);
+        if (nd >= 2) t->dimensions.pitches[nd - 2] = row_pitch;
+        uint64_t p = t->memory_layout.slice_pitch;
+        for (size_t i = nd; i-- > 0;) {
+            if (i + 3 > nd) continue; // last two handled above
+            t->dimensions.pitches[i] = p;
+            p *= shape[i];
+        }
+
+        // GemmAlgorithm kept for API compatibility (work_configuration.zig:110-193, `.local`
+        // branch): largest block <= 64 dividing the (evened) row count and the row pitch.  The
+        // HIP kernels choose their own macro tile per call.
+        GemmAlgorithm alg = GemmAlgorithm::a2x2;
+        const uint64_t h = rows + rows % 2, w = row_pitch + row_pitch % 2;
+        for (int b = 2, i = 0; b <= 64; b *= 2, ++i)
+            if (h % b == 0 && w % b == 0) alg = static_cast<GemmAlgorithm>(i);
+        t->work_configuration.gemm_algorithm_per_device.assign(context->command_queues.size(), alg);
+
+        int rc = wk_malloc(context->device, t->memory_layout.size, &t->buffer);
+        if (rc) {
+            delete t;
+            throw Error(rc);
+        }
+        return t;
+    }
+
+    // Tensor.alloc = empty + fill.zeroes (main.zig:265-277)
+    static Tensor *alloc(const Context *context, Pipeline *pipeline, const std::vector<uint64_t> &shape,
+                         CreateConfig config = {}) {
+        Tensor *t = empty(context, pipeline, shape, config);
+        int rc = wk_memset_async(pipeline->command_queue->stream, t->buffer, 0, t->memory_layout.size);
+        if (rc) {
+            wk_free(context->device, t->buffer);
+            delete t;
+            throw Error(rc);
+        }
+        pipeline->append(1);
+        return t;
+    }
+
+    // Tensor.release drains the pipeline first (main.zig:253-263)
+    void release(Pipeline *pipeline) {
+        pipeline->waitAndCleanup();
+        wk_free(context->device, buffer);
+        delete this;
+    }
+};
+
+namespace helpers {
+// src/tensor/helpers.zig:53-57
+template <typename T> void eqlTensorsShape(const Tensor<T> *a, const Tensor<T> *b) {
+    if (a->dimensions.shape != b->dimensions.shape) throw Error(WK_E_UNQUAL_TENSORS_SHAPE);
+}
+} // namespace helpers
+
+namespace memory {
+// HOST -> DEVICE of the logical region (src/tensor/memory/read_from_buffer.zig:13-63)
+template <typename T> void readFromBuffer(Pipeline *pipeline, Tensor<T> *tensor, const T *buffer, size_t len) {
+    if (len != tensor->dimensions.number_of_elements_without_padding) throw Error(WK_E_INVALID_BUFFER);
+    const size_t width = (size_t)tensor->cols() * sizeof(T), rows = (size_t)tensor->rows(), depth = (size_t)tensor->depth();
+    check(wk_copy_h2d_rect_async(pipeline->command_queue->stream, tensor->buffer,
+                                 (size_t)tensor->memory_layout.row_pitch * sizeof(T),
+                                 (size_t)tensor->memory_layout.slice_pitch * sizeof(T), buffer, width, width * rows, width,
+                                 rows, depth));
+    pipeline->append(1);
+}
+// DEVICE -> HOST of the logical region (src/tensor/memory/write_to_buffer.zig:13-63)
+template <typename T> void writeToBuffer(Pipeline *pipeline, Tensor<T> *tensor, T *buffer, size_t len) {
+    if (len != tensor->dimensions.number_of_elements_without_padding) throw Error(WK_E_INVALID_BUFFER);
+    const size_t width = (size_t)tensor->cols() * sizeof(T), rows = (size_t)tensor->rows(), depth = (size_t)tensor->depth();
+    check(wk_copy_d2h_rect_async(pipeline->command_queue->stream, buffer, width, width * rows, tensor->buffer,
+                                 (size_t)tensor->memory_layout.row_pitch * sizeof(T),
+                                 (size_t)tensor->memory_layout.slice_pitch * sizeof(T), width, rows, depth));
+    pipeline->append(1);
+}
+} // namespace memory
+
+namespace fill {
+// src/tensor/fill.zig:70-95
+template <typename T> void zeroes(Pipeline *pipeline, Tensor<T> *tensor) {
+    check(wk_memset_async(pipeline->command_queue->stream, tensor->buffer, 0, tensor->memory_layout.size));
+    pipeline->append(1);
+}
+// src/tensor/fill.zig:16-57
+template <typename T> void constant(Pipeline *pipeline, Tensor<T> *tensor, T value) {
+    const uint64_t shape3[3] = {tensor->depth(), tensor->rows(), tensor->cols()};
+    check(wk_fill(pipeline->command_queue->stream, core::getTypeIndex<T>(), tensor->buffer, shape3,
+                  tensor->memory_layout.row_pitch, tensor->memory_layout.slice_pitch, &value));
+    pipeline->append(1);
+}
+template <typename T> void one(Pipeline *pipeline, Tensor<T> *tensor) { constant<T>(pipeline, tensor, core::getOne<T>()); }
+} // namespace fill
+
+// src/tensor/identity.zig:16-70
+template <typename T> void identity(Pipeline *pipeline, Tensor<T> *tensor) {
+    const uint64_t size = tensor->dimensions.shape[0];
+    for (uint64_t s : tensor->dimensions.shape)
+        if (s != size) throw Error(WK_E_INVALID_VALUE);
+    fill::zeroes<T>(pipeline, tensor);
+    uint64_t pitch_sum = 0;
+    for (uint64_t p : tensor->dimensions.pitches) pitch_sum += p;
+    check(wk_identity(pipeline->command_queue->stream, core::getTypeIndex<T>(), tensor->buffer, size, pitch_sum));
+    pipeline->append(1);
+}
+
+namespace blas {
+
+enum class Operation : uint8_t { no_transpose = 0, transpose = 1 }; // src/blas/gemm.zig:25-29
+
+// src/blas/axpy.zig:93-169.  alpha == nullopt: y += x; alpha == -1: y -= x; else y += alpha*x.
+template <typename T> void axpy(Pipeline *pipeline, Tensor<T> *x, std::optional<T> alpha, Tensor<T> *y) {
+    helpers::eqlTensorsShape<T>(x, y);
+    const uint64_t shape3[3] = {x->depth(), x->rows(), x->cols()};
+    const T a = alpha.value_or(T{});
+    check(wk_axpy(pipeline->command_queue->stream, core::getTypeIndex<T>(), shape3, x->buffer, x->memory_layout.row_pitch,
+                  x->memory_layout.slice_pitch, y->buffer, y->memory_layout.row_pitch, y->memory_layout.slice_pitch,
+                  alpha ? &a : nullptr));
+    pipeline->append(1);
+}
+
+// src/blas/gemm.zig:60-359.  n_size = rows of C, m_size = columns of C (the reference's naming).
+template <typename T> struct PackedTensors {
+    uint64_t m_size = 0, n_size = 0, k_size = 0;
+    Tensor<T> *packed_a = nullptr, *packed_b = nullptr; // never allocated: no pack pass on this device
+    bool vectors_enabled = false;
+    GemmAlgorithm algorithm = GemmAlgorithm::a2x2;
+
+    static PackedTensors *init(Pipeline *pipeline, Tensor<T> *result_tensor, uint64_t k_size, bool vectors_enabled) {
+        const auto &shape = result_tensor->dimensions.shape;
+        if (shape.size() != 2) throw Error(WK_E_INVALID_VALUE);
+        const uint32_t id = pipeline->command_queue->wekua_id;
+        return initWithDimensions(pipeline, shape[0], shape[1], k_size,
+                                  result_tensor->work_configuration.gemm_algorithm_per_device[id], vectors_enabled);
+    }
+    static PackedTensors *initWithDimensions(Pipeline *pipeline, uint64_t n_size, uint64_t m_size, uint64_t k_size,
+                                             GemmAlgorithm recommended_algorithm, bool vectors_enabled) {
+        (void)pipeline;
+        if (!n_size || !m_size || !k_size) throw Error(WK_E_INVALID_VALUE);
+        PackedTensors *p = new PackedTensors;
+        p->n_size = n_size;
+        p->m_size = m_size;
+        p->k_size = k_size;
+        p->vectors_enabled = !core::isComplex<T>() && vectors_enabled;
+        p->algorithm = recommended_algorithm;
+        return p;
+    }
+    void deinit(Pipeline *pipeline) {
+        pipeline->waitAndCleanup(); // the reference's deinit releases two tensors, each draining the pipeline
+        delete this;
+    }
+    // gemm.zig:250-270
+    void validateTensors(const Tensor<T> *a, Operation op_a, const Tensor<T> *b, Operation op_b) const {
+        const auto &as = a->dimensions.shape, &bs = b->dimensions.shape;
+        if (as.size() != 2 || bs.size() != 2) throw Error(WK_E_INVALID_VALUE);
+        bool valid = op_a == Operation::no_transpose ? (as[0] == n_size && as[1] == k_size)
+                                                     : (as[1] == n_size && as[0] == k_size);
+        valid &= op_b == Operation::no_transpose ? (bs[0] == k_size && bs[1] == m_size)
+                                                 : (bs[1] == k_size && bs[0] == m_size);
+        if (!valid) throw Error(WK_E_INVALID_VALUE);
+    }
+    // gemm.zig:272-357: validation only; nothing is re-tiled in memory
+    void pack(Pipeline *pipeline, Tensor<T> *a, Operation op_a, Tensor<T> *b, Operation op_b) {
+        (void)pipeline;
+        validateTensors(a, op_a, b, op_b);
+    }
+};
+
+// src/blas/gemm.zig:442-485
+template <typename T>
+void validateTensors(const Tensor<T> *a, const Tensor<T> *b, const Tensor<T> *c, Operation op_a, Operation op_b) {
+    if (a->context != b->context || a->context != c->context) throw Error(WK_E_UNQUAL_TENSORS_CONTEXT);
+    const auto &as = a->dimensions.shape, &bs = b->dimensions.shape, &cs = c->dimensions.shape;
+    if (cs.size() != 2 || as.size() != 2 || bs.size() != 2) throw Error(WK_E_INVALID_VALUE);
+    const uint64_t a_m = as[0], a_k = as[1], b_k = bs[0], b_n = bs[1], c_m = cs[0], c_n = cs[1];
+    bool match;
+    if (op_a == Operation::transpose)
+        match = op_b == Operation::no_transpose ? (a_m == b_k && b_n == c_n && a_k == c_m)
+                                                : (a_m == b_n && b_k == c_n && a_k == c_m);
+    else
+        match = op_b == Operation::no_transpose ? (a_k == b_k && b_n == c_n && a_m == c_m)
+                                                : (a_k == b_n && b_k == c_n && a_m == c_m);
+    if (!match) throw Error(WK_E_INVALID_VALUE);
+}
+
+// src/blas/gemm.zig:834-874
+template <typename T>
+void gemm(Pipeline *pipeline, std::optional<T> alpha, Tensor<T> *a, Operation op_a, Tensor<T> *b, Operation op_b,
+          std::optional<T> beta, Tensor<T> *c, PackedTensors<T> *packed_tensors = nullptr) {
+    validateTensors<T>(a, b, c, op_a, op_b);
+    if (packed_tensors) packed_tensors->pack(pipeline, a, op_a, b, op_b);
+    const uint64_t M = c->dimensions.shape[0], N = c->dimensions.shape[1];
+    const uint64_t K = a->dimensions.shape[op_a == Operation::transpose ? 0 : 1];
+    const T av = alpha.value_or(T{}), bv = beta.value_or(T{});
+    check(wk_gemm(pipeline->command_queue->stream, core::getTypeIndex<T>(), (int)op_a, (int)op_b, M, N, K,
+                  alpha ? &av : nullptr, a->buffer, a->memory_layout.row_pitch, b->buffer, b->memory_layout.row_pitch,
+                  beta ? &bv : nullptr, c->buffer, c->memory_layout.row_pitch, nullptr, 0));
+    pipeline->append(1);
+}
+
+} // namespace blas
+
+using GemmOperation = blas::Operation;
+template <typename T> using GemmPackedTensors = blas::PackedTensors<T>;
+
+} // namespace wekua

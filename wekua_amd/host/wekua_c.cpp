@@ -1,0 +1,299 @@
+// wekua_c.cpp -- flat C entry points over the C++ host mirror (wekua.hpp), one per public
+// function of the reference's Zig API on the gemm/axpy path, with the element type passed as
+// the dtype id of src/core/types.zig getTypeIndex.  This is what the Python package binds, so
+// the parity tests exercise the same host logic (validation, layout, option handling) a C++
+// caller gets.  Every function returns a WK_E_* code (the Zig error name) and never throws.
+#include "wekua.hpp"
+
+#include <new>
+
+using namespace wekua;
+using wekua::blas::Operation;
+
+namespace {
+
+struct TensorHandle {
+    int dtype;
+    void *tensor; // Tensor<T>*
+};
+
+struct PackedHandle {
+    int dtype;
+    void *packed; // blas::PackedTensors<T>*
+};
+
+template <typename F> int guard(F &&f) {
+    try {
+        f();
+        return WK_OK;
+    } catch (const Error &e) {
+        return e.code;
+    } catch (const std::bad_alloc &) {
+        return WK_E_OUT_OF_MEMORY;
+    } catch (...) {
+        return WK_E_INVALID_VALUE;
+    }
+}
+
+template <typename F> void dispatch(int dtype, F &&f) {
+    using namespace wekua::core;
+    switch (dtype) {
+    case 0: f.template operator()<int8_t>(); break;
+    case 1: f.template operator()<uint8_t>(); break;
+    case 2: f.template operator()<int16_t>(); break;
+    case 3: f.template operator()<uint16_t>(); break;
+    case 4: f.template operator()<int32_t>(); break;
+    case 5: f.template operator()<uint32_t>(); break;
+    case 6: f.template operator()<int64_t>(); break;
+    case 7: f.template operator()<uint64_t>(); break;
+    case 8: f.template operator()<float>(); break;
+    case 9: f.template operator()<double>(); break;
+    case 10: f.template operator()<Complex<int8_t>>(); break;
+    case 11: f.template operator()<Complex<uint8_t>>(); break;
+    case 12: f.template operator()<Complex<int16_t>>(); break;
+    case 13: f.template operator()<Complex<uint16_t>>(); break;
+    case 14: f.template operator()<Complex<int32_t>>(); break;
+    case 15: f.template operator()<Complex<uint32_t>>(); break;
+    case 16: f.template operator()<Complex<int64_t>>(); break;
+    case 17: f.template operator()<Complex<uint64_t>>(); break;
+    case 18: f.template operator()<Complex<float>>(); break;
+    case 19: f.template operator()<Complex<double>>(); break;
+    default: throw Error(WK_E_TYPE_NOT_SUPPORTED);
+    }
+}
+
+template <typename T> std::optional<T> opt_scalar(const void *p) {
+    if (!p) return std::nullopt;
+    T v;
+    std::memcpy(&v, p, sizeof(T));
+    return v;
+}
+
+} // namespace
+
+extern "C" {
+
+struct wkz_tensor_info {
+    int dtype;
+    int ndim;
+    uint64_t shape[8];
+    uint64_t pitches[8];
+    uint64_t number_of_elements;
+    uint64_t number_of_elements_without_padding;
+    uint64_t row_pitch, row_pitch_for_vectors, slice_pitch, slice_pitch_for_vectors, number_of_vectors;
+    uint64_t size;
+    int vectors_enabled;
+    int gemm_algorithm;
+    void *buffer;
+};
+
+// ---- Context / Pipeline --------------------------------------------------------------------
+int wkz_context_init_from_device_type(int device_type, void **out) {
+    return guard([&] { *out = Context::initFromDeviceType(static_cast<core::DeviceType>(device_type)); });
+}
+int wkz_context_init_from_best_device(int device_type, void **out) {
+    return guard([&] { *out = Context::initFromBestDevice(static_cast<core::DeviceType>(device_type)); });
+}
+int wkz_context_init(int ordinal, void **out) {
+    return guard([&] { *out = Context::init(ordinal); });
+}
+void wkz_context_deinit(void *ctx) {
+    if (ctx) static_cast<Context *>(ctx)->deinit();
+}
+int wkz_context_num_queues(void *ctx) { return (int)static_cast<Context *>(ctx)->command_queues.size(); }
+void *wkz_context_stream(void *ctx, int queue) { return static_cast<Context *>(ctx)->command_queues[queue].stream; }
+void *wkz_context_device(void *ctx) { return static_cast<Context *>(ctx)->device; }
+
+int wkz_pipeline_init(void *ctx, int queue, void **out) {
+    return guard([&] {
+        Context *c = static_cast<Context *>(ctx);
+        if (queue < 0 || (size_t)queue >= c->command_queues.size()) throw Error(WK_E_INVALID_VALUE);
+        *out = Pipeline::init(&c->command_queues[queue]);
+    });
+}
+void wkz_pipeline_deinit(void *p) {
+    if (p) static_cast<Pipeline *>(p)->deinit();
+}
+int wkz_pipeline_prealloc(void *p, uint64_t n) {
+    return guard([&] { static_cast<Pipeline *>(p)->prealloc(n); });
+}
+int wkz_pipeline_wait_and_cleanup(void *p) {
+    return guard([&] { static_cast<Pipeline *>(p)->waitAndCleanup(); });
+}
+uint64_t wkz_pipeline_pending(void *p) { return static_cast<Pipeline *>(p)->events.size(); }
+uint64_t wkz_pipeline_prev_events(void *p) { return static_cast<Pipeline *>(p)->prevEvents().second; }
+void wkz_pipeline_clear(void *p) { static_cast<Pipeline *>(p)->clear(); }
+
+// ---- Tensor ----------------------------------------------------------------------------------
+static int tensor_create(void *ctx, void *pipeline, int dtype, const uint64_t *shape, int ndim, int vectors_enabled,
+                         bool zero, void **out) {
+    return guard([&] {
+        if (!out || ndim < 0 || ndim > 8 || (ndim > 0 && !shape)) throw Error(WK_E_INVALID_VALUE);
+        std::vector<uint64_t> shp(shape, shape + ndim);
+        CreateConfig cfg;
+        cfg.vectors_enabled = vectors_enabled != 0;
+        dispatch(dtype, [&]<typename T>() {
+            Tensor<T> *t = zero ? Tensor<T>::alloc(static_cast<Context *>(ctx), static_cast<Pipeline *>(pipeline), shp, cfg)
+                                : Tensor<T>::empty(static_cast<Context *>(ctx), static_cast<Pipeline *>(pipeline), shp, cfg);
+            *out = new TensorHandle{dtype, t};
+        });
+    });
+}
+int wkz_tensor_alloc(void *ctx, void *pipeline, int dtype, const uint64_t *shape, int ndim, int vectors_enabled, void **out) {
+    return tensor_create(ctx, pipeline, dtype, shape, ndim, vectors_enabled, true, out);
+}
+int wkz_tensor_empty(void *ctx, void *pipeline, int dtype, const uint64_t *shape, int ndim, int vectors_enabled, void **out) {
+    return tensor_create(ctx, pipeline, dtype, shape, ndim, vectors_enabled, false, out);
+}
+int wkz_tensor_release(void *tensor, void *pipeline) {
+    return guard([&] {
+        TensorHandle *h = static_cast<TensorHandle *>(tensor);
+        dispatch(h->dtype, [&]<typename T>() { static_cast<Tensor<T> *>(h->tensor)->release(static_cast<Pipeline *>(pipeline)); });
+        delete h;
+    });
+}
+int wkz_tensor_get_info(void *tensor, wkz_tensor_info *info) {
+    return guard([&] {
+        TensorHandle *h = static_cast<TensorHandle *>(tensor);
+        dispatch(h->dtype, [&]<typename T>() {
+            const Tensor<T> *t = static_cast<Tensor<T> *>(h->tensor);
+            std::memset(info, 0, sizeof *info);
+            info->dtype = h->dtype;
+            info->ndim = (int)t->dimensions.shape.size();
+            for (int i = 0; i < info->ndim; ++i) {
+                info->shape[i] = t->dimensions.shape[i];
+                info->pitches[i] = t->dimensions.pitches[i];
+            }
+            info->number_of_elements = t->dimensions.number_of_elements;
+            info->number_of_elements_without_padding = t->dimensions.number_of_elements_without_padding;
+            info->row_pitch = t->memory_layout.row_pitch;
+            info->row_pitch_for_vectors = t->memory_layout.row_pitch_for_vectors;
+            info->slice_pitch = t->memory_layout.slice_pitch;
+            info->slice_pitch_for_vectors = t->memory_layout.slice_pitch_for_vectors;
+            info->number_of_vectors = t->memory_layout.number_of_vectors;
+            info->size = t->memory_layout.size;
+            info->vectors_enabled = t->flags.vectors_enabled;
+            info->gemm_algorithm = (int)t->work_configuration.gemm_algorithm_per_device[0];
+            info->buffer = t->buffer;
+        });
+    });
+}
+
+// ---- memory / fill / identity ------------------------------------------------------------------
+int wkz_read_from_buffer(void *pipeline, void *tensor, const void *host, uint64_t len) {
+    return guard([&] {
+        TensorHandle *h = static_cast<TensorHandle *>(tensor);
+        dispatch(h->dtype, [&]<typename T>() {
+            memory::readFromBuffer<T>(static_cast<Pipeline *>(pipeline), static_cast<Tensor<T> *>(h->tensor),
+                                      static_cast<const T *>(host), (size_t)len);
+        });
+    });
+}
+int wkz_write_to_buffer(void *pipeline, void *tensor, void *host, uint64_t len) {
+    return guard([&] {
+        TensorHandle *h = static_cast<TensorHandle *>(tensor);
+        dispatch(h->dtype, [&]<typename T>() {
+            memory::writeToBuffer<T>(static_cast<Pipeline *>(pipeline), static_cast<Tensor<T> *>(h->tensor),
+                                     static_cast<T *>(host), (size_t)len);
+        });
+    });
+}
+int wkz_fill_zeroes(void *pipeline, void *tensor) {
+    return guard([&] {
+        TensorHandle *h = static_cast<TensorHandle *>(tensor);
+        dispatch(h->dtype, [&]<typename T>() { fill::zeroes<T>(static_cast<Pipeline *>(pipeline), static_cast<Tensor<T> *>(h->tensor)); });
+    });
+}
+int wkz_fill_one(void *pipeline, void *tensor) {
+    return guard([&] {
+        TensorHandle *h = static_cast<TensorHandle *>(tensor);
+        dispatch(h->dtype, [&]<typename T>() { fill::one<T>(static_cast<Pipeline *>(pipeline), static_cast<Tensor<T> *>(h->tensor)); });
+    });
+}
+int wkz_fill_constant(void *pipeline, void *tensor, const void *host_scalar) {
+    return guard([&] {
+        TensorHandle *h = static_cast<TensorHandle *>(tensor);
+        if (!host_scalar) throw Error(WK_E_INVALID_VALUE);
+        dispatch(h->dtype, [&]<typename T>() {
+            fill::constant<T>(static_cast<Pipeline *>(pipeline), static_cast<Tensor<T> *>(h->tensor), *opt_scalar<T>(host_scalar));
+        });
+    });
+}
+int wkz_identity(void *pipeline, void *tensor) {
+    return guard([&] {
+        TensorHandle *h = static_cast<TensorHandle *>(tensor);
+        dispatch(h->dtype, [&]<typename T>() { identity<T>(static_cast<Pipeline *>(pipeline), static_cast<Tensor<T> *>(h->tensor)); });
+    });
+}
+
+// ---- blas -----------------------------------------------------------------------------------------
+int wkz_axpy(void *pipeline, void *x, const void *host_alpha, void *y) {
+    return guard([&] {
+        TensorHandle *hx = static_cast<TensorHandle *>(x), *hy = static_cast<TensorHandle *>(y);
+        if (hx->dtype != hy->dtype) throw Error(WK_E_UNQUAL_TENSORS_ATTRIBUTE); // Zig rejects this at compile time
+        dispatch(hx->dtype, [&]<typename T>() {
+            blas::axpy<T>(static_cast<Pipeline *>(pipeline), static_cast<Tensor<T> *>(hx->tensor), opt_scalar<T>(host_alpha),
+                          static_cast<Tensor<T> *>(hy->tensor));
+        });
+    });
+}
+
+int wkz_packed_init(void *pipeline, void *result_tensor, uint64_t k_size, int vectors_enabled, void **out) {
+    return guard([&] {
+        TensorHandle *h = static_cast<TensorHandle *>(result_tensor);
+        dispatch(h->dtype, [&]<typename T>() {
+            auto *p = blas::PackedTensors<T>::init(static_cast<Pipeline *>(pipeline), static_cast<Tensor<T> *>(h->tensor), k_size,
+                                                   vectors_enabled != 0);
+            *out = new PackedHandle{h->dtype, p};
+        });
+    });
+}
+int wkz_packed_init_with_dimensions(void *pipeline, int dtype, uint64_t n_size, uint64_t m_size, uint64_t k_size,
+                                    int recommended_algorithm, int vectors_enabled, void **out) {
+    return guard([&] {
+        dispatch(dtype, [&]<typename T>() {
+            auto *p = blas::PackedTensors<T>::initWithDimensions(static_cast<Pipeline *>(pipeline), n_size, m_size, k_size,
+                                                                 static_cast<GemmAlgorithm>(recommended_algorithm),
+                                                                 vectors_enabled != 0);
+            *out = new PackedHandle{dtype, p};
+        });
+    });
+}
+int wkz_packed_deinit(void *packed, void *pipeline) {
+    return guard([&] {
+        PackedHandle *h = static_cast<PackedHandle *>(packed);
+        dispatch(h->dtype, [&]<typename T>() { static_cast<blas::PackedTensors<T> *>(h->packed)->deinit(static_cast<Pipeline *>(pipeline)); });
+        delete h;
+    });
+}
+int wkz_packed_pack(void *packed, void *pipeline, void *a, int op_a, void *b, int op_b) {
+    return guard([&] {
+        PackedHandle *h = static_cast<PackedHandle *>(packed);
+        TensorHandle *ha = static_cast<TensorHandle *>(a), *hb = static_cast<TensorHandle *>(b);
+        if (ha->dtype != h->dtype || hb->dtype != h->dtype) throw Error(WK_E_UNQUAL_TENSORS_ATTRIBUTE);
+        dispatch(h->dtype, [&]<typename T>() {
+            static_cast<blas::PackedTensors<T> *>(h->packed)->pack(static_cast<Pipeline *>(pipeline),
+                                                                   static_cast<Tensor<T> *>(ha->tensor), static_cast<Operation>(op_a),
+                                                                   static_cast<Tensor<T> *>(hb->tensor), static_cast<Operation>(op_b));
+        });
+    });
+}
+
+int wkz_gemm(void *pipeline, const void *host_alpha, void *a, int op_a, void *b, int op_b, const void *host_beta, void *c,
+             void *packed) {
+    return guard([&] {
+        TensorHandle *ha = static_cast<TensorHandle *>(a), *hb = static_cast<TensorHandle *>(b), *hc = static_cast<TensorHandle *>(c);
+        PackedHandle *hp = static_cast<PackedHandle *>(packed);
+        if (ha->dtype != hb->dtype || ha->dtype != hc->dtype || (hp && hp->dtype != ha->dtype))
+            throw Error(WK_E_UNQUAL_TENSORS_ATTRIBUTE);
+        if ((op_a != 0 && op_a != 1) || (op_b != 0 && op_b != 1)) throw Error(WK_E_INVALID_VALUE);
+        dispatch(ha->dtype, [&]<typename T>() {
+            blas::gemm<T>(static_cast<Pipeline *>(pipeline), opt_scalar<T>(host_alpha), static_cast<Tensor<T> *>(ha->tensor),
+                          static_cast<Operation>(op_a), static_cast<Tensor<T> *>(hb->tensor), static_cast<Operation>(op_b),
+                          opt_scalar<T>(host_beta), static_cast<Tensor<T> *>(hc->tensor),
+                          hp ? static_cast<blas::PackedTensors<T> *>(hp->packed) : nullptr);
+        });
+    });
+}
+
+} // extern "C"
