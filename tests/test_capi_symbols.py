@@ -41,7 +41,7 @@ def test_binding_covers_every_declared_symbol():
 
 def test_header_compiles_as_plain_c():
     """The boundary is a C ABI: the header must be valid C, not only C++."""
-    src = '#include "wekua_hip.h"\nint main(void){ return wk_gemm == 0; }\n'
+    src = '#include "wekua_hip.h"\nint main(void){ int (*f)(wk_stream*, int, int, int, uint64_t, uint64_t, uint64_t, const void*, const void*, uint64_t, const void*, uint64_t, const void*, void*, uint64_t, void*, size_t) = wk_gemm; return f != wk_gemm; }\n'
     res = subprocess.run(["gcc", "-std=c99", "-Wall", "-Werror", "-fsyntax-only", "-I", os.path.join(ROOT, "include"),
                           "-x", "c", "-"], input=src, text=True, capture_output=True)
     assert res.returncode == 0, res.stderr
