@@ -1,0 +1,167 @@
+"""GPU: the benchmark configurations (BASELINE.json `configs`) at their real sizes.
+
+Shapes the oracle finishes in seconds are compared entry by entry with it.  The large ones
+(>= 4096^3) are checked through properties that do not need a second full product:
+  * 1024 sampled entries against float64 dot products (tolerance 1e-5*sqrt(K) / 1e-12*sqrt(K)
+    relative to sum|a||b|, as stated for the task);
+  * every entry, in aggregate: C @ 1 must equal alpha * A (B 1) + beta * C0 1 (linearity), an
+    O(n^2) identity evaluated in float64.
+int32 is compared bit for bit: for |entries| <= 2^20 and K = 2048 every partial sum stays
+below 2^53, so a float64 product is exact and is then reduced mod 2^32.
+"""
+import numpy as np
+import pytest
+
+import oracle
+from helpers import F32_TOL, F64_TOL, assert_gemm_close
+from wekua_amd import synth
+
+pytestmark = pytest.mark.gpu
+OPS = [(0, 0), (0, 1), (1, 0), (1, 1)]
+
+
+def run(dev, dtype, alpha, a, op_a, b, op_b, beta, c):
+    M, N = c.shape
+    K = a.shape[0] if op_a else a.shape[1]
+    dA, dB, dC = dev.upload(a), dev.upload(b), dev.upload(c)
+    dev.gemm(dtype, op_a, op_b, M, N, K, alpha, dA, a.shape[1], dB, b.shape[1], beta, dC, N)
+    out = dC.download(c.dtype, c.shape)
+    for d in (dA, dB, dC):
+        d.free()
+    return out
+
+
+def operands(rd, M, N, K, op_a, op_b, cfg):
+    a = synth.uniform(synth.config_seed(cfg, 0), (K, M) if op_a else (M, K), rd)
+    b = synth.uniform(synth.config_seed(cfg, 1), (N, K) if op_b else (K, N), rd)
+    c = synth.uniform(synth.config_seed(cfg, 2), (M, N), rd)
+    return a, b, c
+
+
+def check_by_properties(dtype, got, alpha, a, op_a, b, op_b, beta, c, K):
+    tol = (F32_TOL if dtype == "f32" else F64_TOL) * np.sqrt(K)
+    assert np.isfinite(got).all()
+    A = a.T if op_a else a
+    B = b.T if op_b else b
+    al = 1.0 if alpha is None else float(alpha)
+    be = 0.0 if beta is None else float(beta)
+    M, N = got.shape
+    # sampled entries
+    rng = np.random.default_rng(123)
+    ii = rng.integers(0, M, 1024)
+    jj = rng.integers(0, N, 1024)
+    Ar = A[ii].astype(np.float64)
+    Bc = B[:, jj].astype(np.float64).T
+    want = al * np.einsum("ik,ik->i", Ar, Bc) + be * c[ii, jj].astype(np.float64)
+    bound = abs(al) * np.einsum("ik,ik->i", np.abs(Ar), np.abs(Bc)) + abs(be) * np.abs(c[ii, jj]).astype(np.float64)
+    err = np.abs(got[ii, jj].astype(np.float64) - want) / bound
+    assert err.max() <= tol, f"sampled entries: {err.max():.3e} > {tol:.3e}"
+    # linearity over all entries: row sums
+    ones = np.ones(N, dtype=np.float64)
+    rhs = al * (A.astype(np.float64) @ (B.astype(np.float64) @ ones)) + be * (c.astype(np.float64) @ ones)
+    rb = abs(al) * (np.abs(A).astype(np.float64) @ (np.abs(B).astype(np.float64) @ ones)) + abs(be) * (np.abs(c).astype(np.float64) @ ones)
+    lhs = got.astype(np.float64) @ ones
+    rerr = np.abs(lhs - rhs) / rb
+    assert rerr.max() <= tol, f"row sums: {rerr.max():.3e} > {tol:.3e}"
+    # and column sums (catches a transposed block that row sums of a symmetric layout would not)
+    onesM = np.ones(M, dtype=np.float64)
+    rhs = al * ((onesM @ A.astype(np.float64)) @ B.astype(np.float64)) + be * (onesM @ c.astype(np.float64))
+    cb = abs(al) * ((onesM @ np.abs(A).astype(np.float64)) @ np.abs(B).astype(np.float64)) + abs(be) * (onesM @ np.abs(c).astype(np.float64))
+    cerr = np.abs(onesM @ got.astype(np.float64) - rhs) / cb
+    assert cerr.max() <= tol, f"column sums: {cerr.max():.3e} > {tol:.3e}"
+
+
+def test_config1_f32_512(dev):
+    """f32 C = 1.0*A*B + 0.0*C at 512^3 (C initially zero), also the reference CPU path's own case."""
+    a, b, _ = operands(np.float32, 512, 512, 512, 0, 0, 1)
+    c = np.zeros((512, 512), np.float32)
+    got = run(dev, "f32", 1.0, a, 0, b, 0, 0.0, c)
+    want = oracle.gemm("f32", 1.0, a, 0, b, 0, 0.0, c, vector_width=8, packed=True)   # the CPU device's own path
+    assert_gemm_close("f32", got, want, 1.0, a, 0, b, 0, 0.0, c, 512, what="config 1")
+    exact = oracle.semantic_gemm("f32", 1.0, a, 0, b, 0, 0.0, c)     # long-double accumulation
+    assert_gemm_close("f32", got, exact, 1.0, a, 0, b, 0, 0.0, c, 512, what="config 1 vs exact")
+
+
+@pytest.mark.parametrize("n", [1024, 2048])
+@pytest.mark.parametrize("op_a,op_b", OPS)
+def test_config3_f32_square_vs_oracle(dev, n, op_a, op_b):
+    a, b, c = operands(np.float32, n, n, n, op_a, op_b, 3)
+    got = run(dev, "f32", 1.5, a, op_a, b, op_b, 0.5, c)
+    want = oracle.gemm("f32", 1.5, a, op_a, b, op_b, 0.5, c, vector_width=8, packed=True)
+    assert_gemm_close("f32", got, want, 1.5, a, op_a, b, op_b, 0.5, c, n, what=f"config 3 n={n}")
+
+
+@pytest.mark.parametrize("n", [4096, 8192])
+@pytest.mark.parametrize("op_a,op_b", OPS)
+def test_config3_f32_square_large(dev, n, op_a, op_b):
+    a, b, c = operands(np.float32, n, n, n, op_a, op_b, 3)
+    got = run(dev, "f32", 1.5, a, op_a, b, op_b, 0.5, c)
+    check_by_properties("f32", got, 1.5, a, op_a, b, op_b, 0.5, c, n)
+
+
+@pytest.mark.parametrize("op_a,op_b", OPS)
+def test_config3_f32_ragged_1000(dev, op_a, op_b):
+    a, b, c = operands(np.float32, 1000, 1000, 1000, op_a, op_b, 3)
+    got = run(dev, "f32", 1.5, a, op_a, b, op_b, 0.5, c)
+    want = oracle.gemm("f32", 1.5, a, op_a, b, op_b, 0.5, c, vector_width=8, packed=True)
+    assert_gemm_close("f32", got, want, 1.5, a, op_a, b, op_b, 0.5, c, 1000, what="config 3 1000^3")
+
+
+@pytest.mark.parametrize("op_a,op_b", OPS)
+def test_config3_f32_ragged_4097x4095x4093(dev, op_a, op_b):
+    M, N, K = 4097, 4095, 4093
+    a, b, c = operands(np.float32, M, N, K, op_a, op_b, 3)
+    got = run(dev, "f32", 1.5, a, op_a, b, op_b, 0.5, c)
+    check_by_properties("f32", got, 1.5, a, op_a, b, op_b, 0.5, c, K)
+
+
+def test_config4_f64_4096(dev):
+    a, b, c = operands(np.float64, 4096, 4096, 4096, 0, 0, 4)
+    got = run(dev, "f64", 1.0, a, 0, b, 0, 1.0, c)
+    check_by_properties("f64", got, 1.0, a, 0, b, 0, 1.0, c, 4096)
+
+
+def test_config4_f64_tall_skinny(dev):
+    M, N, K = 8192, 256, 8192
+    a, b, c = operands(np.float64, M, N, K, 0, 0, 4)
+    got = run(dev, "f64", 1.0, a, 0, b, 0, 1.0, c)
+    check_by_properties("f64", got, 1.0, a, 0, b, 0, 1.0, c, K)
+    # small enough for a full float64 reference as well (numpy's own BLAS, a third opinion)
+    ref = a @ b + c
+    bound = np.abs(a) @ np.abs(b) + np.abs(c)
+    assert (np.abs(got - ref) / bound).max() <= F64_TOL * np.sqrt(K)
+
+
+def _exact_int32(alpha, a, b, beta, c):
+    prod = a.astype(np.float64) @ b.astype(np.float64)          # exact: every partial sum < 2^53
+    assert np.abs(prod).max() < 2.0 ** 53
+    p = prod.astype(np.int64)
+    al = 1 if alpha is None else alpha
+    out = p * al + (0 if beta is None else beta) * c.astype(np.int64)
+    if alpha is None and beta is None:
+        out = p
+    return (out & 0xFFFFFFFF).astype(np.uint32).view(np.int32)
+
+
+@pytest.mark.parametrize("alpha,beta", [(None, None), (3, -2)])
+def test_config4_int32_2048_bit_exact(dev, alpha, beta):
+    n = 2048
+    a = synth.integers(synth.config_seed(4, 3), (n, n), np.int32, -100, 100)
+    b = synth.integers(synth.config_seed(4, 4), (n, n), np.int32, -100, 100)
+    c = synth.integers(synth.config_seed(4, 5), (n, n), np.int32, -100, 100)
+    got = run(dev, "i32", alpha, a, 0, b, 0, beta, c)
+    assert np.array_equal(got, _exact_int32(alpha, a, b, beta, c))
+
+
+def test_config4_int32_overflow_forcing(dev):
+    """Entries up to 2^20 with K = 2048: products reach 2^40 and sums wrap many times."""
+    M, N, K = 512, 384, 2048
+    a = synth.integers(11, (M, K), np.int32, -2 ** 20, 2 ** 20)
+    b = synth.integers(12, (K, N), np.int32, -2 ** 20, 2 ** 20)
+    c = synth.integers(13, (M, N), np.int32, -2 ** 31, 2 ** 31 - 1)
+    want = _exact_int32(65537, a, b, -3, c)
+    assert (np.abs(a.astype(np.float64) @ b.astype(np.float64)) > 2.0 ** 31).any()   # it really overflows
+    got = run(dev, "i32", 65537, a, 0, b, 0, -3, c)
+    assert np.array_equal(got, want)
+    # the C restatement of the reference's kernels wraps identically
+    assert np.array_equal(oracle.gemm("i32", 65537, a, 0, b, 0, -3, c), want)
