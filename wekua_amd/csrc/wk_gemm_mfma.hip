@@ -310,8 +310,9 @@ template <int ROWS, int BK, bool KCONTIG> struct SlabD {
     static constexpr int SIZE = KCONTIG ? ROWS * LD : BK * LD;
 };
 
-template <int BM, int BN, int BK, int WAVES_M, int WAVES_N, bool A_K, bool B_K, bool EDGE>
-__global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void gemm_f64_mfma_kernel(MArgs<double> g) {
+template <int BM, int BN, int BK, int WAVES_M, int WAVES_N, int OCC, bool A_K, bool B_K, bool EDGE>
+__global__ __launch_bounds__(WAVES_M *WAVES_N * 64) __attribute__((amdgpu_waves_per_eu(OCC)))
+void gemm_f64_mfma_kernel(MArgs<double> g) {
     constexpr int NT = WAVES_M * WAVES_N * 64;
     constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N;
     constexpr int FM = WM / 16, FN = WN / 16;
@@ -333,6 +334,8 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void gemm_f64_mfma_kernel(MA
     uint32_t tile_m, tile_n;
     tile_coords(g.tiles_m, g.tiles_n, tile_m, tile_n);
     const uint32_t m0 = tile_m * BM, n0 = tile_n * BN;
+    // one solo iteration = FM*FN*BK/4 matrix instructions of 64 clocks = FM*FN*BK/8 sleep units
+    startup_stagger(g.num_cus, OCC, FM * FN * BK / 8 > 0 ? FM * FN * BK / 8 : 1);
 
     f64x4 acc[FM][FN];
 #pragma unroll
@@ -409,10 +412,41 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void gemm_f64_mfma_kernel(MA
     };
 
     const uint32_t ktiles = (g.K + BK - 1) / BK;
+    constexpr int S = BK / 8;
+
+    // fragments of step s: lane holds k = 8*s + 2*lq + t, t = 0..1 (two instructions per 8 k)
+    auto read_frags = [&](int buf, int s, f64x2 *af, f64x2 *bf) {
+        const double *as = As + buf * SA::SIZE + (A_K ? (wm * WM + l16) * SA::LD : wm * WM + l16);
+        const double *bs = Bs + buf * SB::SIZE + (B_K ? (wn * WN + l16) * SB::LD : wn * WN + l16);
+#pragma unroll
+        for (int i = 0; i < FM; ++i) {
+            if constexpr (A_K) {
+                af[i] = *reinterpret_cast<const f64x2 *>(as + i * 16 * SA::LD + 8 * s + 2 * lq);
+            } else {
+#pragma unroll
+                for (int t = 0; t < 2; ++t) af[i][t] = as[(8 * s + 2 * lq + t) * SA::LD + i * 16];
+            }
+        }
+#pragma unroll
+        for (int j = 0; j < FN; ++j) {
+            if constexpr (B_K) {
+                bf[j] = *reinterpret_cast<const f64x2 *>(bs + j * 16 * SB::LD + 8 * s + 2 * lq);
+            } else {
+#pragma unroll
+                for (int t = 0; t < 2; ++t) bf[j][t] = bs[(8 * s + 2 * lq + t) * SB::LD + j * 16];
+            }
+        }
+    };
+
     load_a(0);
     load_b(0);
     store_ab(0);
     __syncthreads();
+
+    // same schedule as the f32 kernel: double-buffered fragments, hand-over in front of the last
+    // step's matrix instructions, next slab requested at the top of the iteration
+    f64x2 af[2][FM], bf[2][FN];
+    read_frags(0, 0, af[0], bf[0]);
 
     for (uint32_t kt = 0; kt < ktiles; ++kt) {
         const int cur = kt & 1;
@@ -421,29 +455,14 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void gemm_f64_mfma_kernel(MA
             load_a((kt + 1) * BK);
             load_b((kt + 1) * BK);
         }
-        const double *as = As + cur * SA::SIZE + (A_K ? (wm * WM + l16) * SA::LD : wm * WM + l16);
-        const double *bs = Bs + cur * SB::SIZE + (B_K ? (wn * WN + l16) * SB::LD : wn * WN + l16);
 #pragma unroll
-        for (int s = 0; s < BK / 8; ++s) {
-            // lane holds k = 8*s + 2*lq + t, t = 0..1  (two instructions per 8 k)
-            f64x2 af[FM], bf[FN];
-#pragma unroll
-            for (int i = 0; i < FM; ++i) {
-                if constexpr (A_K) {
-                    af[i] = *reinterpret_cast<const f64x2 *>(as + i * 16 * SA::LD + 8 * s + 2 * lq);
-                } else {
-#pragma unroll
-                    for (int t = 0; t < 2; ++t) af[i][t] = as[(8 * s + 2 * lq + t) * SA::LD + i * 16];
-                }
-            }
-#pragma unroll
-            for (int j = 0; j < FN; ++j) {
-                if constexpr (B_K) {
-                    bf[j] = *reinterpret_cast<const f64x2 *>(bs + j * 16 * SB::LD + 8 * s + 2 * lq);
-                } else {
-#pragma unroll
-                    for (int t = 0; t < 2; ++t) bf[j][t] = bs[(8 * s + 2 * lq + t) * SB::LD + j * 16];
-                }
+        for (int s = 0; s < S; ++s) {
+            if (s + 1 < S) {
+                read_frags(cur, s + 1, af[(s + 1) & 1], bf[(s + 1) & 1]);
+            } else if (more) {
+                store_ab(cur ^ 1);
+                __syncthreads();
+                read_frags(cur ^ 1, 0, af[(s + 1) & 1], bf[(s + 1) & 1]);
             }
 #pragma unroll
             for (int t = 0; t < 2; ++t)
@@ -451,10 +470,8 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void gemm_f64_mfma_kernel(MA
                 for (int i = 0; i < FM; ++i)
 #pragma unroll
                     for (int j = 0; j < FN; ++j)
-                        acc[i][j] = __builtin_amdgcn_mfma_f64_16x16x4f64(af[i][t], bf[j][t], acc[i][j], 0, 0, 0);
+                        acc[i][j] = __builtin_amdgcn_mfma_f64_16x16x4f64(af[s & 1][i][t], bf[s & 1][j][t], acc[i][j], 0, 0, 0);
         }
-        if (more) store_ab(cur ^ 1);
-        __syncthreads();
     }
 
     const double alpha = g.alpha, beta = g.beta;
@@ -537,10 +554,10 @@ int launch_f32(hipStream_t st, const GemmProblem &p, bool edge) {
 #undef WK_CASE
 }
 
-template <int BM, int BN, int BK, int WMS, int WNS, bool AK, bool BKC, bool EDGE>
+template <int BM, int BN, int BK, int WMS, int WNS, int OCC, bool AK, bool BKC, bool EDGE>
 int launch_f64_one(hipStream_t st, const GemmProblem &p) {
     constexpr size_t lds = 2 * (SlabD<BM, BK, AK>::SIZE + SlabD<BN, BK, BKC>::SIZE) * sizeof(double);
-    auto kern = gemm_f64_mfma_kernel<BM, BN, BK, WMS, WNS, AK, BKC, EDGE>;
+    auto kern = gemm_f64_mfma_kernel<BM, BN, BK, WMS, WNS, OCC, AK, BKC, EDGE>;
     static int attr_rc = set_lds(kern, lds);
     if (attr_rc) return attr_rc;
     MArgs<double> g = make_args<double>(p, BM, BN);
@@ -548,12 +565,12 @@ int launch_f64_one(hipStream_t st, const GemmProblem &p) {
     return launch_status();
 }
 
-template <int BM, int BN, int BK, int WMS, int WNS>
+template <int BM, int BN, int BK, int WMS, int WNS, int OCC>
 int launch_f64(hipStream_t st, const GemmProblem &p, bool edge) {
     const int sel = (p.op_a ? 0 : 2) | (p.op_b ? 1 : 0);
 #define WK_CASE(AK, BKC)                                                                                   \
-    return edge ? launch_f64_one<BM, BN, BK, WMS, WNS, AK, BKC, true>(st, p)                               \
-                : launch_f64_one<BM, BN, BK, WMS, WNS, AK, BKC, false>(st, p)
+    return edge ? launch_f64_one<BM, BN, BK, WMS, WNS, OCC, AK, BKC, true>(st, p)                               \
+                : launch_f64_one<BM, BN, BK, WMS, WNS, OCC, AK, BKC, false>(st, p)
     switch (sel) {
     case 0: WK_CASE(false, false);
     case 1: WK_CASE(false, true);
@@ -573,8 +590,9 @@ const VariantDesc k_variants[] = {
     {"mfma_f32_256x128", WK_F32, 256, 128, 16, &launch_f32<256, 128, 16, 2, 2, 2>},
     {"mfma_f32_128x128", WK_F32, 128, 128, 16, &launch_f32<128, 128, 16, 2, 2, 3>},
     {"mfma_f32_64x64", WK_F32, 64, 64, 16, &launch_f32<64, 64, 16, 2, 2, 4>},
-    {"mfma_f64_128x128", WK_F64, 128, 128, 16, &launch_f64<128, 128, 16, 2, 2>},
-    {"mfma_f64_64x64", WK_F64, 64, 64, 16, &launch_f64<64, 64, 16, 2, 2>},
+    {"mfma_f64_128x128", WK_F64, 128, 128, 16, &launch_f64<128, 128, 16, 2, 2, 2>},
+    {"mfma_f64_64x64", WK_F64, 64, 64, 16, &launch_f64<64, 64, 16, 2, 2, 4>},
+    {"mfma_f64_128x64", WK_F64, 128, 64, 16, &launch_f64<128, 64, 16, 2, 2, 3>},
 };
 constexpr int k_num_variants = sizeof(k_variants) / sizeof(k_variants[0]);
 
