@@ -41,30 +41,60 @@ def read_traffic(name: str):
         return None
 
 
-def gemm_leg(dev, raw, synth, n, steps, warmup):
+def gemm_leg(wk, synth, n, steps, warmup):
+    """The headline call through the reference-shaped API: Tensor.alloc + memory.readFromBuffer, then
+    `steps` calls of blas.gemm(pipeline, 1.5, A, N, B, N, 0.5, C, null) on one pipeline."""
     rd = np.float32
     t0 = time.time()
     a = synth.uniform(synth.config_seed(3, 0), (n, n), rd)
     b = synth.uniform(synth.config_seed(3, 1), (n, n), rd)
     c = synth.uniform(synth.config_seed(3, 2), (n, n), rd)
-    dA, dB, dC = dev.upload(a), dev.upload(b), dev.upload(c)
-    log(f"[bench] gemm operands {n}x{n} f32 generated + uploaded in {time.time() - t0:.1f}s")
-    variant = dev.lib.wk_gemm_variant(raw.dtype_id("f32"), 0, 0, n, n, n, n, n, n, dA.ptr, dB.ptr, dC.ptr).decode()
+    ctx = wk.Context.initFromDeviceType(wk.DeviceType.all)
+    pipeline = wk.Pipeline.init(ctx.command_queues[0])
+    A = wk.Tensor.alloc("f32", ctx, pipeline, (n, n))
+    B = wk.Tensor.alloc("f32", ctx, pipeline, (n, n))
+    C = wk.Tensor.alloc("f32", ctx, pipeline, (n, n))
+    for t, h in ((A, a), (B, b), (C, c)):
+        wk.memory.readFromBuffer(pipeline, t, h)
+    pipeline.waitAndCleanup()
+    log(f"[bench] gemm operands {n}x{n} f32 generated + uploaded in {time.time() - t0:.1f}s "
+        f"(row pitch {A.row_pitch} elements)")
+    lib = wk._capi.load()
+    variant = lib.wk_gemm_variant(wk.dtype_id("f32"), 0, 0, n, n, n, A.row_pitch, B.row_pitch, C.row_pitch,
+                                  A.buffer, B.buffer, C.buffer).decode()
+    N_ = wk.blas.Operation.no_transpose
 
     def step():
-        dev.gemm("f32", 0, 0, n, n, n, 1.5, dA, n, dB, n, 0.5, dC, n)
+        wk.blas.gemm(pipeline, 1.5, A, N_, B, N_, 0.5, C, None)
 
     for _ in range(warmup):
         step()
-    dev.sync()
-    # timed region: exactly `steps` calls; wall clock for `value`, stream events for the kernel time
+    pipeline.waitAndCleanup()
+    # timed region: exactly `steps` calls.  Wall clock (sync on both sides) gives `value`; events
+    # recorded on the pipeline's own stream around the same launches give the kernel time.
+    stream = wk._lib().wkz_context_stream(ctx._h, 0)
+    device = wk._lib().wkz_context_device(ctx._h)
+    import ctypes
+    e0, e1 = ctypes.c_void_p(), ctypes.c_void_p()
+    wk._capi.check(lib.wk_event_create(device, ctypes.byref(e0)))
+    wk._capi.check(lib.wk_event_create(device, ctypes.byref(e1)))
     t0 = time.perf_counter()
-    kernel_ms = dev.time_stream_ms(step, steps)
-    dev.sync()
+    wk._capi.check(lib.wk_event_record(e0, stream))
+    for _ in range(steps):
+        step()
+    wk._capi.check(lib.wk_event_record(e1, stream))
+    pipeline.waitAndCleanup()
     wall_ms = (time.perf_counter() - t0) * 1e3 / steps
+    ms = ctypes.c_float()
+    wk._capi.check(lib.wk_event_elapsed_ms(e0, e1, ctypes.byref(ms)))
+    kernel_ms = ms.value / steps
+    lib.wk_event_destroy(e0)
+    lib.wk_event_destroy(e1)
     flops = 2.0 * n * n * n
-    for d in (dA, dB, dC):
-        d.free()
+    for t in (A, B, C):
+        t.release(pipeline)
+    pipeline.deinit()
+    ctx.deinit()
     return {
         "variant": variant, "wall_ms": wall_ms, "kernel_ms": kernel_ms,
         "tflops_wall": flops / wall_ms / 1e9, "tflops_kernel": flops / kernel_ms / 1e9,
@@ -114,19 +144,22 @@ def main():
     ap.add_argument("--axpy-log2n", type=int, default=28)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-rows", type=int, default=8192)
+    ap.add_argument("--calibrate", action="store_true",
+                    help="also launch the plain 1 GiB copy kernel a few times, so that a profiler run of this "
+                         "command holds a kernel of known HBM traffic to scale byte counters against")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build uses one GPU; --gpus N with N > 1 is not supported "
               "(the hot path has no cross-GPU exchange: see DESIGN.md on sharding)", file=sys.stderr)
         sys.exit(2)
 
-    from wekua_amd import raw, synth   # fails loudly if libwekua_hip.so is missing
+    import wekua_amd as wk                # fails loudly if the native libraries are missing
+    from wekua_amd import raw, synth
 
+    g = gemm_leg(wk, synth, args.n, args.steps, args.warmup)
     dev = raw.Device(0)
     props = dev.props()
     log(f"[bench] device: {props.name.decode()} {props.arch.decode()} CUs={props.compute_units}")
-
-    g = gemm_leg(dev, raw, synth, args.n, args.steps, args.warmup)
     log(f"[bench] gemm f32 {args.n}^3 [{g['variant']}]: {g['kernel_ms']:.3f} ms/launch (events), "
         f"{g['wall_ms']:.3f} ms/step (wall) -> {g['tflops_kernel']:.1f} TFLOP/s")
 
@@ -134,6 +167,15 @@ def main():
     ax64 = axpy_leg(dev, raw, synth, "f64", args.axpy_log2n, max(args.steps, 20), args.warmup)
     log(f"[bench] axpy f32 2^{args.axpy_log2n}: {ax['us']:.1f} us -> {ax['gbs']:.0f} GB/s; "
         f"f64: {ax64['us']:.1f} us -> {ax64['gbs']:.0f} GB/s")
+    if args.calibrate:
+        nbytes = 1 << 30
+        src, dst = dev.malloc(nbytes), dev.malloc(nbytes)
+        from wekua_amd._capi import check
+        check(dev.lib.wk_memset_async(dev.stream, src.ptr, 1, nbytes), "memset")
+        ms = dev.time_stream_ms(lambda: check(dev.lib.wk_copy_kernel(dev.stream, dst.ptr, src.ptr, nbytes), "copy"), 5)
+        log(f"[bench] calibration copy 1 GiB: {ms * 1e3:.1f} us -> {2 * nbytes / ms / 1e6:.0f} GB/s (read + write)")
+        src.free()
+        dst.free()
     dev.close()
 
     cpu = None

@@ -17,8 +17,8 @@
 //        are 4-byte reads, 32 consecutive lanes on consecutive addresses;
 //     both give lane l the k values k0 + KL*(l / ROWS) + t for t = 0..KL-1, so the two
 //     operands of one instruction always agree on k;
-//   * work-groups are renumbered so that the 8 XCDs (each with its own L2) get contiguous
-//     runs of tiles, and tiles are walked in groups of GROUP_M rows for L2 reuse;
+//   * tiles are walked in groups of GROUP_M = 8 tile rows, which with the round-robin dispatch
+//     of work-groups over the 8 XCDs makes all XCDs stream the same panel of B together;
 //   * the epilogue applies the reference's option semantics (src/blas/gemm.zig:500-501,
 //     591-602): store / alpha*acc / alpha*acc + beta*C_old.
 //
@@ -39,7 +39,6 @@ typedef double f64x2 __attribute__((ext_vector_type(2)));
 typedef double f64x4 __attribute__((ext_vector_type(4)));
 
 constexpr int GROUP_M = 8;
-constexpr int NUM_XCD = 8;
 
 template <typename T> struct MArgs {
     const T *A, *B;
@@ -67,11 +66,16 @@ __device__ __forceinline__ void startup_stagger(uint32_t num_cus, uint32_t occup
     for (uint32_t i = 0; i < n; ++i) __builtin_amdgcn_s_sleep(2); // 2 * 64 clocks
 }
 
-// blockIdx.x -> (tile_m, tile_n): XCD-contiguous renumbering, then grouped row-major walk.
+// blockIdx.x -> (tile_m, tile_n): grouped walk, GROUP_M tile rows at a time.
+// Work-groups are dealt to the 8 XCDs round-robin (work-group b runs on XCD b % 8), so with
+// GROUP_M = 8 every XCD owns one tile row of the group and all XCDs sweep the SAME columns of B at
+// the same time: B is fetched from HBM once per sweep and served to the other XCDs from the
+// shared 256 MB Infinity Cache, while the A panel of a tile row stays in that XCD's own L2.
+// Renumbering so that each XCD gets a compact 8x8 block of tiles (better per-XCD L2 reuse on
+// paper) was measured slower (130 vs 135-139 TFLOP/s at 8192^3) and with more L2 misses: the XCDs
+// then stream disjoint panels and together exceed the Infinity Cache.
 __device__ __forceinline__ void tile_coords(uint32_t tiles_m, uint32_t tiles_n, uint32_t &tm, uint32_t &tn) {
-    const uint32_t nb = gridDim.x;
-    uint32_t pid = blockIdx.x;
-    if ((nb % NUM_XCD) == 0) pid = (pid % NUM_XCD) * (nb / NUM_XCD) + pid / NUM_XCD;
+    const uint32_t pid = blockIdx.x;
     const uint32_t group_size = GROUP_M * tiles_n;
     const uint32_t group = pid / group_size;
     const uint32_t first_m = group * GROUP_M;
