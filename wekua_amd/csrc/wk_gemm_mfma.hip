@@ -22,11 +22,12 @@
 //   * the epilogue applies the reference's option semantics (src/blas/gemm.zig:500-501,
 //     591-602): store / alpha*acc / alpha*acc + beta*C_old.
 //
-// The EDGE instantiation bounds-checks every global access (ragged M, N, K, unaligned
-// leading dimensions); the interior instantiation assumes M % BM == N % BN == K % BK == 0
-// and 16-byte aligned rows.
+// The EDGE instantiation bounds-checks every global access (ragged M, N, K) and uses
+// element-aligned 16-byte loads, so odd leading dimensions keep full-width loads; the interior
+// instantiation assumes M % BM == N % BN == K % BK == 0 and 16-byte aligned rows.
 #include "wk_internal.hpp"
 
+#include <cstdlib>
 #include <cstring>
 
 using namespace wk;
@@ -37,6 +38,10 @@ typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 typedef double f64x2 __attribute__((ext_vector_type(2)));
 typedef double f64x4 __attribute__((ext_vector_type(4)));
+// 16-byte vectors that are only element-aligned: gfx950 global loads take any dword-aligned
+// address, so rows with an odd leading dimension still move 16 bytes per lane
+struct __attribute__((packed, aligned(4))) f32x4_u { f32x4 v; };
+struct __attribute__((packed, aligned(8))) f64x2_u { f64x2 v; };
 
 constexpr int GROUP_M = 8;
 
@@ -47,6 +52,7 @@ template <typename T> struct MArgs {
     uint32_t lda, ldb, ldc;
     uint32_t tiles_m, tiles_n;
     uint32_t num_cus; // compute units of the device (0 disables the start-up stagger)
+    uint32_t xcd_remap; // 1: renumber work-groups so that each XCD gets a contiguous run of tiles
     int epi;
     T alpha, beta;
 };
@@ -67,15 +73,16 @@ __device__ __forceinline__ void startup_stagger(uint32_t num_cus, uint32_t occup
 }
 
 // blockIdx.x -> (tile_m, tile_n): grouped walk, GROUP_M tile rows at a time.
-// Work-groups are dealt to the 8 XCDs round-robin (work-group b runs on XCD b % 8), so with
-// GROUP_M = 8 every XCD owns one tile row of the group and all XCDs sweep the SAME columns of B at
-// the same time: B is fetched from HBM once per sweep and served to the other XCDs from the
-// shared 256 MB Infinity Cache, while the A panel of a tile row stays in that XCD's own L2.
-// Renumbering so that each XCD gets a compact 8x8 block of tiles (better per-XCD L2 reuse on
-// paper) was measured slower (130 vs 135-139 TFLOP/s at 8192^3) and with more L2 misses: the XCDs
-// then stream disjoint panels and together exceed the Infinity Cache.
-__device__ __forceinline__ void tile_coords(uint32_t tiles_m, uint32_t tiles_n, uint32_t &tm, uint32_t &tn) {
-    const uint32_t pid = blockIdx.x;
+// Work-groups are dealt to the 8 XCDs round-robin (work-group b runs on XCD b % 8; checked by
+// reading the XCC_ID register).  Without renumbering and with GROUP_M = 8 every XCD owns one tile
+// row of the group and all XCDs sweep the SAME columns of B at the same time: B is fetched from
+// HBM once per sweep and served to the other XCDs from the shared 256 MB Infinity Cache, while
+// the A panel of a tile row stays in that XCD's own L2.  That is the right order for launches of
+// several rounds.  With renumbering (remap) each XCD gets a compact block of tiles, which wins
+// when the whole launch is resident at once and lives in the L2s.
+__device__ __forceinline__ void tile_coords(uint32_t tiles_m, uint32_t tiles_n, uint32_t &tm, uint32_t &tn, uint32_t remap = 0) {
+    uint32_t pid = blockIdx.x;
+    if (remap && (gridDim.x % 8) == 0) pid = (pid % 8) * (gridDim.x / 8) + pid / 8;
     const uint32_t group_size = GROUP_M * tiles_n;
     const uint32_t group = pid / group_size;
     const uint32_t first_m = group * GROUP_M;
@@ -115,7 +122,7 @@ void gemm_f32_mfma_kernel(MArgs<float> g) {
     const int l32 = lane & 31, lhi = lane >> 5;
 
     uint32_t tile_m, tile_n;
-    tile_coords(g.tiles_m, g.tiles_n, tile_m, tile_n);
+    tile_coords(g.tiles_m, g.tiles_n, tile_m, tile_n, g.xcd_remap);
     const uint32_t m0 = tile_m * BM, n0 = tile_n * BN;
     // one solo iteration = FM*FN*BK/2 matrix instructions of 64 clocks = FM*FN*BK/4 sleep units
     startup_stagger(g.num_cus, OCC, FM * FN * BK / 4);
@@ -156,8 +163,8 @@ void gemm_f32_mfma_kernel(MArgs<float> g) {
             } else {
                 f32x4 v = {0.f, 0.f, 0.f, 0.f};
                 if (r < r_lim) {
-                    if (c + 3 < c_lim && ((reinterpret_cast<uintptr_t>(p) & 15u) == 0)) {
-                        v = *reinterpret_cast<const f32x4 *>(p);
+                    if (c + 3 < c_lim) {
+                        v = reinterpret_cast<const f32x4_u *>(p)->v;
                     } else {
                         if (c + 0 < c_lim) v[0] = p[0];
                         if (c + 1 < c_lim) v[1] = p[1];
@@ -336,7 +343,7 @@ void gemm_f64_mfma_kernel(MArgs<double> g) {
     const int l16 = lane & 15, lq = lane >> 4; // lq = 0..3
 
     uint32_t tile_m, tile_n;
-    tile_coords(g.tiles_m, g.tiles_n, tile_m, tile_n);
+    tile_coords(g.tiles_m, g.tiles_n, tile_m, tile_n, g.xcd_remap);
     const uint32_t m0 = tile_m * BM, n0 = tile_n * BN;
     // one solo iteration = FM*FN*BK/4 matrix instructions of 64 clocks = FM*FN*BK/8 sleep units
     startup_stagger(g.num_cus, OCC, FM * FN * BK / 8 > 0 ? FM * FN * BK / 8 : 1);
@@ -373,8 +380,8 @@ void gemm_f64_mfma_kernel(MArgs<double> g) {
             } else {
                 f64x2 v = {0.0, 0.0};
                 if (r < r_lim) {
-                    if (c + 1 < c_lim && ((reinterpret_cast<uintptr_t>(p) & 15u) == 0)) {
-                        v = *reinterpret_cast<const f64x2 *>(p);
+                    if (c + 1 < c_lim) {
+                        v = reinterpret_cast<const f64x2_u *>(p)->v;
                     } else {
                         if (c + 0 < c_lim) v[0] = p[0];
                         if (c + 1 < c_lim) v[1] = p[1];
@@ -499,14 +506,6 @@ void gemm_f64_mfma_kernel(MArgs<double> g) {
 
 // ------------------------------------------------------------------------------ dispatch ---
 
-struct Variant {
-    const char *name;
-    int dtype;
-    int bm, bn, bk;
-    size_t lds_bytes[4]; // per (op_a, op_b)
-    int (*launch)(hipStream_t, const GemmProblem &, bool edge);
-};
-
 template <typename T> MArgs<T> make_args(const GemmProblem &p, int bm, int bn) {
     MArgs<T> g;
     g.A = static_cast<const T *>(p.A);
@@ -517,6 +516,11 @@ template <typename T> MArgs<T> make_args(const GemmProblem &p, int bm, int bn) {
     g.tiles_m = (uint32_t)((p.M + bm - 1) / bm);
     g.tiles_n = (uint32_t)((p.N + bn - 1) / bn);
     g.num_cus = p.num_cus;
+    // Small launches (every tile resident at once) run out of the per-XCD L2: give each XCD a
+    // compact run of tiles.  Large launches stream from the shared Infinity Cache: keep the XCDs on
+    // the same B panel (see tile_coords).  Measured: 1024^3 f32 48 -> 62 TFLOP/s with the
+    // renumbering, 8192^3 138 -> 131 with it.
+    g.xcd_remap = (uint64_t)g.tiles_m * g.tiles_n <= 4ull * (p.num_cus ? p.num_cus : 256u) ? 1u : 0u;
     g.epi = p.epi;
     std::memcpy(&g.alpha, p.alpha, sizeof(T));
     std::memcpy(&g.beta, p.beta, sizeof(T));
@@ -587,16 +591,17 @@ int launch_f64(hipStream_t st, const GemmProblem &p, bool edge) {
 struct VariantDesc {
     const char *name;
     int dtype, bm, bn, bk;
+    double efficiency; // relative matrix-pipe efficiency of the tile shape (0: never auto-selected)
     int (*launch)(hipStream_t, const GemmProblem &, bool);
 };
 
 const VariantDesc k_variants[] = {
-    {"mfma_f32_256x128", WK_F32, 256, 128, 16, &launch_f32<256, 128, 16, 2, 2, 2>},
-    {"mfma_f32_128x128", WK_F32, 128, 128, 16, &launch_f32<128, 128, 16, 2, 2, 3>},
-    {"mfma_f32_64x64", WK_F32, 64, 64, 16, &launch_f32<64, 64, 16, 2, 2, 4>},
-    {"mfma_f64_128x128", WK_F64, 128, 128, 16, &launch_f64<128, 128, 16, 2, 2, 2>},
-    {"mfma_f64_64x64", WK_F64, 64, 64, 16, &launch_f64<64, 64, 16, 2, 2, 4>},
-    {"mfma_f64_128x64", WK_F64, 128, 64, 16, &launch_f64<128, 64, 16, 2, 2, 3>},
+    {"mfma_f32_256x128", WK_F32, 256, 128, 16, 1.00, &launch_f32<256, 128, 16, 2, 2, 2>},
+    {"mfma_f32_128x128", WK_F32, 128, 128, 16, 0.96, &launch_f32<128, 128, 16, 2, 2, 3>},
+    {"mfma_f32_64x64", WK_F32, 64, 64, 16, 0.85, &launch_f32<64, 64, 16, 2, 2, 4>},
+    {"mfma_f64_128x128", WK_F64, 128, 128, 16, 1.00, &launch_f64<128, 128, 16, 2, 2, 2>},
+    {"mfma_f64_64x64", WK_F64, 64, 64, 16, 0.92, &launch_f64<64, 64, 16, 2, 2, 4>},
+    {"mfma_f64_128x64", WK_F64, 128, 64, 16, 0.97, &launch_f64<128, 64, 16, 2, 2, 3>},
 };
 constexpr int k_num_variants = sizeof(k_variants) / sizeof(k_variants[0]);
 
@@ -619,20 +624,31 @@ int wk::gemm_mfma_variant_dtype(int variant) {
     return (variant >= 0 && variant < k_num_variants) ? k_variants[variant].dtype : -1;
 }
 
-// Largest macro tile that still yields at least ~2 work-groups per CU; small problems take
-// smaller tiles so that the 256 CUs are not left idle.
+// Kernel choice by a small cost model.  The matrix pipes of a CU are saturated by the work-groups
+// resident on it, so a launch takes about (tiles on the busiest CU) x (tile area / efficiency):
+//     cost = ceil(tiles / CUs) * BM * BN / efficiency
+// with the efficiency of each macro tile relative to the largest measured at 4096^3 on MI355X
+// (f32: 122 / 118 / 106 TFLOP/s; f64 similarly).  This picks big tiles for big problems, small
+// tiles when the big ones would leave CUs idle (1024^3, tall-skinny) or quantise badly
+// (4097 x 4095: 544 tiles of 256x128 put three tiles on some CUs and two on the rest).
 int wk::gemm_mfma_pick(const GemmProblem &p) {
     if (p.dtype != WK_F32 && p.dtype != WK_F64) return -1;
     if (p.M > 0x7fffffffull || p.N > 0x7fffffffull || p.K > 0x7fffffffull || p.lda > 0x7fffffffull ||
         p.ldb > 0x7fffffffull || p.ldc > 0x7fffffffull)
         return -1;
+    const double cus = p.num_cus ? (double)p.num_cus : 256.0;
     int best = -1;
+    double best_cost = 0.0;
     for (int v = 0; v < k_num_variants; ++v) {
-        if (k_variants[v].dtype != p.dtype) continue;
-        const uint64_t tiles = ((p.M + k_variants[v].bm - 1) / k_variants[v].bm) *
-                               ((p.N + k_variants[v].bn - 1) / k_variants[v].bn);
-        best = v;
-        if (tiles >= 512) break;
+        const VariantDesc &d = k_variants[v];
+        if (d.dtype != p.dtype || d.efficiency <= 0.0) continue;
+        const double tiles = (double)((p.M + d.bm - 1) / d.bm) * (double)((p.N + d.bn - 1) / d.bn);
+        const double rounds = (double)(uint64_t)((tiles + cus - 1.0) / cus);
+        const double cost = rounds * d.bm * d.bn / d.efficiency;
+        if (best < 0 || cost < best_cost) {
+            best = v;
+            best_cost = cost;
+        }
     }
     return best;
 }
