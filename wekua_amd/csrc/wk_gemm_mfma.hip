@@ -100,7 +100,7 @@ template <int ROWS, int BK, bool KCONTIG> struct Slab {
     static constexpr int SIZE = KCONTIG ? ROWS * LD : BK * LD;
 };
 
-template <int BM, int BN, int BK, int WAVES_M, int WAVES_N, int OCC, bool LOAD_AHEAD, bool A_K, bool B_K, bool EDGE>
+template <int BM, int BN, int BK, int WAVES_M, int WAVES_N, int OCC, bool A_K, bool B_K, bool EDGE>
 __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) __attribute__((amdgpu_waves_per_eu(OCC)))
 void gemm_f32_mfma_kernel(MArgs<float> g) {
     constexpr int NT = WAVES_M * WAVES_N * 64;
@@ -135,7 +135,7 @@ void gemm_f32_mfma_kernel(MArgs<float> g) {
 #pragma unroll
             for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
 
-    f32x4 ra[A_V4], rb[B_V4];
+    f32x4 ra[A_V4], rb[B_V4]; // staging registers: global -> LDS
 
     // ---- global -> registers -----------------------------------------------------------
     // KCONTIG: slab is ROWS x BK, q -> (row = q / (BK/4), c4 = q % (BK/4)), address row*ld + k0 + 4*c4
@@ -193,11 +193,9 @@ void gemm_f32_mfma_kernel(MArgs<float> g) {
     };
 
     using std::integral_constant;
-    auto load_a = [&](uint32_t k0) {
+    auto load_ab = [&](uint32_t k0) {
         gload(ra, g.A, g.lda, m0, g.M, k0, integral_constant<bool, A_K>{}, integral_constant<int, BM>{},
               integral_constant<int, A_V4>{});
-    };
-    auto load_b = [&](uint32_t k0) {
         gload(rb, g.B, g.ldb, n0, g.N, k0, integral_constant<bool, B_K>{}, integral_constant<int, BN>{},
               integral_constant<int, B_V4>{});
     };
@@ -235,37 +233,25 @@ void gemm_f32_mfma_kernel(MArgs<float> g) {
         }
     };
 
-    load_a(0);
-    load_b(0);
+    load_ab(0);
     store_ab(0);
-    if (LOAD_AHEAD && ktiles > 1) {
-        load_a(BK);
-        load_b(BK);
-    }
     __syncthreads();
 
     // Fragment registers are double-buffered: the LDS reads for step s+1 are issued before the
     // matrix instructions of step s, and the slab hand-over (LDS store of the next slab, barrier,
-    // first fragment read of the next slab) sits in front of the last step's matrix
-    // instructions, so that LDS latency and barrier skew are covered by matrix work of the
-    // same wavefront instead of relying on another wavefront to fill the pipe.
+    // first fragment reload) sits in front of the last step's matrix instructions, so that LDS
+    // latency and barrier skew are covered by matrix work of the same wavefront.
+    // Slab kt+1 is requested from global memory at the top of iteration kt.  Requesting it a whole
+    // iteration (refill right after the hand-over) or one and a half iterations earlier (a second
+    // staging register set) was measured and changes nothing (134-138 TFLOP/s at 8192^3 in all
+    // three schedules), so the simplest one is kept.
     f32x4 af[2][FM], bf[2][FN];
     read_frags(0, 0, af[0], bf[0]);
 
-    // Global prefetch, two schedules (LOAD_AHEAD):
-    //   false: slab kt+1 is requested at the top of iteration kt and written to LDS in that
-    //          iteration's hand-over (half an iteration of matrix work covers the latency);
-    //   true : the staging registers are refilled with slab kt+2 right after the hand-over,
-    //          from inside the last step's matrix work (a whole iteration covers the latency;
-    //          the refill is unconditional -- the tail re-fetches the final slab -- so that
-    //          the loop body stays one basic block).
     for (uint32_t kt = 0; kt < ktiles; ++kt) {
         const int cur = kt & 1;
         const bool more = kt + 1 < ktiles;
-        if (!LOAD_AHEAD && more) {
-            load_a((kt + 1) * BK);
-            load_b((kt + 1) * BK);
-        }
+        if (more) load_ab((kt + 1) * BK);
 #pragma unroll
         for (int s = 0; s < S; ++s) {
             if (s + 1 < S) {
@@ -276,18 +262,12 @@ void gemm_f32_mfma_kernel(MArgs<float> g) {
                 read_frags(cur ^ 1, 0, af[(s + 1) & 1], bf[(s + 1) & 1]);
             }
 #pragma unroll
-            for (int t = 0; t < 4; ++t) {
+            for (int t = 0; t < 4; ++t)
 #pragma unroll
                 for (int i = 0; i < FM; ++i)
 #pragma unroll
                     for (int j = 0; j < FN; ++j)
                         acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(af[s & 1][i][t], bf[s & 1][j][t], acc[i][j], 0, 0, 0);
-                if (LOAD_AHEAD && s == S - 1 && t == 0) {
-                    const uint32_t knext = min(kt + 2, ktiles - 1) * BK;
-                    load_a(knext);
-                    load_b(knext);
-                }
-            }
         }
     }
 
@@ -536,10 +516,10 @@ template <typename K> int set_lds(K kernel, size_t bytes) {
     return WK_OK;
 }
 
-template <int BM, int BN, int BK, int WMS, int WNS, int OCC, bool LA, bool AK, bool BKC, bool EDGE>
+template <int BM, int BN, int BK, int WMS, int WNS, int OCC, bool AK, bool BKC, bool EDGE>
 int launch_f32_one(hipStream_t st, const GemmProblem &p) {
     constexpr size_t lds = 2 * (Slab<BM, BK, AK>::SIZE + Slab<BN, BK, BKC>::SIZE) * sizeof(float);
-    auto kern = gemm_f32_mfma_kernel<BM, BN, BK, WMS, WNS, OCC, LA, AK, BKC, EDGE>;
+    auto kern = gemm_f32_mfma_kernel<BM, BN, BK, WMS, WNS, OCC, AK, BKC, EDGE>;
     static int attr_rc = set_lds(kern, lds);
     if (attr_rc) return attr_rc;
     MArgs<float> g = make_args<float>(p, BM, BN);
@@ -547,12 +527,12 @@ int launch_f32_one(hipStream_t st, const GemmProblem &p) {
     return launch_status();
 }
 
-template <int BM, int BN, int BK, int WMS, int WNS, int OCC, bool LA = false>
+template <int BM, int BN, int BK, int WMS, int WNS, int OCC>
 int launch_f32(hipStream_t st, const GemmProblem &p, bool edge) {
     const int sel = (p.op_a ? 0 : 2) | (p.op_b ? 1 : 0); // bit1: A k-contiguous, bit0: B k-contiguous
 #define WK_CASE(AK, BKC)                                                                                   \
-    return edge ? launch_f32_one<BM, BN, BK, WMS, WNS, OCC, LA, AK, BKC, true>(st, p)                          \
-                : launch_f32_one<BM, BN, BK, WMS, WNS, OCC, LA, AK, BKC, false>(st, p)
+    return edge ? launch_f32_one<BM, BN, BK, WMS, WNS, OCC, AK, BKC, true>(st, p)                          \
+                : launch_f32_one<BM, BN, BK, WMS, WNS, OCC, AK, BKC, false>(st, p)
     switch (sel) {
     case 0: WK_CASE(false, false);
     case 1: WK_CASE(false, true);
