@@ -171,6 +171,43 @@ const char *wk_gemm_variant(int dtype, int op_a, int op_b, uint64_t M, uint64_t 
  * Returns WK_E_INVALID_VALUE for an unknown name. */
 int wk_gemm_force_variant(const char *name);
 
+/* ---- around the hot path: what one MLP training step needs besides gemm / axpy -----------------
+ * (f32 and f64 only; every tensor is a logical {depth, rows, cols} region with its own pitches) */
+enum { WK_ACT_NONE = -1, WK_ACT_SIGMOID = 0, WK_ACT_TANH = 1 };
+/* math.dot, the in-place Hadamard product x *= y: src/math/basic.zig:18-77, kernels/dot.cl */
+int  wk_hadamard(wk_stream *s, int dtype, const uint64_t shape3[3], void *x, uint64_t x_row_pitch, uint64_t x_slice_pitch,
+                 const void *y, uint64_t y_row_pitch, uint64_t y_slice_pitch);
+/* Activation.run in place: Sigmoid 1/(1+exp(-x)) (src/nn/activation/kernels/sigmoid.cl:3-19),
+ * Tanh (src/nn/activation/tanh.zig:16-31 -> math.tanh, src/math/kernels/trig.cl) */
+int  wk_activation(wk_stream *s, int dtype, int kind, const uint64_t shape3[3], void *x, uint64_t row_pitch, uint64_t slice_pitch);
+/* Activation.getDerivative from the activation OUTPUT y: sigmoid_dev y(1-y) (sigmoid.cl:21-38),
+ * tanh_dev 1-y^2 (src/nn/activation/kernels/tanh.cl) */
+int  wk_activation_dev(wk_stream *s, int dtype, int kind, const uint64_t shape3[3], const void *out, uint64_t out_row_pitch,
+                       uint64_t out_slice_pitch, void *dev, uint64_t dev_row_pitch, uint64_t dev_slice_pitch);
+/* Linear.addBias (src/nn/layer/kernels/bias.cl: out[r][c] += bias[c]) fused with the activation that
+ * follows it in Linear.forward (src/nn/layer/linear.zig:480-525).  bias may be NULL, kind WK_ACT_NONE. */
+int  wk_bias_activation(wk_stream *s, int dtype, int kind, uint64_t rows, uint64_t cols, void *out, uint64_t out_pitch,
+                        const void *bias);
+/* Linear.getBiasSensitivity: bias_grad[c] = sum_r sens[r][c] (src/nn/layer/kernels/bias_step.cl) */
+int  wk_bias_step(wk_stream *s, int dtype, uint64_t rows, uint64_t cols, const void *sens, uint64_t pitch, void *bias_grad);
+/* loss.mse kernel: err = expected - output; error = err^2; dev = -2*err when dev != NULL
+ * (src/nn/loss/kernels/mse.cl:3-35, src/nn/loss/mse.zig:63-132) */
+int  wk_mse(wk_stream *s, int dtype, const uint64_t shape3[3], const void *output, uint64_t out_row_pitch, uint64_t out_slice_pitch,
+            const void *expected, uint64_t exp_row_pitch, uint64_t exp_slice_pitch, void *error, uint64_t err_row_pitch,
+            uint64_t err_slice_pitch, void *dev, uint64_t dev_row_pitch, uint64_t dev_slice_pitch);
+/* math.sum / math.mean (src/math/basic.zig:128-244): scale * sum of the logical elements into one
+ * element at dev_result; workspace holds wk_sum_workspace_bytes(dtype) bytes of device memory. */
+size_t wk_sum_workspace_bytes(int dtype);
+int  wk_sum(wk_stream *s, int dtype, const uint64_t shape3[3], const void *x, uint64_t row_pitch, uint64_t slice_pitch,
+            void *workspace, void *dev_result, double scale);
+/* Adam update.  The reference's Zig tree has no Adam (src/nn/optimizers/adam.zig is empty); this is
+ * the textbook rule with the reference's sibling optimizers' epsilon placement (rmsprop.cl:54):
+ * m = b1 m + (1-b1) g; v = b2 v + (1-b2) g^2; w -= lr/(1-b1^t) * m / (sqrt(v/(1-b2^t)) + eps).
+ * m and v share one layout. */
+int  wk_adam_step(wk_stream *s, int dtype, const uint64_t shape3[3], void *w, uint64_t w_row_pitch, uint64_t w_slice_pitch,
+                  const void *g, uint64_t g_row_pitch, uint64_t g_slice_pitch, void *m, void *v, uint64_t mv_row_pitch,
+                  uint64_t mv_slice_pitch, double lr, double beta1, double beta2, double eps, uint64_t step);
+
 /* A plain device-to-device streaming copy kernel of known size, used only to calibrate
  * profiler byte counters against a known amount of traffic. */
 int wk_copy_kernel(wk_stream *s, void *dst, const void *src, size_t bytes);

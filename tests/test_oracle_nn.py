@@ -1,0 +1,170 @@
+"""CPU: pins the numpy restatement of the nn kernels and of the MLP training step (oracle/nn.py)
+against the reference's own known answers where it holds any, and against mathematics elsewhere
+(central differences, closed forms, brute force on tiny inputs)."""
+import numpy as np
+import pytest
+
+from oracle import nn as onn
+
+FLOATS = [np.float32, np.float64]
+
+
+# ---- the reference's own known answers -----------------------------------------------------------
+
+@pytest.mark.parametrize("dt", FLOATS)
+def test_dot_known_answer(dt):
+    # src/math/basic.zig:258-320: [1,2,3,4] * [2,3,4,5] = [2,6,12,20]
+    x = np.arange(1, 5, dtype=dt)
+    y = np.arange(2, 6, dtype=dt)
+    assert np.array_equal(onn.hadamard(x, y), np.array([2, 6, 12, 20], dtype=dt))
+
+
+@pytest.mark.parametrize("dt", FLOATS)
+def test_sum_and_mean_known_answers(dt):
+    # src/math/basic.zig:322-366: sum [1..5] = 15;  :368-420: mean [2,4,6,8] = 5
+    assert onn.tensor_sum(np.arange(1, 6, dtype=dt)) == dt(15)
+    assert abs(float(onn.tensor_mean(np.array([2, 4, 6, 8], dtype=dt))) - 5.0) < 1e-5
+
+
+@pytest.mark.parametrize("dt", FLOATS)
+def test_tanh_known_answer(dt):
+    # src/math/trig.zig:397-450: tanh(0) = 0, tanh(1) ~ 0.7616 within 1e-4
+    got = onn.activation(onn.TANH, np.array([0, 1], dtype=dt))
+    assert abs(float(got[0])) < 1e-4 and abs(float(got[1]) - 0.7616) < 1e-4
+
+
+# ---- mathematics ---------------------------------------------------------------------------------
+
+def test_sum_matches_exact_rational_sum():
+    rng = np.random.default_rng(1)
+    x = rng.integers(-1000, 1000, size=(7, 13)).astype(np.float64)  # exactly representable
+    assert onn.tensor_sum(x) == float(sum(int(v) for v in x.ravel()))
+    assert onn.tensor_mean(x) == onn.tensor_sum(x) / x.size
+
+
+def test_sigmoid_special_values_and_symmetry():
+    x = np.array([-30.0, -2.0, 0.0, 2.0, 30.0])
+    y = onn.activation(onn.SIGMOID, x)
+    assert y[2] == 0.5
+    assert np.allclose(y + y[::-1], 1.0, atol=1e-15)  # s(x) + s(-x) = 1
+    assert np.allclose(y[3], 1.0 / (1.0 + np.exp(-2.0)))
+    assert np.allclose(np.log(y[3] / (1 - y[3])), 2.0)  # logit inverts it
+
+
+@pytest.mark.parametrize("kind", [onn.SIGMOID, onn.TANH])
+def test_activation_derivative_against_central_differences(kind):
+    x = np.linspace(-3, 3, 41)
+    h = 1e-6
+    numeric = (onn.activation(kind, x + h) - onn.activation(kind, x - h)) / (2 * h)
+    assert np.allclose(onn.activation_dev(kind, onn.activation(kind, x)), numeric, atol=1e-9)
+
+
+def test_bias_and_bias_step_brute_force():
+    rng = np.random.default_rng(2)
+    out = rng.standard_normal((5, 3))
+    bias = rng.standard_normal(3)
+    got = onn.bias_add(out, bias)
+    for r in range(5):
+        for c in range(3):
+            assert got[r, c] == out[r, c] + bias[c]
+    ints = rng.integers(-50, 50, size=(6, 4)).astype(np.float64)
+    assert np.array_equal(onn.bias_step(ints), np.array([sum(ints[:, c]) for c in range(4)]))
+
+
+def test_mse_brute_force():
+    out = np.array([[0.25, 1.0], [2.0, -1.0]])
+    exp = np.array([[1.0, 1.0], [0.0, 0.5]])
+    err, dev = onn.mse(out, exp)
+    assert np.array_equal(err, np.array([[0.5625, 0.0], [4.0, 2.25]]))
+    assert np.array_equal(dev, np.array([[-1.5, 0.0], [4.0, -3.0]]))  # d/d out of (exp - out)^2
+
+
+def _random_layers(rng, sizes, acts, deep=1, bias=True):
+    layers = []
+    for (i, o), act in zip(zip(sizes[:-1], sizes[1:]), acts):
+        w = [rng.uniform(-0.7, 0.7, size=(o, i if d == 0 else o)) for d in range(deep)]
+        b = [rng.uniform(-0.3, 0.3, size=o) if bias else None for _ in range(deep)]
+        layers.append({"w": w, "b": b, "act": act})
+    return layers
+
+
+def _loss(x, expected, layers):
+    out = onn.mlp_forward(x, layers)[-1][-1]
+    return float(np.sum((expected - out) ** 2))
+
+
+@pytest.mark.parametrize("deep", [1, 2])
+def test_network_gradients_against_central_differences(deep):
+    """The reference's loss derivative is -2(expected - output) without a 1/N factor, so backward
+    yields the gradient of the SUM of squared errors."""
+    rng = np.random.default_rng(3)
+    sizes, acts = [3, 5, 4, 2], [onn.TANH, onn.SIGMOID, onn.TANH]
+    layers = _random_layers(rng, sizes, acts, deep=deep)
+    x = rng.standard_normal((6, 3))
+    expected = rng.uniform(-1, 1, size=(6, 2))
+    caches = onn.mlp_forward(x, layers)
+    _, sens = onn.mse(caches[-1][-1], expected)
+    grads = onn.mlp_backward(x, layers, caches, sens)
+    h = 1e-6
+    for li, layer in enumerate(layers):
+        for d in range(deep):
+            for kind, params, got in (("w", layer["w"], grads[li][0]), ("b", layer["b"], grads[li][1])):
+                p = params[d]
+                numeric = np.zeros_like(p)
+                it = np.nditer(p, flags=["multi_index"])
+                for _ in it:
+                    idx = it.multi_index
+                    keep = p[idx]
+                    p[idx] = keep + h
+                    up = _loss(x, expected, layers)
+                    p[idx] = keep - h
+                    down = _loss(x, expected, layers)
+                    p[idx] = keep
+                    numeric[idx] = (up - down) / (2 * h)
+                assert np.allclose(got[d], numeric, rtol=1e-6, atol=1e-8), (li, d, kind)
+
+
+def test_layer_without_activation_gets_zero_gradients():
+    # linear.zig:606-611: the sensitivity is multiplied by the derivative tensor, which nothing fills
+    rng = np.random.default_rng(4)
+    layers = _random_layers(rng, [3, 2], [None])
+    x = rng.standard_normal((4, 3))
+    caches = onn.mlp_forward(x, layers)
+    _, sens = onn.mse(caches[-1][-1], np.zeros((4, 2)))
+    g, bg = onn.mlp_backward(x, layers, caches, sens)[0]
+    assert not g[0].any() and not bg[0].any()
+
+
+def test_gd_step_reduces_the_loss_and_equals_axpy():
+    rng = np.random.default_rng(5)
+    layers = _random_layers(rng, [2, 10, 1], [onn.SIGMOID, onn.SIGMOID])
+    x = np.array([[1, 1], [0, 1], [1, 0], [0, 0]], dtype=np.float64)
+    y = np.array([[0], [1], [1], [0]], dtype=np.float64)
+    before = _loss(x, y, layers)
+    w0 = layers[0]["w"][0].copy()
+    _, _, grads, _ = onn.mlp_step(x, y, layers, ("gd", 0.1))
+    assert np.array_equal(layers[0]["w"][0], w0 + (-0.1) * grads[0][0][0])
+    assert _loss(x, y, layers) < before
+    for _ in range(3000):  # examples/xor_neural_network.zig trains this network with GD
+        onn.mlp_step(x, y, layers, ("gd", 1.0))
+    assert _loss(x, y, layers) < 0.05
+
+
+@pytest.mark.parametrize("dt", FLOATS)
+def test_adam_first_step_closed_form(dt):
+    # m0 = v0 = 0: m_hat = g, v_hat = g^2, so dw = -lr * g / (|g| + eps)
+    g = np.array([0.5, -2.0, 1e-3, 3.0], dtype=dt)
+    w = np.ones(4, dtype=dt)
+    lr, eps = 1e-3, 1e-8
+    w1, m, v = onn.adam_update(w, g, np.zeros(4, dt), np.zeros(4, dt), lr, 0.9, 0.999, eps, 1)
+    want = 1.0 - lr * g.astype(np.float64) / (np.abs(g.astype(np.float64)) + eps)
+    assert np.allclose(w1, want, rtol=4 * np.finfo(dt).eps)
+    assert np.allclose(m, 0.1 * g, rtol=1e-6) and np.allclose(v, 0.001 * g * g, rtol=1e-5)
+
+
+def test_adam_converges_on_a_quadratic():
+    w = np.array([5.0, -3.0])
+    m = v = np.zeros(2)
+    for t in range(1, 4001):
+        w, m, v = onn.adam_update(w, 2 * w, m, v, 1e-2, 0.9, 0.999, 1e-8, t)
+    assert np.all(np.abs(w) < 1e-3)

@@ -81,6 +81,30 @@ HOST_SIGNATURES = {
     "wkz_packed_deinit": (ci, [vp, vp]),
     "wkz_packed_pack": (ci, [vp, vp, vp, ci, vp, ci]),
     "wkz_gemm": (ci, [vp, vp, vp, ci, vp, ci, vp, vp, vp]),
+    # math / nn (the MLP training step)
+    "wkz_math_dot": (ci, [vp, vp, vp]),
+    "wkz_math_sum": (ci, [vp, vp, vp]),
+    "wkz_math_mean": (ci, [vp, vp, vp]),
+    "wkz_nn_activation_run": (ci, [ci, vp, vp]),
+    "wkz_nn_activation_get_derivative": (ci, [ci, vp, vp, vp]),
+    "wkz_nn_linear_init": (ci, [vp, vp, ci, u64, u64, ci, u64, ci, u64p, ctypes.POINTER(vp)]),
+    "wkz_nn_sequential_init": (ci, [ci, ctypes.POINTER(vp)]),
+    "wkz_nn_sequential_append": (ci, [vp, vp]),
+    "wkz_nn_layer_deinit": (ci, [vp, vp]),
+    "wkz_nn_layer_tensor": (ci, [vp, vp, ci, u64, u64p, ctypes.POINTER(vp)]),
+    "wkz_tensor_handle_drop": (None, [vp]),
+    "wkz_nn_layer_forward": (ci, [vp, vp, vp, vp, ctypes.POINTER(vp)]),
+    "wkz_nn_layer_backward": (ci, [vp, vp, vp, vp, vp]),
+    "wkz_nn_cache_init": (ci, [vp, vp, u64, ctypes.POINTER(vp), u64, ctypes.POINTER(vp)]),
+    "wkz_nn_cache_deinit": (ci, [vp, vp]),
+    "wkz_nn_cache_get_layer_cache": (vp, [vp, u64]),
+    "wkz_nn_cache_error_tensor": (ci, [vp, ctypes.POINTER(vp)]),
+    "wkz_nn_loss_mse": (ci, [ci, vp, vp, vp, vp, vp]),
+    "wkz_nn_gd_init": (ci, [ci, ctypes.c_double, ctypes.POINTER(vp)]),
+    "wkz_nn_adam_init": (ci, [ci, ctypes.c_double, ctypes.c_double, ctypes.c_double, ctypes.c_double, ctypes.POINTER(vp)]),
+    "wkz_nn_optimizer_step": (ci, [vp, vp, vp]),
+    "wkz_nn_optimizer_zero": (ci, [vp, vp]),
+    "wkz_nn_optimizer_deinit": (ci, [vp, vp]),
 }
 
 _host = None
@@ -236,7 +260,21 @@ class Tensor:
 
     def release(self, pipeline: Pipeline) -> None:
         if self._h:
+            if getattr(self, "_borrowed", False):
+                raise ValueError("this tensor belongs to a layer or cache; release that instead")
             _check(_lib().wkz_tensor_release(self._h, pipeline._h), "Tensor.release")
+            self._h = None
+
+    @classmethod
+    def _borrow(cls, handle, dtype: str, context: Context) -> "Tensor":
+        """View of a tensor owned by a layer or a cache; only the handle wrapper is dropped."""
+        t = cls(handle, dtype, context)
+        t._borrowed = True
+        return t
+
+    def __del__(self):
+        if getattr(self, "_borrowed", False) and self._h and _host is not None:
+            _host.wkz_tensor_handle_drop(self._h)
             self._h = None
 
     def host_shape(self):
@@ -336,5 +374,8 @@ class blas:
                                packed_tensors._h if packed_tensors is not None else None), "blas.gemm")
 
 
-__all__ = ["Context", "Pipeline", "Tensor", "CommandQueue", "DeviceType", "memory", "fill", "identity", "blas",
+from . import nn  # noqa: E402  (needs the classes above)
+from .nn import math  # noqa: E402,F401
+
+__all__ = ["nn", "math", "Context", "Pipeline", "Tensor", "CommandQueue", "DeviceType", "memory", "fill", "identity", "blas",
            "GemmPackedTensors", "WekuaError", "DTYPE_NAMES", "dtype_id", "elem_size", "is_complex", "real_np_dtype"]

@@ -66,6 +66,16 @@ SIGNATURES = {
     "wk_gemm_variant": (ctypes.c_char_p, [ci, ci, ci, u64, u64, u64, u64, u64, u64, vp, vp, vp]),
     "wk_gemm_force_variant": (ci, [ctypes.c_char_p]),
     "wk_copy_kernel": (ci, [vp, vp, vp, sz]),
+    "wk_hadamard": (ci, [vp, ci, u64p, vp, u64, u64, vp, u64, u64]),
+    "wk_activation": (ci, [vp, ci, ci, u64p, vp, u64, u64]),
+    "wk_activation_dev": (ci, [vp, ci, ci, u64p, vp, u64, u64, vp, u64, u64]),
+    "wk_bias_activation": (ci, [vp, ci, ci, u64, u64, vp, u64, vp]),
+    "wk_bias_step": (ci, [vp, ci, u64, u64, vp, u64, vp]),
+    "wk_mse": (ci, [vp, ci, u64p, vp, u64, u64, vp, u64, u64, vp, u64, u64, vp, u64, u64]),
+    "wk_sum_workspace_bytes": (sz, [ci]),
+    "wk_sum": (ci, [vp, ci, u64p, vp, u64, u64, vp, vp, ctypes.c_double]),
+    "wk_adam_step": (ci, [vp, ci, u64p, vp, u64, u64, vp, u64, u64, vp, vp, u64, u64, ctypes.c_double, ctypes.c_double,
+                          ctypes.c_double, ctypes.c_double, u64]),
 }
 
 _lib = None

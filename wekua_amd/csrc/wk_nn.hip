@@ -1,0 +1,323 @@
+// Element-wise and reduction kernels the MLP training step needs around gemm / axpy:
+// bias add (+ activation), activation derivative, Hadamard product, bias gradient (column
+// sums), MSE with its derivative, a whole-tensor sum, and an Adam update.
+//
+// Reference kernels restated here:  src/nn/layer/kernels/{bias,bias_step}.cl,
+// src/nn/activation/kernels/{sigmoid,tanh}.cl, src/math/kernels/{dot,sum,trig}.cl,
+// src/nn/loss/kernels/mse.cl.  All are HBM-bound streaming passes over row-pitched 2-D/3-D
+// tensors: one 16-byte vector per lane, rows addressed through their pitch so that only the
+// logical region is touched.  f32 and f64 only (what the MLP configuration uses).
+#include "wk_internal.hpp"
+
+#include <cmath>
+#include <cstring>
+
+using namespace wk;
+
+namespace {
+
+constexpr int EW_BLOCK = 256;
+
+struct Region {
+    uint64_t depth, rows, cols;
+};
+
+// One tensor operand of an element-wise pass.
+template <typename T> struct Opnd {
+    T *p;
+    uint64_t rp, sp;
+};
+
+template <typename T> __device__ __forceinline__ T act_forward(int kind, T x) {
+    if (kind == WK_ACT_SIGMOID) return T(1) / (T(1) + exp(-x));
+    if (kind == WK_ACT_TANH) return tanh(x);
+    return x;
+}
+template <typename T> __device__ __forceinline__ T act_derivative(int kind, T y) {
+    if (kind == WK_ACT_SIGMOID) return y * (T(1) - y);
+    if (kind == WK_ACT_TANH) return T(1) - y * y;
+    return T(1);
+}
+
+// Generic element-wise driver: F(idx3, element pointers...) over the logical region, VE
+// elements of a row per thread when every operand allows 16-byte accesses.
+// WMASK: bit i set = operand i is written back (the others are read-only inputs).
+template <typename T, int NOPS, int WMASK, bool VEC, typename F>
+__global__ __launch_bounds__(EW_BLOCK) void ew_kernel(Region rg, Opnd<T> o0, Opnd<T> o1, Opnd<T> o2, Opnd<T> o3, F f) {
+    constexpr int VE = VEC ? 16 / sizeof(T) : 1;
+    const uint64_t cols_v = (rg.cols + VE - 1) / VE;
+    const uint64_t total = rg.depth * rg.rows * cols_v;
+    for (uint64_t idx = blockIdx.x * (uint64_t)blockDim.x + threadIdx.x; idx < total;
+         idx += (uint64_t)gridDim.x * blockDim.x) {
+        const uint64_t cv = idx % cols_v;
+        const uint64_t ij = idx / cols_v;
+        const uint64_t j = ij % rg.rows, i = ij / rg.rows;
+        const uint64_t c = cv * VE;
+        T *p0 = o0.p + i * o0.sp + j * o0.rp + c;
+        T *p1 = NOPS > 1 ? o1.p + i * o1.sp + j * o1.rp + c : nullptr;
+        T *p2 = NOPS > 2 ? o2.p + i * o2.sp + j * o2.rp + c : nullptr;
+        T *p3 = NOPS > 3 ? o3.p + i * o3.sp + j * o3.rp + c : nullptr;
+        if (VEC && c + VE <= rg.cols) {
+            T v0[VE], v1[VE], v2[VE], v3[VE];
+            __builtin_memcpy(v0, p0, 16);
+            if (NOPS > 1) __builtin_memcpy(v1, p1, 16);
+            if (NOPS > 2) __builtin_memcpy(v2, p2, 16);
+            if (NOPS > 3) __builtin_memcpy(v3, p3, 16);
+#pragma unroll
+            for (int e = 0; e < VE; ++e) f(c + e, v0[e], v1[e], v2[e], v3[e]);
+            if (WMASK & 1) __builtin_memcpy(p0, v0, 16);
+            if (NOPS > 1 && (WMASK & 2)) __builtin_memcpy(p1, v1, 16);
+            if (NOPS > 2 && (WMASK & 4)) __builtin_memcpy(p2, v2, 16);
+            if (NOPS > 3 && (WMASK & 8)) __builtin_memcpy(p3, v3, 16);
+        } else {
+            for (int e = 0; e < VE && c + e < rg.cols; ++e) {
+                T a = p0[e], b = NOPS > 1 ? p1[e] : T(0), cc = NOPS > 2 ? p2[e] : T(0), d = NOPS > 3 ? p3[e] : T(0);
+                f(c + e, a, b, cc, d);
+                if (WMASK & 1) p0[e] = a;
+                if (NOPS > 1 && (WMASK & 2)) p1[e] = b;
+                if (NOPS > 2 && (WMASK & 4)) p2[e] = cc;
+                if (NOPS > 3 && (WMASK & 8)) p3[e] = d;
+            }
+        }
+    }
+}
+
+template <typename T> bool vec_ok(const Opnd<T> &o) {
+    constexpr uint64_t VE = 16 / sizeof(T);
+    return !o.p || ((reinterpret_cast<uintptr_t>(o.p) & 15u) == 0 && o.rp % VE == 0 && o.sp % VE == 0);
+}
+
+template <typename T, int NOPS, int WMASK, typename F>
+int ew_launch(wk_stream *s, const Region &rg, Opnd<T> o0, Opnd<T> o1, Opnd<T> o2, Opnd<T> o3, F f) {
+    const bool vec = vec_ok(o0) && vec_ok(o1) && vec_ok(o2) && vec_ok(o3);
+    const uint64_t ve = vec ? 16 / sizeof(T) : 1;
+    const uint64_t total = rg.depth * rg.rows * ((rg.cols + ve - 1) / ve);
+    const uint64_t want = (total + EW_BLOCK - 1) / EW_BLOCK;
+    const unsigned grid = (unsigned)(want < 256ull * 256 ? (want ? want : 1) : 256ull * 256);
+    if (vec) hipLaunchKernelGGL((ew_kernel<T, NOPS, WMASK, true, F>), dim3(grid), dim3(EW_BLOCK), 0, s->stream, rg, o0, o1, o2, o3, f);
+    else hipLaunchKernelGGL((ew_kernel<T, NOPS, WMASK, false, F>), dim3(grid), dim3(EW_BLOCK), 0, s->stream, rg, o0, o1, o2, o3, f);
+    return launch_status();
+}
+
+int check_region(const uint64_t shape3[3], Region &rg) {
+    if (!shape3) return WK_E_INVALID_VALUE;
+    rg = {shape3[0], shape3[1], shape3[2]};
+    if (!rg.depth || !rg.rows || !rg.cols) return WK_E_INVALID_VALUE;
+    return WK_OK;
+}
+
+template <typename T> int check_opnd(const Region &rg, const void *p, uint64_t rp, uint64_t sp) {
+    if (!p) return WK_E_INVALID_VALUE;
+    if (rg.rows > 1 && rp < rg.cols) return WK_E_INVALID_VALUE;
+    if (rg.depth > 1 && sp < rg.rows * rp) return WK_E_INVALID_VALUE;
+    return WK_OK;
+}
+
+template <typename F> int dispatch_float(int dtype, F &&f) {
+    if (dtype == WK_F32) return f.template operator()<float>();
+    if (dtype == WK_F64) return f.template operator()<double>();
+    return dtype >= 0 && dtype < WK_DTYPE_COUNT ? WK_E_TYPE_NOT_SUPPORTED : WK_E_TYPE_NOT_SUPPORTED;
+}
+
+// ---- column sums (bias_step.cl): one thread per column walks the rows; consecutive threads read
+// consecutive addresses of each row, so every row access is one coalesced run. --------------
+template <typename T>
+__global__ __launch_bounds__(256) void colsum_kernel(const T *__restrict__ x, uint64_t rows, uint64_t cols, uint64_t pitch,
+                                                     T *__restrict__ out) {
+    // blockDim = (64, 4): 64 columns per block, rows split 4 ways, combined through LDS
+    __shared__ T part[4][64];
+    const uint64_t c = blockIdx.x * 64ull + threadIdx.x;
+    T acc = T(0);
+    if (c < cols)
+        for (uint64_t r = threadIdx.y; r < rows; r += 4) acc += x[r * pitch + c];
+    part[threadIdx.y][threadIdx.x] = acc;
+    __syncthreads();
+    if (threadIdx.y == 0 && c < cols) out[c] = (part[0][threadIdx.x] + part[1][threadIdx.x]) + (part[2][threadIdx.x] + part[3][threadIdx.x]);
+}
+
+// ---- whole-tensor sum (math.sum + host finish, src/math/basic.zig:128-203): two fixed-shape
+// passes so that the result does not depend on scheduling. ------------------------------------
+constexpr int SUM_PARTIALS = 1024;
+
+template <typename T>
+__global__ __launch_bounds__(256) void sum_pass1_kernel(const T *__restrict__ x, Region rg, uint64_t rp, uint64_t sp,
+                                                        T *__restrict__ partials) {
+    __shared__ T red[256];
+    const uint64_t total = rg.depth * rg.rows * rg.cols;
+    T acc = T(0);
+    for (uint64_t idx = blockIdx.x * 256ull + threadIdx.x; idx < total; idx += (uint64_t)SUM_PARTIALS * 256ull) {
+        const uint64_t k = idx % rg.cols;
+        const uint64_t ij = idx / rg.cols;
+        acc += x[(ij / rg.rows) * sp + (ij % rg.rows) * rp + k];
+    }
+    red[threadIdx.x] = acc;
+    __syncthreads();
+    for (int st = 128; st > 0; st >>= 1) {
+        if ((int)threadIdx.x < st) red[threadIdx.x] += red[threadIdx.x + st];
+        __syncthreads();
+    }
+    if (threadIdx.x == 0) partials[blockIdx.x] = red[0];
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void sum_pass2_kernel(const T *__restrict__ partials, T *__restrict__ out, T scale) {
+    __shared__ T red[256];
+    T acc = T(0);
+    for (int i = threadIdx.x; i < SUM_PARTIALS; i += 256) acc += partials[i];
+    red[threadIdx.x] = acc;
+    __syncthreads();
+    for (int st = 128; st > 0; st >>= 1) {
+        if ((int)threadIdx.x < st) red[threadIdx.x] += red[threadIdx.x + st];
+        __syncthreads();
+    }
+    if (threadIdx.x == 0) out[0] = red[0] * scale;
+}
+
+} // namespace
+
+extern "C" {
+
+int wk_hadamard(wk_stream *s, int dtype, const uint64_t shape3[3], void *x, uint64_t xrp, uint64_t xsp, const void *y,
+                uint64_t yrp, uint64_t ysp) {
+    int rc = bind(s);
+    if (rc) return rc;
+    Region rg;
+    if ((rc = check_region(shape3, rg))) return rc;
+    return dispatch_float(dtype, [&]<typename T>() -> int {
+        if (check_opnd<T>(rg, x, xrp, xsp) || check_opnd<T>(rg, y, yrp, ysp)) return WK_E_INVALID_VALUE;
+        return ew_launch<T, 2, 1>(s, rg, Opnd<T>{(T *)x, xrp, xsp}, Opnd<T>{(T *)y, yrp, ysp}, Opnd<T>{}, Opnd<T>{},
+                               [] __device__(uint64_t, T &a, T &b, T &, T &) { a *= b; });
+    });
+}
+
+int wk_activation(wk_stream *s, int dtype, int kind, const uint64_t shape3[3], void *x, uint64_t xrp, uint64_t xsp) {
+    int rc = bind(s);
+    if (rc) return rc;
+    Region rg;
+    if ((rc = check_region(shape3, rg))) return rc;
+    if (kind != WK_ACT_SIGMOID && kind != WK_ACT_TANH) return WK_E_INVALID_VALUE;
+    return dispatch_float(dtype, [&]<typename T>() -> int {
+        if (check_opnd<T>(rg, x, xrp, xsp)) return WK_E_INVALID_VALUE;
+        return ew_launch<T, 1, 1>(s, rg, Opnd<T>{(T *)x, xrp, xsp}, Opnd<T>{}, Opnd<T>{}, Opnd<T>{},
+                               [kind] __device__(uint64_t, T &a, T &, T &, T &) { a = act_forward<T>(kind, a); });
+    });
+}
+
+int wk_activation_dev(wk_stream *s, int dtype, int kind, const uint64_t shape3[3], const void *out, uint64_t orp,
+                      uint64_t osp, void *dev, uint64_t drp, uint64_t dsp) {
+    int rc = bind(s);
+    if (rc) return rc;
+    Region rg;
+    if ((rc = check_region(shape3, rg))) return rc;
+    if (kind != WK_ACT_SIGMOID && kind != WK_ACT_TANH) return WK_E_INVALID_VALUE;
+    return dispatch_float(dtype, [&]<typename T>() -> int {
+        if (check_opnd<T>(rg, out, orp, osp) || check_opnd<T>(rg, dev, drp, dsp)) return WK_E_INVALID_VALUE;
+        return ew_launch<T, 2, 1>(s, rg, Opnd<T>{(T *)dev, drp, dsp}, Opnd<T>{(T *)out, orp, osp}, Opnd<T>{}, Opnd<T>{},
+                               [kind] __device__(uint64_t, T &d, T &y, T &, T &) { d = act_derivative<T>(kind, y); });
+    });
+}
+
+int wk_bias_activation(wk_stream *s, int dtype, int kind, uint64_t rows, uint64_t cols, void *out, uint64_t out_pitch,
+                       const void *bias) {
+    int rc = bind(s);
+    if (rc) return rc;
+    if (!rows || !cols || !out || out_pitch < cols) return WK_E_INVALID_VALUE;
+    if (kind != WK_ACT_NONE && kind != WK_ACT_SIGMOID && kind != WK_ACT_TANH) return WK_E_INVALID_VALUE;
+    const Region rg{1, rows, cols};
+    return dispatch_float(dtype, [&]<typename T>() -> int {
+        const T *b = static_cast<const T *>(bias); // may be null: activation only
+        return ew_launch<T, 1, 1>(s, rg, Opnd<T>{(T *)out, out_pitch, 0}, Opnd<T>{}, Opnd<T>{}, Opnd<T>{},
+                               [kind, b] __device__(uint64_t c, T &a, T &, T &, T &) {
+                                   if (b) a += b[c];
+                                   a = act_forward<T>(kind, a);
+                               });
+    });
+}
+
+int wk_bias_step(wk_stream *s, int dtype, uint64_t rows, uint64_t cols, const void *sens, uint64_t pitch, void *bias_grad) {
+    int rc = bind(s);
+    if (rc) return rc;
+    if (!rows || !cols || !sens || !bias_grad || pitch < cols) return WK_E_INVALID_VALUE;
+    return dispatch_float(dtype, [&]<typename T>() -> int {
+        hipLaunchKernelGGL((colsum_kernel<T>), dim3((unsigned)((cols + 63) / 64)), dim3(64, 4), 0, s->stream,
+                           static_cast<const T *>(sens), rows, cols, pitch, static_cast<T *>(bias_grad));
+        return launch_status();
+    });
+}
+
+int wk_mse(wk_stream *s, int dtype, const uint64_t shape3[3], const void *output, uint64_t orp, uint64_t osp,
+           const void *expected, uint64_t erp, uint64_t esp, void *error, uint64_t rrp, uint64_t rsp, void *dev,
+           uint64_t drp, uint64_t dsp) {
+    int rc = bind(s);
+    if (rc) return rc;
+    Region rg;
+    if ((rc = check_region(shape3, rg))) return rc;
+    return dispatch_float(dtype, [&]<typename T>() -> int {
+        if (check_opnd<T>(rg, output, orp, osp) || check_opnd<T>(rg, expected, erp, esp) || check_opnd<T>(rg, error, rrp, rsp))
+            return WK_E_INVALID_VALUE;
+        if (dev) {
+            if (check_opnd<T>(rg, dev, drp, dsp)) return WK_E_INVALID_VALUE;
+            return ew_launch<T, 4, 3>(s, rg, Opnd<T>{(T *)error, rrp, rsp}, Opnd<T>{(T *)dev, drp, dsp},
+                                   Opnd<T>{(T *)output, orp, osp}, Opnd<T>{(T *)expected, erp, esp},
+                                   [] __device__(uint64_t, T &err2, T &d, T &o, T &e) {
+                                       const T err = e - o;
+                                       err2 = err * err;
+                                       d = T(-2) * err;
+                                   });
+        }
+        return ew_launch<T, 3, 1>(s, rg, Opnd<T>{(T *)error, rrp, rsp}, Opnd<T>{(T *)output, orp, osp},
+                               Opnd<T>{(T *)expected, erp, esp}, Opnd<T>{},
+                               [] __device__(uint64_t, T &err2, T &o, T &e, T &) {
+                                   const T err = e - o;
+                                   err2 = err * err;
+                               });
+    });
+}
+
+size_t wk_sum_workspace_bytes(int dtype) { return SUM_PARTIALS * wk_dtype_size(dtype); }
+
+int wk_sum(wk_stream *s, int dtype, const uint64_t shape3[3], const void *x, uint64_t xrp, uint64_t xsp, void *workspace,
+           void *dev_result, double scale) {
+    int rc = bind(s);
+    if (rc) return rc;
+    Region rg;
+    if ((rc = check_region(shape3, rg))) return rc;
+    if (!workspace || !dev_result) return WK_E_INVALID_VALUE;
+    return dispatch_float(dtype, [&]<typename T>() -> int {
+        if (check_opnd<T>(rg, x, xrp, xsp)) return WK_E_INVALID_VALUE;
+        hipLaunchKernelGGL((sum_pass1_kernel<T>), dim3(SUM_PARTIALS), dim3(256), 0, s->stream, static_cast<const T *>(x), rg,
+                           xrp, xsp, static_cast<T *>(workspace));
+        int lrc = launch_status();
+        if (lrc) return lrc;
+        hipLaunchKernelGGL((sum_pass2_kernel<T>), dim3(1), dim3(256), 0, s->stream, static_cast<const T *>(workspace),
+                           static_cast<T *>(dev_result), static_cast<T>(scale));
+        return launch_status();
+    });
+}
+
+int wk_adam_step(wk_stream *s, int dtype, const uint64_t shape3[3], void *w, uint64_t wrp, uint64_t wsp, const void *g,
+                 uint64_t grp, uint64_t gsp, void *m, void *v, uint64_t mrp, uint64_t msp, double lr, double beta1,
+                 double beta2, double eps, uint64_t step) {
+    int rc = bind(s);
+    if (rc) return rc;
+    Region rg;
+    if ((rc = check_region(shape3, rg))) return rc;
+    if (step == 0) return WK_E_INVALID_VALUE;
+    const double bc1 = 1.0 - std::pow(beta1, (double)step), bc2 = 1.0 - std::pow(beta2, (double)step);
+    return dispatch_float(dtype, [&]<typename T>() -> int {
+        if (check_opnd<T>(rg, w, wrp, wsp) || check_opnd<T>(rg, g, grp, gsp) || check_opnd<T>(rg, m, mrp, msp) ||
+            check_opnd<T>(rg, v, mrp, msp))
+            return WK_E_INVALID_VALUE;
+        const T b1 = (T)beta1, b2 = (T)beta2, ib1 = (T)(1.0 - beta1), ib2 = (T)(1.0 - beta2);
+        const T step_size = (T)(lr / bc1), inv_sqrt_bc2 = (T)(1.0 / std::sqrt(bc2)), e = (T)eps;
+        return ew_launch<T, 4, 7>(s, rg, Opnd<T>{(T *)w, wrp, wsp}, Opnd<T>{(T *)m, mrp, msp}, Opnd<T>{(T *)v, mrp, msp},
+                               Opnd<T>{(T *)g, grp, gsp},
+                               [=] __device__(uint64_t, T &wv, T &mv, T &vv, T &gv) {
+                                   mv = b1 * mv + ib1 * gv;
+                                   vv = b2 * vv + ib2 * gv * gv;
+                                   wv -= step_size * mv / (sqrt(vv) * inv_sqrt_bc2 + e);
+                               });
+    });
+}
+
+} // extern "C"

@@ -4,6 +4,7 @@
 // the parity tests exercise the same host logic (validation, layout, option handling) a C++
 // caller gets.  Every function returns a WK_E_* code (the Zig error name) and never throws.
 #include "wekua.hpp"
+#include "wekua_nn.hpp"
 
 #include <new>
 
@@ -21,6 +22,28 @@ struct PackedHandle {
     int dtype;
     void *packed; // blas::PackedTensors<T>*
 };
+
+// nn objects exist for f32 and f64 only, like the reference's (src/nn/optimizers/gd.zig:17-20)
+struct LayerHandle {
+    int dtype;
+    void *layer; // nn::Layer<T>*
+};
+struct CacheHandle {
+    int dtype;
+    void *cache; // nn::Cache<T>*
+};
+struct OptimizerHandle {
+    int dtype;
+    void *optimizer; // nn::optimizers::Optimizer<T>*
+};
+
+template <typename F> void dispatch_real(int dtype, F &&f) {
+    switch (dtype) {
+    case 8: f.template operator()<float>(); break;
+    case 9: f.template operator()<double>(); break;
+    default: throw Error(WK_E_TYPE_NOT_SUPPORTED);
+    }
+}
 
 template <typename F> int guard(F &&f) {
     try {
@@ -293,6 +316,253 @@ int wkz_gemm(void *pipeline, const void *host_alpha, void *a, int op_a, void *b,
                           opt_scalar<T>(host_beta), static_cast<Tensor<T> *>(hc->tensor),
                           hp ? static_cast<blas::PackedTensors<T> *>(hp->packed) : nullptr);
         });
+    });
+}
+
+// ---- math ------------------------------------------------------------------------------------------
+int wkz_math_dot(void *pipeline, void *x, void *y) {
+    return guard([&] {
+        TensorHandle *hx = static_cast<TensorHandle *>(x), *hy = static_cast<TensorHandle *>(y);
+        if (hx->dtype != hy->dtype) throw Error(WK_E_UNQUAL_TENSORS_ATTRIBUTE);
+        dispatch_real(hx->dtype, [&]<typename T>() {
+            math::dot<T>(static_cast<Pipeline *>(pipeline), static_cast<Tensor<T> *>(hx->tensor), static_cast<Tensor<T> *>(hy->tensor));
+        });
+    });
+}
+static int reduce(void *pipeline, void *x, void *host_result, bool mean) {
+    return guard([&] {
+        TensorHandle *hx = static_cast<TensorHandle *>(x);
+        if (!host_result) throw Error(WK_E_INVALID_VALUE);
+        dispatch_real(hx->dtype, [&]<typename T>() {
+            Tensor<T> *t = static_cast<Tensor<T> *>(hx->tensor);
+            const T r = mean ? math::mean<T>(static_cast<Pipeline *>(pipeline), t) : math::sum<T>(static_cast<Pipeline *>(pipeline), t);
+            std::memcpy(host_result, &r, sizeof(T));
+        });
+    });
+}
+int wkz_math_sum(void *pipeline, void *x, void *host_result) { return reduce(pipeline, x, host_result, false); }
+int wkz_math_mean(void *pipeline, void *x, void *host_result) { return reduce(pipeline, x, host_result, true); }
+
+// ---- nn: activations ---------------------------------------------------------------------------------
+int wkz_nn_activation_run(int kind, void *pipeline, void *tensor) {
+    return guard([&] {
+        TensorHandle *h = static_cast<TensorHandle *>(tensor);
+        dispatch_real(h->dtype, [&]<typename T>() {
+            nn::Activation<T>{kind}.run(static_cast<Pipeline *>(pipeline), static_cast<Tensor<T> *>(h->tensor));
+        });
+    });
+}
+int wkz_nn_activation_get_derivative(int kind, void *pipeline, void *output, void *derivative) {
+    return guard([&] {
+        TensorHandle *ho = static_cast<TensorHandle *>(output), *hd = static_cast<TensorHandle *>(derivative);
+        if (ho->dtype != hd->dtype) throw Error(WK_E_UNQUAL_TENSORS_ATTRIBUTE);
+        dispatch_real(ho->dtype, [&]<typename T>() {
+            nn::Activation<T>{kind}.getDerivative(static_cast<Pipeline *>(pipeline), static_cast<Tensor<T> *>(ho->tensor),
+                                                  static_cast<Tensor<T> *>(hd->tensor));
+        });
+    });
+}
+
+// ---- nn: layers ------------------------------------------------------------------------------------------
+// activation_kind: WK_ACT_NONE for a layer without activation; seed: NULL draws it from the clock
+int wkz_nn_linear_init(void *ctx, void *pipeline, int dtype, uint64_t input, uint64_t output, int activation_kind, uint64_t deep,
+                       int enable_bias, const uint64_t *seed, void **out) {
+    return guard([&] {
+        if (!out) throw Error(WK_E_INVALID_VALUE);
+        if (activation_kind != WK_ACT_NONE && activation_kind != WK_ACT_SIGMOID && activation_kind != WK_ACT_TANH)
+            throw Error(WK_E_INVALID_VALUE);
+        dispatch_real(dtype, [&]<typename T>() {
+            nn::ExtraParams extra;
+            extra.deep = (size_t)deep;
+            extra.enable_bias = enable_bias != 0;
+            if (seed) extra.seed = *seed;
+            std::optional<nn::Activation<T>> acti;
+            if (activation_kind != WK_ACT_NONE) acti = nn::Activation<T>{activation_kind};
+            nn::Layer<T> *l =
+                nn::Linear<T>::init(static_cast<Context *>(ctx), static_cast<Pipeline *>(pipeline), input, output, acti, extra);
+            *out = new LayerHandle{dtype, l};
+        });
+    });
+}
+int wkz_nn_sequential_init(int dtype, void **out) {
+    return guard([&] {
+        if (!out) throw Error(WK_E_INVALID_VALUE);
+        dispatch_real(dtype, [&]<typename T>() {
+            nn::Layer<T> *l = nn::Sequential<T>::init();
+            *out = new LayerHandle{dtype, l};
+        });
+    });
+}
+// the sequence takes ownership of `layer`; its handle is consumed
+int wkz_nn_sequential_append(void *sequential, void *layer) {
+    return guard([&] {
+        LayerHandle *hs = static_cast<LayerHandle *>(sequential), *hl = static_cast<LayerHandle *>(layer);
+        if (hs->dtype != hl->dtype) throw Error(WK_E_UNQUAL_TENSORS_ATTRIBUTE);
+        dispatch_real(hs->dtype, [&]<typename T>() {
+            auto *seq = dynamic_cast<nn::Sequential<T> *>(static_cast<nn::Layer<T> *>(hs->layer));
+            if (!seq) throw Error(WK_E_INVALID_VALUE);
+            seq->append(static_cast<nn::Layer<T> *>(hl->layer));
+        });
+        delete hl;
+    });
+}
+int wkz_nn_layer_deinit(void *layer, void *pipeline) {
+    return guard([&] {
+        LayerHandle *h = static_cast<LayerHandle *>(layer);
+        dispatch_real(h->dtype, [&]<typename T>() { static_cast<nn::Layer<T> *>(h->layer)->deinit(static_cast<Pipeline *>(pipeline)); });
+        delete h;
+    });
+}
+// Borrowed views of a layer's tensors.  which: 0 weights, 1 bias, 2 gradients, 3 bias gradients
+// (2 and 3 need the layer's cache), 4 cached output, 5 sensitivity (index ignored).  *count
+// receives the list length; *out a tensor handle to pass to wkz_tensor_handle_drop (never to
+// wkz_tensor_release), or NULL for an absent bias.
+int wkz_nn_layer_tensor(void *layer, void *layer_cache, int which, uint64_t index, uint64_t *count, void **out) {
+    return guard([&] {
+        LayerHandle *h = static_cast<LayerHandle *>(layer);
+        if ((which >= 2 && !layer_cache) || which < 0 || which > 5) throw Error(WK_E_INVALID_VALUE);
+        dispatch_real(h->dtype, [&]<typename T>() {
+            nn::Layer<T> *l = static_cast<nn::Layer<T> *>(h->layer);
+            std::vector<Tensor<T> *> list;
+            switch (which) {
+            case 0: list = l->getWeights(); break;
+            case 1: list = l->getBias(); break;
+            case 2: list = l->getGradients(layer_cache); break;
+            case 3: list = l->getBiasGradients(layer_cache); break;
+            case 4: list = {l->getCachedOutput(layer_cache)}; break;
+            default: list = {l->getSensitivity(layer_cache)}; break;
+            }
+            if (count) *count = list.size();
+            if (out) {
+                if (index >= list.size()) throw Error(WK_E_INVALID_COORDINATES);
+                *out = list[index] ? new TensorHandle{h->dtype, list[index]} : nullptr;
+            }
+        });
+    });
+}
+void wkz_tensor_handle_drop(void *tensor) { delete static_cast<TensorHandle *>(tensor); }
+
+int wkz_nn_layer_forward(void *layer, void *pipeline, void *input, void *layer_cache, void **out) {
+    return guard([&] {
+        LayerHandle *h = static_cast<LayerHandle *>(layer);
+        TensorHandle *hi = static_cast<TensorHandle *>(input);
+        if (hi->dtype != h->dtype) throw Error(WK_E_UNQUAL_TENSORS_ATTRIBUTE);
+        if (!layer_cache) throw Error(WK_E_INVALID_VALUE);
+        dispatch_real(h->dtype, [&]<typename T>() {
+            Tensor<T> *o = static_cast<nn::Layer<T> *>(h->layer)->forward(static_cast<Pipeline *>(pipeline),
+                                                                          static_cast<Tensor<T> *>(hi->tensor), layer_cache);
+            if (out) *out = new TensorHandle{h->dtype, o};
+        });
+    });
+}
+int wkz_nn_layer_backward(void *layer, void *pipeline, void *layer_cache, void *input, void *input_gradient) {
+    return guard([&] {
+        LayerHandle *h = static_cast<LayerHandle *>(layer);
+        TensorHandle *hi = static_cast<TensorHandle *>(input), *hg = static_cast<TensorHandle *>(input_gradient);
+        if (hi->dtype != h->dtype || (hg && hg->dtype != h->dtype)) throw Error(WK_E_UNQUAL_TENSORS_ATTRIBUTE);
+        if (!layer_cache) throw Error(WK_E_INVALID_VALUE);
+        dispatch_real(h->dtype, [&]<typename T>() {
+            static_cast<nn::Layer<T> *>(h->layer)->backward(static_cast<Pipeline *>(pipeline), layer_cache,
+                                                            static_cast<Tensor<T> *>(hi->tensor),
+                                                            hg ? static_cast<Tensor<T> *>(hg->tensor) : nullptr);
+        });
+    });
+}
+
+// ---- nn: cache, loss, optimizers ----------------------------------------------------------------------
+int wkz_nn_cache_init(void *ctx, void *pipeline, uint64_t number_of_elements, void *const *layers, uint64_t num_layers, void **out) {
+    return guard([&] {
+        if (!out || !layers || num_layers == 0) throw Error(WK_E_INVALID_VALUE);
+        const int dtype = static_cast<LayerHandle *>(layers[0])->dtype;
+        for (uint64_t i = 1; i < num_layers; ++i)
+            if (static_cast<LayerHandle *>(layers[i])->dtype != dtype) throw Error(WK_E_UNQUAL_TENSORS_ATTRIBUTE);
+        dispatch_real(dtype, [&]<typename T>() {
+            std::vector<const nn::Layer<T> *> list;
+            for (uint64_t i = 0; i < num_layers; ++i) list.push_back(static_cast<nn::Layer<T> *>(static_cast<LayerHandle *>(layers[i])->layer));
+            *out = new CacheHandle{
+                dtype, nn::Cache<T>::init(static_cast<Context *>(ctx), static_cast<Pipeline *>(pipeline), number_of_elements, list)};
+        });
+    });
+}
+int wkz_nn_cache_deinit(void *cache, void *pipeline) {
+    return guard([&] {
+        CacheHandle *h = static_cast<CacheHandle *>(cache);
+        dispatch_real(h->dtype, [&]<typename T>() { static_cast<nn::Cache<T> *>(h->cache)->deinit(static_cast<Pipeline *>(pipeline)); });
+        delete h;
+    });
+}
+void *wkz_nn_cache_get_layer_cache(void *cache, uint64_t index) {
+    CacheHandle *h = static_cast<CacheHandle *>(cache);
+    void *r = nullptr;
+    guard([&] {
+        dispatch_real(h->dtype, [&]<typename T>() {
+            auto *c = static_cast<nn::Cache<T> *>(h->cache);
+            if (index < c->slots.size()) r = c->getLayerCache((size_t)index);
+        });
+    });
+    return r;
+}
+int wkz_nn_cache_error_tensor(void *cache, void **out) {
+    return guard([&] {
+        CacheHandle *h = static_cast<CacheHandle *>(cache);
+        dispatch_real(h->dtype, [&]<typename T>() { *out = new TensorHandle{h->dtype, static_cast<nn::Cache<T> *>(h->cache)->error_tensor}; });
+    });
+}
+// host_error_result may be NULL (no mean is computed, nothing synchronises)
+int wkz_nn_loss_mse(int calculate_derivative, void *pipeline, void *output, void *expected, void *cache, void *host_error_result) {
+    return guard([&] {
+        CacheHandle *hc = static_cast<CacheHandle *>(cache);
+        TensorHandle *ho = static_cast<TensorHandle *>(output), *he = static_cast<TensorHandle *>(expected);
+        if (ho->dtype != hc->dtype || he->dtype != hc->dtype) throw Error(WK_E_UNQUAL_TENSORS_ATTRIBUTE);
+        dispatch_real(hc->dtype, [&]<typename T>() {
+            T result{};
+            nn::loss::mse<T>(calculate_derivative != 0, static_cast<Pipeline *>(pipeline), static_cast<Tensor<T> *>(ho->tensor),
+                             static_cast<Tensor<T> *>(he->tensor), static_cast<nn::Cache<T> *>(hc->cache),
+                             host_error_result ? &result : nullptr);
+            if (host_error_result) std::memcpy(host_error_result, &result, sizeof(T));
+        });
+    });
+}
+int wkz_nn_gd_init(int dtype, double lr, void **out) {
+    return guard([&] {
+        if (!out) throw Error(WK_E_INVALID_VALUE);
+        dispatch_real(dtype, [&]<typename T>() {
+            nn::optimizers::Optimizer<T> *o = nn::optimizers::GD<T>::init((T)lr);
+            *out = new OptimizerHandle{dtype, o};
+        });
+    });
+}
+// eps < 0 selects the default (the machine epsilon of the element type)
+int wkz_nn_adam_init(int dtype, double lr, double beta1, double beta2, double eps, void **out) {
+    return guard([&] {
+        if (!out) throw Error(WK_E_INVALID_VALUE);
+        dispatch_real(dtype, [&]<typename T>() {
+            nn::optimizers::Optimizer<T> *o = nn::optimizers::Adam<T>::init(lr, beta1, beta2, eps);
+            *out = new OptimizerHandle{dtype, o};
+        });
+    });
+}
+int wkz_nn_optimizer_step(void *optimizer, void *pipeline, void *cache) {
+    return guard([&] {
+        OptimizerHandle *h = static_cast<OptimizerHandle *>(optimizer);
+        CacheHandle *hc = static_cast<CacheHandle *>(cache);
+        if (hc->dtype != h->dtype) throw Error(WK_E_UNQUAL_TENSORS_ATTRIBUTE);
+        dispatch_real(h->dtype, [&]<typename T>() {
+            static_cast<nn::optimizers::Optimizer<T> *>(h->optimizer)->step(static_cast<Pipeline *>(pipeline), static_cast<nn::Cache<T> *>(hc->cache));
+        });
+    });
+}
+int wkz_nn_optimizer_zero(void *optimizer, void *pipeline) {
+    return guard([&] {
+        OptimizerHandle *h = static_cast<OptimizerHandle *>(optimizer);
+        dispatch_real(h->dtype, [&]<typename T>() { static_cast<nn::optimizers::Optimizer<T> *>(h->optimizer)->zero(static_cast<Pipeline *>(pipeline)); });
+    });
+}
+int wkz_nn_optimizer_deinit(void *optimizer, void *pipeline) {
+    return guard([&] {
+        OptimizerHandle *h = static_cast<OptimizerHandle *>(optimizer);
+        dispatch_real(h->dtype, [&]<typename T>() { static_cast<nn::optimizers::Optimizer<T> *>(h->optimizer)->deinit(static_cast<Pipeline *>(pipeline)); });
+        delete h;
     });
 }
 

@@ -34,6 +34,15 @@ def uniform(seed: int, shape, dtype, lo: float = -1.0, hi: float = 1.0) -> np.nd
     return out.reshape(shape)
 
 
+def normal(seed: int, shape, dtype) -> np.ndarray:
+    """Standard normal values (Box-Muller on two splitmix64 streams, evaluated in float64)."""
+    n = int(np.prod(shape))
+    u1 = 1.0 - uniform(seed, (n,), np.float64, 0.0, 1.0)  # (0, 1]
+    u2 = uniform(seed ^ 0x5A5A5A5A5A5A5A5A, (n,), np.float64, 0.0, 1.0)
+    z = np.sqrt(-2.0 * np.log(u1)) * np.cos(2.0 * np.pi * u2)
+    return z.astype(dtype).reshape(shape)
+
+
 def integers(seed: int, shape, dtype, lo: int, hi: int) -> np.ndarray:
     """Uniform integers in [lo, hi] of `dtype` (values are reduced into the dtype's range)."""
     dtype = np.dtype(dtype)
