@@ -144,6 +144,7 @@ def main():
     ap.add_argument("--axpy-log2n", type=int, default=28)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-rows", type=int, default=8192)
+    ap.add_argument("--no-mlp", action="store_true", help="skip the MLP training step leg (BASELINE configuration 5)")
     ap.add_argument("--calibrate", action="store_true",
                     help="also launch the plain 1 GiB copy kernel a few times, so that a profiler run of this "
                          "command holds a kernel of known HBM traffic to scale byte counters against")
@@ -178,6 +179,17 @@ def main():
         dst.free()
     dev.close()
 
+    mlp = None
+    if not args.no_mlp:
+        from wekua_amd import benchmark
+        m = benchmark.time_mlp_step(steps=max(args.steps, 10), warmup=args.warmup)
+        log(f"[bench] mlp step 1024-4096-4096-1024 f32 batch 2048 adam: {m['stream_ms']:.3f} ms/step "
+            f"-> {m['tflops']:.1f} TFLOP/s over its GEMM flops")
+        mlp = {"workload": "MLP training step 1024-4096-4096-1024, f32, batch 2048, tanh/tanh/sigmoid, MSE, Adam lr=1e-3 "
+                           "(BASELINE config 5): forward + loss + backward + update",
+               "ms_per_step": m["stream_ms"], "wall_ms_per_step": m["wall_ms"], "gemm_flops_per_step": m["flops"],
+               "value": m["tflops"], "unit": "TFLOP/s", "frac_of_f32_matrix_peak": m["tflops"] / F32_MATRIX_PEAK_TFLOPS}
+
     cpu = None
     if not args.no_cpu_baseline:
         cores = min(os.cpu_count() or 1, int(os.environ.get("OMP_NUM_THREADS", "16") or 16), 16)
@@ -210,6 +222,7 @@ def main():
                               "frac": ax["gbs"] / HBM_PEAK_GBS, "traffic": read_traffic("axpy_f32_2p28"),
                               "bytes_per_launch": ax["bytes"]},
                  "f64": {"value": ax64["gbs"], "us_per_call": ax64["us"], "frac": ax64["gbs"] / HBM_PEAK_GBS}},
+        "mlp_step": mlp,
         "cpu_baseline": cpu,
     }
     print(json.dumps(out), flush=True)

@@ -81,7 +81,7 @@ def test_f32_every_variant(dev, variant, op_a, op_b):
         dev.lib.wk_gemm_force_variant(b"auto")
 
 
-@pytest.mark.parametrize("variant", ["tile64", "mfma_f64_64x64", "mfma_f64_128x128"])
+@pytest.mark.parametrize("variant", ["tile64", "mfma_f64_64x64", "mfma_f64_128x64", "mfma_f64_128x128"])
 @pytest.mark.parametrize("op_a,op_b", OPS)
 def test_f64_every_variant(dev, variant, op_a, op_b):
     assert dev.lib.wk_gemm_force_variant(variant.encode()) == 0

@@ -4,7 +4,8 @@ times over 1-D sizes, on GPU 0.
 
     python -m wekua_amd.benchmark gemm [--dtype f32] [--sizes 1024 2048 ...] [--variant NAME]
     python -m wekua_amd.benchmark axpy [--dtype f32]
-    python -m wekua_amd.benchmark configs        # every BASELINE configuration, one line each
+    python -m wekua_amd.benchmark configs        # every BASELINE GEMM / AXPY configuration, one line each
+    python -m wekua_amd.benchmark mlp [--dtype f32] [--sizes 1024 4096 4096 1024] [--batch 2048] [--optimizer adam]
 
 Unlike the reference's harness the inputs are seeded (wekua_amd.synth), times come from
 events on the kernel's stream, and every line also gives the rate (TFLOP/s or GB/s).
@@ -104,6 +105,90 @@ def cmd_configs(dev, args):
         print(f"{name:34s} {ms:9.4f} {rate:9.2f} {unit:8s} {v}")
 
 
+def mlp_flops(sizes, batch):
+    """Multiply-adds of the GEMMs of one training step, as flops: forward and weight gradients over
+    every layer, input sensitivities over every layer but the first."""
+    pairs = list(zip(sizes[:-1], sizes[1:]))
+    fwd = sum(2.0 * batch * i * o for i, o in pairs)
+    return 2 * fwd + sum(2.0 * batch * i * o for i, o in pairs[1:])
+
+
+def time_mlp_step(dtype="f32", sizes=(1024, 4096, 4096, 1024), batch=2048, optimizer="adam", lr=1e-3, steps=20, warmup=3,
+                  seed=None):
+    """One training step of BASELINE configuration 5 through the reference-shaped API: Sequential of
+    Linear layers (tanh hidden, sigmoid output), loss.mse with derivative, backward, optimizer step.
+    Returns ms per step from events on the pipeline's stream and from the wall clock."""
+    import ctypes
+    import time
+
+    import wekua_amd as wk
+    from wekua_amd import nn
+
+    seed = synth.config_seed(5, 0) if seed is None else seed
+    rd = raw.real_np_dtype(dtype)
+    ctx = wk.Context.initFromDeviceType(wk.DeviceType.all)
+    pipeline = wk.Pipeline.init(ctx.command_queues[0])
+    seq = nn.Sequential.init(dtype)
+    n_layers = len(sizes) - 1
+    for i in range(n_layers):
+        act = nn.Sigmoid.init() if i == n_layers - 1 else nn.Tanh.init()
+        seq.append(nn.Linear.init(dtype, ctx, pipeline, sizes[i], sizes[i + 1], act, seed=seed + i))
+    x = wk.Tensor.alloc(dtype, ctx, pipeline, (batch, sizes[0]))
+    y = wk.Tensor.alloc(dtype, ctx, pipeline, (batch, sizes[-1]))
+    wk.memory.readFromBuffer(pipeline, x, synth.normal(synth.config_seed(5, 8), (batch, sizes[0]), rd))
+    wk.memory.readFromBuffer(pipeline, y, synth.uniform(synth.config_seed(5, 9), (batch, sizes[-1]), rd, 0.0, 1.0))
+    cache = nn.Cache.init(ctx, pipeline, batch, [seq])
+    lc = cache.getLayerCache(0)
+    opt = nn.optimizers.Adam.init(dtype, lr) if optimizer == "adam" else nn.optimizers.GD.init(dtype, lr)
+
+    def step():
+        out = seq.forward(pipeline, x, lc)
+        nn.loss.mse(True, pipeline, out, y, cache, None)
+        seq.backward(pipeline, lc, x, None)
+        opt.step(pipeline, cache)
+
+    for _ in range(warmup):
+        step()
+    pipeline.waitAndCleanup()
+    lib = wk._capi.load()
+    stream = wk._lib().wkz_context_stream(ctx._h, 0)
+    device = wk._lib().wkz_context_device(ctx._h)
+    e0, e1 = ctypes.c_void_p(), ctypes.c_void_p()
+    wk._capi.check(lib.wk_event_create(device, ctypes.byref(e0)))
+    wk._capi.check(lib.wk_event_create(device, ctypes.byref(e1)))
+    t0 = time.perf_counter()
+    wk._capi.check(lib.wk_event_record(e0, stream))
+    for _ in range(steps):
+        step()
+    wk._capi.check(lib.wk_event_record(e1, stream))
+    pipeline.waitAndCleanup()
+    wall_ms = (time.perf_counter() - t0) * 1e3 / steps
+    ms = ctypes.c_float()
+    wk._capi.check(lib.wk_event_elapsed_ms(e0, e1, ctypes.byref(ms)))
+    loss = np.zeros(1, dtype=rd)
+    nn.loss.mse(False, pipeline, seq.forward(pipeline, x, lc), y, cache, loss)
+    lib.wk_event_destroy(e0)
+    lib.wk_event_destroy(e1)
+    opt.deinit(pipeline)
+    cache.deinit(pipeline)
+    seq.deinit(pipeline)
+    x.release(pipeline)
+    y.release(pipeline)
+    pipeline.deinit()
+    ctx.deinit()
+    flops = mlp_flops(sizes, batch)
+    return {"stream_ms": ms.value / steps, "wall_ms": wall_ms, "flops": flops, "tflops": flops / (ms.value / steps) / 1e9,
+            "loss_after": float(loss[0])}
+
+
+def cmd_mlp(args):
+    r = time_mlp_step(args.dtype, tuple(args.sizes), args.batch, args.optimizer, args.lr, args.steps, args.warmup)
+    print(f"mlp {'-'.join(map(str, args.sizes))} {args.dtype} batch {args.batch} {args.optimizer}: "
+          f"{r['stream_ms']:.3f} ms/step on the stream, {r['wall_ms']:.3f} ms/step wall, "
+          f"{r['tflops']:.1f} TFLOP/s over {r['flops'] / 1e9:.1f} GFLOP of GEMM work, "
+          f"mse after {args.steps + args.warmup} steps {r['loss_after']:.5f}")
+
+
 def main(argv=None):
     ap = argparse.ArgumentParser(prog="python -m wekua_amd.benchmark")
     sub = ap.add_subparsers(dest="cmd", required=True)
@@ -115,7 +200,18 @@ def main(argv=None):
     a.add_argument("--dtype", default="f32")
     c = sub.add_parser("configs")
     c.add_argument("--variant", default="auto")
+    m = sub.add_parser("mlp")
+    m.add_argument("--dtype", default="f32")
+    m.add_argument("--sizes", type=int, nargs="+", default=[1024, 4096, 4096, 1024])
+    m.add_argument("--batch", type=int, default=2048)
+    m.add_argument("--optimizer", choices=["adam", "gd"], default="adam")
+    m.add_argument("--lr", type=float, default=1e-3)
+    m.add_argument("--steps", type=int, default=20)
+    m.add_argument("--warmup", type=int, default=3)
     args = ap.parse_args(argv)
+    if args.cmd == "mlp":
+        cmd_mlp(args)
+        return 0
     dev = raw.Device(0)
     try:
         if getattr(args, "variant", "auto") != "auto":

@@ -571,17 +571,18 @@ int launch_f64(hipStream_t st, const GemmProblem &p, bool edge) {
 struct VariantDesc {
     const char *name;
     int dtype, bm, bn, bk;
-    double efficiency; // relative matrix-pipe efficiency of the tile shape (0: never auto-selected)
+    double efficiency; // fraction of the matrix peak this tile shape sustains over many rounds (0: never auto-selected)
+    double fill;       // start-up and drain of a launch, in units of one round of tiles
     int (*launch)(hipStream_t, const GemmProblem &, bool);
 };
 
 const VariantDesc k_variants[] = {
-    {"mfma_f32_256x128", WK_F32, 256, 128, 16, 1.00, &launch_f32<256, 128, 16, 2, 2, 2>},
-    {"mfma_f32_128x128", WK_F32, 128, 128, 16, 0.96, &launch_f32<128, 128, 16, 2, 2, 3>},
-    {"mfma_f32_64x64", WK_F32, 64, 64, 16, 0.85, &launch_f32<64, 64, 16, 2, 2, 4>},
-    {"mfma_f64_128x128", WK_F64, 128, 128, 16, 1.00, &launch_f64<128, 128, 16, 2, 2, 2>},
-    {"mfma_f64_64x64", WK_F64, 64, 64, 16, 0.92, &launch_f64<64, 64, 16, 2, 2, 4>},
-    {"mfma_f64_128x64", WK_F64, 128, 64, 16, 0.97, &launch_f64<128, 64, 16, 2, 2, 3>},
+    {"mfma_f32_256x128", WK_F32, 256, 128, 16, 0.943, 0.25, &launch_f32<256, 128, 16, 2, 2, 2>},
+    {"mfma_f32_128x128", WK_F32, 128, 128, 16, 0.885, 0.25, &launch_f32<128, 128, 16, 2, 2, 3>},
+    {"mfma_f32_64x64", WK_F32, 64, 64, 16, 0.730, 0.10, &launch_f32<64, 64, 16, 2, 2, 4>},
+    {"mfma_f64_128x128", WK_F64, 128, 128, 16, 0.908, 0.20, &launch_f64<128, 128, 16, 2, 2, 2>},
+    {"mfma_f64_64x64", WK_F64, 64, 64, 16, 0.800, 0.22, &launch_f64<64, 64, 16, 2, 2, 4>},
+    {"mfma_f64_128x64", WK_F64, 128, 64, 16, 0.863, 0.25, &launch_f64<128, 64, 16, 2, 2, 3>},
 };
 constexpr int k_num_variants = sizeof(k_variants) / sizeof(k_variants[0]);
 
@@ -605,12 +606,16 @@ int wk::gemm_mfma_variant_dtype(int variant) {
 }
 
 // Kernel choice by a small cost model.  The matrix pipes of a CU are saturated by the work-groups
-// resident on it, so a launch takes about (tiles on the busiest CU) x (tile area / efficiency):
-//     cost = ceil(tiles / CUs) * BM * BN / efficiency
-// with the efficiency of each macro tile relative to the largest measured at 4096^3 on MI355X
-// (f32: 122 / 118 / 106 TFLOP/s; f64 similarly).  This picks big tiles for big problems, small
-// tiles when the big ones would leave CUs idle (1024^3, tall-skinny) or quantise badly
-// (4097 x 4095: 544 tiles of 256x128 put three tiles on some CUs and two on the rest).
+// resident on it, so a launch takes about (tiles on the busiest CU + a start-up/drain share) x
+// (tile area / efficiency):
+//     cost = (ceil(tiles / CUs) + fill) * BM * BN / efficiency
+// `efficiency` and `fill` are fitted per macro tile to times measured on MI355X over launches of
+// one to sixteen rounds (f32 256x128: 123 TFLOP/s at one tile per CU, 130 at two, 143.6 at eight;
+// 128x128: 112 / 128 / 137 at one / two / sixteen; f64 alike).  This picks big tiles for big
+// problems, the next size down while the big one would run a single round (a lone work-group per
+// CU has nothing to overlap its hand-overs and epilogue with), small tiles when the others would
+// leave CUs idle (1024^3, tall-skinny) or quantise badly (4097 x 4095: 544 tiles of 256x128 put
+// three tiles on some CUs and two on the rest).
 int wk::gemm_mfma_pick(const GemmProblem &p) {
     if (p.dtype != WK_F32 && p.dtype != WK_F64) return -1;
     if (p.M > 0x7fffffffull || p.N > 0x7fffffffull || p.K > 0x7fffffffull || p.lda > 0x7fffffffull ||
@@ -624,7 +629,7 @@ int wk::gemm_mfma_pick(const GemmProblem &p) {
         if (d.dtype != p.dtype || d.efficiency <= 0.0) continue;
         const double tiles = (double)((p.M + d.bm - 1) / d.bm) * (double)((p.N + d.bn - 1) / d.bn);
         const double rounds = (double)(uint64_t)((tiles + cus - 1.0) / cus);
-        const double cost = rounds * d.bm * d.bn / d.efficiency;
+        const double cost = (rounds + d.fill) * d.bm * d.bn / d.efficiency;
         if (best < 0 || cost < best_cost) {
             best = v;
             best_cost = cost;

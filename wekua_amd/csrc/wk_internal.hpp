@@ -16,7 +16,13 @@ struct wk_device {
 struct wk_stream {
     wk_device *dev;
     hipStream_t stream;
+    // Device memory for partial results of two-pass reductions launched on this stream (the
+    // stream is in order, so consecutive users never overlap).  Allocated with the stream.
+    void *scratch;
+    size_t scratch_bytes;
 };
+
+constexpr size_t WK_STREAM_SCRATCH_BYTES = 1u << 20;
 
 struct wk_event {
     wk_device *dev;

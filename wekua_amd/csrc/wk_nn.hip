@@ -119,20 +119,37 @@ template <typename F> int dispatch_float(int dtype, F &&f) {
     return dtype >= 0 && dtype < WK_DTYPE_COUNT ? WK_E_TYPE_NOT_SUPPORTED : WK_E_TYPE_NOT_SUPPORTED;
 }
 
-// ---- column sums (bias_step.cl): one thread per column walks the rows; consecutive threads read
-// consecutive addresses of each row, so every row access is one coalesced run. --------------
+// ---- column sums (bias_step.cl).  Rows are cut into `chunks` bands; a block of 64 x 4 threads
+// sums 64 columns of one band (consecutive lanes read consecutive addresses of a row, four rows
+// in flight per block) and writes one partial per column; a second pass adds the bands in a fixed
+// order, so the result does not depend on scheduling. --------------------------------------------
+constexpr int COLSUM_ROWS_PER_BAND = 32;
+constexpr int COLSUM_MAX_BANDS = 64;
+
 template <typename T>
-__global__ __launch_bounds__(256) void colsum_kernel(const T *__restrict__ x, uint64_t rows, uint64_t cols, uint64_t pitch,
-                                                     T *__restrict__ out) {
-    // blockDim = (64, 4): 64 columns per block, rows split 4 ways, combined through LDS
+__global__ __launch_bounds__(256) void colsum_bands_kernel(const T *__restrict__ x, uint64_t rows, uint64_t cols, uint64_t pitch,
+                                                           uint64_t band_rows, T *__restrict__ partial) {
     __shared__ T part[4][64];
     const uint64_t c = blockIdx.x * 64ull + threadIdx.x;
+    const uint64_t r0 = blockIdx.y * band_rows;
+    const uint64_t r1 = r0 + band_rows < rows ? r0 + band_rows : rows;
     T acc = T(0);
     if (c < cols)
-        for (uint64_t r = threadIdx.y; r < rows; r += 4) acc += x[r * pitch + c];
+        for (uint64_t r = r0 + threadIdx.y; r < r1; r += 4) acc += x[r * pitch + c];
     part[threadIdx.y][threadIdx.x] = acc;
     __syncthreads();
-    if (threadIdx.y == 0 && c < cols) out[c] = (part[0][threadIdx.x] + part[1][threadIdx.x]) + (part[2][threadIdx.x] + part[3][threadIdx.x]);
+    if (threadIdx.y == 0 && c < cols)
+        partial[blockIdx.y * cols + c] = (part[0][threadIdx.x] + part[1][threadIdx.x]) + (part[2][threadIdx.x] + part[3][threadIdx.x]);
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void colsum_finish_kernel(const T *__restrict__ partial, uint64_t bands, uint64_t cols,
+                                                            T *__restrict__ out) {
+    const uint64_t c = blockIdx.x * 256ull + threadIdx.x;
+    if (c >= cols) return;
+    T acc = T(0);
+    for (uint64_t b = 0; b < bands; ++b) acc += partial[b * cols + c];
+    out[c] = acc;
 }
 
 // ---- whole-tensor sum (math.sum + host finish, src/math/basic.zig:128-203): two fixed-shape
@@ -238,9 +255,23 @@ int wk_bias_step(wk_stream *s, int dtype, uint64_t rows, uint64_t cols, const vo
     int rc = bind(s);
     if (rc) return rc;
     if (!rows || !cols || !sens || !bias_grad || pitch < cols) return WK_E_INVALID_VALUE;
+    if ((cols + 63) / 64 > 0x7fffffffull) return WK_E_INVALID_VALUE;
     return dispatch_float(dtype, [&]<typename T>() -> int {
-        hipLaunchKernelGGL((colsum_kernel<T>), dim3((unsigned)((cols + 63) / 64)), dim3(64, 4), 0, s->stream,
-                           static_cast<const T *>(sens), rows, cols, pitch, static_cast<T *>(bias_grad));
+        // as many bands as the stream's scratch holds partials for; one band writes the result directly
+        uint64_t bands = (rows + COLSUM_ROWS_PER_BAND - 1) / COLSUM_ROWS_PER_BAND;
+        if (bands > COLSUM_MAX_BANDS) bands = COLSUM_MAX_BANDS;
+        const uint64_t fit = s->scratch_bytes / (cols * sizeof(T));
+        if (bands > fit) bands = fit;
+        if (bands < 2) bands = 1;
+        const uint64_t band_rows = (rows + bands - 1) / bands;
+        bands = (rows + band_rows - 1) / band_rows;
+        T *partial = bands > 1 ? static_cast<T *>(s->scratch) : static_cast<T *>(bias_grad);
+        hipLaunchKernelGGL((colsum_bands_kernel<T>), dim3((unsigned)((cols + 63) / 64), (unsigned)bands), dim3(64, 4), 0,
+                           s->stream, static_cast<const T *>(sens), rows, cols, pitch, band_rows, partial);
+        int lrc = launch_status();
+        if (lrc || bands == 1) return lrc;
+        hipLaunchKernelGGL((colsum_finish_kernel<T>), dim3((unsigned)((cols + 255) / 256)), dim3(256), 0, s->stream,
+                           static_cast<const T *>(partial), bands, cols, static_cast<T *>(bias_grad));
         return launch_status();
     });
 }

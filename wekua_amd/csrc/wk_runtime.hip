@@ -98,12 +98,22 @@ int wk_stream_create(wk_device *dev, wk_stream **out) {
     wk_stream *s = new (std::nothrow) wk_stream;
     if (!s) return WK_E_OUT_OF_MEMORY;
     s->dev = dev;
+    s->scratch = nullptr;
+    s->scratch_bytes = 0;
     hipError_t e = hipStreamCreateWithFlags(&s->stream, hipStreamNonBlocking);
     if (e != hipSuccess) {
         (void)hipGetLastError();
         delete s;
         return hip_code(e);
     }
+    e = hipMalloc(&s->scratch, WK_STREAM_SCRATCH_BYTES);
+    if (e != hipSuccess) {
+        (void)hipGetLastError();
+        (void)hipStreamDestroy(s->stream);
+        delete s;
+        return hip_code(e);
+    }
+    s->scratch_bytes = WK_STREAM_SCRATCH_BYTES;
     *out = s;
     return WK_OK;
 }
@@ -113,6 +123,7 @@ void wk_stream_destroy(wk_stream *s) {
     if (hipSetDevice(s->dev->ordinal) == hipSuccess) {
         (void)hipStreamSynchronize(s->stream);
         (void)hipStreamDestroy(s->stream);
+        if (s->scratch) (void)hipFree(s->scratch);
     }
     (void)hipGetLastError();
     delete s;
