@@ -7,8 +7,10 @@ times over 1-D sizes, on GPU 0.
     python -m wekua_amd.benchmark configs        # every BASELINE GEMM / AXPY configuration, one line each
     python -m wekua_amd.benchmark mlp [--dtype f32] [--sizes 1024 4096 4096 1024] [--batch 2048] [--optimizer adam]
 
+Everything goes through the reference-shaped API (Tensor.alloc, memory.readFromBuffer, blas.*).
 Unlike the reference's harness the inputs are seeded (wekua_amd.synth), times come from
-events on the kernel's stream, and every line also gives the rate (TFLOP/s or GB/s).
+events on the pipeline's stream after a warm-up by time, and every line also gives the rate
+(TFLOP/s or GB/s).
 """
 from __future__ import annotations
 
@@ -28,77 +30,123 @@ def _operand(rd, shape, seed):
     return synth.integers(seed, shape, rd, -100, 100)
 
 
-def time_gemm(dev, dtype, M, N, K, op_a, op_b, alpha, beta, iters=10, warmup=2):
+class Session:
+    """One Context + Pipeline and the event pair used to time launches on the pipeline's stream."""
+
+    def __init__(self):
+        import ctypes
+
+        import wekua_amd as wk
+        self.wk, self.ct = wk, ctypes
+        self.ctx = wk.Context.initFromDeviceType(wk.DeviceType.all)
+        self.pipeline = wk.Pipeline.init(self.ctx.command_queues[0])
+        self.lib = wk._capi.load()
+        self.stream = wk._lib().wkz_context_stream(self.ctx._h, 0)
+        device = wk._lib().wkz_context_device(self.ctx._h)
+        self.e0, self.e1 = ctypes.c_void_p(), ctypes.c_void_p()
+        wk._capi.check(self.lib.wk_event_create(device, ctypes.byref(self.e0)))
+        wk._capi.check(self.lib.wk_event_create(device, ctypes.byref(self.e1)))
+
+    def close(self):
+        self.lib.wk_event_destroy(self.e0)
+        self.lib.wk_event_destroy(self.e1)
+        self.pipeline.deinit()
+        self.ctx.deinit()
+
+    def tensor(self, dtype, host):
+        t = self.wk.Tensor.alloc(dtype, self.ctx, self.pipeline, host.shape)
+        self.wk.memory.readFromBuffer(self.pipeline, t, host)
+        return t
+
+    def time_ms(self, call, iters, warm_seconds=0.15):
+        """ms per call from events on the stream, after keeping the device busy for `warm_seconds`
+        (short kernels measured right after an upload see the clocks still ramping)."""
+        import time
+        t0 = time.perf_counter()
+        while True:
+            for _ in range(4):
+                call()
+            self.pipeline.waitAndCleanup()
+            if time.perf_counter() - t0 >= warm_seconds:
+                break
+        check = self.wk._capi.check
+        check(self.lib.wk_event_record(self.e0, self.stream))
+        for _ in range(iters):
+            call()
+        check(self.lib.wk_event_record(self.e1, self.stream))
+        self.pipeline.waitAndCleanup()
+        ms = self.ct.c_float()
+        check(self.lib.wk_event_elapsed_ms(self.e0, self.e1, self.ct.byref(ms)))
+        return ms.value / iters
+
+
+def time_gemm(ses, dtype, M, N, K, op_a, op_b, alpha, beta, iters=10):
+    """blas.gemm on tensors created by Tensor.alloc (so with the library's own row pitches)."""
     rd = raw.real_np_dtype(dtype)
-    a = _operand(rd, (K, M) if op_a else (M, K), 1)
-    b = _operand(rd, (N, K) if op_b else (K, N), 2)
-    c = _operand(rd, (M, N), 3)
-    dA, dB, dC = dev.upload(a), dev.upload(b), dev.upload(c)
-    call = lambda: dev.gemm(dtype, op_a, op_b, M, N, K, alpha, dA, a.shape[1], dB, b.shape[1], beta, dC, N)
-    for _ in range(warmup):
-        call()
-    dev.sync()
-    ms = dev.time_stream_ms(call, iters)
-    variant = dev.lib.wk_gemm_variant(raw.dtype_id(dtype), op_a, op_b, M, N, K, a.shape[1], b.shape[1], N,
-                                      dA.ptr, dB.ptr, dC.ptr).decode()
-    for d in (dA, dB, dC):
-        d.free()
+    wk = ses.wk
+    A = ses.tensor(dtype, _operand(rd, (K, M) if op_a else (M, K), 1))
+    B = ses.tensor(dtype, _operand(rd, (N, K) if op_b else (K, N), 2))
+    C = ses.tensor(dtype, _operand(rd, (M, N), 3))
+    ses.pipeline.waitAndCleanup()
+    ms = ses.time_ms(lambda: wk.blas.gemm(ses.pipeline, alpha, A, op_a, B, op_b, beta, C, None), iters)
+    variant = ses.lib.wk_gemm_variant(raw.dtype_id(dtype), op_a, op_b, M, N, K, A.row_pitch, B.row_pitch, C.row_pitch,
+                                      A.buffer, B.buffer, C.buffer).decode()
+    for t in (A, B, C):
+        t.release(ses.pipeline)
     return ms, variant
 
 
-def time_axpy(dev, dtype, n, iters=50, warmup=3):
+def time_axpy(ses, dtype, n, iters=50):
     rd = raw.real_np_dtype(dtype)
-    x, y = _operand(rd, (n,), 1), _operand(rd, (n,), 2)
-    dx, dy = dev.upload(x), dev.upload(y)
-    call = lambda: dev.axpy(dtype, (1, 1, n), dx, n, n, 0.75 if rd.kind == "f" else 3, dy, n, n)
-    for _ in range(warmup):
-        call()
-    dev.sync()
-    ms = dev.time_stream_ms(call, iters)
-    dx.free()
-    dy.free()
+    wk = ses.wk
+    x, y = ses.tensor(dtype, _operand(rd, (n,), 1)), ses.tensor(dtype, _operand(rd, (n,), 2))
+    ses.pipeline.waitAndCleanup()
+    alpha = 0.75 if rd.kind == "f" else 3
+    ms = ses.time_ms(lambda: wk.blas.axpy(ses.pipeline, x, alpha, y), iters)
+    x.release(ses.pipeline)
+    y.release(ses.pipeline)
     return ms
 
 
-def cmd_gemm(dev, args):
+def cmd_gemm(ses, args):
     print(f"{'dtype':5s} {'n':>6s} {'op':2s} {'ms':>9s} {'TFLOP/s':>9s}  kernel")
     for n in args.sizes:
         for op_a, op_b, name in OPS:
-            ms, variant = time_gemm(dev, args.dtype, n, n, n, op_a, op_b, 1.5 if args.dtype[0] == "f" else 3,
+            ms, variant = time_gemm(ses, args.dtype, n, n, n, op_a, op_b, 1.5 if args.dtype[0] == "f" else 3,
                                     0.5 if args.dtype[0] == "f" else 2)
             print(f"{args.dtype:5s} {n:6d} {name:2s} {ms:9.4f} {2.0 * n ** 3 / ms / 1e9:9.2f}  {variant}", flush=True)
 
 
-def cmd_axpy(dev, args):
+def cmd_axpy(ses, args):
     print(f"{'dtype':5s} {'n':>10s} {'us':>9s} {'GB/s':>8s}")
     for lg in range(12, 29):
         n = 1 << lg
-        ms = time_axpy(dev, args.dtype, n)
+        ms = time_axpy(ses, args.dtype, n)
         nbytes = 3 * n * raw.elem_size(args.dtype)
         print(f"{args.dtype:5s} {n:10d} {ms * 1e3:9.2f} {nbytes / ms / 1e6:8.0f}", flush=True)
 
 
-def cmd_configs(dev, args):
+def cmd_configs(ses, args):
     rows = []
-    ms, v = time_gemm(dev, "f32", 512, 512, 512, 0, 0, 1.0, 0.0)
+    ms, v = time_gemm(ses, "f32", 512, 512, 512, 0, 0, 1.0, 0.0)
     rows.append(("1 f32 512^3 NN a=1 b=0", ms, 2 * 512 ** 3 / ms / 1e9, "TFLOP/s", v))
     for dt in ("f32", "f64"):
         for lg in (20, 24, 28):
-            ms = time_axpy(dev, dt, 1 << lg)
+            ms = time_axpy(ses, dt, 1 << lg)
             rows.append((f"2 axpy {dt} n=2^{lg}", ms, 3 * (1 << lg) * raw.elem_size(dt) / ms / 1e6, "GB/s", "axpy_stream"))
     for n in (1024, 2048, 4096, 8192):
         for op_a, op_b, name in OPS:
-            ms, v = time_gemm(dev, "f32", n, n, n, op_a, op_b, 1.5, 0.5)
+            ms, v = time_gemm(ses, "f32", n, n, n, op_a, op_b, 1.5, 0.5)
             rows.append((f"3 f32 {n}^3 {name}", ms, 2.0 * n ** 3 / ms / 1e9, "TFLOP/s", v))
     for (M, N, K) in ((1000, 1000, 1000), (4097, 4095, 4093)):
         for op_a, op_b, name in OPS:
-            ms, v = time_gemm(dev, "f32", M, N, K, op_a, op_b, 1.5, 0.5)
+            ms, v = time_gemm(ses, "f32", M, N, K, op_a, op_b, 1.5, 0.5)
             rows.append((f"3 f32 {M}x{N}x{K} {name}", ms, 2.0 * M * N * K / ms / 1e9, "TFLOP/s", v))
-    ms, v = time_gemm(dev, "f64", 4096, 4096, 4096, 0, 0, 1.0, 1.0)
+    ms, v = time_gemm(ses, "f64", 4096, 4096, 4096, 0, 0, 1.0, 1.0)
     rows.append(("4 f64 4096^3 NN", ms, 2.0 * 4096 ** 3 / ms / 1e9, "TFLOP/s", v))
-    ms, v = time_gemm(dev, "f64", 8192, 256, 8192, 0, 0, 1.0, 1.0)
+    ms, v = time_gemm(ses, "f64", 8192, 256, 8192, 0, 0, 1.0, 1.0)
     rows.append(("4 f64 8192x256x8192 NN", ms, 2.0 * 8192 * 256 * 8192 / ms / 1e9, "TFLOP/s", v))
-    ms, v = time_gemm(dev, "i32", 2048, 2048, 2048, 0, 0, 3, -2)
+    ms, v = time_gemm(ses, "i32", 2048, 2048, 2048, 0, 0, 3, -2)
     rows.append(("4 i32 2048^3 NN", ms, 2.0 * 2048 ** 3 / ms / 1e9, "TOP/s", v))
     print(f"{'config':34s} {'ms':>9s} {'rate':>9s} unit     kernel")
     for name, ms, rate, unit, v in rows:
@@ -212,13 +260,13 @@ def main(argv=None):
     if args.cmd == "mlp":
         cmd_mlp(args)
         return 0
-    dev = raw.Device(0)
+    ses = Session()
     try:
         if getattr(args, "variant", "auto") != "auto":
-            raw.check(dev.lib.wk_gemm_force_variant(args.variant.encode()), "wk_gemm_force_variant")
-        {"gemm": cmd_gemm, "axpy": cmd_axpy, "configs": cmd_configs}[args.cmd](dev, args)
+            raw.check(ses.lib.wk_gemm_force_variant(args.variant.encode()), "wk_gemm_force_variant")
+        {"gemm": cmd_gemm, "axpy": cmd_axpy, "configs": cmd_configs}[args.cmd](ses, args)
     finally:
-        dev.close()
+        ses.close()
     return 0
 
 

@@ -121,8 +121,8 @@ template <typename F> int dispatch_float(int dtype, F &&f) {
 
 // ---- column sums (bias_step.cl).  Rows are cut into `chunks` bands; a block of 64 x 4 threads
 // sums 64 columns of one band (consecutive lanes read consecutive addresses of a row, four rows
-// in flight per block) and writes one partial per column; a second pass adds the bands in a fixed
-// order, so the result does not depend on scheduling. --------------------------------------------
+// in flight per block) and writes one partial per column; a second pass runs the same kernel over
+// the partials, so the order of additions is fixed and the result does not depend on scheduling. --------------------------------------------
 constexpr int COLSUM_ROWS_PER_BAND = 32;
 constexpr int COLSUM_MAX_BANDS = 64;
 
@@ -140,16 +140,6 @@ __global__ __launch_bounds__(256) void colsum_bands_kernel(const T *__restrict__
     __syncthreads();
     if (threadIdx.y == 0 && c < cols)
         partial[blockIdx.y * cols + c] = (part[0][threadIdx.x] + part[1][threadIdx.x]) + (part[2][threadIdx.x] + part[3][threadIdx.x]);
-}
-
-template <typename T>
-__global__ __launch_bounds__(256) void colsum_finish_kernel(const T *__restrict__ partial, uint64_t bands, uint64_t cols,
-                                                            T *__restrict__ out) {
-    const uint64_t c = blockIdx.x * 256ull + threadIdx.x;
-    if (c >= cols) return;
-    T acc = T(0);
-    for (uint64_t b = 0; b < bands; ++b) acc += partial[b * cols + c];
-    out[c] = acc;
 }
 
 // ---- whole-tensor sum (math.sum + host finish, src/math/basic.zig:128-203): two fixed-shape
@@ -270,8 +260,9 @@ int wk_bias_step(wk_stream *s, int dtype, uint64_t rows, uint64_t cols, const vo
                            s->stream, static_cast<const T *>(sens), rows, cols, pitch, band_rows, partial);
         int lrc = launch_status();
         if (lrc || bands == 1) return lrc;
-        hipLaunchKernelGGL((colsum_finish_kernel<T>), dim3((unsigned)((cols + 255) / 256)), dim3(256), 0, s->stream,
-                           static_cast<const T *>(partial), bands, cols, static_cast<T *>(bias_grad));
+        // second pass: the same kernel over the bands x cols matrix of partials, as one band
+        hipLaunchKernelGGL((colsum_bands_kernel<T>), dim3((unsigned)((cols + 63) / 64), 1), dim3(64, 4), 0, s->stream,
+                           static_cast<const T *>(partial), bands, cols, cols, bands, static_cast<T *>(bias_grad));
         return launch_status();
     });
 }

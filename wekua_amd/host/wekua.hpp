@@ -25,7 +25,7 @@
 //     prevEvents()/append() bookkeeping callers rely on; waitAndCleanup() syncs the stream;
 //   * Tensor rows are padded to 16 bytes (the per-lane load width of gfx950), not to an
 //     even vector count, row counts are not padded at all, and row pitches that are a
-//     multiple of 1 KiB are skewed by 1056 bytes to avoid cache-set / channel aliasing;
+//     multiple of 1 KiB and at least 16 KiB are skewed by 512 bytes to avoid channel aliasing;
 //   * PackedTensors allocates nothing: the HIP kernels tile straight from the row-major
 //     operands through LDS, so pack() only validates.
 #pragma once
@@ -277,12 +277,13 @@ template <typename T> struct Tensor {
 
         uint64_t row_pitch = cols;
         if (vw > 1 && row_pitch % vw) row_pitch += vw - row_pitch % vw;
-        // Rows whose byte pitch is a multiple of 1 KiB land on the same L2 sets and memory
-        // channels (measured on MI355X: f32 gemm at 8192^3 runs at 135 TFLOP/s with a pitch of
-        // 32768 bytes and 139 with 32768 + 1056).  The layout is ours to choose, so such pitches
-        // are skewed by 1056 bytes.
-        if (rows * depth > 1 && row_pitch * sizeof(T) >= 4096 && (row_pitch * sizeof(T)) % 1024 == 0)
-            row_pitch += 1056 / sizeof(T);
+        // Long rows whose byte pitch is a multiple of 1 KiB land on the same memory channels
+        // (measured on MI355X, f32 gemm NN: 8192^3 runs at 135.8 TFLOP/s with a pitch of 32768
+        // bytes and at 140 with 32768 + 512; 4096^3 and 2048^3 do not care; at 1024^3 any skew
+        // costs a quarter of the rate).  The layout is ours to choose, so pitches from 16 KiB
+        // up are skewed by 512 bytes, which keeps row starts on cache-line boundaries.
+        if (rows * depth > 1 && row_pitch * sizeof(T) >= 16384 && (row_pitch * sizeof(T)) % 1024 == 0)
+            row_pitch += 512 / sizeof(T);
 
         t->dimensions.number_of_elements_without_padding = depth * rows * cols;
         t->memory_layout.row_pitch = row_pitch;
