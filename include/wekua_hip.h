@@ -208,6 +208,32 @@ int  wk_adam_step(wk_stream *s, int dtype, const uint64_t shape3[3], void *w, ui
                   const void *g, uint64_t g_row_pitch, uint64_t g_slice_pitch, void *m, void *v, uint64_t mv_row_pitch,
                   uint64_t mv_slice_pitch, double lr, double beta1, double beta2, double eps, uint64_t step);
 
+/* ---- tensor support operations (src/tensor) --------------------------------------------------- */
+#define WK_MAX_DIMS 8
+/* transpose (src/tensor/transpose.zig:14-105, kernels/transpose.cl): swaps dimensions dim0 != dim1 of an
+ * ndim-dimensional tensor (ndim <= WK_MAX_DIMS).  `shape` and `src_pitches` describe the source,
+ * `dst_pitches` the destination, whose shape is `shape` with the two dimensions exchanged; pitches are
+ * element strides per dimension (the last is 1), as Tensor.dimensions.pitches (src/tensor/main.zig:198-220). */
+int  wk_transpose(wk_stream *s, int dtype, int ndim, const uint64_t *shape, const uint64_t *src_pitches,
+                  const uint64_t *dst_pitches, int dim0, int dim1, const void *src, void *dst);
+/* random.uniform (src/tensor/random/uniform.zig:60-135, kernels/uniform.cl).  host_min == NULL: floats
+ * hash / 2^64 in [0, 1], integers the low bits of the hash.  Otherwise host_min / host_range point to
+ * one value of the real component type and every value is min + hash / 2^64 * range, formed in double.
+ * The hash is the reference's; it is keyed on the LOGICAL element index (complex: 2*index, 2*index + 1),
+ * where the reference keys it on the index in its padded layout, so the two streams agree exactly when
+ * the reference's tensor has no padding. */
+int  wk_random_uniform(wk_stream *s, int dtype, const uint64_t shape3[3], void *ptr, uint64_t row_pitch, uint64_t slice_pitch,
+                       uint64_t seed, const void *host_min, const void *host_range);
+/* The hash random.uniform draws from (kernels/uniform.cl:31-55), on the host. */
+uint64_t wk_random_hash(uint64_t index, uint64_t seed);
+/* toComplex / toReal (src/tensor/convertions/to_complex.zig:52-98, to_real.zig:51-97): copy a real
+ * tensor into the real (space 0) or imaginary (space 1) components of a complex one, or back.
+ * real_dtype is the id of the component type (0..9); pitches are in elements of each tensor's own type. */
+int  wk_to_complex(wk_stream *s, int real_dtype, const uint64_t shape3[3], const void *src, uint64_t src_row_pitch,
+                   uint64_t src_slice_pitch, void *dst, uint64_t dst_row_pitch, uint64_t dst_slice_pitch, int space);
+int  wk_to_real(wk_stream *s, int real_dtype, const uint64_t shape3[3], const void *src, uint64_t src_row_pitch,
+                uint64_t src_slice_pitch, void *dst, uint64_t dst_row_pitch, uint64_t dst_slice_pitch, int space);
+
 /* A plain device-to-device streaming copy kernel of known size, used only to calibrate
  * profiler byte counters against a known amount of traffic. */
 int wk_copy_kernel(wk_stream *s, void *dst, const void *src, size_t bytes);

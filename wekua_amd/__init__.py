@@ -81,6 +81,14 @@ HOST_SIGNATURES = {
     "wkz_packed_deinit": (ci, [vp, vp]),
     "wkz_packed_pack": (ci, [vp, vp, vp, ci, vp, ci]),
     "wkz_gemm": (ci, [vp, vp, vp, ci, vp, ci, vp, vp, vp]),
+    # tensor support operations
+    "wkz_memory_copy": (ci, [vp, vp, vp]),
+    "wkz_get_value": (ci, [vp, vp, u64p, u64, vp]),
+    "wkz_put_value": (ci, [vp, vp, u64p, u64, vp]),
+    "wkz_transpose": (ci, [vp, vp, vp, u64, u64]),
+    "wkz_random_uniform": (ci, [vp, vp, u64p, vp, vp]),
+    "wkz_to_complex": (ci, [vp, vp, vp, ci]),
+    "wkz_to_real": (ci, [vp, vp, vp, ci]),
     # math / nn (the MLP training step)
     "wkz_math_dot": (ci, [vp, vp, vp]),
     "wkz_math_sum": (ci, [vp, vp, vp]),
@@ -299,6 +307,29 @@ class memory:
         _check(_lib().wkz_write_to_buffer(pipeline._h, tensor._h, buffer.ctypes.data, n), "memory.writeToBuffer")
 
 
+    @staticmethod
+    def copy(pipeline: Pipeline, src: Tensor, dst: Tensor) -> None:
+        """memory.copy (src/tensor/memory/copy.zig): DEVICE -> DEVICE of the logical region."""
+        _check(_lib().wkz_memory_copy(pipeline._h, src._h, dst._h), "memory.copy")
+
+    @staticmethod
+    def getValue(pipeline: Pipeline, tensor: Tensor, coor, scalar: np.ndarray) -> None:
+        """memory.getValue: non-blocking read of one element into `scalar` (a 1-element array of the
+        tensor's dtype; complex: 2 elements), valid after pipeline.waitAndCleanup()."""
+        c = (u64 * max(len(coor), 1))(*coor)
+        if scalar.dtype != real_np_dtype(tensor.dtype) or scalar.size != (2 if is_complex(tensor.dtype) else 1):
+            raise TypeError("getValue needs an array holding exactly one element of the tensor's dtype")
+        _check(_lib().wkz_get_value(pipeline._h, tensor._h, c, len(coor), scalar.ctypes.data), "memory.getValue")
+
+    @staticmethod
+    def putValue(pipeline: Pipeline, tensor: Tensor, coor, value) -> None:
+        """memory.putValue: write one element."""
+        c = (u64 * max(len(coor), 1))(*coor)
+        keep, p = _scalar_ptr(tensor.dtype, value)
+        _check(_lib().wkz_put_value(pipeline._h, tensor._h, c, len(coor), p), "memory.putValue")
+        pipeline._keepalive = getattr(pipeline, "_keepalive", []) + [keep]
+
+
 class fill:
     @staticmethod
     def zeroes(pipeline: Pipeline, tensor: Tensor) -> None:
@@ -316,6 +347,43 @@ class fill:
 
 def identity(pipeline: Pipeline, tensor: Tensor) -> None:
     _check(_lib().wkz_identity(pipeline._h, tensor._h), "identity")
+
+
+def transpose(pipeline: Pipeline, result_tensor: Tensor, tensor: Tensor, dim0: int, dim1: int) -> None:
+    """tensor.transpose (src/tensor/transpose.zig): result = tensor with dim0 and dim1 exchanged."""
+    _check(_lib().wkz_transpose(pipeline._h, result_tensor._h, tensor._h, dim0, dim1), "transpose")
+
+
+class Space(enum.IntEnum):
+    real = 0
+    imag = 1
+
+
+class random:
+    @staticmethod
+    def uniform(pipeline: Pipeline, tensor: Tensor, seed=None, min_value=None, max_value=None) -> None:
+        """random.uniform (src/tensor/random/uniform.zig): seed None draws it from the clock; without
+        min/max floats land in [0, 1] and integers take the low bits of the hash."""
+        sub = DTYPE_NAMES[dtype_id(tensor.dtype) % 10]
+        seed_arg = ctypes.byref(u64(seed)) if seed is not None else None
+        _k1, pmin = _scalar_ptr(sub, min_value)
+        _k2, pmax = _scalar_ptr(sub, max_value)
+        _check(_lib().wkz_random_uniform(pipeline._h, tensor._h, seed_arg, pmin, pmax), "random.uniform")
+
+    @staticmethod
+    def hash(index: int, seed: int) -> int:
+        """The 64-bit hash random.uniform draws from."""
+        return int(_capi.load().wk_random_hash(index, seed))
+
+
+class convertions:
+    @staticmethod
+    def toComplex(pipeline: Pipeline, src: Tensor, dst: Tensor, space: Space) -> None:
+        _check(_lib().wkz_to_complex(pipeline._h, src._h, dst._h, int(space)), "toComplex")
+
+    @staticmethod
+    def toReal(pipeline: Pipeline, src: Tensor, dst: Tensor, space: Space) -> None:
+        _check(_lib().wkz_to_real(pipeline._h, src._h, dst._h, int(space)), "toReal")
 
 
 class GemmPackedTensors:
@@ -377,5 +445,5 @@ class blas:
 from . import nn  # noqa: E402  (needs the classes above)
 from .nn import math  # noqa: E402,F401
 
-__all__ = ["nn", "math", "Context", "Pipeline", "Tensor", "CommandQueue", "DeviceType", "memory", "fill", "identity", "blas",
+__all__ = ["nn", "math", "transpose", "random", "convertions", "Space", "Context", "Pipeline", "Tensor", "CommandQueue", "DeviceType", "memory", "fill", "identity", "blas",
            "GemmPackedTensors", "WekuaError", "DTYPE_NAMES", "dtype_id", "elem_size", "is_complex", "real_np_dtype"]

@@ -76,6 +76,11 @@ SIGNATURES = {
     "wk_sum": (ci, [vp, ci, u64p, vp, u64, u64, vp, vp, ctypes.c_double]),
     "wk_adam_step": (ci, [vp, ci, u64p, vp, u64, u64, vp, u64, u64, vp, vp, u64, u64, ctypes.c_double, ctypes.c_double,
                           ctypes.c_double, ctypes.c_double, u64]),
+    "wk_transpose": (ci, [vp, ci, ci, u64p, u64p, u64p, ci, ci, vp, vp]),
+    "wk_random_uniform": (ci, [vp, ci, u64p, vp, u64, u64, u64, vp, vp]),
+    "wk_random_hash": (u64, [u64, u64]),
+    "wk_to_complex": (ci, [vp, ci, u64p, vp, u64, u64, vp, u64, u64, ci]),
+    "wk_to_real": (ci, [vp, ci, u64p, vp, u64, u64, vp, u64, u64, ci]),
 }
 
 _lib = None

@@ -30,9 +30,11 @@
 //     operands through LDS, so pack() only validates.
 #pragma once
 
+#include <chrono>
 #include <cstdint>
 #include <cstring>
 #include <exception>
+#include <limits>
 #include <optional>
 #include <string>
 #include <type_traits>
@@ -65,6 +67,7 @@ template <typename T> struct scalar_of { using type = T; };
 template <typename R> struct scalar_of<Complex<R>> { using type = R; };
 
 template <typename T> constexpr bool isComplex() { return is_complex<T>::value; }
+enum class Space : uint8_t { real = 0, imag = 1 }; // src/core/types.zig:1-4
 
 // getTypeId: 0..9 over the scalar type (types.zig:88-104)
 template <typename T> constexpr int getTypeId() {
@@ -372,6 +375,42 @@ template <typename T> void writeToBuffer(Pipeline *pipeline, Tensor<T> *tensor, 
                                  (size_t)tensor->memory_layout.slice_pitch * sizeof(T), width, rows, depth));
     pipeline->append(1);
 }
+// DEVICE -> DEVICE of the logical region (src/tensor/memory/copy.zig:84-98)
+template <typename T> void copy(Pipeline *pipeline, Tensor<T> *src, Tensor<T> *dst) {
+    helpers::eqlTensorsShape<T>(src, dst);
+    const size_t width = (size_t)src->cols() * sizeof(T);
+    check(wk_copy_d2d_rect_async(pipeline->command_queue->stream, dst->buffer, (size_t)dst->memory_layout.row_pitch * sizeof(T),
+                                 (size_t)dst->memory_layout.slice_pitch * sizeof(T), src->buffer,
+                                 (size_t)src->memory_layout.row_pitch * sizeof(T),
+                                 (size_t)src->memory_layout.slice_pitch * sizeof(T), width, (size_t)src->rows(),
+                                 (size_t)src->depth()));
+    pipeline->append(1);
+}
+// element offset of a coordinate (get_value.zig:18-27): InvalidCoordinates on rank or range mismatch
+template <typename T> size_t elementOffset(const Tensor<T> *tensor, const std::vector<uint64_t> &coor) {
+    const auto &shape = tensor->dimensions.shape;
+    if (coor.size() != shape.size()) throw Error(WK_E_INVALID_COORDINATES);
+    size_t offset = 0;
+    for (size_t i = 0; i < coor.size(); ++i) {
+        if (coor[i] >= shape[i]) throw Error(WK_E_INVALID_COORDINATES);
+        offset += (size_t)(coor[i] * tensor->dimensions.pitches[i]);
+    }
+    return offset;
+}
+// src/tensor/memory/get_value.zig:11-47: non-blocking read of one element into *scalar
+template <typename T> void getValue(Pipeline *pipeline, Tensor<T> *tensor, const std::vector<uint64_t> &coor, T *scalar) {
+    const size_t offset = elementOffset<T>(tensor, coor);
+    check(wk_copy_d2h_rect_async(pipeline->command_queue->stream, scalar, sizeof(T), sizeof(T),
+                                 static_cast<const T *>(tensor->buffer) + offset, sizeof(T), sizeof(T), sizeof(T), 1, 1));
+    pipeline->append(1);
+}
+// src/tensor/memory/put_value.zig:11-47
+template <typename T> void putValue(Pipeline *pipeline, Tensor<T> *tensor, const std::vector<uint64_t> &coor, const T *scalar) {
+    const size_t offset = elementOffset<T>(tensor, coor);
+    check(wk_copy_h2d_rect_async(pipeline->command_queue->stream, static_cast<T *>(tensor->buffer) + offset, sizeof(T), sizeof(T),
+                                 scalar, sizeof(T), sizeof(T), sizeof(T), 1, 1));
+    pipeline->append(1);
+}
 } // namespace memory
 
 namespace fill {
@@ -401,6 +440,77 @@ template <typename T> void identity(Pipeline *pipeline, Tensor<T> *tensor) {
     check(wk_identity(pipeline->command_queue->stream, core::getTypeIndex<T>(), tensor->buffer, size, pitch_sum));
     pipeline->append(1);
 }
+
+// src/tensor/transpose.zig:14-105: result = tensor with dimensions dim0 and dim1 exchanged
+template <typename T> void transpose(Pipeline *pipeline, Tensor<T> *result_tensor, Tensor<T> *tensor, uint64_t dim0, uint64_t dim1) {
+    const auto &shape_a = result_tensor->dimensions.shape, &shape_b = tensor->dimensions.shape;
+    if (shape_a.size() != shape_b.size()) throw Error(WK_E_UNQUAL_TENSORS_DIMENSION);
+    if (dim0 >= shape_a.size() || dim1 >= shape_a.size()) throw Error(WK_E_INVALID_VALUE);
+    if (tensor->dimensions.number_of_elements_without_padding != result_tensor->dimensions.number_of_elements_without_padding)
+        throw Error(WK_E_UNQUAL_TENSORS_DIMENSION);
+    if (shape_a[dim0] != shape_b[dim1] || shape_a[dim1] != shape_b[dim0]) throw Error(WK_E_INVALID_VALUE);
+    if (dim0 == dim1) {
+        memory::copy<T>(pipeline, tensor, result_tensor);
+        return;
+    }
+    // the kernel walks the source, so every other dimension has to agree too (the reference's
+    // kernel would write out of the result's bounds otherwise)
+    for (size_t x = 0; x < shape_a.size(); ++x)
+        if (x != dim0 && x != dim1 && shape_a[x] != shape_b[x]) throw Error(WK_E_INVALID_VALUE);
+    check(wk_transpose(pipeline->command_queue->stream, core::getTypeIndex<T>(), (int)shape_b.size(), shape_b.data(),
+                       tensor->dimensions.pitches.data(), result_tensor->dimensions.pitches.data(), (int)dim0, (int)dim1,
+                       tensor->buffer, result_tensor->buffer));
+    pipeline->append(1);
+}
+
+namespace random {
+// src/tensor/random/uniform.zig:60-135.  seed == nullopt draws it from the clock, as there.
+template <typename T>
+void uniform(Pipeline *pipeline, Tensor<T> *tensor, std::optional<uint64_t> seed,
+             std::optional<typename core::scalar_of<T>::type> min_value, std::optional<typename core::scalar_of<T>::type> max_value) {
+    using Sub = typename core::scalar_of<T>::type;
+    const uint64_t global_seed =
+        seed ? *seed : (uint64_t)std::chrono::duration_cast<std::chrono::seconds>(std::chrono::system_clock::now().time_since_epoch()).count();
+    const uint64_t shape3[3] = {tensor->depth(), tensor->rows(), tensor->cols()};
+    Sub mn{}, range{};
+    const bool range_defined = min_value.has_value() || max_value.has_value();
+    if (range_defined) {
+        mn = min_value.value_or(std::numeric_limits<Sub>::lowest());
+        const Sub mx = max_value.value_or(std::numeric_limits<Sub>::max());
+        if constexpr (std::is_integral_v<Sub>) {
+            using U = std::make_unsigned_t<Sub>;
+            range = (Sub)(U)((U)mx - (U)mn); // wraps like the reference's release build when the span exceeds the type
+        } else {
+            range = mx - mn;
+        }
+    }
+    check(wk_random_uniform(pipeline->command_queue->stream, core::getTypeIndex<T>(), shape3, tensor->buffer,
+                            tensor->memory_layout.row_pitch, tensor->memory_layout.slice_pitch, global_seed,
+                            range_defined ? &mn : nullptr, range_defined ? &range : nullptr));
+    pipeline->append(1);
+}
+} // namespace random
+
+namespace convertions {
+// src/tensor/convertions/to_complex.zig:52-98
+template <typename R> void toComplex(Pipeline *pipeline, Tensor<R> *src, Tensor<core::Complex<R>> *dst, core::Space space) {
+    if (src->dimensions.shape != dst->dimensions.shape) throw Error(WK_E_UNQUAL_TENSORS_SHAPE);
+    const uint64_t shape3[3] = {src->depth(), src->rows(), src->cols()};
+    check(wk_to_complex(pipeline->command_queue->stream, core::getTypeIndex<R>(), shape3, src->buffer, src->memory_layout.row_pitch,
+                        src->memory_layout.slice_pitch, dst->buffer, dst->memory_layout.row_pitch, dst->memory_layout.slice_pitch,
+                        (int)space));
+    pipeline->append(1);
+}
+// src/tensor/convertions/to_real.zig:51-97
+template <typename R> void toReal(Pipeline *pipeline, Tensor<core::Complex<R>> *src, Tensor<R> *dst, core::Space space) {
+    if (src->dimensions.shape != dst->dimensions.shape) throw Error(WK_E_UNQUAL_TENSORS_SHAPE);
+    const uint64_t shape3[3] = {src->depth(), src->rows(), src->cols()};
+    check(wk_to_real(pipeline->command_queue->stream, core::getTypeIndex<R>(), shape3, src->buffer, src->memory_layout.row_pitch,
+                     src->memory_layout.slice_pitch, dst->buffer, dst->memory_layout.row_pitch, dst->memory_layout.slice_pitch,
+                     (int)space));
+    pipeline->append(1);
+}
+} // namespace convertions
 
 namespace blas {
 

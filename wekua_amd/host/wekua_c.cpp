@@ -37,6 +37,21 @@ struct OptimizerHandle {
     void *optimizer; // nn::optimizers::Optimizer<T>*
 };
 
+template <typename F> void dispatch_real_component(int dtype, F &&f) {
+    switch (dtype) {
+    case 0: f.template operator()<int8_t>(); break;
+    case 1: f.template operator()<uint8_t>(); break;
+    case 2: f.template operator()<int16_t>(); break;
+    case 3: f.template operator()<uint16_t>(); break;
+    case 4: f.template operator()<int32_t>(); break;
+    case 5: f.template operator()<uint32_t>(); break;
+    case 6: f.template operator()<int64_t>(); break;
+    case 7: f.template operator()<uint64_t>(); break;
+    case 8: f.template operator()<float>(); break;
+    case 9: f.template operator()<double>(); break;
+    default: throw Error(WK_E_TYPE_NOT_SUPPORTED);
+    }
+}
 template <typename F> void dispatch_real(int dtype, F &&f) {
     switch (dtype) {
     case 8: f.template operator()<float>(); break;
@@ -246,6 +261,78 @@ int wkz_identity(void *pipeline, void *tensor) {
     return guard([&] {
         TensorHandle *h = static_cast<TensorHandle *>(tensor);
         dispatch(h->dtype, [&]<typename T>() { identity<T>(static_cast<Pipeline *>(pipeline), static_cast<Tensor<T> *>(h->tensor)); });
+    });
+}
+
+// ---- tensor support operations --------------------------------------------------------------------
+int wkz_memory_copy(void *pipeline, void *src, void *dst) {
+    return guard([&] {
+        TensorHandle *hs = static_cast<TensorHandle *>(src), *hd = static_cast<TensorHandle *>(dst);
+        if (hs->dtype != hd->dtype) throw Error(WK_E_UNQUAL_TENSORS_ATTRIBUTE);
+        dispatch(hs->dtype, [&]<typename T>() {
+            memory::copy<T>(static_cast<Pipeline *>(pipeline), static_cast<Tensor<T> *>(hs->tensor), static_cast<Tensor<T> *>(hd->tensor));
+        });
+    });
+}
+int wkz_get_value(void *pipeline, void *tensor, const uint64_t *coor, uint64_t ncoor, void *host_scalar) {
+    return guard([&] {
+        TensorHandle *h = static_cast<TensorHandle *>(tensor);
+        if (!host_scalar || (ncoor && !coor)) throw Error(WK_E_INVALID_VALUE);
+        dispatch(h->dtype, [&]<typename T>() {
+            memory::getValue<T>(static_cast<Pipeline *>(pipeline), static_cast<Tensor<T> *>(h->tensor),
+                                std::vector<uint64_t>(coor, coor + ncoor), static_cast<T *>(host_scalar));
+        });
+    });
+}
+int wkz_put_value(void *pipeline, void *tensor, const uint64_t *coor, uint64_t ncoor, const void *host_scalar) {
+    return guard([&] {
+        TensorHandle *h = static_cast<TensorHandle *>(tensor);
+        if (!host_scalar || (ncoor && !coor)) throw Error(WK_E_INVALID_VALUE);
+        dispatch(h->dtype, [&]<typename T>() {
+            memory::putValue<T>(static_cast<Pipeline *>(pipeline), static_cast<Tensor<T> *>(h->tensor),
+                                std::vector<uint64_t>(coor, coor + ncoor), static_cast<const T *>(host_scalar));
+        });
+    });
+}
+int wkz_transpose(void *pipeline, void *result, void *tensor, uint64_t dim0, uint64_t dim1) {
+    return guard([&] {
+        TensorHandle *hr = static_cast<TensorHandle *>(result), *ht = static_cast<TensorHandle *>(tensor);
+        if (hr->dtype != ht->dtype) throw Error(WK_E_UNQUAL_TENSORS_ATTRIBUTE);
+        dispatch(ht->dtype, [&]<typename T>() {
+            transpose<T>(static_cast<Pipeline *>(pipeline), static_cast<Tensor<T> *>(hr->tensor), static_cast<Tensor<T> *>(ht->tensor), dim0,
+                         dim1);
+        });
+    });
+}
+// seed, host_min, host_max: NULL for an absent (null) argument; min / max are of the real component type
+int wkz_random_uniform(void *pipeline, void *tensor, const uint64_t *seed, const void *host_min, const void *host_max) {
+    return guard([&] {
+        TensorHandle *h = static_cast<TensorHandle *>(tensor);
+        dispatch(h->dtype, [&]<typename T>() {
+            using Sub = typename core::scalar_of<T>::type;
+            random::uniform<T>(static_cast<Pipeline *>(pipeline), static_cast<Tensor<T> *>(h->tensor),
+                               seed ? std::optional<uint64_t>(*seed) : std::nullopt, opt_scalar<Sub>(host_min), opt_scalar<Sub>(host_max));
+        });
+    });
+}
+int wkz_to_complex(void *pipeline, void *src, void *dst, int space) {
+    return guard([&] {
+        TensorHandle *hs = static_cast<TensorHandle *>(src), *hd = static_cast<TensorHandle *>(dst);
+        if (hd->dtype != hs->dtype + 10 || (space != 0 && space != 1)) throw Error(WK_E_UNQUAL_TENSORS_ATTRIBUTE);
+        dispatch_real_component(hs->dtype, [&]<typename R>() {
+            convertions::toComplex<R>(static_cast<Pipeline *>(pipeline), static_cast<Tensor<R> *>(hs->tensor),
+                                      static_cast<Tensor<core::Complex<R>> *>(hd->tensor), static_cast<core::Space>(space));
+        });
+    });
+}
+int wkz_to_real(void *pipeline, void *src, void *dst, int space) {
+    return guard([&] {
+        TensorHandle *hs = static_cast<TensorHandle *>(src), *hd = static_cast<TensorHandle *>(dst);
+        if (hs->dtype != hd->dtype + 10 || (space != 0 && space != 1)) throw Error(WK_E_UNQUAL_TENSORS_ATTRIBUTE);
+        dispatch_real_component(hd->dtype, [&]<typename R>() {
+            convertions::toReal<R>(static_cast<Pipeline *>(pipeline), static_cast<Tensor<core::Complex<R>> *>(hs->tensor),
+                                   static_cast<Tensor<R> *>(hd->tensor), static_cast<core::Space>(space));
+        });
     });
 }
 
