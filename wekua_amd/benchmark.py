@@ -5,6 +5,7 @@ times over 1-D sizes, on GPU 0.
     python -m wekua_amd.benchmark gemm [--dtype f32] [--sizes 1024 2048 ...] [--variant NAME]
     python -m wekua_amd.benchmark axpy [--dtype f32]
     python -m wekua_amd.benchmark configs        # every BASELINE GEMM / AXPY configuration, one line each
+    python -m wekua_amd.benchmark tensor         # transpose / copy / random.uniform / toComplex streaming rates
     python -m wekua_amd.benchmark mlp [--dtype f32] [--sizes 1024 4096 4096 1024] [--batch 2048] [--optimizer adam]
 
 Everything goes through the reference-shaped API (Tensor.alloc, memory.readFromBuffer, blas.*).
@@ -153,6 +154,42 @@ def cmd_configs(ses, args):
         print(f"{name:34s} {ms:9.4f} {rate:9.2f} {unit:8s} {v}")
 
 
+def cmd_tensor(ses, args):
+    """Streaming rates of the tensor support operations (algorithmic bytes: one read and one write of
+    every element, one write for random.uniform)."""
+    wk = ses.wk
+    print(f"{'operation':44s} {'us':>9s} {'GB/s':>8s}")
+    for dtype, shape, d0, d1 in (("f32", (8192, 8192), 0, 1), ("f64", (8192, 8192), 0, 1), ("cf64", (4096, 4096), 0, 1),
+                                 ("u8", (16384, 16384), 0, 1), ("f32", (64, 1024, 1024), 0, 1), ("f32", (64, 1024, 1024), 1, 2),
+                                 ("f32", (1024, 64, 1024), 0, 2)):
+        x = wk.Tensor.alloc(dtype, ses.ctx, ses.pipeline, shape)
+        rshape = list(shape)
+        rshape[d0], rshape[d1] = rshape[d1], rshape[d0]
+        r = wk.Tensor.alloc(dtype, ses.ctx, ses.pipeline, rshape)
+        wk.random.uniform(ses.pipeline, x, 1)
+        ms = ses.time_ms(lambda: wk.transpose(ses.pipeline, r, x, d0, d1), 20)
+        nbytes = 2.0 * np.prod(shape) * raw.elem_size(dtype)
+        print(f"{'transpose ' + dtype + ' ' + 'x'.join(map(str, shape)) + f' dims {d0},{d1}':44s} {ms * 1e3:9.1f} {nbytes / ms / 1e6:8.0f}",
+              flush=True)
+        x.release(ses.pipeline)
+        r.release(ses.pipeline)
+    x = wk.Tensor.alloc("f32", ses.ctx, ses.pipeline, (8192, 8192))
+    y = wk.Tensor.alloc("f32", ses.ctx, ses.pipeline, (8192, 8192))
+    z = wk.Tensor.alloc("cf32", ses.ctx, ses.pipeline, (8192, 8192))
+    n = 8192.0 * 8192
+    for name, call, nbytes in (
+            ("memory.copy f32 8192x8192", lambda: wk.memory.copy(ses.pipeline, x, y), 8 * n),
+            ("random.uniform f32 8192x8192", lambda: wk.random.uniform(ses.pipeline, x, 7), 4 * n),
+            ("random.uniform f32 8192x8192 in [-1, 1]", lambda: wk.random.uniform(ses.pipeline, x, 7, -1.0, 1.0), 4 * n),
+            ("random.uniform cf32 8192x8192", lambda: wk.random.uniform(ses.pipeline, z, 7), 8 * n),
+            ("toComplex f32 -> cf32 8192x8192", lambda: wk.convertions.toComplex(ses.pipeline, x, z, wk.Space.real), 8 * n),
+            ("toReal cf32 -> f32 8192x8192", lambda: wk.convertions.toReal(ses.pipeline, z, x, wk.Space.imag), 8 * n)):
+        ms = ses.time_ms(call, 20)
+        print(f"{name:44s} {ms * 1e3:9.1f} {nbytes / ms / 1e6:8.0f}", flush=True)
+    for t in (x, y, z):
+        t.release(ses.pipeline)
+
+
 def mlp_flops(sizes, batch):
     """Multiply-adds of the GEMMs of one training step, as flops: forward and weight gradients over
     every layer, input sensitivities over every layer but the first."""
@@ -246,6 +283,7 @@ def main(argv=None):
     g.add_argument("--variant", default="auto")
     a = sub.add_parser("axpy")
     a.add_argument("--dtype", default="f32")
+    sub.add_parser("tensor")
     c = sub.add_parser("configs")
     c.add_argument("--variant", default="auto")
     m = sub.add_parser("mlp")
@@ -264,7 +302,7 @@ def main(argv=None):
     try:
         if getattr(args, "variant", "auto") != "auto":
             raw.check(ses.lib.wk_gemm_force_variant(args.variant.encode()), "wk_gemm_force_variant")
-        {"gemm": cmd_gemm, "axpy": cmd_axpy, "configs": cmd_configs}[args.cmd](ses, args)
+        {"gemm": cmd_gemm, "axpy": cmd_axpy, "configs": cmd_configs, "tensor": cmd_tensor}[args.cmd](ses, args)
     finally:
         ses.close()
     return 0

@@ -38,35 +38,80 @@ __device__ __forceinline__ void batch_offsets(const TransposeArgs &a, uint64_t b
     }
 }
 
-// The contiguous dimension takes part in the swap: tiles go through LDS so that both the read
+// The contiguous dimension takes part in the swap: T x T tiles go through LDS so that both the read
 // (along source columns) and the write (along what becomes the destination's contiguous
-// dimension) are runs of consecutive addresses.
-template <typename E, int TILE>
+// dimension) are runs of consecutive addresses.  With VEC every lane moves 16 bytes (VE elements)
+// per access on both sides; the host grants VEC only when bases and pitches allow it.
+template <typename E, int T, bool VEC>
 __global__ __launch_bounds__(256) void transpose_tiled_kernel(const E *__restrict__ src, E *__restrict__ dst, TransposeArgs a,
                                                               uint64_t tiles_c) {
-    __shared__ E tile[TILE][TILE + 1];
-    constexpr int RY = 256 / TILE;
-    const int tx = threadIdx.x % TILE, ty = threadIdx.x / TILE;
+    constexpr int VE = VEC ? 16 / (int)sizeof(E) : 1;
+    constexpr int VPR = T / VE;            // vectors per tile row
+    constexpr int ITERS = T * VPR / 256;   // vectors per thread
+    static_assert(T % VE == 0 && (T * VPR) % 256 == 0, "tile must split evenly over 256 threads");
+    __shared__ E tile[T][T + 1];
     const uint64_t tr = blockIdx.x / tiles_c, tc = blockIdx.x % tiles_c;
     uint64_t so, dof;
     batch_offsets(a, blockIdx.y, so, dof);
-    const uint64_t r0 = tr * TILE, c0 = tc * TILE;
-    for (int r = ty; r < TILE; r += RY)
-        if (r0 + r < a.rows && c0 + tx < a.cols) tile[r][tx] = src[so + (r0 + r) * a.src_row_pitch + c0 + tx];
+    const uint64_t r0 = tr * T, c0 = tc * T;
+#pragma unroll
+    for (int it = 0; it < ITERS; ++it) {
+        const int v = it * 256 + (int)threadIdx.x;
+        const int r = v / VPR, c = (v % VPR) * VE;
+        if (r0 + r >= a.rows) continue;
+        const E *p = src + so + (r0 + r) * a.src_row_pitch + c0 + c;
+        if (VEC && c0 + c + VE <= a.cols) {
+            E tmp[VE];
+            __builtin_memcpy(tmp, __builtin_assume_aligned(p, 16), 16);
+#pragma unroll
+            for (int e = 0; e < VE; ++e) tile[r][c + e] = tmp[e];
+        } else {
+            for (int e = 0; e < VE; ++e)
+                if (c0 + c + e < a.cols) tile[r][c + e] = p[e];
+        }
+    }
     __syncthreads();
-    for (int c = ty; c < TILE; c += RY)
-        if (c0 + c < a.cols && r0 + tx < a.rows) dst[dof + (c0 + c) * a.dst_row_pitch + r0 + tx] = tile[tx][c];
+#pragma unroll
+    for (int it = 0; it < ITERS; ++it) {
+        const int v = it * 256 + (int)threadIdx.x;
+        const int c = v / VPR, r = (v % VPR) * VE; // destination row = source column c
+        if (c0 + c >= a.cols) continue;
+        E *p = dst + dof + (c0 + c) * a.dst_row_pitch + r0 + r;
+        if (VEC && r0 + r + VE <= a.rows) {
+            E tmp[VE];
+#pragma unroll
+            for (int e = 0; e < VE; ++e) tmp[e] = tile[r + e][c];
+            __builtin_memcpy(__builtin_assume_aligned(p, 16), tmp, 16);
+        } else {
+            for (int e = 0; e < VE; ++e)
+                if (r0 + r + e < a.rows) p[e] = tile[r + e][c];
+        }
+    }
 }
 
 // The contiguous dimension stays where it is: whole rows move, reads and writes both run along it.
-template <typename E>
-__global__ __launch_bounds__(256) void transpose_rows_kernel(const E *__restrict__ src, E *__restrict__ dst, TransposeArgs a) {
-    uint64_t so, dof;
-    batch_offsets(a, blockIdx.y, so, dof);
-    const uint64_t total = a.rows * a.cols;
-    for (uint64_t idx = blockIdx.x * 256ull + threadIdx.x; idx < total; idx += (uint64_t)gridDim.x * 256ull) {
-        const uint64_t r = idx / a.cols, c = idx % a.cols;
-        dst[dof + r * a.dst_row_pitch + c] = src[so + r * a.src_row_pitch + c];
+// blockIdx.y walks (batch, row) pairs, blockIdx.x the columns.
+template <typename E, bool VEC>
+__global__ __launch_bounds__(256) void transpose_rows_kernel(const E *__restrict__ src, E *__restrict__ dst, TransposeArgs a,
+                                                             uint64_t total_rows) {
+    constexpr int VE = VEC ? 16 / (int)sizeof(E) : 1;
+    const uint64_t cols_v = (a.cols + VE - 1) / VE;
+    for (uint64_t br = blockIdx.y; br < total_rows; br += gridDim.y) {
+        uint64_t so, dof;
+        batch_offsets(a, br / a.rows, so, dof);
+        const uint64_t r = br % a.rows;
+        const E *sp = src + so + r * a.src_row_pitch;
+        E *dp = dst + dof + r * a.dst_row_pitch;
+        for (uint64_t cv = blockIdx.x * 256ull + threadIdx.x; cv < cols_v; cv += (uint64_t)gridDim.x * 256ull) {
+            const uint64_t c = cv * VE;
+            if (VEC && c + VE <= a.cols) {
+                E tmp[VE];
+                __builtin_memcpy(tmp, __builtin_assume_aligned(sp + c, 16), 16);
+                __builtin_memcpy(__builtin_assume_aligned(dp + c, 16), tmp, 16);
+            } else {
+                for (int e = 0; e < VE && c + e < a.cols; ++e) dp[c + e] = sp[c + e];
+            }
+        }
     }
 }
 
@@ -114,21 +159,36 @@ __device__ __forceinline__ R uniform_value(uint64_t h, MinT min_value, MinT rang
     }
 }
 
+// blockIdx.y walks the rows (all slices), blockIdx.x the columns: one division per row, none per element.
 template <typename R, bool CPLX, bool IS_FLOAT, bool RANGED, typename MinT>
-__global__ __launch_bounds__(256) void uniform_kernel(R *__restrict__ out, uint64_t depth, uint64_t rows, uint64_t cols,
+__global__ __launch_bounds__(256) void uniform_kernel(R *__restrict__ out, uint64_t rows, uint64_t cols, uint64_t total_rows,
                                                       uint64_t row_pitch, uint64_t slice_pitch, uint64_t seed, MinT min_value,
                                                       MinT range) {
-    const uint64_t total = depth * rows * cols;
-    for (uint64_t idx = blockIdx.x * 256ull + threadIdx.x; idx < total; idx += (uint64_t)gridDim.x * 256ull) {
-        const uint64_t k = idx % cols, ij = idx / cols;
-        const uint64_t off = (ij / rows) * slice_pitch + (ij % rows) * row_pitch + k;
-        if constexpr (CPLX) {
-            out[2 * off] = uniform_value<R, IS_FLOAT, RANGED, MinT>(wk_hash64(idx << 1, seed), min_value, range);
-            out[2 * off + 1] = uniform_value<R, IS_FLOAT, RANGED, MinT>(wk_hash64((idx << 1) + 1, seed), min_value, range);
-        } else {
-            out[off] = uniform_value<R, IS_FLOAT, RANGED, MinT>(wk_hash64(idx, seed), min_value, range);
+    for (uint64_t row = blockIdx.y; row < total_rows; row += gridDim.y) {
+        const uint64_t off0 = (row / rows) * slice_pitch + (row % rows) * row_pitch;
+        const uint64_t idx0 = row * cols;
+        for (uint64_t k = blockIdx.x * 256ull + threadIdx.x; k < cols; k += (uint64_t)gridDim.x * 256ull) {
+            const uint64_t idx = idx0 + k, off = off0 + k;
+            if constexpr (CPLX) {
+                out[2 * off] = uniform_value<R, IS_FLOAT, RANGED, MinT>(wk_hash64(idx << 1, seed), min_value, range);
+                out[2 * off + 1] = uniform_value<R, IS_FLOAT, RANGED, MinT>(wk_hash64((idx << 1) + 1, seed), min_value, range);
+            } else {
+                out[off] = uniform_value<R, IS_FLOAT, RANGED, MinT>(wk_hash64(idx, seed), min_value, range);
+            }
         }
     }
+}
+
+// grid for the row-wise kernels: x over 256-column chunks, y over rows, about 16k blocks at most
+dim3 row_grid(uint64_t cols, uint64_t total_rows) {
+    uint64_t gx = (cols + 255) / 256;
+    if (gx < 1) gx = 1;
+    if (gx > 16384) gx = 16384;
+    uint64_t gy = (16384 + gx - 1) / gx;
+    if (gy > total_rows) gy = total_rows;
+    if (gy > 65535) gy = 65535;
+    if (gy < 1) gy = 1;
+    return dim3((unsigned)gx, (unsigned)gy);
 }
 
 unsigned grid_for(uint64_t total) {
@@ -139,8 +199,8 @@ unsigned grid_for(uint64_t total) {
 template <typename R, typename S, bool IS_FLOAT>
 int launch_uniform(wk_stream *s, bool cplx, void *ptr, const uint64_t shape3[3], uint64_t rp, uint64_t sp, uint64_t seed,
                    const void *host_min, const void *host_range) {
-    const uint64_t total = shape3[0] * shape3[1] * shape3[2];
-    const unsigned grid = grid_for(total);
+    const uint64_t total_rows = shape3[0] * shape3[1];
+    const dim3 grid = row_grid(shape3[2], total_rows);
     R *out = static_cast<R *>(ptr);
     S mn{}, rg{};
     if (host_min) {
@@ -148,8 +208,8 @@ int launch_uniform(wk_stream *s, bool cplx, void *ptr, const uint64_t shape3[3],
         std::memcpy(&rg, host_range, sizeof(S));
     }
 #define WK_U(CP, RA)                                                                                                        \
-    hipLaunchKernelGGL((uniform_kernel<R, CP, IS_FLOAT, RA, S>), dim3(grid), dim3(256), 0, s->stream, out, shape3[0], shape3[1], \
-                       shape3[2], rp, sp, seed, mn, rg)
+    hipLaunchKernelGGL((uniform_kernel<R, CP, IS_FLOAT, RA, S>), grid, dim3(256), 0, s->stream, out, shape3[1], shape3[2],      \
+                       total_rows, rp, sp, seed, mn, rg)
     if (cplx) {
         if (host_min) WK_U(true, true);
         else WK_U(true, false);
@@ -163,16 +223,17 @@ int launch_uniform(wk_stream *s, bool cplx, void *ptr, const uint64_t shape3[3],
 
 // ---- real <-> complex -------------------------------------------------------------------------
 template <typename E, bool TO_COMPLEX>
-__global__ __launch_bounds__(256) void complex_part_kernel(const E *__restrict__ src, E *__restrict__ dst, uint64_t depth,
-                                                           uint64_t rows, uint64_t cols, uint64_t srp, uint64_t ssp, uint64_t drp,
-                                                           uint64_t dsp, unsigned part) {
-    const uint64_t total = depth * rows * cols;
-    for (uint64_t idx = blockIdx.x * 256ull + threadIdx.x; idx < total; idx += (uint64_t)gridDim.x * 256ull) {
-        const uint64_t k = idx % cols, ij = idx / cols;
-        const uint64_t i = ij / rows, j = ij % rows;
-        const uint64_t so = i * ssp + j * srp + k, dof = i * dsp + j * drp + k;
-        if constexpr (TO_COMPLEX) dst[2 * dof + part] = src[so];
-        else dst[dof] = src[2 * so + part];
+__global__ __launch_bounds__(256) void complex_part_kernel(const E *__restrict__ src, E *__restrict__ dst, uint64_t rows,
+                                                           uint64_t cols, uint64_t total_rows, uint64_t srp, uint64_t ssp,
+                                                           uint64_t drp, uint64_t dsp, unsigned part) {
+    for (uint64_t row = blockIdx.y; row < total_rows; row += gridDim.y) {
+        const uint64_t i = row / rows, j = row % rows;
+        const E *sp = src + (TO_COMPLEX ? 1 : 2) * (i * ssp + j * srp);
+        E *dp = dst + (TO_COMPLEX ? 2 : 1) * (i * dsp + j * drp);
+        for (uint64_t k = blockIdx.x * 256ull + threadIdx.x; k < cols; k += (uint64_t)gridDim.x * 256ull) {
+            if constexpr (TO_COMPLEX) dp[2 * k + part] = sp[k];
+            else dp[k] = sp[2 * k + part];
+        }
     }
 }
 
@@ -228,22 +289,36 @@ int wk_transpose(wk_stream *s, int dtype, int ndim, const uint64_t *shape, const
         batches *= shape[x];
         ++a.nbatch;
     }
-    if (batches > 65535) {
-        // fold: the y dimension of a grid is limited; such shapes (more than 65535 slices) take
-        // one launch per chunk of slices through the x dimension instead -- not needed by any
-        // caller of this library yet, reported rather than silently mishandled
-        return WK_E_INVALID_VALUE;
-    }
+    // the tiled kernel puts one batch entry on each blockIdx.y; the y dimension of a grid is limited
+    if (tiled && batches > 65535) return WK_E_INVALID_VALUE;
+    const bool aligned16 = ((reinterpret_cast<uintptr_t>(src) | reinterpret_cast<uintptr_t>(dst)) & 15u) == 0;
     return dispatch_elem_size(es, [&]<typename E>() -> int {
         if (tiled) {
-            constexpr int TILE = sizeof(E) == 16 ? 32 : 64;
-            const uint64_t tiles_r = (a.rows + TILE - 1) / TILE, tiles_c = (a.cols + TILE - 1) / TILE;
+            // tile edge: at least 128 bytes of every row segment (64 elements of 4 and 8 bytes, 128 of 1 and 2, 32 of 16)
+            constexpr int T = sizeof(E) == 16 ? 32 : (sizeof(E) >= 4 ? 64 : 128);
+            constexpr uint64_t VE = 16 / sizeof(E);
+            bool vec = aligned16 && a.src_row_pitch % VE == 0 && a.dst_row_pitch % VE == 0;
+            for (int x = 0; x < a.nbatch; ++x) vec = vec && a.bsrc[x] % VE == 0 && a.bdst[x] % VE == 0;
+            const uint64_t tiles_r = (a.rows + T - 1) / T, tiles_c = (a.cols + T - 1) / T;
             if (tiles_r * tiles_c > 0x7fffffffull) return WK_E_INVALID_VALUE;
-            hipLaunchKernelGGL((transpose_tiled_kernel<E, TILE>), dim3((unsigned)(tiles_r * tiles_c), (unsigned)batches), dim3(256),
-                               0, s->stream, static_cast<const E *>(src), static_cast<E *>(dst), a, tiles_c);
+            const dim3 grid((unsigned)(tiles_r * tiles_c), (unsigned)batches);
+            if (vec)
+                hipLaunchKernelGGL((transpose_tiled_kernel<E, T, true>), grid, dim3(256), 0, s->stream, static_cast<const E *>(src),
+                                   static_cast<E *>(dst), a, tiles_c);
+            else
+                hipLaunchKernelGGL((transpose_tiled_kernel<E, T, false>), grid, dim3(256), 0, s->stream, static_cast<const E *>(src),
+                                   static_cast<E *>(dst), a, tiles_c);
         } else {
-            hipLaunchKernelGGL((transpose_rows_kernel<E>), dim3(grid_for(a.rows * a.cols), (unsigned)batches), dim3(256), 0,
-                               s->stream, static_cast<const E *>(src), static_cast<E *>(dst), a);
+            const uint64_t total_rows = batches * a.rows;
+            constexpr uint64_t VE = 16 / sizeof(E);
+            bool vec = aligned16 && a.src_row_pitch % VE == 0 && a.dst_row_pitch % VE == 0;
+            for (int x = 0; x < a.nbatch; ++x) vec = vec && a.bsrc[x] % VE == 0 && a.bdst[x] % VE == 0;
+            if (vec)
+                hipLaunchKernelGGL((transpose_rows_kernel<E, true>), row_grid((a.cols + VE - 1) / VE, total_rows), dim3(256), 0,
+                                   s->stream, static_cast<const E *>(src), static_cast<E *>(dst), a, total_rows);
+            else
+                hipLaunchKernelGGL((transpose_rows_kernel<E, false>), row_grid(a.cols, total_rows), dim3(256), 0, s->stream,
+                                   static_cast<const E *>(src), static_cast<E *>(dst), a, total_rows);
         }
         return launch_status();
     });
@@ -281,10 +356,10 @@ int wk_to_complex(wk_stream *s, int real_dtype, const uint64_t shape3[3], const 
     if (rc) return rc;
     if ((rc = check_part_args(shape3, src, srp, ssp, dst, drp, dsp, space))) return rc;
     if (real_dtype < 0 || real_dtype >= 10) return WK_E_TYPE_NOT_SUPPORTED;
-    const uint64_t total = shape3[0] * shape3[1] * shape3[2];
+    const uint64_t total_rows = shape3[0] * shape3[1];
     return dispatch_elem_size(wk_dtype_size(real_dtype), [&]<typename E>() -> int {
-        hipLaunchKernelGGL((complex_part_kernel<E, true>), dim3(grid_for(total)), dim3(256), 0, s->stream,
-                           static_cast<const E *>(src), static_cast<E *>(dst), shape3[0], shape3[1], shape3[2], srp, ssp, drp, dsp,
+        hipLaunchKernelGGL((complex_part_kernel<E, true>), row_grid(shape3[2], total_rows), dim3(256), 0, s->stream,
+                           static_cast<const E *>(src), static_cast<E *>(dst), shape3[1], shape3[2], total_rows, srp, ssp, drp, dsp,
                            (unsigned)space);
         return launch_status();
     });
@@ -296,10 +371,10 @@ int wk_to_real(wk_stream *s, int real_dtype, const uint64_t shape3[3], const voi
     if (rc) return rc;
     if ((rc = check_part_args(shape3, src, srp, ssp, dst, drp, dsp, space))) return rc;
     if (real_dtype < 0 || real_dtype >= 10) return WK_E_TYPE_NOT_SUPPORTED;
-    const uint64_t total = shape3[0] * shape3[1] * shape3[2];
+    const uint64_t total_rows = shape3[0] * shape3[1];
     return dispatch_elem_size(wk_dtype_size(real_dtype), [&]<typename E>() -> int {
-        hipLaunchKernelGGL((complex_part_kernel<E, false>), dim3(grid_for(total)), dim3(256), 0, s->stream,
-                           static_cast<const E *>(src), static_cast<E *>(dst), shape3[0], shape3[1], shape3[2], srp, ssp, drp, dsp,
+        hipLaunchKernelGGL((complex_part_kernel<E, false>), row_grid(shape3[2], total_rows), dim3(256), 0, s->stream,
+                           static_cast<const E *>(src), static_cast<E *>(dst), shape3[1], shape3[2], total_rows, srp, ssp, drp, dsp,
                            (unsigned)space);
         return launch_status();
     });
