@@ -22,9 +22,10 @@
 //   * the epilogue applies the reference's option semantics (src/blas/gemm.zig:500-501,
 //     591-602): store / alpha*acc / alpha*acc + beta*C_old.
 //
-// The EDGE instantiation bounds-checks every global access (ragged M, N, K) and uses
-// element-aligned 16-byte loads, so odd leading dimensions keep full-width loads; the interior
-// instantiation assumes M % BM == N % BN == K % BK == 0 and 16-byte aligned rows.
+// The EDGE instantiation handles ragged M, N, K and rows that are only element-aligned: tiles on
+// the border of C and the slab holding the k tail bounds-check every global access, everything
+// else takes unchecked element-aligned 16-byte loads.  The interior instantiation assumes
+// M % BM == N % BN == K % BK == 0 and 16-byte aligned rows.
 #include "wk_internal.hpp"
 
 #include <cstdlib>
@@ -140,11 +141,14 @@ void gemm_f32_mfma_kernel(MArgs<float> g) {
     // ---- global -> registers -----------------------------------------------------------
     // KCONTIG: slab is ROWS x BK, q -> (row = q / (BK/4), c4 = q % (BK/4)), address row*ld + k0 + 4*c4
     // else   : slab is BK x ROWS, q -> (k = q / (ROWS/4), c4 = q % (ROWS/4)), address (k0+k)*ld + 4*c4
+    // CHECK: bounds-check every access (edge tiles and the k tail); otherwise the slab lies inside
+    // the operand and only the alignment of the 16-byte load differs between the instantiations.
     auto gload = [&](f32x4 *dst, const float *__restrict__ base, uint32_t ld, uint32_t row0, uint32_t row_lim,
-                     uint32_t k0, auto kc_tag, auto rows_tag, auto nv_tag) {
+                     uint32_t k0, auto kc_tag, auto rows_tag, auto nv_tag, auto check_tag) {
         constexpr bool KC = decltype(kc_tag)::value;
         constexpr int ROWS = decltype(rows_tag)::value;
         constexpr int NV = decltype(nv_tag)::value;
+        constexpr bool CHECK = decltype(check_tag)::value;
 #pragma unroll
         for (int i = 0; i < NV; ++i) {
             const int q = tid + i * NT;
@@ -160,27 +164,35 @@ void gemm_f32_mfma_kernel(MArgs<float> g) {
             const float *p = base + (size_t)r * ld + c;
             if constexpr (!EDGE) {
                 dst[i] = *reinterpret_cast<const f32x4 *>(p);
+            } else if constexpr (!CHECK) {
+                dst[i] = reinterpret_cast<const f32x4_u *>(p)->v;
             } else {
-                f32x4 v = {0.f, 0.f, 0.f, 0.f};
-                if (r < r_lim) {
-                    if (c + 3 < c_lim) {
-                        v = reinterpret_cast<const f32x4_u *>(p)->v;
-                    } else {
-                        if (c + 0 < c_lim) v[0] = p[0];
-                        if (c + 1 < c_lim) v[1] = p[1];
-                        if (c + 2 < c_lim) v[2] = p[2];
-                        if (c + 3 < c_lim) v[3] = p[3];
-                    }
+                // Clamp the address into the operand and load one raw vector; nothing here depends
+                // on the loaded value, so the request stays in flight across the matrix work.  The
+                // lanes that do not exist are sorted out when the vector is stored to LDS (fixup).
+                const uint32_t rr = r < r_lim ? r : r_lim - 1;
+                const uint32_t cc = c + 4 <= c_lim ? c : (c_lim >= 4 ? c_lim - 4 : 0);
+                const float *q = base + (size_t)rr * ld + cc;
+                f32x4 v;
+                if (c_lim >= 4) { // uniform: operands narrower than one vector are read by element
+                    v = reinterpret_cast<const f32x4_u *>(q)->v;
+                } else {
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) v[e] = (uint32_t)e < c_lim ? q[e] : 0.f;
                 }
                 dst[i] = v;
             }
         }
     };
     // ---- registers -> LDS ------------------------------------------------------------------
-    auto sstore = [&](float *slab, const f32x4 *src, auto kc_tag, auto rows_tag, auto nv_tag) {
+    // FIX: the vectors came from the clamped loads of a checked slab: element e of the vector
+    // that should start at column c sits at index (c - cc) + e of what was loaded, if it exists.
+    auto sstore = [&](float *slab, const f32x4 *src, uint32_t row0, uint32_t row_lim, uint32_t k0, auto kc_tag, auto rows_tag,
+                      auto nv_tag, auto fix_tag) {
         constexpr bool KC = decltype(kc_tag)::value;
         constexpr int ROWS = decltype(rows_tag)::value;
         constexpr int NV = decltype(nv_tag)::value;
+        constexpr bool FIX = decltype(fix_tag)::value;
         constexpr int LD = Slab<ROWS, BK, KC>::LD;
 #pragma unroll
         for (int i = 0; i < NV; ++i) {
@@ -188,22 +200,67 @@ void gemm_f32_mfma_kernel(MArgs<float> g) {
             int off;
             if constexpr (KC) off = (q / (BK / 4)) * LD + 4 * (q % (BK / 4));
             else off = (q / (ROWS / 4)) * LD + 4 * (q % (ROWS / 4));
-            *reinterpret_cast<f32x4 *>(slab + off) = src[i];
+            f32x4 v = src[i];
+            if constexpr (FIX) {
+                // keeps the compiler from folding this path into the unchecked one as selects, which
+                // would charge every interior slab for the lane sorting
+                asm volatile("" ::: "memory");
+                uint32_t r, c, r_lim, c_lim;
+                if constexpr (KC) {
+                    r = row0 + q / (BK / 4); c = k0 + 4 * (q % (BK / 4));
+                    r_lim = row_lim; c_lim = g.K;
+                } else {
+                    r = k0 + q / (ROWS / 4); c = row0 + 4 * (q % (ROWS / 4));
+                    r_lim = g.K; c_lim = row_lim;
+                }
+                const uint32_t cc = c + 4 <= c_lim ? c : (c_lim >= 4 ? c_lim - 4 : 0);
+                const uint32_t shift = c - cc;
+                const f32x4 t = v;
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    const uint32_t idx = shift + e;
+                    float x = t[3];
+                    x = idx == 2 ? t[2] : x;
+                    x = idx == 1 ? t[1] : x;
+                    x = idx == 0 ? t[0] : x;
+                    const bool ok = (r < r_lim) & (c + e < c_lim);
+                    v[e] = ok ? x : 0.f;
+                }
+            }
+            *reinterpret_cast<f32x4 *>(slab + off) = v;
         }
     };
 
     using std::integral_constant;
+    // In the bounds-checked instantiation most work is still interior: a tile that lies inside C
+    // needs checks only on the slab that holds the k tail.  The choice is uniform over the work-group.
+    const bool tile_inside = !EDGE || (m0 + BM <= g.M && n0 + BN <= g.N);
+    const uint32_t k_inside = g.K - g.K % BK; // slabs starting below this are complete
     auto load_ab = [&](uint32_t k0) {
-        gload(ra, g.A, g.lda, m0, g.M, k0, integral_constant<bool, A_K>{}, integral_constant<int, BM>{},
-              integral_constant<int, A_V4>{});
-        gload(rb, g.B, g.ldb, n0, g.N, k0, integral_constant<bool, B_K>{}, integral_constant<int, BN>{},
-              integral_constant<int, B_V4>{});
+        if (!EDGE || (tile_inside && k0 < k_inside)) {
+            gload(ra, g.A, g.lda, m0, g.M, k0, integral_constant<bool, A_K>{}, integral_constant<int, BM>{},
+                  integral_constant<int, A_V4>{}, std::false_type{});
+            gload(rb, g.B, g.ldb, n0, g.N, k0, integral_constant<bool, B_K>{}, integral_constant<int, BN>{},
+                  integral_constant<int, B_V4>{}, std::false_type{});
+        } else {
+            gload(ra, g.A, g.lda, m0, g.M, k0, integral_constant<bool, A_K>{}, integral_constant<int, BM>{},
+                  integral_constant<int, A_V4>{}, std::true_type{});
+            gload(rb, g.B, g.ldb, n0, g.N, k0, integral_constant<bool, B_K>{}, integral_constant<int, BN>{},
+                  integral_constant<int, B_V4>{}, std::true_type{});
+        }
     };
-    auto store_ab = [&](int buf) {
-        sstore(As + buf * SA::SIZE, ra, integral_constant<bool, A_K>{}, integral_constant<int, BM>{},
-               integral_constant<int, A_V4>{});
-        sstore(Bs + buf * SB::SIZE, rb, integral_constant<bool, B_K>{}, integral_constant<int, BN>{},
-               integral_constant<int, B_V4>{});
+    auto store_ab = [&](int buf, uint32_t k0) {
+        if (!EDGE || (tile_inside && k0 < k_inside)) {
+            sstore(As + buf * SA::SIZE, ra, m0, g.M, k0, integral_constant<bool, A_K>{}, integral_constant<int, BM>{},
+                   integral_constant<int, A_V4>{}, std::false_type{});
+            sstore(Bs + buf * SB::SIZE, rb, n0, g.N, k0, integral_constant<bool, B_K>{}, integral_constant<int, BN>{},
+                   integral_constant<int, B_V4>{}, std::false_type{});
+        } else {
+            sstore(As + buf * SA::SIZE, ra, m0, g.M, k0, integral_constant<bool, A_K>{}, integral_constant<int, BM>{},
+                   integral_constant<int, A_V4>{}, std::true_type{});
+            sstore(Bs + buf * SB::SIZE, rb, n0, g.N, k0, integral_constant<bool, B_K>{}, integral_constant<int, BN>{},
+                   integral_constant<int, B_V4>{}, std::true_type{});
+        }
     };
 
     const uint32_t ktiles = (g.K + BK - 1) / BK;
@@ -234,7 +291,7 @@ void gemm_f32_mfma_kernel(MArgs<float> g) {
     };
 
     load_ab(0);
-    store_ab(0);
+    store_ab(0, 0);
     __syncthreads();
 
     // Fragment registers are double-buffered: the LDS reads for step s+1 are issued before the
@@ -257,7 +314,7 @@ void gemm_f32_mfma_kernel(MArgs<float> g) {
             if (s + 1 < S) {
                 read_frags(cur, s + 1, af[(s + 1) & 1], bf[(s + 1) & 1]);
             } else if (more) {
-                store_ab(cur ^ 1);
+                store_ab(cur ^ 1, (kt + 1) * BK);
                 __syncthreads();
                 read_frags(cur ^ 1, 0, af[(s + 1) & 1], bf[(s + 1) & 1]);
             }
@@ -271,22 +328,33 @@ void gemm_f32_mfma_kernel(MArgs<float> g) {
         }
     }
 
-    // ---- epilogue: acc register r of lane l is C[8*(r/4) + 4*(l/32) + r%4][l%32] of its 32x32 block
+    // ---- epilogue: acc register r of lane l is C[8*(r/4) + 4*(l/32) + r%4][l%32] of its 32x32 block.
+    // The reads of C_old (beta given) are issued for a whole 32x32 block before any is used; in the
+    // bounds-checked instantiation their addresses are clamped into C instead of being skipped, so
+    // that they stay one batch of independent loads (a load inside a branch is waited for on the spot).
     const float alpha = g.alpha, beta = g.beta;
 #pragma unroll
     for (int i = 0; i < FM; ++i)
 #pragma unroll
         for (int j = 0; j < FN; ++j) {
             const uint32_t col = n0 + wn * WN + j * 32 + l32;
+            const uint32_t colc = EDGE ? min(col, g.N - 1) : col;
+            float old[16];
+            if (g.epi == EPI_ALPHA_BETA) {
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    const uint32_t row = m0 + wm * WM + i * 32 + 8 * (r / 4) + 4 * lhi + (r % 4);
+                    const uint32_t rowc = EDGE ? min(row, g.M - 1) : row;
+                    old[r] = g.C[(size_t)rowc * g.ldc + colc];
+                }
+            }
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
                 const uint32_t row = m0 + wm * WM + i * 32 + 8 * (r / 4) + 4 * lhi + (r % 4);
-                if (EDGE && (row >= g.M || col >= g.N)) continue;
-                float *p = g.C + (size_t)row * g.ldc + col;
                 float v = acc[i][j][r];
                 if (g.epi == EPI_ALPHA) v = alpha * v;
-                else if (g.epi == EPI_ALPHA_BETA) v = alpha * v + beta * (*p);
-                *p = v;
+                else if (g.epi == EPI_ALPHA_BETA) v = alpha * v + beta * old[r];
+                if (!EDGE || ((row < g.M) & (col < g.N))) g.C[(size_t)row * g.ldc + col] = v;
             }
         }
 }
@@ -339,10 +407,11 @@ void gemm_f64_mfma_kernel(MArgs<double> g) {
     f64x2 ra[A_V2], rb[B_V2];
 
     auto gload = [&](f64x2 *dst, const double *__restrict__ base, uint32_t ld, uint32_t row0, uint32_t row_lim,
-                     uint32_t k0, auto kc_tag, auto rows_tag, auto nv_tag) {
+                     uint32_t k0, auto kc_tag, auto rows_tag, auto nv_tag, auto check_tag) {
         constexpr bool KC = decltype(kc_tag)::value;
         constexpr int ROWS = decltype(rows_tag)::value;
         constexpr int NV = decltype(nv_tag)::value;
+        constexpr bool CHECK = decltype(check_tag)::value;
 #pragma unroll
         for (int i = 0; i < NV; ++i) {
             const int q = tid + i * NT;
@@ -357,24 +426,30 @@ void gemm_f64_mfma_kernel(MArgs<double> g) {
             const double *p = base + (size_t)r * ld + c;
             if constexpr (!EDGE) {
                 dst[i] = *reinterpret_cast<const f64x2 *>(p);
+            } else if constexpr (!CHECK) {
+                dst[i] = reinterpret_cast<const f64x2_u *>(p)->v;
             } else {
-                f64x2 v = {0.0, 0.0};
-                if (r < r_lim) {
-                    if (c + 1 < c_lim) {
-                        v = reinterpret_cast<const f64x2_u *>(p)->v;
-                    } else {
-                        if (c + 0 < c_lim) v[0] = p[0];
-                        if (c + 1 < c_lim) v[1] = p[1];
-                    }
+                // clamped raw load; the fixup happens at the LDS store, as in the f32 kernel
+                const uint32_t rr = r < r_lim ? r : r_lim - 1;
+                const uint32_t cc = c + 2 <= c_lim ? c : (c_lim >= 2 ? c_lim - 2 : 0);
+                const double *q = base + (size_t)rr * ld + cc;
+                f64x2 v;
+                if (c_lim >= 2) {
+                    v = reinterpret_cast<const f64x2_u *>(q)->v;
+                } else {
+                    v[0] = q[0];
+                    v[1] = 0.0;
                 }
                 dst[i] = v;
             }
         }
     };
-    auto sstore = [&](double *slab, const f64x2 *src, auto kc_tag, auto rows_tag, auto nv_tag) {
+    auto sstore = [&](double *slab, const f64x2 *src, uint32_t row0, uint32_t row_lim, uint32_t k0, auto kc_tag, auto rows_tag,
+                      auto nv_tag, auto fix_tag) {
         constexpr bool KC = decltype(kc_tag)::value;
         constexpr int ROWS = decltype(rows_tag)::value;
         constexpr int NV = decltype(nv_tag)::value;
+        constexpr bool FIX = decltype(fix_tag)::value;
         constexpr int LD = SlabD<ROWS, BK, KC>::LD;
 #pragma unroll
         for (int i = 0; i < NV; ++i) {
@@ -382,24 +457,60 @@ void gemm_f64_mfma_kernel(MArgs<double> g) {
             int off;
             if constexpr (KC) off = (q / (BK / 2)) * LD + 2 * (q % (BK / 2));
             else off = (q / (ROWS / 2)) * LD + 2 * (q % (ROWS / 2));
-            *reinterpret_cast<f64x2 *>(slab + off) = src[i];
+            f64x2 v = src[i];
+            if constexpr (FIX) {
+                asm volatile("" ::: "memory"); // as in the f32 kernel: keep this a branch, not selects
+                uint32_t r, c, r_lim, c_lim;
+                if constexpr (KC) {
+                    r = row0 + q / (BK / 2); c = k0 + 2 * (q % (BK / 2));
+                    r_lim = row_lim; c_lim = g.K;
+                } else {
+                    r = k0 + q / (ROWS / 2); c = row0 + 2 * (q % (ROWS / 2));
+                    r_lim = g.K; c_lim = row_lim;
+                }
+                const uint32_t cc = c + 2 <= c_lim ? c : (c_lim >= 2 ? c_lim - 2 : 0);
+                const uint32_t shift = c - cc;
+                const f64x2 t = v;
+#pragma unroll
+                for (int e = 0; e < 2; ++e) {
+                    const double x = shift + e == 0 ? t[0] : t[1];
+                    const bool ok = (r < r_lim) & (c + e < c_lim);
+                    v[e] = ok ? x : 0.0;
+                }
+            }
+            *reinterpret_cast<f64x2 *>(slab + off) = v;
         }
     };
 
     using std::integral_constant;
-    auto load_a = [&](uint32_t k0) {
-        gload(ra, g.A, g.lda, m0, g.M, k0, integral_constant<bool, A_K>{}, integral_constant<int, BM>{},
-              integral_constant<int, A_V2>{});
+    // interior tiles of the bounds-checked instantiation check only the slab with the k tail
+    const bool tile_inside = !EDGE || (m0 + BM <= g.M && n0 + BN <= g.N);
+    const uint32_t k_inside = g.K - g.K % BK;
+    auto load_ab = [&](uint32_t k0) {
+        if (!EDGE || (tile_inside && k0 < k_inside)) {
+            gload(ra, g.A, g.lda, m0, g.M, k0, integral_constant<bool, A_K>{}, integral_constant<int, BM>{},
+                  integral_constant<int, A_V2>{}, std::false_type{});
+            gload(rb, g.B, g.ldb, n0, g.N, k0, integral_constant<bool, B_K>{}, integral_constant<int, BN>{},
+                  integral_constant<int, B_V2>{}, std::false_type{});
+        } else {
+            gload(ra, g.A, g.lda, m0, g.M, k0, integral_constant<bool, A_K>{}, integral_constant<int, BM>{},
+                  integral_constant<int, A_V2>{}, std::true_type{});
+            gload(rb, g.B, g.ldb, n0, g.N, k0, integral_constant<bool, B_K>{}, integral_constant<int, BN>{},
+                  integral_constant<int, B_V2>{}, std::true_type{});
+        }
     };
-    auto load_b = [&](uint32_t k0) {
-        gload(rb, g.B, g.ldb, n0, g.N, k0, integral_constant<bool, B_K>{}, integral_constant<int, BN>{},
-              integral_constant<int, B_V2>{});
-    };
-    auto store_ab = [&](int buf) {
-        sstore(As + buf * SA::SIZE, ra, integral_constant<bool, A_K>{}, integral_constant<int, BM>{},
-               integral_constant<int, A_V2>{});
-        sstore(Bs + buf * SB::SIZE, rb, integral_constant<bool, B_K>{}, integral_constant<int, BN>{},
-               integral_constant<int, B_V2>{});
+    auto store_ab = [&](int buf, uint32_t k0) {
+        if (!EDGE || (tile_inside && k0 < k_inside)) {
+            sstore(As + buf * SA::SIZE, ra, m0, g.M, k0, integral_constant<bool, A_K>{}, integral_constant<int, BM>{},
+                   integral_constant<int, A_V2>{}, std::false_type{});
+            sstore(Bs + buf * SB::SIZE, rb, n0, g.N, k0, integral_constant<bool, B_K>{}, integral_constant<int, BN>{},
+                   integral_constant<int, B_V2>{}, std::false_type{});
+        } else {
+            sstore(As + buf * SA::SIZE, ra, m0, g.M, k0, integral_constant<bool, A_K>{}, integral_constant<int, BM>{},
+                   integral_constant<int, A_V2>{}, std::true_type{});
+            sstore(Bs + buf * SB::SIZE, rb, n0, g.N, k0, integral_constant<bool, B_K>{}, integral_constant<int, BN>{},
+                   integral_constant<int, B_V2>{}, std::true_type{});
+        }
     };
 
     const uint32_t ktiles = (g.K + BK - 1) / BK;
@@ -429,9 +540,8 @@ void gemm_f64_mfma_kernel(MArgs<double> g) {
         }
     };
 
-    load_a(0);
-    load_b(0);
-    store_ab(0);
+    load_ab(0);
+    store_ab(0, 0);
     __syncthreads();
 
     // same schedule as the f32 kernel: double-buffered fragments, hand-over in front of the last
@@ -442,16 +552,13 @@ void gemm_f64_mfma_kernel(MArgs<double> g) {
     for (uint32_t kt = 0; kt < ktiles; ++kt) {
         const int cur = kt & 1;
         const bool more = kt + 1 < ktiles;
-        if (more) {
-            load_a((kt + 1) * BK);
-            load_b((kt + 1) * BK);
-        }
+        if (more) load_ab((kt + 1) * BK);
 #pragma unroll
         for (int s = 0; s < S; ++s) {
             if (s + 1 < S) {
                 read_frags(cur, s + 1, af[(s + 1) & 1], bf[(s + 1) & 1]);
             } else if (more) {
-                store_ab(cur ^ 1);
+                store_ab(cur ^ 1, (kt + 1) * BK);
                 __syncthreads();
                 read_frags(cur ^ 1, 0, af[(s + 1) & 1], bf[(s + 1) & 1]);
             }
@@ -471,15 +578,23 @@ void gemm_f64_mfma_kernel(MArgs<double> g) {
 #pragma unroll
         for (int j = 0; j < FN; ++j) {
             const uint32_t col = n0 + wn * WN + j * 16 + l16;
+            const uint32_t colc = EDGE ? min(col, g.N - 1) : col;
+            double old[4];
+            if (g.epi == EPI_ALPHA_BETA) { // batched, clamped reads of C_old (see the f32 kernel)
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    const uint32_t row = m0 + wm * WM + i * 16 + 4 * r + lq;
+                    const uint32_t rowc = EDGE ? min(row, g.M - 1) : row;
+                    old[r] = g.C[(size_t)rowc * g.ldc + colc];
+                }
+            }
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
                 const uint32_t row = m0 + wm * WM + i * 16 + 4 * r + lq;
-                if (EDGE && (row >= g.M || col >= g.N)) continue;
-                double *p = g.C + (size_t)row * g.ldc + col;
                 double v = acc[i][j][r];
                 if (g.epi == EPI_ALPHA) v = alpha * v;
-                else if (g.epi == EPI_ALPHA_BETA) v = alpha * v + beta * (*p);
-                *p = v;
+                else if (g.epi == EPI_ALPHA_BETA) v = alpha * v + beta * old[r];
+                if (!EDGE || ((row < g.M) & (col < g.N))) g.C[(size_t)row * g.ldc + col] = v;
             }
         }
 }
@@ -579,9 +694,9 @@ struct VariantDesc {
 const VariantDesc k_variants[] = {
     {"mfma_f32_256x128", WK_F32, 256, 128, 16, 0.943, 0.25, &launch_f32<256, 128, 16, 2, 2, 2>},
     {"mfma_f32_128x128", WK_F32, 128, 128, 16, 0.885, 0.25, &launch_f32<128, 128, 16, 2, 2, 3>},
-    {"mfma_f32_64x64", WK_F32, 64, 64, 16, 0.730, 0.10, &launch_f32<64, 64, 16, 2, 2, 4>},
+    {"mfma_f32_64x64", WK_F32, 64, 64, 32, 0.780, 0.10, &launch_f32<64, 64, 32, 2, 2, 4>},
     {"mfma_f64_128x128", WK_F64, 128, 128, 16, 0.908, 0.20, &launch_f64<128, 128, 16, 2, 2, 2>},
-    {"mfma_f64_64x64", WK_F64, 64, 64, 16, 0.800, 0.22, &launch_f64<64, 64, 16, 2, 2, 4>},
+    {"mfma_f64_64x64", WK_F64, 64, 64, 32, 0.800, 0.22, &launch_f64<64, 64, 32, 2, 2, 2>},
     {"mfma_f64_128x64", WK_F64, 128, 64, 16, 0.863, 0.25, &launch_f64<128, 64, 16, 2, 2, 3>},
 };
 constexpr int k_num_variants = sizeof(k_variants) / sizeof(k_variants[0]);
@@ -616,6 +731,10 @@ int wk::gemm_mfma_variant_dtype(int variant) {
 // CU has nothing to overlap its hand-overs and epilogue with), small tiles when the others would
 // leave CUs idle (1024^3, tall-skinny) or quantise badly (4097 x 4095: 544 tiles of 256x128 put
 // three tiles on some CUs and two on the rest).
+// The 64x64 tiles use k-slabs of 32: with one or two small tiles per CU the matrix work of a slab
+// is shorter than the latency of the global loads behind it, and the deeper slab halves the number
+// of such waits (f32 1024^3: 76 -> 84 TFLOP/s, 2048x1024x4096: 116 -> 130; f64 8192x256x8192:
+// 56 -> 60); the larger tiles measured no better with it.
 int wk::gemm_mfma_pick(const GemmProblem &p) {
     if (p.dtype != WK_F32 && p.dtype != WK_F64) return -1;
     if (p.M > 0x7fffffffull || p.N > 0x7fffffffull || p.K > 0x7fffffffull || p.lda > 0x7fffffffull ||
