@@ -314,6 +314,9 @@ void gemm_f32_mfma_kernel(MArgs<float> g) {
             if (s + 1 < S) {
                 read_frags(cur, s + 1, af[(s + 1) & 1], bf[(s + 1) & 1]);
             } else if (more) {
+                // (placing the barrier behind the first or second quarter of this step's matrix
+                // instructions, so that the LDS stores complete underneath them, measured 7 % slower
+                // at 8192^3 NN)
                 store_ab(cur ^ 1, (kt + 1) * BK);
                 __syncthreads();
                 read_frags(cur ^ 1, 0, af[(s + 1) & 1], bf[(s + 1) & 1]);
