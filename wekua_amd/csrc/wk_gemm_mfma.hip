@@ -136,7 +136,12 @@ void gemm_f32_mfma_kernel(MArgs<float> g) {
 #pragma unroll
             for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
 
-    f32x4 ra[A_V4], rb[B_V4]; // staging registers: global -> LDS
+    // Staging registers, global -> LDS.  The small tile keeps two sets and requests slab kt+2 while
+    // slab kt is computed: with one or two 64x64 tiles on a CU a slab's matrix work is shorter than
+    // the latency of a global load, so one slab of lead time does not cover it.  The large tiles
+    // measured no different with the deeper lead and keep one set.
+    constexpr int PF = (BM * BN <= 64 * 64) ? 2 : 1;
+    f32x4 ra[PF][A_V4], rb[PF][B_V4];
 
     // ---- global -> registers -----------------------------------------------------------
     // KCONTIG: slab is ROWS x BK, q -> (row = q / (BK/4), c4 = q % (BK/4)), address row*ld + k0 + 4*c4
@@ -236,7 +241,7 @@ void gemm_f32_mfma_kernel(MArgs<float> g) {
     // needs checks only on the slab that holds the k tail.  The choice is uniform over the work-group.
     const bool tile_inside = !EDGE || (m0 + BM <= g.M && n0 + BN <= g.N);
     const uint32_t k_inside = g.K - g.K % BK; // slabs starting below this are complete
-    auto load_ab = [&](uint32_t k0) {
+    auto load_ab = [&](uint32_t k0, f32x4 *ra, f32x4 *rb) {
         if (!EDGE || (tile_inside && k0 < k_inside)) {
             gload(ra, g.A, g.lda, m0, g.M, k0, integral_constant<bool, A_K>{}, integral_constant<int, BM>{},
                   integral_constant<int, A_V4>{}, std::false_type{});
@@ -249,7 +254,7 @@ void gemm_f32_mfma_kernel(MArgs<float> g) {
                   integral_constant<int, B_V4>{}, std::true_type{});
         }
     };
-    auto store_ab = [&](int buf, uint32_t k0) {
+    auto store_ab = [&](int buf, uint32_t k0, const f32x4 *ra, const f32x4 *rb) {
         if (!EDGE || (tile_inside && k0 < k_inside)) {
             sstore(As + buf * SA::SIZE, ra, m0, g.M, k0, integral_constant<bool, A_K>{}, integral_constant<int, BM>{},
                    integral_constant<int, A_V4>{}, std::false_type{});
@@ -290,44 +295,132 @@ void gemm_f32_mfma_kernel(MArgs<float> g) {
         }
     };
 
-    load_ab(0);
-    store_ab(0, 0);
+    load_ab(0, ra[0], rb[0]);
+    store_ab(0, 0, ra[0], rb[0]);
+    if (PF == 2 && ktiles > 1) load_ab(BK, ra[PF - 1], rb[PF - 1]);
     __syncthreads();
 
     // Fragment registers are double-buffered: the LDS reads for step s+1 are issued before the
     // matrix instructions of step s, and the slab hand-over (LDS store of the next slab, barrier,
     // first fragment reload) sits in front of the last step's matrix instructions, so that LDS
     // latency and barrier skew are covered by matrix work of the same wavefront.
-    // Slab kt+1 is requested from global memory at the top of iteration kt.  Requesting it a whole
-    // iteration (refill right after the hand-over) or one and a half iterations earlier (a second
-    // staging register set) was measured and changes nothing (134-138 TFLOP/s at 8192^3 in all
-    // three schedules), so the simplest one is kept.
+    // With one staging set slab kt+1 is requested from global memory at the top of iteration kt
+    // (requesting it a whole iteration earlier was measured on the large tiles and changes nothing);
+    // with two sets slab kt+2 is requested there and slab kt+1, requested an iteration ago, is the
+    // one handed over.
+    //
+    // The loop exists in three spellings of the same schedule.  How two co-resident work-groups
+    // interleave on a CU depends on the instruction order the compiler derives from the spelling,
+    // and the rate moves by up to 10 % with it; each tile (for 256x128: each operand layout) uses the one that measured fastest on
+    // MI355X (same box, same process, f32, alpha and beta given):
+    //   LOOP 0  `if (more)` around the hand-over, written out      256x128: NN 142.0, NT 133.4, TN 129.4
+    //   LOOP 1  the same inside a lambda                            256x128: NN 129.3, NT 131.6, TN 128.6;
+    //                                                               128x128 at 2048x4096x4096: 136.4 (LOOP 0: 127.3, LOOP 2: 125.3)
+    //   LOOP 2  last slab peeled, hand-over fenced                  256x128: NN 133.4, NT 134.3, TN 131.1;
+    //           (sched_barrier) so that matrix instructions         64x64 at 1024^3: 90.8 (LOOP 1: 88.7), 2048^3: 122.8 (115-120)
+    //           are not hoisted above the barrier
+    constexpr int LOOP = (BM * BN <= 64 * 64) ? 2 : (BM * BN <= 128 * 128 ? 1 : ((A_K && !B_K) ? 0 : 2));
+    static_assert(LOOP == 2 || PF == 1, "only the peeled loop knows the two-set prefetch");
     f32x4 af[2][FM], bf[2][FN];
     read_frags(0, 0, af[0], bf[0]);
 
-    for (uint32_t kt = 0; kt < ktiles; ++kt) {
-        const int cur = kt & 1;
-        const bool more = kt + 1 < ktiles;
-        if (more) load_ab((kt + 1) * BK);
+    auto mfma_step = [&](int s) {
 #pragma unroll
-        for (int s = 0; s < S; ++s) {
-            if (s + 1 < S) {
-                read_frags(cur, s + 1, af[(s + 1) & 1], bf[(s + 1) & 1]);
-            } else if (more) {
-                // (placing the barrier behind the first or second quarter of this step's matrix
-                // instructions, so that the LDS stores complete underneath them, measured 7 % slower
-                // at 8192^3 NN)
-                store_ab(cur ^ 1, (kt + 1) * BK);
-                __syncthreads();
-                read_frags(cur ^ 1, 0, af[(s + 1) & 1], bf[(s + 1) & 1]);
+        for (int t = 0; t < 4; ++t)
+#pragma unroll
+            for (int i = 0; i < FM; ++i)
+#pragma unroll
+                for (int j = 0; j < FN; ++j)
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(af[s & 1][i][t], bf[s & 1][j][t], acc[i][j], 0, 0, 0);
+    };
+
+    if constexpr (LOOP == 0) {
+        for (uint32_t kt = 0; kt < ktiles; ++kt) {
+            const int cur = kt & 1;
+            const bool more = kt + 1 < ktiles;
+            if (more) load_ab((kt + 1) * BK, ra[0], rb[0]);
+#pragma unroll
+            for (int s = 0; s < S; ++s) {
+                if (s + 1 < S) {
+                    read_frags(cur, s + 1, af[(s + 1) & 1], bf[(s + 1) & 1]);
+                } else if (more) {
+                    store_ab(cur ^ 1, (kt + 1) * BK, ra[0], rb[0]);
+                    __syncthreads();
+                    read_frags(cur ^ 1, 0, af[(s + 1) & 1], bf[(s + 1) & 1]);
+                }
+#pragma unroll
+                for (int t = 0; t < 4; ++t)
+#pragma unroll
+                    for (int i = 0; i < FM; ++i)
+#pragma unroll
+                        for (int j = 0; j < FN; ++j)
+                            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(af[s & 1][i][t], bf[s & 1][j][t], acc[i][j], 0, 0, 0);
             }
+        }
+    } else if constexpr (LOOP == 1) {
+        auto iteration = [&](uint32_t kt) {
+            const int cur = kt & 1;
+            const bool more = kt + 1 < ktiles;
+            if (more) load_ab((kt + 1) * BK, ra[0], rb[0]);
 #pragma unroll
-            for (int t = 0; t < 4; ++t)
+            for (int s = 0; s < S; ++s) {
+                if (s + 1 < S) {
+                    read_frags(cur, s + 1, af[(s + 1) & 1], bf[(s + 1) & 1]);
+                } else if (more) {
+                    store_ab(cur ^ 1, (kt + 1) * BK, ra[0], rb[0]);
+                    __syncthreads();
+                    read_frags(cur ^ 1, 0, af[(s + 1) & 1], bf[(s + 1) & 1]);
+                }
+                mfma_step(s);
+            }
+        };
+        for (uint32_t kt = 0; kt < ktiles; ++kt) iteration(kt);
+    } else {
+        // one iteration that hands over to slab kt+1; P = parity of kt, a compile-time constant so
+        // that the staging sets stay in registers
+        auto iteration = [&](uint32_t kt, auto parity_tag) {
+            constexpr int P = decltype(parity_tag)::value;
+            const int cur = kt & 1;
+            if constexpr (PF == 1) {
+                load_ab((kt + 1) * BK, ra[0], rb[0]);
+            } else {
+                if (kt + 2 < ktiles) load_ab((kt + 2) * BK, ra[P], rb[P]); // set P held slab kt, already in LDS
+            }
+            constexpr int NEXT = PF == 1 ? 0 : 1 - P; // the set holding slab kt+1
 #pragma unroll
-                for (int i = 0; i < FM; ++i)
+            for (int s = 0; s < S; ++s) {
+                if (s + 1 < S) {
+                    read_frags(cur, s + 1, af[(s + 1) & 1], bf[(s + 1) & 1]);
+                } else {
+                    __builtin_amdgcn_sched_barrier(0);
+                    store_ab(cur ^ 1, (kt + 1) * BK, ra[NEXT], rb[NEXT]);
+                    __syncthreads();
+                    read_frags(cur ^ 1, 0, af[(s + 1) & 1], bf[(s + 1) & 1]);
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+                mfma_step(s);
+            }
+        };
+        uint32_t kt = 0;
+        if constexpr (PF == 1) {
+            for (; kt + 1 < ktiles; ++kt) iteration(kt, integral_constant<int, 0>{});
+        } else {
+            for (; kt + 2 < ktiles; kt += 2) {
+                iteration(kt, integral_constant<int, 0>{});
+                iteration(kt + 1, integral_constant<int, 1>{});
+            }
+            if (kt + 1 < ktiles) {
+                iteration(kt, integral_constant<int, 0>{});
+                ++kt;
+            }
+        }
+        {   // last slab: nothing to hand over
+            const int cur = kt & 1;
 #pragma unroll
-                    for (int j = 0; j < FN; ++j)
-                        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(af[s & 1][i][t], bf[s & 1][j][t], acc[i][j], 0, 0, 0);
+            for (int s = 0; s < S; ++s) {
+                if (s + 1 < S) read_frags(cur, s + 1, af[(s + 1) & 1], bf[(s + 1) & 1]);
+                mfma_step(s);
+            }
         }
     }
 
