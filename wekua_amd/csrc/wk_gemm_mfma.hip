@@ -500,7 +500,9 @@ void gemm_f64_mfma_kernel(MArgs<double> g) {
 #pragma unroll
             for (int r = 0; r < 4; ++r) acc[i][j][r] = 0.0;
 
-    f64x2 ra[A_V2], rb[B_V2];
+    // two staging sets for the small tile, as in the f32 kernel
+    constexpr int PF = (BM * BN <= 64 * 64) ? 2 : 1;
+    f64x2 ra[PF][A_V2], rb[PF][B_V2];
 
     auto gload = [&](f64x2 *dst, const double *__restrict__ base, uint32_t ld, uint32_t row0, uint32_t row_lim,
                      uint32_t k0, auto kc_tag, auto rows_tag, auto nv_tag, auto check_tag) {
@@ -582,7 +584,7 @@ void gemm_f64_mfma_kernel(MArgs<double> g) {
     // interior tiles of the bounds-checked instantiation check only the slab with the k tail
     const bool tile_inside = !EDGE || (m0 + BM <= g.M && n0 + BN <= g.N);
     const uint32_t k_inside = g.K - g.K % BK;
-    auto load_ab = [&](uint32_t k0) {
+    auto load_ab = [&](uint32_t k0, f64x2 *ra, f64x2 *rb) {
         if (!EDGE || (tile_inside && k0 < k_inside)) {
             gload(ra, g.A, g.lda, m0, g.M, k0, integral_constant<bool, A_K>{}, integral_constant<int, BM>{},
                   integral_constant<int, A_V2>{}, std::false_type{});
@@ -595,7 +597,7 @@ void gemm_f64_mfma_kernel(MArgs<double> g) {
                   integral_constant<int, B_V2>{}, std::true_type{});
         }
     };
-    auto store_ab = [&](int buf, uint32_t k0) {
+    auto store_ab = [&](int buf, uint32_t k0, const f64x2 *ra, const f64x2 *rb) {
         if (!EDGE || (tile_inside && k0 < k_inside)) {
             sstore(As + buf * SA::SIZE, ra, m0, g.M, k0, integral_constant<bool, A_K>{}, integral_constant<int, BM>{},
                    integral_constant<int, A_V2>{}, std::false_type{});
@@ -636,35 +638,84 @@ void gemm_f64_mfma_kernel(MArgs<double> g) {
         }
     };
 
-    load_ab(0);
-    store_ab(0, 0);
+    load_ab(0, ra[0], rb[0]);
+    store_ab(0, 0, ra[0], rb[0]);
+    if (PF == 2 && ktiles > 1) load_ab(BK, ra[PF - 1], rb[PF - 1]);
     __syncthreads();
 
-    // same schedule as the f32 kernel: double-buffered fragments, hand-over in front of the last
-    // step's matrix instructions, next slab requested at the top of the iteration
+    // Same schedule as the f32 kernel: double-buffered fragments, hand-over in front of the last
+    // step's matrix instructions.  The large tiles request slab kt+1 at the top of iteration kt
+    // around an `if (more)`; the small tile requests slab kt+2 there (two staging sets), runs its
+    // last slab after the loop and fences the hand-over against reordering.
     f64x2 af[2][FM], bf[2][FN];
     read_frags(0, 0, af[0], bf[0]);
 
-    for (uint32_t kt = 0; kt < ktiles; ++kt) {
-        const int cur = kt & 1;
-        const bool more = kt + 1 < ktiles;
-        if (more) load_ab((kt + 1) * BK);
+    auto mfma_step = [&](int s) {
+#pragma unroll
+        for (int t = 0; t < 2; ++t)
+#pragma unroll
+            for (int i = 0; i < FM; ++i)
+#pragma unroll
+                for (int j = 0; j < FN; ++j)
+                    acc[i][j] = __builtin_amdgcn_mfma_f64_16x16x4f64(af[s & 1][i][t], bf[s & 1][j][t], acc[i][j], 0, 0, 0);
+    };
+
+    if constexpr (PF == 1) {
+        for (uint32_t kt = 0; kt < ktiles; ++kt) {
+            const int cur = kt & 1;
+            const bool more = kt + 1 < ktiles;
+            if (more) load_ab((kt + 1) * BK, ra[0], rb[0]);
+#pragma unroll
+            for (int s = 0; s < S; ++s) {
+                if (s + 1 < S) {
+                    read_frags(cur, s + 1, af[(s + 1) & 1], bf[(s + 1) & 1]);
+                } else if (more) {
+                    store_ab(cur ^ 1, (kt + 1) * BK, ra[0], rb[0]);
+                    __syncthreads();
+                    read_frags(cur ^ 1, 0, af[(s + 1) & 1], bf[(s + 1) & 1]);
+                }
+#pragma unroll
+                for (int t = 0; t < 2; ++t)
+#pragma unroll
+                    for (int i = 0; i < FM; ++i)
+#pragma unroll
+                        for (int j = 0; j < FN; ++j)
+                            acc[i][j] = __builtin_amdgcn_mfma_f64_16x16x4f64(af[s & 1][i][t], bf[s & 1][j][t], acc[i][j], 0, 0, 0);
+            }
+        }
+    } else {
+        auto iteration = [&](uint32_t kt, auto parity_tag) {
+            constexpr int P = decltype(parity_tag)::value;
+            const int cur = kt & 1;
+            if (kt + 2 < ktiles) load_ab((kt + 2) * BK, ra[P], rb[P]);
+#pragma unroll
+            for (int s = 0; s < S; ++s) {
+                if (s + 1 < S) {
+                    read_frags(cur, s + 1, af[(s + 1) & 1], bf[(s + 1) & 1]);
+                } else {
+                    __builtin_amdgcn_sched_barrier(0);
+                    store_ab(cur ^ 1, (kt + 1) * BK, ra[1 - P], rb[1 - P]);
+                    __syncthreads();
+                    read_frags(cur ^ 1, 0, af[(s + 1) & 1], bf[(s + 1) & 1]);
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+                mfma_step(s);
+            }
+        };
+        uint32_t kt = 0;
+        for (; kt + 2 < ktiles; kt += 2) {
+            iteration(kt, integral_constant<int, 0>{});
+            iteration(kt + 1, integral_constant<int, 1>{});
+        }
+        if (kt + 1 < ktiles) {
+            iteration(kt, integral_constant<int, 0>{});
+            ++kt;
+        }
+        const int cur = kt & 1; // last slab: nothing to hand over
 #pragma unroll
         for (int s = 0; s < S; ++s) {
-            if (s + 1 < S) {
-                read_frags(cur, s + 1, af[(s + 1) & 1], bf[(s + 1) & 1]);
-            } else if (more) {
-                store_ab(cur ^ 1, (kt + 1) * BK);
-                __syncthreads();
-                read_frags(cur ^ 1, 0, af[(s + 1) & 1], bf[(s + 1) & 1]);
-            }
-#pragma unroll
-            for (int t = 0; t < 2; ++t)
-#pragma unroll
-                for (int i = 0; i < FM; ++i)
-#pragma unroll
-                    for (int j = 0; j < FN; ++j)
-                        acc[i][j] = __builtin_amdgcn_mfma_f64_16x16x4f64(af[s & 1][i][t], bf[s & 1][j][t], acc[i][j], 0, 0, 0);
+            if (s + 1 < S) read_frags(cur, s + 1, af[(s + 1) & 1], bf[(s + 1) & 1]);
+            mfma_step(s);
         }
     }
 
@@ -792,7 +843,7 @@ const VariantDesc k_variants[] = {
     {"mfma_f32_128x128", WK_F32, 128, 128, 16, 0.885, 0.25, &launch_f32<128, 128, 16, 2, 2, 3>},
     {"mfma_f32_64x64", WK_F32, 64, 64, 32, 0.780, 0.10, &launch_f32<64, 64, 32, 2, 2, 4>},
     {"mfma_f64_128x128", WK_F64, 128, 128, 16, 0.908, 0.20, &launch_f64<128, 128, 16, 2, 2, 2>},
-    {"mfma_f64_64x64", WK_F64, 64, 64, 32, 0.800, 0.22, &launch_f64<64, 64, 32, 2, 2, 2>},
+    {"mfma_f64_64x64", WK_F64, 64, 64, 32, 0.840, 0.05, &launch_f64<64, 64, 32, 2, 2, 2>},
     {"mfma_f64_128x64", WK_F64, 128, 64, 16, 0.863, 0.25, &launch_f64<128, 64, 16, 2, 2, 3>},
 };
 constexpr int k_num_variants = sizeof(k_variants) / sizeof(k_variants[0]);
