@@ -101,6 +101,45 @@ def test_integer_wraparound_bit_exact(dev, dtype, op_a, op_b):
             check(dev, dtype, M, N, K, op_a, op_b, alpha, beta, seed=21)   # full-range entries: overflow is the norm
 
 
+@pytest.mark.parametrize("dtype", ["i32", "u32"])
+@pytest.mark.parametrize("variant", ["tile64", "mfma_{}_64x128"])
+@pytest.mark.parametrize("op_a,op_b", OPS)
+def test_int32_every_variant_bit_exact(dev, dtype, variant, op_a, op_b):
+    """The int8-matrix-core decomposition and the vector-ALU kernel against the exact product modulo
+    2^32 on full-range entries: interior shapes (aligned), ragged shapes, K not a multiple of the slab,
+    every alpha / beta combination."""
+    variant = variant.format(dtype)
+    assert dev.lib.wk_gemm_force_variant(variant.encode()) == 0
+    try:
+        for (M, N, K) in [(64, 128, 32), (128, 256, 64), (192, 128, 416), (1, 1, 1), (65, 129, 33), (200, 300, 77), (63, 127, 500)]:
+            for alpha, beta in [(None, None), (3, None), (-5 if dtype == "i32" else 4000000000, 7), (None, 1)]:
+                check(dev, dtype, M, N, K, op_a, op_b, alpha, beta, seed=23)
+    finally:
+        dev.lib.wk_gemm_force_variant(b"auto")
+
+
+def test_int32_matrix_core_extremes(dev):
+    """Inputs built from the byte values that stress the signed-digit split: 0x00, 0x7f, 0x80, 0xff in
+    every byte position, so that every digit pair hits -128 * -128 and the row / column sum
+    corrections wrap many times."""
+    import oracle
+    vals = np.array([0x00000000, 0x7f7f7f7f, 0x80808080, 0xffffffff, 0x80000000, 0x7fffffff, 0x00800080, 0xff00ff00,
+                     0x01010101, 0x807f807f], dtype=np.uint32)
+    M, N, K = 128, 128, 320
+    rng = np.random.default_rng(77)
+    a = vals[rng.integers(0, len(vals), (M, K))].view(np.int32)
+    b = vals[rng.integers(0, len(vals), (K, N))].view(np.int32)
+    c = vals[rng.integers(0, len(vals), (M, N))].view(np.int32)
+    assert dev.lib.wk_gemm_variant(4, 0, 0, M, N, K, K, N, N, None, None, None).decode() == "mfma_i32_64x128"
+    dA, dB, dC = dev.upload(a), dev.upload(b), dev.upload(c)
+    dev.gemm("i32", 0, 0, M, N, K, -3, dA, K, dB, N, 5, dC, N)
+    got = dC.download(np.int32, (M, N))
+    want = oracle.semantic_gemm("i32", -3, a, 0, b, 0, 5, c)
+    assert np.array_equal(got, want)
+    for d in (dA, dB, dC):
+        d.free()
+
+
 @pytest.mark.parametrize("dtype", ["cf32", "cf64", "ci32", "cu16", "ci8", "ci64"])
 def test_complex(dev, dtype):
     for op_a, op_b in OPS:

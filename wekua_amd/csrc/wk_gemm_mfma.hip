@@ -845,11 +845,14 @@ const VariantDesc k_variants[] = {
     {"mfma_f64_128x128", WK_F64, 128, 128, 16, 0.908, 0.20, &launch_f64<128, 128, 16, 2, 2, 2>},
     {"mfma_f64_64x64", WK_F64, 64, 64, 32, 0.840, 0.05, &launch_f64<64, 64, 32, 2, 2, 2>},
     {"mfma_f64_128x64", WK_F64, 128, 64, 16, 0.863, 0.25, &launch_f64<128, 64, 16, 2, 2, 3>},
+    // 32-bit integers through the int8 matrix cores (wk_gemm_imfma.hip); same kernel for both signs
+    {"mfma_i32_64x128", WK_I32, 64, 128, 32, 1.0, 0.25, &gemm_i32_mfma_launch},
+    {"mfma_u32_64x128", WK_U32, 64, 128, 32, 1.0, 0.25, &gemm_i32_mfma_launch},
 };
 constexpr int k_num_variants = sizeof(k_variants) / sizeof(k_variants[0]);
 
 bool needs_edge(const GemmProblem &p, const VariantDesc &v) {
-    const size_t es = p.dtype == WK_F32 ? 4 : 8;
+    const size_t es = p.dtype == WK_F64 ? 8 : 4;
     const uint64_t vec = 16 / es;
     if (p.M % v.bm || p.N % v.bn || p.K % v.bk) return true;
     if (p.lda % vec || p.ldb % vec) return true;
@@ -883,7 +886,7 @@ int wk::gemm_mfma_variant_dtype(int variant) {
 // of such waits (f32 1024^3: 76 -> 84 TFLOP/s, 2048x1024x4096: 116 -> 130; f64 8192x256x8192:
 // 56 -> 60); the larger tiles measured no better with it.
 int wk::gemm_mfma_pick(const GemmProblem &p) {
-    if (p.dtype != WK_F32 && p.dtype != WK_F64) return -1;
+    if (p.dtype != WK_F32 && p.dtype != WK_F64 && p.dtype != WK_I32 && p.dtype != WK_U32) return -1;
     if (p.M > 0x7fffffffull || p.N > 0x7fffffffull || p.K > 0x7fffffffull || p.lda > 0x7fffffffull ||
         p.ldb > 0x7fffffffull || p.ldc > 0x7fffffffull)
         return -1;
