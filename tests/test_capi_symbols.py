@@ -68,7 +68,7 @@ def test_host_only_entry_points():
     v = lambda dt, n: lib.wk_gemm_variant(dt, 0, 0, n, n, n, n, n, n, None, None, None).decode()
     assert v(8, 8192).startswith("mfma_f32")
     assert v(9, 4096).startswith("mfma_f64")
-    assert v(4, 2048) == "mfma_i32_64x128" and v(5, 2048) == "mfma_u32_64x128"
+    assert v(4, 2048) == "mfma_i32_128x128" and v(5, 2048) == "mfma_u32_128x128" and v(4, 1024) == "mfma_i32_64x128"
     assert v(2, 2048) == "tile64" and v(6, 2048) == "tile64" and v(14, 512) == "tile64"
     assert v(18, 512) == "tile64"
     assert lib.wk_gemm_variant(8, 0, 0, 0, 4, 4, 4, 4, 4, None, None, None).decode() == "invalid"

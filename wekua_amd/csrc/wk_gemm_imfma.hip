@@ -16,7 +16,7 @@
 // So one 32-bit product costs ten int8 matrix products; against the vector ALU (a 32-bit
 // multiply-add per lane and clock at best) that is still several times faster.
 //
-// Work-group: 256 threads = 2 x 2 waves, macro tile 64 x 128, wave tile 32 x 64 (two 32x32 blocks),
+// Work-group: BM/32 x 2 waves (256 or 512 threads), macro tile BM x 128 with BM = 64 or 128, wave tile 32 x 64 (two 32x32 blocks),
 // four accumulator sets (one per shift i+j).  k-slab 32.  LDS holds, per operand and slab, four
 // digit planes [row slot][32 bytes of k + 8 pad]; the loader XORs with c and transposes 4x4 bytes with
 // v_perm_b32 so that every plane dword holds one digit of four consecutive k.
@@ -32,17 +32,18 @@ typedef int i32x16 __attribute__((ext_vector_type(16)));
 typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
 struct __attribute__((packed, aligned(4))) u32x4_u { u32x4 v; };
 
-constexpr int BM = 64, BN = 128, BK = 32, NT = 256;
+constexpr int BN = 128, BK = 32; // BM (64 or 128) and the thread count 4 * BM are template parameters
 // LDS geometry of a digit plane.  Row r of an operand lives at row slot (r % 4) * P + r / 4 and a
 // slot is LDB = 40 bytes: the loader of an m/n-contiguous operand writes one dword to each of four
 // ADJACENT rows per lane, lanes 16 bytes (four rows) apart, and without the regrouping those stores
 // hit two banks 16 ways.  With it (found by enumerating strides and group pitches) loader stores are
 // at most 2-way and the 8-byte fragment reads 2-way, which is their minimum.
 constexpr int LDB = BK + 8;
-constexpr int P_A = 20, P_B = 36;            // row-slot pitch of the four residue groups
-constexpr int PLANE_A = 4 * P_A * LDB, PLANE_B = 4 * P_B * LDB;
+// row-slot pitch of the four residue groups: 20 for a 64-row operand, 36 for a 128-row one
+constexpr int group_pitch(int rows) { return rows == 64 ? 20 : 36; }
+constexpr int plane_bytes(int rows) { return 4 * group_pitch(rows) * LDB; }
+constexpr int slab_bytes(int bm) { return 4 * (plane_bytes(bm) + plane_bytes(BN)); }
 template <int P> __device__ __forceinline__ constexpr int slot(int r) { return (r & 3) * P + (r >> 2); }
-constexpr int SLAB_BYTES = 4 * (PLANE_A + PLANE_B);
 constexpr uint32_t CBIAS = 0x80808080u;
 
 struct IArgs {
@@ -68,9 +69,12 @@ __device__ __forceinline__ void digit_planes(const uint32_t e[4], uint32_t p[4])
 
 // A_K / B_K: operand is k-contiguous in storage (A for op N, B for op T).  EDGE: ragged sizes or
 // rows that are only element-aligned.
-template <bool A_K, bool B_K, bool EDGE>
-__global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(2)))
+template <int BM, bool A_K, bool B_K, bool EDGE>
+__global__ __launch_bounds__(4 * BM) __attribute__((amdgpu_waves_per_eu(2)))
 void gemm_i32_mfma_kernel(IArgs g) {
+    constexpr int NT = 4 * BM;               // BM/32 x 2 waves
+    constexpr int P_A = group_pitch(BM), P_B = group_pitch(BN);
+    constexpr int PLANE_A = plane_bytes(BM), PLANE_B = plane_bytes(BN), SLAB_BYTES = slab_bytes(BM);
     extern __shared__ __align__(16) unsigned char lds_raw[];
     unsigned char *slabs = lds_raw;                                               // [2][SLAB_BYTES]
     uint32_t *row_sum = reinterpret_cast<uint32_t *>(lds_raw + 2 * SLAB_BYTES);   // [BM]
@@ -99,9 +103,11 @@ void gemm_i32_mfma_kernel(IArgs g) {
             for (int r = 0; r < 16; ++r) acc[s][b][r] = 0;
 
     // ---- loader --------------------------------------------------------------------------------
-    // k-contiguous operand of ROWS rows: vector q -> (row = q / 8, k = 4 * (q % 8)), NV = ROWS / 32 per thread.
-    // otherwise a thread owns one patch of 4 k x 4 rows: patch q -> (k = 4 * (q / (ROWS/4)), row = 4 * (q % (ROWS/4))).
-    constexpr int A_NV = A_K ? BM / 32 : 4, B_NV = B_K ? BN / 32 : 4;
+    // k-contiguous operand of ROWS rows: vector q -> (row = q / 8, k = 4 * (q % 8)), ROWS * 8 / NT per thread.
+    // otherwise a thread owns one patch of 4 k x 4 rows: patch q -> (k = 4 * (q / (ROWS/4)), row = 4 * (q % (ROWS/4)));
+    // there are ROWS * 2 patches; A's go to the first threads, B's to the last, so that with 512 threads
+    // two patch-loaded operands land on different threads.
+    constexpr int A_NV = A_K ? BM * 8 / NT : 4, B_NV = B_K ? BN * 8 / NT : 4;
     u32x4 ra[A_NV], rb[B_NV];
     uint32_t sum_a[4] = {0, 0, 0, 0}, sum_b[4] = {0, 0, 0, 0}; // KC: one per vector (its row); else one per patch column
 
@@ -124,31 +130,34 @@ void gemm_i32_mfma_kernel(IArgs g) {
         }
     };
     auto gload = [&](u32x4 *dst, const uint32_t *base, uint32_t ld, uint32_t row0, uint32_t row_lim, uint32_t k0, auto kc_tag,
-                     auto rows_tag) {
+                     auto rows_tag, auto first_tag) {
         constexpr bool KC = decltype(kc_tag)::value;
         constexpr int ROWS = decltype(rows_tag)::value;
+        constexpr int T0 = decltype(first_tag)::value; // first thread of the patch loaders
         if constexpr (KC) {
 #pragma unroll
-            for (int i = 0; i < ROWS / 32; ++i) {
+            for (int i = 0; i < ROWS * 8 / NT; ++i) {
                 const int q = tid + i * NT;
                 dst[i] = load_vec(base, ld, row0 + q / 8, row_lim, k0 + 4 * (q % 8), g.K);
             }
         } else {
-            if (tid < ROWS * 2) {
-                const uint32_t k = k0 + 4 * (tid / (ROWS / 4)), c = row0 + 4 * (tid % (ROWS / 4));
+            const int pq = tid - T0;
+            if (pq >= 0 && pq < ROWS * 2) {
+                const uint32_t k = k0 + 4 * (pq / (ROWS / 4)), c = row0 + 4 * (pq % (ROWS / 4));
 #pragma unroll
                 for (int t = 0; t < 4; ++t) dst[t] = load_vec(base, ld, k + t, g.K, c, row_lim);
             }
         }
     };
     // registers -> digit planes in LDS; also adds the raw elements into the running sums
-    auto sstore = [&](unsigned char *planes, int plane_bytes, const u32x4 *src, uint32_t *sums, auto kc_tag, auto rows_tag) {
+    auto sstore = [&](unsigned char *planes, const u32x4 *src, uint32_t *sums, auto kc_tag, auto rows_tag, auto first_tag) {
         constexpr bool KC = decltype(kc_tag)::value;
         constexpr int ROWS = decltype(rows_tag)::value;
-        constexpr int P = ROWS == BM ? P_A : P_B;
+        constexpr int T0 = decltype(first_tag)::value;
+        constexpr int P = group_pitch(ROWS), plane_bytes = 4 * P * LDB;
         if constexpr (KC) {
 #pragma unroll
-            for (int i = 0; i < ROWS / 32; ++i) {
+            for (int i = 0; i < ROWS * 8 / NT; ++i) {
                 const int q = tid + i * NT;
                 const uint32_t e[4] = {src[i][0], src[i][1], src[i][2], src[i][3]};
                 uint32_t p[4];
@@ -159,8 +168,9 @@ void gemm_i32_mfma_kernel(IArgs g) {
                 for (int d = 0; d < 4; ++d) *reinterpret_cast<uint32_t *>(planes + d * plane_bytes + off) = p[d];
             }
         } else {
-            if (tid < ROWS * 2) {
-                const int koff = 4 * (tid / (ROWS / 4)), row = 4 * (tid % (ROWS / 4));
+            const int pq = tid - T0;
+            if (pq >= 0 && pq < ROWS * 2) {
+                const int koff = 4 * (pq / (ROWS / 4)), row = 4 * (pq % (ROWS / 4));
 #pragma unroll
                 for (int c = 0; c < 4; ++c) {
                     const uint32_t e[4] = {src[0][c], src[1][c], src[2][c], src[3][c]};
@@ -175,14 +185,15 @@ void gemm_i32_mfma_kernel(IArgs g) {
         }
     };
     using std::integral_constant;
+    constexpr int T0_A = 0, T0_B = NT - BN * 2;
     auto load_ab = [&](uint32_t k0) {
-        gload(ra, g.A, g.lda, m0, g.M, k0, integral_constant<bool, A_K>{}, integral_constant<int, BM>{});
-        gload(rb, g.B, g.ldb, n0, g.N, k0, integral_constant<bool, B_K>{}, integral_constant<int, BN>{});
+        gload(ra, g.A, g.lda, m0, g.M, k0, integral_constant<bool, A_K>{}, integral_constant<int, BM>{}, integral_constant<int, T0_A>{});
+        gload(rb, g.B, g.ldb, n0, g.N, k0, integral_constant<bool, B_K>{}, integral_constant<int, BN>{}, integral_constant<int, T0_B>{});
     };
     auto store_ab = [&](int buf) {
         unsigned char *s = slabs + buf * SLAB_BYTES;
-        sstore(s, PLANE_A, ra, sum_a, integral_constant<bool, A_K>{}, integral_constant<int, BM>{});
-        sstore(s + 4 * PLANE_A, PLANE_B, rb, sum_b, integral_constant<bool, B_K>{}, integral_constant<int, BN>{});
+        sstore(s, ra, sum_a, integral_constant<bool, A_K>{}, integral_constant<int, BM>{}, integral_constant<int, T0_A>{});
+        sstore(s + 4 * PLANE_A, rb, sum_b, integral_constant<bool, B_K>{}, integral_constant<int, BN>{}, integral_constant<int, T0_B>{});
     };
 
     // ---- matrix work of one slab ----------------------------------------------------------------
@@ -234,19 +245,21 @@ void gemm_i32_mfma_kernel(IArgs g) {
     // ---- row / column sums of the raw elements ------------------------------------------------------
     if constexpr (A_K) {
 #pragma unroll
-        for (int i = 0; i < BM / 32; ++i) atomicAdd(&row_sum[(tid + i * NT) / 8], sum_a[i]);
+        for (int i = 0; i < BM * 8 / NT; ++i) atomicAdd(&row_sum[(tid + i * NT) / 8], sum_a[i]);
     } else {
-        if (tid < BM * 2)
+        const int pq = tid - T0_A;
+        if (pq >= 0 && pq < BM * 2)
 #pragma unroll
-            for (int c = 0; c < 4; ++c) atomicAdd(&row_sum[4 * (tid % (BM / 4)) + c], sum_a[c]);
+            for (int c = 0; c < 4; ++c) atomicAdd(&row_sum[4 * (pq % (BM / 4)) + c], sum_a[c]);
     }
     if constexpr (B_K) {
 #pragma unroll
-        for (int i = 0; i < BN / 32; ++i) atomicAdd(&col_sum[(tid + i * NT) / 8], sum_b[i]);
+        for (int i = 0; i < BN * 8 / NT; ++i) atomicAdd(&col_sum[(tid + i * NT) / 8], sum_b[i]);
     } else {
-        if (tid < BN * 2)
+        const int pq = tid - T0_B;
+        if (pq >= 0 && pq < BN * 2)
 #pragma unroll
-            for (int c = 0; c < 4; ++c) atomicAdd(&col_sum[4 * (tid % (BN / 4)) + c], sum_b[c]);
+            for (int c = 0; c < 4; ++c) atomicAdd(&col_sum[4 * (pq % (BN / 4)) + c], sum_b[c]);
     }
     __syncthreads();
 
@@ -278,9 +291,10 @@ void gemm_i32_mfma_kernel(IArgs g) {
     }
 }
 
-template <bool AK, bool BKC, bool EDGE> int launch_one(hipStream_t st, const GemmProblem &p) {
-    constexpr size_t lds = 2 * SLAB_BYTES + (BM + BN) * sizeof(uint32_t);
-    auto kern = gemm_i32_mfma_kernel<AK, BKC, EDGE>;
+template <int BM, bool AK, bool BKC, bool EDGE> int launch_one(hipStream_t st, const GemmProblem &p) {
+    constexpr int NT = 4 * BM;
+    constexpr size_t lds = 2 * slab_bytes(BM) + (BM + BN) * sizeof(uint32_t);
+    auto kern = gemm_i32_mfma_kernel<BM, AK, BKC, EDGE>;
     static const hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
                                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     if (attr != hipSuccess) { (void)hipGetLastError(); return hip_code(attr); }
@@ -299,11 +313,9 @@ template <bool AK, bool BKC, bool EDGE> int launch_one(hipStream_t st, const Gem
     return launch_status();
 }
 
-} // namespace
-
-int wk::gemm_i32_mfma_launch(hipStream_t st, const GemmProblem &p, bool edge) {
+template <int BM> int launch_bm(hipStream_t st, const GemmProblem &p, bool edge) {
     const int sel = (p.op_a ? 0 : 2) | (p.op_b ? 1 : 0); // bit1: A k-contiguous, bit0: B k-contiguous
-#define WK_CASE(AK, BKC) return edge ? launch_one<AK, BKC, true>(st, p) : launch_one<AK, BKC, false>(st, p)
+#define WK_CASE(AK, BKC) return edge ? launch_one<BM, AK, BKC, true>(st, p) : launch_one<BM, AK, BKC, false>(st, p)
     switch (sel) {
     case 0: WK_CASE(false, false);
     case 1: WK_CASE(false, true);
@@ -312,3 +324,8 @@ int wk::gemm_i32_mfma_launch(hipStream_t st, const GemmProblem &p, bool edge) {
     }
 #undef WK_CASE
 }
+
+} // namespace
+
+int wk::gemm_i32_mfma_launch_64(hipStream_t st, const GemmProblem &p, bool edge) { return launch_bm<64>(st, p, edge); }
+int wk::gemm_i32_mfma_launch_128(hipStream_t st, const GemmProblem &p, bool edge) { return launch_bm<128>(st, p, edge); }

@@ -166,7 +166,8 @@ int gemm_generic_launch(hipStream_t st, const GemmProblem &p);
 // MFMA kernels for f32 / f64 / i32 / u32 (wk_gemm_mfma.hip); `variant` indexes mfma_variant_name()
 int gemm_mfma_launch(hipStream_t st, const GemmProblem &p, int variant);
 // i32 / u32 on the int8 matrix cores (wk_gemm_imfma.hip); reached through the variant table
-int gemm_i32_mfma_launch(hipStream_t st, const GemmProblem &p, bool edge);
+int gemm_i32_mfma_launch_64(hipStream_t st, const GemmProblem &p, bool edge);  // macro tile 64 x 128
+int gemm_i32_mfma_launch_128(hipStream_t st, const GemmProblem &p, bool edge); // macro tile 128 x 128
 int gemm_mfma_pick(const GemmProblem &p);        // -1: not applicable
 const char *gemm_mfma_variant_name(int variant); // nullptr past the end
 int gemm_mfma_variant_dtype(int variant);
