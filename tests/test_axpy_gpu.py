@@ -20,7 +20,10 @@ def run_axpy(dev, dtype, x, alpha, y, pitched=False):
     x3 = x.reshape((depth, rows, cols) + tail)
     y3 = y.reshape((depth, rows, cols) + tail)
     if pitched:
-        xrp, yrp = cols + 3, cols + 5
+        if pitched == "aligned":  # row starts on 16-byte boundaries for every dtype: the vector row kernel
+            xrp, yrp = (cols + 15) // 16 * 16 + 16, (cols + 15) // 16 * 16 + 32
+        else:
+            xrp, yrp = cols + 3, cols + 5
         xs = np.full((depth, rows + 1, xrp) + tail, 55, dtype=x.dtype)
         ys = np.full((depth, rows + 2, yrp) + tail, 66, dtype=y.dtype)
         xs[:, :rows, :cols] = x3
@@ -72,6 +75,25 @@ def test_axpy_all_dtypes_shapes_alphas(dev, dtype):
             x = make_operand(dtype, shape, 7)
             y = make_operand(dtype, shape, 8)
             got = run_axpy(dev, dtype, x, alpha, y)
+            want = expect(dtype, x, alpha, y)
+            if oracle.is_float(dtype) and cx:
+                np.testing.assert_allclose(got, want, rtol=1e-5 if dtype.endswith("f32") else 1e-13,
+                                           atol=1e-6 if dtype.endswith("f32") else 1e-14)
+            else:
+                assert np.array_equal(got, want), f"{dtype} shape={shape} alpha={alpha}"
+
+
+@pytest.mark.parametrize("dtype", ALL_DTYPES)
+def test_axpy_aligned_pitched_rows(dev, dtype):
+    """Rows with gaps between them whose starts are 16-byte aligned (the layout of every 2-D / 3-D
+    Tensor): full vectors plus a per-row tail, nothing written into the gaps."""
+    signed = oracle.real_np_dtype(dtype).kind != "u"
+    cx = oracle.is_complex(dtype)
+    for shape in [(3, 16), (5, 37), (2, 3, 70), (7, 1), (4, 300), (33, 1025)]:
+        for alpha in ([None, (2, 1)] + ([(-1, 0)] if signed else []) if cx else [None, 3] + ([-1] if signed else [])):
+            x = make_operand(dtype, shape, 19)
+            y = make_operand(dtype, shape, 20)
+            got = run_axpy(dev, dtype, x, alpha, y, pitched="aligned")
             want = expect(dtype, x, alpha, y)
             if oracle.is_float(dtype) and cx:
                 np.testing.assert_allclose(got, want, rtol=1e-5 if dtype.endswith("f32") else 1e-13,

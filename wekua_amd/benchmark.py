@@ -98,9 +98,11 @@ def time_gemm(ses, dtype, M, N, K, op_a, op_b, alpha, beta, iters=10):
 
 
 def time_axpy(ses, dtype, n, iters=50):
+    """n: element count of a 1-D tensor, or a shape tuple (2-D / 3-D tensors have pitched rows)."""
     rd = raw.real_np_dtype(dtype)
     wk = ses.wk
-    x, y = ses.tensor(dtype, _operand(rd, (n,), 1)), ses.tensor(dtype, _operand(rd, (n,), 2))
+    shape = n if isinstance(n, tuple) else (n,)
+    x, y = ses.tensor(dtype, _operand(rd, shape, 1)), ses.tensor(dtype, _operand(rd, shape, 2))
     ses.pipeline.waitAndCleanup()
     alpha = 0.75 if rd.kind == "f" else 3
     ms = ses.time_ms(lambda: wk.blas.axpy(ses.pipeline, x, alpha, y), iters)
@@ -125,6 +127,10 @@ def cmd_axpy(ses, args):
         ms = time_axpy(ses, args.dtype, n)
         nbytes = 3 * n * raw.elem_size(args.dtype)
         print(f"{args.dtype:5s} {n:10d} {ms * 1e3:9.2f} {nbytes / ms / 1e6:8.0f}", flush=True)
+    for shape in ((8192, 8192), (4096, 4096), (2048, 4096), (1000, 1000), (16, 1024, 4096)):
+        ms = time_axpy(ses, args.dtype, shape)
+        nbytes = 3 * int(np.prod(shape)) * raw.elem_size(args.dtype)
+        print(f"{args.dtype:5s} {'x'.join(map(str, shape)):>10s} {ms * 1e3:9.2f} {nbytes / ms / 1e6:8.0f}", flush=True)
 
 
 def cmd_configs(ses, args):

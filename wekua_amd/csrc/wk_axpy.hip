@@ -95,6 +95,40 @@ __global__ __launch_bounds__(PITCHED_BLOCK) void axpy_pitched_kernel(const T *__
     }
 }
 
+// Pitched rows whose starts and pitches are 16-byte aligned (every 2-D / 3-D Tensor of the host
+// mirror): blockIdx.y walks the rows of all slices, blockIdx.x the 16-byte vectors of a row, so no
+// lane divides anything per element and every access is a full vector; the < VE tail of each row
+// is done by element.
+template <typename T, int MODE>
+__global__ __launch_bounds__(256) void axpy_rows_kernel(const T *__restrict__ x, T *__restrict__ y, uint64_t rows, uint64_t cols,
+                                                        uint64_t total_rows, uint64_t xrp, uint64_t xsp, uint64_t yrp,
+                                                        uint64_t ysp, typename elem_traits<T>::acc alpha) {
+    constexpr int VE = 16 / sizeof(T);
+    const uint64_t nvec = cols / VE;
+    for (uint64_t row = blockIdx.y; row < total_rows; row += gridDim.y) {
+        const uint64_t i = row / rows, j = row % rows;
+        const T *xr_ = x + i * xsp + j * xrp;
+        T *yr_ = y + i * ysp + j * yrp;
+        const u32x4 *xv = reinterpret_cast<const u32x4 *>(xr_);
+        u32x4 *yv = reinterpret_cast<u32x4 *>(yr_);
+        for (uint64_t v = blockIdx.x * 256ull + threadIdx.x; v < nvec; v += (uint64_t)gridDim.x * 256ull) {
+            const u32x4 xq = __builtin_nontemporal_load(xv + v), yq = __builtin_nontemporal_load(yv + v);
+            T xe[VE], ye[VE];
+            __builtin_memcpy(xe, &xq, 16);
+            __builtin_memcpy(ye, &yq, 16);
+#pragma unroll
+            for (int e = 0; e < VE; ++e) ye[e] = axpy_elem<T, MODE>(xe[e], ye[e], alpha);
+            u32x4 out;
+            __builtin_memcpy(&out, ye, 16);
+            __builtin_nontemporal_store(out, yv + v);
+        }
+        if (blockIdx.x == 0) {
+            const uint64_t k = nvec * VE + threadIdx.x;
+            if (k < cols) yr_[k] = axpy_elem<T, MODE>(xr_[k], yr_[k], alpha);
+        }
+    }
+}
+
 // isSubstracting, src/blas/axpy.zig:66-91
 template <typename T> bool is_subtracting(int dtype, const void *host_alpha) {
     using R = typename elem_traits<T>::real;
@@ -132,6 +166,18 @@ int launch(wk_stream *s, const uint64_t shape3[3], const T *x, uint64_t xrp, uin
         if (blocks > 0x7fffffffull) return WK_E_INVALID_VALUE;
         hipLaunchKernelGGL((axpy_stream_kernel<T, MODE>), dim3((unsigned)blocks), dim3(AXPY_BLOCK), 0, s->stream, x, y, n,
                            alpha);
+        return launch_status();
+    }
+    const bool rows_aligned = aligned && xrp % VE == 0 && yrp % VE == 0 && xsp % VE == 0 && ysp % VE == 0;
+    if (rows_aligned && c >= VE) {
+        const uint64_t total_rows = d * r;
+        uint64_t gx = (c / VE + 255) / 256;
+        if (gx > 16384) gx = 16384;
+        uint64_t gy = (16384 + gx - 1) / gx;
+        if (gy > total_rows) gy = total_rows;
+        if (gy > 65535) gy = 65535;
+        hipLaunchKernelGGL((axpy_rows_kernel<T, MODE>), dim3((unsigned)gx, (unsigned)gy), dim3(256), 0, s->stream, x, y, r, c,
+                           total_rows, xrp, xsp, yrp, ysp, alpha);
         return launch_status();
     }
     const uint64_t want = (n + PITCHED_BLOCK - 1) / PITCHED_BLOCK;
