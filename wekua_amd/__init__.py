@@ -89,6 +89,7 @@ HOST_SIGNATURES = {
     "wkz_random_uniform": (ci, [vp, vp, u64p, vp, vp]),
     "wkz_to_complex": (ci, [vp, vp, vp, ci]),
     "wkz_to_real": (ci, [vp, vp, vp, ci]),
+    "wkz_print": (ci, [vp, vp, ctypes.c_char_p, u64, u64p]),
     # math / nn (the MLP training step)
     "wkz_math_dot": (ci, [vp, vp, vp]),
     "wkz_math_sum": (ci, [vp, vp, vp]),
@@ -354,6 +355,21 @@ def transpose(pipeline: Pipeline, result_tensor: Tensor, tensor: Tensor, dim0: i
     _check(_lib().wkz_transpose(pipeline._h, result_tensor._h, tensor._h, dim0, dim1), "transpose")
 
 
+def printZ(pipeline: Pipeline, tensor: Tensor) -> str:
+    """tensor.printZ (src/tensor/print.zig): the text `print` writes."""
+    need = u64()
+    _check(_lib().wkz_print(pipeline._h, tensor._h, None, 0, ctypes.byref(need)), "printZ")
+    buf = ctypes.create_string_buffer(need.value + 1)
+    _check(_lib().wkz_print(pipeline._h, tensor._h, buf, need.value + 1, None), "printZ")
+    return buf.value.decode()
+
+
+def print_tensor(pipeline: Pipeline, tensor: Tensor) -> None:
+    """tensor.print (`print` is taken in Python)."""
+    import sys
+    sys.stdout.write(printZ(pipeline, tensor))
+
+
 class Space(enum.IntEnum):
     real = 0
     imag = 1
@@ -445,5 +461,5 @@ class blas:
 from . import nn  # noqa: E402  (needs the classes above)
 from .nn import math  # noqa: E402,F401
 
-__all__ = ["nn", "math", "transpose", "random", "convertions", "Space", "Context", "Pipeline", "Tensor", "CommandQueue", "DeviceType", "memory", "fill", "identity", "blas",
+__all__ = ["nn", "math", "printZ", "print_tensor", "transpose", "random", "convertions", "Space", "Context", "Pipeline", "Tensor", "CommandQueue", "DeviceType", "memory", "fill", "identity", "blas",
            "GemmPackedTensors", "WekuaError", "DTYPE_NAMES", "dtype_id", "elem_size", "is_complex", "real_np_dtype"]

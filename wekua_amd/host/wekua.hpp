@@ -30,8 +30,12 @@
 //     operands through LDS, so pack() only validates.
 #pragma once
 
+#include <algorithm>
+#include <charconv>
 #include <chrono>
+#include <cmath>
 #include <cstdint>
+#include <cstdio>
 #include <cstring>
 #include <exception>
 #include <limits>
@@ -511,6 +515,223 @@ template <typename R> void toReal(Pipeline *pipeline, Tensor<core::Complex<R>> *
     pipeline->append(1);
 }
 } // namespace convertions
+
+// ---- print (src/tensor/print.zig) -----------------------------------------------------------------
+// Host-side text rendering of a tensor: the first and last entries of every dimension, numpy style.
+// The layout rules (how many items per row, "..." elision, widths, brackets, the trailing
+// shape / dtype line) follow print.zig:103-361; number formatting follows Zig's `{d}` / `{e}`
+// (exponent without sign padding: 1.50000e0, 1.00000e-3).
+namespace print_detail {
+inline void pad(std::string &o, size_t n) { o.append(n, ' '); }
+inline void right(std::string &o, const std::string &v, size_t width) {
+    if (v.size() < width) o.append(width - v.size(), ' ');
+    o += v;
+    o += ',';
+}
+// Zig renders a float by taking the shortest decimal that round-trips in ITS type (so 0.3f is "3",
+// exponent -1, not 0.30000001192...) and then rounding that decimal, half up, to the requested
+// number of fraction digits.
+struct Decimal {
+    bool negative;
+    std::string digits; // d1 d2 d3 ...: value = d1.d2d3... * 10^exponent
+    int exponent;
+};
+template <typename F> Decimal shortest(F v) {
+    char buf[64];
+    auto r = std::to_chars(buf, buf + sizeof buf, v, std::chars_format::scientific);
+    std::string t(buf, r.ptr);
+    Decimal d{false, "", 0};
+    size_t i = 0;
+    if (t[0] == '-') d.negative = true, i = 1;
+    for (; i < t.size() && t[i] != 'e'; ++i)
+        if (t[i] != '.') d.digits += t[i];
+    d.exponent = std::atoi(t.c_str() + i + 1);
+    return d;
+}
+// keeps `keep` leading digits of d.digits (may be <= 0), rounding half up; returns true on a carry out
+inline bool round_digits(std::string &digits, long keep) {
+    if (keep < 0) {
+        digits.clear();
+        return false;
+    }
+    if ((long)digits.size() <= keep) {
+        digits.append(keep - digits.size(), '0');
+        return false;
+    }
+    const bool up = digits[keep] >= '5';
+    digits.resize(keep);
+    if (!up) return false;
+    for (long i = keep; i-- > 0;) {
+        if (digits[i] != '9') {
+            ++digits[i];
+            return false;
+        }
+        digits[i] = '0';
+    }
+    return true;
+}
+template <typename F> std::string special(F v) { return std::isnan(v) ? "nan" : v < 0 ? "-inf" : "inf"; }
+template <typename F> std::string zig_e(F v, int prec) {
+    if (!std::isfinite(v)) return special(v);
+    Decimal d = shortest(v);
+    if (round_digits(d.digits, prec + 1)) {
+        d.digits.insert(d.digits.begin(), '1');
+        d.digits.pop_back();
+        ++d.exponent;
+    }
+    std::string o = d.negative ? "-" : "";
+    o += d.digits[0];
+    if (prec > 0) o += "." + d.digits.substr(1);
+    return o + "e" + std::to_string(d.exponent);
+}
+template <typename F> std::string zig_d(F v, int prec) {
+    if (!std::isfinite(v)) return special(v);
+    Decimal d = shortest(v);
+    long int_digits = (long)d.exponent + 1; // digits in front of the point (<= 0: leading zeros behind it)
+    std::string digits = d.digits;
+    if (int_digits <= 0) {
+        digits.insert(0, (size_t)(1 - int_digits), '0');
+        int_digits = 1;
+    }
+    if (round_digits(digits, int_digits + prec)) {
+        digits.insert(digits.begin(), '1');
+        ++int_digits;
+    }
+    std::string o = d.negative ? "-" : "";
+    o += digits.substr(0, int_digits);
+    if (prec > 0) o += "." + digits.substr(int_digits);
+    return o;
+}
+template <typename I> std::string int_str(I v) { return std::to_string((long long)v); }
+template <> inline std::string int_str<uint64_t>(uint64_t v) { return std::to_string(v); }
+
+template <typename T> void vector(std::string &o, size_t padding, const T *buf, uint64_t cols) {
+    using Sub = typename core::scalar_of<T>::type;
+    constexpr bool cplx = core::isComplex<T>();
+    pad(o, padding);
+    auto loop = [&](uint64_t head, uint64_t max_items, size_t ell_width, auto &&item) {
+        for (uint64_t i = 0; i < head && i < cols; ++i) item(i);
+        if (cols > head) {
+            uint64_t dec = head + 1;
+            if (cols > max_items) {
+                dec = head;
+                right(o, "...", ell_width);
+            }
+            for (uint64_t i = std::max<uint64_t>(head, cols - dec); i < cols; ++i) item(i);
+        }
+    };
+    if constexpr (std::is_integral_v<Sub>) {
+        const std::string ext = std::is_signed_v<Sub> ? int_str(std::numeric_limits<Sub>::min()) : int_str(std::numeric_limits<Sub>::max());
+        const std::string widest = cplx ? (std::is_signed_v<Sub> ? ext + ext + "j" : ext + "+" + ext + "j") : ext;
+        const size_t width = widest.size() + 1;
+        uint64_t max_items = std::max<uint64_t>(cplx ? 3 : 5, 65 / widest.size());
+        if (max_items % 2 == 0) ++max_items;
+        const uint64_t head = std::min<uint64_t>(cols, (max_items - 1) / 2);
+        loop(head, max_items, width, [&](uint64_t i) {
+            if constexpr (cplx) {
+                const Sub re = buf[i].real, im = buf[i].imag;
+                std::string v;
+                if (re != 0 && im != 0) v = int_str(re) + (im < 0 ? "" : "+") + int_str(im) + "j";
+                else if (im != 0) v = int_str(im) + "j";
+                else v = int_str(re);
+                right(o, v, width);
+            } else {
+                right(o, int_str(buf[i]), width);
+            }
+        });
+    } else if constexpr (cplx) {
+        loop(2, 5, 24, [&](uint64_t i) {
+            const Sub re = buf[i].real, im = buf[i].imag;
+            const bool rz = std::fabs(re) < 1e-8, iz = std::fabs(im) < 1e-8;
+            std::string v;
+            if (!rz && !iz) v = zig_e(re, 2) + (im < 0 ? "" : "+") + zig_e(im, 2) + "j";
+            else if (rz && !iz) v = zig_e(im, 5) + "j";
+            else v = zig_e(re, 5);
+            right(o, v, 24);
+        });
+    } else {
+        loop(4, 9, 14, [&](uint64_t i) {
+            const T v = buf[i];
+            right(o, (10000.0 - std::fabs((double)v)) > 1e-8 ? zig_d(v, 8) : zig_e(v, 5), 14);
+        });
+    }
+}
+
+template <typename T>
+void dim(std::string &o, size_t padding, const T *buf, const uint64_t *shape, const uint64_t *pitches, size_t nd) {
+    pad(o, padding);
+    o += '[';
+    if (nd > 2) {
+        o += '\n';
+        const uint64_t n = shape[0], pitch = pitches[0];
+        for (uint64_t i = 0; i < std::min<uint64_t>(2, n); ++i) dim<T>(o, padding + 2, buf + i * pitch, shape + 1, pitches + 1, nd - 1);
+        if (n > 2) {
+            if (n > 4) {
+                o += '\n';
+                pad(o, padding + 2);
+                o += "... \n";
+            }
+            for (uint64_t i = std::max<uint64_t>(2, n - 2); i < n; ++i) dim<T>(o, padding + 2, buf + i * pitch, shape + 1, pitches + 1, nd - 1);
+        }
+        o += '\n';
+    } else if (nd == 1) {
+        vector<T>(o, padding, buf, shape[0]);
+    } else {
+        const uint64_t rows = shape[0], cols = shape[1], pitch = pitches[0];
+        for (uint64_t i = 0; i < std::min<uint64_t>(2, rows); ++i) {
+            o += '\n';
+            vector<T>(o, padding + 2, buf + i * pitch, cols);
+        }
+        if (rows > 2) {
+            if (rows > 4) {
+                o += '\n';
+                pad(o, padding + 2);
+                o += " ... ";
+            }
+            for (uint64_t i = std::max<uint64_t>(2, rows - 2); i < rows; ++i) {
+                o += '\n';
+                vector<T>(o, padding + 2, buf + i * pitch, cols);
+            }
+        }
+        o += '\n';
+    }
+    pad(o, padding);
+    o += "],";
+    if (padding > 0) o += '\n';
+}
+template <typename T> const char *type_name() {
+    using Sub = typename core::scalar_of<T>::type;
+    if constexpr (std::is_same_v<Sub, float>) return "f32";
+    else if constexpr (std::is_same_v<Sub, double>) return "f64";
+    else if constexpr (std::is_signed_v<Sub>) return sizeof(Sub) == 1 ? "i8" : sizeof(Sub) == 2 ? "i16" : sizeof(Sub) == 4 ? "i32" : "i64";
+    else return sizeof(Sub) == 1 ? "u8" : sizeof(Sub) == 2 ? "u16" : sizeof(Sub) == 4 ? "u32" : "u64";
+}
+} // namespace print_detail
+
+// printZ (print.zig:316-361): drains the pipeline, copies the buffer to the host, renders it
+template <typename T> std::string printZ(Pipeline *pipeline, Tensor<T> *tensor) {
+    std::vector<T> host(tensor->dimensions.number_of_elements);
+    check(wk_copy_d2h_rect_async(pipeline->command_queue->stream, host.data(), tensor->memory_layout.size, tensor->memory_layout.size,
+                                 tensor->buffer, tensor->memory_layout.size, tensor->memory_layout.size, tensor->memory_layout.size,
+                                 1, 1));
+    pipeline->append(1);
+    pipeline->waitAndCleanup();
+    std::string o = "Tensor(";
+    const auto &shape = tensor->dimensions.shape;
+    print_detail::dim<T>(o, 0, host.data(), shape.data(), tensor->dimensions.pitches.data(), shape.size());
+    o += " shape=(" + std::to_string(shape[0]);
+    for (size_t i = 1; i < shape.size(); ++i) o += ", " + std::to_string(shape[i]);
+    o += ')';
+    o += core::isComplex<T>() ? std::string(", dtype=complex_") + print_detail::type_name<T>() + ")\n"
+                              : std::string(", dtype=") + print_detail::type_name<T>() + ")\n";
+    return o;
+}
+// print (print.zig:363-382): to standard output
+template <typename T> void print(Pipeline *pipeline, Tensor<T> *tensor) {
+    const std::string o = printZ<T>(pipeline, tensor);
+    std::fwrite(o.data(), 1, o.size(), stdout);
+    std::fflush(stdout);
+}
 
 namespace blas {
 

@@ -336,6 +336,23 @@ int wkz_to_real(void *pipeline, void *src, void *dst, int space) {
     });
 }
 
+// printZ into a caller buffer: returns the text length (without terminator) through *needed; copies at
+// most capacity - 1 bytes plus a terminator.  Call with capacity 0 to size the buffer.
+int wkz_print(void *pipeline, void *tensor, char *out, uint64_t capacity, uint64_t *needed) {
+    return guard([&] {
+        TensorHandle *h = static_cast<TensorHandle *>(tensor);
+        dispatch(h->dtype, [&]<typename T>() {
+            const std::string text = printZ<T>(static_cast<Pipeline *>(pipeline), static_cast<Tensor<T> *>(h->tensor));
+            if (needed) *needed = text.size();
+            if (out && capacity) {
+                const size_t n = std::min<size_t>(text.size(), capacity - 1);
+                std::memcpy(out, text.data(), n);
+                out[n] = 0;
+            }
+        });
+    });
+}
+
 // ---- blas -----------------------------------------------------------------------------------------
 int wkz_axpy(void *pipeline, void *x, const void *host_alpha, void *y) {
     return guard([&] {
