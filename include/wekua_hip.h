@@ -99,7 +99,10 @@ int  wk_event_record(wk_event *e, wk_stream *s);          /* the event a cl enqu
 int  wk_event_sync(wk_event *e);                          /* cl.event.wait */
 int  wk_event_elapsed_ms(wk_event *start, wk_event *stop, float *out_ms);
 
-/* ---- memory: cl.buffer.create/release (src/tensor/main.zig:229-234,253-263) ----------- */
+/* ---- memory: cl.buffer.create/release (src/tensor/main.zig:229-234,253-263) -----------
+ * Pointers from wk_malloc are at least 1 KiB aligned and must go back through wk_free (blocks of
+ * 1 MiB and more start 0 / 3 / 6 / 9 KiB into their device allocation in turn, which spreads
+ * streams that are walked in step over the memory channels; WK_ALLOC_COLOURS=0 disables it). */
 int  wk_malloc(wk_device *dev, size_t bytes, void **out_dptr);
 int  wk_free(wk_device *dev, void *dptr);
 int  wk_mem_info(wk_device *dev, size_t *free_bytes, size_t *total_bytes);

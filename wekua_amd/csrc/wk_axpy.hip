@@ -96,23 +96,25 @@ __global__ __launch_bounds__(PITCHED_BLOCK) void axpy_pitched_kernel(const T *__
 }
 
 // Pitched rows whose starts and pitches are 16-byte aligned (every 2-D / 3-D Tensor of the host
-// mirror): blockIdx.y walks the rows of all slices, blockIdx.x the 16-byte vectors of a row, so no
-// lane divides anything per element and every access is a full vector; the < VE tail of each row
-// is done by element.
+// mirror): the same shape as the stream kernel -- one wavefront per work-group, one 16-byte vector
+// per lane, streaming stores -- with blockIdx.x over the vectors of a row, blockIdx.y over the rows
+// and blockIdx.z over the slices, so nothing is divided anywhere; the < VE tail of each row is done
+// by element.
 template <typename T, int MODE>
-__global__ __launch_bounds__(256) void axpy_rows_kernel(const T *__restrict__ x, T *__restrict__ y, uint64_t rows, uint64_t cols,
-                                                        uint64_t total_rows, uint64_t xrp, uint64_t xsp, uint64_t yrp,
-                                                        uint64_t ysp, typename elem_traits<T>::acc alpha) {
+__global__ __launch_bounds__(AXPY_BLOCK) void axpy_rows_kernel(const T *__restrict__ x, T *__restrict__ y, uint64_t rows,
+                                                               uint64_t cols, uint64_t depth, uint64_t xrp, uint64_t xsp,
+                                                               uint64_t yrp, uint64_t ysp, typename elem_traits<T>::acc alpha) {
     constexpr int VE = 16 / sizeof(T);
     const uint64_t nvec = cols / VE;
-    for (uint64_t row = blockIdx.y; row < total_rows; row += gridDim.y) {
-        const uint64_t i = row / rows, j = row % rows;
+    const uint64_t v = (uint64_t)blockIdx.x * AXPY_BLOCK + threadIdx.x;
+    for (uint64_t i = blockIdx.z; i < depth; i += gridDim.z)
+    for (uint64_t j = blockIdx.y; j < rows; j += gridDim.y) {
         const T *xr_ = x + i * xsp + j * xrp;
         T *yr_ = y + i * ysp + j * yrp;
-        const u32x4 *xv = reinterpret_cast<const u32x4 *>(xr_);
-        u32x4 *yv = reinterpret_cast<u32x4 *>(yr_);
-        for (uint64_t v = blockIdx.x * 256ull + threadIdx.x; v < nvec; v += (uint64_t)gridDim.x * 256ull) {
-            const u32x4 xq = __builtin_nontemporal_load(xv + v), yq = __builtin_nontemporal_load(yv + v);
+        if (v < nvec) {
+            const u32x4 *xv = reinterpret_cast<const u32x4 *>(xr_) + v;
+            u32x4 *yv = reinterpret_cast<u32x4 *>(yr_) + v;
+            const u32x4 xq = __builtin_nontemporal_load(xv), yq = __builtin_nontemporal_load(yv);
             T xe[VE], ye[VE];
             __builtin_memcpy(xe, &xq, 16);
             __builtin_memcpy(ye, &yq, 16);
@@ -120,7 +122,7 @@ __global__ __launch_bounds__(256) void axpy_rows_kernel(const T *__restrict__ x,
             for (int e = 0; e < VE; ++e) ye[e] = axpy_elem<T, MODE>(xe[e], ye[e], alpha);
             u32x4 out;
             __builtin_memcpy(&out, ye, 16);
-            __builtin_nontemporal_store(out, yv + v);
+            asm volatile("global_store_dwordx4 %0, %1, off nt sc0 sc1" ::"v"(yv), "v"(out) : "memory");
         }
         if (blockIdx.x == 0) {
             const uint64_t k = nvec * VE + threadIdx.x;
@@ -170,14 +172,11 @@ int launch(wk_stream *s, const uint64_t shape3[3], const T *x, uint64_t xrp, uin
     }
     const bool rows_aligned = aligned && xrp % VE == 0 && yrp % VE == 0 && xsp % VE == 0 && ysp % VE == 0;
     if (rows_aligned && c >= VE) {
-        const uint64_t total_rows = d * r;
-        uint64_t gx = (c / VE + 255) / 256;
-        if (gx > 16384) gx = 16384;
-        uint64_t gy = (16384 + gx - 1) / gx;
-        if (gy > total_rows) gy = total_rows;
-        if (gy > 65535) gy = 65535;
-        hipLaunchKernelGGL((axpy_rows_kernel<T, MODE>), dim3((unsigned)gx, (unsigned)gy), dim3(256), 0, s->stream, x, y, r, c,
-                           total_rows, xrp, xsp, yrp, ysp, alpha);
+        const uint64_t gx = (c / VE + AXPY_BLOCK - 1) / AXPY_BLOCK;
+        if (gx > 0x7fffffffull) return WK_E_INVALID_VALUE;
+        const uint64_t gy = r < 65535 ? r : 65535, gz = d < 65535 ? d : 65535;
+        hipLaunchKernelGGL((axpy_rows_kernel<T, MODE>), dim3((unsigned)gx, (unsigned)gy, (unsigned)gz), dim3(AXPY_BLOCK), 0, s->stream, x, y, r,
+                           c, d, xrp, xsp, yrp, ysp, alpha);
         return launch_status();
     }
     const uint64_t want = (n + PITCHED_BLOCK - 1) / PITCHED_BLOCK;

@@ -5,7 +5,10 @@
 
 #include <cstdio>
 #include <cstring>
+#include <cstdlib>
+#include <mutex>
 #include <new>
+#include <unordered_map>
 
 using namespace wk;
 
@@ -184,11 +187,42 @@ int wk_event_elapsed_ms(wk_event *start, wk_event *stop, float *out_ms) {
     return WK_OK;
 }
 
+// Allocation colouring.  Two streams that a kernel walks in step (x and y of AXPY) run 1.5-2.5 % faster
+// on MI355X when their base addresses differ by an odd number of KiB from 3 KiB up than when they
+// share their offset inside a 4 KiB block, which is what two fresh hipMalloc blocks do (measured on
+// AXPY, n = 2^28 f32, over 24 base separations: same offset 6.49-6.81 TB/s, mean 6.71; +3 KiB
+// 6.78-6.85, mean 6.82; +5 / +7 KiB the same; +2 KiB no gain; +4 KiB worse).  Successive large
+// allocations therefore start 0, 3, 6, 9 KiB into their block, which makes every pair of neighbours
+// in allocation order differ by +3 KiB or -9 KiB.  WK_ALLOC_COLOURS=0 in the environment turns it off.
+namespace {
+constexpr size_t COLOUR_MIN_BYTES = size_t(1) << 20, COLOUR_STEP = 3072;
+std::mutex g_colour_mutex;
+std::unordered_map<void *, void *> g_coloured; // pointer handed out -> block to free
+unsigned g_next_colour = 0;
+bool colouring_enabled() {
+    static const bool on = [] {
+        const char *v = std::getenv("WK_ALLOC_COLOURS");
+        return !(v && v[0] == '0');
+    }();
+    return on;
+}
+} // namespace
+
 int wk_malloc(wk_device *dev, size_t bytes, void **out_dptr) {
     if (!dev || !out_dptr || bytes == 0) return WK_E_INVALID_VALUE;
     *out_dptr = nullptr;
     WK_HIP_TRY(hipSetDevice(dev->ordinal));
-    WK_HIP_TRY(hipMalloc(out_dptr, bytes));
+    if (bytes < COLOUR_MIN_BYTES || !colouring_enabled()) {
+        WK_HIP_TRY(hipMalloc(out_dptr, bytes));
+        return WK_OK;
+    }
+    std::lock_guard<std::mutex> lock(g_colour_mutex);
+    const size_t colour = (g_next_colour & 3u) * COLOUR_STEP;
+    void *block = nullptr;
+    WK_HIP_TRY(hipMalloc(&block, bytes + colour));
+    ++g_next_colour;
+    *out_dptr = static_cast<char *>(block) + colour;
+    if (colour) g_coloured.emplace(*out_dptr, block);
     return WK_OK;
 }
 
@@ -196,6 +230,14 @@ int wk_free(wk_device *dev, void *dptr) {
     if (!dev) return WK_E_INVALID_VALUE;
     if (!dptr) return WK_OK;
     WK_HIP_TRY(hipSetDevice(dev->ordinal));
+    {
+        std::lock_guard<std::mutex> lock(g_colour_mutex);
+        auto it = g_coloured.find(dptr);
+        if (it != g_coloured.end()) {
+            dptr = it->second;
+            g_coloured.erase(it);
+        }
+    }
     WK_HIP_TRY(hipFree(dptr));
     return WK_OK;
 }
