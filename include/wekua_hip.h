@@ -156,10 +156,14 @@ int  wk_axpy(wk_stream *s, int dtype, const uint64_t shape3[3],
  *     beta set              -> C = (alpha or 1)*op(A)op(B) + beta*C_old; C_old is read and
  *                              multiplied even when beta == 0 (NaN/Inf propagate).
  *   Integers wrap modulo 2^width; f32/f64 accumulate in their own precision.
- *   The reference's PackedTensors pass (gemm.zig:60-359) has no counterpart: tiles are
- *   staged through LDS straight from the row-major operands.
- *   workspace may be NULL when wk_gemm_workspace_bytes() returns 0 (it currently
- *   always does); it is reserved for split-K variants. */
+ *   The reference's PackedTensors pass (gemm.zig:60-359, 705-720: pack A and B into two scratch
+ *   tensors before every product) survives for i32 / u32 only: with `workspace` of at least
+ *   wk_gemm_workspace_bytes() bytes of device memory (16-byte aligned; what blas.PackedTensors
+ *   holds) large products first pack both operands into signed-digit planes there and then run a
+ *   leaner matrix-core kernel; the result is the same bits either way.  Every other type stages
+ *   its tiles through LDS straight from the row-major operands, asks for 0 bytes and ignores the
+ *   workspace, which may always be NULL.  The workspace is overwritten by every call that uses it:
+ *   calls sharing one must be ordered on one stream. */
 int    wk_gemm(wk_stream *s, int dtype, int op_a, int op_b, uint64_t M, uint64_t N, uint64_t K,
                const void *host_alpha, const void *A, uint64_t lda, const void *B, uint64_t ldb,
                const void *host_beta, void *C, uint64_t ldc, void *workspace, size_t workspace_bytes);
@@ -169,6 +173,10 @@ size_t wk_gemm_workspace_bytes(int dtype, int op_a, int op_b, uint64_t M, uint64
  * "tile64", ...).  For benchmarks and profiles; not part of the reference's surface. */
 const char *wk_gemm_variant(int dtype, int op_a, int op_b, uint64_t M, uint64_t N, uint64_t K,
                             uint64_t lda, uint64_t ldb, uint64_t ldc, const void *A, const void *B, const void *C);
+/* The same for a call that brings workspace_bytes bytes of workspace ("mfma_i32_packed", ...). */
+const char *wk_gemm_variant_with_workspace(int dtype, int op_a, int op_b, uint64_t M, uint64_t N, uint64_t K,
+                                           uint64_t lda, uint64_t ldb, uint64_t ldc, const void *A, const void *B,
+                                           const void *C, size_t workspace_bytes);
 
 /* Test/benchmark knob: force a gemm variant by name ("auto" restores selection).
  * Returns WK_E_INVALID_VALUE for an unknown name. */

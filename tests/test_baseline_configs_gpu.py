@@ -165,3 +165,46 @@ def test_config4_int32_overflow_forcing(dev):
     assert np.array_equal(got, want)
     # the C restatement of the reference's kernels wraps identically
     assert np.array_equal(oracle.gemm("i32", 65537, a, 0, b, 0, -3, c), want)
+
+
+@pytest.mark.parametrize("op_a,op_b", OPS)
+def test_config4_int32_large_with_packed_tensors(op_a, op_b):
+    """The int32 product the way benchmark/gemm.zig drives it: through blas.gemm with a
+    GemmPackedTensors, at a size where the library takes its pack pass + packed kernel."""
+    import wekua_amd as wk
+    from wekua_amd import raw
+    M, N, K = 4096, 4096, 2048
+    a = synth.integers(synth.config_seed(4, 6), (K, M) if op_a else (M, K), np.int32, -100, 100)
+    b = synth.integers(synth.config_seed(4, 7), (N, K) if op_b else (K, N), np.int32, -100, 100)
+    c = synth.integers(synth.config_seed(4, 8), (M, N), np.int32, -100, 100)
+    want = _exact_int32(3, a.T if op_a else a, b.T if op_b else b, -2, c)
+    context = wk.Context.initFromDeviceType(wk.DeviceType.all)
+    pipeline = wk.Pipeline.init(context.command_queues[0])
+    try:
+        tensors = []
+        for host in (a, b, c):
+            t = wk.Tensor.alloc("i32", context, pipeline, host.shape)
+            wk.memory.readFromBuffer(pipeline, t, host)
+            tensors.append(t)
+        A, B, C = tensors
+        packed = wk.GemmPackedTensors.init(pipeline, C, K, True)
+        assert packed.workspace_bytes > 0
+        name = wk._capi.load().wk_gemm_variant_with_workspace(raw.dtype_id("i32"), op_a, op_b, M, N, K, A.row_pitch, B.row_pitch,
+                                                        C.row_pitch, A.buffer, B.buffer, C.buffer, packed.workspace_bytes)
+        assert name == b"mfma_i32_packed"
+        wk.blas.gemm(pipeline, 3, A, op_a, B, op_b, -2, C, packed)
+        got = np.empty((M, N), dtype=np.int32)
+        wk.memory.writeToBuffer(pipeline, C, got)
+        pipeline.waitAndCleanup()
+        assert np.array_equal(got, want)
+        # second call on the same handle (the workspace is reused) from the new C
+        wk.blas.gemm(pipeline, None, A, op_a, B, op_b, None, C, packed)
+        wk.memory.writeToBuffer(pipeline, C, got)
+        pipeline.waitAndCleanup()
+        assert np.array_equal(got, _exact_int32(None, a.T if op_a else a, b.T if op_b else b, None, c))
+        packed.deinit(pipeline)
+        for t in tensors:
+            t.release(pipeline)
+    finally:
+        pipeline.deinit()
+        context.deinit()

@@ -12,8 +12,9 @@ pytestmark = pytest.mark.gpu
 OPS = list(itertools.product((0, 1), (0, 1)))
 
 
-def run_gemm(dev, dtype, alpha, a, op_a, b, op_b, beta, c, lda=None, ldb=None, ldc=None):
-    """Uploads dense operands (optionally re-pitched), runs wk_gemm, returns C as dense numpy."""
+def run_gemm(dev, dtype, alpha, a, op_a, b, op_b, beta, c, lda=None, ldb=None, ldc=None, packed=False):
+    """Uploads dense operands (optionally re-pitched), runs wk_gemm, returns C as dense numpy.
+    packed: bring the workspace wk_gemm_workspace_bytes asks for (poisoned first)."""
     cx = oracle.is_complex(dtype)
 
     def dims(m):
@@ -34,10 +35,16 @@ def run_gemm(dev, dtype, alpha, a, op_a, b, op_b, beta, c, lda=None, ldb=None, l
     bp, ldb = pitched(b, ldb)
     cp, ldc = pitched(c, ldc)
     dA, dB, dC = dev.upload(ap), dev.upload(bp), dev.upload(cp)
-    dev.gemm(dtype, op_a, op_b, M, N, K, alpha, dA, lda, dB, ldb, beta, dC, ldc)
+    ws = None
+    if packed:
+        from wekua_amd import raw
+        need = dev.lib.wk_gemm_workspace_bytes(raw.dtype_id(dtype), op_a, op_b, M, N, K)
+        assert need > 0
+        ws = dev.upload(np.full(need, 0x5a, dtype=np.uint8))
+    dev.gemm(dtype, op_a, op_b, M, N, K, alpha, dA, lda, dB, ldb, beta, dC, ldc, workspace=ws)
     dev.sync()
     out = dC.download(cp.dtype, cp.shape)
-    for d in (dA, dB, dC):
+    for d in (dA, dB, dC) + ((ws,) if ws is not None else ()):
         d.free()
     if out.shape[1] != N:
         gaps = out[:, N:]
@@ -46,9 +53,9 @@ def run_gemm(dev, dtype, alpha, a, op_a, b, op_b, beta, c, lda=None, ldb=None, l
     return out
 
 
-def check(dev, dtype, M, N, K, op_a, op_b, alpha, beta, seed=1, int_range=None, **ld):
+def check(dev, dtype, M, N, K, op_a, op_b, alpha, beta, seed=1, int_range=None, **kw):
     a, b, c = gemm_operands(dtype, M, N, K, op_a, op_b, seed, int_range)
-    got = run_gemm(dev, dtype, alpha, a, op_a, b, op_b, beta, c, **ld)
+    got = run_gemm(dev, dtype, alpha, a, op_a, b, op_b, beta, c, **kw)
     if M * N * K <= 64 ** 3 * 8:
         want = oracle.semantic_gemm(dtype, alpha, a, op_a, b, op_b, beta, c)
     else:
@@ -102,20 +109,45 @@ def test_integer_wraparound_bit_exact(dev, dtype, op_a, op_b):
 
 
 @pytest.mark.parametrize("dtype", ["i32", "u32"])
-@pytest.mark.parametrize("variant", ["tile64", "mfma_{}_64x128", "mfma_{}_128x128"])
+@pytest.mark.parametrize("variant", ["tile64", "mfma_{}_64x128", "mfma_{}_128x128", "mfma_{}_packed"])
 @pytest.mark.parametrize("op_a,op_b", OPS)
 def test_int32_every_variant_bit_exact(dev, dtype, variant, op_a, op_b):
-    """The int8-matrix-core decomposition and the vector-ALU kernel against the exact product modulo
-    2^32 on full-range entries: interior shapes (aligned), ragged shapes, K not a multiple of the slab,
-    every alpha / beta combination."""
+    """The int8-matrix-core decomposition (fused and with the pack pass) and the vector-ALU kernel
+    against the exact product modulo 2^32 on full-range entries: interior shapes (aligned), ragged
+    shapes, K not a multiple of the slab, every alpha / beta combination."""
     variant = variant.format(dtype)
+    packed = variant.endswith("packed")
     assert dev.lib.wk_gemm_force_variant(variant.encode()) == 0
     try:
         for (M, N, K) in [(64, 128, 32), (128, 256, 64), (192, 128, 416), (1, 1, 1), (65, 129, 33), (200, 300, 77), (63, 127, 500)]:
             for alpha, beta in [(None, None), (3, None), (-5 if dtype == "i32" else 4000000000, 7), (None, 1)]:
-                check(dev, dtype, M, N, K, op_a, op_b, alpha, beta, seed=23)
+                check(dev, dtype, M, N, K, op_a, op_b, alpha, beta, seed=23, packed=packed)
+        if packed:   # unaligned leading dimensions take the element-wise reader of the pack pass
+            check(dev, dtype, 130, 70, 200, op_a, op_b, 3, 7, seed=24, packed=True,
+                  lda=(130 if op_a else 200) + 3, ldb=(200 if op_b else 70) + 5, ldc=70 + 7)
     finally:
         dev.lib.wk_gemm_force_variant(b"auto")
+
+
+def test_int32_packed_needs_its_workspace(dev):
+    """Forced packed variant without a workspace (or with one that is too small) is an error, not a
+    silent fall-back; with automatic choice a missing workspace just means the fused kernel."""
+    from wekua_amd import raw
+    a, b, c = gemm_operands("i32", 128, 128, 64, 0, 0, 3)
+    dA, dB, dC = dev.upload(a), dev.upload(b), dev.upload(c)
+    small = dev.malloc(1024)
+    assert dev.lib.wk_gemm_force_variant(b"mfma_i32_packed") == 0
+    try:
+        lib, p = dev.lib, (dA.ptr, dB.ptr, dC.ptr)
+        assert lib.wk_gemm(dev.stream, raw.dtype_id("i32"), 0, 0, 128, 128, 64, None, p[0], 64, p[1], 128, None, p[2], 128, None, 0) == 1
+        assert lib.wk_gemm(dev.stream, raw.dtype_id("i32"), 0, 0, 128, 128, 64, None, p[0], 64, p[1], 128, None, p[2], 128, small.ptr, 1024) == 1
+    finally:
+        dev.lib.wk_gemm_force_variant(b"auto")
+    dev.gemm("i32", 0, 0, 128, 128, 64, None, dA, 64, dB, 128, None, dC, 128)
+    assert np.array_equal(dC.download(np.int32, (128, 128)), oracle.semantic_gemm("i32", None, a, 0, b, 0, None, c))
+    assert dev.lib.wk_gemm_workspace_bytes(raw.dtype_id("f32"), 0, 0, 128, 128, 64) == 0
+    for d in (dA, dB, dC, small):
+        d.free()
 
 
 def test_int32_matrix_core_extremes(dev):
@@ -138,6 +170,27 @@ def test_int32_matrix_core_extremes(dev):
     assert np.array_equal(got, want)
     for d in (dA, dB, dC):
         d.free()
+    assert dev.lib.wk_gemm_force_variant(b"mfma_i32_packed") == 0
+    try:
+        assert np.array_equal(run_gemm(dev, "i32", -3, a, 0, b, 0, 5, c, packed=True), want)
+    finally:
+        dev.lib.wk_gemm_force_variant(b"auto")
+
+
+@pytest.mark.parametrize("op_a,op_b", OPS)
+def test_int32_with_workspace_mid_size(dev, op_a, op_b):
+    """Mid-size ragged problem with and without a workspace under the automatic choice (which takes
+    the packed path only for much larger products) and with the packed path forced: all bit-exact."""
+    M, N, K = 768, 896, 300
+    a, b, c = gemm_operands("u32", M, N, K, op_a, op_b, 5)
+    want = oracle.gemm("u32", 7, a, op_a, b, op_b, 3, c)
+    assert np.array_equal(run_gemm(dev, "u32", 7, a, op_a, b, op_b, 3, c, packed=True), want)
+    assert np.array_equal(run_gemm(dev, "u32", 7, a, op_a, b, op_b, 3, c), want)
+    assert dev.lib.wk_gemm_force_variant(b"mfma_u32_packed") == 0
+    try:
+        assert np.array_equal(run_gemm(dev, "u32", 7, a, op_a, b, op_b, 3, c, packed=True), want)
+    finally:
+        dev.lib.wk_gemm_force_variant(b"auto")
 
 
 @pytest.mark.parametrize("dtype", ["cf32", "cf64", "ci32", "cu16", "ci8", "ci64"])

@@ -79,6 +79,7 @@ HOST_SIGNATURES = {
     "wkz_packed_init": (ci, [vp, vp, u64, ci, ctypes.POINTER(vp)]),
     "wkz_packed_init_with_dimensions": (ci, [vp, ci, u64, u64, u64, ci, ci, ctypes.POINTER(vp)]),
     "wkz_packed_deinit": (ci, [vp, vp]),
+    "wkz_packed_workspace_bytes": (ci, [vp, u64p]),
     "wkz_packed_pack": (ci, [vp, vp, vp, ci, vp, ci]),
     "wkz_gemm": (ci, [vp, vp, vp, ci, vp, ci, vp, vp, vp]),
     # tensor support operations
@@ -403,11 +404,18 @@ class convertions:
 
 
 class GemmPackedTensors:
-    """blas.GemmPackedTensors (src/blas/gemm.zig:60-359).  Holds no device memory here."""
+    """blas.GemmPackedTensors (src/blas/gemm.zig:60-359).  Holds device memory only for i32 / u32:
+    the workspace of the library's pack pass (`workspace_bytes`)."""
 
     def __init__(self, handle, dtype):
         self._h = handle
         self.dtype = dtype
+
+    @property
+    def workspace_bytes(self) -> int:
+        n = u64()
+        _check(_lib().wkz_packed_workspace_bytes(self._h, ctypes.byref(n)), "GemmPackedTensors.workspace_bytes")
+        return n.value
 
     @classmethod
     def init(cls, pipeline: Pipeline, result_tensor: Tensor, k_size: int, vectors_enabled: bool) -> "GemmPackedTensors":

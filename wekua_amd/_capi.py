@@ -64,6 +64,7 @@ SIGNATURES = {
     "wk_gemm": (ci, [vp, ci, ci, ci, u64, u64, u64, vp, vp, u64, vp, u64, vp, vp, u64, vp, sz]),
     "wk_gemm_workspace_bytes": (sz, [ci, ci, ci, u64, u64, u64]),
     "wk_gemm_variant": (ctypes.c_char_p, [ci, ci, ci, u64, u64, u64, u64, u64, u64, vp, vp, vp]),
+    "wk_gemm_variant_with_workspace": (ctypes.c_char_p, [ci, ci, ci, u64, u64, u64, u64, u64, u64, vp, vp, vp, sz]),
     "wk_gemm_force_variant": (ci, [ctypes.c_char_p]),
     "wk_copy_kernel": (ci, [vp, vp, vp, sz]),
     "wk_hadamard": (ci, [vp, ci, u64p, vp, u64, u64, vp, u64, u64]),

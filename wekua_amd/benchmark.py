@@ -88,10 +88,14 @@ def time_gemm(ses, dtype, M, N, K, op_a, op_b, alpha, beta, iters=10):
     A = ses.tensor(dtype, _operand(rd, (K, M) if op_a else (M, K), 1))
     B = ses.tensor(dtype, _operand(rd, (N, K) if op_b else (K, N), 2))
     C = ses.tensor(dtype, _operand(rd, (M, N), 3))
+    # as benchmark/gemm.zig:186-196 does: one GemmPackedTensors for the run, passed to every call
+    packed = wk.GemmPackedTensors.init(ses.pipeline, C, K, True)
     ses.pipeline.waitAndCleanup()
-    ms = ses.time_ms(lambda: wk.blas.gemm(ses.pipeline, alpha, A, op_a, B, op_b, beta, C, None), iters)
-    variant = ses.lib.wk_gemm_variant(raw.dtype_id(dtype), op_a, op_b, M, N, K, A.row_pitch, B.row_pitch, C.row_pitch,
-                                      A.buffer, B.buffer, C.buffer).decode()
+    ms = ses.time_ms(lambda: wk.blas.gemm(ses.pipeline, alpha, A, op_a, B, op_b, beta, C, packed), iters)
+    variant = ses.lib.wk_gemm_variant_with_workspace(raw.dtype_id(dtype), op_a, op_b, M, N, K, A.row_pitch, B.row_pitch,
+                                                     C.row_pitch, A.buffer, B.buffer, C.buffer,
+                                                     packed.workspace_bytes).decode()
+    packed.deinit(ses.pipeline)
     for t in (A, B, C):
         t.release(ses.pipeline)
     return ms, variant

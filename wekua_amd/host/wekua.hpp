@@ -26,8 +26,9 @@
 //   * Tensor rows are padded to 16 bytes (the per-lane load width of gfx950), not to an
 //     even vector count, row counts are not padded at all, and row pitches that are a
 //     multiple of 1 KiB and at least 16 KiB are skewed by 512 bytes to avoid channel aliasing;
-//   * PackedTensors allocates nothing: the HIP kernels tile straight from the row-major
-//     operands through LDS, so pack() only validates.
+//   * PackedTensors holds device memory only for i32 / u32 (the signed-digit planes of the
+//     int8 matrix-core product, filled by a pack pass inside gemm); for every other type the
+//     HIP kernels tile straight from the row-major operands through LDS and pack() only validates.
 #pragma once
 
 #include <algorithm>
@@ -751,9 +752,13 @@ template <typename T> void axpy(Pipeline *pipeline, Tensor<T> *x, std::optional<
 // src/blas/gemm.zig:60-359.  n_size = rows of C, m_size = columns of C (the reference's naming).
 template <typename T> struct PackedTensors {
     uint64_t m_size = 0, n_size = 0, k_size = 0;
-    Tensor<T> *packed_a = nullptr, *packed_b = nullptr; // never allocated: no pack pass on this device
+    Tensor<T> *packed_a = nullptr, *packed_b = nullptr; // never allocated: the packed form is not a tensor here
     bool vectors_enabled = false;
     GemmAlgorithm algorithm = GemmAlgorithm::a2x2;
+    // device memory the library's gemm packs into (wk_gemm_workspace_bytes; zero bytes for most types)
+    wk_device *device = nullptr;
+    void *workspace = nullptr;
+    size_t workspace_bytes = 0;
 
     static PackedTensors *init(Pipeline *pipeline, Tensor<T> *result_tensor, uint64_t k_size, bool vectors_enabled) {
         const auto &shape = result_tensor->dimensions.shape;
@@ -764,7 +769,6 @@ template <typename T> struct PackedTensors {
     }
     static PackedTensors *initWithDimensions(Pipeline *pipeline, uint64_t n_size, uint64_t m_size, uint64_t k_size,
                                              GemmAlgorithm recommended_algorithm, bool vectors_enabled) {
-        (void)pipeline;
         if (!n_size || !m_size || !k_size) throw Error(WK_E_INVALID_VALUE);
         PackedTensors *p = new PackedTensors;
         p->n_size = n_size;
@@ -772,10 +776,20 @@ template <typename T> struct PackedTensors {
         p->k_size = k_size;
         p->vectors_enabled = !core::isComplex<T>() && vectors_enabled;
         p->algorithm = recommended_algorithm;
+        p->device = pipeline->command_queue->context->device;
+        p->workspace_bytes = wk_gemm_workspace_bytes(core::getTypeIndex<T>(), 0, 0, n_size, m_size, k_size);
+        if (p->workspace_bytes) {
+            const int rc = wk_malloc(p->device, p->workspace_bytes, &p->workspace);
+            if (rc) {
+                delete p;
+                throw Error(rc);
+            }
+        }
         return p;
     }
     void deinit(Pipeline *pipeline) {
         pipeline->waitAndCleanup(); // the reference's deinit releases two tensors, each draining the pipeline
+        if (workspace) wk_free(device, workspace);
         delete this;
     }
     // gemm.zig:250-270
@@ -788,7 +802,7 @@ template <typename T> struct PackedTensors {
                                                  : (bs[1] == k_size && bs[0] == m_size);
         if (!valid) throw Error(WK_E_INVALID_VALUE);
     }
-    // gemm.zig:272-357: validation only; nothing is re-tiled in memory
+    // gemm.zig:272-357: validation; the pack pass itself runs inside wk_gemm, on the workspace
     void pack(Pipeline *pipeline, Tensor<T> *a, Operation op_a, Tensor<T> *b, Operation op_b) {
         (void)pipeline;
         validateTensors(a, op_a, b, op_b);
@@ -823,7 +837,8 @@ void gemm(Pipeline *pipeline, std::optional<T> alpha, Tensor<T> *a, Operation op
     const T av = alpha.value_or(T{}), bv = beta.value_or(T{});
     check(wk_gemm(pipeline->command_queue->stream, core::getTypeIndex<T>(), (int)op_a, (int)op_b, M, N, K,
                   alpha ? &av : nullptr, a->buffer, a->memory_layout.row_pitch, b->buffer, b->memory_layout.row_pitch,
-                  beta ? &bv : nullptr, c->buffer, c->memory_layout.row_pitch, nullptr, 0));
+                  beta ? &bv : nullptr, c->buffer, c->memory_layout.row_pitch, packed_tensors ? packed_tensors->workspace : nullptr,
+                  packed_tensors ? packed_tensors->workspace_bytes : 0));
     pipeline->append(1);
 }
 

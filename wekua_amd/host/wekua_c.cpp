@@ -393,6 +393,13 @@ int wkz_packed_deinit(void *packed, void *pipeline) {
         delete h;
     });
 }
+// bytes of device memory the handle holds for the library's pack pass (0 for most types)
+int wkz_packed_workspace_bytes(void *packed, uint64_t *out) {
+    return guard([&] {
+        PackedHandle *h = static_cast<PackedHandle *>(packed);
+        dispatch(h->dtype, [&]<typename T>() { *out = static_cast<blas::PackedTensors<T> *>(h->packed)->workspace_bytes; });
+    });
+}
 int wkz_packed_pack(void *packed, void *pipeline, void *a, int op_a, void *b, int op_b) {
     return guard([&] {
         PackedHandle *h = static_cast<PackedHandle *>(packed);
