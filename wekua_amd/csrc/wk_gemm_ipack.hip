@@ -37,7 +37,7 @@ struct __attribute__((packed, aligned(4))) u32x4_u { u32x4 v; };
 
 constexpr uint32_t CBIAS = 0x80808080u;
 constexpr int TILE = 128, BK = 32, BLOCK_BYTES = 1024, GROUP_BYTES = 4 * BLOCK_BYTES; // 4 digits of one (32 rows, 32 k)
-constexpr int PACK_THREADS = 256, GEMM_THREADS = 512;
+constexpr int PACK_THREADS = 256;
 constexpr uint32_t MAX_KSPLIT = 16;
 
 struct Layout {
@@ -160,15 +160,28 @@ struct PArgs {
     uint32_t alpha, beta;
 };
 
-constexpr int STAGE_BYTES = 2 * (TILE / 32) * GROUP_BYTES; // A: 4 groups of 4 KiB, then B: 4 groups
+// BM x 128 tile, BM / 32 x 2 waves.  BM = 128 (one 8-wave work-group per CU) is what is launched.
+// BM = 64 -- two independent 4-wave work-groups per CU, so that the two waves of a SIMD are not held
+// in the same phase by one barrier -- was measured and is slower (8192^3: 207 against 222 TOP/s): it
+// copies half as much again per matrix instruction.
+template <int BM> struct PackedTile {
+    static constexpr int NT = BM * 4;                       // threads
+    static constexpr int GROUPS = BM / 32 + TILE / 32;      // 4 KiB groups per slab: A row blocks, then B column blocks
+    static constexpr int STAGE_BYTES = GROUPS * GROUP_BYTES;
+    static constexpr int GROUPS_PER_PASS = NT * 16 / GROUP_BYTES; // 1 or 2
+    static constexpr int PASSES = GROUPS / GROUPS_PER_PASS;
+    static constexpr size_t LDS_BYTES = 2 * STAGE_BYTES + (BM + TILE) * sizeof(uint32_t);
+};
 
-template <bool EDGE>
-__global__ __launch_bounds__(GEMM_THREADS) __attribute__((amdgpu_waves_per_eu(2)))
+template <int BM, bool EDGE>
+__global__ __launch_bounds__(BM * 4) __attribute__((amdgpu_waves_per_eu(2)))
 void gemm_i32_packed_kernel(PArgs g) {
+    using TL = PackedTile<BM>;
+    constexpr int STAGE_BYTES = TL::STAGE_BYTES, PASSES = TL::PASSES, A_GROUPS = BM / 32;
     extern __shared__ __align__(16) unsigned char lds_raw[];
     unsigned char *stages = lds_raw;                                              // [2][STAGE_BYTES]
-    uint32_t *row_sum = reinterpret_cast<uint32_t *>(lds_raw + 2 * STAGE_BYTES);  // [TILE]
-    uint32_t *col_sum = row_sum + TILE;                                           // [TILE]
+    uint32_t *row_sum = reinterpret_cast<uint32_t *>(lds_raw + 2 * STAGE_BYTES);  // [BM]
+    uint32_t *col_sum = row_sum + BM;                                             // [TILE]
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wm = wave >> 1, wn = wave & 1, l32 = lane & 31, lhi = lane >> 5;
@@ -179,11 +192,11 @@ void gemm_i32_packed_kernel(PArgs g) {
         tile_m = first_m + in_group % gsz;
         tile_n = in_group / gsz;
     }
-    const uint32_t m0 = tile_m * TILE, n0 = tile_n * TILE;
+    const uint32_t m0 = tile_m * BM, n0 = tile_n * TILE;
 
-    if (tid < 2 * TILE) {
-        const uint32_t *src = tid < TILE ? g.sums_a + m0 + tid : g.sums_b + n0 + (tid - TILE);
-        const uint32_t stride = tid < TILE ? g.Mp : g.Np;
+    if (tid < BM + TILE) {
+        const uint32_t *src = tid < BM ? g.sums_a + m0 + tid : g.sums_b + n0 + (tid - BM);
+        const uint32_t stride = tid < BM ? g.Mp : g.Np;
         uint32_t s = 0;
         for (uint32_t i = 0; i < g.ksplit; ++i) s += src[(size_t)i * stride];
         row_sum[tid] = s; // col_sum follows row_sum
@@ -197,40 +210,40 @@ void gemm_i32_packed_kernel(PArgs g) {
 #pragma unroll
             for (int r = 0; r < 16; ++r) acc[s][b][r] = 0;
 
-    // Copy of one slab: 8 groups of 4 KiB; pass i moves groups 2i and 2i + 1 (threads 0..255 / 256..511).
-    // Each of the four group streams of this thread is a buffer resource (scalar registers) over the
-    // KB * 4 KiB of that group; a load is resource + scalar slab offset + the lane's fixed 32-bit
-    // offset, so the loop holds no vector address arithmetic (whose result registers the compiler
-    // would share with the load destinations, waiting for every load in flight first).
+    // Copy of one slab: GROUPS groups of 4 KiB; pass i moves group(s) i * GROUPS_PER_PASS (+ tid / 256).
+    // Each group stream of this thread is a buffer resource (scalar registers) over the KB * 4 KiB of
+    // that group; a load is resource + scalar slab offset + the lane's fixed 32-bit offset, so the
+    // loop holds no vector address arithmetic (whose result registers the compiler would share with
+    // the load destinations, waiting for every load in flight first).
     const int grp = __builtin_amdgcn_readfirstlane(tid >> 8);
     const int within = (tid & 255) * 16;
-    __amdgpu_buffer_rsrc_t src[4];
+    __amdgpu_buffer_rsrc_t src[PASSES];
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-        const int gi = 2 * i + grp; // 0..3: A row blocks, 4..7: B column blocks
-        const unsigned char *p = gi < 4 ? g.planes_a + (size_t)(tile_m * 4 + gi) * g.KB * GROUP_BYTES
-                                        : g.planes_b + (size_t)(tile_n * 4 + gi - 4) * g.KB * GROUP_BYTES;
+    for (int i = 0; i < PASSES; ++i) {
+        const int gi = TL::GROUPS_PER_PASS * i + grp; // < A_GROUPS: A row blocks, then B column blocks
+        const unsigned char *p = gi < A_GROUPS ? g.planes_a + (size_t)(tile_m * A_GROUPS + gi) * g.KB * GROUP_BYTES
+                                               : g.planes_b + (size_t)(tile_n * 4 + gi - A_GROUPS) * g.KB * GROUP_BYTES;
         src[i] = __builtin_amdgcn_make_buffer_rsrc(const_cast<unsigned char *>(p), 0, (int)(g.KB * GROUP_BYTES), 0x00020000);
     }
     // Two register sets: the slab loaded in step kb is stored to LDS at the end of step kb + 1 and
     // used in step kb + 2, so a load has two slabs of matrix work to arrive.
-    u32x4 staged[2][4];
     // (past the end the last slab is loaded again and dropped: no branch, so the loads stay where
     // they are written, ahead of the matrix work)
+    u32x4 staged[2][PASSES];
     auto gload = [&](u32x4 *dst, uint32_t kb) {
         const int off = (int)(min(kb, g.KB - 1) * GROUP_BYTES);
 #pragma unroll
-        for (int i = 0; i < 4; ++i) dst[i] = __builtin_amdgcn_raw_buffer_load_b128(src[i], within, off, 0);
+        for (int i = 0; i < PASSES; ++i) dst[i] = __builtin_amdgcn_raw_buffer_load_b128(src[i], within, off, 0);
         __builtin_amdgcn_sched_barrier(0);
     };
     auto sstore = [&](const u32x4 *from, int buf) {
 #pragma unroll
-        for (int i = 0; i < 4; ++i)
-            *reinterpret_cast<u32x4 *>(stages + buf * STAGE_BYTES + (2 * i + grp) * GROUP_BYTES + within) = from[i];
+        for (int i = 0; i < PASSES; ++i)
+            *reinterpret_cast<u32x4 *>(stages + buf * STAGE_BYTES + (TL::GROUPS_PER_PASS * i + grp) * GROUP_BYTES + within) = from[i];
     };
     auto compute = [&](int buf) {
         const unsigned char *sa = stages + buf * STAGE_BYTES + wm * GROUP_BYTES + lane * 16;
-        const unsigned char *sb = stages + buf * STAGE_BYTES + (4 + wn * 2) * GROUP_BYTES + lane * 16;
+        const unsigned char *sb = stages + buf * STAGE_BYTES + (A_GROUPS + wn * 2) * GROUP_BYTES + lane * 16;
         i32x4 a[4], b[2][4];
 #pragma unroll
         for (int d = 0; d < 4; ++d) {
@@ -294,13 +307,14 @@ void gemm_i32_packed_kernel(PArgs g) {
     }
 }
 
-template <bool EDGE> int launch_packed(hipStream_t st, const PArgs &g) {
-    constexpr size_t lds = 2 * STAGE_BYTES + 2 * TILE * sizeof(uint32_t);
-    auto kern = gemm_i32_packed_kernel<EDGE>;
+template <int BM, bool EDGE> int launch_packed(hipStream_t st, PArgs g) {
+    constexpr size_t lds = PackedTile<BM>::LDS_BYTES;
+    auto kern = gemm_i32_packed_kernel<BM, EDGE>;
     static const hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
                                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     if (attr != hipSuccess) { (void)hipGetLastError(); return hip_code(attr); }
-    hipLaunchKernelGGL(kern, dim3(g.tiles_m * g.tiles_n), dim3(GEMM_THREADS), lds, st, g);
+    g.tiles_m = g.Mp / BM;
+    hipLaunchKernelGGL(kern, dim3(g.tiles_m * g.tiles_n), dim3(PackedTile<BM>::NT), lds, st, g);
     return launch_status();
 }
 
@@ -349,5 +363,6 @@ int wk::gemm_i32_packed_launch(hipStream_t st, const GemmProblem &p, void *works
     g.epi = p.epi;
     std::memcpy(&g.alpha, p.alpha, 4);
     std::memcpy(&g.beta, p.beta, 4);
-    return p.M % TILE != 0 || p.N % TILE != 0 ? launch_packed<true>(st, g) : launch_packed<false>(st, g);
+    const bool edge = p.M % TILE != 0 || p.N % TILE != 0;
+    return edge ? launch_packed<128, true>(st, g) : launch_packed<128, false>(st, g);
 }
