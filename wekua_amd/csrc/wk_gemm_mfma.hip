@@ -244,8 +244,21 @@ void gemm_f32_mfma_kernel(MArgs<float> g) {
     // needs checks only on the slab that holds the k tail.  The choice is uniform over the work-group.
     const bool tile_inside = !EDGE || (m0 + BM <= g.M && n0 + BN <= g.N);
     const uint32_t k_inside = g.K - g.K % BK; // slabs starting below this are complete
-    auto load_ab = [&](uint32_t k0, f32x4 *ra, f32x4 *rb) {
-        if (!EDGE || (tile_inside && k0 < k_inside)) {
+    // An edge tile away from the k tail needs less than the full treatment: rows and columns beyond
+    // the matrix only feed entries of C that are never stored, so the clamped loads (which keep the
+    // addresses inside the operand and deliver copies of valid data) can go to LDS as they are.  The
+    // one exception is a vector that straddles the end of a row of storage, whose valid elements
+    // arrive shifted: that happens only when the contiguous extent is not a multiple of the vector.
+    const bool fix_a_always = !A_K && g.M % 4 != 0, fix_b_always = !B_K && g.N % 4 != 0;
+    // How a slab is treated is a compile-time flavour of the loop that handles it, so that the loops
+    // over complete slabs carry no trace of the checked paths:
+    //   PLAIN    the slab lies inside both operands (the only flavour of the unchecked instantiation)
+    //   CLAMPED  edge tile, complete slab: clamped loads, stored as they are unless a row end is straddled
+    //   ANY      decided per slab at run time (the iterations that touch the k tail)
+    enum { PLAIN = 0, CLAMPED = 1, ANY = 2 };
+    auto load_ab = [&](uint32_t k0, f32x4 *ra, f32x4 *rb, auto flavour_tag) {
+        constexpr int FL = decltype(flavour_tag)::value;
+        if (FL == PLAIN || (FL == ANY && tile_inside && k0 < k_inside)) {
             gload(ra, g.A, g.lda, m0, g.M, k0, integral_constant<bool, A_K>{}, integral_constant<int, BM>{},
                   integral_constant<int, A_V4>{}, std::false_type{});
             gload(rb, g.B, g.ldb, n0, g.N, k0, integral_constant<bool, B_K>{}, integral_constant<int, BN>{},
@@ -257,19 +270,24 @@ void gemm_f32_mfma_kernel(MArgs<float> g) {
                   integral_constant<int, B_V4>{}, std::true_type{});
         }
     };
-    auto store_ab = [&](int buf, uint32_t k0, const f32x4 *ra, const f32x4 *rb) {
-        if (!EDGE || (tile_inside && k0 < k_inside)) {
+    auto store_ab = [&](int buf, uint32_t k0, const f32x4 *ra, const f32x4 *rb, auto flavour_tag) {
+        constexpr int FL = decltype(flavour_tag)::value;
+        const bool complete = FL != ANY || k0 < k_inside;
+        const bool plain = FL == PLAIN || (FL == ANY && tile_inside && complete);
+        if (plain || (complete && !fix_a_always))
             sstore(As + buf * SA::SIZE, ra, m0, g.M, k0, integral_constant<bool, A_K>{}, integral_constant<int, BM>{},
                    integral_constant<int, A_V4>{}, std::false_type{});
-            sstore(Bs + buf * SB::SIZE, rb, n0, g.N, k0, integral_constant<bool, B_K>{}, integral_constant<int, BN>{},
-                   integral_constant<int, B_V4>{}, std::false_type{});
-        } else {
+        else
             sstore(As + buf * SA::SIZE, ra, m0, g.M, k0, integral_constant<bool, A_K>{}, integral_constant<int, BM>{},
                    integral_constant<int, A_V4>{}, std::true_type{});
+        if (plain || (complete && !fix_b_always))
+            sstore(Bs + buf * SB::SIZE, rb, n0, g.N, k0, integral_constant<bool, B_K>{}, integral_constant<int, BN>{},
+                   integral_constant<int, B_V4>{}, std::false_type{});
+        else
             sstore(Bs + buf * SB::SIZE, rb, n0, g.N, k0, integral_constant<bool, B_K>{}, integral_constant<int, BN>{},
                    integral_constant<int, B_V4>{}, std::true_type{});
-        }
     };
+    using AnyFlavour = integral_constant<int, EDGE ? ANY : PLAIN>;
 
     const uint32_t ktiles = (g.K + BK - 1) / BK;
     constexpr int S = BK / 8; // fragment steps per k-slab (8 values of k each)
@@ -298,9 +316,9 @@ void gemm_f32_mfma_kernel(MArgs<float> g) {
         }
     };
 
-    load_ab(0, ra[0], rb[0]);
-    store_ab(0, 0, ra[0], rb[0]);
-    if (PF == 2 && ktiles > 1) load_ab(BK, ra[PF - 1], rb[PF - 1]);
+    load_ab(0, ra[0], rb[0], AnyFlavour{});
+    store_ab(0, 0, ra[0], rb[0], AnyFlavour{});
+    if (PF == 2 && ktiles > 1) load_ab(BK, ra[PF - 1], rb[PF - 1], AnyFlavour{});
     __syncthreads();
 
     // Fragment registers are double-buffered: the LDS reads for step s+1 are issued before the
@@ -322,7 +340,8 @@ void gemm_f32_mfma_kernel(MArgs<float> g) {
     //   LOOP 2  last slab peeled, hand-over fenced                  256x128: NN 133.4, NT 134.3, TN 131.1;
     //           (sched_barrier) so that matrix instructions         64x64 at 1024^3: 90.8 (LOOP 1: 88.7), 2048^3: 122.8 (115-120)
     //           are not hoisted above the barrier
-    constexpr int LOOP = (BM * BN <= 64 * 64) ? 2 : (BM * BN <= 128 * 128 ? 1 : ((A_K && !B_K) ? 0 : 2));
+    // (the bounds-checked instantiation always takes LOOP 2, whose iterations exist per flavour)
+    constexpr int LOOP = EDGE ? 2 : (BM * BN <= 64 * 64) ? 2 : (BM * BN <= 128 * 128 ? 1 : ((A_K && !B_K) ? 0 : 2));
     static_assert(LOOP == 2 || PF == 1, "only the peeled loop knows the two-set prefetch");
     f32x4 af[2][FM], bf[2][FN];
     read_frags(0, 0, af[0], bf[0]);
@@ -341,13 +360,13 @@ void gemm_f32_mfma_kernel(MArgs<float> g) {
         for (uint32_t kt = 0; kt < ktiles; ++kt) {
             const int cur = kt & 1;
             const bool more = kt + 1 < ktiles;
-            if (more) load_ab((kt + 1) * BK, ra[0], rb[0]);
+            if (more) load_ab((kt + 1) * BK, ra[0], rb[0], AnyFlavour{});
 #pragma unroll
             for (int s = 0; s < S; ++s) {
                 if (s + 1 < S) {
                     read_frags(cur, s + 1, af[(s + 1) & 1], bf[(s + 1) & 1]);
                 } else if (more) {
-                    store_ab(cur ^ 1, (kt + 1) * BK, ra[0], rb[0]);
+                    store_ab(cur ^ 1, (kt + 1) * BK, ra[0], rb[0], AnyFlavour{});
                     __syncthreads();
                     read_frags(cur ^ 1, 0, af[(s + 1) & 1], bf[(s + 1) & 1]);
                 }
@@ -364,13 +383,13 @@ void gemm_f32_mfma_kernel(MArgs<float> g) {
         auto iteration = [&](uint32_t kt) {
             const int cur = kt & 1;
             const bool more = kt + 1 < ktiles;
-            if (more) load_ab((kt + 1) * BK, ra[0], rb[0]);
+            if (more) load_ab((kt + 1) * BK, ra[0], rb[0], AnyFlavour{});
 #pragma unroll
             for (int s = 0; s < S; ++s) {
                 if (s + 1 < S) {
                     read_frags(cur, s + 1, af[(s + 1) & 1], bf[(s + 1) & 1]);
                 } else if (more) {
-                    store_ab(cur ^ 1, (kt + 1) * BK, ra[0], rb[0]);
+                    store_ab(cur ^ 1, (kt + 1) * BK, ra[0], rb[0], AnyFlavour{});
                     __syncthreads();
                     read_frags(cur ^ 1, 0, af[(s + 1) & 1], bf[(s + 1) & 1]);
                 }
@@ -381,13 +400,13 @@ void gemm_f32_mfma_kernel(MArgs<float> g) {
     } else {
         // one iteration that hands over to slab kt+1; P = parity of kt, a compile-time constant so
         // that the staging sets stay in registers
-        auto iteration = [&](uint32_t kt, auto parity_tag) {
+        auto iteration = [&](uint32_t kt, auto parity_tag, auto flavour_tag) __attribute__((always_inline)) {
             constexpr int P = decltype(parity_tag)::value;
             const int cur = kt & 1;
             if constexpr (PF == 1) {
-                load_ab((kt + 1) * BK, ra[0], rb[0]);
+                load_ab((kt + 1) * BK, ra[0], rb[0], flavour_tag);
             } else {
-                if (kt + 2 < ktiles) load_ab((kt + 2) * BK, ra[P], rb[P]); // set P held slab kt, already in LDS
+                if (kt + 2 < ktiles) load_ab((kt + 2) * BK, ra[P], rb[P], flavour_tag); // set P held slab kt, already in LDS
             }
             constexpr int NEXT = PF == 1 ? 0 : 1 - P; // the set holding slab kt+1
 #pragma unroll
@@ -396,7 +415,7 @@ void gemm_f32_mfma_kernel(MArgs<float> g) {
                     read_frags(cur, s + 1, af[(s + 1) & 1], bf[(s + 1) & 1]);
                 } else {
                     __builtin_amdgcn_sched_barrier(0);
-                    store_ab(cur ^ 1, (kt + 1) * BK, ra[NEXT], rb[NEXT]);
+                    store_ab(cur ^ 1, (kt + 1) * BK, ra[NEXT], rb[NEXT], flavour_tag);
                     __syncthreads();
                     read_frags(cur ^ 1, 0, af[(s + 1) & 1], bf[(s + 1) & 1]);
                     __builtin_amdgcn_sched_barrier(0);
@@ -404,18 +423,48 @@ void gemm_f32_mfma_kernel(MArgs<float> g) {
                 mfma_step(s);
             }
         };
+        // iterations kt .. end-1 in one flavour; with two staging sets the set index is the parity of kt
+        auto run = [&](uint32_t &kt, uint32_t end, auto flavour_tag) __attribute__((always_inline)) {
+            if constexpr (PF == 1) {
+                for (; kt < end; ++kt) iteration(kt, integral_constant<int, 0>{}, flavour_tag);
+            } else {
+                if ((kt & 1) && kt < end) {
+                    iteration(kt, integral_constant<int, 1>{}, flavour_tag);
+                    ++kt;
+                }
+                for (; kt + 1 < end; kt += 2) {
+                    iteration(kt, integral_constant<int, 0>{}, flavour_tag);
+                    iteration(kt + 1, integral_constant<int, 1>{}, flavour_tag);
+                }
+                if (kt < end) {
+                    iteration(kt, integral_constant<int, 0>{}, flavour_tag);
+                    ++kt;
+                }
+            }
+        };
         uint32_t kt = 0;
-        if constexpr (PF == 1) {
-            for (; kt + 1 < ktiles; ++kt) iteration(kt, integral_constant<int, 0>{});
+        if constexpr (!EDGE) {
+            if constexpr (PF == 1) {
+                for (; kt + 1 < ktiles; ++kt) iteration(kt, integral_constant<int, 0>{}, AnyFlavour{});
+            } else {
+                for (; kt + 2 < ktiles; kt += 2) {
+                    iteration(kt, integral_constant<int, 0>{}, AnyFlavour{});
+                    iteration(kt + 1, integral_constant<int, 1>{}, AnyFlavour{});
+                }
+                if (kt + 1 < ktiles) {
+                    iteration(kt, integral_constant<int, 0>{}, AnyFlavour{});
+                    ++kt;
+                }
+            }
         } else {
-            for (; kt + 2 < ktiles; kt += 2) {
-                iteration(kt, integral_constant<int, 0>{});
-                iteration(kt + 1, integral_constant<int, 1>{});
-            }
-            if (kt + 1 < ktiles) {
-                iteration(kt, integral_constant<int, 0>{});
-                ++kt;
-            }
+            // Iteration kt stores slab kt + 1 and requests slab kt + PF: the iterations before
+            // `main_end` touch complete slabs only and run in a flavour fixed for the tile.
+            const bool has_tail = g.K % BK != 0;
+            const uint32_t hand_overs = ktiles - 1;
+            const uint32_t main_end = has_tail ? (hand_overs > (uint32_t)PF ? hand_overs - PF : 0u) : hand_overs;
+            if (tile_inside) run(kt, main_end, integral_constant<int, PLAIN>{});
+            else run(kt, main_end, integral_constant<int, CLAMPED>{});
+            run(kt, hand_overs, integral_constant<int, ANY>{});
         }
         {   // last slab: nothing to hand over
             const int cur = kt & 1;
