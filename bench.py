@@ -190,6 +190,23 @@ def main():
                "ms_per_step": m["stream_ms"], "wall_ms_per_step": m["wall_ms"], "gemm_flops_per_step": m["flops"],
                "value": m["tflops"], "unit": "TFLOP/s", "frac_of_f32_matrix_peak": m["tflops"] / F32_MATRIX_PEAK_TFLOPS}
 
+    other = None
+    if not args.no_mlp:   # the remaining benchmark configurations, a few launches each
+        from wekua_amd import benchmark
+        ses = benchmark.Session()
+        try:
+            other = {}
+            for key, dtype, (M, N, K), alpha, beta, unit in (("f64_gemm_4096", "f64", (4096, 4096, 4096), 1.0, 1.0, "TFLOP/s"),
+                                                             ("f64_gemm_8192x256x8192", "f64", (8192, 256, 8192), 1.0, 1.0, "TFLOP/s"),
+                                                             ("i32_gemm_2048", "i32", (2048, 2048, 2048), 3, -2, "TOP/s"),
+                                                             ("f32_gemm_1000", "f32", (1000, 1000, 1000), 1.5, 0.5, "TFLOP/s"),
+                                                             ("f32_gemm_4097x4095x4093", "f32", (4097, 4095, 4093), 1.5, 0.5, "TFLOP/s")):
+                ms, variant = benchmark.time_gemm(ses, dtype, M, N, K, 0, 0, alpha, beta)
+                other[key] = {"ms": ms, "value": 2.0 * M * N * K / ms / 1e9, "unit": unit, "kernel": variant}
+                log(f"[bench] {key}: {ms:.4f} ms -> {other[key]['value']:.1f} {unit} [{variant}]")
+        finally:
+            ses.close()
+
     cpu = None
     if not args.no_cpu_baseline:
         cores = min(os.cpu_count() or 1, int(os.environ.get("OMP_NUM_THREADS", "16") or 16), 16)
@@ -223,6 +240,7 @@ def main():
                               "bytes_per_launch": ax["bytes"]},
                  "f64": {"value": ax64["gbs"], "us_per_call": ax64["us"], "frac": ax64["gbs"] / HBM_PEAK_GBS}},
         "mlp_step": mlp,
+        "configs": other,
         "cpu_baseline": cpu,
     }
     print(json.dumps(out), flush=True)
