@@ -636,8 +636,13 @@ void gemm_f64_mfma_kernel(MArgs<double> g) {
     // interior tiles of the bounds-checked instantiation check only the slab with the k tail
     const bool tile_inside = !EDGE || (m0 + BM <= g.M && n0 + BN <= g.N);
     const uint32_t k_inside = g.K - g.K % BK;
-    auto load_ab = [&](uint32_t k0, f64x2 *ra, f64x2 *rb) {
-        if (!EDGE || (tile_inside && k0 < k_inside)) {
+    // slab flavours as in the f32 kernel: PLAIN inside both operands, CLAMPED for complete slabs of an
+    // edge tile (stored as loaded unless a 2-element vector straddles a row end), ANY decided per slab
+    const bool fix_a_always = !A_K && g.M % 2 != 0, fix_b_always = !B_K && g.N % 2 != 0;
+    enum { PLAIN = 0, CLAMPED = 1, ANY = 2 };
+    auto load_ab = [&](uint32_t k0, f64x2 *ra, f64x2 *rb, auto flavour_tag) {
+        constexpr int FL = decltype(flavour_tag)::value;
+        if (FL == PLAIN || (FL == ANY && tile_inside && k0 < k_inside)) {
             gload(ra, g.A, g.lda, m0, g.M, k0, integral_constant<bool, A_K>{}, integral_constant<int, BM>{},
                   integral_constant<int, A_V2>{}, std::false_type{});
             gload(rb, g.B, g.ldb, n0, g.N, k0, integral_constant<bool, B_K>{}, integral_constant<int, BN>{},
@@ -649,19 +654,24 @@ void gemm_f64_mfma_kernel(MArgs<double> g) {
                   integral_constant<int, B_V2>{}, std::true_type{});
         }
     };
-    auto store_ab = [&](int buf, uint32_t k0, const f64x2 *ra, const f64x2 *rb) {
-        if (!EDGE || (tile_inside && k0 < k_inside)) {
+    auto store_ab = [&](int buf, uint32_t k0, const f64x2 *ra, const f64x2 *rb, auto flavour_tag) {
+        constexpr int FL = decltype(flavour_tag)::value;
+        const bool complete = FL != ANY || k0 < k_inside;
+        const bool plain = FL == PLAIN || (FL == ANY && tile_inside && complete);
+        if (plain || (complete && !fix_a_always))
             sstore(As + buf * SA::SIZE, ra, m0, g.M, k0, integral_constant<bool, A_K>{}, integral_constant<int, BM>{},
                    integral_constant<int, A_V2>{}, std::false_type{});
-            sstore(Bs + buf * SB::SIZE, rb, n0, g.N, k0, integral_constant<bool, B_K>{}, integral_constant<int, BN>{},
-                   integral_constant<int, B_V2>{}, std::false_type{});
-        } else {
+        else
             sstore(As + buf * SA::SIZE, ra, m0, g.M, k0, integral_constant<bool, A_K>{}, integral_constant<int, BM>{},
                    integral_constant<int, A_V2>{}, std::true_type{});
+        if (plain || (complete && !fix_b_always))
+            sstore(Bs + buf * SB::SIZE, rb, n0, g.N, k0, integral_constant<bool, B_K>{}, integral_constant<int, BN>{},
+                   integral_constant<int, B_V2>{}, std::false_type{});
+        else
             sstore(Bs + buf * SB::SIZE, rb, n0, g.N, k0, integral_constant<bool, B_K>{}, integral_constant<int, BN>{},
                    integral_constant<int, B_V2>{}, std::true_type{});
-        }
     };
+    using AnyFlavour = integral_constant<int, EDGE ? ANY : PLAIN>;
 
     const uint32_t ktiles = (g.K + BK - 1) / BK;
     constexpr int S = BK / 8;
@@ -690,9 +700,9 @@ void gemm_f64_mfma_kernel(MArgs<double> g) {
         }
     };
 
-    load_ab(0, ra[0], rb[0]);
-    store_ab(0, 0, ra[0], rb[0]);
-    if (PF == 2 && ktiles > 1) load_ab(BK, ra[PF - 1], rb[PF - 1]);
+    load_ab(0, ra[0], rb[0], AnyFlavour{});
+    store_ab(0, 0, ra[0], rb[0], AnyFlavour{});
+    if (PF == 2 && ktiles > 1) load_ab(BK, ra[PF - 1], rb[PF - 1], AnyFlavour{});
     __syncthreads();
 
     // Same schedule as the f32 kernel: double-buffered fragments, hand-over in front of the last
@@ -712,17 +722,17 @@ void gemm_f64_mfma_kernel(MArgs<double> g) {
                     acc[i][j] = __builtin_amdgcn_mfma_f64_16x16x4f64(af[s & 1][i][t], bf[s & 1][j][t], acc[i][j], 0, 0, 0);
     };
 
-    if constexpr (PF == 1) {
+    if constexpr (PF == 1 && !EDGE) {
         for (uint32_t kt = 0; kt < ktiles; ++kt) {
             const int cur = kt & 1;
             const bool more = kt + 1 < ktiles;
-            if (more) load_ab((kt + 1) * BK, ra[0], rb[0]);
+            if (more) load_ab((kt + 1) * BK, ra[0], rb[0], AnyFlavour{});
 #pragma unroll
             for (int s = 0; s < S; ++s) {
                 if (s + 1 < S) {
                     read_frags(cur, s + 1, af[(s + 1) & 1], bf[(s + 1) & 1]);
                 } else if (more) {
-                    store_ab(cur ^ 1, (kt + 1) * BK, ra[0], rb[0]);
+                    store_ab(cur ^ 1, (kt + 1) * BK, ra[0], rb[0], AnyFlavour{});
                     __syncthreads();
                     read_frags(cur ^ 1, 0, af[(s + 1) & 1], bf[(s + 1) & 1]);
                 }
@@ -736,17 +746,23 @@ void gemm_f64_mfma_kernel(MArgs<double> g) {
             }
         }
     } else {
-        auto iteration = [&](uint32_t kt, auto parity_tag) {
+        // (the bounds-checked instantiation of every tile takes this loop, whose iterations exist per flavour)
+        auto iteration = [&](uint32_t kt, auto parity_tag, auto flavour_tag) __attribute__((always_inline)) {
             constexpr int P = decltype(parity_tag)::value;
             const int cur = kt & 1;
-            if (kt + 2 < ktiles) load_ab((kt + 2) * BK, ra[P], rb[P]);
+            if constexpr (PF == 1) {
+                load_ab((kt + 1) * BK, ra[0], rb[0], flavour_tag);
+            } else {
+                if (kt + 2 < ktiles) load_ab((kt + 2) * BK, ra[P], rb[P], flavour_tag);
+            }
+            constexpr int NEXT = PF == 1 ? 0 : 1 - P;
 #pragma unroll
             for (int s = 0; s < S; ++s) {
                 if (s + 1 < S) {
                     read_frags(cur, s + 1, af[(s + 1) & 1], bf[(s + 1) & 1]);
                 } else {
                     __builtin_amdgcn_sched_barrier(0);
-                    store_ab(cur ^ 1, (kt + 1) * BK, ra[1 - P], rb[1 - P]);
+                    store_ab(cur ^ 1, (kt + 1) * BK, ra[NEXT], rb[NEXT], flavour_tag);
                     __syncthreads();
                     read_frags(cur ^ 1, 0, af[(s + 1) & 1], bf[(s + 1) & 1]);
                     __builtin_amdgcn_sched_barrier(0);
@@ -754,14 +770,41 @@ void gemm_f64_mfma_kernel(MArgs<double> g) {
                 mfma_step(s);
             }
         };
+        auto run = [&](uint32_t &kt, uint32_t end, auto flavour_tag) __attribute__((always_inline)) {
+            if constexpr (PF == 1) {
+                for (; kt < end; ++kt) iteration(kt, integral_constant<int, 0>{}, flavour_tag);
+            } else {
+                if ((kt & 1) && kt < end) {
+                    iteration(kt, integral_constant<int, 1>{}, flavour_tag);
+                    ++kt;
+                }
+                for (; kt + 1 < end; kt += 2) {
+                    iteration(kt, integral_constant<int, 0>{}, flavour_tag);
+                    iteration(kt + 1, integral_constant<int, 1>{}, flavour_tag);
+                }
+                if (kt < end) {
+                    iteration(kt, integral_constant<int, 0>{}, flavour_tag);
+                    ++kt;
+                }
+            }
+        };
         uint32_t kt = 0;
-        for (; kt + 2 < ktiles; kt += 2) {
-            iteration(kt, integral_constant<int, 0>{});
-            iteration(kt + 1, integral_constant<int, 1>{});
-        }
-        if (kt + 1 < ktiles) {
-            iteration(kt, integral_constant<int, 0>{});
-            ++kt;
+        if constexpr (!EDGE) {
+            for (; kt + 2 < ktiles; kt += 2) {
+                iteration(kt, integral_constant<int, 0>{}, AnyFlavour{});
+                iteration(kt + 1, integral_constant<int, 1>{}, AnyFlavour{});
+            }
+            if (kt + 1 < ktiles) {
+                iteration(kt, integral_constant<int, 0>{}, AnyFlavour{});
+                ++kt;
+            }
+        } else {
+            const bool has_tail = g.K % BK != 0;
+            const uint32_t hand_overs = ktiles - 1;
+            const uint32_t main_end = has_tail ? (hand_overs > (uint32_t)PF ? hand_overs - PF : 0u) : hand_overs;
+            if (tile_inside) run(kt, main_end, integral_constant<int, PLAIN>{});
+            else run(kt, main_end, integral_constant<int, CLAMPED>{});
+            run(kt, hand_overs, integral_constant<int, ANY>{});
         }
         const int cur = kt & 1; // last slab: nothing to hand over
 #pragma unroll
