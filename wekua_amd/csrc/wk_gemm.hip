@@ -88,7 +88,8 @@ int wk_gemm(wk_stream *s, int dtype, int op_a, int op_b, uint64_t M, uint64_t N,
     p.num_cus = (uint32_t)s->dev->props.multiProcessorCount;
     if (is_int32(dtype)) {
         const int forced = g_forced.load(std::memory_order_relaxed);
-        const bool fits = workspace && workspace_bytes >= gemm_i32_packed_workspace_bytes(M, N, K);
+        const size_t need = gemm_i32_packed_workspace_bytes(M, N, K);
+        const bool fits = need && workspace && workspace_bytes >= need && (reinterpret_cast<uintptr_t>(workspace) & 15u) == 0;
         if (forced == -3 && !fits) return WK_E_INVALID_VALUE;
         if (fits && (forced == -3 || (forced == -2 && packed_pays(p))))
             return gemm_i32_packed_launch(s->stream, p, workspace, workspace_bytes);
@@ -116,7 +117,8 @@ const char *wk_gemm_variant_with_workspace(int dtype, int op_a, int op_b, uint64
     const char *plain = wk_gemm_variant(dtype, op_a, op_b, M, N, K, lda, ldb, ldc, A, B, C);
     if (!is_int32(dtype) || !std::strcmp(plain, "invalid")) return plain;
     const int forced = g_forced.load(std::memory_order_relaxed);
-    const bool fits = workspace_bytes && workspace_bytes >= gemm_i32_packed_workspace_bytes(M, N, K);
+    const size_t need = gemm_i32_packed_workspace_bytes(M, N, K);
+    const bool fits = need && workspace_bytes >= need;
     GemmProblem p;
     p.M = M; p.N = N; p.K = K;
     if (forced == -3) return fits ? k_packed_names[dtype == WK_U32] : "invalid";

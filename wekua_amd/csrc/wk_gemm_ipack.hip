@@ -320,12 +320,17 @@ template <int BM, bool EDGE> int launch_packed(hipStream_t st, PArgs g) {
 
 } // namespace
 
-size_t wk::gemm_i32_packed_workspace_bytes(uint64_t M, uint64_t N, uint64_t K) { return make_layout(M, N, K).total; }
+// 0: this problem cannot take the packed path (a group stream of KB * 4 KiB must fit the 31-bit extent
+// of a buffer resource, the dimensions 31 bits)
+size_t wk::gemm_i32_packed_workspace_bytes(uint64_t M, uint64_t N, uint64_t K) {
+    if (!M || !N || !K || M > 0x7fffffffull || N > 0x7fffffffull || K > (0x7fffffffull / GROUP_BYTES) * BK) return 0;
+    return make_layout(M, N, K).total;
+}
 
 int wk::gemm_i32_packed_launch(hipStream_t st, const GemmProblem &p, void *workspace, size_t workspace_bytes) {
+    if (!gemm_i32_packed_workspace_bytes(p.M, p.N, p.K)) return WK_E_INVALID_VALUE;
     const Layout w = make_layout(p.M, p.N, p.K);
     if (!workspace || workspace_bytes < w.total || (reinterpret_cast<uintptr_t>(workspace) & 15u)) return WK_E_INVALID_VALUE;
-    if (p.M > 0x7fffffffull || p.N > 0x7fffffffull || p.K > 0x7fffffffull) return WK_E_INVALID_VALUE;
     unsigned char *ws = static_cast<unsigned char *>(workspace);
 
     PackArgs pa;
