@@ -127,3 +127,30 @@ def test_int32_gemm_packed_planes_beyond_4_gib(env):
     packed.deinit(pipeline)
     for t in (a, b, c):
         t.release(pipeline)
+
+
+def test_transpose_and_copy_beyond_4_gib(env):
+    """transpose of a 32768 x 40000 f32 tensor (5.2 GB) into a skew-pitched 40000 x 32768 one, and
+    memory.copy of the result: sampled rows of both against the generator's values."""
+    context, pipeline, _rawdev = env
+    R, C = 32768, 40000
+    src = wk.Tensor.alloc("f32", context, pipeline, (R, C))
+    dst = wk.Tensor.alloc("f32", context, pipeline, (C, R))
+    wk.random.uniform(pipeline, src, 41)
+    wk.transpose(pipeline, dst, src, 0, 1)
+    rows = (0, 1, 20000, 32000, 39998, 39999)          # row j of dst starts at byte j * pitch * 4: beyond 2^32 from j = 32641
+    assert 32000 * dst.row_pitch * 4 < 2 ** 32 < 39998 * dst.row_pitch * 4
+
+    def check(tensor):
+        for j in rows:
+            got = window(env, tensor, j * tensor.row_pitch, R, np.float32)
+            idx = np.arange(R, dtype=np.uint64) * np.uint64(C) + np.uint64(j)     # src[i][j]
+            want = ot._component(ot.hash64(idx, 41), np.dtype(np.float32), None, None)
+            assert np.array_equal(got, want), f"row {j}"
+    check(dst)
+    src.release(pipeline)
+    dup = wk.Tensor.alloc("f32", context, pipeline, (C, R))
+    wk.memory.copy(pipeline, dst, dup)
+    check(dup)
+    dst.release(pipeline)
+    dup.release(pipeline)
