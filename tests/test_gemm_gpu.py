@@ -241,3 +241,22 @@ def test_invalid_arguments(dev):
     assert lib.wk_gemm(dev.stream, 8, 0, 0, 4, 4, 4, None, None, 4, p, 4, None, p, 4, None, 0) == 1
     assert lib.wk_gemm(None, 8, 0, 0, 4, 4, 4, None, p, 4, p, 4, None, p, 4, None, 0) == 1
     buf.free()
+
+
+@pytest.mark.parametrize("dtype,variant", [("f32", "mfma_f32_64x64"), ("f32", "mfma_f32_128x128"), ("f32", "mfma_f32_256x128"),
+                                           ("f64", "mfma_f64_64x64"), ("f64", "mfma_f64_128x64"), ("f64", "mfma_f64_128x128")])
+def test_every_k_around_the_slab_boundaries(dev, dtype, variant):
+    """Every K from 1 to 100 on a ragged tile and on a tile-aligned shape: the bounds-checked kernels
+    choose per-flavour loops from the number of complete slabs (k-slab 16 or 32, one or two slabs of
+    prefetch), so every count of slabs from one to a handful, with and without a k tail, must agree."""
+    assert dev.lib.wk_gemm_force_variant(variant.encode()) == 0
+    try:
+        for K in range(1, 101):
+            op_a, op_b = K % 2, (K // 2) % 2
+            check(dev, dtype, 70, 45, K, op_a, op_b, 1.5, 0.5, seed=100 + K)
+            if K % 7 == 0:
+                check(dev, dtype, 256, 128, K, op_a, op_b, None, None, seed=300 + K)
+                check(dev, dtype, 130, 257, K, 1 - op_a, op_b, 2.0, None, seed=400 + K, lda=(130 if 1 - op_a else K) + 1,
+                      ldb=(K if op_b else 257) + 3, ldc=257 + 5)
+    finally:
+        dev.lib.wk_gemm_force_variant(b"auto")
