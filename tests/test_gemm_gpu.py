@@ -260,3 +260,17 @@ def test_every_k_around_the_slab_boundaries(dev, dtype, variant):
                       ldb=(K if op_b else 257) + 3, ldc=257 + 5)
     finally:
         dev.lib.wk_gemm_force_variant(b"auto")
+
+
+@pytest.mark.parametrize("variant", ["mfma_i32_64x128", "mfma_i32_128x128", "mfma_i32_packed"])
+def test_int32_every_k(dev, variant):
+    """K from 1 to 70 (one to three k-slabs, every tail length; for the pack pass also fewer k-blocks
+    than k-ranges of its grid) on a ragged shape, full-range entries, bit-exact."""
+    packed = variant.endswith("packed")
+    assert dev.lib.wk_gemm_force_variant(variant.encode()) == 0
+    try:
+        for K in range(1, 71):
+            op_a, op_b = K % 2, (K // 2) % 2
+            check(dev, "i32", 70, 130, K, op_a, op_b, -7, 3, seed=500 + K, packed=packed)
+    finally:
+        dev.lib.wk_gemm_force_variant(b"auto")
