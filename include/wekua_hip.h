@@ -199,6 +199,14 @@ int  wk_activation_dev(wk_stream *s, int dtype, int kind, const uint64_t shape3[
  * follows it in Linear.forward (src/nn/layer/linear.zig:480-525).  bias may be NULL, kind WK_ACT_NONE. */
 int  wk_bias_activation(wk_stream *s, int dtype, int kind, uint64_t rows, uint64_t cols, void *out, uint64_t out_pitch,
                         const void *bias);
+/* One matrix of Linear.forward in one call (src/nn/layer/linear.zig:480-525: blas.gemm, addBias,
+ * act.run): C = act(op(A)op(B) + bias[col]), f32 / f64.  For op N, T (x times the transposed weight
+ * matrix, what Linear runs) bias and activation are applied in the epilogue of the matrix-core kernel,
+ * to the same bits as wk_gemm followed by wk_bias_activation; any other layout runs those two.
+ * bias may be NULL, kind WK_ACT_NONE. */
+int  wk_gemm_bias_activation(wk_stream *s, int dtype, int op_a, int op_b, uint64_t M, uint64_t N, uint64_t K,
+                             const void *A, uint64_t lda, const void *B, uint64_t ldb, void *C, uint64_t ldc,
+                             const void *bias, int kind);
 /* Linear.getBiasSensitivity: bias_grad[c] = sum_r sens[r][c] (src/nn/layer/kernels/bias_step.cl) */
 int  wk_bias_step(wk_stream *s, int dtype, uint64_t rows, uint64_t cols, const void *sens, uint64_t pitch, void *bias_grad);
 /* loss.mse kernel: err = expected - output; error = err^2; dev = -2*err when dev != NULL

@@ -99,6 +99,29 @@ int wk_gemm(wk_stream *s, int dtype, int op_a, int op_b, uint64_t M, uint64_t N,
     return gemm_generic_launch(s->stream, p);
 }
 
+int wk_gemm_bias_activation(wk_stream *s, int dtype, int op_a, int op_b, uint64_t M, uint64_t N, uint64_t K, const void *A,
+                            uint64_t lda, const void *B, uint64_t ldb, void *C, uint64_t ldc, const void *bias, int kind) {
+    int rc = bind(s);
+    if (rc) return rc;
+    if (kind != WK_ACT_NONE && kind != WK_ACT_SIGMOID && kind != WK_ACT_TANH) return WK_E_INVALID_VALUE;
+    if (dtype != WK_F32 && dtype != WK_F64) return WK_E_TYPE_NOT_SUPPORTED;
+    GemmProblem p;
+    rc = build_problem(p, dtype, op_a, op_b, M, N, K, nullptr, A, lda, B, ldb, nullptr, C, ldc);
+    if (rc) return rc;
+    p.num_cus = (uint32_t)s->dev->props.multiProcessorCount;
+    const int v = choose(p);
+    if (v >= 0 && gemm_mfma_fuses(p, v) && (bias || kind != WK_ACT_NONE)) {
+        p.ext = true;
+        p.ext_bias = bias;
+        p.ext_act = kind;
+        return gemm_mfma_launch(s->stream, p, v);
+    }
+    // no fused kernel for this layout or variant: the product, then the element-wise pass
+    rc = v >= 0 ? gemm_mfma_launch(s->stream, p, v) : gemm_generic_launch(s->stream, p);
+    if (rc || (!bias && kind == WK_ACT_NONE)) return rc;
+    return wk_bias_activation(s, dtype, kind, M, N, C, ldc, bias);
+}
+
 const char *wk_gemm_variant(int dtype, int op_a, int op_b, uint64_t M, uint64_t N, uint64_t K, uint64_t lda, uint64_t ldb,
                             uint64_t ldc, const void *A, const void *B, const void *C) {
     GemmProblem p;

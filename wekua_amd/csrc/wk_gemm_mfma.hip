@@ -56,6 +56,9 @@ template <typename T> struct MArgs {
     uint32_t xcd_remap; // 1: renumber work-groups so that each XCD gets a contiguous run of tiles
     int epi;
     T alpha, beta;
+    // epilogue extension (kernels instantiated with EXT): C = act(acc + bias[col]); bias may be null
+    const T *bias;
+    int act;
 };
 
 // Work-groups that share a CU start in lock step (the whole first wave of work-groups is
@@ -104,7 +107,7 @@ template <int ROWS, int BK, bool KCONTIG> struct Slab {
     static constexpr int SIZE = KCONTIG ? ROWS * LD : BK * LD;
 };
 
-template <int BM, int BN, int BK, int WAVES_M, int WAVES_N, int OCC, bool A_K, bool B_K, bool EDGE>
+template <int BM, int BN, int BK, int WAVES_M, int WAVES_N, int OCC, bool A_K, bool B_K, bool EDGE, bool EXT = false>
 __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) __attribute__((amdgpu_waves_per_eu(OCC)))
 void gemm_f32_mfma_kernel(MArgs<float> g) {
     constexpr int NT = WAVES_M * WAVES_N * 64;
@@ -487,6 +490,10 @@ void gemm_f32_mfma_kernel(MArgs<float> g) {
         for (int j = 0; j < FN; ++j) {
             const uint32_t col = n0 + wn * WN + j * 32 + l32;
             const uint32_t colc = EDGE ? min(col, g.N - 1) : col;
+            float bias_v = 0.f;
+            if constexpr (EXT) {
+                if (g.bias) bias_v = g.bias[colc];
+            }
             float old[16];
             if (g.epi == EPI_ALPHA_BETA) {
 #pragma unroll
@@ -502,6 +509,10 @@ void gemm_f32_mfma_kernel(MArgs<float> g) {
                 float v = acc[i][j][r];
                 if (g.epi == EPI_ALPHA) v = alpha * v;
                 else if (g.epi == EPI_ALPHA_BETA) v = alpha * v + beta * old[r];
+                if constexpr (EXT) {
+                    if (g.bias) v += bias_v;
+                    v = act_forward<float>(g.act, v);
+                }
                 if (!EDGE || ((row < g.M) & (col < g.N))) g.C[(size_t)row * g.ldc + col] = v;
             }
         }
@@ -517,7 +528,7 @@ template <int ROWS, int BK, bool KCONTIG> struct SlabD {
     static constexpr int SIZE = KCONTIG ? ROWS * LD : BK * LD;
 };
 
-template <int BM, int BN, int BK, int WAVES_M, int WAVES_N, int OCC, bool A_K, bool B_K, bool EDGE>
+template <int BM, int BN, int BK, int WAVES_M, int WAVES_N, int OCC, bool A_K, bool B_K, bool EDGE, bool EXT = false>
 __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) __attribute__((amdgpu_waves_per_eu(OCC)))
 void gemm_f64_mfma_kernel(MArgs<double> g) {
     constexpr int NT = WAVES_M * WAVES_N * 64;
@@ -821,6 +832,10 @@ void gemm_f64_mfma_kernel(MArgs<double> g) {
         for (int j = 0; j < FN; ++j) {
             const uint32_t col = n0 + wn * WN + j * 16 + l16;
             const uint32_t colc = EDGE ? min(col, g.N - 1) : col;
+            double bias_v = 0.;
+            if constexpr (EXT) {
+                if (g.bias) bias_v = g.bias[colc];
+            }
             double old[4];
             if (g.epi == EPI_ALPHA_BETA) { // batched, clamped reads of C_old (see the f32 kernel)
 #pragma unroll
@@ -836,6 +851,10 @@ void gemm_f64_mfma_kernel(MArgs<double> g) {
                 double v = acc[i][j][r];
                 if (g.epi == EPI_ALPHA) v = alpha * v;
                 else if (g.epi == EPI_ALPHA_BETA) v = alpha * v + beta * old[r];
+                if constexpr (EXT) {
+                    if (g.bias) v += bias_v;
+                    v = act_forward<double>(g.act, v);
+                }
                 if (!EDGE || ((row < g.M) & (col < g.N))) g.C[(size_t)row * g.ldc + col] = v;
             }
         }
@@ -861,6 +880,8 @@ template <typename T> MArgs<T> make_args(const GemmProblem &p, int bm, int bn) {
     g.epi = p.epi;
     std::memcpy(&g.alpha, p.alpha, sizeof(T));
     std::memcpy(&g.beta, p.beta, sizeof(T));
+    g.bias = static_cast<const T *>(p.ext_bias);
+    g.act = p.ext_act;
     return g;
 }
 
@@ -873,10 +894,10 @@ template <typename K> int set_lds(K kernel, size_t bytes) {
     return WK_OK;
 }
 
-template <int BM, int BN, int BK, int WMS, int WNS, int OCC, bool AK, bool BKC, bool EDGE>
+template <int BM, int BN, int BK, int WMS, int WNS, int OCC, bool AK, bool BKC, bool EDGE, bool EXT = false>
 int launch_f32_one(hipStream_t st, const GemmProblem &p) {
     constexpr size_t lds = 2 * (Slab<BM, BK, AK>::SIZE + Slab<BN, BK, BKC>::SIZE) * sizeof(float);
-    auto kern = gemm_f32_mfma_kernel<BM, BN, BK, WMS, WNS, OCC, AK, BKC, EDGE>;
+    auto kern = gemm_f32_mfma_kernel<BM, BN, BK, WMS, WNS, OCC, AK, BKC, EDGE, EXT>;
     static int attr_rc = set_lds(kern, lds);
     if (attr_rc) return attr_rc;
     MArgs<float> g = make_args<float>(p, BM, BN);
@@ -887,6 +908,11 @@ int launch_f32_one(hipStream_t st, const GemmProblem &p) {
 template <int BM, int BN, int BK, int WMS, int WNS, int OCC>
 int launch_f32(hipStream_t st, const GemmProblem &p, bool edge) {
     const int sel = (p.op_a ? 0 : 2) | (p.op_b ? 1 : 0); // bit1: A k-contiguous, bit0: B k-contiguous
+    if (p.ext) { // fused bias + activation: instantiated for op N, T only (see gemm_mfma_fuses)
+        if (sel != 3) return WK_E_INVALID_VALUE;
+        return edge ? launch_f32_one<BM, BN, BK, WMS, WNS, OCC, true, true, true, true>(st, p)
+                    : launch_f32_one<BM, BN, BK, WMS, WNS, OCC, true, true, false, true>(st, p);
+    }
 #define WK_CASE(AK, BKC)                                                                                   \
     return edge ? launch_f32_one<BM, BN, BK, WMS, WNS, OCC, AK, BKC, true>(st, p)                          \
                 : launch_f32_one<BM, BN, BK, WMS, WNS, OCC, AK, BKC, false>(st, p)
@@ -899,10 +925,10 @@ int launch_f32(hipStream_t st, const GemmProblem &p, bool edge) {
 #undef WK_CASE
 }
 
-template <int BM, int BN, int BK, int WMS, int WNS, int OCC, bool AK, bool BKC, bool EDGE>
+template <int BM, int BN, int BK, int WMS, int WNS, int OCC, bool AK, bool BKC, bool EDGE, bool EXT = false>
 int launch_f64_one(hipStream_t st, const GemmProblem &p) {
     constexpr size_t lds = 2 * (SlabD<BM, BK, AK>::SIZE + SlabD<BN, BK, BKC>::SIZE) * sizeof(double);
-    auto kern = gemm_f64_mfma_kernel<BM, BN, BK, WMS, WNS, OCC, AK, BKC, EDGE>;
+    auto kern = gemm_f64_mfma_kernel<BM, BN, BK, WMS, WNS, OCC, AK, BKC, EDGE, EXT>;
     static int attr_rc = set_lds(kern, lds);
     if (attr_rc) return attr_rc;
     MArgs<double> g = make_args<double>(p, BM, BN);
@@ -913,6 +939,11 @@ int launch_f64_one(hipStream_t st, const GemmProblem &p) {
 template <int BM, int BN, int BK, int WMS, int WNS, int OCC>
 int launch_f64(hipStream_t st, const GemmProblem &p, bool edge) {
     const int sel = (p.op_a ? 0 : 2) | (p.op_b ? 1 : 0);
+    if (p.ext) {
+        if (sel != 3) return WK_E_INVALID_VALUE;
+        return edge ? launch_f64_one<BM, BN, BK, WMS, WNS, OCC, true, true, true, true>(st, p)
+                    : launch_f64_one<BM, BN, BK, WMS, WNS, OCC, true, true, false, true>(st, p);
+    }
 #define WK_CASE(AK, BKC)                                                                                   \
     return edge ? launch_f64_one<BM, BN, BK, WMS, WNS, OCC, AK, BKC, true>(st, p)                               \
                 : launch_f64_one<BM, BN, BK, WMS, WNS, OCC, AK, BKC, false>(st, p)
@@ -948,6 +979,18 @@ const VariantDesc k_variants[] = {
     {"mfma_u32_128x128", WK_U32, 128, 128, 32, 1.0, 0.25, &gemm_i32_mfma_launch_128},
 };
 constexpr int k_num_variants = sizeof(k_variants) / sizeof(k_variants[0]);
+
+} // namespace
+
+// The fused epilogue is instantiated for the f32 / f64 kernels of this file and for op N, T only
+// (x * W^T, the product Linear.forward makes).
+bool wk::gemm_mfma_fuses(const GemmProblem &p, int variant) {
+    if (variant < 0 || variant >= k_num_variants) return false;
+    const VariantDesc &v = k_variants[variant];
+    return (v.dtype == WK_F32 || v.dtype == WK_F64) && v.dtype == p.dtype && !p.op_a && p.op_b;
+}
+
+namespace {
 
 bool needs_edge(const GemmProblem &p, const VariantDesc &v) {
     const size_t es = p.dtype == WK_F64 ? 8 : 4;

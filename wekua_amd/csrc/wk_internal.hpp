@@ -159,6 +159,11 @@ struct GemmProblem {
     uint32_t num_cus;                 // compute units of the device the stream belongs to
     alignas(16) unsigned char alpha[16];  // one element of dtype (valid when epi != EPI_STORE)
     alignas(16) unsigned char beta[16];   // one element of dtype (valid when epi == EPI_ALPHA_BETA)
+    // fused epilogue of Linear.forward: C = act(op(A)op(B) + bias[col]); only the f32 / f64 matrix-core
+    // kernels for op N, T carry it (gemm_mfma_fuses)
+    bool ext = false;
+    const void *ext_bias = nullptr;   // N elements of dtype, or null
+    int ext_act = -1;                 // WK_ACT_*
 };
 
 // generic LDS-tiled VALU kernel, every dtype and shape (wk_gemm_generic.hip)
@@ -171,8 +176,20 @@ int gemm_i32_mfma_launch_128(hipStream_t st, const GemmProblem &p, bool edge); /
 // i32 / u32 with a pack pass into caller-provided workspace (wk_gemm_ipack.hip)
 size_t gemm_i32_packed_workspace_bytes(uint64_t M, uint64_t N, uint64_t K);
 int gemm_i32_packed_launch(hipStream_t st, const GemmProblem &p, void *workspace, size_t workspace_bytes);
+bool gemm_mfma_fuses(const GemmProblem &p, int variant); // variant can run p with the fused bias + activation epilogue
 int gemm_mfma_pick(const GemmProblem &p);        // -1: not applicable
 const char *gemm_mfma_variant_name(int variant); // nullptr past the end
 int gemm_mfma_variant_dtype(int variant);
+
+
+#ifdef __HIPCC__
+// activation of nn.activation.{Sigmoid,Tanh} (src/nn/activation/kernels/{sigmoid,tanh}.cl), shared by
+// the element-wise kernels and the fused GEMM epilogue so that both give the same bits
+template <typename T> __device__ __forceinline__ T act_forward(int kind, T x) {
+    if (kind == WK_ACT_SIGMOID) return T(1) / (T(1) + exp(-x));
+    if (kind == WK_ACT_TANH) return tanh(x);
+    return x;
+}
+#endif
 
 } // namespace wk

@@ -28,11 +28,6 @@ template <typename T> struct Opnd {
     uint64_t rp, sp;
 };
 
-template <typename T> __device__ __forceinline__ T act_forward(int kind, T x) {
-    if (kind == WK_ACT_SIGMOID) return T(1) / (T(1) + exp(-x));
-    if (kind == WK_ACT_TANH) return tanh(x);
-    return x;
-}
 template <typename T> __device__ __forceinline__ T act_derivative(int kind, T y) {
     if (kind == WK_ACT_SIGMOID) return y * (T(1) - y);
     if (kind == WK_ACT_TANH) return T(1) - y * y;

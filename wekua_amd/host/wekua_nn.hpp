@@ -219,19 +219,18 @@ template <typename T> struct Linear : Layer<T> {
     }
 
     // forward (linear.zig:480-525): out = in * W^T, then addBias and the activation -- here one
-    // fused pass over the output with the same arithmetic
+    // call: bias and activation run in the epilogue of the matrix-core kernel
     TensorT *forward(Pipeline *pipeline, TensorT *input, void *cache) const override {
         LinearCache *c = static_cast<LinearCache *>(cache);
         for (size_t i = 0; i < weights.size(); ++i) {
             TensorT *out = c->outputs[i];
-            blas::gemm<T>(pipeline, std::nullopt, input, blas::Operation::no_transpose, weights[i], blas::Operation::transpose,
-                          std::nullopt, out, nullptr);
-            if (bias_enabled || activation) {
-                check(wk_bias_activation(pipeline->command_queue->stream, core::getTypeIndex<T>(),
-                                         activation ? activation->kind : WK_ACT_NONE, out->rows(), out->cols(), out->buffer,
-                                         out->memory_layout.row_pitch, bias_enabled ? bias[i]->buffer : nullptr));
-                pipeline->append(1);
-            }
+            blas::validateTensors<T>(input, weights[i], out, blas::Operation::no_transpose, blas::Operation::transpose);
+            check(wk_gemm_bias_activation(pipeline->command_queue->stream, core::getTypeIndex<T>(), 0, 1, out->rows(), out->cols(),
+                                          input->cols(), input->buffer, input->memory_layout.row_pitch, weights[i]->buffer,
+                                          weights[i]->memory_layout.row_pitch, out->buffer, out->memory_layout.row_pitch,
+                                          bias_enabled ? bias[i]->buffer : nullptr,
+                                          activation ? activation->kind : WK_ACT_NONE));
+            pipeline->append(1);
             input = out;
         }
         return input;
