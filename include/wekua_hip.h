@@ -157,10 +157,11 @@ int  wk_axpy(wk_stream *s, int dtype, const uint64_t shape3[3],
  *                              multiplied even when beta == 0 (NaN/Inf propagate).
  *   Integers wrap modulo 2^width; f32/f64 accumulate in their own precision.
  *   The reference's PackedTensors pass (gemm.zig:60-359, 705-720: pack A and B into two scratch
- *   tensors before every product) survives for i32 / u32 only: with `workspace` of at least
- *   wk_gemm_workspace_bytes() bytes of device memory (16-byte aligned; what blas.PackedTensors
- *   holds) large products first pack both operands into signed-digit planes there and then run a
- *   leaner matrix-core kernel; the result is the same bits either way.  Every other type stages
+ *   tensors before every product) survives for the 8-, 16- and 32-bit integers: with `workspace` of
+ *   at least wk_gemm_workspace_bytes() bytes of device memory (16-byte aligned; what
+ *   blas.PackedTensors holds) products that are large enough first pack both operands into
+ *   signed-digit planes there and then run a lean int8 matrix-core kernel (for 8 and 16 bits the
+ *   only matrix-core path); the result is the same bits either way.  Every other type stages
  *   its tiles through LDS straight from the row-major operands, asks for 0 bytes and ignores the
  *   workspace, which may always be NULL.  The workspace is overwritten by every call that uses it:
  *   calls sharing one must be ordered on one stream. */

@@ -274,3 +274,38 @@ def test_int32_every_k(dev, variant):
             check(dev, "i32", 70, 130, K, op_a, op_b, -7, 3, seed=500 + K, packed=packed)
     finally:
         dev.lib.wk_gemm_force_variant(b"auto")
+
+
+@pytest.mark.parametrize("dtype", ["i8", "u8", "i16", "u16"])
+@pytest.mark.parametrize("op_a,op_b", OPS)
+def test_narrow_integers_packed_bit_exact(dev, dtype, op_a, op_b):
+    """8- and 16-bit integers on the int8 matrix cores (pack pass + packed kernel with one or two digits
+    per element) against the exact product modulo 2^8 / 2^16: full-range entries, aligned and ragged
+    shapes, K around the slab boundaries (a slab is 128 / 64 values of k), odd leading dimensions."""
+    signed = dtype.startswith("i")
+    assert dev.lib.wk_gemm_force_variant(f"mfma_{dtype}_packed".encode()) == 0
+    try:
+        for (M, N, K) in [(128, 128, 128), (256, 128, 64), (1, 1, 1), (65, 129, 33), (200, 300, 77), (63, 127, 500), (130, 70, 129)]:
+            for alpha, beta in [(None, None), (3, None), (-5 if signed else 201, 7), (None, 1)]:
+                check(dev, dtype, M, N, K, op_a, op_b, alpha, beta, seed=61, packed=True)
+        for K in (31, 32, 63, 64, 65, 127, 128, 191, 192, 257):
+            check(dev, dtype, 70, 45, K, op_a, op_b, 3, 2, seed=62 + K, packed=True)
+        check(dev, dtype, 130, 70, 200, op_a, op_b, 3, 7, seed=64, packed=True,
+              lda=(130 if op_a else 200) + 3, ldb=(200 if op_b else 70) + 5, ldc=70 + 7)
+    finally:
+        dev.lib.wk_gemm_force_variant(b"auto")
+
+
+@pytest.mark.parametrize("dtype", ["i8", "u16"])
+def test_narrow_integers_with_workspace_automatic(dev, dtype):
+    """With a workspace the automatic choice takes the matrix cores from a few hundred cubed up; the
+    result equals the vector-ALU kernel's (no workspace) and the oracle's."""
+    M, N, K = 768, 640, 1024
+    a, b, c = gemm_operands(dtype, M, N, K, 0, 1, 7)
+    from wekua_amd import raw
+    need = dev.lib.wk_gemm_workspace_bytes(raw.dtype_id(dtype), 0, 1, M, N, K)
+    assert dev.lib.wk_gemm_variant_with_workspace(raw.dtype_id(dtype), 0, 1, M, N, K, K, K, N, None, None, None, need) \
+        == f"mfma_{dtype}_packed".encode()
+    want = oracle.gemm(dtype, 3, a, 0, b, 1, 5, c)
+    assert np.array_equal(run_gemm(dev, dtype, 3, a, 0, b, 1, 5, c, packed=True), want)
+    assert np.array_equal(run_gemm(dev, dtype, 3, a, 0, b, 1, 5, c), want)

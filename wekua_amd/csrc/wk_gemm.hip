@@ -10,18 +10,25 @@ using namespace wk;
 
 namespace {
 
-// -3: the packed int32 path whenever a workspace comes along; -2: automatic; -1: generic tile kernel;
+// -3: the packed integer path whenever a workspace comes along; -2: automatic; -1: generic tile kernel;
 // >= 0: index into the MFMA variant table
 std::atomic<int> g_forced{-2};
 
 const char *k_generic_name = "tile64";
-const char *k_packed_names[2] = {"mfma_i32_packed", "mfma_u32_packed"};
+// indexed by dtype (WK_I8 .. WK_U32)
+const char *k_packed_names[6] = {"mfma_i8_packed", "mfma_u8_packed", "mfma_i16_packed", "mfma_u16_packed",
+                                 "mfma_i32_packed", "mfma_u32_packed"};
 
 bool is_int32(int dtype) { return dtype == WK_I32 || dtype == WK_U32; }
-// The pack pass reads A and B once more and writes as much.  Measured against the fused kernel on
-// MI355X (all four layouts): 1024^3 -8 %, 2048^3 equal, 4096^3 +9..10 %, 8192^3 +13..18 %.
+bool has_packed_path(int dtype) { return dtype >= WK_I8 && dtype <= WK_U32; }
+// The pack pass reads A and B once more and writes as much.  32-bit, measured against the fused
+// matrix-core kernel on MI355X (all four layouts): 1024^3 -8 %, 2048^3 equal, 4096^3 +9..10 %,
+// 8192^3 +13..18 %.  8- and 16-bit integers have only the vector-ALU kernel (36-45 TOP/s) beside it:
+// the two launches of the packed path take 16-20 us up to 1024^3, which that kernel beats below ~700^3.
 bool packed_pays(const GemmProblem &p) {
-    return p.M >= 1024 && p.N >= 1024 && (double)p.M * (double)p.N * (double)p.K >= 3.0e10;
+    const double work = (double)p.M * (double)p.N * (double)p.K;
+    if (is_int32(p.dtype)) return p.M >= 1024 && p.N >= 1024 && work >= 3.0e10;
+    return p.M >= 256 && p.N >= 256 && work >= 4.0e8;
 }
 
 int build_problem(GemmProblem &p, int dtype, int op_a, int op_b, uint64_t M, uint64_t N, uint64_t K,
@@ -73,8 +80,8 @@ int choose(const GemmProblem &p) {
 extern "C" {
 
 size_t wk_gemm_workspace_bytes(int dtype, int, int, uint64_t M, uint64_t N, uint64_t K) {
-    if (!is_int32(dtype) || !M || !N || !K) return 0;
-    return gemm_i32_packed_workspace_bytes(M, N, K);
+    if (!has_packed_path(dtype) || !M || !N || !K) return 0;
+    return gemm_int_packed_workspace_bytes(dtype, M, N, K);
 }
 
 int wk_gemm(wk_stream *s, int dtype, int op_a, int op_b, uint64_t M, uint64_t N, uint64_t K, const void *host_alpha,
@@ -86,13 +93,13 @@ int wk_gemm(wk_stream *s, int dtype, int op_a, int op_b, uint64_t M, uint64_t N,
     rc = build_problem(p, dtype, op_a, op_b, M, N, K, host_alpha, A, lda, B, ldb, host_beta, C, ldc);
     if (rc) return rc;
     p.num_cus = (uint32_t)s->dev->props.multiProcessorCount;
-    if (is_int32(dtype)) {
+    if (has_packed_path(dtype)) {
         const int forced = g_forced.load(std::memory_order_relaxed);
-        const size_t need = gemm_i32_packed_workspace_bytes(M, N, K);
+        const size_t need = gemm_int_packed_workspace_bytes(dtype, M, N, K);
         const bool fits = need && workspace && workspace_bytes >= need && (reinterpret_cast<uintptr_t>(workspace) & 15u) == 0;
         if (forced == -3 && !fits) return WK_E_INVALID_VALUE;
         if (fits && (forced == -3 || (forced == -2 && packed_pays(p))))
-            return gemm_i32_packed_launch(s->stream, p, workspace, workspace_bytes);
+            return gemm_int_packed_launch(s->stream, p, workspace, workspace_bytes);
     }
     const int v = choose(p);
     if (v >= 0) return gemm_mfma_launch(s->stream, p, v);
@@ -138,20 +145,21 @@ const char *wk_gemm_variant_with_workspace(int dtype, int op_a, int op_b, uint64
                                            uint64_t ldb, uint64_t ldc, const void *A, const void *B, const void *C,
                                            size_t workspace_bytes) {
     const char *plain = wk_gemm_variant(dtype, op_a, op_b, M, N, K, lda, ldb, ldc, A, B, C);
-    if (!is_int32(dtype) || !std::strcmp(plain, "invalid")) return plain;
+    if (!has_packed_path(dtype) || !std::strcmp(plain, "invalid")) return plain;
     const int forced = g_forced.load(std::memory_order_relaxed);
-    const size_t need = gemm_i32_packed_workspace_bytes(M, N, K);
+    const size_t need = gemm_int_packed_workspace_bytes(dtype, M, N, K);
     const bool fits = need && workspace_bytes >= need;
     GemmProblem p;
-    p.M = M; p.N = N; p.K = K;
-    if (forced == -3) return fits ? k_packed_names[dtype == WK_U32] : "invalid";
-    return fits && forced == -2 && packed_pays(p) ? k_packed_names[dtype == WK_U32] : plain;
+    p.dtype = dtype; p.M = M; p.N = N; p.K = K;
+    if (forced == -3) return fits ? k_packed_names[dtype] : "invalid";
+    return fits && forced == -2 && packed_pays(p) ? k_packed_names[dtype] : plain;
 }
 
 int wk_gemm_force_variant(const char *name) {
     if (!name || !std::strcmp(name, "auto")) { g_forced.store(-2); return WK_OK; }
     if (!std::strcmp(name, k_generic_name)) { g_forced.store(-1); return WK_OK; }
-    if (!std::strcmp(name, k_packed_names[0]) || !std::strcmp(name, k_packed_names[1])) { g_forced.store(-3); return WK_OK; }
+    for (const char *packed : k_packed_names)
+        if (!std::strcmp(name, packed)) { g_forced.store(-3); return WK_OK; }
     for (int v = 0; gemm_mfma_variant_name(v); ++v)
         if (!std::strcmp(name, gemm_mfma_variant_name(v))) { g_forced.store(v); return WK_OK; }
     return WK_E_INVALID_VALUE;

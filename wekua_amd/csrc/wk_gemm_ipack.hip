@@ -21,6 +21,11 @@
 //
 // Workspace: 128 bytes per (padded row, 32 k) of each operand + the partial sums; for 2048^3 that
 // is 2 x 16 MiB.  The pack pass costs what reading A and B once and writing as much costs.
+//
+// 8- and 16-bit integers take the same two passes with one or two digits per element (modulo 2^8 only
+// the pair (0,0) survives, modulo 2^16 the pairs with i + j <= 1): a slab is then four or two k-blocks
+// of 32, so that it is 4 KiB per 32 rows whatever the width, and the matrix work per slab is 4 x 1 or
+// 2 x 3 instructions per 32 x 32 block instead of 10.  Their only other kernel is the vector-ALU one.
 #include "wk_internal.hpp"
 
 #include <cstring>
@@ -35,29 +40,35 @@ typedef int i32x4 __attribute__((ext_vector_type(4)));
 typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
 struct __attribute__((packed, aligned(4))) u32x4_u { u32x4 v; };
 
-constexpr uint32_t CBIAS = 0x80808080u;
-constexpr int TILE = 128, BK = 32, BLOCK_BYTES = 1024, GROUP_BYTES = 4 * BLOCK_BYTES; // 4 digits of one (32 rows, 32 k)
+constexpr int TILE = 128, BK = 32, BLOCK_BYTES = 1024, GROUP_BYTES = 4 * BLOCK_BYTES; // one slab of 32 rows: 4 blocks
+// element of D bytes = D digits; c = 0x80 in every byte; a slab holds 4 / D k-blocks of D digit blocks
+template <typename E> struct Digits {
+    static constexpr int D = sizeof(E), KB_PER_SLAB = 4 / D;
+    static constexpr uint32_t CBIAS = D == 1 ? 0x80u : D == 2 ? 0x8080u : 0x80808080u;
+};
 constexpr int PACK_THREADS = 256;
 constexpr uint32_t MAX_KSPLIT = 16;
 
 struct Layout {
-    uint64_t Mp, Np, KB, ksplit;
+    uint64_t Mp, Np, KB, slabs, ksplit; // KB: k-blocks of 32, padded to whole slabs
     size_t planes_a, planes_b, sums_a, sums_b, total; // byte offsets into the workspace
 };
 
-Layout make_layout(uint64_t M, uint64_t N, uint64_t K) {
+Layout make_layout(int digits, uint64_t M, uint64_t N, uint64_t K) {
     Layout w;
+    const uint64_t per_slab = 4 / digits;
     w.Mp = (M + TILE - 1) / TILE * TILE;
     w.Np = (N + TILE - 1) / TILE * TILE;
-    w.KB = (K + BK - 1) / BK;
+    w.KB = ((K + BK - 1) / BK + per_slab - 1) / per_slab * per_slab;
+    w.slabs = w.KB / per_slab;
     // enough work-groups in the pack launch to fill the chip: (Mp + Np) / 32 row blocks x ksplit
     uint64_t ks = 2048 / ((w.Mp + w.Np) / 32);
     ks = ks < 1 ? 1 : ks > MAX_KSPLIT ? MAX_KSPLIT : ks;
     if (ks > w.KB) ks = w.KB;
     w.ksplit = ks;
     w.planes_a = 0;
-    w.planes_b = w.planes_a + (size_t)w.Mp / 32 * w.KB * GROUP_BYTES;
-    w.sums_a = w.planes_b + (size_t)w.Np / 32 * w.KB * GROUP_BYTES;
+    w.planes_b = w.planes_a + (size_t)w.Mp / 32 * w.slabs * GROUP_BYTES;
+    w.sums_a = w.planes_b + (size_t)w.Np / 32 * w.slabs * GROUP_BYTES;
     w.sums_b = w.sums_a + (size_t)w.ksplit * w.Mp * 4;
     w.total = w.sums_b + (size_t)w.ksplit * w.Np * 4;
     return w;
@@ -65,6 +76,7 @@ Layout make_layout(uint64_t M, uint64_t N, uint64_t K) {
 
 // 4x4 byte transpose: e[t] = element at k+t (bytes = digits 0..3) -> p[d] = digit d of k+0..k+3, signed form
 __device__ __forceinline__ void digit_planes(const uint32_t e[4], uint32_t p[4]) {
+    constexpr uint32_t CBIAS = 0x80808080u;
     const uint32_t a = e[0] ^ CBIAS, b = e[1] ^ CBIAS, c = e[2] ^ CBIAS, d = e[3] ^ CBIAS;
     const uint32_t ab_lo = __builtin_amdgcn_perm(b, a, 0x05010400u), ab_hi = __builtin_amdgcn_perm(b, a, 0x07030602u);
     const uint32_t cd_lo = __builtin_amdgcn_perm(d, c, 0x05010400u), cd_hi = __builtin_amdgcn_perm(d, c, 0x07030602u);
@@ -74,8 +86,18 @@ __device__ __forceinline__ void digit_planes(const uint32_t e[4], uint32_t p[4])
     p[3] = __builtin_amdgcn_perm(cd_hi, ab_hi, 0x07060302u);
 }
 
+// the same for D = 1 or 2 digits: p[d] = byte d of the four (zero-extended) elements, signed form
+template <int D> __device__ __forceinline__ void digit_planes_narrow(const uint32_t e[4], uint32_t p[D]) {
+    constexpr uint32_t c = D == 1 ? 0x80u : 0x8080u;
+    const uint32_t a = e[0] ^ c, b = e[1] ^ c, cc = e[2] ^ c, d = e[3] ^ c;
+#pragma unroll
+    for (int i = 0; i < D; ++i)
+        p[i] = ((a >> (8 * i)) & 0xffu) | (((b >> (8 * i)) & 0xffu) << 8) | (((cc >> (8 * i)) & 0xffu) << 16) |
+               (((d >> (8 * i)) & 0xffu) << 24);
+}
+
 struct PackOperand {
-    const uint32_t *src;   // element (r, k) at src[r * ld + k] (k-contiguous) or src[k * ld + r]
+    const void *src;       // element (r, k) at src[r * ld + k] (k-contiguous) or src[k * ld + r]
     uint32_t ld, rows, row_blocks; // true rows; padded rows / 32
     unsigned char *planes;
     uint32_t *sums;        // [ksplit][row_blocks * 32]
@@ -88,10 +110,14 @@ struct PackArgs {
 
 // blockIdx.x: row block of A, then of B; blockIdx.y: k-range.  Wave w of the work-group takes the
 // k-blocks start + w, start + w + 4, ...; lane l the row l % 32 and the 16 k of half l / 32.
+template <typename E>
 __global__ __launch_bounds__(PACK_THREADS) void ipack_kernel(PackArgs g) {
+    constexpr int D = Digits<E>::D;
+    constexpr uint32_t CBIAS = Digits<E>::CBIAS;
     __shared__ uint32_t partial[PACK_THREADS];
     const int which = blockIdx.x >= g.op[0].row_blocks;
     const PackOperand &o = g.op[which];
+    const E *src = static_cast<const E *>(o.src);
     const uint32_t rb = blockIdx.x - (which ? g.op[0].row_blocks : 0u);
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, l32 = lane & 31, half = lane >> 5;
     const uint32_t row = rb * 32 + l32;
@@ -102,20 +128,23 @@ __global__ __launch_bounds__(PACK_THREADS) void ipack_kernel(PackArgs g) {
         const uint32_t k0 = kb * BK + 16 * half;
         uint32_t e[16];
         if (o.k_contiguous) {
-            const uint32_t *p = o.src + (size_t)row * o.ld + k0;
+            const E *p = src + (size_t)row * o.ld + k0;
             if (row_ok && o.vector_ok && k0 + 16 <= g.K) {
+                u32x4 vec[D];
 #pragma unroll
-                for (int q = 0; q < 4; ++q) {
-                    const u32x4 v = *reinterpret_cast<const u32x4 *>(p + 4 * q);
-                    e[4 * q] = v[0]; e[4 * q + 1] = v[1]; e[4 * q + 2] = v[2]; e[4 * q + 3] = v[3];
+                for (int q = 0; q < D; ++q) vec[q] = *reinterpret_cast<const u32x4 *>(reinterpret_cast<const unsigned char *>(p) + 16 * q);
+                E raw[16];
+                __builtin_memcpy(raw, vec, 16 * D);
+#pragma unroll
+                for (int j = 0; j < 16; ++j) {
+                    e[j] = raw[j];
+                    sum += e[j];
                 }
-#pragma unroll
-                for (int j = 0; j < 16; ++j) sum += e[j];
             } else {
 #pragma unroll
                 for (int j = 0; j < 16; ++j) {
                     const bool ok = row_ok && k0 + j < g.K;
-                    const uint32_t v = ok ? p[j] : 0u;
+                    const uint32_t v = ok ? (uint32_t)p[j] : 0u;
                     sum += v;
                     e[j] = ok ? v : CBIAS; // CBIAS has all-zero signed digits
                 }
@@ -124,22 +153,24 @@ __global__ __launch_bounds__(PACK_THREADS) void ipack_kernel(PackArgs g) {
 #pragma unroll
             for (int j = 0; j < 16; ++j) {
                 const bool ok = row_ok && k0 + j < g.K;
-                const uint32_t v = ok ? o.src[(size_t)(k0 + j) * o.ld + row] : 0u;
+                const uint32_t v = ok ? (uint32_t)src[(size_t)(k0 + j) * o.ld + row] : 0u;
                 sum += v;
                 e[j] = ok ? v : CBIAS;
             }
         }
-        u32x4 out[4];
+        u32x4 out[D];
 #pragma unroll
         for (int q = 0; q < 4; ++q) {
-            uint32_t p4[4];
-            digit_planes(e + 4 * q, p4);
+            uint32_t pd[D];
+            if constexpr (D == 4) digit_planes(e + 4 * q, pd);
+            else digit_planes_narrow<D>(e + 4 * q, pd);
 #pragma unroll
-            for (int d = 0; d < 4; ++d) out[d][q] = p4[d];
+            for (int d = 0; d < D; ++d) out[d][q] = pd[d];
         }
-        unsigned char *dst = o.planes + ((size_t)rb * g.KB + kb) * GROUP_BYTES + lane * 16;
+        // block (rb, kb, d) is the (kb * D + d)-th of its row block
+        unsigned char *dst = o.planes + ((size_t)rb * g.KB * D + (size_t)kb * D) * BLOCK_BYTES + lane * 16;
 #pragma unroll
-        for (int d = 0; d < 4; ++d) *reinterpret_cast<u32x4 *>(dst + d * BLOCK_BYTES) = out[d];
+        for (int d = 0; d < D; ++d) *reinterpret_cast<u32x4 *>(dst + d * BLOCK_BYTES) = out[d];
     }
     partial[tid] = sum;
     __syncthreads();
@@ -154,8 +185,8 @@ __global__ __launch_bounds__(PACK_THREADS) void ipack_kernel(PackArgs g) {
 struct PArgs {
     const unsigned char *planes_a, *planes_b;
     const uint32_t *sums_a, *sums_b;
-    uint32_t *C;
-    uint32_t M, N, K, KB, Mp, Np, ksplit, ldc, tiles_m, tiles_n;
+    void *C;
+    uint32_t M, N, K, slabs, Mp, Np, ksplit, ldc, tiles_m, tiles_n;
     int epi;
     uint32_t alpha, beta;
 };
@@ -173,10 +204,12 @@ template <int BM> struct PackedTile {
     static constexpr size_t LDS_BYTES = 2 * STAGE_BYTES + (BM + TILE) * sizeof(uint32_t);
 };
 
-template <int BM, bool EDGE>
+template <typename E, int BM, bool EDGE>
 __global__ __launch_bounds__(BM * 4) __attribute__((amdgpu_waves_per_eu(2)))
-void gemm_i32_packed_kernel(PArgs g) {
+void gemm_int_packed_kernel(PArgs g) {
     using TL = PackedTile<BM>;
+    constexpr int D = Digits<E>::D, KB_PER_SLAB = Digits<E>::KB_PER_SLAB;
+    constexpr uint32_t CBIAS = Digits<E>::CBIAS;
     constexpr int STAGE_BYTES = TL::STAGE_BYTES, PASSES = TL::PASSES, A_GROUPS = BM / 32;
     extern __shared__ __align__(16) unsigned char lds_raw[];
     unsigned char *stages = lds_raw;                                              // [2][STAGE_BYTES]
@@ -202,9 +235,9 @@ void gemm_i32_packed_kernel(PArgs g) {
         row_sum[tid] = s; // col_sum follows row_sum
     }
 
-    i32x16 acc[4][2];
+    i32x16 acc[D][2]; // one set per shift i + j
 #pragma unroll
-    for (int s = 0; s < 4; ++s)
+    for (int s = 0; s < D; ++s)
 #pragma unroll
         for (int b = 0; b < 2; ++b)
 #pragma unroll
@@ -221,9 +254,9 @@ void gemm_i32_packed_kernel(PArgs g) {
 #pragma unroll
     for (int i = 0; i < PASSES; ++i) {
         const int gi = TL::GROUPS_PER_PASS * i + grp; // < A_GROUPS: A row blocks, then B column blocks
-        const unsigned char *p = gi < A_GROUPS ? g.planes_a + (size_t)(tile_m * A_GROUPS + gi) * g.KB * GROUP_BYTES
-                                               : g.planes_b + (size_t)(tile_n * 4 + gi - A_GROUPS) * g.KB * GROUP_BYTES;
-        src[i] = __builtin_amdgcn_make_buffer_rsrc(const_cast<unsigned char *>(p), 0, (int)(g.KB * GROUP_BYTES), 0x00020000);
+        const unsigned char *p = gi < A_GROUPS ? g.planes_a + (size_t)(tile_m * A_GROUPS + gi) * g.slabs * GROUP_BYTES
+                                               : g.planes_b + (size_t)(tile_n * 4 + gi - A_GROUPS) * g.slabs * GROUP_BYTES;
+        src[i] = __builtin_amdgcn_make_buffer_rsrc(const_cast<unsigned char *>(p), 0, (int)(g.slabs * GROUP_BYTES), 0x00020000);
     }
     // Two register sets: the slab loaded in step kb is stored to LDS at the end of step kb + 1 and
     // used in step kb + 2, so a load has two slabs of matrix work to arrive.
@@ -231,7 +264,7 @@ void gemm_i32_packed_kernel(PArgs g) {
     // they are written, ahead of the matrix work)
     u32x4 staged[2][PASSES];
     auto gload = [&](u32x4 *dst, uint32_t kb) {
-        const int off = (int)(min(kb, g.KB - 1) * GROUP_BYTES);
+        const int off = (int)(min(kb, g.slabs - 1) * GROUP_BYTES);
 #pragma unroll
         for (int i = 0; i < PASSES; ++i) dst[i] = __builtin_amdgcn_raw_buffer_load_b128(src[i], within, off, 0);
         __builtin_amdgcn_sched_barrier(0);
@@ -244,27 +277,30 @@ void gemm_i32_packed_kernel(PArgs g) {
     auto compute = [&](int buf) {
         const unsigned char *sa = stages + buf * STAGE_BYTES + wm * GROUP_BYTES + lane * 16;
         const unsigned char *sb = stages + buf * STAGE_BYTES + (A_GROUPS + wn * 2) * GROUP_BYTES + lane * 16;
+        // the four blocks of a group: k-block f / D of the slab, digit f % D
         i32x4 a[4], b[2][4];
 #pragma unroll
-        for (int d = 0; d < 4; ++d) {
-            a[d] = *reinterpret_cast<const i32x4 *>(sa + d * BLOCK_BYTES);
-            b[0][d] = *reinterpret_cast<const i32x4 *>(sb + d * BLOCK_BYTES);
-            b[1][d] = *reinterpret_cast<const i32x4 *>(sb + GROUP_BYTES + d * BLOCK_BYTES);
+        for (int f = 0; f < 4; ++f) {
+            a[f] = *reinterpret_cast<const i32x4 *>(sa + f * BLOCK_BYTES);
+            b[0][f] = *reinterpret_cast<const i32x4 *>(sb + f * BLOCK_BYTES);
+            b[1][f] = *reinterpret_cast<const i32x4 *>(sb + GROUP_BYTES + f * BLOCK_BYTES);
         }
 #pragma unroll
-        for (int s = 0; s < 4; ++s)
+        for (int kbl = 0; kbl < KB_PER_SLAB; ++kbl)
 #pragma unroll
-            for (int i = 0; i <= s; ++i)
+            for (int s = 0; s < D; ++s)
 #pragma unroll
-                for (int blk = 0; blk < 2; ++blk)
-                    acc[s][blk] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a[i], b[blk][s - i], acc[s][blk], 0, 0, 0);
+                for (int i = 0; i <= s; ++i)
+#pragma unroll
+                    for (int blk = 0; blk < 2; ++blk)
+                        acc[s][blk] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a[kbl * D + i], b[blk][kbl * D + s - i], acc[s][blk], 0, 0, 0);
     };
     // one step: slab kb is in LDS stage `cur`, slab kb + 1 in flight in staged[other]
     auto step = [&](uint32_t kb, auto cur_tag) {
         constexpr int cur = decltype(cur_tag)::value;
         gload(staged[cur], kb + 2);
         compute(cur);
-        if (kb + 1 < g.KB) {
+        if (kb + 1 < g.slabs) {
             sstore(staged[cur ^ 1], cur ^ 1);
             __syncthreads();
         }
@@ -274,13 +310,15 @@ void gemm_i32_packed_kernel(PArgs g) {
     gload(staged[1], 1);
     sstore(staged[0], 0);
     __syncthreads();
-    for (uint32_t kb = 0; kb < g.KB; kb += 2) {
+    for (uint32_t kb = 0; kb < g.slabs; kb += 2) {
         step(kb, std::integral_constant<int, 0>{});
-        if (kb + 1 < g.KB) step(kb + 1, std::integral_constant<int, 1>{});
+        if (kb + 1 < g.slabs) step(kb + 1, std::integral_constant<int, 1>{});
     }
 
     // epilogue: register r of lane l is C[8*(r/4) + 4*(l/32) + r%4][l%32] of its 32x32 block
+    // (all of it modulo 2^32; the store keeps the low 8 * D bits, which is the product modulo 2^(8 D))
     const uint32_t kc2 = g.K * (CBIAS * CBIAS);
+    E *C = static_cast<E *>(g.C);
 #pragma unroll
     for (int blk = 0; blk < 2; ++blk) {
         const uint32_t lcol = wn * 64 + blk * 32 + l32, col = n0 + lcol;
@@ -291,25 +329,26 @@ void gemm_i32_packed_kernel(PArgs g) {
             for (int r = 0; r < 16; ++r) {
                 const uint32_t row = m0 + wm * 32 + 8 * (r / 4) + 4 * lhi + (r % 4);
                 const uint32_t rowc = EDGE ? min(row, g.M - 1) : row, colc = EDGE ? min(col, g.N - 1) : col;
-                old[r] = g.C[(size_t)rowc * g.ldc + colc];
+                old[r] = C[(size_t)rowc * g.ldc + colc];
             }
         }
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
             const uint32_t lrow = wm * 32 + 8 * (r / 4) + 4 * lhi + (r % 4), row = m0 + lrow;
-            uint32_t v = (uint32_t)acc[0][blk][r] + ((uint32_t)acc[1][blk][r] << 8) + ((uint32_t)acc[2][blk][r] << 16) +
-                         ((uint32_t)acc[3][blk][r] << 24);
+            uint32_t v = 0;
+#pragma unroll
+            for (int s = 0; s < D; ++s) v += (uint32_t)acc[s][blk][r] << (8 * s);
             v += CBIAS * (row_sum[lrow] + csum) - kc2;
             if (g.epi == EPI_ALPHA) v = g.alpha * v;
             else if (g.epi == EPI_ALPHA_BETA) v = g.alpha * v + g.beta * old[r];
-            if (!EDGE || ((row < g.M) & (col < g.N))) g.C[(size_t)row * g.ldc + col] = v;
+            if (!EDGE || ((row < g.M) & (col < g.N))) C[(size_t)row * g.ldc + col] = (E)v;
         }
     }
 }
 
-template <int BM, bool EDGE> int launch_packed(hipStream_t st, PArgs g) {
+template <typename E, int BM, bool EDGE> int launch_packed(hipStream_t st, PArgs g) {
     constexpr size_t lds = PackedTile<BM>::LDS_BYTES;
-    auto kern = gemm_i32_packed_kernel<BM, EDGE>;
+    auto kern = gemm_int_packed_kernel<E, BM, EDGE>;
     static const hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
                                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     if (attr != hipSuccess) { (void)hipGetLastError(); return hip_code(attr); }
@@ -318,39 +357,35 @@ template <int BM, bool EDGE> int launch_packed(hipStream_t st, PArgs g) {
     return launch_status();
 }
 
-} // namespace
-
-// 0: this problem cannot take the packed path (a group stream of KB * 4 KiB must fit the 31-bit extent
-// of a buffer resource, the dimensions 31 bits)
-size_t wk::gemm_i32_packed_workspace_bytes(uint64_t M, uint64_t N, uint64_t K) {
-    if (!M || !N || !K || M > 0x7fffffffull || N > 0x7fffffffull || K > (0x7fffffffull / GROUP_BYTES) * BK) return 0;
-    return make_layout(M, N, K).total;
+int digits_of(int dtype) {
+    switch (dtype) {
+    case WK_I8: case WK_U8: return 1;
+    case WK_I16: case WK_U16: return 2;
+    case WK_I32: case WK_U32: return 4;
+    default: return 0;
+    }
 }
 
-int wk::gemm_i32_packed_launch(hipStream_t st, const GemmProblem &p, void *workspace, size_t workspace_bytes) {
-    if (!gemm_i32_packed_workspace_bytes(p.M, p.N, p.K)) return WK_E_INVALID_VALUE;
-    const Layout w = make_layout(p.M, p.N, p.K);
-    if (!workspace || workspace_bytes < w.total || (reinterpret_cast<uintptr_t>(workspace) & 15u)) return WK_E_INVALID_VALUE;
-    unsigned char *ws = static_cast<unsigned char *>(workspace);
-
+template <typename E> int launch_typed(hipStream_t st, const GemmProblem &p, unsigned char *ws, const Layout &w) {
+    constexpr int D = Digits<E>::D;
     PackArgs pa;
     auto operand = [&](PackOperand &o, const void *src, uint64_t ld, uint64_t rows, uint64_t rows_p, bool kc, size_t planes,
                        size_t sums) {
-        o.src = static_cast<const uint32_t *>(src);
+        o.src = src;
         o.ld = (uint32_t)ld;
         o.rows = (uint32_t)rows;
         o.row_blocks = (uint32_t)(rows_p / 32);
         o.planes = ws + planes;
         o.sums = reinterpret_cast<uint32_t *>(ws + sums);
         o.k_contiguous = kc;
-        o.vector_ok = kc && ld % 4 == 0 && (reinterpret_cast<uintptr_t>(src) & 15u) == 0;
+        o.vector_ok = kc && (ld * D) % 16 == 0 && (reinterpret_cast<uintptr_t>(src) & 15u) == 0;
     };
     operand(pa.op[0], p.A, p.lda, p.M, w.Mp, !p.op_a, w.planes_a, w.sums_a); // A is k-contiguous for op N
     operand(pa.op[1], p.B, p.ldb, p.N, w.Np, p.op_b != 0, w.planes_b, w.sums_b); // B for op T
     pa.K = (uint32_t)p.K;
     pa.KB = (uint32_t)w.KB;
     pa.kb_per_split = (uint32_t)((w.KB + w.ksplit - 1) / w.ksplit);
-    hipLaunchKernelGGL(ipack_kernel, dim3((unsigned)((w.Mp + w.Np) / 32), (unsigned)w.ksplit), dim3(PACK_THREADS), 0, st, pa);
+    hipLaunchKernelGGL(ipack_kernel<E>, dim3((unsigned)((w.Mp + w.Np) / 32), (unsigned)w.ksplit), dim3(PACK_THREADS), 0, st, pa);
     int rc = launch_status();
     if (rc) return rc;
 
@@ -359,15 +394,39 @@ int wk::gemm_i32_packed_launch(hipStream_t st, const GemmProblem &p, void *works
     g.planes_b = ws + w.planes_b;
     g.sums_a = reinterpret_cast<const uint32_t *>(ws + w.sums_a);
     g.sums_b = reinterpret_cast<const uint32_t *>(ws + w.sums_b);
-    g.C = static_cast<uint32_t *>(p.C);
+    g.C = p.C;
     g.M = (uint32_t)p.M; g.N = (uint32_t)p.N; g.K = (uint32_t)p.K;
-    g.KB = (uint32_t)w.KB; g.Mp = (uint32_t)w.Mp; g.Np = (uint32_t)w.Np; g.ksplit = (uint32_t)w.ksplit;
+    g.slabs = (uint32_t)w.slabs; g.Mp = (uint32_t)w.Mp; g.Np = (uint32_t)w.Np; g.ksplit = (uint32_t)w.ksplit;
     g.ldc = (uint32_t)p.ldc;
     g.tiles_m = (uint32_t)(w.Mp / TILE);
     g.tiles_n = (uint32_t)(w.Np / TILE);
     g.epi = p.epi;
-    std::memcpy(&g.alpha, p.alpha, 4);
-    std::memcpy(&g.beta, p.beta, 4);
+    g.alpha = g.beta = 0;
+    std::memcpy(&g.alpha, p.alpha, D); // little-endian: zero-extended element
+    std::memcpy(&g.beta, p.beta, D);
     const bool edge = p.M % TILE != 0 || p.N % TILE != 0;
-    return edge ? launch_packed<128, true>(st, g) : launch_packed<128, false>(st, g);
+    return edge ? launch_packed<E, 128, true>(st, g) : launch_packed<E, 128, false>(st, g);
+}
+
+} // namespace
+
+// 0: this problem cannot take the packed path (not an 8/16/32-bit integer type; a group stream of
+// slabs * 4 KiB must fit the 31-bit extent of a buffer resource, the dimensions 31 bits)
+size_t wk::gemm_int_packed_workspace_bytes(int dtype, uint64_t M, uint64_t N, uint64_t K) {
+    const int digits = digits_of(dtype);
+    if (!digits || !M || !N || !K || M > 0x7fffffffull || N > 0x7fffffffull) return 0;
+    if (K > (0x7fffffffull / GROUP_BYTES - 1) * BK * (4 / digits)) return 0;
+    return make_layout(digits, M, N, K).total;
+}
+
+int wk::gemm_int_packed_launch(hipStream_t st, const GemmProblem &p, void *workspace, size_t workspace_bytes) {
+    const size_t need = gemm_int_packed_workspace_bytes(p.dtype, p.M, p.N, p.K);
+    if (!need || !workspace || workspace_bytes < need || (reinterpret_cast<uintptr_t>(workspace) & 15u)) return WK_E_INVALID_VALUE;
+    const Layout w = make_layout(digits_of(p.dtype), p.M, p.N, p.K);
+    unsigned char *ws = static_cast<unsigned char *>(workspace);
+    switch (digits_of(p.dtype)) {
+    case 1: return launch_typed<uint8_t>(st, p, ws, w);
+    case 2: return launch_typed<uint16_t>(st, p, ws, w);
+    default: return launch_typed<uint32_t>(st, p, ws, w);
+    }
 }

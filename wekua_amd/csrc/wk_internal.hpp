@@ -173,9 +173,9 @@ int gemm_mfma_launch(hipStream_t st, const GemmProblem &p, int variant);
 // i32 / u32 on the int8 matrix cores (wk_gemm_imfma.hip); reached through the variant table
 int gemm_i32_mfma_launch_64(hipStream_t st, const GemmProblem &p, bool edge);  // macro tile 64 x 128
 int gemm_i32_mfma_launch_128(hipStream_t st, const GemmProblem &p, bool edge); // macro tile 128 x 128
-// i32 / u32 with a pack pass into caller-provided workspace (wk_gemm_ipack.hip)
-size_t gemm_i32_packed_workspace_bytes(uint64_t M, uint64_t N, uint64_t K);
-int gemm_i32_packed_launch(hipStream_t st, const GemmProblem &p, void *workspace, size_t workspace_bytes);
+// 8/16/32-bit integers with a pack pass into caller-provided workspace (wk_gemm_ipack.hip)
+size_t gemm_int_packed_workspace_bytes(int dtype, uint64_t M, uint64_t N, uint64_t K); // 0: not applicable
+int gemm_int_packed_launch(hipStream_t st, const GemmProblem &p, void *workspace, size_t workspace_bytes);
 bool gemm_mfma_fuses(const GemmProblem &p, int variant); // variant can run p with the fused bias + activation epilogue
 int gemm_mfma_pick(const GemmProblem &p);        // -1: not applicable
 const char *gemm_mfma_variant_name(int variant); // nullptr past the end

@@ -26,8 +26,8 @@
 //   * Tensor rows are padded to 16 bytes (the per-lane load width of gfx950), not to an
 //     even vector count, row counts are not padded at all, and row pitches that are a
 //     multiple of 1 KiB and at least 16 KiB are skewed by 512 bytes to avoid channel aliasing;
-//   * PackedTensors holds device memory only for i32 / u32 (the signed-digit planes of the
-//     int8 matrix-core product, filled by a pack pass inside gemm); for every other type the
+//   * PackedTensors holds device memory only for the 8/16/32-bit integers (the signed-digit planes of
+//     the int8 matrix-core product, filled by a pack pass inside gemm); for every other type the
 //     HIP kernels tile straight from the row-major operands through LDS and pack() only validates.
 #pragma once
 
