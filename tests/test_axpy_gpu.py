@@ -161,3 +161,15 @@ def test_axpy_invalid_arguments(dev):
     assert lib.wk_axpy(dev.stream, 25, s3, p, 8, 16, p, 8, 16, None) == 9     # bad dtype
     assert lib.wk_axpy(dev.stream, 8, s3, None, 8, 16, p, 8, 16, None) == 1   # null
     buf.free()
+
+
+@pytest.mark.parametrize("shape", [(70001, 24), (66000, 2, 8), (3, 66001, 4)])
+def test_axpy_pitched_rows_beyond_grid_limits(dev, shape):
+    """More rows or slices than one grid dimension holds (65535): the pitched-row kernel walks the
+    rest in a loop."""
+    x = make_operand("f32", shape, 29)
+    y = make_operand("f32", shape, 30)
+    got = run_axpy(dev, "f32", x, 0.75, y, pitched="aligned")
+    assert np.array_equal(got, expect("f32", x, 0.75, y))
+    gi = run_axpy(dev, "i16", make_operand("i16", shape, 31), -3, make_operand("i16", shape, 32), pitched="aligned")
+    assert np.array_equal(gi, expect("i16", make_operand("i16", shape, 31), -3, make_operand("i16", shape, 32)))
