@@ -67,9 +67,23 @@ def build_host(verbose: bool = False) -> str:
     return LIB_HOST
 
 
+def build_example(verbose: bool = False) -> str:
+    """The C++ usage example of the host mirror (benchmark/gemm.zig's flow); built to keep it compiling."""
+    src = os.path.join(HOST, "example_gemm.cpp")
+    if not os.path.exists(src):
+        return ""
+    exe = os.path.join(OBJ, "example_gemm")
+    out = _run(["g++", "-O2", "-std=c++20", "-Wall", "-Wextra", "-I" + INCLUDE, "-I" + HOST, src, "-o", exe,
+                "-L" + PKG, "-lwekua_hip", "-Wl,-rpath," + PKG])
+    if verbose and out.strip():
+        print(out)
+    return exe
+
+
 def build_all(verbose: bool = False):
     build_hip(verbose)
     build_host(verbose)
+    build_example(verbose)
 
 
 if __name__ == "__main__":
