@@ -101,7 +101,7 @@ struct PackOperand {
     uint32_t ld, rows, row_blocks; // true rows; padded rows / 32
     unsigned char *planes;
     uint32_t *sums;        // [ksplit][row_blocks * 32]
-    uint32_t k_contiguous, vector_ok; // vector_ok: 16-byte loads along k are aligned
+    uint32_t k_contiguous, vector_ok; // vector_ok: 16-byte loads along the contiguous direction are aligned
 };
 struct PackArgs {
     PackOperand op[2];
@@ -115,6 +115,7 @@ __global__ __launch_bounds__(PACK_THREADS) void ipack_kernel(PackArgs g) {
     constexpr int D = Digits<E>::D;
     constexpr uint32_t CBIAS = Digits<E>::CBIAS;
     __shared__ uint32_t partial[PACK_THREADS];
+    __shared__ __align__(16) unsigned char gather_tile[(PACK_THREADS / 64) * 32 * (32 * (D < 4 ? D : 1) + 4)];
     const int which = blockIdx.x >= g.op[0].row_blocks;
     const PackOperand &o = g.op[which];
     const E *src = static_cast<const E *>(o.src);
@@ -149,6 +150,34 @@ __global__ __launch_bounds__(PACK_THREADS) void ipack_kernel(PackArgs g) {
                     e[j] = ok ? v : CBIAS; // CBIAS has all-zero signed digits
                 }
             }
+        } else if (D < 4 && o.vector_ok && rb * 32 + 32 <= o.rows && kb * BK + BK <= g.K) {
+            // Row-contiguous storage of a narrow type, block inside the operand: a lane gathering its
+            // 16 k from 16 rows would load one element at a time (32 * D bytes per row and wave
+            // instruction).  Instead the wave copies the 32 k-rows x 32 * D bytes of the block with
+            // 16-byte loads (2 D lanes per row), parks them in its own LDS tile and every lane picks
+            // its column out of that.  The tile is private to the wave: LDS executes a wave's
+            // instructions in order, the fences only pin the compiler.
+            constexpr int LANES_PER_ROW = 2 * D, ROWS_PER_LOAD = 64 / LANES_PER_ROW, PITCH = 32 * D + 4;
+            unsigned char *tile = gather_tile + wave * (32 * PITCH);
+            const int seg = lane % LANES_PER_ROW;
+            const unsigned char *base = reinterpret_cast<const unsigned char *>(src) + (size_t)rb * 32 * D + seg * 16;
+#pragma unroll
+            for (int q = 0; q < D; ++q) {
+                const int k = q * ROWS_PER_LOAD + lane / LANES_PER_ROW;
+                const u32x4 v = *reinterpret_cast<const u32x4 *>(base + (size_t)(kb * BK + k) * o.ld * D);
+                uint32_t *dst = reinterpret_cast<uint32_t *>(tile + k * PITCH + seg * 16);
+                dst[0] = v[0]; dst[1] = v[1]; dst[2] = v[2]; dst[3] = v[3];
+            }
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+            __builtin_amdgcn_wave_barrier();
+            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+#pragma unroll
+            for (int j = 0; j < 16; ++j) {
+                e[j] = *reinterpret_cast<const E *>(tile + (16 * half + j) * PITCH + l32 * D);
+                sum += e[j];
+            }
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+            __builtin_amdgcn_wave_barrier(); // the tile is overwritten by the next block
         } else {
 #pragma unroll
             for (int j = 0; j < 16; ++j) {
@@ -378,7 +407,8 @@ template <typename E> int launch_typed(hipStream_t st, const GemmProblem &p, uns
         o.planes = ws + planes;
         o.sums = reinterpret_cast<uint32_t *>(ws + sums);
         o.k_contiguous = kc;
-        o.vector_ok = kc && (ld * D) % 16 == 0 && (reinterpret_cast<uintptr_t>(src) & 15u) == 0;
+        // 16-byte loads along the contiguous direction (k, or for the narrow types also the rows) are aligned
+        o.vector_ok = (kc || D < 4) && (ld * D) % 16 == 0 && (reinterpret_cast<uintptr_t>(src) & 15u) == 0;
     };
     operand(pa.op[0], p.A, p.lda, p.M, w.Mp, !p.op_a, w.planes_a, w.sums_a); // A is k-contiguous for op N
     operand(pa.op[1], p.B, p.ldb, p.N, w.Np, p.op_b != 0, w.planes_b, w.sums_b); // B for op T
