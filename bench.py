@@ -151,7 +151,7 @@ def main():
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build uses one GPU; --gpus N with N > 1 is not supported "
-              "(the hot path has no cross-GPU exchange: see DESIGN.md on sharding)", file=sys.stderr)
+              "(GEMM and AXPY shard over GPUs without any exchange step: every GPU would run this same benchmark on its share)", file=sys.stderr)
         sys.exit(2)
 
     import wekua_amd as wk                # fails loudly if the native libraries are missing
