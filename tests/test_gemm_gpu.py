@@ -309,3 +309,26 @@ def test_narrow_integers_with_workspace_automatic(dev, dtype):
     want = oracle.gemm(dtype, 3, a, 0, b, 1, 5, c)
     assert np.array_equal(run_gemm(dev, dtype, 3, a, 0, b, 1, 5, c, packed=True), want)
     assert np.array_equal(run_gemm(dev, dtype, 3, a, 0, b, 1, 5, c), want)
+
+
+@pytest.mark.parametrize("dtype", ["f32", "f64", "i32", "u8", "i16"])
+def test_seeded_random_problems(dev, dtype):
+    """Sixty seeded random problems per type under the automatic kernel choice: shapes up to 400 (so
+    that every tile of the cost model and both bounds-checked flavours come up), random transposes,
+    option combinations and leading-dimension padding; the integer types also with a workspace."""
+    rng = np.random.default_rng({"f32": 1, "f64": 2, "i32": 3, "u8": 4, "i16": 5}[dtype])
+    integer = dtype[0] in "iu"
+    for case in range(60):
+        M, N, K = (int(v) for v in rng.integers(1, 401, 3))
+        if case % 5 == 0:
+            M, N, K = (M + 63) // 64 * 64, (N + 63) // 64 * 64, (K + 31) // 32 * 32    # tile-aligned: the unchecked kernels
+        op_a, op_b = int(rng.integers(0, 2)), int(rng.integers(0, 2))
+        mode = int(rng.integers(0, 4))
+        if integer:
+            alpha, beta = [(None, None), (3, None), (5, 7), (None, 1)][mode]
+        else:
+            alpha, beta = [(None, None), (2.0, None), (1.5, 0.5), (None, -0.25)][mode]
+        pad = int(rng.integers(0, 3)) * int(rng.integers(1, 9))
+        a_cols, b_cols = (M if op_a else K), (K if op_b else N)
+        kw = dict(lda=a_cols + pad, ldb=b_cols + pad, ldc=N + pad) if pad else {}
+        check(dev, dtype, M, N, K, op_a, op_b, alpha, beta, seed=1000 + case, packed=integer and case % 2 == 0, **kw)
