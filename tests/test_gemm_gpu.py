@@ -332,3 +332,33 @@ def test_seeded_random_problems(dev, dtype):
         a_cols, b_cols = (M if op_a else K), (K if op_b else N)
         kw = dict(lda=a_cols + pad, ldb=b_cols + pad, ldc=N + pad) if pad else {}
         check(dev, dtype, M, N, K, op_a, op_b, alpha, beta, seed=1000 + case, packed=integer and case % 2 == 0, **kw)
+
+
+@pytest.mark.parametrize("dtype", ["cf32", "cf64"])
+@pytest.mark.parametrize("op_a,op_b", OPS)
+def test_complex_float_through_the_real_matrix_cores(dev, dtype, op_a, op_b):
+    """cf32 / cf64 with a workspace: B is expanded to its real 2K x 2N form (alpha folded in),
+    transposed operands are turned first, beta scales C beforehand, and the product is the real
+    matrix-core kernel on (M, 2N, 2K).  Against the oracle to the float tolerance of the real types,
+    for every option combination, ragged shapes and padded leading dimensions."""
+    assert dev.lib.wk_gemm_force_variant(f"mfma_{dtype}_packed".encode()) == 0
+    try:
+        for (M, N, K) in [(5, 7, 3), (33, 17, 65), (64, 96, 48), (128, 128, 64), (130, 70, 200), (257, 129, 17)]:
+            for alpha, beta in [(None, None), ((2, 1), None), ((2, 1), (1, -1)), (None, (0.5, 0.25))]:
+                check(dev, dtype, M, N, K, op_a, op_b, alpha, beta, seed=71, packed=True)
+        check(dev, dtype, 70, 45, 33, op_a, op_b, (1.5, -0.5), (0.25, 2), seed=72, packed=True,
+              lda=(70 if op_a else 33) + 3, ldb=(33 if op_b else 45) + 5, ldc=45 + 7)
+    finally:
+        dev.lib.wk_gemm_force_variant(b"auto")
+
+
+def test_complex_float_nan_in_c_propagates_with_beta(dev):
+    """beta given: C_old is read and multiplied (so NaN propagates) also on the packed path."""
+    a, b, c = gemm_operands("cf32", 64, 64, 64, 0, 0, 5)
+    c[:] = np.nan
+    assert dev.lib.wk_gemm_force_variant(b"mfma_cf32_packed") == 0
+    try:
+        assert np.isnan(run_gemm(dev, "cf32", (1, 0), a, 0, b, 0, (0, 0), c, packed=True)).all()
+        assert np.isfinite(run_gemm(dev, "cf32", (1, 0), a, 0, b, 0, None, c, packed=True)).all()
+    finally:
+        dev.lib.wk_gemm_force_variant(b"auto")

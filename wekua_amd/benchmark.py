@@ -55,7 +55,8 @@ class Session:
         self.ctx.deinit()
 
     def tensor(self, dtype, host):
-        t = self.wk.Tensor.alloc(dtype, self.ctx, self.pipeline, host.shape)
+        shape = host.shape[:-1] if dtype.startswith("c") else host.shape   # complex: trailing (re, im) axis
+        t = self.wk.Tensor.alloc(dtype, self.ctx, self.pipeline, shape)
         self.wk.memory.readFromBuffer(self.pipeline, t, host)
         return t
 
@@ -85,9 +86,10 @@ def time_gemm(ses, dtype, M, N, K, op_a, op_b, alpha, beta, iters=10):
     """blas.gemm on tensors created by Tensor.alloc (so with the library's own row pitches)."""
     rd = raw.real_np_dtype(dtype)
     wk = ses.wk
-    A = ses.tensor(dtype, _operand(rd, (K, M) if op_a else (M, K), 1))
-    B = ses.tensor(dtype, _operand(rd, (N, K) if op_b else (K, N), 2))
-    C = ses.tensor(dtype, _operand(rd, (M, N), 3))
+    tail = (2,) if dtype.startswith("c") else ()
+    A = ses.tensor(dtype, _operand(rd, ((K, M) if op_a else (M, K)) + tail, 1))
+    B = ses.tensor(dtype, _operand(rd, ((N, K) if op_b else (K, N)) + tail, 2))
+    C = ses.tensor(dtype, _operand(rd, (M, N) + tail, 3))
     # as benchmark/gemm.zig:186-196 does: one GemmPackedTensors for the run, passed to every call
     packed = wk.GemmPackedTensors.init(ses.pipeline, C, K, True)
     ses.pipeline.waitAndCleanup()
@@ -117,11 +119,16 @@ def time_axpy(ses, dtype, n, iters=50):
 
 def cmd_gemm(ses, args):
     print(f"{'dtype':5s} {'n':>6s} {'op':2s} {'ms':>9s} {'TFLOP/s':>9s}  kernel")
+    cplx = args.dtype.startswith("c")
+    is_float = args.dtype.lstrip("c")[0] == "f"
+    alpha, beta = (1.5, 0.5) if is_float else (3, 2)
+    if cplx:
+        alpha, beta = (alpha, 0.5 if is_float else 1), (beta, 0.25 if is_float else -1)
+    ops = 8.0 if cplx else 2.0   # a complex multiply-add counted as four real ones
     for n in args.sizes:
         for op_a, op_b, name in OPS:
-            ms, variant = time_gemm(ses, args.dtype, n, n, n, op_a, op_b, 1.5 if args.dtype[0] == "f" else 3,
-                                    0.5 if args.dtype[0] == "f" else 2)
-            print(f"{args.dtype:5s} {n:6d} {name:2s} {ms:9.4f} {2.0 * n ** 3 / ms / 1e9:9.2f}  {variant}", flush=True)
+            ms, variant = time_gemm(ses, args.dtype, n, n, n, op_a, op_b, alpha, beta)
+            print(f"{args.dtype:5s} {n:6d} {name:2s} {ms:9.4f} {ops * n ** 3 / ms / 1e9:9.2f}  {variant}", flush=True)
 
 
 def cmd_axpy(ses, args):

@@ -18,6 +18,17 @@ const char *k_generic_name = "tile64";
 // indexed by dtype (WK_I8 .. WK_U32)
 const char *k_packed_names[6] = {"mfma_i8_packed", "mfma_u8_packed", "mfma_i16_packed", "mfma_u16_packed",
                                  "mfma_i32_packed", "mfma_u32_packed"};
+const char *k_complex_packed_names[2] = {"mfma_cf32_packed", "mfma_cf64_packed"};
+bool is_complex_float(int dtype) { return dtype == WK_CF32 || dtype == WK_CF64; }
+// Two to four extra launches over the operands.  Measured against the generic kernel on MI355X: 512^3
+// 4x faster (cf32 0.137 -> 0.034 ms), 1024^3 3.7x, 4096^3 1.8x; the launches alone cost ~15 us.
+bool complex_packed_pays(const GemmProblem &p) {
+    return p.M >= 64 && p.N >= 64 && p.K >= 64 && (double)p.M * (double)p.N * (double)p.K >= 1.6e7;
+}
+int transpose_for_gemm(void *ctx, int dtype, uint64_t rows, uint64_t cols, const void *src, uint64_t ld, void *dst) {
+    const uint64_t shape[2] = {rows, cols}, src_pitches[2] = {ld, 1}, dst_pitches[2] = {rows, 1};
+    return wk_transpose(static_cast<wk_stream *>(ctx), dtype, 2, shape, src_pitches, dst_pitches, 0, 1, src, dst);
+}
 
 bool is_int32(int dtype) { return dtype == WK_I32 || dtype == WK_U32; }
 bool has_packed_path(int dtype) { return dtype >= WK_I8 && dtype <= WK_U32; }
@@ -80,7 +91,9 @@ int choose(const GemmProblem &p) {
 extern "C" {
 
 size_t wk_gemm_workspace_bytes(int dtype, int, int, uint64_t M, uint64_t N, uint64_t K) {
-    if (!has_packed_path(dtype) || !M || !N || !K) return 0;
+    if (!M || !N || !K) return 0;
+    if (is_complex_float(dtype)) return gemm_complex_packed_workspace_bytes(dtype, M, N, K);
+    if (!has_packed_path(dtype)) return 0;
     return gemm_int_packed_workspace_bytes(dtype, M, N, K);
 }
 
@@ -100,6 +113,19 @@ int wk_gemm(wk_stream *s, int dtype, int op_a, int op_b, uint64_t M, uint64_t N,
         if (forced == -3 && !fits) return WK_E_INVALID_VALUE;
         if (fits && (forced == -3 || (forced == -2 && packed_pays(p))))
             return gemm_int_packed_launch(s->stream, p, workspace, workspace_bytes);
+    }
+    if (is_complex_float(dtype)) {
+        const int forced = g_forced.load(std::memory_order_relaxed);
+        const size_t need = gemm_complex_packed_workspace_bytes(dtype, M, N, K);
+        const bool fits = need && workspace && workspace_bytes >= need && (reinterpret_cast<uintptr_t>(workspace) & 15u) == 0;
+        if (forced == -3 && !fits) return WK_E_INVALID_VALUE;
+        if (fits && (forced == -3 || (forced == -2 && complex_packed_pays(p)))) {
+            GemmProblem real;
+            rc = gemm_complex_packed_prepare(s->stream, p, workspace, workspace_bytes, &transpose_for_gemm, s, real);
+            if (rc) return rc;
+            const int rv = gemm_mfma_pick(real);
+            return rv >= 0 ? gemm_mfma_launch(s->stream, real, rv) : gemm_generic_launch(s->stream, real);
+        }
     }
     const int v = choose(p);
     if (v >= 0) return gemm_mfma_launch(s->stream, p, v);
@@ -145,7 +171,17 @@ const char *wk_gemm_variant_with_workspace(int dtype, int op_a, int op_b, uint64
                                            uint64_t ldb, uint64_t ldc, const void *A, const void *B, const void *C,
                                            size_t workspace_bytes) {
     const char *plain = wk_gemm_variant(dtype, op_a, op_b, M, N, K, lda, ldb, ldc, A, B, C);
-    if (!has_packed_path(dtype) || !std::strcmp(plain, "invalid")) return plain;
+    if (!std::strcmp(plain, "invalid")) return plain;
+    if (is_complex_float(dtype)) {
+        const int forced = g_forced.load(std::memory_order_relaxed);
+        const size_t need = gemm_complex_packed_workspace_bytes(dtype, M, N, K);
+        const bool fits = need && workspace_bytes >= need;
+        GemmProblem q;
+        q.M = M; q.N = N; q.K = K;
+        if (forced == -3) return fits ? k_complex_packed_names[dtype == WK_CF64] : "invalid";
+        return fits && forced == -2 && complex_packed_pays(q) ? k_complex_packed_names[dtype == WK_CF64] : plain;
+    }
+    if (!has_packed_path(dtype)) return plain;
     const int forced = g_forced.load(std::memory_order_relaxed);
     const size_t need = gemm_int_packed_workspace_bytes(dtype, M, N, K);
     const bool fits = need && workspace_bytes >= need;
@@ -159,6 +195,8 @@ int wk_gemm_force_variant(const char *name) {
     if (!name || !std::strcmp(name, "auto")) { g_forced.store(-2); return WK_OK; }
     if (!std::strcmp(name, k_generic_name)) { g_forced.store(-1); return WK_OK; }
     for (const char *packed : k_packed_names)
+        if (!std::strcmp(name, packed)) { g_forced.store(-3); return WK_OK; }
+    for (const char *packed : k_complex_packed_names)
         if (!std::strcmp(name, packed)) { g_forced.store(-3); return WK_OK; }
     for (int v = 0; gemm_mfma_variant_name(v); ++v)
         if (!std::strcmp(name, gemm_mfma_variant_name(v))) { g_forced.store(v); return WK_OK; }
