@@ -172,6 +172,20 @@ int    wk_gemm(wk_stream *s, int dtype, int op_a, int op_b, uint64_t M, uint64_t
                const void *host_beta, void *C, uint64_t ldc, void *workspace, size_t workspace_bytes);
 size_t wk_gemm_workspace_bytes(int dtype, int op_a, int op_b, uint64_t M, uint64_t N, uint64_t K);
 
+/* wk_gemm for a caller whose op(B) has not changed since the previous call: the workspace still
+ * holds B's packed form (digit planes and column sums of an integer B; the real 2K x 2N form of a
+ * complex B, which has alpha folded in), so only A is packed again.  The reference packs both
+ * operands before every product (gemm.zig:713-719) although its callers' B is usually a weight
+ * matrix that changes once per step; this is the entry point behind blas.PackedTensors.keepB.
+ * The caller guarantees: the previous call that used this workspace was a wk_gemm or
+ * wk_gemm_packed_b_kept with the same dtype, op_b, M, N, K and B contents (for cf32 / cf64 also the
+ * same alpha, present or absent alike), and nothing else has written the workspace since.  A
+ * violated guarantee gives a wrong product, never an access outside the operands.  Problems that
+ * do not use the workspace run exactly as under wk_gemm. */
+int    wk_gemm_packed_b_kept(wk_stream *s, int dtype, int op_a, int op_b, uint64_t M, uint64_t N, uint64_t K,
+                             const void *host_alpha, const void *A, uint64_t lda, const void *B, uint64_t ldb,
+                             const void *host_beta, void *C, uint64_t ldc, void *workspace, size_t workspace_bytes);
+
 /* Name of the kernel variant wk_gemm() would launch for these arguments ("mfma_f32_256x128",
  * "tile64", ...).  For benchmarks and profiles; not part of the reference's surface. */
 const char *wk_gemm_variant(int dtype, int op_a, int op_b, uint64_t M, uint64_t N, uint64_t K,

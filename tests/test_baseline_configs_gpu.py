@@ -208,3 +208,56 @@ def test_config4_int32_large_with_packed_tensors(op_a, op_b):
     finally:
         pipeline.deinit()
         context.deinit()
+
+
+@pytest.mark.parametrize("dtype,shape", [("i8", (768, 640, 1024)), ("cf32", (256, 320, 256))])
+def test_packed_tensors_keep_b_across_calls(dtype, shape):
+    """GemmPackedTensors.keepB: B is packed by the first blas.gemm and stays packed while the same B
+    tensor comes back; a changed B shows only after invalidateB() (so the stale product in between is
+    the proof that the pack pass of B was skipped); another B tensor is packed without being asked."""
+    import wekua_amd as wk
+    from helpers import assert_gemm_close, gemm_operands
+    M, N, K = shape
+    a1, b1, c0 = gemm_operands(dtype, M, N, K, 0, 1, 61)
+    a2, b2, _ = gemm_operands(dtype, M, N, K, 0, 1, 62)
+    context = wk.Context.initFromDeviceType(wk.DeviceType.all)
+    pipeline = wk.Pipeline.init(context.command_queues[0])
+    try:
+        A = wk.Tensor.alloc(dtype, context, pipeline, (M, K))
+        B = wk.Tensor.alloc(dtype, context, pipeline, (N, K))
+        B_other = wk.Tensor.alloc(dtype, context, pipeline, (N, K))
+        C = wk.Tensor.alloc(dtype, context, pipeline, (M, N))
+        packed = wk.GemmPackedTensors.init(pipeline, C, K, True)
+        assert packed.workspace_bytes > 0
+        packed.keepB(True)
+
+        def product(b_tensor, a_host, b_host_expected):
+            wk.blas.gemm(pipeline, None, A, 0, b_tensor, 1, None, C, packed)
+            got = np.empty_like(c0)
+            wk.memory.writeToBuffer(pipeline, C, got)
+            pipeline.waitAndCleanup()
+            want = oracle.gemm(dtype, None, a_host, 0, b_host_expected, 1, None, c0)
+            assert_gemm_close(dtype, got, want, None, a_host, 0, b_host_expected, 1, None, c0, K, what=dtype)
+
+        wk.memory.readFromBuffer(pipeline, A, a1)
+        wk.memory.readFromBuffer(pipeline, B, b1)
+        wk.memory.readFromBuffer(pipeline, B_other, b2)
+        product(B, a1, b1)                       # packs A and B
+        wk.memory.readFromBuffer(pipeline, A, a2)
+        product(B, a2, b1)                       # packs A only
+        wk.memory.readFromBuffer(pipeline, B, b2)
+        product(B, a2, b1)                       # B changed behind the handle's back: still the kept form
+        packed.invalidateB()
+        product(B, a2, b2)
+        wk.memory.readFromBuffer(pipeline, B, b1)
+        product(B_other, a2, b2)                 # another tensor: packed afresh
+        product(B, a2, b1)                       # and back
+        packed.keepB(False)
+        wk.memory.readFromBuffer(pipeline, B, b2)
+        product(B, a2, b2)                       # off: every call packs both, as the reference does
+        packed.deinit(pipeline)
+        for t in (A, B, B_other, C):
+            t.release(pipeline)
+    finally:
+        pipeline.deinit()
+        context.deinit()

@@ -362,3 +362,62 @@ def test_complex_float_nan_in_c_propagates_with_beta(dev):
         assert np.isfinite(run_gemm(dev, "cf32", (1, 0), a, 0, b, 0, None, c, packed=True)).all()
     finally:
         dev.lib.wk_gemm_force_variant(b"auto")
+
+
+@pytest.mark.parametrize("dtype", ["i8", "u16", "i32", "cf32", "cf64"])
+@pytest.mark.parametrize("op_a,op_b", OPS)
+def test_packed_b_kept_across_calls(dev, dtype, op_a, op_b):
+    """wk_gemm_packed_b_kept: after one wk_gemm with a workspace, later calls with a new A pack only A.
+    To show that B's packed form in the workspace is what the product reads, B's own buffer is
+    overwritten with other values before the second call: the result must still be the product
+    with the first B.  A third, ordinary wk_gemm then sees the new B."""
+    from wekua_amd import raw
+    forced = f"mfma_{dtype}_packed".encode()
+    assert dev.lib.wk_gemm_force_variant(forced) == 0
+    try:
+        for (M, N, K), alpha, beta in [((128, 128, 64), None, None), ((130, 70, 200), (2, 1) if dtype.startswith("c") else 3, None),
+                                       ((65, 129, 33), (1.5, -0.5) if dtype.startswith("c") else 2,
+                                        (0.25, 2) if dtype.startswith("c") else 5)]:
+            a1, b1, c0 = gemm_operands(dtype, M, N, K, op_a, op_b, 81)
+            a2, b2, _ = gemm_operands(dtype, M, N, K, op_a, op_b, 82)
+            dA, dB, dC = dev.upload(a1), dev.upload(b1), dev.upload(c0)
+            need = dev.lib.wk_gemm_workspace_bytes(raw.dtype_id(dtype), op_a, op_b, M, N, K)
+            ws = dev.upload(np.full(need, 0x5a, dtype=np.uint8))
+            lda, ldb = a1.shape[1], b1.shape[1]
+
+            def product(a, b, b_kept):
+                dC.write(c0)
+                dev.gemm(dtype, op_a, op_b, M, N, K, alpha, dA, lda, dB, ldb, beta, dC, N, workspace=ws, b_kept=b_kept)
+                dev.sync()
+                got = dC.download(c0.dtype, c0.shape)
+                want = oracle.gemm(dtype, alpha, a, op_a, b, op_b, beta, c0)
+                assert_gemm_close(dtype, got, want, alpha, a, op_a, b, op_b, beta, c0, K,
+                                  what=f"{dtype} {M}x{N}x{K} op=({op_a},{op_b}) b_kept={b_kept}")
+
+            product(a1, b1, False)
+            dA.write(a2)
+            dB.write(b2)                    # B's buffer changes; its packed form in the workspace does not
+            product(a2, b1, True)
+            dA.write(a1)
+            product(a1, b1, True)           # and again, A back to the first
+            product(a1, b2, False)          # an ordinary call packs the new B
+            dA.write(a2)
+            product(a2, b2, True)
+            for d in (dA, dB, dC, ws):
+                d.free()
+    finally:
+        dev.lib.wk_gemm_force_variant(b"auto")
+
+
+def test_packed_b_kept_is_plain_gemm_without_a_workspace_path(dev):
+    """Types and sizes that do not use the workspace: the entry point is wk_gemm."""
+    for dtype, (M, N, K) in [("f32", (130, 70, 200)), ("i64", (33, 17, 65)), ("i32", (64, 64, 64))]:
+        a, b, c = gemm_operands(dtype, M, N, K, 0, 1, 83)
+        dA, dB, dC = dev.upload(a), dev.upload(b), dev.upload(c)
+        dev.gemm(dtype, 0, 1, M, N, K, None, dA, K, dB, K, None, dC, N, b_kept=True)
+        dev.sync()
+        got = dC.download(c.dtype, c.shape)
+        want = oracle.semantic_gemm(dtype, None, a, 0, b, 1, None, c)
+        assert_gemm_close(dtype, got, want, None, a, 0, b, 1, None, c, K, what=dtype)
+        for d in (dA, dB, dC):
+            d.free()

@@ -81,6 +81,8 @@ HOST_SIGNATURES = {
     "wkz_packed_deinit": (ci, [vp, vp]),
     "wkz_packed_workspace_bytes": (ci, [vp, u64p]),
     "wkz_packed_pack": (ci, [vp, vp, vp, ci, vp, ci]),
+    "wkz_packed_keep_b": (ci, [vp, ci]),
+    "wkz_packed_invalidate_b": (ci, [vp]),
     "wkz_gemm": (ci, [vp, vp, vp, ci, vp, ci, vp, vp, vp]),
     # tensor support operations
     "wkz_memory_copy": (ci, [vp, vp, vp]),
@@ -404,8 +406,10 @@ class convertions:
 
 
 class GemmPackedTensors:
-    """blas.GemmPackedTensors (src/blas/gemm.zig:60-359).  Holds device memory only for i32 / u32:
-    the workspace of the library's pack pass (`workspace_bytes`)."""
+    """blas.GemmPackedTensors (src/blas/gemm.zig:60-359).  Holds device memory only for the types
+    whose gemm has a pack pass (8/16/32-bit integers, cf32, cf64): its workspace (`workspace_bytes`).
+    keepB / invalidateB have no counterpart in the reference, which packs both operands on every
+    call: they let a constant B (weights) stay packed across calls."""
 
     def __init__(self, handle, dtype):
         self._h = handle
@@ -437,6 +441,14 @@ class GemmPackedTensors:
         if self._h:
             _check(_lib().wkz_packed_deinit(self._h, pipeline._h), "GemmPackedTensors.deinit")
             self._h = None
+
+    def keepB(self, on: bool) -> None:
+        """While on, gemm calls after the first with the same B tensor, op_b, pipeline queue and alpha
+        skip B's pack pass; call invalidateB() after B's contents change."""
+        _check(_lib().wkz_packed_keep_b(self._h, int(on)), "GemmPackedTensors.keepB")
+
+    def invalidateB(self) -> None:
+        _check(_lib().wkz_packed_invalidate_b(self._h), "GemmPackedTensors.invalidateB")
 
     def pack(self, pipeline: Pipeline, a: Tensor, op_a: int, b: Tensor, op_b: int) -> None:
         _check(_lib().wkz_packed_pack(self._h, pipeline._h, a._h, int(op_a), b._h, int(op_b)), "GemmPackedTensors.pack")

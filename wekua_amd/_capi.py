@@ -62,6 +62,7 @@ SIGNATURES = {
     "wk_identity": (ci, [vp, ci, vp, u64, u64]),
     "wk_axpy": (ci, [vp, ci, u64p, vp, u64, u64, vp, u64, u64, vp]),
     "wk_gemm": (ci, [vp, ci, ci, ci, u64, u64, u64, vp, vp, u64, vp, u64, vp, vp, u64, vp, sz]),
+    "wk_gemm_packed_b_kept": (ci, [vp, ci, ci, ci, u64, u64, u64, vp, vp, u64, vp, u64, vp, vp, u64, vp, sz]),
     "wk_gemm_workspace_bytes": (sz, [ci, ci, ci, u64, u64, u64]),
     "wk_gemm_variant": (ctypes.c_char_p, [ci, ci, ci, u64, u64, u64, u64, u64, u64, vp, vp, vp]),
     "wk_gemm_variant_with_workspace": (ctypes.c_char_p, [ci, ci, ci, u64, u64, u64, u64, u64, u64, vp, vp, vp, sz]),

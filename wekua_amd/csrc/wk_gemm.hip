@@ -97,15 +97,16 @@ size_t wk_gemm_workspace_bytes(int dtype, int, int, uint64_t M, uint64_t N, uint
     return gemm_int_packed_workspace_bytes(dtype, M, N, K);
 }
 
-int wk_gemm(wk_stream *s, int dtype, int op_a, int op_b, uint64_t M, uint64_t N, uint64_t K, const void *host_alpha,
-            const void *A, uint64_t lda, const void *B, uint64_t ldb, const void *host_beta, void *C, uint64_t ldc,
-            void *workspace, size_t workspace_bytes) {
+static int gemm_entry(wk_stream *s, int dtype, int op_a, int op_b, uint64_t M, uint64_t N, uint64_t K, const void *host_alpha,
+                      const void *A, uint64_t lda, const void *B, uint64_t ldb, const void *host_beta, void *C, uint64_t ldc,
+                      void *workspace, size_t workspace_bytes, bool reuse_b) {
     int rc = bind(s);
     if (rc) return rc;
     GemmProblem p;
     rc = build_problem(p, dtype, op_a, op_b, M, N, K, host_alpha, A, lda, B, ldb, host_beta, C, ldc);
     if (rc) return rc;
     p.num_cus = (uint32_t)s->dev->props.multiProcessorCount;
+    p.reuse_b = reuse_b;
     if (has_packed_path(dtype)) {
         const int forced = g_forced.load(std::memory_order_relaxed);
         const size_t need = gemm_int_packed_workspace_bytes(dtype, M, N, K);
@@ -130,6 +131,20 @@ int wk_gemm(wk_stream *s, int dtype, int op_a, int op_b, uint64_t M, uint64_t N,
     const int v = choose(p);
     if (v >= 0) return gemm_mfma_launch(s->stream, p, v);
     return gemm_generic_launch(s->stream, p);
+}
+
+int wk_gemm(wk_stream *s, int dtype, int op_a, int op_b, uint64_t M, uint64_t N, uint64_t K, const void *host_alpha,
+            const void *A, uint64_t lda, const void *B, uint64_t ldb, const void *host_beta, void *C, uint64_t ldc,
+            void *workspace, size_t workspace_bytes) {
+    return gemm_entry(s, dtype, op_a, op_b, M, N, K, host_alpha, A, lda, B, ldb, host_beta, C, ldc, workspace, workspace_bytes,
+                      false);
+}
+
+int wk_gemm_packed_b_kept(wk_stream *s, int dtype, int op_a, int op_b, uint64_t M, uint64_t N, uint64_t K,
+                          const void *host_alpha, const void *A, uint64_t lda, const void *B, uint64_t ldb, const void *host_beta,
+                          void *C, uint64_t ldc, void *workspace, size_t workspace_bytes) {
+    return gemm_entry(s, dtype, op_a, op_b, M, N, K, host_alpha, A, lda, B, ldb, host_beta, C, ldc, workspace, workspace_bytes,
+                      true);
 }
 
 int wk_gemm_bias_activation(wk_stream *s, int dtype, int op_a, int op_b, uint64_t M, uint64_t N, uint64_t K, const void *A,

@@ -68,9 +68,12 @@ int prepare(hipStream_t st, const GemmProblem &p, const void *b_src, uint64_t ld
     std::memcpy(alpha, p.alpha, sizeof alpha);
     std::memcpy(beta, p.beta, sizeof beta);
     const bool has_alpha = p.epi != EPI_STORE;
-    hipLaunchKernelGGL(expand_b_kernel<R>, dim3(grid_for(p.K * p.N)), dim3(CP_BLOCK), 0, st, static_cast<const R *>(b_src), ldb, p.K,
-                       p.N, static_cast<R *>(bx), has_alpha, alpha[0], alpha[1]);
-    int rc = launch_status();
+    int rc = WK_OK;
+    if (!p.reuse_b) {
+        hipLaunchKernelGGL(expand_b_kernel<R>, dim3(grid_for(p.K * p.N)), dim3(CP_BLOCK), 0, st, static_cast<const R *>(b_src), ldb,
+                           p.K, p.N, static_cast<R *>(bx), has_alpha, alpha[0], alpha[1]);
+        rc = launch_status();
+    }
     if (rc || p.epi != EPI_ALPHA_BETA) return rc;
     hipLaunchKernelGGL(cscale_kernel<R>, dim3(grid_for(p.M * p.N)), dim3(CP_BLOCK), 0, st, static_cast<R *>(p.C), p.ldc, p.M, p.N,
                        beta[0], beta[1]);
@@ -109,7 +112,7 @@ int wk::gemm_complex_packed_prepare(hipStream_t st, const GemmProblem &p, void *
     }
     const void *b_src = p.B;
     uint64_t ldb = p.ldb;
-    if (p.op_b) { // stored N x K
+    if (p.op_b && !p.reuse_b) { // stored N x K
         const int rc = transpose(ctx, p.dtype, p.N, p.K, p.B, p.ldb, bt);
         if (rc) return rc;
         b_src = bt;

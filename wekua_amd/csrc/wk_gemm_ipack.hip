@@ -415,7 +415,10 @@ template <typename E> int launch_typed(hipStream_t st, const GemmProblem &p, uns
     pa.K = (uint32_t)p.K;
     pa.KB = (uint32_t)w.KB;
     pa.kb_per_split = (uint32_t)((w.KB + w.ksplit - 1) / w.ksplit);
-    hipLaunchKernelGGL(ipack_kernel<E>, dim3((unsigned)((w.Mp + w.Np) / 32), (unsigned)w.ksplit), dim3(PACK_THREADS), 0, st, pa);
+    // A's row blocks come first in the grid: with B's planes and column sums kept from the previous
+    // call only those are launched
+    const uint64_t row_blocks = (p.reuse_b ? w.Mp : w.Mp + w.Np) / 32;
+    hipLaunchKernelGGL(ipack_kernel<E>, dim3((unsigned)row_blocks, (unsigned)w.ksplit), dim3(PACK_THREADS), 0, st, pa);
     int rc = launch_status();
     if (rc) return rc;
 

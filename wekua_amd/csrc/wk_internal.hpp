@@ -164,6 +164,8 @@ struct GemmProblem {
     bool ext = false;
     const void *ext_bias = nullptr;   // N elements of dtype, or null
     int ext_act = -1;                 // WK_ACT_*
+    // the workspace still holds op(B)'s packed form from the previous call (wk_gemm_packed_b_kept)
+    bool reuse_b = false;
 };
 
 // generic LDS-tiled VALU kernel, every dtype and shape (wk_gemm_generic.hip)

@@ -760,6 +760,33 @@ template <typename T> struct PackedTensors {
     wk_device *device = nullptr;
     void *workspace = nullptr;
     size_t workspace_bytes = 0;
+    // No counterpart in the reference, which packs both operands before every product
+    // (gemm.zig:713-719).  keepB(true) declares B a constant operand (weights): gemm calls after the
+    // first with the same B tensor, op_b, queue and alpha (alpha is folded into the packed B of the
+    // complex types) leave B's packed form in the workspace as it is and pack only A.  After B's
+    // contents change, invalidateB() makes the next call pack it again.
+    bool keep_b = false;
+    const Tensor<T> *kept_b = nullptr;
+    Operation kept_op_b = Operation::no_transpose;
+    const void *kept_stream = nullptr;
+    std::optional<T> kept_alpha;
+    void keepB(bool on) {
+        keep_b = on;
+        kept_b = nullptr;
+    }
+    void invalidateB() { kept_b = nullptr; }
+    // true when the workspace holds this B already; records the operand otherwise
+    bool holdsB(const Tensor<T> *b, Operation op_b, const void *stream, const std::optional<T> &alpha) {
+        if (!keep_b) return false;
+        const bool same_alpha = alpha.has_value() == kept_alpha.has_value() &&
+                                (!alpha || std::memcmp(&*alpha, &*kept_alpha, sizeof(T)) == 0);
+        if (kept_b == b && kept_op_b == op_b && kept_stream == stream && same_alpha) return true;
+        kept_b = b;
+        kept_op_b = op_b;
+        kept_stream = stream;
+        kept_alpha = alpha;
+        return false;
+    }
 
     static PackedTensors *init(Pipeline *pipeline, Tensor<T> *result_tensor, uint64_t k_size, bool vectors_enabled) {
         const auto &shape = result_tensor->dimensions.shape;
@@ -836,10 +863,13 @@ void gemm(Pipeline *pipeline, std::optional<T> alpha, Tensor<T> *a, Operation op
     const uint64_t M = c->dimensions.shape[0], N = c->dimensions.shape[1];
     const uint64_t K = a->dimensions.shape[op_a == Operation::transpose ? 0 : 1];
     const T av = alpha.value_or(T{}), bv = beta.value_or(T{});
-    check(wk_gemm(pipeline->command_queue->stream, core::getTypeIndex<T>(), (int)op_a, (int)op_b, M, N, K,
-                  alpha ? &av : nullptr, a->buffer, a->memory_layout.row_pitch, b->buffer, b->memory_layout.row_pitch,
-                  beta ? &bv : nullptr, c->buffer, c->memory_layout.row_pitch, packed_tensors ? packed_tensors->workspace : nullptr,
-                  packed_tensors ? packed_tensors->workspace_bytes : 0));
+    wk_stream *stream = pipeline->command_queue->stream;
+    const bool b_kept = packed_tensors && packed_tensors->holdsB(b, op_b, stream, alpha);
+    check((b_kept ? wk_gemm_packed_b_kept : wk_gemm)(
+        stream, core::getTypeIndex<T>(), (int)op_a, (int)op_b, M, N, K, alpha ? &av : nullptr, a->buffer,
+        a->memory_layout.row_pitch, b->buffer, b->memory_layout.row_pitch, beta ? &bv : nullptr, c->buffer,
+        c->memory_layout.row_pitch, packed_tensors ? packed_tensors->workspace : nullptr,
+        packed_tensors ? packed_tensors->workspace_bytes : 0));
     pipeline->append(1);
 }
 

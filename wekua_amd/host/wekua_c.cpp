@@ -400,6 +400,18 @@ int wkz_packed_workspace_bytes(void *packed, uint64_t *out) {
         dispatch(h->dtype, [&]<typename T>() { *out = static_cast<blas::PackedTensors<T> *>(h->packed)->workspace_bytes; });
     });
 }
+int wkz_packed_keep_b(void *packed, int on) {
+    return guard([&] {
+        PackedHandle *h = static_cast<PackedHandle *>(packed);
+        dispatch(h->dtype, [&]<typename T>() { static_cast<blas::PackedTensors<T> *>(h->packed)->keepB(on != 0); });
+    });
+}
+int wkz_packed_invalidate_b(void *packed) {
+    return guard([&] {
+        PackedHandle *h = static_cast<PackedHandle *>(packed);
+        dispatch(h->dtype, [&]<typename T>() { static_cast<blas::PackedTensors<T> *>(h->packed)->invalidateB(); });
+    });
+}
 int wkz_packed_pack(void *packed, void *pipeline, void *a, int op_a, void *b, int op_b) {
     return guard([&] {
         PackedHandle *h = static_cast<PackedHandle *>(packed);

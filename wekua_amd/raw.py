@@ -113,12 +113,15 @@ class Device:
 
     # -- the hot path ---------------------------------------------------------------------
     def gemm(self, dtype: str, op_a: int, op_b: int, M: int, N: int, K: int, alpha, A: "DeviceBuffer", lda: int,
-             B: "DeviceBuffer", ldb: int, beta, C: "DeviceBuffer", ldc: int, workspace: "DeviceBuffer | None" = None) -> None:
+             B: "DeviceBuffer", ldb: int, beta, C: "DeviceBuffer", ldc: int, workspace: "DeviceBuffer | None" = None,
+             b_kept: bool = False) -> None:
+        """wk_gemm; b_kept: wk_gemm_packed_b_kept (the workspace still holds B's packed form)."""
         a, b = scalar_bytes(dtype, alpha), scalar_bytes(dtype, beta)
-        check(self.lib.wk_gemm(self.stream, dtype_id(dtype), op_a, op_b, M, N, K,
-                               ctypes.cast(a, ctypes.c_void_p) if a is not None else None, A.ptr, lda, B.ptr, ldb,
-                               ctypes.cast(b, ctypes.c_void_p) if b is not None else None, C.ptr, ldc,
-                               workspace.ptr if workspace is not None else None, workspace.nbytes if workspace is not None else 0),
+        entry = self.lib.wk_gemm_packed_b_kept if b_kept else self.lib.wk_gemm
+        check(entry(self.stream, dtype_id(dtype), op_a, op_b, M, N, K,
+                    ctypes.cast(a, ctypes.c_void_p) if a is not None else None, A.ptr, lda, B.ptr, ldb,
+                    ctypes.cast(b, ctypes.c_void_p) if b is not None else None, C.ptr, ldc,
+                    workspace.ptr if workspace is not None else None, workspace.nbytes if workspace is not None else 0),
               "wk_gemm")
 
     def axpy(self, dtype: str, shape3, x: "DeviceBuffer", xrp: int, xsp: int, alpha, y: "DeviceBuffer", yrp: int,
