@@ -76,7 +76,8 @@ def test_float_small_shapes(dev, dtype, op_a, op_b, alpha, beta):
         check(dev, dtype, M, N, K, op_a, op_b, alpha, beta)
 
 
-@pytest.mark.parametrize("variant", ["tile64", "mfma_f32_64x64", "mfma_f32_128x128", "mfma_f32_256x128"])
+@pytest.mark.parametrize("variant", ["tile64", "mfma_f32_64x64", "mfma_f32_64x64s2", "mfma_f32_64x64s4", "mfma_f32_128x128",
+                                     "mfma_f32_256x128"])
 @pytest.mark.parametrize("op_a,op_b", OPS)
 def test_f32_every_variant(dev, variant, op_a, op_b):
     import ctypes
@@ -88,7 +89,7 @@ def test_f32_every_variant(dev, variant, op_a, op_b):
         dev.lib.wk_gemm_force_variant(b"auto")
 
 
-@pytest.mark.parametrize("variant", ["tile64", "mfma_f64_64x64", "mfma_f64_128x64", "mfma_f64_128x128"])
+@pytest.mark.parametrize("variant", ["tile64", "mfma_f64_64x64", "mfma_f64_64x64s2", "mfma_f64_128x64", "mfma_f64_128x128"])
 @pytest.mark.parametrize("op_a,op_b", OPS)
 def test_f64_every_variant(dev, variant, op_a, op_b):
     assert dev.lib.wk_gemm_force_variant(variant.encode()) == 0
@@ -243,8 +244,9 @@ def test_invalid_arguments(dev):
     buf.free()
 
 
-@pytest.mark.parametrize("dtype,variant", [("f32", "mfma_f32_64x64"), ("f32", "mfma_f32_128x128"), ("f32", "mfma_f32_256x128"),
-                                           ("f64", "mfma_f64_64x64"), ("f64", "mfma_f64_128x64"), ("f64", "mfma_f64_128x128")])
+@pytest.mark.parametrize("dtype,variant", [("f32", "mfma_f32_64x64"), ("f32", "mfma_f32_64x64s2"), ("f32", "mfma_f32_64x64s4"),
+                                           ("f32", "mfma_f32_128x128"), ("f32", "mfma_f32_256x128"),
+                                           ("f64", "mfma_f64_64x64"), ("f64", "mfma_f64_64x64s2"), ("f64", "mfma_f64_128x64"), ("f64", "mfma_f64_128x128")])
 def test_every_k_around_the_slab_boundaries(dev, dtype, variant):
     """Every K from 1 to 100 on a ragged tile and on a tile-aligned shape: the bounds-checked kernels
     choose per-flavour loops from the number of complete slabs (k-slab 16 or 32, one or two slabs of
@@ -258,8 +260,30 @@ def test_every_k_around_the_slab_boundaries(dev, dtype, variant):
                 check(dev, dtype, 256, 128, K, op_a, op_b, None, None, seed=300 + K)
                 check(dev, dtype, 130, 257, K, 1 - op_a, op_b, 2.0, None, seed=400 + K, lda=(130 if 1 - op_a else K) + 1,
                       ldb=(K if op_b else 257) + 3, ldc=257 + 5)
+        for K in (127, 128, 129, 191, 192, 193, 255, 256, 257, 320, 333):    # several slabs of 64 as well
+            op_a, op_b = K % 2, (K // 2) % 2
+            check(dev, dtype, 70, 45, K, op_a, op_b, 1.5, 0.5, seed=500 + K)
+            check(dev, dtype, 128, 192, K, 1 - op_a, op_b, None, None, seed=600 + K)
     finally:
         dev.lib.wk_gemm_force_variant(b"auto")
+
+
+def test_one_round_launches_take_the_k_split_tiles(dev):
+    """Launches of one round (f32: up to two) of the 64x64 tile with K >= 256 go to its k-split twins;
+    the automatic choice is checked by name and its result against the oracle, all four layouts."""
+    from wekua_amd import raw
+
+    def name(dtype, M, N, K):
+        return dev.lib.wk_gemm_variant(raw.dtype_id(dtype), 0, 0, M, N, K, K, N, N, None, None, None)
+    assert name("f32", 1024, 1024, 1024) == b"mfma_f32_64x64s4"     # the name query assumes 256 compute units
+    assert name("f32", 2048, 1024, 1024) == b"mfma_f32_64x64s2"
+    assert name("f32", 1024, 1024, 128) == b"mfma_f32_64x64"
+    assert name("f64", 1024, 1024, 1024) == b"mfma_f64_64x64s2"
+    assert name("f64", 2048, 2048, 2048) != b"mfma_f64_64x64s2"
+    for dtype in ("f32", "f64"):
+        for op_a, op_b in OPS:
+            check(dev, dtype, 1024, 960, 300, op_a, op_b, 1.5, 0.5, seed=93)
+            check(dev, dtype, 1000, 1000, 257, op_a, op_b, None, None, seed=94)
 
 
 @pytest.mark.parametrize("variant", ["mfma_i32_64x128", "mfma_i32_128x128", "mfma_i32_packed"])

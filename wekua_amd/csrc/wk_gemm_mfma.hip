@@ -107,24 +107,29 @@ template <int ROWS, int BK, bool KCONTIG> struct Slab {
     static constexpr int SIZE = KCONTIG ? ROWS * LD : BK * LD;
 };
 
-template <int BM, int BN, int BK, int WAVES_M, int WAVES_N, int OCC, bool A_K, bool B_K, bool EDGE, bool EXT = false>
-__global__ __launch_bounds__(WAVES_M *WAVES_N * 64) __attribute__((amdgpu_waves_per_eu(OCC)))
+// KS > 1: KS groups of WAVES_M x WAVES_N wavefronts share the macro tile and split every k-slab of
+// KS * BK values between them (group kg multiplies the k values kg * BK .. kg * BK + BK - 1 of the
+// slab); their accumulators are added through LDS before the epilogue.  For launches that put a
+// single small work-group on a CU this doubles the wavefronts a SIMD can switch between.
+template <int BM, int BN, int BK, int WAVES_M, int WAVES_N, int OCC, bool A_K, bool B_K, bool EDGE, bool EXT = false, int KS = 1>
+__global__ __launch_bounds__(WAVES_M *WAVES_N * 64 * KS) __attribute__((amdgpu_waves_per_eu(OCC)))
 void gemm_f32_mfma_kernel(MArgs<float> g) {
-    constexpr int NT = WAVES_M * WAVES_N * 64;
+    constexpr int NT = WAVES_M * WAVES_N * 64 * KS;
+    constexpr int BKT = BK * KS; // k values per LDS slab
     constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N;
     constexpr int FM = WM / 32, FN = WN / 32;
     static_assert(WM % 32 == 0 && WN % 32 == 0 && BK % 8 == 0, "tile shape");
-    using SA = Slab<BM, BK, A_K>;
-    using SB = Slab<BN, BK, B_K>;
-    constexpr int A_V4 = BM * BK / 4 / NT, B_V4 = BN * BK / 4 / NT; // 16-byte loads per thread per slab
-    static_assert(A_V4 * NT * 4 == BM * BK && B_V4 * NT * 4 == BN * BK, "slab must divide over the threads");
+    using SA = Slab<BM, BKT, A_K>;
+    using SB = Slab<BN, BKT, B_K>;
+    constexpr int A_V4 = BM * BKT / 4 / NT, B_V4 = BN * BKT / 4 / NT; // 16-byte loads per thread per slab
+    static_assert(A_V4 * NT * 4 == BM * BKT && B_V4 * NT * 4 == BN * BKT, "slab must divide over the threads");
 
     extern __shared__ __align__(16) float lds[];
     float *As = lds;                     // [2][SA::SIZE]
     float *Bs = lds + 2 * SA::SIZE;      // [2][SB::SIZE]
 
     const int tid = threadIdx.x;
-    const int lane = tid & 63, wave = tid >> 6;
+    const int lane = tid & 63, wave = (tid >> 6) % (WAVES_M * WAVES_N), kg = (tid >> 6) / (WAVES_M * WAVES_N);
     const int wm = wave / WAVES_N, wn = wave % WAVES_N;
     const int l32 = lane & 31, lhi = lane >> 5;
 
@@ -166,7 +171,7 @@ void gemm_f32_mfma_kernel(MArgs<float> g) {
             uint32_t r, c;     // r: index along the row-of-storage direction, c: first of 4 contiguous
             uint32_t r_lim, c_lim;
             if constexpr (KC) {
-                r = row0 + q / (BK / 4); c = k0 + 4 * (q % (BK / 4));
+                r = row0 + q / (BKT / 4); c = k0 + 4 * (q % (BKT / 4));
                 r_lim = row_lim; c_lim = g.K;
             } else {
                 r = k0 + q / (ROWS / 4); c = row0 + 4 * (q % (ROWS / 4));
@@ -204,12 +209,12 @@ void gemm_f32_mfma_kernel(MArgs<float> g) {
         constexpr int ROWS = decltype(rows_tag)::value;
         constexpr int NV = decltype(nv_tag)::value;
         constexpr bool FIX = decltype(fix_tag)::value;
-        constexpr int LD = Slab<ROWS, BK, KC>::LD;
+        constexpr int LD = Slab<ROWS, BKT, KC>::LD;
 #pragma unroll
         for (int i = 0; i < NV; ++i) {
             const int q = tid + i * NT;
             int off;
-            if constexpr (KC) off = (q / (BK / 4)) * LD + 4 * (q % (BK / 4));
+            if constexpr (KC) off = (q / (BKT / 4)) * LD + 4 * (q % (BKT / 4));
             else off = (q / (ROWS / 4)) * LD + 4 * (q % (ROWS / 4));
             f32x4 v = src[i];
             if constexpr (FIX) {
@@ -218,7 +223,7 @@ void gemm_f32_mfma_kernel(MArgs<float> g) {
                 asm volatile("" ::: "memory");
                 uint32_t r, c, r_lim, c_lim;
                 if constexpr (KC) {
-                    r = row0 + q / (BK / 4); c = k0 + 4 * (q % (BK / 4));
+                    r = row0 + q / (BKT / 4); c = k0 + 4 * (q % (BKT / 4));
                     r_lim = row_lim; c_lim = g.K;
                 } else {
                     r = k0 + q / (ROWS / 4); c = row0 + 4 * (q % (ROWS / 4));
@@ -246,7 +251,7 @@ void gemm_f32_mfma_kernel(MArgs<float> g) {
     // In the bounds-checked instantiation most work is still interior: a tile that lies inside C
     // needs checks only on the slab that holds the k tail.  The choice is uniform over the work-group.
     const bool tile_inside = !EDGE || (m0 + BM <= g.M && n0 + BN <= g.N);
-    const uint32_t k_inside = g.K - g.K % BK; // slabs starting below this are complete
+    const uint32_t k_inside = g.K - g.K % BKT; // slabs starting below this are complete
     // An edge tile away from the k tail needs less than the full treatment: rows and columns beyond
     // the matrix only feed entries of C that are never stored, so the clamped loads (which keep the
     // addresses inside the operand and deliver copies of valid data) can go to LDS as they are.  The
@@ -292,7 +297,7 @@ void gemm_f32_mfma_kernel(MArgs<float> g) {
     };
     using AnyFlavour = integral_constant<int, EDGE ? ANY : PLAIN>;
 
-    const uint32_t ktiles = (g.K + BK - 1) / BK;
+    const uint32_t ktiles = (g.K + BKT - 1) / BKT;
     constexpr int S = BK / 8; // fragment steps per k-slab (8 values of k each)
 
     // fragments of step s of LDS buffer `buf`: lane holds k = 8*s + 4*lhi + t, t = 0..3
@@ -302,26 +307,26 @@ void gemm_f32_mfma_kernel(MArgs<float> g) {
 #pragma unroll
         for (int i = 0; i < FM; ++i) {
             if constexpr (A_K) {
-                af[i] = *reinterpret_cast<const f32x4 *>(as + i * 32 * SA::LD + 8 * s + 4 * lhi);
+                af[i] = *reinterpret_cast<const f32x4 *>(as + i * 32 * SA::LD + kg * BK + 8 * s + 4 * lhi);
             } else {
 #pragma unroll
-                for (int t = 0; t < 4; ++t) af[i][t] = as[(8 * s + 4 * lhi + t) * SA::LD + i * 32];
+                for (int t = 0; t < 4; ++t) af[i][t] = as[(kg * BK + 8 * s + 4 * lhi + t) * SA::LD + i * 32];
             }
         }
 #pragma unroll
         for (int j = 0; j < FN; ++j) {
             if constexpr (B_K) {
-                bf[j] = *reinterpret_cast<const f32x4 *>(bs + j * 32 * SB::LD + 8 * s + 4 * lhi);
+                bf[j] = *reinterpret_cast<const f32x4 *>(bs + j * 32 * SB::LD + kg * BK + 8 * s + 4 * lhi);
             } else {
 #pragma unroll
-                for (int t = 0; t < 4; ++t) bf[j][t] = bs[(8 * s + 4 * lhi + t) * SB::LD + j * 32];
+                for (int t = 0; t < 4; ++t) bf[j][t] = bs[(kg * BK + 8 * s + 4 * lhi + t) * SB::LD + j * 32];
             }
         }
     };
 
     load_ab(0, ra[0], rb[0], AnyFlavour{});
     store_ab(0, 0, ra[0], rb[0], AnyFlavour{});
-    if (PF == 2 && ktiles > 1) load_ab(BK, ra[PF - 1], rb[PF - 1], AnyFlavour{});
+    if (PF == 2 && ktiles > 1) load_ab(BKT, ra[PF - 1], rb[PF - 1], AnyFlavour{});
     __syncthreads();
 
     // Fragment registers are double-buffered: the LDS reads for step s+1 are issued before the
@@ -363,13 +368,13 @@ void gemm_f32_mfma_kernel(MArgs<float> g) {
         for (uint32_t kt = 0; kt < ktiles; ++kt) {
             const int cur = kt & 1;
             const bool more = kt + 1 < ktiles;
-            if (more) load_ab((kt + 1) * BK, ra[0], rb[0], AnyFlavour{});
+            if (more) load_ab((kt + 1) * BKT, ra[0], rb[0], AnyFlavour{});
 #pragma unroll
             for (int s = 0; s < S; ++s) {
                 if (s + 1 < S) {
                     read_frags(cur, s + 1, af[(s + 1) & 1], bf[(s + 1) & 1]);
                 } else if (more) {
-                    store_ab(cur ^ 1, (kt + 1) * BK, ra[0], rb[0], AnyFlavour{});
+                    store_ab(cur ^ 1, (kt + 1) * BKT, ra[0], rb[0], AnyFlavour{});
                     __syncthreads();
                     read_frags(cur ^ 1, 0, af[(s + 1) & 1], bf[(s + 1) & 1]);
                 }
@@ -386,13 +391,13 @@ void gemm_f32_mfma_kernel(MArgs<float> g) {
         auto iteration = [&](uint32_t kt) {
             const int cur = kt & 1;
             const bool more = kt + 1 < ktiles;
-            if (more) load_ab((kt + 1) * BK, ra[0], rb[0], AnyFlavour{});
+            if (more) load_ab((kt + 1) * BKT, ra[0], rb[0], AnyFlavour{});
 #pragma unroll
             for (int s = 0; s < S; ++s) {
                 if (s + 1 < S) {
                     read_frags(cur, s + 1, af[(s + 1) & 1], bf[(s + 1) & 1]);
                 } else if (more) {
-                    store_ab(cur ^ 1, (kt + 1) * BK, ra[0], rb[0], AnyFlavour{});
+                    store_ab(cur ^ 1, (kt + 1) * BKT, ra[0], rb[0], AnyFlavour{});
                     __syncthreads();
                     read_frags(cur ^ 1, 0, af[(s + 1) & 1], bf[(s + 1) & 1]);
                 }
@@ -407,9 +412,9 @@ void gemm_f32_mfma_kernel(MArgs<float> g) {
             constexpr int P = decltype(parity_tag)::value;
             const int cur = kt & 1;
             if constexpr (PF == 1) {
-                load_ab((kt + 1) * BK, ra[0], rb[0], flavour_tag);
+                load_ab((kt + 1) * BKT, ra[0], rb[0], flavour_tag);
             } else {
-                if (kt + 2 < ktiles) load_ab((kt + 2) * BK, ra[P], rb[P], flavour_tag); // set P held slab kt, already in LDS
+                if (kt + 2 < ktiles) load_ab((kt + 2) * BKT, ra[P], rb[P], flavour_tag); // set P held slab kt, already in LDS
             }
             constexpr int NEXT = PF == 1 ? 0 : 1 - P; // the set holding slab kt+1
 #pragma unroll
@@ -418,7 +423,7 @@ void gemm_f32_mfma_kernel(MArgs<float> g) {
                     read_frags(cur, s + 1, af[(s + 1) & 1], bf[(s + 1) & 1]);
                 } else {
                     __builtin_amdgcn_sched_barrier(0);
-                    store_ab(cur ^ 1, (kt + 1) * BK, ra[NEXT], rb[NEXT], flavour_tag);
+                    store_ab(cur ^ 1, (kt + 1) * BKT, ra[NEXT], rb[NEXT], flavour_tag);
                     __syncthreads();
                     read_frags(cur ^ 1, 0, af[(s + 1) & 1], bf[(s + 1) & 1]);
                     __builtin_amdgcn_sched_barrier(0);
@@ -462,7 +467,7 @@ void gemm_f32_mfma_kernel(MArgs<float> g) {
         } else {
             // Iteration kt stores slab kt + 1 and requests slab kt + PF: the iterations before
             // `main_end` touch complete slabs only and run in a flavour fixed for the tile.
-            const bool has_tail = g.K % BK != 0;
+            const bool has_tail = g.K % BKT != 0;
             const uint32_t hand_overs = ktiles - 1;
             const uint32_t main_end = has_tail ? (hand_overs > (uint32_t)PF ? hand_overs - PF : 0u) : hand_overs;
             if (tile_inside) run(kt, main_end, integral_constant<int, PLAIN>{});
@@ -476,6 +481,33 @@ void gemm_f32_mfma_kernel(MArgs<float> g) {
                 if (s + 1 < S) read_frags(cur, s + 1, af[(s + 1) & 1], bf[(s + 1) & 1]);
                 mfma_step(s);
             }
+        }
+    }
+
+    if constexpr (KS > 1) {
+        // the groups' partial tiles meet in LDS (the slabs are done with): [group - 1][wave][i][j][r][lane]
+        static_assert((KS - 1) * BM * BN <= 2 * (SA::SIZE + SB::SIZE), "partial tiles must fit the slab buffers");
+        __syncthreads();
+        if (kg > 0) {
+            float *dst = lds + (size_t)((kg - 1) * WAVES_M * WAVES_N + wave) * FM * FN * 16 * 64 + lane;
+#pragma unroll
+            for (int i = 0; i < FM; ++i)
+#pragma unroll
+                for (int j = 0; j < FN; ++j)
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) dst[((i * FN + j) * 16 + r) * 64] = acc[i][j][r];
+        }
+        __syncthreads();
+        if (kg > 0) return;
+#pragma unroll
+        for (int q = 1; q < KS; ++q) {
+            const float *src = lds + (size_t)((q - 1) * WAVES_M * WAVES_N + wave) * FM * FN * 16 * 64 + lane;
+#pragma unroll
+            for (int i = 0; i < FM; ++i)
+#pragma unroll
+                for (int j = 0; j < FN; ++j)
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) acc[i][j][r] += src[((i * FN + j) * 16 + r) * 64];
         }
     }
 
@@ -528,24 +560,25 @@ template <int ROWS, int BK, bool KCONTIG> struct SlabD {
     static constexpr int SIZE = KCONTIG ? ROWS * LD : BK * LD;
 };
 
-template <int BM, int BN, int BK, int WAVES_M, int WAVES_N, int OCC, bool A_K, bool B_K, bool EDGE, bool EXT = false>
-__global__ __launch_bounds__(WAVES_M *WAVES_N * 64) __attribute__((amdgpu_waves_per_eu(OCC)))
+template <int BM, int BN, int BK, int WAVES_M, int WAVES_N, int OCC, bool A_K, bool B_K, bool EDGE, bool EXT = false, int KS = 1>
+__global__ __launch_bounds__(WAVES_M *WAVES_N * 64 * KS) __attribute__((amdgpu_waves_per_eu(OCC)))
 void gemm_f64_mfma_kernel(MArgs<double> g) {
-    constexpr int NT = WAVES_M * WAVES_N * 64;
+    constexpr int NT = WAVES_M * WAVES_N * 64 * KS; // KS groups of wavefronts split each slab, as in the f32 kernel
+    constexpr int BKT = BK * KS;
     constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N;
     constexpr int FM = WM / 16, FN = WN / 16;
     static_assert(WM % 16 == 0 && WN % 16 == 0 && BK % 8 == 0, "tile shape");
-    using SA = SlabD<BM, BK, A_K>;
-    using SB = SlabD<BN, BK, B_K>;
-    constexpr int A_V2 = BM * BK / 2 / NT, B_V2 = BN * BK / 2 / NT;
-    static_assert(A_V2 * NT * 2 == BM * BK && B_V2 * NT * 2 == BN * BK, "slab must divide over the threads");
+    using SA = SlabD<BM, BKT, A_K>;
+    using SB = SlabD<BN, BKT, B_K>;
+    constexpr int A_V2 = BM * BKT / 2 / NT, B_V2 = BN * BKT / 2 / NT;
+    static_assert(A_V2 * NT * 2 == BM * BKT && B_V2 * NT * 2 == BN * BKT, "slab must divide over the threads");
 
     extern __shared__ __align__(16) float lds[];
     double *As = reinterpret_cast<double *>(lds);
     double *Bs = As + 2 * SA::SIZE;
 
     const int tid = threadIdx.x;
-    const int lane = tid & 63, wave = tid >> 6;
+    const int lane = tid & 63, wave = (tid >> 6) % (WAVES_M * WAVES_N), kg = (tid >> 6) / (WAVES_M * WAVES_N);
     const int wm = wave / WAVES_N, wn = wave % WAVES_N;
     const int l16 = lane & 15, lq = lane >> 4; // lq = 0..3
 
@@ -578,7 +611,7 @@ void gemm_f64_mfma_kernel(MArgs<double> g) {
             const int q = tid + i * NT;
             uint32_t r, c, r_lim, c_lim;
             if constexpr (KC) {
-                r = row0 + q / (BK / 2); c = k0 + 2 * (q % (BK / 2));
+                r = row0 + q / (BKT / 2); c = k0 + 2 * (q % (BKT / 2));
                 r_lim = row_lim; c_lim = g.K;
             } else {
                 r = k0 + q / (ROWS / 2); c = row0 + 2 * (q % (ROWS / 2));
@@ -611,19 +644,19 @@ void gemm_f64_mfma_kernel(MArgs<double> g) {
         constexpr int ROWS = decltype(rows_tag)::value;
         constexpr int NV = decltype(nv_tag)::value;
         constexpr bool FIX = decltype(fix_tag)::value;
-        constexpr int LD = SlabD<ROWS, BK, KC>::LD;
+        constexpr int LD = SlabD<ROWS, BKT, KC>::LD;
 #pragma unroll
         for (int i = 0; i < NV; ++i) {
             const int q = tid + i * NT;
             int off;
-            if constexpr (KC) off = (q / (BK / 2)) * LD + 2 * (q % (BK / 2));
+            if constexpr (KC) off = (q / (BKT / 2)) * LD + 2 * (q % (BKT / 2));
             else off = (q / (ROWS / 2)) * LD + 2 * (q % (ROWS / 2));
             f64x2 v = src[i];
             if constexpr (FIX) {
                 asm volatile("" ::: "memory"); // as in the f32 kernel: keep this a branch, not selects
                 uint32_t r, c, r_lim, c_lim;
                 if constexpr (KC) {
-                    r = row0 + q / (BK / 2); c = k0 + 2 * (q % (BK / 2));
+                    r = row0 + q / (BKT / 2); c = k0 + 2 * (q % (BKT / 2));
                     r_lim = row_lim; c_lim = g.K;
                 } else {
                     r = k0 + q / (ROWS / 2); c = row0 + 2 * (q % (ROWS / 2));
@@ -646,7 +679,7 @@ void gemm_f64_mfma_kernel(MArgs<double> g) {
     using std::integral_constant;
     // interior tiles of the bounds-checked instantiation check only the slab with the k tail
     const bool tile_inside = !EDGE || (m0 + BM <= g.M && n0 + BN <= g.N);
-    const uint32_t k_inside = g.K - g.K % BK;
+    const uint32_t k_inside = g.K - g.K % BKT;
     // slab flavours as in the f32 kernel: PLAIN inside both operands, CLAMPED for complete slabs of an
     // edge tile (stored as loaded unless a 2-element vector straddles a row end), ANY decided per slab
     const bool fix_a_always = !A_K && g.M % 2 != 0, fix_b_always = !B_K && g.N % 2 != 0;
@@ -684,7 +717,7 @@ void gemm_f64_mfma_kernel(MArgs<double> g) {
     };
     using AnyFlavour = integral_constant<int, EDGE ? ANY : PLAIN>;
 
-    const uint32_t ktiles = (g.K + BK - 1) / BK;
+    const uint32_t ktiles = (g.K + BKT - 1) / BKT;
     constexpr int S = BK / 8;
 
     // fragments of step s: lane holds k = 8*s + 2*lq + t, t = 0..1 (two instructions per 8 k)
@@ -694,26 +727,26 @@ void gemm_f64_mfma_kernel(MArgs<double> g) {
 #pragma unroll
         for (int i = 0; i < FM; ++i) {
             if constexpr (A_K) {
-                af[i] = *reinterpret_cast<const f64x2 *>(as + i * 16 * SA::LD + 8 * s + 2 * lq);
+                af[i] = *reinterpret_cast<const f64x2 *>(as + i * 16 * SA::LD + kg * BK + 8 * s + 2 * lq);
             } else {
 #pragma unroll
-                for (int t = 0; t < 2; ++t) af[i][t] = as[(8 * s + 2 * lq + t) * SA::LD + i * 16];
+                for (int t = 0; t < 2; ++t) af[i][t] = as[(kg * BK + 8 * s + 2 * lq + t) * SA::LD + i * 16];
             }
         }
 #pragma unroll
         for (int j = 0; j < FN; ++j) {
             if constexpr (B_K) {
-                bf[j] = *reinterpret_cast<const f64x2 *>(bs + j * 16 * SB::LD + 8 * s + 2 * lq);
+                bf[j] = *reinterpret_cast<const f64x2 *>(bs + j * 16 * SB::LD + kg * BK + 8 * s + 2 * lq);
             } else {
 #pragma unroll
-                for (int t = 0; t < 2; ++t) bf[j][t] = bs[(8 * s + 2 * lq + t) * SB::LD + j * 16];
+                for (int t = 0; t < 2; ++t) bf[j][t] = bs[(kg * BK + 8 * s + 2 * lq + t) * SB::LD + j * 16];
             }
         }
     };
 
     load_ab(0, ra[0], rb[0], AnyFlavour{});
     store_ab(0, 0, ra[0], rb[0], AnyFlavour{});
-    if (PF == 2 && ktiles > 1) load_ab(BK, ra[PF - 1], rb[PF - 1], AnyFlavour{});
+    if (PF == 2 && ktiles > 1) load_ab(BKT, ra[PF - 1], rb[PF - 1], AnyFlavour{});
     __syncthreads();
 
     // Same schedule as the f32 kernel: double-buffered fragments, hand-over in front of the last
@@ -737,13 +770,13 @@ void gemm_f64_mfma_kernel(MArgs<double> g) {
         for (uint32_t kt = 0; kt < ktiles; ++kt) {
             const int cur = kt & 1;
             const bool more = kt + 1 < ktiles;
-            if (more) load_ab((kt + 1) * BK, ra[0], rb[0], AnyFlavour{});
+            if (more) load_ab((kt + 1) * BKT, ra[0], rb[0], AnyFlavour{});
 #pragma unroll
             for (int s = 0; s < S; ++s) {
                 if (s + 1 < S) {
                     read_frags(cur, s + 1, af[(s + 1) & 1], bf[(s + 1) & 1]);
                 } else if (more) {
-                    store_ab(cur ^ 1, (kt + 1) * BK, ra[0], rb[0], AnyFlavour{});
+                    store_ab(cur ^ 1, (kt + 1) * BKT, ra[0], rb[0], AnyFlavour{});
                     __syncthreads();
                     read_frags(cur ^ 1, 0, af[(s + 1) & 1], bf[(s + 1) & 1]);
                 }
@@ -762,9 +795,9 @@ void gemm_f64_mfma_kernel(MArgs<double> g) {
             constexpr int P = decltype(parity_tag)::value;
             const int cur = kt & 1;
             if constexpr (PF == 1) {
-                load_ab((kt + 1) * BK, ra[0], rb[0], flavour_tag);
+                load_ab((kt + 1) * BKT, ra[0], rb[0], flavour_tag);
             } else {
-                if (kt + 2 < ktiles) load_ab((kt + 2) * BK, ra[P], rb[P], flavour_tag);
+                if (kt + 2 < ktiles) load_ab((kt + 2) * BKT, ra[P], rb[P], flavour_tag);
             }
             constexpr int NEXT = PF == 1 ? 0 : 1 - P;
 #pragma unroll
@@ -773,7 +806,7 @@ void gemm_f64_mfma_kernel(MArgs<double> g) {
                     read_frags(cur, s + 1, af[(s + 1) & 1], bf[(s + 1) & 1]);
                 } else {
                     __builtin_amdgcn_sched_barrier(0);
-                    store_ab(cur ^ 1, (kt + 1) * BK, ra[NEXT], rb[NEXT], flavour_tag);
+                    store_ab(cur ^ 1, (kt + 1) * BKT, ra[NEXT], rb[NEXT], flavour_tag);
                     __syncthreads();
                     read_frags(cur ^ 1, 0, af[(s + 1) & 1], bf[(s + 1) & 1]);
                     __builtin_amdgcn_sched_barrier(0);
@@ -810,7 +843,7 @@ void gemm_f64_mfma_kernel(MArgs<double> g) {
                 ++kt;
             }
         } else {
-            const bool has_tail = g.K % BK != 0;
+            const bool has_tail = g.K % BKT != 0;
             const uint32_t hand_overs = ktiles - 1;
             const uint32_t main_end = has_tail ? (hand_overs > (uint32_t)PF ? hand_overs - PF : 0u) : hand_overs;
             if (tile_inside) run(kt, main_end, integral_constant<int, PLAIN>{});
@@ -822,6 +855,34 @@ void gemm_f64_mfma_kernel(MArgs<double> g) {
         for (int s = 0; s < S; ++s) {
             if (s + 1 < S) read_frags(cur, s + 1, af[(s + 1) & 1], bf[(s + 1) & 1]);
             mfma_step(s);
+        }
+    }
+
+    if constexpr (KS > 1) {
+        // partial tiles of the groups through LDS: [group - 1][wave][i][j][r][lane]
+        static_assert((KS - 1) * BM * BN <= 2 * (SA::SIZE + SB::SIZE), "partial tiles must fit the slab buffers");
+        double *red = reinterpret_cast<double *>(lds);
+        __syncthreads();
+        if (kg > 0) {
+            double *dst = red + (size_t)((kg - 1) * WAVES_M * WAVES_N + wave) * FM * FN * 4 * 64 + lane;
+#pragma unroll
+            for (int i = 0; i < FM; ++i)
+#pragma unroll
+                for (int j = 0; j < FN; ++j)
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) dst[((i * FN + j) * 4 + r) * 64] = acc[i][j][r];
+        }
+        __syncthreads();
+        if (kg > 0) return;
+#pragma unroll
+        for (int q = 1; q < KS; ++q) {
+            const double *src = red + (size_t)((q - 1) * WAVES_M * WAVES_N + wave) * FM * FN * 4 * 64 + lane;
+#pragma unroll
+            for (int i = 0; i < FM; ++i)
+#pragma unroll
+                for (int j = 0; j < FN; ++j)
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) acc[i][j][r] += src[((i * FN + j) * 4 + r) * 64];
         }
     }
 
@@ -894,28 +955,29 @@ template <typename K> int set_lds(K kernel, size_t bytes) {
     return WK_OK;
 }
 
-template <int BM, int BN, int BK, int WMS, int WNS, int OCC, bool AK, bool BKC, bool EDGE, bool EXT = false>
+template <int BM, int BN, int BK, int WMS, int WNS, int OCC, bool AK, bool BKC, bool EDGE, bool EXT = false, int KS = 1>
 int launch_f32_one(hipStream_t st, const GemmProblem &p) {
-    constexpr size_t lds = 2 * (Slab<BM, BK, AK>::SIZE + Slab<BN, BK, BKC>::SIZE) * sizeof(float);
-    auto kern = gemm_f32_mfma_kernel<BM, BN, BK, WMS, WNS, OCC, AK, BKC, EDGE, EXT>;
+    constexpr size_t lds = 2 * (Slab<BM, BK * KS, AK>::SIZE + Slab<BN, BK * KS, BKC>::SIZE) * sizeof(float);
+    auto kern = gemm_f32_mfma_kernel<BM, BN, BK, WMS, WNS, OCC, AK, BKC, EDGE, EXT, KS>;
     static int attr_rc = set_lds(kern, lds);
     if (attr_rc) return attr_rc;
     MArgs<float> g = make_args<float>(p, BM, BN);
-    hipLaunchKernelGGL(kern, dim3(g.tiles_m * g.tiles_n), dim3(WMS * WNS * 64), lds, st, g);
+    hipLaunchKernelGGL(kern, dim3(g.tiles_m * g.tiles_n), dim3(WMS * WNS * 64 * KS), lds, st, g);
     return launch_status();
 }
 
-template <int BM, int BN, int BK, int WMS, int WNS, int OCC>
+// BK: k values one group of wavefronts multiplies per slab; KS groups share a slab of BK * KS
+template <int BM, int BN, int BK, int WMS, int WNS, int OCC, int KS = 1>
 int launch_f32(hipStream_t st, const GemmProblem &p, bool edge) {
     const int sel = (p.op_a ? 0 : 2) | (p.op_b ? 1 : 0); // bit1: A k-contiguous, bit0: B k-contiguous
     if (p.ext) { // fused bias + activation: instantiated for op N, T only (see gemm_mfma_fuses)
         if (sel != 3) return WK_E_INVALID_VALUE;
-        return edge ? launch_f32_one<BM, BN, BK, WMS, WNS, OCC, true, true, true, true>(st, p)
-                    : launch_f32_one<BM, BN, BK, WMS, WNS, OCC, true, true, false, true>(st, p);
+        return edge ? launch_f32_one<BM, BN, BK, WMS, WNS, OCC, true, true, true, true, KS>(st, p)
+                    : launch_f32_one<BM, BN, BK, WMS, WNS, OCC, true, true, false, true, KS>(st, p);
     }
 #define WK_CASE(AK, BKC)                                                                                   \
-    return edge ? launch_f32_one<BM, BN, BK, WMS, WNS, OCC, AK, BKC, true>(st, p)                          \
-                : launch_f32_one<BM, BN, BK, WMS, WNS, OCC, AK, BKC, false>(st, p)
+    return edge ? launch_f32_one<BM, BN, BK, WMS, WNS, OCC, AK, BKC, true, false, KS>(st, p)                          \
+                : launch_f32_one<BM, BN, BK, WMS, WNS, OCC, AK, BKC, false, false, KS>(st, p)
     switch (sel) {
     case 0: WK_CASE(false, false);
     case 1: WK_CASE(false, true);
@@ -925,28 +987,28 @@ int launch_f32(hipStream_t st, const GemmProblem &p, bool edge) {
 #undef WK_CASE
 }
 
-template <int BM, int BN, int BK, int WMS, int WNS, int OCC, bool AK, bool BKC, bool EDGE, bool EXT = false>
+template <int BM, int BN, int BK, int WMS, int WNS, int OCC, bool AK, bool BKC, bool EDGE, bool EXT = false, int KS = 1>
 int launch_f64_one(hipStream_t st, const GemmProblem &p) {
-    constexpr size_t lds = 2 * (SlabD<BM, BK, AK>::SIZE + SlabD<BN, BK, BKC>::SIZE) * sizeof(double);
-    auto kern = gemm_f64_mfma_kernel<BM, BN, BK, WMS, WNS, OCC, AK, BKC, EDGE, EXT>;
+    constexpr size_t lds = 2 * (SlabD<BM, BK * KS, AK>::SIZE + SlabD<BN, BK * KS, BKC>::SIZE) * sizeof(double);
+    auto kern = gemm_f64_mfma_kernel<BM, BN, BK, WMS, WNS, OCC, AK, BKC, EDGE, EXT, KS>;
     static int attr_rc = set_lds(kern, lds);
     if (attr_rc) return attr_rc;
     MArgs<double> g = make_args<double>(p, BM, BN);
-    hipLaunchKernelGGL(kern, dim3(g.tiles_m * g.tiles_n), dim3(WMS * WNS * 64), lds, st, g);
+    hipLaunchKernelGGL(kern, dim3(g.tiles_m * g.tiles_n), dim3(WMS * WNS * 64 * KS), lds, st, g);
     return launch_status();
 }
 
-template <int BM, int BN, int BK, int WMS, int WNS, int OCC>
+template <int BM, int BN, int BK, int WMS, int WNS, int OCC, int KS = 1>
 int launch_f64(hipStream_t st, const GemmProblem &p, bool edge) {
     const int sel = (p.op_a ? 0 : 2) | (p.op_b ? 1 : 0);
     if (p.ext) {
         if (sel != 3) return WK_E_INVALID_VALUE;
-        return edge ? launch_f64_one<BM, BN, BK, WMS, WNS, OCC, true, true, true, true>(st, p)
-                    : launch_f64_one<BM, BN, BK, WMS, WNS, OCC, true, true, false, true>(st, p);
+        return edge ? launch_f64_one<BM, BN, BK, WMS, WNS, OCC, true, true, true, true, KS>(st, p)
+                    : launch_f64_one<BM, BN, BK, WMS, WNS, OCC, true, true, false, true, KS>(st, p);
     }
 #define WK_CASE(AK, BKC)                                                                                   \
-    return edge ? launch_f64_one<BM, BN, BK, WMS, WNS, OCC, AK, BKC, true>(st, p)                               \
-                : launch_f64_one<BM, BN, BK, WMS, WNS, OCC, AK, BKC, false>(st, p)
+    return edge ? launch_f64_one<BM, BN, BK, WMS, WNS, OCC, AK, BKC, true, false, KS>(st, p)                               \
+                : launch_f64_one<BM, BN, BK, WMS, WNS, OCC, AK, BKC, false, false, KS>(st, p)
     switch (sel) {
     case 0: WK_CASE(false, false);
     case 1: WK_CASE(false, true);
@@ -958,18 +1020,24 @@ int launch_f64(hipStream_t st, const GemmProblem &p, bool edge) {
 
 struct VariantDesc {
     const char *name;
-    int dtype, bm, bn, bk;
-    double efficiency; // fraction of the matrix peak this tile shape sustains over many rounds (0: never auto-selected)
+    int dtype, bm, bn, bk; // bk: k values per LDS slab
+    double efficiency; // fraction of the matrix peak this tile shape sustains over many rounds (0: never chosen by cost)
     double fill;       // start-up and drain of a launch, in units of one round of tiles
     int (*launch)(hipStream_t, const GemmProblem &, bool);
+    // k-split twins of this tile (more wavefronts per work-group, each slab shared between groups of
+    // them): the variant to take instead when the launch is one round of tiles / at most two
+    const char *one_round = nullptr, *two_rounds = nullptr;
 };
 
 const VariantDesc k_variants[] = {
     {"mfma_f32_256x128", WK_F32, 256, 128, 16, 0.943, 0.25, &launch_f32<256, 128, 16, 2, 2, 2>},
     {"mfma_f32_128x128", WK_F32, 128, 128, 16, 0.885, 0.25, &launch_f32<128, 128, 16, 2, 2, 3>},
-    {"mfma_f32_64x64", WK_F32, 64, 64, 32, 0.780, 0.10, &launch_f32<64, 64, 32, 2, 2, 4>},
+    {"mfma_f32_64x64", WK_F32, 64, 64, 32, 0.780, 0.10, &launch_f32<64, 64, 32, 2, 2, 4>, "mfma_f32_64x64s4", "mfma_f32_64x64s2"},
+    {"mfma_f32_64x64s2", WK_F32, 64, 64, 32, 0.0, 0.10, &launch_f32<64, 64, 16, 2, 2, 4, 2>}, // 2 groups x 16 k
+    {"mfma_f32_64x64s4", WK_F32, 64, 64, 64, 0.0, 0.10, &launch_f32<64, 64, 16, 2, 2, 4, 4>}, // 4 groups x 16 k
     {"mfma_f64_128x128", WK_F64, 128, 128, 16, 0.908, 0.20, &launch_f64<128, 128, 16, 2, 2, 2>},
-    {"mfma_f64_64x64", WK_F64, 64, 64, 32, 0.840, 0.05, &launch_f64<64, 64, 32, 2, 2, 2>},
+    {"mfma_f64_64x64", WK_F64, 64, 64, 32, 0.840, 0.05, &launch_f64<64, 64, 32, 2, 2, 2>, "mfma_f64_64x64s2", nullptr},
+    {"mfma_f64_64x64s2", WK_F64, 64, 64, 64, 0.0, 0.05, &launch_f64<64, 64, 32, 2, 2, 2, 2>}, // 2 groups x 32 k
     {"mfma_f64_128x64", WK_F64, 128, 64, 16, 0.863, 0.25, &launch_f64<128, 64, 16, 2, 2, 3>},
     // 32-bit integers through the int8 matrix cores (wk_gemm_imfma.hip); same kernel for both signs
     // (efficiency here is relative between the two integer tiles: 196-202 against 155-192 TOP/s)
@@ -1044,6 +1112,18 @@ int wk::gemm_mfma_pick(const GemmProblem &p) {
             best = v;
             best_cost = cost;
         }
+    }
+    // A launch of one round (f32: up to two) of the small tile leaves each SIMD one or two wavefronts,
+    // which stall together at every hand-over: the k-split twin of the tile gives it two to four.
+    // Measured on MI355X, f32: 1024^3 90.8 -> 101.8 TFLOP/s, 1000^3 64 -> 76, 1024x1024x4096 102 -> 119,
+    // 2048x1024x1024 (two rounds) 108 -> 113; f64: 1024^3 47 -> 53, 1000^3 36.6 -> 42.9.  From three
+    // rounds on, and for short k, the plain tile is as fast or faster.
+    if (best >= 0 && p.K >= 256) {
+        const VariantDesc &d = k_variants[best];
+        const double tiles = (double)((p.M + d.bm - 1) / d.bm) * (double)((p.N + d.bn - 1) / d.bn);
+        const char *twin = tiles <= cus ? d.one_round : (tiles <= 2.0 * cus ? d.two_rounds : nullptr);
+        for (int v = 0; twin && v < k_num_variants; ++v)
+            if (!std::strcmp(k_variants[v].name, twin)) return v;
     }
     return best;
 }
