@@ -76,8 +76,8 @@ def test_float_small_shapes(dev, dtype, op_a, op_b, alpha, beta):
         check(dev, dtype, M, N, K, op_a, op_b, alpha, beta)
 
 
-@pytest.mark.parametrize("variant", ["tile64", "mfma_f32_64x64", "mfma_f32_64x64s2", "mfma_f32_64x64s4", "mfma_f32_128x128",
-                                     "mfma_f32_256x128"])
+@pytest.mark.parametrize("variant", ["tile64", "mfma_f32_64x64", "mfma_f32_64x64s2", "mfma_f32_64x64s4", "mfma_f32_32x32s4",
+                                     "mfma_f32_128x128", "mfma_f32_256x128"])
 @pytest.mark.parametrize("op_a,op_b", OPS)
 def test_f32_every_variant(dev, variant, op_a, op_b):
     import ctypes
@@ -245,7 +245,7 @@ def test_invalid_arguments(dev):
 
 
 @pytest.mark.parametrize("dtype,variant", [("f32", "mfma_f32_64x64"), ("f32", "mfma_f32_64x64s2"), ("f32", "mfma_f32_64x64s4"),
-                                           ("f32", "mfma_f32_128x128"), ("f32", "mfma_f32_256x128"),
+                                           ("f32", "mfma_f32_32x32s4"), ("f32", "mfma_f32_128x128"), ("f32", "mfma_f32_256x128"),
                                            ("f64", "mfma_f64_64x64"), ("f64", "mfma_f64_64x64s2"), ("f64", "mfma_f64_128x64"), ("f64", "mfma_f64_128x128")])
 def test_every_k_around_the_slab_boundaries(dev, dtype, variant):
     """Every K from 1 to 100 on a ragged tile and on a tile-aligned shape: the bounds-checked kernels
@@ -278,12 +278,16 @@ def test_one_round_launches_take_the_k_split_tiles(dev):
     assert name("f32", 1024, 1024, 1024) == b"mfma_f32_64x64s4"     # the name query assumes 256 compute units
     assert name("f32", 2048, 1024, 1024) == b"mfma_f32_64x64s2"
     assert name("f32", 1024, 1024, 128) == b"mfma_f32_64x64"
+    assert name("f32", 512, 512, 512) == b"mfma_f32_32x32s4"       # 64 tiles of 64x64 would leave most CUs idle
+    assert name("f32", 768, 768, 768) == b"mfma_f32_32x32s4"
+    assert name("f32", 896, 896, 896) == b"mfma_f32_64x64s4"
     assert name("f64", 1024, 1024, 1024) == b"mfma_f64_64x64s2"
     assert name("f64", 2048, 2048, 2048) != b"mfma_f64_64x64s2"
     for dtype in ("f32", "f64"):
         for op_a, op_b in OPS:
             check(dev, dtype, 1024, 960, 300, op_a, op_b, 1.5, 0.5, seed=93)
             check(dev, dtype, 1000, 1000, 257, op_a, op_b, None, None, seed=94)
+            check(dev, dtype, 500, 333, 129, op_a, op_b, 2.0, None, seed=95)
 
 
 @pytest.mark.parametrize("variant", ["mfma_i32_64x128", "mfma_i32_128x128", "mfma_i32_packed"])

@@ -1027,16 +1027,21 @@ struct VariantDesc {
     // k-split twins of this tile (more wavefronts per work-group, each slab shared between groups of
     // them): the variant to take instead when the launch is one round of tiles / at most two
     const char *one_round = nullptr, *two_rounds = nullptr;
+    // and the quarter-size tile (one wavefront's 32x32, k split over four of them) for launches
+    // whose tiles of this size would leave a quarter of the CUs or more without work
+    const char *sparse = nullptr;
 };
 
 const VariantDesc k_variants[] = {
     {"mfma_f32_256x128", WK_F32, 256, 128, 16, 0.943, 0.25, &launch_f32<256, 128, 16, 2, 2, 2>},
     {"mfma_f32_128x128", WK_F32, 128, 128, 16, 0.885, 0.25, &launch_f32<128, 128, 16, 2, 2, 3>},
-    {"mfma_f32_64x64", WK_F32, 64, 64, 32, 0.780, 0.10, &launch_f32<64, 64, 32, 2, 2, 4>, "mfma_f32_64x64s4", "mfma_f32_64x64s2"},
+    {"mfma_f32_64x64", WK_F32, 64, 64, 32, 0.780, 0.10, &launch_f32<64, 64, 32, 2, 2, 4>, "mfma_f32_64x64s4", "mfma_f32_64x64s2",
+     "mfma_f32_32x32s4"},
     {"mfma_f32_64x64s2", WK_F32, 64, 64, 32, 0.0, 0.10, &launch_f32<64, 64, 16, 2, 2, 4, 2>}, // 2 groups x 16 k
     {"mfma_f32_64x64s4", WK_F32, 64, 64, 64, 0.0, 0.10, &launch_f32<64, 64, 16, 2, 2, 4, 4>}, // 4 groups x 16 k
+    {"mfma_f32_32x32s4", WK_F32, 32, 32, 64, 0.0, 0.10, &launch_f32<32, 32, 16, 1, 1, 4, 4>}, // one wavefront's tile, 4 groups
     {"mfma_f64_128x128", WK_F64, 128, 128, 16, 0.908, 0.20, &launch_f64<128, 128, 16, 2, 2, 2>},
-    {"mfma_f64_64x64", WK_F64, 64, 64, 32, 0.840, 0.05, &launch_f64<64, 64, 32, 2, 2, 2>, "mfma_f64_64x64s2", nullptr},
+    {"mfma_f64_64x64", WK_F64, 64, 64, 32, 0.840, 0.05, &launch_f64<64, 64, 32, 2, 2, 2>, "mfma_f64_64x64s2", nullptr, nullptr},
     {"mfma_f64_64x64s2", WK_F64, 64, 64, 64, 0.0, 0.05, &launch_f64<64, 64, 32, 2, 2, 2, 2>}, // 2 groups x 32 k
     {"mfma_f64_128x64", WK_F64, 128, 64, 16, 0.863, 0.25, &launch_f64<128, 64, 16, 2, 2, 3>},
     // 32-bit integers through the int8 matrix cores (wk_gemm_imfma.hip); same kernel for both signs
@@ -1118,10 +1123,14 @@ int wk::gemm_mfma_pick(const GemmProblem &p) {
     // Measured on MI355X, f32: 1024^3 90.8 -> 101.8 TFLOP/s, 1000^3 64 -> 76, 1024x1024x4096 102 -> 119,
     // 2048x1024x1024 (two rounds) 108 -> 113; f64: 1024^3 47 -> 53, 1000^3 36.6 -> 42.9.  From three
     // rounds on, and for short k, the plain tile is as fast or faster.
-    if (best >= 0 && p.K >= 256) {
+    // Below three quarters of a round the quarter-size tile spreads the work over the idle CUs
+    // (f32 512^3: 13.1 -> 6.9 us, 512x512x2048: 43.5 -> 15.7 us, 768^3: 18.5 -> 14.8 us; at 1024^3 it loses).
+    if (best >= 0 && p.K >= 64) {
         const VariantDesc &d = k_variants[best];
         const double tiles = (double)((p.M + d.bm - 1) / d.bm) * (double)((p.N + d.bn - 1) / d.bn);
-        const char *twin = tiles <= cus ? d.one_round : (tiles <= 2.0 * cus ? d.two_rounds : nullptr);
+        const char *twin = nullptr;
+        if (tiles <= 0.75 * cus && d.sparse) twin = d.sparse; // (f64: measured several times slower, not built)
+        else if (p.K >= 256) twin = tiles <= cus ? d.one_round : (tiles <= 2.0 * cus ? d.two_rounds : nullptr);
         for (int v = 0; twin && v < k_num_variants; ++v)
             if (!std::strcmp(k_variants[v].name, twin)) return v;
     }
