@@ -161,9 +161,10 @@ int  wk_axpy(wk_stream *s, int dtype, const uint64_t shape3[3],
  *   at least wk_gemm_workspace_bytes() bytes of device memory (16-byte aligned; what
  *   blas.PackedTensors holds) products that are large enough first pack both operands into
  *   signed-digit planes there and then run a lean int8 matrix-core kernel (for 8 and 16 bits the
- *   only matrix-core path); the result is the same bits either way.  cf32 / cf64 use a workspace
- *   too: B is rebuilt there as its real 2K x 2N form (transposed operands are turned first) and the
- *   product runs on the real f32 / f64 matrix-core kernels, to the float tolerance.  Every other type stages
+ *   only matrix-core path); the result is the same bits either way.  cf32 / cf64 and the complex
+ *   8/16/32-bit integers use a workspace too: B is rebuilt there as its real 2K x 2N form
+ *   (transposed operands are turned first) and the product runs on the real matrix-core kernels
+ *   (floats: to the float tolerance; integers: the same bits).  Every other type stages
  *   its tiles through LDS straight from the row-major operands, asks for 0 bytes and ignores the
  *   workspace, which may always be NULL.  The workspace is overwritten by every call that uses it:
  *   calls sharing one must be ordered on one stream. */

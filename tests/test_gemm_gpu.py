@@ -339,6 +339,25 @@ def test_narrow_integers_with_workspace_automatic(dev, dtype):
     assert np.array_equal(run_gemm(dev, dtype, 3, a, 0, b, 1, 5, c), want)
 
 
+def test_complex_integers_with_workspace_automatic(dev):
+    """ci16 at a size where the automatic choice takes the pack passes: same bits as the generic
+    kernel (no workspace) and the oracle."""
+    from wekua_amd import raw
+    dtype, (M, N, K) = "ci16", (512, 384, 512)
+    a, b, c = gemm_operands(dtype, M, N, K, 1, 0, 9)
+    need = dev.lib.wk_gemm_workspace_bytes(raw.dtype_id(dtype), 1, 0, M, N, K)
+    assert dev.lib.wk_gemm_variant_with_workspace(raw.dtype_id(dtype), 1, 0, M, N, K, M, N, N, None, None, None, need) \
+        == b"mfma_ci16_packed"
+    want = oracle.gemm(dtype, (3, -2), a, 1, b, 0, (5, 1), c)
+    assert np.array_equal(run_gemm(dev, dtype, (3, -2), a, 1, b, 0, (5, 1), c, packed=True), want)
+    assert np.array_equal(run_gemm(dev, dtype, (3, -2), a, 1, b, 0, (5, 1), c), want)
+    # cu32 at a size below its own pack pass: the real product runs on the fused int8 matrix-core kernel
+    for (M, N, K, op_a, op_b) in [(256, 192, 320, 0, 1), (130, 70, 200, 1, 1)]:
+        a, b, c = gemm_operands("cu32", M, N, K, op_a, op_b, 10)
+        want = oracle.gemm("cu32", (4000000000, 7), a, op_a, b, op_b, (1, 2), c)
+        assert np.array_equal(run_gemm(dev, "cu32", (4000000000, 7), a, op_a, b, op_b, (1, 2), c, packed=True), want)
+
+
 @pytest.mark.parametrize("dtype", ["f32", "f64", "i32", "u8", "i16"])
 def test_seeded_random_problems(dev, dtype):
     """Sixty seeded random problems per type under the automatic kernel choice: shapes up to 400 (so
@@ -362,19 +381,22 @@ def test_seeded_random_problems(dev, dtype):
         check(dev, dtype, M, N, K, op_a, op_b, alpha, beta, seed=1000 + case, packed=integer and case % 2 == 0, **kw)
 
 
-@pytest.mark.parametrize("dtype", ["cf32", "cf64"])
+@pytest.mark.parametrize("dtype", ["cf32", "cf64", "ci8", "cu8", "ci16", "cu16", "ci32", "cu32"])
 @pytest.mark.parametrize("op_a,op_b", OPS)
-def test_complex_float_through_the_real_matrix_cores(dev, dtype, op_a, op_b):
-    """cf32 / cf64 with a workspace: B is expanded to its real 2K x 2N form (alpha folded in),
+def test_complex_through_the_real_matrix_cores(dev, dtype, op_a, op_b):
+    """Complex types with a workspace: B is expanded to its real 2K x 2N form (alpha folded in),
     transposed operands are turned first, beta scales C beforehand, and the product is the real
-    matrix-core kernel on (M, 2N, 2K).  Against the oracle to the float tolerance of the real types,
-    for every option combination, ragged shapes and padded leading dimensions."""
+    matrix-core path on (M, 2N, 2K) -- the f32 / f64 kernel, or for the complex integers the packed
+    int8 matrix-core path, where every step is exact modulo 2^width.  Against the oracle (floats to
+    the tolerance of the real types, integers bit for bit on full-range entries), for every option
+    combination, ragged shapes and padded leading dimensions."""
     assert dev.lib.wk_gemm_force_variant(f"mfma_{dtype}_packed".encode()) == 0
+    fl = dtype[1] == "f"
     try:
         for (M, N, K) in [(5, 7, 3), (33, 17, 65), (64, 96, 48), (128, 128, 64), (130, 70, 200), (257, 129, 17)]:
-            for alpha, beta in [(None, None), ((2, 1), None), ((2, 1), (1, -1)), (None, (0.5, 0.25))]:
+            for alpha, beta in [(None, None), ((2, 1), None), ((2, 1), (1, -1)), (None, (0.5, 0.25) if fl else (3, 125))]:
                 check(dev, dtype, M, N, K, op_a, op_b, alpha, beta, seed=71, packed=True)
-        check(dev, dtype, 70, 45, 33, op_a, op_b, (1.5, -0.5), (0.25, 2), seed=72, packed=True,
+        check(dev, dtype, 70, 45, 33, op_a, op_b, (1.5, -0.5) if fl else (-7, 5), (0.25, 2) if fl else (2, -3), seed=72, packed=True,
               lda=(70 if op_a else 33) + 3, ldb=(33 if op_b else 45) + 5, ldc=45 + 7)
     finally:
         dev.lib.wk_gemm_force_variant(b"auto")
@@ -392,7 +414,7 @@ def test_complex_float_nan_in_c_propagates_with_beta(dev):
         dev.lib.wk_gemm_force_variant(b"auto")
 
 
-@pytest.mark.parametrize("dtype", ["i8", "u16", "i32", "cf32", "cf64"])
+@pytest.mark.parametrize("dtype", ["i8", "u16", "i32", "cf32", "cf64", "ci16", "cu32"])
 @pytest.mark.parametrize("op_a,op_b", OPS)
 def test_packed_b_kept_across_calls(dev, dtype, op_a, op_b):
     """wk_gemm_packed_b_kept: after one wk_gemm with a workspace, later calls with a new A pack only A.

@@ -407,7 +407,8 @@ class convertions:
 
 class GemmPackedTensors:
     """blas.GemmPackedTensors (src/blas/gemm.zig:60-359).  Holds device memory only for the types
-    whose gemm has a pack pass (8/16/32-bit integers, cf32, cf64): its workspace (`workspace_bytes`).
+    whose gemm has a pack pass (8/16/32-bit integers, their complex types, cf32, cf64): its workspace
+    (`workspace_bytes`).
     keepB / invalidateB have no counterpart in the reference, which packs both operands on every
     call: they let a constant B (weights) stay packed across calls."""
 

@@ -18,11 +18,21 @@ const char *k_generic_name = "tile64";
 // indexed by dtype (WK_I8 .. WK_U32)
 const char *k_packed_names[6] = {"mfma_i8_packed", "mfma_u8_packed", "mfma_i16_packed", "mfma_u16_packed",
                                  "mfma_i32_packed", "mfma_u32_packed"};
-const char *k_complex_packed_names[2] = {"mfma_cf32_packed", "mfma_cf64_packed"};
+const char *k_complex_packed_names[8] = {"mfma_ci8_packed",  "mfma_cu8_packed",  "mfma_ci16_packed", "mfma_cu16_packed",
+                                         "mfma_ci32_packed", "mfma_cu32_packed", "mfma_cf32_packed", "mfma_cf64_packed"};
 bool is_complex_float(int dtype) { return dtype == WK_CF32 || dtype == WK_CF64; }
+bool is_complex_small_int(int dtype) { return dtype >= WK_COMPLEX + WK_I8 && dtype <= WK_COMPLEX + WK_U32; }
+bool has_complex_packed_path(int dtype) { return is_complex_float(dtype) || is_complex_small_int(dtype); }
+const char *complex_packed_name(int dtype) {
+    return k_complex_packed_names[is_complex_float(dtype) ? 6 + (dtype == WK_CF64) : dtype - WK_COMPLEX];
+}
 // Two to four extra launches over the operands.  Measured against the generic kernel on MI355X: 512^3
 // 4x faster (cf32 0.137 -> 0.034 ms), 1024^3 3.7x, 4096^3 1.8x; the launches alone cost ~15 us.
 bool complex_packed_pays(const GemmProblem &p) {
+    // Complex integers have only the generic kernel beside this path, and it is slow for them
+    // (ci32 128^3: 37 us against 26; 512^3: 136 against 45; ci8 / ci16 256^3: 66 against 20-22).
+    if (is_complex_small_int(p.dtype))
+        return p.M >= 64 && p.N >= 64 && p.K >= 64 && (double)p.M * (double)p.N * (double)p.K >= 2.0e6;
     return p.M >= 64 && p.N >= 64 && p.K >= 64 && (double)p.M * (double)p.N * (double)p.K >= 1.6e7;
 }
 int transpose_for_gemm(void *ctx, int dtype, uint64_t rows, uint64_t cols, const void *src, uint64_t ld, void *dst) {
@@ -92,7 +102,7 @@ extern "C" {
 
 size_t wk_gemm_workspace_bytes(int dtype, int, int, uint64_t M, uint64_t N, uint64_t K) {
     if (!M || !N || !K) return 0;
-    if (is_complex_float(dtype)) return gemm_complex_packed_workspace_bytes(dtype, M, N, K);
+    if (has_complex_packed_path(dtype)) return gemm_complex_packed_workspace_bytes(dtype, M, N, K);
     if (!has_packed_path(dtype)) return 0;
     return gemm_int_packed_workspace_bytes(dtype, M, N, K);
 }
@@ -115,15 +125,22 @@ static int gemm_entry(wk_stream *s, int dtype, int op_a, int op_b, uint64_t M, u
         if (fits && (forced == -3 || (forced == -2 && packed_pays(p))))
             return gemm_int_packed_launch(s->stream, p, workspace, workspace_bytes);
     }
-    if (is_complex_float(dtype)) {
+    if (has_complex_packed_path(dtype)) {
         const int forced = g_forced.load(std::memory_order_relaxed);
         const size_t need = gemm_complex_packed_workspace_bytes(dtype, M, N, K);
         const bool fits = need && workspace && workspace_bytes >= need && (reinterpret_cast<uintptr_t>(workspace) & 15u) == 0;
         if (forced == -3 && !fits) return WK_E_INVALID_VALUE;
         if (fits && (forced == -3 || (forced == -2 && complex_packed_pays(p)))) {
             GemmProblem real;
-            rc = gemm_complex_packed_prepare(s->stream, p, workspace, workspace_bytes, &transpose_for_gemm, s, real);
+            void *rest = nullptr;
+            size_t rest_bytes = 0;
+            rc = gemm_complex_packed_prepare(s->stream, p, workspace, workspace_bytes, &transpose_for_gemm, s, real, &rest,
+                                             &rest_bytes);
             if (rc) return rc;
+            // the real product: 8 / 16 bits have no other matrix-core path than the packed one; 32 bits take
+            // it where it pays against the fused kernel (ci32 1024^3: 78 us fused, 88 packed; 1536^3: 249 / 242)
+            if (is_complex_small_int(dtype) && (forced == -3 || !is_int32(real.dtype) || packed_pays(real)))
+                return gemm_int_packed_launch(s->stream, real, rest, rest_bytes);
             const int rv = gemm_mfma_pick(real);
             return rv >= 0 ? gemm_mfma_launch(s->stream, real, rv) : gemm_generic_launch(s->stream, real);
         }
@@ -187,14 +204,14 @@ const char *wk_gemm_variant_with_workspace(int dtype, int op_a, int op_b, uint64
                                            size_t workspace_bytes) {
     const char *plain = wk_gemm_variant(dtype, op_a, op_b, M, N, K, lda, ldb, ldc, A, B, C);
     if (!std::strcmp(plain, "invalid")) return plain;
-    if (is_complex_float(dtype)) {
+    if (has_complex_packed_path(dtype)) {
         const int forced = g_forced.load(std::memory_order_relaxed);
         const size_t need = gemm_complex_packed_workspace_bytes(dtype, M, N, K);
         const bool fits = need && workspace_bytes >= need;
         GemmProblem q;
-        q.M = M; q.N = N; q.K = K;
-        if (forced == -3) return fits ? k_complex_packed_names[dtype == WK_CF64] : "invalid";
-        return fits && forced == -2 && complex_packed_pays(q) ? k_complex_packed_names[dtype == WK_CF64] : plain;
+        q.dtype = dtype; q.M = M; q.N = N; q.K = K;
+        if (forced == -3) return fits ? complex_packed_name(dtype) : "invalid";
+        return fits && forced == -2 && complex_packed_pays(q) ? complex_packed_name(dtype) : plain;
     }
     if (!has_packed_path(dtype)) return plain;
     const int forced = g_forced.load(std::memory_order_relaxed);

@@ -1,4 +1,4 @@
-// Complex float GEMM through the real matrix-core kernels, for callers that bring a workspace
+// Complex GEMM (float and 8/16/32-bit integer components) through the real matrix-core kernels, for callers that bring a workspace
 // (blas.PackedTensors, the reference's pack pass: src/blas/gemm.zig:272-357, 705-720).
 //
 // With interleaved storage a complex M x K matrix IS a real M x 2K matrix, and
@@ -11,9 +11,13 @@
 // on (M, 2N, 2K): 8 M N K real flop, the same count as four real products per complex one.
 // Rounding differs from the reference's three-multiplication complex product
 // (wekua_cl_lib.cl:648-653) only within the stated float tolerance.
+// For the complex integer types everything is arithmetic modulo 2^width, where the identity is exact:
+// the passes compute in unsigned 32-bit and truncate (signed and unsigned share the bits), and the real
+// product is the packed int8 matrix-core path on (M, 2N, 2K) in the section of the workspace behind B~.
 #include "wk_internal.hpp"
 
 #include <cstring>
+#include <type_traits>
 
 using namespace wk;
 
@@ -21,37 +25,44 @@ namespace {
 
 constexpr int CP_BLOCK = 256;
 
+// the type the passes compute in: wraparound arithmetic for the integers without promotion to signed int
+template <typename R> using Wide = std::conditional_t<std::is_integral_v<R>, uint32_t, R>;
+
 // one thread per complex element of B (K x N, row pitch ldb complex elements)
 template <typename R>
 __global__ __launch_bounds__(CP_BLOCK) void expand_b_kernel(const R *__restrict__ B, uint64_t ldb, uint64_t K, uint64_t N,
-                                                            R *__restrict__ Bx, bool has_alpha, R ar, R ai) {
+                                                            R *__restrict__ Bx, bool has_alpha, R alpha_r, R alpha_i) {
+    using W = Wide<R>;
+    const W ar = alpha_r, ai = alpha_i;
     const uint64_t total = K * N;
     for (uint64_t idx = blockIdx.x * (uint64_t)CP_BLOCK + threadIdx.x; idx < total; idx += (uint64_t)gridDim.x * CP_BLOCK) {
         const uint64_t k = idx / N, n = idx - k * N;
-        R br = B[(k * ldb + n) * 2], bi = B[(k * ldb + n) * 2 + 1];
+        W br = B[(k * ldb + n) * 2], bi = B[(k * ldb + n) * 2 + 1];
         if (has_alpha) {
-            const R tr = ar * br - ai * bi, ti = ar * bi + ai * br;
+            const W tr = ar * br - ai * bi, ti = ar * bi + ai * br;
             br = tr;
             bi = ti;
         }
         R *row0 = Bx + (2 * k) * (2 * N) + 2 * n, *row1 = row0 + 2 * N;
-        row0[0] = br;
-        row0[1] = bi;
-        row1[0] = -bi;
-        row1[1] = br;
+        row0[0] = (R)br;
+        row0[1] = (R)bi;
+        row1[0] = (R)(W(0) - bi);
+        row1[1] = (R)br;
     }
 }
 
 // C = beta * C over the logical M x N complex region
 template <typename R>
-__global__ __launch_bounds__(CP_BLOCK) void cscale_kernel(R *__restrict__ C, uint64_t ldc, uint64_t M, uint64_t N, R br, R bi) {
+__global__ __launch_bounds__(CP_BLOCK) void cscale_kernel(R *__restrict__ C, uint64_t ldc, uint64_t M, uint64_t N, R beta_r, R beta_i) {
+    using W = Wide<R>;
+    const W br = beta_r, bi = beta_i;
     const uint64_t total = M * N;
     for (uint64_t idx = blockIdx.x * (uint64_t)CP_BLOCK + threadIdx.x; idx < total; idx += (uint64_t)gridDim.x * CP_BLOCK) {
         const uint64_t m = idx / N, n = idx - m * N;
         R *p = C + (m * ldc + n) * 2;
-        const R cr = p[0], ci = p[1];
-        p[0] = br * cr - bi * ci;
-        p[1] = br * ci + bi * cr;
+        const W cr = p[0], ci = p[1];
+        p[0] = (R)(br * cr - bi * ci);
+        p[1] = (R)(br * ci + bi * cr);
     }
 }
 
@@ -80,27 +91,49 @@ int prepare(hipStream_t st, const GemmProblem &p, const void *b_src, uint64_t ld
     return launch_status();
 }
 
-} // namespace
+// component type of a complex dtype this file handles, or -1
+int real_of(int dtype) {
+    if (dtype == WK_CF32) return WK_F32;
+    if (dtype == WK_CF64) return WK_F64;
+    if (dtype >= WK_COMPLEX + WK_I8 && dtype <= WK_COMPLEX + WK_U32) return dtype - WK_COMPLEX;
+    return -1;
+}
 
-size_t wk::gemm_complex_packed_workspace_bytes(int dtype, uint64_t M, uint64_t N, uint64_t K) {
-    if ((dtype != WK_CF32 && dtype != WK_CF64) || !M || !N || !K) return 0;
-    if (M > 0x3fffffffull || N > 0x3fffffffull || K > 0x3fffffffull) return 0; // the real problem doubles N and K
-    const size_t es = dtype == WK_CF32 ? 8 : 16;
+// bytes of the section holding the turned operands and B~
+size_t section_bytes(int dtype, uint64_t M, uint64_t N, uint64_t K) {
+    const size_t es = wk_dtype_size(dtype);
     return align16(M * K * es) + align16(K * N * es) + align16(2 * K * N * es);
 }
 
-// Fills `real` with the f32 / f64 problem whose result is the complex one, after enqueueing the passes
+} // namespace
+
+size_t wk::gemm_complex_packed_workspace_bytes(int dtype, uint64_t M, uint64_t N, uint64_t K) {
+    const int rd = real_of(dtype);
+    if (rd < 0 || !M || !N || !K) return 0;
+    if (M > 0x3fffffffull || N > 0x3fffffffull || K > 0x3fffffffull) return 0; // the real problem doubles N and K
+    const size_t section = section_bytes(dtype, M, N, K);
+    if (rd == WK_F32 || rd == WK_F64) return section;
+    const size_t product = gemm_int_packed_workspace_bytes(rd, M, 2 * N, 2 * K); // digit planes of the real operands
+    return product ? section + product : 0;
+}
+
+// Fills `real` with the real problem whose result is the complex one, after enqueueing the passes
 // that build its operands in the workspace.  `transpose` turns an R x C complex matrix (row pitch ld)
-// into its C x R transpose with row pitch R.
+// into its C x R transpose with row pitch R.  `rest` / `rest_bytes`: what lies behind the section
+// used here (the workspace of the real integer product; empty for the float types).
 int wk::gemm_complex_packed_prepare(hipStream_t st, const GemmProblem &p, void *workspace, size_t workspace_bytes,
                                     int (*transpose)(void *ctx, int dtype, uint64_t rows, uint64_t cols, const void *src, uint64_t ld,
                                                      void *dst),
-                                    void *ctx, GemmProblem &real) {
+                                    void *ctx, GemmProblem &real, void **rest, size_t *rest_bytes) {
     const size_t need = gemm_complex_packed_workspace_bytes(p.dtype, p.M, p.N, p.K);
     if (!need || !workspace || workspace_bytes < need || (reinterpret_cast<uintptr_t>(workspace) & 15u)) return WK_E_INVALID_VALUE;
-    const size_t es = p.dtype == WK_CF32 ? 8 : 16;
+    const int rd = real_of(p.dtype);
+    const size_t es = wk_dtype_size(p.dtype);
     unsigned char *ws = static_cast<unsigned char *>(workspace);
     unsigned char *at = ws, *bt = at + align16(p.M * p.K * es), *bx = bt + align16(p.K * p.N * es);
+    const size_t section = section_bytes(p.dtype, p.M, p.N, p.K);
+    *rest = ws + section;
+    *rest_bytes = workspace_bytes - section;
 
     const void *a_real = p.A;
     uint64_t lda_real = 2 * p.lda;
@@ -118,29 +151,38 @@ int wk::gemm_complex_packed_prepare(hipStream_t st, const GemmProblem &p, void *
         b_src = bt;
         ldb = p.N;
     }
-    const int rc = p.dtype == WK_CF32 ? prepare<float>(st, p, b_src, ldb, bx) : prepare<double>(st, p, b_src, ldb, bx);
+    int rc;
+    switch (es) {
+    case 2: rc = prepare<uint8_t>(st, p, b_src, ldb, bx); break;
+    case 4: rc = prepare<uint16_t>(st, p, b_src, ldb, bx); break;
+    case 8: rc = rd == WK_F32 ? prepare<float>(st, p, b_src, ldb, bx) : prepare<uint32_t>(st, p, b_src, ldb, bx); break;
+    default: rc = prepare<double>(st, p, b_src, ldb, bx); break;
+    }
     if (rc) return rc;
 
     real = GemmProblem{};
-    real.dtype = p.dtype == WK_CF32 ? WK_F32 : WK_F64;
+    real.dtype = rd;
     real.op_a = real.op_b = 0;
     real.M = p.M; real.N = 2 * p.N; real.K = 2 * p.K;
     real.A = a_real; real.lda = lda_real;
     real.B = bx; real.ldb = 2 * p.N;
     real.C = p.C; real.ldc = 2 * p.ldc;
     real.num_cus = p.num_cus;
+    real.reuse_b = p.reuse_b;
     std::memset(real.alpha, 0, sizeof real.alpha);
     std::memset(real.beta, 0, sizeof real.beta);
     if (p.epi == EPI_ALPHA_BETA) { // C was scaled by beta already, alpha is inside B~: C = 1 * acc + 1 * C
         real.epi = EPI_ALPHA_BETA;
-        if (real.dtype == WK_F32) {
+        if (rd == WK_F32) {
             const float one = 1.f;
             std::memcpy(real.alpha, &one, 4);
             std::memcpy(real.beta, &one, 4);
-        } else {
+        } else if (rd == WK_F64) {
             const double one = 1.;
             std::memcpy(real.alpha, &one, 8);
             std::memcpy(real.beta, &one, 8);
+        } else {
+            real.alpha[0] = real.beta[0] = 1; // little-endian integer one of any width
         }
     } else {
         real.epi = EPI_STORE;

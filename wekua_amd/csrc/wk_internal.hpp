@@ -179,12 +179,13 @@ int gemm_i32_mfma_launch_128(hipStream_t st, const GemmProblem &p, bool edge); /
 size_t gemm_int_packed_workspace_bytes(int dtype, uint64_t M, uint64_t N, uint64_t K); // 0: not applicable
 int gemm_int_packed_launch(hipStream_t st, const GemmProblem &p, void *workspace, size_t workspace_bytes);
 constexpr int WK_CF32 = WK_COMPLEX + WK_F32, WK_CF64 = WK_COMPLEX + WK_F64;
-// cf32 / cf64 through the real matrix-core kernels, operands rebuilt in caller-provided workspace (wk_gemm_cpack.hip)
+// cf32 / cf64 and the complex 8/16/32-bit integers through the real matrix-core kernels, operands
+// rebuilt in caller-provided workspace (wk_gemm_cpack.hip)
 size_t gemm_complex_packed_workspace_bytes(int dtype, uint64_t M, uint64_t N, uint64_t K); // 0: not applicable
 int gemm_complex_packed_prepare(hipStream_t st, const GemmProblem &p, void *workspace, size_t workspace_bytes,
                                 int (*transpose)(void *ctx, int dtype, uint64_t rows, uint64_t cols, const void *src, uint64_t ld,
                                                  void *dst),
-                                void *ctx, GemmProblem &real);
+                                void *ctx, GemmProblem &real, void **rest, size_t *rest_bytes);
 bool gemm_mfma_fuses(const GemmProblem &p, int variant); // variant can run p with the fused bias + activation epilogue
 int gemm_mfma_pick(const GemmProblem &p);        // -1: not applicable
 const char *gemm_mfma_variant_name(int variant); // nullptr past the end

@@ -27,8 +27,8 @@
 //     even vector count, row counts are not padded at all, and row pitches that are a
 //     multiple of 1 KiB and at least 16 KiB are skewed by 512 bytes to avoid channel aliasing;
 //   * PackedTensors holds device memory only for the 8/16/32-bit integers (the signed-digit planes of
-//     the int8 matrix-core product) and for cf32 / cf64 (operands rebuilt as real matrices), both
-//     filled by a pack pass inside gemm; for every other type the
+//     the int8 matrix-core product), for cf32 / cf64 and for the complex 8/16/32-bit integers
+//     (operands rebuilt as real matrices), all filled by pack passes inside gemm; for every other type the
 //     HIP kernels tile straight from the row-major operands through LDS and pack() only validates.
 #pragma once
 
