@@ -324,6 +324,18 @@ def test_narrow_integers_packed_bit_exact(dev, dtype, op_a, op_b):
         dev.lib.wk_gemm_force_variant(b"auto")
 
 
+@pytest.mark.parametrize("dtype", ["u8", "i16"])
+def test_narrow_integers_packed_large_tile(dev, dtype):
+    """From one 256 x 128 tile per compute unit up the packed kernel runs that tile (64 x 64 per
+    wavefront): an aligned and a ragged problem of that many tiles with a short K, bit-exact."""
+    assert dev.lib.wk_gemm_force_variant(f"mfma_{dtype}_packed".encode()) == 0
+    try:
+        check(dev, dtype, 4096, 2048, 128, 0, 1, None, None, seed=65, packed=True)
+        check(dev, dtype, 4096 + 77, 2048 + 5, 96, 1, 0, 3, 7, seed=66, packed=True)
+    finally:
+        dev.lib.wk_gemm_force_variant(b"auto")
+
+
 @pytest.mark.parametrize("dtype", ["i8", "u16"])
 def test_narrow_integers_with_workspace_automatic(dev, dtype):
     """With a workspace the automatic choice takes the matrix cores from a few hundred cubed up; the

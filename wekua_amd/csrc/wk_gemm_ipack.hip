@@ -57,7 +57,8 @@ struct Layout {
 Layout make_layout(int digits, uint64_t M, uint64_t N, uint64_t K) {
     Layout w;
     const uint64_t per_slab = 4 / digits;
-    w.Mp = (M + TILE - 1) / TILE * TILE;
+    const uint64_t m_tile = digits < 4 ? 256 : TILE; // the narrow types may run the 256-row tile
+    w.Mp = (M + m_tile - 1) / m_tile * m_tile;
     w.Np = (N + TILE - 1) / TILE * TILE;
     w.KB = ((K + BK - 1) / BK + per_slab - 1) / per_slab * per_slab;
     w.slabs = w.KB / per_slab;
@@ -224,8 +225,14 @@ struct PArgs {
 // BM = 64 -- two independent 4-wave work-groups per CU, so that the two waves of a SIMD are not held
 // in the same phase by one barrier -- was measured and is slower (8192^3: 207 against 222 TOP/s): it
 // copies half as much again per matrix instruction.
-template <int BM> struct PackedTile {
-    static constexpr int NT = BM * 4;                       // threads
+// WMF: 32-row blocks of A per wavefront.  With WMF = 1 a wavefront's tile is 32 x 64 and it reads
+// three 4 KiB groups from LDS per eight (8-bit: per slab) matrix instructions, which for one and two
+// digits is as long as the matrix work itself; WMF = 2 (64 x 64) reads four groups per sixteen.  The
+// 32-bit type, with ten digit products per group pair, is not short of LDS bandwidth and its four
+// accumulator sets leave no room for the larger tile.
+template <int BM, int WMF = 1> struct PackedTile {
+    static constexpr int WAVES_M = BM / (32 * WMF);
+    static constexpr int NT = WAVES_M * 2 * 64;             // threads
     static constexpr int GROUPS = BM / 32 + TILE / 32;      // 4 KiB groups per slab: A row blocks, then B column blocks
     static constexpr int STAGE_BYTES = GROUPS * GROUP_BYTES;
     static constexpr int GROUPS_PER_PASS = NT * 16 / GROUP_BYTES; // 1 or 2
@@ -233,10 +240,11 @@ template <int BM> struct PackedTile {
     static constexpr size_t LDS_BYTES = 2 * STAGE_BYTES + (BM + TILE) * sizeof(uint32_t);
 };
 
-template <typename E, int BM, bool EDGE>
-__global__ __launch_bounds__(BM * 4) __attribute__((amdgpu_waves_per_eu(2)))
+template <typename E, int BM, bool EDGE, int WMF = 1>
+__global__ __launch_bounds__(BM / (32 * WMF) * 128) __attribute__((amdgpu_waves_per_eu(2)))
 void gemm_int_packed_kernel(PArgs g) {
-    using TL = PackedTile<BM>;
+    using TL = PackedTile<BM, WMF>;
+    static_assert(BM + TILE <= TL::NT && TL::GROUPS % TL::GROUPS_PER_PASS == 0, "tile shape");
     constexpr int D = Digits<E>::D, KB_PER_SLAB = Digits<E>::KB_PER_SLAB;
     constexpr uint32_t CBIAS = Digits<E>::CBIAS;
     constexpr int STAGE_BYTES = TL::STAGE_BYTES, PASSES = TL::PASSES, A_GROUPS = BM / 32;
@@ -264,13 +272,15 @@ void gemm_int_packed_kernel(PArgs g) {
         row_sum[tid] = s; // col_sum follows row_sum
     }
 
-    i32x16 acc[D][2]; // one set per shift i + j
+    i32x16 acc[D][WMF][2]; // one set per shift i + j
 #pragma unroll
     for (int s = 0; s < D; ++s)
 #pragma unroll
-        for (int b = 0; b < 2; ++b)
+        for (int am = 0; am < WMF; ++am)
 #pragma unroll
-            for (int r = 0; r < 16; ++r) acc[s][b][r] = 0;
+            for (int b = 0; b < 2; ++b)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) acc[s][am][b][r] = 0;
 
     // Copy of one slab: GROUPS groups of 4 KiB; pass i moves group(s) i * GROUPS_PER_PASS (+ tid / 256).
     // Each group stream of this thread is a buffer resource (scalar registers) over the KB * 4 KiB of
@@ -304,13 +314,14 @@ void gemm_int_packed_kernel(PArgs g) {
             *reinterpret_cast<u32x4 *>(stages + buf * STAGE_BYTES + (TL::GROUPS_PER_PASS * i + grp) * GROUP_BYTES + within) = from[i];
     };
     auto compute = [&](int buf) {
-        const unsigned char *sa = stages + buf * STAGE_BYTES + wm * GROUP_BYTES + lane * 16;
+        const unsigned char *sa = stages + buf * STAGE_BYTES + wm * WMF * GROUP_BYTES + lane * 16;
         const unsigned char *sb = stages + buf * STAGE_BYTES + (A_GROUPS + wn * 2) * GROUP_BYTES + lane * 16;
         // the four blocks of a group: k-block f / D of the slab, digit f % D
-        i32x4 a[4], b[2][4];
+        i32x4 a[WMF][4], b[2][4];
 #pragma unroll
         for (int f = 0; f < 4; ++f) {
-            a[f] = *reinterpret_cast<const i32x4 *>(sa + f * BLOCK_BYTES);
+#pragma unroll
+            for (int am = 0; am < WMF; ++am) a[am][f] = *reinterpret_cast<const i32x4 *>(sa + am * GROUP_BYTES + f * BLOCK_BYTES);
             b[0][f] = *reinterpret_cast<const i32x4 *>(sb + f * BLOCK_BYTES);
             b[1][f] = *reinterpret_cast<const i32x4 *>(sb + GROUP_BYTES + f * BLOCK_BYTES);
         }
@@ -321,8 +332,11 @@ void gemm_int_packed_kernel(PArgs g) {
 #pragma unroll
                 for (int i = 0; i <= s; ++i)
 #pragma unroll
-                    for (int blk = 0; blk < 2; ++blk)
-                        acc[s][blk] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a[kbl * D + i], b[blk][kbl * D + s - i], acc[s][blk], 0, 0, 0);
+                    for (int am = 0; am < WMF; ++am)
+#pragma unroll
+                        for (int blk = 0; blk < 2; ++blk)
+                            acc[s][am][blk] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a[am][kbl * D + i], b[blk][kbl * D + s - i],
+                                                                                   acc[s][am][blk], 0, 0, 0);
     };
     // one step: slab kb is in LDS stage `cur`, slab kb + 1 in flight in staged[other]
     auto step = [&](uint32_t kb, auto cur_tag) {
@@ -349,6 +363,8 @@ void gemm_int_packed_kernel(PArgs g) {
     const uint32_t kc2 = g.K * (CBIAS * CBIAS);
     E *C = static_cast<E *>(g.C);
 #pragma unroll
+    for (int am = 0; am < WMF; ++am)
+#pragma unroll
     for (int blk = 0; blk < 2; ++blk) {
         const uint32_t lcol = wn * 64 + blk * 32 + l32, col = n0 + lcol;
         const uint32_t csum = col_sum[lcol];
@@ -356,17 +372,17 @@ void gemm_int_packed_kernel(PArgs g) {
         if (g.epi == EPI_ALPHA_BETA) {
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
-                const uint32_t row = m0 + wm * 32 + 8 * (r / 4) + 4 * lhi + (r % 4);
+                const uint32_t row = m0 + (wm * WMF + am) * 32 + 8 * (r / 4) + 4 * lhi + (r % 4);
                 const uint32_t rowc = EDGE ? min(row, g.M - 1) : row, colc = EDGE ? min(col, g.N - 1) : col;
                 old[r] = C[(size_t)rowc * g.ldc + colc];
             }
         }
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
-            const uint32_t lrow = wm * 32 + 8 * (r / 4) + 4 * lhi + (r % 4), row = m0 + lrow;
+            const uint32_t lrow = (wm * WMF + am) * 32 + 8 * (r / 4) + 4 * lhi + (r % 4), row = m0 + lrow;
             uint32_t v = 0;
 #pragma unroll
-            for (int s = 0; s < D; ++s) v += (uint32_t)acc[s][blk][r] << (8 * s);
+            for (int s = 0; s < D; ++s) v += (uint32_t)acc[s][am][blk][r] << (8 * s);
             v += CBIAS * (row_sum[lrow] + csum) - kc2;
             if (g.epi == EPI_ALPHA) v = g.alpha * v;
             else if (g.epi == EPI_ALPHA_BETA) v = g.alpha * v + g.beta * old[r];
@@ -375,14 +391,14 @@ void gemm_int_packed_kernel(PArgs g) {
     }
 }
 
-template <typename E, int BM, bool EDGE> int launch_packed(hipStream_t st, PArgs g) {
-    constexpr size_t lds = PackedTile<BM>::LDS_BYTES;
-    auto kern = gemm_int_packed_kernel<E, BM, EDGE>;
+template <typename E, int BM, bool EDGE, int WMF = 1> int launch_packed(hipStream_t st, PArgs g) {
+    constexpr size_t lds = PackedTile<BM, WMF>::LDS_BYTES;
+    auto kern = gemm_int_packed_kernel<E, BM, EDGE, WMF>;
     static const hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
                                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     if (attr != hipSuccess) { (void)hipGetLastError(); return hip_code(attr); }
-    g.tiles_m = g.Mp / BM;
-    hipLaunchKernelGGL(kern, dim3(g.tiles_m * g.tiles_n), dim3(PackedTile<BM>::NT), lds, st, g);
+    g.tiles_m = (g.M + BM - 1) / BM;
+    hipLaunchKernelGGL(kern, dim3(g.tiles_m * g.tiles_n), dim3(PackedTile<BM, WMF>::NT), lds, st, g);
     return launch_status();
 }
 
@@ -437,6 +453,17 @@ template <typename E> int launch_typed(hipStream_t st, const GemmProblem &p, uns
     g.alpha = g.beta = 0;
     std::memcpy(&g.alpha, p.alpha, D); // little-endian: zero-extended element
     std::memcpy(&g.beta, p.beta, D);
+    if constexpr (D < 4) {
+        // One and two digits: the 256 x 128 tile with 64 x 64 per wavefront once it fills the chip
+        // (measured against the 128 x 128 tile on MI355X: u16 4096^3 569 -> 661 TOP/s, 8192^3 607 -> 728;
+        // i8 8192^3 1535 -> 1690; below one tile per CU the smaller tile wins: i8 2048^3 663 against 511).
+        // These products move one byte per 170 operations even so and are bound by what the L2 delivers.
+        const uint64_t tiles256 = ((p.M + 255) / 256) * ((p.N + TILE - 1) / TILE);
+        if (tiles256 >= (p.num_cus ? p.num_cus : 256u)) {
+            const bool edge = p.M % 256 != 0 || p.N % TILE != 0;
+            return edge ? launch_packed<E, 256, true, 2>(st, g) : launch_packed<E, 256, false, 2>(st, g);
+        }
+    }
     const bool edge = p.M % TILE != 0 || p.N % TILE != 0;
     return edge ? launch_packed<E, 128, true>(st, g) : launch_packed<E, 128, false>(st, g);
 }
