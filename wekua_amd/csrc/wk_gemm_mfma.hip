@@ -111,7 +111,7 @@ template <int ROWS, int BK, bool KCONTIG> struct Slab {
 // KS * BK values between them (group kg multiplies the k values kg * BK .. kg * BK + BK - 1 of the
 // slab); their accumulators are added through LDS before the epilogue.  For launches that put a
 // single small work-group on a CU this doubles the wavefronts a SIMD can switch between.
-template <int BM, int BN, int BK, int WAVES_M, int WAVES_N, int OCC, bool A_K, bool B_K, bool EDGE, bool EXT = false, int KS = 1>
+template <int BM, int BN, int BK, int WAVES_M, int WAVES_N, int OCC, bool A_K, bool B_K, bool EDGE, bool EXT = false, int KS = 1, int LSEL = -1>
 __global__ __launch_bounds__(WAVES_M *WAVES_N * 64 * KS) __attribute__((amdgpu_waves_per_eu(OCC)))
 void gemm_f32_mfma_kernel(MArgs<float> g) {
     constexpr int NT = WAVES_M * WAVES_N * 64 * KS;
@@ -147,11 +147,14 @@ void gemm_f32_mfma_kernel(MArgs<float> g) {
 #pragma unroll
             for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
 
-    // Staging registers, global -> LDS.  The small tile keeps two sets and requests slab kt+2 while
-    // slab kt is computed: with one or two 64x64 tiles on a CU a slab's matrix work is shorter than
-    // the latency of a global load, so one slab of lead time does not cover it.  The large tiles
-    // measured no different with the deeper lead and keep one set.
-    constexpr int PF = (BM * BN <= 64 * 64) ? 2 : 1;
+    // Which spelling of the main loop (described below); the bounds-checked instantiation has the
+    // peeled ones only.
+    // Staging registers, global -> LDS: one set.  (LOOP 2 on the small tile keeps two and requests
+    // slab kt+2 while slab kt is computed: with one or two 64x64 tiles on a CU a slab's matrix work is
+    // shorter than the latency of a global load.  LOOP 3 gets the same lead from one set.)
+    constexpr int LOOP_WANTED = LSEL >= 0 ? LSEL : (BM * BN <= 128 * 128) ? 3 : B_K ? 3 : (A_K ? 0 : 2);
+    constexpr int LOOP = (EDGE && LOOP_WANTED < 2) ? 2 : LOOP_WANTED;
+    constexpr int PF = (BM * BN <= 64 * 64 && LOOP == 2) ? 2 : 1;
     f32x4 ra[PF][A_V4], rb[PF][B_V4];
 
     // ---- global -> registers -----------------------------------------------------------
@@ -326,7 +329,7 @@ void gemm_f32_mfma_kernel(MArgs<float> g) {
 
     load_ab(0, ra[0], rb[0], AnyFlavour{});
     store_ab(0, 0, ra[0], rb[0], AnyFlavour{});
-    if (PF == 2 && ktiles > 1) load_ab(BKT, ra[PF - 1], rb[PF - 1], AnyFlavour{});
+    if ((PF == 2 || LOOP == 3) && ktiles > 1) load_ab(BKT, ra[PF - 1], rb[PF - 1], AnyFlavour{});
     __syncthreads();
 
     // Fragment registers are double-buffered: the LDS reads for step s+1 are issued before the
@@ -338,7 +341,7 @@ void gemm_f32_mfma_kernel(MArgs<float> g) {
     // with two sets slab kt+2 is requested there and slab kt+1, requested an iteration ago, is the
     // one handed over.
     //
-    // The loop exists in three spellings of the same schedule.  How two co-resident work-groups
+    // The loop exists in four spellings, three of the same schedule and one that stores early.  How two co-resident work-groups
     // interleave on a CU depends on the instruction order the compiler derives from the spelling,
     // and the rate moves by up to 10 % with it; each tile (for 256x128: each operand layout) uses the one that measured fastest on
     // MI355X (same box, same process, f32, alpha and beta given):
@@ -348,9 +351,11 @@ void gemm_f32_mfma_kernel(MArgs<float> g) {
     //   LOOP 2  last slab peeled, hand-over fenced                  256x128: NN 133.4, NT 134.3, TN 131.1;
     //           (sched_barrier) so that matrix instructions         64x64 at 1024^3: 90.8 (LOOP 1: 88.7), 2048^3: 122.8 (115-120)
     //           are not hoisted above the barrier
-    // (the bounds-checked instantiation always takes LOOP 2, whose iterations exist per flavour)
-    constexpr int LOOP = EDGE ? 2 : (BM * BN <= 64 * 64) ? 2 : (BM * BN <= 128 * 128 ? 1 : ((A_K && !B_K) ? 0 : 2));
-    static_assert(LOOP == 2 || PF == 1, "only the peeled loop knows the two-set prefetch");
+    //   LOOP 3  LOOP 2 with an early store: slab kt+1, requested    256x128: NT 143.3, TT 141.2, NN 132.7, TN 127.2;
+    //           a whole iteration ago, goes to the free LDS        128x128: faster than LOOP 1 on every layout and shape tried
+    //           buffer at the top of iteration kt and slab kt+2     (4096^3 NT 109 -> 141, 2048x4096x4096 NN 126 -> 133);
+    //           is requested into the same registers               64x64: +1..3 % over LOOP 2 with two staging sets
+    // (the bounds-checked instantiation takes LOOP 2 or 3, whose iterations exist per flavour)
     f32x4 af[2][FM], bf[2][FN];
     read_frags(0, 0, af[0], bf[0]);
 
@@ -406,12 +411,20 @@ void gemm_f32_mfma_kernel(MArgs<float> g) {
         };
         for (uint32_t kt = 0; kt < ktiles; ++kt) iteration(kt);
     } else {
-        // one iteration that hands over to slab kt+1; P = parity of kt, a compile-time constant so
-        // that the staging sets stay in registers
+        // LOOP 2 and 3: one iteration that hands over to slab kt+1; P = parity of kt, a compile-time
+        // constant so that the staging sets stay in registers.  EARLY (LOOP 3): slab kt+1 was requested
+        // an iteration ago and goes to the free LDS buffer at the top of iteration kt, slab kt+2 is then
+        // requested into the same registers, and only the barrier and the first fragment reads of the
+        // next slab sit between the matrix instructions of two slabs.
+        constexpr bool EARLY = LOOP == 3;
+        constexpr int LEAD = (PF == 2 || EARLY) ? 2 : 1; // iteration kt requests slab kt + LEAD
         auto iteration = [&](uint32_t kt, auto parity_tag, auto flavour_tag) __attribute__((always_inline)) {
             constexpr int P = decltype(parity_tag)::value;
             const int cur = kt & 1;
-            if constexpr (PF == 1) {
+            if constexpr (EARLY) {
+                store_ab(cur ^ 1, (kt + 1) * BKT, ra[0], rb[0], flavour_tag);
+                if (kt + 2 < ktiles) load_ab((kt + 2) * BKT, ra[0], rb[0], flavour_tag);
+            } else if constexpr (PF == 1) {
                 load_ab((kt + 1) * BKT, ra[0], rb[0], flavour_tag);
             } else {
                 if (kt + 2 < ktiles) load_ab((kt + 2) * BKT, ra[P], rb[P], flavour_tag); // set P held slab kt, already in LDS
@@ -423,7 +436,7 @@ void gemm_f32_mfma_kernel(MArgs<float> g) {
                     read_frags(cur, s + 1, af[(s + 1) & 1], bf[(s + 1) & 1]);
                 } else {
                     __builtin_amdgcn_sched_barrier(0);
-                    store_ab(cur ^ 1, (kt + 1) * BKT, ra[NEXT], rb[NEXT], flavour_tag);
+                    if constexpr (!EARLY) store_ab(cur ^ 1, (kt + 1) * BKT, ra[NEXT], rb[NEXT], flavour_tag);
                     __syncthreads();
                     read_frags(cur ^ 1, 0, af[(s + 1) & 1], bf[(s + 1) & 1]);
                     __builtin_amdgcn_sched_barrier(0);
@@ -431,9 +444,10 @@ void gemm_f32_mfma_kernel(MArgs<float> g) {
                 mfma_step(s);
             }
         };
-        // iterations kt .. end-1 in one flavour; with two staging sets the set index is the parity of kt
+        // iterations kt .. end-1 in one flavour, two per trip; with two staging sets the set index is
+        // the parity of kt
         auto run = [&](uint32_t &kt, uint32_t end, auto flavour_tag) __attribute__((always_inline)) {
-            if constexpr (PF == 1) {
+            if constexpr (PF == 1 && !EARLY) {
                 for (; kt < end; ++kt) iteration(kt, integral_constant<int, 0>{}, flavour_tag);
             } else {
                 if ((kt & 1) && kt < end) {
@@ -452,7 +466,7 @@ void gemm_f32_mfma_kernel(MArgs<float> g) {
         };
         uint32_t kt = 0;
         if constexpr (!EDGE) {
-            if constexpr (PF == 1) {
+            if constexpr (PF == 1 && !EARLY) {
                 for (; kt + 1 < ktiles; ++kt) iteration(kt, integral_constant<int, 0>{}, AnyFlavour{});
             } else {
                 for (; kt + 2 < ktiles; kt += 2) {
@@ -465,11 +479,11 @@ void gemm_f32_mfma_kernel(MArgs<float> g) {
                 }
             }
         } else {
-            // Iteration kt stores slab kt + 1 and requests slab kt + PF: the iterations before
+            // Iteration kt stores slab kt + 1 and requests slab kt + LEAD: the iterations before
             // `main_end` touch complete slabs only and run in a flavour fixed for the tile.
             const bool has_tail = g.K % BKT != 0;
             const uint32_t hand_overs = ktiles - 1;
-            const uint32_t main_end = has_tail ? (hand_overs > (uint32_t)PF ? hand_overs - PF : 0u) : hand_overs;
+            const uint32_t main_end = has_tail ? (hand_overs > (uint32_t)LEAD ? hand_overs - LEAD : 0u) : hand_overs;
             if (tile_inside) run(kt, main_end, integral_constant<int, PLAIN>{});
             else run(kt, main_end, integral_constant<int, CLAMPED>{});
             run(kt, hand_overs, integral_constant<int, ANY>{});
@@ -955,10 +969,10 @@ template <typename K> int set_lds(K kernel, size_t bytes) {
     return WK_OK;
 }
 
-template <int BM, int BN, int BK, int WMS, int WNS, int OCC, bool AK, bool BKC, bool EDGE, bool EXT = false, int KS = 1>
+template <int BM, int BN, int BK, int WMS, int WNS, int OCC, bool AK, bool BKC, bool EDGE, bool EXT = false, int KS = 1, int LSEL = -1>
 int launch_f32_one(hipStream_t st, const GemmProblem &p) {
     constexpr size_t lds = 2 * (Slab<BM, BK * KS, AK>::SIZE + Slab<BN, BK * KS, BKC>::SIZE) * sizeof(float);
-    auto kern = gemm_f32_mfma_kernel<BM, BN, BK, WMS, WNS, OCC, AK, BKC, EDGE, EXT, KS>;
+    auto kern = gemm_f32_mfma_kernel<BM, BN, BK, WMS, WNS, OCC, AK, BKC, EDGE, EXT, KS, LSEL>;
     static int attr_rc = set_lds(kern, lds);
     if (attr_rc) return attr_rc;
     MArgs<float> g = make_args<float>(p, BM, BN);
@@ -967,17 +981,17 @@ int launch_f32_one(hipStream_t st, const GemmProblem &p) {
 }
 
 // BK: k values one group of wavefronts multiplies per slab; KS groups share a slab of BK * KS
-template <int BM, int BN, int BK, int WMS, int WNS, int OCC, int KS = 1>
+template <int BM, int BN, int BK, int WMS, int WNS, int OCC, int KS = 1, int LSEL = -1>
 int launch_f32(hipStream_t st, const GemmProblem &p, bool edge) {
     const int sel = (p.op_a ? 0 : 2) | (p.op_b ? 1 : 0); // bit1: A k-contiguous, bit0: B k-contiguous
     if (p.ext) { // fused bias + activation: instantiated for op N, T only (see gemm_mfma_fuses)
         if (sel != 3) return WK_E_INVALID_VALUE;
-        return edge ? launch_f32_one<BM, BN, BK, WMS, WNS, OCC, true, true, true, true, KS>(st, p)
-                    : launch_f32_one<BM, BN, BK, WMS, WNS, OCC, true, true, false, true, KS>(st, p);
+        return edge ? launch_f32_one<BM, BN, BK, WMS, WNS, OCC, true, true, true, true, KS, LSEL>(st, p)
+                    : launch_f32_one<BM, BN, BK, WMS, WNS, OCC, true, true, false, true, KS, LSEL>(st, p);
     }
 #define WK_CASE(AK, BKC)                                                                                   \
-    return edge ? launch_f32_one<BM, BN, BK, WMS, WNS, OCC, AK, BKC, true, false, KS>(st, p)                          \
-                : launch_f32_one<BM, BN, BK, WMS, WNS, OCC, AK, BKC, false, false, KS>(st, p)
+    return edge ? launch_f32_one<BM, BN, BK, WMS, WNS, OCC, AK, BKC, true, false, KS, LSEL>(st, p)                          \
+                : launch_f32_one<BM, BN, BK, WMS, WNS, OCC, AK, BKC, false, false, KS, LSEL>(st, p)
     switch (sel) {
     case 0: WK_CASE(false, false);
     case 1: WK_CASE(false, true);
