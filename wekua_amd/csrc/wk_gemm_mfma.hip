@@ -152,7 +152,7 @@ void gemm_f32_mfma_kernel(MArgs<float> g) {
     // Staging registers, global -> LDS: one set.  (LOOP 2 on the small tile keeps two and requests
     // slab kt+2 while slab kt is computed: with one or two 64x64 tiles on a CU a slab's matrix work is
     // shorter than the latency of a global load.  LOOP 3 gets the same lead from one set.)
-    constexpr int LOOP_WANTED = LSEL >= 0 ? LSEL : (BM * BN <= 128 * 128) ? 3 : B_K ? 3 : (A_K ? 0 : 2);
+    constexpr int LOOP_WANTED = LSEL >= 0 ? LSEL : (BM * BN <= 128 * 128) ? 3 : B_K ? 3 : (A_K ? 0 : 5);
     constexpr int LOOP = (EDGE && LOOP_WANTED < 2) ? 2 : LOOP_WANTED;
     constexpr int PF = (BM * BN <= 64 * 64 && LOOP == 2) ? 2 : 1;
     f32x4 ra[PF][A_V4], rb[PF][B_V4];
@@ -267,36 +267,53 @@ void gemm_f32_mfma_kernel(MArgs<float> g) {
     //   CLAMPED  edge tile, complete slab: clamped loads, stored as they are unless a row end is straddled
     //   ANY      decided per slab at run time (the iterations that touch the k tail)
     enum { PLAIN = 0, CLAMPED = 1, ANY = 2 };
-    auto load_ab = [&](uint32_t k0, f32x4 *ra, f32x4 *rb, auto flavour_tag) {
+    // W: which operands (bit 0: A, bit 1: B)
+    auto load_sel = [&](uint32_t k0, f32x4 *ra, f32x4 *rb, auto flavour_tag, auto which_tag) {
         constexpr int FL = decltype(flavour_tag)::value;
+        constexpr int W = decltype(which_tag)::value;
         if (FL == PLAIN || (FL == ANY && tile_inside && k0 < k_inside)) {
-            gload(ra, g.A, g.lda, m0, g.M, k0, integral_constant<bool, A_K>{}, integral_constant<int, BM>{},
-                  integral_constant<int, A_V4>{}, std::false_type{});
-            gload(rb, g.B, g.ldb, n0, g.N, k0, integral_constant<bool, B_K>{}, integral_constant<int, BN>{},
-                  integral_constant<int, B_V4>{}, std::false_type{});
+            if constexpr (W & 1)
+                gload(ra, g.A, g.lda, m0, g.M, k0, integral_constant<bool, A_K>{}, integral_constant<int, BM>{},
+                      integral_constant<int, A_V4>{}, std::false_type{});
+            if constexpr (W & 2)
+                gload(rb, g.B, g.ldb, n0, g.N, k0, integral_constant<bool, B_K>{}, integral_constant<int, BN>{},
+                      integral_constant<int, B_V4>{}, std::false_type{});
         } else {
-            gload(ra, g.A, g.lda, m0, g.M, k0, integral_constant<bool, A_K>{}, integral_constant<int, BM>{},
-                  integral_constant<int, A_V4>{}, std::true_type{});
-            gload(rb, g.B, g.ldb, n0, g.N, k0, integral_constant<bool, B_K>{}, integral_constant<int, BN>{},
-                  integral_constant<int, B_V4>{}, std::true_type{});
+            if constexpr (W & 1)
+                gload(ra, g.A, g.lda, m0, g.M, k0, integral_constant<bool, A_K>{}, integral_constant<int, BM>{},
+                      integral_constant<int, A_V4>{}, std::true_type{});
+            if constexpr (W & 2)
+                gload(rb, g.B, g.ldb, n0, g.N, k0, integral_constant<bool, B_K>{}, integral_constant<int, BN>{},
+                      integral_constant<int, B_V4>{}, std::true_type{});
         }
     };
-    auto store_ab = [&](int buf, uint32_t k0, const f32x4 *ra, const f32x4 *rb, auto flavour_tag) {
+    auto store_sel = [&](int buf, uint32_t k0, const f32x4 *ra, const f32x4 *rb, auto flavour_tag, auto which_tag) {
         constexpr int FL = decltype(flavour_tag)::value;
+        constexpr int W = decltype(which_tag)::value;
         const bool complete = FL != ANY || k0 < k_inside;
         const bool plain = FL == PLAIN || (FL == ANY && tile_inside && complete);
-        if (plain || (complete && !fix_a_always))
-            sstore(As + buf * SA::SIZE, ra, m0, g.M, k0, integral_constant<bool, A_K>{}, integral_constant<int, BM>{},
-                   integral_constant<int, A_V4>{}, std::false_type{});
-        else
-            sstore(As + buf * SA::SIZE, ra, m0, g.M, k0, integral_constant<bool, A_K>{}, integral_constant<int, BM>{},
-                   integral_constant<int, A_V4>{}, std::true_type{});
-        if (plain || (complete && !fix_b_always))
-            sstore(Bs + buf * SB::SIZE, rb, n0, g.N, k0, integral_constant<bool, B_K>{}, integral_constant<int, BN>{},
-                   integral_constant<int, B_V4>{}, std::false_type{});
-        else
-            sstore(Bs + buf * SB::SIZE, rb, n0, g.N, k0, integral_constant<bool, B_K>{}, integral_constant<int, BN>{},
-                   integral_constant<int, B_V4>{}, std::true_type{});
+        if constexpr (W & 1) {
+            if (plain || (complete && !fix_a_always))
+                sstore(As + buf * SA::SIZE, ra, m0, g.M, k0, integral_constant<bool, A_K>{}, integral_constant<int, BM>{},
+                       integral_constant<int, A_V4>{}, std::false_type{});
+            else
+                sstore(As + buf * SA::SIZE, ra, m0, g.M, k0, integral_constant<bool, A_K>{}, integral_constant<int, BM>{},
+                       integral_constant<int, A_V4>{}, std::true_type{});
+        }
+        if constexpr (W & 2) {
+            if (plain || (complete && !fix_b_always))
+                sstore(Bs + buf * SB::SIZE, rb, n0, g.N, k0, integral_constant<bool, B_K>{}, integral_constant<int, BN>{},
+                       integral_constant<int, B_V4>{}, std::false_type{});
+            else
+                sstore(Bs + buf * SB::SIZE, rb, n0, g.N, k0, integral_constant<bool, B_K>{}, integral_constant<int, BN>{},
+                       integral_constant<int, B_V4>{}, std::true_type{});
+        }
+    };
+    auto load_ab = [&](uint32_t k0, f32x4 *ra, f32x4 *rb, auto flavour_tag) {
+        load_sel(k0, ra, rb, flavour_tag, integral_constant<int, 3>{});
+    };
+    auto store_ab = [&](int buf, uint32_t k0, const f32x4 *ra, const f32x4 *rb, auto flavour_tag) {
+        store_sel(buf, k0, ra, rb, flavour_tag, integral_constant<int, 3>{});
     };
     using AnyFlavour = integral_constant<int, EDGE ? ANY : PLAIN>;
 
@@ -329,7 +346,9 @@ void gemm_f32_mfma_kernel(MArgs<float> g) {
 
     load_ab(0, ra[0], rb[0], AnyFlavour{});
     store_ab(0, 0, ra[0], rb[0], AnyFlavour{});
-    if ((PF == 2 || LOOP == 3) && ktiles > 1) load_ab(BKT, ra[PF - 1], rb[PF - 1], AnyFlavour{});
+    if (PF == 2 && ktiles > 1) load_ab(BKT, ra[PF - 1], rb[PF - 1], AnyFlavour{});
+    if (LOOP >= 3 && ktiles > 1) // the operands that are stored early are requested a slab ahead
+        load_sel(BKT, ra[0], rb[0], AnyFlavour{}, integral_constant<int, LOOP == 3 ? 3 : LOOP == 4 ? 1 : 2>{});
     __syncthreads();
 
     // Fragment registers are double-buffered: the LDS reads for step s+1 are issued before the
@@ -355,7 +374,9 @@ void gemm_f32_mfma_kernel(MArgs<float> g) {
     //           a whole iteration ago, goes to the free LDS        128x128: faster than LOOP 1 on every layout and shape tried
     //           buffer at the top of iteration kt and slab kt+2     (4096^3 NT 109 -> 141, 2048x4096x4096 NN 126 -> 133);
     //           is requested into the same registers               64x64: +1..3 % over LOOP 2 with two staging sets
-    // (the bounds-checked instantiation takes LOOP 2 or 3, whose iterations exist per flavour)
+    //   LOOP 4 / 5  LOOP 3 for A only / for B only, the other     256x128 TN: LOOP 5 136.1 (LOOP 2: 133.3, LOOP 4: 132.7);
+    //           operand stored late as in LOOP 2                    NN: 140.2 / 135.9, TT: 136.2 / 138.6 -- behind their own
+    // (the bounds-checked instantiation takes LOOP 2 and up, whose iterations exist per flavour)
     f32x4 af[2][FM], bf[2][FN];
     read_frags(0, 0, af[0], bf[0]);
 
@@ -416,14 +437,18 @@ void gemm_f32_mfma_kernel(MArgs<float> g) {
         // an iteration ago and goes to the free LDS buffer at the top of iteration kt, slab kt+2 is then
         // requested into the same registers, and only the barrier and the first fragment reads of the
         // next slab sit between the matrix instructions of two slabs.
-        constexpr bool EARLY = LOOP == 3;
+        constexpr bool EARLY = LOOP >= 3;
+        constexpr int EW = LOOP == 3 ? 3 : LOOP == 4 ? 1 : LOOP == 5 ? 2 : 0; // operands stored early (bit 0: A, bit 1: B)
+        using Early = integral_constant<int, EW>;
+        using Late = integral_constant<int, 3 - EW>;
         constexpr int LEAD = (PF == 2 || EARLY) ? 2 : 1; // iteration kt requests slab kt + LEAD
         auto iteration = [&](uint32_t kt, auto parity_tag, auto flavour_tag) __attribute__((always_inline)) {
             constexpr int P = decltype(parity_tag)::value;
             const int cur = kt & 1;
             if constexpr (EARLY) {
-                store_ab(cur ^ 1, (kt + 1) * BKT, ra[0], rb[0], flavour_tag);
-                if (kt + 2 < ktiles) load_ab((kt + 2) * BKT, ra[0], rb[0], flavour_tag);
+                store_sel(cur ^ 1, (kt + 1) * BKT, ra[0], rb[0], flavour_tag, Early{});
+                if (kt + 2 < ktiles) load_sel((kt + 2) * BKT, ra[0], rb[0], flavour_tag, Early{});
+                if constexpr (EW != 3) load_sel((kt + 1) * BKT, ra[0], rb[0], flavour_tag, Late{});
             } else if constexpr (PF == 1) {
                 load_ab((kt + 1) * BKT, ra[0], rb[0], flavour_tag);
             } else {
@@ -437,6 +462,7 @@ void gemm_f32_mfma_kernel(MArgs<float> g) {
                 } else {
                     __builtin_amdgcn_sched_barrier(0);
                     if constexpr (!EARLY) store_ab(cur ^ 1, (kt + 1) * BKT, ra[NEXT], rb[NEXT], flavour_tag);
+                    else if constexpr (EW != 3) store_sel(cur ^ 1, (kt + 1) * BKT, ra[0], rb[0], flavour_tag, Late{});
                     __syncthreads();
                     read_frags(cur ^ 1, 0, af[(s + 1) & 1], bf[(s + 1) & 1]);
                     __builtin_amdgcn_sched_barrier(0);
