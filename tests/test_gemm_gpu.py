@@ -89,7 +89,8 @@ def test_f32_every_variant(dev, variant, op_a, op_b):
         dev.lib.wk_gemm_force_variant(b"auto")
 
 
-@pytest.mark.parametrize("variant", ["tile64", "mfma_f64_64x64", "mfma_f64_64x64s2", "mfma_f64_128x64", "mfma_f64_128x128"])
+@pytest.mark.parametrize("variant", ["tile64", "mfma_f64_64x64", "mfma_f64_64x64s2", "mfma_f64_32x32s4", "mfma_f64_128x64",
+                                     "mfma_f64_128x128"])
 @pytest.mark.parametrize("op_a,op_b", OPS)
 def test_f64_every_variant(dev, variant, op_a, op_b):
     assert dev.lib.wk_gemm_force_variant(variant.encode()) == 0
@@ -246,7 +247,8 @@ def test_invalid_arguments(dev):
 
 @pytest.mark.parametrize("dtype,variant", [("f32", "mfma_f32_64x64"), ("f32", "mfma_f32_64x64s2"), ("f32", "mfma_f32_64x64s4"),
                                            ("f32", "mfma_f32_32x32s4"), ("f32", "mfma_f32_128x128"), ("f32", "mfma_f32_256x128"),
-                                           ("f64", "mfma_f64_64x64"), ("f64", "mfma_f64_64x64s2"), ("f64", "mfma_f64_128x64"), ("f64", "mfma_f64_128x128")])
+                                           ("f64", "mfma_f64_64x64"), ("f64", "mfma_f64_64x64s2"), ("f64", "mfma_f64_32x32s4"),
+                                           ("f64", "mfma_f64_128x64"), ("f64", "mfma_f64_128x128")])
 def test_every_k_around_the_slab_boundaries(dev, dtype, variant):
     """Every K from 1 to 100 on a ragged tile and on a tile-aligned shape: the bounds-checked kernels
     choose per-flavour loops from the number of complete slabs (k-slab 16 or 32, one or two slabs of
@@ -283,6 +285,7 @@ def test_one_round_launches_take_the_k_split_tiles(dev):
     assert name("f32", 896, 896, 896) == b"mfma_f32_64x64s4"
     assert name("f64", 1024, 1024, 1024) == b"mfma_f64_64x64s2"
     assert name("f64", 2048, 2048, 2048) != b"mfma_f64_64x64s2"
+    assert name("f64", 512, 512, 512) == b"mfma_f64_32x32s4"
     for dtype in ("f32", "f64"):
         for op_a, op_b in OPS:
             check(dev, dtype, 1024, 960, 300, op_a, op_b, 1.5, 0.5, seed=93)

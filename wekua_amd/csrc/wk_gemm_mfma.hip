@@ -1081,8 +1081,12 @@ const VariantDesc k_variants[] = {
     {"mfma_f32_64x64s4", WK_F32, 64, 64, 64, 0.0, 0.10, &launch_f32<64, 64, 16, 2, 2, 4, 4>}, // 4 groups x 16 k
     {"mfma_f32_32x32s4", WK_F32, 32, 32, 64, 0.0, 0.10, &launch_f32<32, 32, 16, 1, 1, 4, 4>}, // one wavefront's tile, 4 groups
     {"mfma_f64_128x128", WK_F64, 128, 128, 16, 0.908, 0.20, &launch_f64<128, 128, 16, 2, 2, 2>},
-    {"mfma_f64_64x64", WK_F64, 64, 64, 32, 0.840, 0.05, &launch_f64<64, 64, 32, 2, 2, 2>, "mfma_f64_64x64s2", nullptr, nullptr},
+    {"mfma_f64_64x64", WK_F64, 64, 64, 32, 0.840, 0.05, &launch_f64<64, 64, 32, 2, 2, 2>, "mfma_f64_64x64s2", nullptr,
+     "mfma_f64_32x32s4"},
     {"mfma_f64_64x64s2", WK_F64, 64, 64, 64, 0.0, 0.05, &launch_f64<64, 64, 32, 2, 2, 2, 2>}, // 2 groups x 32 k
+    // (two wavefronts per SIMD: with a 128-register budget its staging sets and fragments spill and it
+    // runs several times slower than the 64x64 tile)
+    {"mfma_f64_32x32s4", WK_F64, 32, 32, 64, 0.0, 0.05, &launch_f64<32, 32, 16, 1, 1, 2, 4>},
     {"mfma_f64_128x64", WK_F64, 128, 64, 16, 0.863, 0.25, &launch_f64<128, 64, 16, 2, 2, 3>},
     // 32-bit integers through the int8 matrix cores (wk_gemm_imfma.hip); same kernel for both signs
     // (efficiency here is relative between the two integer tiles: 196-202 against 155-192 TOP/s)
@@ -1169,7 +1173,7 @@ int wk::gemm_mfma_pick(const GemmProblem &p) {
         const VariantDesc &d = k_variants[best];
         const double tiles = (double)((p.M + d.bm - 1) / d.bm) * (double)((p.N + d.bn - 1) / d.bn);
         const char *twin = nullptr;
-        if (tiles <= 0.75 * cus && d.sparse) twin = d.sparse; // (f64: measured several times slower, not built)
+        if (tiles <= 0.75 * cus && d.sparse) twin = d.sparse; // (f64 512^3: 21.5 -> 10.3 us, 512x512x2048: 74 -> 32 us)
         else if (p.K >= 256) twin = tiles <= cus ? d.one_round : (tiles <= 2.0 * cus ? d.two_rounds : nullptr);
         for (int v = 0; twin && v < k_num_variants; ++v)
             if (!std::strcmp(k_variants[v].name, twin)) return v;
