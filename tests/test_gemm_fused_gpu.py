@@ -46,7 +46,7 @@ def both(dev, dtype, M, N, K, op_a, op_b, kind, with_bias, seed, ld_extra=0):
 
 
 @pytest.mark.parametrize("dtype,variant", [("f32", "auto"), ("f32", "mfma_f32_64x64"), ("f32", "mfma_f32_64x64s2"),
-                                           ("f32", "mfma_f32_64x64s4"), ("f32", "mfma_f32_32x32s4"), ("f64", "mfma_f64_64x64s2"), ("f64", "mfma_f64_32x32s4"), ("f32", "mfma_f32_128x128"),
+                                           ("f32", "mfma_f32_64x64s4"), ("f32", "mfma_f32_32x32s4"), ("f32", "mfma_f32_128x128s2"), ("f64", "mfma_f64_64x64s2"), ("f64", "mfma_f64_32x32s4"), ("f32", "mfma_f32_128x128"),
                                            ("f32", "mfma_f32_256x128"), ("f64", "auto"), ("f64", "mfma_f64_64x64"),
                                            ("f64", "mfma_f64_128x64"), ("f64", "mfma_f64_128x128"), ("f32", "tile64")])
 @pytest.mark.parametrize("kind", ["none", "sigmoid", "tanh"])

@@ -77,7 +77,7 @@ def test_float_small_shapes(dev, dtype, op_a, op_b, alpha, beta):
 
 
 @pytest.mark.parametrize("variant", ["tile64", "mfma_f32_64x64", "mfma_f32_64x64s2", "mfma_f32_64x64s4", "mfma_f32_32x32s4",
-                                     "mfma_f32_128x128", "mfma_f32_256x128"])
+                                     "mfma_f32_128x128", "mfma_f32_128x128s2", "mfma_f32_256x128"])
 @pytest.mark.parametrize("op_a,op_b", OPS)
 def test_f32_every_variant(dev, variant, op_a, op_b):
     import ctypes
@@ -246,7 +246,8 @@ def test_invalid_arguments(dev):
 
 
 @pytest.mark.parametrize("dtype,variant", [("f32", "mfma_f32_64x64"), ("f32", "mfma_f32_64x64s2"), ("f32", "mfma_f32_64x64s4"),
-                                           ("f32", "mfma_f32_32x32s4"), ("f32", "mfma_f32_128x128"), ("f32", "mfma_f32_256x128"),
+                                           ("f32", "mfma_f32_32x32s4"), ("f32", "mfma_f32_128x128"), ("f32", "mfma_f32_128x128s2"),
+                                           ("f32", "mfma_f32_256x128"),
                                            ("f64", "mfma_f64_64x64"), ("f64", "mfma_f64_64x64s2"), ("f64", "mfma_f64_32x32s4"),
                                            ("f64", "mfma_f64_128x64"), ("f64", "mfma_f64_128x128")])
 def test_every_k_around_the_slab_boundaries(dev, dtype, variant):
@@ -283,6 +284,8 @@ def test_one_round_launches_take_the_k_split_tiles(dev):
     assert name("f32", 512, 512, 512) == b"mfma_f32_32x32s4"       # 64 tiles of 64x64 would leave most CUs idle
     assert name("f32", 768, 768, 768) == b"mfma_f32_32x32s4"
     assert name("f32", 896, 896, 896) == b"mfma_f32_64x64s4"
+    assert name("f32", 2048, 2048, 2048) == b"mfma_f32_128x128s2"  # one full round of 128x128 tiles
+    assert name("f32", 1536, 1536, 1536) == b"mfma_f32_64x64"
     assert name("f64", 1024, 1024, 1024) == b"mfma_f64_64x64s2"
     assert name("f64", 2048, 2048, 2048) != b"mfma_f64_64x64s2"
     assert name("f64", 512, 512, 512) == b"mfma_f64_32x32s4"

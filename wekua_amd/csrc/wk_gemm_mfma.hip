@@ -1075,6 +1075,7 @@ struct VariantDesc {
 const VariantDesc k_variants[] = {
     {"mfma_f32_256x128", WK_F32, 256, 128, 16, 0.943, 0.25, &launch_f32<256, 128, 16, 2, 2, 2>},
     {"mfma_f32_128x128", WK_F32, 128, 128, 16, 0.885, 0.25, &launch_f32<128, 128, 16, 2, 2, 3>},
+    {"mfma_f32_128x128s2", WK_F32, 128, 128, 32, 0.0, 0.25, &launch_f32<128, 128, 16, 2, 2, 2, 2>}, // 2 groups x 16 k, see pick
     {"mfma_f32_64x64", WK_F32, 64, 64, 32, 0.780, 0.10, &launch_f32<64, 64, 32, 2, 2, 4>, "mfma_f32_64x64s4", "mfma_f32_64x64s2",
      "mfma_f32_32x32s4"},
     {"mfma_f32_64x64s2", WK_F32, 64, 64, 32, 0.0, 0.10, &launch_f32<64, 64, 16, 2, 2, 4, 2>}, // 2 groups x 16 k
@@ -1161,6 +1162,16 @@ int wk::gemm_mfma_pick(const GemmProblem &p) {
             best = v;
             best_cost = cost;
         }
+    }
+    // f32 problems that are one nearly full round of 128x128 tiles: that tile with two k-groups (eight
+    // wavefronts per CU) beats the four rounds of 64x64 the cost model would take -- 2048^3 126 / 132 /
+    // 120 / 126 -> 130 / 136 / 126 / 131 TFLOP/s (NN / NT / TN / TT), 2048x2048x4096 128 -> 134.  With
+    // fewer tiles (1536^3) or more than one round (3072^3) the 64x64 tile wins.
+    if (p.dtype == WK_F32 && p.K >= 512) {
+        const double tiles128 = (double)((p.M + 127) / 128) * (double)((p.N + 127) / 128);
+        if (tiles128 <= cus && tiles128 >= 0.85 * cus)
+            for (int v = 0; v < k_num_variants; ++v)
+                if (!std::strcmp(k_variants[v].name, "mfma_f32_128x128s2")) return v;
     }
     // A launch of one round (f32: up to two) of the small tile leaves each SIMD one or two wavefronts,
     // which stall together at every hand-over: the k-split twin of the tile gives it two to four.
