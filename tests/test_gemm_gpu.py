@@ -489,3 +489,24 @@ def test_packed_b_kept_is_plain_gemm_without_a_workspace_path(dev):
         assert_gemm_close(dtype, got, want, None, a, 0, b, 1, None, c, K, what=dtype)
         for d in (dA, dB, dC):
             d.free()
+
+
+@pytest.mark.parametrize("dtype", ["f32", "f64"])
+def test_seeded_random_mid_size_problems(dev, dtype):
+    """Sixteen seeded random problems per type with M, N up to 2300 and K up to 700 under the automatic
+    kernel choice: the sizes where it moves between the quarter-size tile, the k-split twins, the plain
+    64x64 tile and the 128x128 tiles, mostly through their bounds-checked instantiations."""
+    from wekua_amd import raw
+    rng = np.random.default_rng({"f32": 11, "f64": 12}[dtype])
+    seen = set()
+    for case in range(16):
+        M, N = (int(v) for v in rng.integers(300, 2301, 2))
+        K = int(rng.integers(64, 701))
+        if case % 4 == 0:
+            M, N, K = (M + 127) // 128 * 128, (N + 127) // 128 * 128, (K + 63) // 64 * 64   # the unchecked kernels
+        op_a, op_b = int(rng.integers(0, 2)), int(rng.integers(0, 2))
+        alpha, beta = [(None, None), (1.5, None), (1.5, 0.5), (None, -0.25)][case % 4]
+        seen.add(dev.lib.wk_gemm_variant(raw.dtype_id(dtype), op_a, op_b, M, N, K, M if op_a else K, K if op_b else N, N, None, None,
+                                         None))
+        check(dev, dtype, M, N, K, op_a, op_b, alpha, beta, seed=700 + case)
+    assert len(seen) >= 3, seen
