@@ -59,7 +59,8 @@ Layout make_layout(int digits, uint64_t M, uint64_t N, uint64_t K) {
     const uint64_t per_slab = 4 / digits;
     const uint64_t m_tile = digits < 4 ? 256 : TILE; // the narrow types may run the 256-row tile
     w.Mp = (M + m_tile - 1) / m_tile * m_tile;
-    w.Np = (N + TILE - 1) / TILE * TILE;
+    const uint64_t n_tile = digits == 1 ? 256 : TILE; // 8-bit: also the 256-column tile
+    w.Np = (N + n_tile - 1) / n_tile * n_tile;
     w.KB = ((K + BK - 1) / BK + per_slab - 1) / per_slab * per_slab;
     w.slabs = w.KB / per_slab;
     // enough work-groups in the pack launch to fill the chip: (Mp + Np) / 32 row blocks x ksplit
@@ -230,28 +231,31 @@ struct PArgs {
 // digits is as long as the matrix work itself; WMF = 2 (64 x 64) reads four groups per sixteen.  The
 // 32-bit type, with ten digit products per group pair, is not short of LDS bandwidth and its four
 // accumulator sets leave no room for the larger tile.
-template <int BM, int WMF = 1> struct PackedTile {
+// BN: columns of the tile (two wavefronts across, BN / 64 blocks of 32 columns each).
+template <int BM, int WMF = 1, int BN = TILE> struct PackedTile {
     static constexpr int WAVES_M = BM / (32 * WMF);
     static constexpr int NT = WAVES_M * 2 * 64;             // threads
-    static constexpr int GROUPS = BM / 32 + TILE / 32;      // 4 KiB groups per slab: A row blocks, then B column blocks
+    static constexpr int GROUPS = BM / 32 + BN / 32;        // 4 KiB groups per slab: A row blocks, then B column blocks
     static constexpr int STAGE_BYTES = GROUPS * GROUP_BYTES;
     static constexpr int GROUPS_PER_PASS = NT * 16 / GROUP_BYTES; // 1 or 2
     static constexpr int PASSES = GROUPS / GROUPS_PER_PASS;
-    static constexpr size_t LDS_BYTES = 2 * STAGE_BYTES + (BM + TILE) * sizeof(uint32_t);
+    static constexpr size_t LDS_BYTES = 2 * STAGE_BYTES + (BM + BN) * sizeof(uint32_t);
 };
 
-template <typename E, int BM, bool EDGE, int WMF = 1>
+template <typename E, int BM, bool EDGE, int WMF = 1, int BN = TILE>
 __global__ __launch_bounds__(BM / (32 * WMF) * 128) __attribute__((amdgpu_waves_per_eu(2)))
 void gemm_int_packed_kernel(PArgs g) {
-    using TL = PackedTile<BM, WMF>;
-    static_assert(BM + TILE <= TL::NT && TL::GROUPS % TL::GROUPS_PER_PASS == 0, "tile shape");
+    using TL = PackedTile<BM, WMF, BN>;
+    constexpr int WNF = BN / 64;        // 32-column blocks of B per wavefront
+    constexpr bool ONE_SET = BN > TILE; // the 256 x 256 tile has registers for one staging set only
+    static_assert(BM + BN <= TL::NT && TL::GROUPS % TL::GROUPS_PER_PASS == 0, "tile shape");
     constexpr int D = Digits<E>::D, KB_PER_SLAB = Digits<E>::KB_PER_SLAB;
     constexpr uint32_t CBIAS = Digits<E>::CBIAS;
     constexpr int STAGE_BYTES = TL::STAGE_BYTES, PASSES = TL::PASSES, A_GROUPS = BM / 32;
     extern __shared__ __align__(16) unsigned char lds_raw[];
     unsigned char *stages = lds_raw;                                              // [2][STAGE_BYTES]
     uint32_t *row_sum = reinterpret_cast<uint32_t *>(lds_raw + 2 * STAGE_BYTES);  // [BM]
-    uint32_t *col_sum = row_sum + BM;                                             // [TILE]
+    uint32_t *col_sum = row_sum + BM;                                             // [BN]
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wm = wave >> 1, wn = wave & 1, l32 = lane & 31, lhi = lane >> 5;
@@ -262,9 +266,9 @@ void gemm_int_packed_kernel(PArgs g) {
         tile_m = first_m + in_group % gsz;
         tile_n = in_group / gsz;
     }
-    const uint32_t m0 = tile_m * BM, n0 = tile_n * TILE;
+    const uint32_t m0 = tile_m * BM, n0 = tile_n * BN;
 
-    if (tid < BM + TILE) {
+    if (tid < BM + BN) {
         const uint32_t *src = tid < BM ? g.sums_a + m0 + tid : g.sums_b + n0 + (tid - BM);
         const uint32_t stride = tid < BM ? g.Mp : g.Np;
         uint32_t s = 0;
@@ -272,13 +276,13 @@ void gemm_int_packed_kernel(PArgs g) {
         row_sum[tid] = s; // col_sum follows row_sum
     }
 
-    i32x16 acc[D][WMF][2]; // one set per shift i + j
+    i32x16 acc[D][WMF][WNF]; // one set per shift i + j
 #pragma unroll
     for (int s = 0; s < D; ++s)
 #pragma unroll
         for (int am = 0; am < WMF; ++am)
 #pragma unroll
-            for (int b = 0; b < 2; ++b)
+            for (int b = 0; b < WNF; ++b)
 #pragma unroll
                 for (int r = 0; r < 16; ++r) acc[s][am][b][r] = 0;
 
@@ -294,14 +298,14 @@ void gemm_int_packed_kernel(PArgs g) {
     for (int i = 0; i < PASSES; ++i) {
         const int gi = TL::GROUPS_PER_PASS * i + grp; // < A_GROUPS: A row blocks, then B column blocks
         const unsigned char *p = gi < A_GROUPS ? g.planes_a + (size_t)(tile_m * A_GROUPS + gi) * g.slabs * GROUP_BYTES
-                                               : g.planes_b + (size_t)(tile_n * 4 + gi - A_GROUPS) * g.slabs * GROUP_BYTES;
+                                               : g.planes_b + (size_t)(tile_n * (BN / 32) + gi - A_GROUPS) * g.slabs * GROUP_BYTES;
         src[i] = __builtin_amdgcn_make_buffer_rsrc(const_cast<unsigned char *>(p), 0, (int)(g.slabs * GROUP_BYTES), 0x00020000);
     }
     // Two register sets: the slab loaded in step kb is stored to LDS at the end of step kb + 1 and
     // used in step kb + 2, so a load has two slabs of matrix work to arrive.
     // (past the end the last slab is loaded again and dropped: no branch, so the loads stay where
     // they are written, ahead of the matrix work)
-    u32x4 staged[2][PASSES];
+    u32x4 staged[ONE_SET ? 1 : 2][PASSES];
     auto gload = [&](u32x4 *dst, uint32_t kb) {
         const int off = (int)(min(kb, g.slabs - 1) * GROUP_BYTES);
 #pragma unroll
@@ -315,15 +319,33 @@ void gemm_int_packed_kernel(PArgs g) {
     };
     auto compute = [&](int buf) {
         const unsigned char *sa = stages + buf * STAGE_BYTES + wm * WMF * GROUP_BYTES + lane * 16;
-        const unsigned char *sb = stages + buf * STAGE_BYTES + (A_GROUPS + wn * 2) * GROUP_BYTES + lane * 16;
+        const unsigned char *sb = stages + buf * STAGE_BYTES + (A_GROUPS + wn * WNF) * GROUP_BYTES + lane * 16;
+        if constexpr (D == 1 && WNF > 2) {
+            // one digit, large tile: a k-block needs only its own fragments, so they are fetched per
+            // k-block instead of all sixteen of the slab at once (which would not fit the registers)
+#pragma unroll
+            for (int kbl = 0; kbl < KB_PER_SLAB; ++kbl) {
+                i32x4 a[WMF], b[WNF];
+#pragma unroll
+                for (int am = 0; am < WMF; ++am) a[am] = *reinterpret_cast<const i32x4 *>(sa + am * GROUP_BYTES + kbl * BLOCK_BYTES);
+#pragma unroll
+                for (int blk = 0; blk < WNF; ++blk) b[blk] = *reinterpret_cast<const i32x4 *>(sb + blk * GROUP_BYTES + kbl * BLOCK_BYTES);
+#pragma unroll
+                for (int am = 0; am < WMF; ++am)
+#pragma unroll
+                    for (int blk = 0; blk < WNF; ++blk)
+                        acc[0][am][blk] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a[am], b[blk], acc[0][am][blk], 0, 0, 0);
+            }
+            return;
+        }
         // the four blocks of a group: k-block f / D of the slab, digit f % D
-        i32x4 a[WMF][4], b[2][4];
+        i32x4 a[WMF][4], b[WNF][4];
 #pragma unroll
         for (int f = 0; f < 4; ++f) {
 #pragma unroll
             for (int am = 0; am < WMF; ++am) a[am][f] = *reinterpret_cast<const i32x4 *>(sa + am * GROUP_BYTES + f * BLOCK_BYTES);
-            b[0][f] = *reinterpret_cast<const i32x4 *>(sb + f * BLOCK_BYTES);
-            b[1][f] = *reinterpret_cast<const i32x4 *>(sb + GROUP_BYTES + f * BLOCK_BYTES);
+#pragma unroll
+            for (int blk = 0; blk < WNF; ++blk) b[blk][f] = *reinterpret_cast<const i32x4 *>(sb + blk * GROUP_BYTES + f * BLOCK_BYTES);
         }
 #pragma unroll
         for (int kbl = 0; kbl < KB_PER_SLAB; ++kbl)
@@ -334,24 +356,38 @@ void gemm_int_packed_kernel(PArgs g) {
 #pragma unroll
                     for (int am = 0; am < WMF; ++am)
 #pragma unroll
-                        for (int blk = 0; blk < 2; ++blk)
+                        for (int blk = 0; blk < WNF; ++blk)
                             acc[s][am][blk] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a[am][kbl * D + i], b[blk][kbl * D + s - i],
                                                                                    acc[s][am][blk], 0, 0, 0);
     };
     // one step: slab kb is in LDS stage `cur`, slab kb + 1 in flight in staged[other]
     auto step = [&](uint32_t kb, auto cur_tag) {
         constexpr int cur = decltype(cur_tag)::value;
-        gload(staged[cur], kb + 2);
-        compute(cur);
-        if (kb + 1 < g.slabs) {
-            sstore(staged[cur ^ 1], cur ^ 1);
-            __syncthreads();
+        if constexpr (ONE_SET) {
+            // one set: slab kb + 1, requested a step ago, goes to the free stage first and slab kb + 2
+            // is requested into the same registers (measured equal to the two-set order on the other tiles)
+            if (kb + 1 < g.slabs) sstore(staged[0], cur ^ 1);
+            gload(staged[0], kb + 2);
+            compute(cur);
+            if (kb + 1 < g.slabs) __syncthreads();
+        } else {
+            gload(staged[cur], kb + 2);
+            compute(cur);
+            if (kb + 1 < g.slabs) {
+                sstore(staged[cur ^ 1], cur ^ 1);
+                __syncthreads();
+            }
         }
     };
 
     gload(staged[0], 0);
-    gload(staged[1], 1);
-    sstore(staged[0], 0);
+    if constexpr (ONE_SET) {
+        sstore(staged[0], 0);
+        gload(staged[0], 1);
+    } else {
+        gload(staged[1], 1);
+        sstore(staged[0], 0);
+    }
     __syncthreads();
     for (uint32_t kb = 0; kb < g.slabs; kb += 2) {
         step(kb, std::integral_constant<int, 0>{});
@@ -365,8 +401,8 @@ void gemm_int_packed_kernel(PArgs g) {
 #pragma unroll
     for (int am = 0; am < WMF; ++am)
 #pragma unroll
-    for (int blk = 0; blk < 2; ++blk) {
-        const uint32_t lcol = wn * 64 + blk * 32 + l32, col = n0 + lcol;
+    for (int blk = 0; blk < WNF; ++blk) {
+        const uint32_t lcol = wn * (BN / 2) + blk * 32 + l32, col = n0 + lcol;
         const uint32_t csum = col_sum[lcol];
         uint32_t old[16];
         if (g.epi == EPI_ALPHA_BETA) {
@@ -391,14 +427,15 @@ void gemm_int_packed_kernel(PArgs g) {
     }
 }
 
-template <typename E, int BM, bool EDGE, int WMF = 1> int launch_packed(hipStream_t st, PArgs g) {
-    constexpr size_t lds = PackedTile<BM, WMF>::LDS_BYTES;
-    auto kern = gemm_int_packed_kernel<E, BM, EDGE, WMF>;
+template <typename E, int BM, bool EDGE, int WMF = 1, int BN = TILE> int launch_packed(hipStream_t st, PArgs g) {
+    constexpr size_t lds = PackedTile<BM, WMF, BN>::LDS_BYTES;
+    auto kern = gemm_int_packed_kernel<E, BM, EDGE, WMF, BN>;
     static const hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
                                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     if (attr != hipSuccess) { (void)hipGetLastError(); return hip_code(attr); }
     g.tiles_m = (g.M + BM - 1) / BM;
-    hipLaunchKernelGGL(kern, dim3(g.tiles_m * g.tiles_n), dim3(PackedTile<BM, WMF>::NT), lds, st, g);
+    g.tiles_n = (g.N + BN - 1) / BN;
+    hipLaunchKernelGGL(kern, dim3(g.tiles_m * g.tiles_n), dim3(PackedTile<BM, WMF, BN>::NT), lds, st, g);
     return launch_status();
 }
 
@@ -459,6 +496,15 @@ template <typename E> int launch_typed(hipStream_t st, const GemmProblem &p, uns
         // i8 8192^3 1535 -> 1690; below one tile per CU the smaller tile wins: i8 2048^3 663 against 511).
         // These products move one byte per 170 operations even so and are bound by what the L2 delivers.
         const uint64_t tiles256 = ((p.M + 255) / 256) * ((p.N + TILE - 1) / TILE);
+        if constexpr (D == 1) {
+            // one digit: from one 256 x 256 tile per CU up that tile (64 x 128 per wavefront, 256 operations
+            // per byte fetched): i8 4096^3 1461 -> 1737 TOP/s, 8192^3 1736 -> 2034, 16384^3 1795 -> 2118
+            const uint64_t tiles256x256 = ((p.M + 255) / 256) * ((p.N + 255) / 256);
+            if (tiles256x256 >= (p.num_cus ? p.num_cus : 256u)) {
+                const bool edge = p.M % 256 != 0 || p.N % 256 != 0;
+                return edge ? launch_packed<E, 256, true, 2, 256>(st, g) : launch_packed<E, 256, false, 2, 256>(st, g);
+            }
+        }
         if (tiles256 >= (p.num_cus ? p.num_cus : 256u)) {
             const bool edge = p.M % 256 != 0 || p.N % TILE != 0;
             return edge ? launch_packed<E, 256, true, 2>(st, g) : launch_packed<E, 256, false, 2>(st, g);
