@@ -179,8 +179,8 @@ size_t wk_gemm_workspace_bytes(int dtype, int op_a, int op_b, uint64_t M, uint64
  * operands before every product (gemm.zig:713-719) although its callers' B is usually a weight
  * matrix that changes once per step; this is the entry point behind blas.PackedTensors.keepB.
  * The caller guarantees: the previous call that used this workspace was a wk_gemm or
- * wk_gemm_packed_b_kept with the same dtype, op_b, M, N, K and B contents (for cf32 / cf64 also the
- * same alpha, present or absent alike), and nothing else has written the workspace since.  A
+ * wk_gemm_packed_b_kept with the same dtype, op_b, M, N, K and B contents (for the complex types also
+ * the same alpha, present or absent alike), and nothing else has written the workspace since.  A
  * violated guarantee gives a wrong product, never an access outside the operands.  Problems that
  * do not use the workspace run exactly as under wk_gemm. */
 int    wk_gemm_packed_b_kept(wk_stream *s, int dtype, int op_a, int op_b, uint64_t M, uint64_t N, uint64_t K,
