@@ -70,7 +70,8 @@ def test_axpy_all_dtypes_shapes_alphas(dev, dtype):
         alphas += [0.75, -1.0 + 1e-9 if dtype.endswith("f64") else -1.0]
     if cx:
         alphas = [None, (2, 0), (2, 1), (0, 0)] + ([(-1, 0), (-1, -1)] if signed else [])
-    for shape in [(1,), (5,), (4,), (2, 3), (2, 2, 2), (3, 5, 7), (1000,), (4099,), (65536 + 3,), (2, 3, 4, 5)]:
+    for shape in [(1,), (5,), (4,), (2, 3), (2, 2, 2), (3, 5, 7), (1000,), (4099,), (65536 + 3,), (2, 3, 4, 5),
+                  (4, 1, 5), (3, 1, 70), (2, 3, 1, 7)]:
         for alpha in alphas:
             x = make_operand(dtype, shape, 7)
             y = make_operand(dtype, shape, 8)
@@ -100,6 +101,39 @@ def test_axpy_aligned_pitched_rows(dev, dtype):
                                            atol=1e-6 if dtype.endswith("f32") else 1e-14)
             else:
                 assert np.array_equal(got, want), f"{dtype} shape={shape} alpha={alpha}"
+
+
+@pytest.mark.parametrize("dtype", ALL_DTYPES)
+@pytest.mark.parametrize("shape", [(4, 1, 5), (3, 1, 70), (2, 3, 1, 7), (5, 1, 1)])
+def test_axpy_single_row_slices_with_padded_pitch(dev, dtype, shape):
+    """Slices of one row whose slice pitch is the padded row pitch (what a Tensor of shape
+    (4, 1, 5) looks like): the logical elements are not contiguous although every slice holds a
+    single row, so the contiguous-stream kernel must not be taken.  Gaps keep their poison."""
+    cx = oracle.is_complex(dtype)
+    depth, cols = int(np.prod(shape[:-2])), shape[-1]
+    tail = (2,) if cx else ()
+    x = make_operand(dtype, shape, 41)
+    y = make_operand(dtype, shape, 42)
+    alpha = (2, 1) if cx else 3
+    ve = max(1, 16 // (x.dtype.itemsize * (2 if cx else 1)))
+    for pitch in ((cols + ve - 1) // ve * ve + ve, cols + 3):       # 16-byte aligned rows; odd pitch
+        xs = np.full((depth, pitch) + tail, 55, dtype=x.dtype)
+        ys = np.full((depth, pitch) + tail, 66, dtype=y.dtype)
+        xs[:, :cols] = x.reshape((depth, cols) + tail)
+        ys[:, :cols] = y.reshape((depth, cols) + tail)
+        dx, dy = dev.upload(xs), dev.upload(ys)
+        dev.axpy(dtype, (depth, 1, cols), dx, pitch, pitch, alpha, dy, pitch, pitch)
+        dev.sync()
+        out = dy.download(ys.dtype, ys.shape)
+        dx.free(); dy.free()
+        assert (out[:, cols:] == 66).all(), "axpy wrote into the padding of a single-row slice"
+        got = np.ascontiguousarray(out[:, :cols]).reshape(y.shape)
+        want = expect(dtype, x, alpha, y)
+        if oracle.is_float(dtype) and cx:
+            np.testing.assert_allclose(got, want, rtol=1e-5 if dtype.endswith("f32") else 1e-13,
+                                       atol=1e-6 if dtype.endswith("f32") else 1e-14)
+        else:
+            assert np.array_equal(got, want), f"{dtype} shape={shape} pitch={pitch}"
 
 
 @pytest.mark.parametrize("dtype", ["f32", "f64", "i32", "u8", "cf32", "ci16"])
@@ -160,6 +194,8 @@ def test_axpy_invalid_arguments(dev):
     assert lib.wk_axpy(dev.stream, 8, s3, p, 4, 16, p, 8, 16, None) == 1      # pitch < cols
     assert lib.wk_axpy(dev.stream, 25, s3, p, 8, 16, p, 8, 16, None) == 9     # bad dtype
     assert lib.wk_axpy(dev.stream, 8, s3, None, 8, 16, p, 8, 16, None) == 1   # null
+    r1 = (ctypes.c_uint64 * 3)(2, 1, 8)
+    assert lib.wk_axpy(dev.stream, 8, r1, p, 0, 4, p, 8, 8, None) == 1        # slice pitch < row of one-row slices
     buf.free()
 
 

@@ -168,3 +168,61 @@ def test_adam_converges_on_a_quadratic():
     for t in range(1, 4001):
         w, m, v = onn.adam_update(w, 2 * w, m, v, 1e-2, 0.9, 0.999, 1e-8, t)
     assert np.all(np.abs(w) < 1e-3)
+
+
+@pytest.mark.parametrize("dt", FLOATS)
+@pytest.mark.parametrize("eps_kind", ["machine", "1e-8"])
+def test_adam_matches_the_library_routine_over_several_steps(dt, eps_kind):
+    """The reference has no Adam (src/nn/optimizers/adam.zig is empty), so the pin is the library
+    routine of the same rule: torch.optim.Adam on CPU tensors, epsilon added outside the
+    bias-corrected root.  Nine steps with fresh random gradients: a wrong exponent in a bias
+    correction, swapped betas or epsilon inside the root all show from step two on."""
+    torch = pytest.importorskip("torch")
+    rng = np.random.default_rng(17)
+    n = 257
+    lr, b1, b2 = 1e-3, 0.9, 0.999
+    eps = float(np.finfo(dt).eps) if eps_kind == "machine" else 1e-8
+    w = rng.standard_normal(n).astype(dt)
+    m = np.zeros(n, dt)
+    v = np.zeros(n, dt)
+    p = torch.tensor(w.copy(), requires_grad=True)
+    opt = torch.optim.Adam([p], lr=lr, betas=(b1, b2), eps=eps, foreach=False, fused=False)
+    m_scale = np.zeros(n)
+    for t in range(1, 10):
+        g = (rng.standard_normal(n) * 10.0 ** rng.integers(-3, 2, n)).astype(dt)
+        w, m, v = onn.adam_update(w, g, m, v, lr, b1, b2, eps, t)
+        m_scale = b1 * m_scale + (1 - b1) * np.abs(g)      # what the sum for m is rounded against
+        p.grad = torch.tensor(g.copy())
+        opt.step()
+        st = opt.state[p]
+        assert w.dtype == dt
+        # one unit in the last place of the weight per step taken (two rounded trajectories; a
+        # wrong rule moves a weight by about lr = 1e-3 per step); the moments to a few roundings
+        assert np.all(np.abs(p.detach().numpy() - w) <= t * np.spacing(np.abs(w).astype(dt))), t
+        assert np.all(np.abs(st["exp_avg"].numpy() - m) <= 8 * np.finfo(dt).eps * m_scale), t
+        assert np.allclose(st["exp_avg_sq"].numpy(), v, rtol=8 * np.finfo(dt).eps, atol=1e-30), t
+
+
+def test_adam_pin_sees_a_wrong_bias_correction():
+    """The comparison above is sharp enough to catch the mistakes it is there for."""
+    torch = pytest.importorskip("torch")
+    rng = np.random.default_rng(3)
+    n = 64
+    w0 = rng.standard_normal(n)
+    gs = [rng.standard_normal(n) for _ in range(5)]
+    p = torch.tensor(w0.copy(), requires_grad=True)
+    opt = torch.optim.Adam([p], lr=1e-3, betas=(0.9, 0.999), eps=1e-8, foreach=False, fused=False)
+    for g in gs:
+        p.grad = torch.tensor(g.copy())
+        opt.step()
+    want = p.detach().numpy()
+
+    def run(b1, b2, tshift):
+        w, m, v = w0.copy(), np.zeros(n), np.zeros(n)
+        for t, g in enumerate(gs, 1):
+            w, m, v = onn.adam_update(w, g, m, v, 1e-3, b1, b2, 1e-8, max(1, t + tshift))
+        return w
+
+    assert np.abs(run(0.9, 0.999, 0) - want).max() <= 1e-15
+    assert np.abs(run(0.999, 0.9, 0) - want).max() > 1e-5      # swapped betas
+    assert np.abs(run(0.9, 0.999, -1) - want).max() > 1e-5     # bias correction one step behind

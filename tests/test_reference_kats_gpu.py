@@ -70,6 +70,23 @@ def test_axpy_with_different_vector_configurations(env, dtype):
     assert np.array_equal(outs[0], kats.iota(dtype, (2, 3), scale=12))
 
 
+@pytest.mark.parametrize("dtype", ["f32", "f64", "i8", "u16", "i64", "cf32", "ci32"])
+@pytest.mark.parametrize("shape", [(4, 1, 5), (3, 1, 70), (2, 3, 1, 7)])
+def test_axpy_tensors_whose_slices_hold_one_padded_row(env, dtype, shape):
+    """Tensors with a row count of one and several slices: the row pitch is padded, so slices are
+    not back to back.  Every logical element must be updated and none skipped."""
+    context, pipeline = env
+    x_h = kats.iota(dtype, shape)
+    y_h = kats.iota(dtype, shape, scale=10)
+    x = upload(context, pipeline, dtype, x_h)
+    y = upload(context, pipeline, dtype, y_h)
+    blas.axpy(pipeline, x, kats.scalar(dtype, 2), y)
+    assert np.array_equal(download(pipeline, y), kats.iota(dtype, shape, scale=12))
+    assert np.array_equal(download(pipeline, x), x_h)
+    x.release(pipeline)
+    y.release(pipeline)
+
+
 def test_axpy_incompatible_tensor_shapes(env):
     """axpy.zig:763-815"""
     context, pipeline = env

@@ -157,8 +157,10 @@ int launch(wk_stream *s, const uint64_t shape3[3], const T *x, uint64_t xrp, uin
            uint64_t ysp, typename elem_traits<T>::acc alpha) {
     const uint64_t d = shape3[0], r = shape3[1], c = shape3[2];
     const uint64_t n = d * r * c;
-    const bool x_dense = (r == 1 || xrp == c) && (d == 1 || xsp == r * xrp);
-    const bool y_dense = (r == 1 || yrp == c) && (d == 1 || ysp == r * yrp);
+    // Dense = the logical elements are one contiguous run.  A single-row slice may still be padded
+    // (pitch > cols), so the slice pitch is held against rows * cols, not rows * row pitch.
+    const bool x_dense = (r == 1 || xrp == c) && (d == 1 || xsp == r * c);
+    const bool y_dense = (r == 1 || yrp == c) && (d == 1 || ysp == r * c);
     const bool aligned = ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(y)) & 15u) == 0;
     constexpr uint64_t VE = 16 / sizeof(T);
     if (x_dense && y_dense && aligned && n >= VE) {
@@ -198,6 +200,7 @@ extern "C" int wk_axpy(wk_stream *s, int dtype, const uint64_t shape3[3], const 
     if (!d || !r || !c) return WK_E_INVALID_VALUE;
     if (r > 1 && (x_row_pitch < c || y_row_pitch < c)) return WK_E_INVALID_VALUE;
     if (d > 1 && (x_slice_pitch < r * x_row_pitch || y_slice_pitch < r * y_row_pitch)) return WK_E_INVALID_VALUE;
+    if (d > 1 && (x_slice_pitch < r * c || y_slice_pitch < r * c)) return WK_E_INVALID_VALUE;
 
     return dispatch_dtype(dtype, [&]<typename T>() -> int {
         using A = typename elem_traits<T>::acc;
