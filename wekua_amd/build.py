@@ -37,7 +37,16 @@ def _run(cmd):
     return res.stdout
 
 
-def build_hip(verbose: bool = False, extra_flags=()) -> str:
+def _stale(obj: str, src: str) -> bool:
+    """True when `obj` is older than its source or than any header it may include."""
+    if not os.path.exists(obj):
+        return True
+    t = os.path.getmtime(obj)
+    deps = [src] + [os.path.join(d, f) for d in (CSRC, INCLUDE) for f in os.listdir(d) if f.endswith((".hpp", ".h", ".inc"))]
+    return any(os.path.getmtime(d) > t for d in deps)
+
+
+def build_hip(verbose: bool = False, extra_flags=(), incremental: bool = False) -> str:
     os.makedirs(OBJ, exist_ok=True)
     objs = []
     jobs = []
@@ -45,6 +54,8 @@ def build_hip(verbose: bool = False, extra_flags=()) -> str:
         for src in HIP_SOURCES:
             obj = os.path.join(OBJ, src.replace(".hip", ".o"))
             objs.append(obj)
+            if incremental and not _stale(obj, os.path.join(CSRC, src)):
+                continue
             cmd = [HIPCC] + HIP_FLAGS + list(extra_flags) + ["-c", os.path.join(CSRC, src), "-o", obj]
             jobs.append(pool.submit(_run, cmd))
         for j in jobs:
@@ -80,12 +91,12 @@ def build_example(verbose: bool = False) -> str:
     return exe
 
 
-def build_all(verbose: bool = False):
-    build_hip(verbose)
+def build_all(verbose: bool = False, incremental: bool = False):
+    build_hip(verbose, incremental=incremental)
     build_host(verbose)
     build_example(verbose)
 
 
 if __name__ == "__main__":
-    build_all(verbose=True)
+    build_all(verbose=True, incremental="--incremental" in sys.argv)
     print("built", LIB_HIP, LIB_HOST if os.path.exists(LIB_HOST) else "")
