@@ -46,6 +46,7 @@ enum {
     WK_E_OUT_OF_MEMORY = 8,            /* std.mem.Allocator.Error.OutOfMemory / hipErrorOutOfMemory */
     WK_E_TYPE_NOT_SUPPORTED = 9,       /* core.KernelsSet.Errors.TypeNotSupported (src/core/kernel.zig:151) */
     WK_E_NO_DEVICE = 10,               /* Context.init: DevicesArrayEmpty (src/core/context.zig:18) */
+    WK_E_SCRATCH_TOO_SMALL = 11,       /* an operand beyond the fixed scratch array of a *_static entry point */
     WK_E_HIP_BASE = 1000               /* WK_E_HIP_BASE + hipError_t: replaces cl.errors.OpenCLError */
 };
 
@@ -227,6 +228,17 @@ int  wk_gemm_bias_activation(wk_stream *s, int dtype, int op_a, int op_b, uint64
                              const void *bias, int kind);
 /* Linear.getBiasSensitivity: bias_grad[c] = sum_r sens[r][c] (src/nn/layer/kernels/bias_step.cl) */
 int  wk_bias_step(wk_stream *s, int dtype, uint64_t rows, uint64_t cols, const void *sens, uint64_t pitch, void *bias_grad);
+/* wk_bias_step for callers that cannot allocate device memory (code under HIP graph capture, tight
+ * serving loops, harnesses that forbid it).  No counterpart in the reference.  Same arguments, same
+ * kernels and bit for bit the same result, but the band partials live in an array that is part of the
+ * library's code object (WK_BIAS_STEP_STATIC_SCRATCH_BYTES per device, held until the process ends),
+ * whose address wk_device_open looks up once per device.  The call itself allocates and frees nothing.
+ * Limit: cols * element size <= WK_BIAS_STEP_STATIC_SCRATCH_BYTES / 2 (131072 f32 or 65536 f64 columns),
+ * beyond it WK_E_SCRATCH_TOO_SMALL; f32 / f64 only.  Every call on a device uses that device's one
+ * array: nothing in it has to start at zero (each partial is written before it is read), but two calls
+ * that overlap on one device -- on different streams or from different threads -- race. */
+#define WK_BIAS_STEP_STATIC_SCRATCH_BYTES (1u << 20)
+int  wk_bias_step_static(wk_stream *s, int dtype, uint64_t rows, uint64_t cols, const void *sens, uint64_t pitch, void *bias_grad);
 /* loss.mse kernel: err = expected - output; error = err^2; dev = -2*err when dev != NULL
  * (src/nn/loss/kernels/mse.cl:3-35, src/nn/loss/mse.zig:63-132) */
 int  wk_mse(wk_stream *s, int dtype, const uint64_t shape3[3], const void *output, uint64_t out_row_pitch, uint64_t out_slice_pitch,

@@ -60,6 +60,7 @@ def test_host_only_entry_points():
              9: "TypeNotSupported", 10: "DevicesArrayEmpty"}
     for code, name in names.items():
         assert lib.wk_strerror(code).decode() == name
+    assert lib.wk_strerror(11).decode().startswith("ScratchTooSmall")
     assert lib.wk_gemm_workspace_bytes(8, 0, 0, 8192, 8192, 8192) == 0
     assert lib.wk_gemm_force_variant(b"no-such-kernel") == 1
     assert lib.wk_gemm_force_variant(b"auto") == 0

@@ -74,6 +74,7 @@ SIGNATURES = {
     "wk_bias_activation": (ci, [vp, ci, ci, u64, u64, vp, u64, vp]),
     "wk_gemm_bias_activation": (ci, [vp, ci, ci, ci, u64, u64, u64, vp, u64, vp, u64, vp, u64, vp, ci]),
     "wk_bias_step": (ci, [vp, ci, u64, u64, vp, u64, vp]),
+    "wk_bias_step_static": (ci, [vp, ci, u64, u64, vp, u64, vp]),
     "wk_mse": (ci, [vp, ci, u64p, vp, u64, u64, vp, u64, u64, vp, u64, u64, vp, u64, u64]),
     "wk_sum_workspace_bytes": (sz, [ci]),
     "wk_sum": (ci, [vp, ci, u64p, vp, u64, u64, vp, vp, ctypes.c_double]),

@@ -49,6 +49,10 @@ inline int hip_code(hipError_t e) {
 // Every launch is followed by this: a bad launch configuration surfaces here, not later.
 inline int launch_status() { return hip_code(hipGetLastError()); }
 
+// Looks up this device's address of the static scratch array of wk_bias_step_static (wk_nn.hip);
+// wk_device_open calls it with the device current.
+int static_scratch_setup(int ordinal);
+
 inline int bind(wk_stream *s) {
     if (!s || !s->dev) return WK_E_INVALID_VALUE;
     WK_HIP_TRY(hipSetDevice(s->dev->ordinal));

@@ -9,6 +9,7 @@
 // logical region is touched.  f32 and f64 only (what the MLP configuration uses).
 #include "wk_internal.hpp"
 
+#include <atomic>
 #include <cmath>
 #include <cstring>
 
@@ -121,6 +122,15 @@ template <typename F> int dispatch_float(int dtype, F &&f) {
 constexpr int COLSUM_ROWS_PER_BAND = 32;
 constexpr int COLSUM_MAX_BANDS = 64;
 
+// Partials of wk_bias_step_static: part of the code object, so it exists on every device the library
+// is loaded on from load time until the process ends, and no call ever allocates it.  In host code
+// this name is only a handle for hipGetSymbolAddress; kernels get the per-device address below.
+constexpr size_t STATIC_SCRATCH_BYTES = WK_BIAS_STEP_STATIC_SCRATCH_BYTES;
+static __device__ __align__(256) unsigned char scratch[STATIC_SCRATCH_BYTES];
+
+constexpr int STATIC_SCRATCH_MAX_DEVICES = 64;
+std::atomic<void *> g_static_scratch[STATIC_SCRATCH_MAX_DEVICES];
+
 template <typename T>
 __global__ __launch_bounds__(256) void colsum_bands_kernel(const T *__restrict__ x, uint64_t rows, uint64_t cols, uint64_t pitch,
                                                            uint64_t band_rows, T *__restrict__ partial) {
@@ -173,6 +183,50 @@ __global__ __launch_bounds__(256) void sum_pass2_kernel(const T *__restrict__ pa
         __syncthreads();
     }
     if (threadIdx.x == 0) out[0] = red[0] * scale;
+}
+
+} // namespace
+
+// Called by wk_device_open with `ordinal` current: every device holds its own copy of the array at
+// its own address, so the address is looked up once per device and kept.
+int wk::static_scratch_setup(int ordinal) {
+    if (ordinal < 0 || ordinal >= STATIC_SCRATCH_MAX_DEVICES) return WK_OK; // such a device has no static entry point
+    if (g_static_scratch[ordinal].load(std::memory_order_acquire)) return WK_OK;
+    void *ptr = nullptr;
+    hipError_t e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+    if (e != hipSuccess) {
+        (void)hipGetLastError();
+        return hip_code(e);
+    }
+    if (!ptr) return WK_E_HIP_BASE + static_cast<int>(hipErrorInvalidSymbol);
+    g_static_scratch[ordinal].store(ptr, std::memory_order_release);
+    return WK_OK;
+}
+
+namespace {
+
+// Column sums of a rows x cols matrix in two launches of colsum_bands_kernel: bands of rows into
+// `partial_buf`, then the bands.  The number of bands depends only on (rows, cols, partial_bytes),
+// so two callers with equally sized buffers add in the same order and get the same bits.
+template <typename T>
+int colsum_two_pass(wk_stream *s, uint64_t rows, uint64_t cols, const T *sens, uint64_t pitch, T *bias_grad,
+                    void *partial_buf, size_t partial_bytes) {
+    uint64_t bands = (rows + COLSUM_ROWS_PER_BAND - 1) / COLSUM_ROWS_PER_BAND;
+    if (bands > COLSUM_MAX_BANDS) bands = COLSUM_MAX_BANDS;
+    const uint64_t fit = partial_bytes / (cols * sizeof(T));
+    if (bands > fit) bands = fit;
+    if (bands < 2) bands = 1; // one band writes the result directly
+    const uint64_t band_rows = (rows + bands - 1) / bands;
+    bands = (rows + band_rows - 1) / band_rows;
+    T *partial = bands > 1 ? static_cast<T *>(partial_buf) : bias_grad;
+    hipLaunchKernelGGL((colsum_bands_kernel<T>), dim3((unsigned)((cols + 63) / 64), (unsigned)bands), dim3(64, 4), 0,
+                       s->stream, sens, rows, cols, pitch, band_rows, partial);
+    int lrc = launch_status();
+    if (lrc || bands == 1) return lrc;
+    // second pass: the same kernel over the bands x cols matrix of partials, as one band
+    hipLaunchKernelGGL((colsum_bands_kernel<T>), dim3((unsigned)((cols + 63) / 64), 1), dim3(64, 4), 0, s->stream,
+                       static_cast<const T *>(partial), bands, cols, cols, bands, bias_grad);
+    return launch_status();
 }
 
 } // namespace
@@ -242,23 +296,27 @@ int wk_bias_step(wk_stream *s, int dtype, uint64_t rows, uint64_t cols, const vo
     if (!rows || !cols || !sens || !bias_grad || pitch < cols) return WK_E_INVALID_VALUE;
     if ((cols + 63) / 64 > 0x7fffffffull) return WK_E_INVALID_VALUE;
     return dispatch_float(dtype, [&]<typename T>() -> int {
-        // as many bands as the stream's scratch holds partials for; one band writes the result directly
-        uint64_t bands = (rows + COLSUM_ROWS_PER_BAND - 1) / COLSUM_ROWS_PER_BAND;
-        if (bands > COLSUM_MAX_BANDS) bands = COLSUM_MAX_BANDS;
-        const uint64_t fit = s->scratch_bytes / (cols * sizeof(T));
-        if (bands > fit) bands = fit;
-        if (bands < 2) bands = 1;
-        const uint64_t band_rows = (rows + bands - 1) / bands;
-        bands = (rows + band_rows - 1) / band_rows;
-        T *partial = bands > 1 ? static_cast<T *>(s->scratch) : static_cast<T *>(bias_grad);
-        hipLaunchKernelGGL((colsum_bands_kernel<T>), dim3((unsigned)((cols + 63) / 64), (unsigned)bands), dim3(64, 4), 0,
-                           s->stream, static_cast<const T *>(sens), rows, cols, pitch, band_rows, partial);
-        int lrc = launch_status();
-        if (lrc || bands == 1) return lrc;
-        // second pass: the same kernel over the bands x cols matrix of partials, as one band
-        hipLaunchKernelGGL((colsum_bands_kernel<T>), dim3((unsigned)((cols + 63) / 64), 1), dim3(64, 4), 0, s->stream,
-                           static_cast<const T *>(partial), bands, cols, cols, bands, static_cast<T *>(bias_grad));
-        return launch_status();
+        // as many bands as the stream's scratch holds partials for
+        return colsum_two_pass<T>(s, rows, cols, static_cast<const T *>(sens), pitch, static_cast<T *>(bias_grad), s->scratch,
+                                  s->scratch_bytes);
+    });
+}
+
+int wk_bias_step_static(wk_stream *s, int dtype, uint64_t rows, uint64_t cols, const void *sens, uint64_t pitch,
+                        void *bias_grad) {
+    int rc = bind(s);
+    if (rc) return rc;
+    if (!rows || !cols || !sens || !bias_grad || pitch < cols) return WK_E_INVALID_VALUE;
+    if (dtype != WK_F32 && dtype != WK_F64) return WK_E_TYPE_NOT_SUPPORTED;
+    const size_t esize = wk_dtype_size(dtype);
+    // at least two bands of partials must fit, whatever the row count: a row is at most half the array
+    if (cols > STATIC_SCRATCH_BYTES / 2 / esize) return WK_E_SCRATCH_TOO_SMALL;
+    const int ordinal = s->dev->ordinal;
+    void *ptr = ordinal < STATIC_SCRATCH_MAX_DEVICES ? g_static_scratch[ordinal].load(std::memory_order_acquire) : nullptr;
+    if (!ptr) return WK_E_INVALID_VALUE; // the device was not opened through wk_device_open
+    return dispatch_float(dtype, [&]<typename T>() -> int {
+        return colsum_two_pass<T>(s, rows, cols, static_cast<const T *>(sens), pitch, static_cast<T *>(bias_grad), ptr,
+                                  STATIC_SCRATCH_BYTES);
     });
 }
 

@@ -27,6 +27,7 @@ const char *wk_strerror(int code) {
     case WK_E_OUT_OF_MEMORY: return "OutOfMemory";
     case WK_E_TYPE_NOT_SUPPORTED: return "TypeNotSupported";
     case WK_E_NO_DEVICE: return "DevicesArrayEmpty";
+    case WK_E_SCRATCH_TOO_SMALL: return "ScratchTooSmall: the operand exceeds the fixed scratch array of this entry point";
     default: break;
     }
     if (code >= WK_E_HIP_BASE) return hipGetErrorString(static_cast<hipError_t>(code - WK_E_HIP_BASE));
@@ -71,6 +72,11 @@ int wk_device_open(int ordinal, wk_device **out) {
         (void)hipGetLastError();
         delete d;
         return hip_code(e);
+    }
+    rc = static_scratch_setup(ordinal);
+    if (rc) {
+        delete d;
+        return rc;
     }
     *out = d;
     return WK_OK;
