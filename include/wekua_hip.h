@@ -197,8 +197,11 @@ const char *wk_gemm_variant_with_workspace(int dtype, int op_a, int op_b, uint64
                                            uint64_t lda, uint64_t ldb, uint64_t ldc, const void *A, const void *B,
                                            const void *C, size_t workspace_bytes);
 
-/* Test/benchmark knob: force a gemm variant by name ("auto" restores selection).
- * Returns WK_E_INVALID_VALUE for an unknown name. */
+/* Test and benchmark knob only, not for product code: force a gemm variant by name ("auto" restores
+ * selection).  Process-wide, read by every wk_gemm call on every stream; changing it while a
+ * PackedTensors keeps B invalidates what that handle remembers.  A forced variant whose kernel
+ * cannot take the problem (a dimension or leading dimension of 2^31 or more) makes wk_gemm return
+ * WK_E_INVALID_VALUE.  Returns WK_E_INVALID_VALUE for an unknown name. */
 int wk_gemm_force_variant(const char *name);
 
 /* ---- around the hot path: what one MLP training step needs besides gemm / axpy -----------------

@@ -252,6 +252,17 @@ def test_packed_tensors_keep_b_across_calls(dtype, shape):
         wk.memory.readFromBuffer(pipeline, B, b1)
         product(B_other, a2, b2)                 # another tensor: packed afresh
         product(B, a2, b1)                       # and back
+        # B released and another tensor created in its place (same shape: the allocators hand back the
+        # same host object and device block more often than not): a different tensor, so it is packed
+        # afresh although every address may match the kept one
+        for _ in range(3):
+            product(B, a2, b1)
+            B.release(pipeline)
+            B = wk.Tensor.alloc(dtype, context, pipeline, (N, K))
+            wk.memory.readFromBuffer(pipeline, B, b2)
+            product(B, a2, b2)
+            wk.memory.readFromBuffer(pipeline, B, b1)
+            packed.invalidateB()
         packed.keepB(False)
         wk.memory.readFromBuffer(pipeline, B, b2)
         product(B, a2, b2)                       # off: every call packs both, as the reference does

@@ -39,6 +39,39 @@ def test_binding_covers_every_declared_symbol():
     assert declared == bound, f"unbound: {declared - bound}; undeclared: {bound - declared}"
 
 
+def _split_args(arglist):
+    """Top-level comma split of a parameter list (brackets of `[3]u64`, `[*:0]const u8` stay whole)."""
+    out, depth, cur = [], 0, ""
+    for ch in arglist:
+        if ch in "([":
+            depth += 1
+        elif ch in ")]":
+            depth -= 1
+        if ch == "," and depth == 0:
+            out.append(cur)
+            cur = ""
+        else:
+            cur += ch
+    if cur.strip() and cur.strip() != "void":
+        out.append(cur)
+    return out
+
+
+def test_zig_binding_in_the_integration_guide_matches_the_header():
+    """The `extern fn` block a wekua maintainer would paste declares exactly the functions of the
+    header, each with the header's number of parameters."""
+    text = re.sub(r"/\*.*?\*/", "", open(HEADER).read(), flags=re.S)
+    header = {m.group(1): len(_split_args(m.group(2)))
+              for m in re.finditer(r"\b(wk_[a-z0-9_]+)\s*\(([^;{]*?)\)\s*;", text, flags=re.S)}
+    doc = open(os.path.join(ROOT, "INTEGRATION.md")).read()
+    zig = {m.group(1): len(_split_args(m.group(2)))
+           for m in re.finditer(r"pub extern fn (wk_[a-z0-9_]+)\(([^;]*?)\)\s*[^;()]*;", doc, flags=re.S)}
+    assert set(header) == set(declared_functions())
+    assert set(zig) == set(header), f"not in the guide: {set(header) - set(zig)}; not in the header: {set(zig) - set(header)}"
+    wrong = {n: (header[n], zig[n]) for n in header if header[n] != zig[n]}
+    assert not wrong, f"parameter counts differ (header, guide): {wrong}"
+
+
 def test_header_compiles_as_plain_c():
     """The boundary is a C ABI: the header must be valid C, not only C++."""
     src = '#include "wekua_hip.h"\nint main(void){ int (*f)(wk_stream*, int, int, int, uint64_t, uint64_t, uint64_t, const void*, const void*, uint64_t, const void*, uint64_t, const void*, void*, uint64_t, void*, size_t) = wk_gemm; return f != wk_gemm; }\n'

@@ -242,6 +242,17 @@ def test_invalid_arguments(dev):
     assert lib.wk_gemm(dev.stream, 20, 0, 0, 4, 4, 4, None, p, 4, p, 4, None, p, 4, None, 0) == 9
     assert lib.wk_gemm(dev.stream, 8, 0, 0, 4, 4, 4, None, None, 4, p, 4, None, p, 4, None, 0) == 1
     assert lib.wk_gemm(None, 8, 0, 0, 4, 4, 4, None, p, 4, p, 4, None, p, 4, None, 0) == 1
+    # a forced matrix-core variant does not get past the 32-bit limits of its kernel either
+    # (automatic selection sends such a problem to the generic kernel); nothing is launched
+    for name, dt in ((b"mfma_f32_64x64", 8), (b"mfma_f64_64x64", 9), (b"mfma_i32_64x128", 4)):
+        if lib.wk_gemm_force_variant(name) != 0:
+            continue
+        try:
+            assert lib.wk_gemm(dev.stream, dt, 0, 0, 4, 4, 4, None, p, 2 ** 31, p, 4, None, p, 4, None, 0) == 1
+            assert lib.wk_gemm(dev.stream, dt, 0, 0, 4, 4, 4, None, p, 4, p, 2 ** 31, None, p, 4, None, 0) == 1
+            assert lib.wk_gemm(dev.stream, dt, 0, 0, 4, 4, 4, None, p, 4, p, 4, None, p, 2 ** 31, None, 0) == 1
+        finally:
+            lib.wk_gemm_force_variant(b"auto")
     buf.free()
 
 

@@ -528,6 +528,10 @@ size_t wk::gemm_int_packed_workspace_bytes(int dtype, uint64_t M, uint64_t N, ui
 int wk::gemm_int_packed_launch(hipStream_t st, const GemmProblem &p, void *workspace, size_t workspace_bytes) {
     const size_t need = gemm_int_packed_workspace_bytes(p.dtype, p.M, p.N, p.K);
     if (!need || !workspace || workspace_bytes < need || (reinterpret_cast<uintptr_t>(workspace) & 15u)) return WK_E_INVALID_VALUE;
+    // 32-bit extents and leading dimensions inside the pack pass and the product kernel
+    if (p.M > 0x7fffffffull || p.N > 0x7fffffffull || p.K > 0x7fffffffull || p.lda > 0x7fffffffull ||
+        p.ldb > 0x7fffffffull || p.ldc > 0x7fffffffull)
+        return WK_E_INVALID_VALUE;
     const Layout w = make_layout(digits_of(p.dtype), p.M, p.N, p.K);
     unsigned char *ws = static_cast<unsigned char *>(workspace);
     switch (digits_of(p.dtype)) {

@@ -1194,6 +1194,11 @@ int wk::gemm_mfma_pick(const GemmProblem &p) {
 
 int wk::gemm_mfma_launch(hipStream_t st, const GemmProblem &p, int variant) {
     if (variant < 0 || variant >= k_num_variants || k_variants[variant].dtype != p.dtype) return WK_E_INVALID_VALUE;
+    // the kernels index with 32 bits per dimension; automatic selection never gets here with more
+    // (gemm_mfma_pick declines), a forced variant is turned away
+    if (p.M > 0x7fffffffull || p.N > 0x7fffffffull || p.K > 0x7fffffffull || p.lda > 0x7fffffffull ||
+        p.ldb > 0x7fffffffull || p.ldc > 0x7fffffffull)
+        return WK_E_INVALID_VALUE;
     const VariantDesc &v = k_variants[variant];
     const uint64_t tiles = ((p.M + v.bm - 1) / v.bm) * ((p.N + v.bn - 1) / v.bn);
     if (tiles > 0x7fffffffull) return WK_E_INVALID_VALUE;

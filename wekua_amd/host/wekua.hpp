@@ -41,6 +41,7 @@
 #include <cstring>
 #include <exception>
 #include <limits>
+#include <atomic>
 #include <optional>
 #include <string>
 #include <type_traits>
@@ -221,6 +222,13 @@ struct CreateConfig {
     bool vectors_enabled = true; // src/tensor/main.zig:35-39 (cl_mem_flags / host_ptr have no HIP meaning)
 };
 
+namespace detail {
+inline uint64_t nextTensorSerial() {
+    static std::atomic<uint64_t> counter{0};
+    return counter.fetch_add(1, std::memory_order_relaxed) + 1;
+}
+} // namespace detail
+
 template <typename T> struct Tensor {
     struct Dimensions {
         std::vector<uint64_t> shape, vl_shape, pitches;
@@ -242,6 +250,9 @@ template <typename T> struct Tensor {
 
     const Context *context = nullptr;
     void *buffer = nullptr; // device memory (hipMalloc)
+    // Unique per tensor ever created in this process (never reused, unlike the address of the object
+    // or of its buffer): what a cache keyed on "this tensor" compares.  No counterpart in the reference.
+    uint64_t serial = 0;
     Dimensions dimensions;
     MemoryLayout memory_layout;
     Flags flags;
@@ -271,6 +282,7 @@ template <typename T> struct Tensor {
 
         Tensor *t = new Tensor;
         t->context = context;
+        t->serial = detail::nextTensorSerial();
         t->dimensions.shape = shape;
         t->dimensions.vl_shape = shape;
 
@@ -765,27 +777,38 @@ template <typename T> struct PackedTensors {
     // first with the same B tensor, op_b, queue and alpha (alpha is folded into the packed B of the
     // complex types) leave B's packed form in the workspace as it is and pack only A.  After B's
     // contents change, invalidateB() makes the next call pack it again.
+    // B is recognised by the tensor's serial (a released B whose address a new tensor reuses is a
+    // different tensor), its buffer and its row pitch, and is recorded only once a product with it
+    // has been enqueued without error.
     bool keep_b = false;
-    const Tensor<T> *kept_b = nullptr;
+    uint64_t kept_b_serial = 0; // 0: the workspace holds no B
+    const void *kept_b_buffer = nullptr;
+    uint64_t kept_b_pitch = 0;
     Operation kept_op_b = Operation::no_transpose;
     const void *kept_stream = nullptr;
     std::optional<T> kept_alpha;
     void keepB(bool on) {
         keep_b = on;
-        kept_b = nullptr;
+        kept_b_serial = 0;
     }
-    void invalidateB() { kept_b = nullptr; }
-    // true when the workspace holds this B already; records the operand otherwise
-    bool holdsB(const Tensor<T> *b, Operation op_b, const void *stream, const std::optional<T> &alpha) {
-        if (!keep_b) return false;
+    void invalidateB() { kept_b_serial = 0; }
+    // true when the workspace holds this B already
+    bool holdsB(const Tensor<T> *b, Operation op_b, const void *stream, const std::optional<T> &alpha) const {
+        if (!keep_b || kept_b_serial == 0) return false;
         const bool same_alpha = alpha.has_value() == kept_alpha.has_value() &&
                                 (!alpha || std::memcmp(&*alpha, &*kept_alpha, sizeof(T)) == 0);
-        if (kept_b == b && kept_op_b == op_b && kept_stream == stream && same_alpha) return true;
-        kept_b = b;
+        return kept_b_serial == b->serial && kept_b_buffer == b->buffer && kept_b_pitch == b->memory_layout.row_pitch &&
+               kept_op_b == op_b && kept_stream == stream && same_alpha;
+    }
+    // after a product with this B went through
+    void recordB(const Tensor<T> *b, Operation op_b, const void *stream, const std::optional<T> &alpha) {
+        if (!keep_b) return;
+        kept_b_serial = b->serial;
+        kept_b_buffer = b->buffer;
+        kept_b_pitch = b->memory_layout.row_pitch;
         kept_op_b = op_b;
         kept_stream = stream;
         kept_alpha = alpha;
-        return false;
     }
 
     static PackedTensors *init(Pipeline *pipeline, Tensor<T> *result_tensor, uint64_t k_size, bool vectors_enabled) {
@@ -865,11 +888,16 @@ void gemm(Pipeline *pipeline, std::optional<T> alpha, Tensor<T> *a, Operation op
     const T av = alpha.value_or(T{}), bv = beta.value_or(T{});
     wk_stream *stream = pipeline->command_queue->stream;
     const bool b_kept = packed_tensors && packed_tensors->holdsB(b, op_b, stream, alpha);
-    check((b_kept ? wk_gemm_packed_b_kept : wk_gemm)(
+    const int rc = (b_kept ? wk_gemm_packed_b_kept : wk_gemm)(
         stream, core::getTypeIndex<T>(), (int)op_a, (int)op_b, M, N, K, alpha ? &av : nullptr, a->buffer,
         a->memory_layout.row_pitch, b->buffer, b->memory_layout.row_pitch, beta ? &bv : nullptr, c->buffer,
         c->memory_layout.row_pitch, packed_tensors ? packed_tensors->workspace : nullptr,
-        packed_tensors ? packed_tensors->workspace_bytes : 0));
+        packed_tensors ? packed_tensors->workspace_bytes : 0);
+    if (packed_tensors) {
+        if (rc) packed_tensors->invalidateB(); // whatever the workspace holds now, it is not trusted
+        else packed_tensors->recordB(b, op_b, stream, alpha);
+    }
+    check(rc);
     pipeline->append(1);
 }
 
