@@ -5,14 +5,26 @@ A "step" is one call of the headline workload: f32 GEMM C = 1.5*A*B + 0.5*C at
 M = N = K = 8192 (no transposes), operands resident in HBM.  The AXPY half of the metric
 (y = 0.75*x + y, f32, n = 2^28) is measured in the same run and reported beside it.
 
-Prints ONE JSON line:  metric/value/unit as BASELINE.json names them, `roofline` for the
-GEMM kernel (MFMA-bound), `axpy` with its own HBM roofline, and `cpu_baseline`: the
-reference-order CPU restatement (oracle/) timed on this box's host cores on a bounded
-sample of the same GEMM.  The oracle is used here only as that timed baseline.
+Prints ONE JSON line:
+  metric / value / unit   as the benchmark definition names them (the headline GEMM, wall clock);
+  roofline                the headline GEMM kernel against the f32 matrix peak, from events on its stream;
+  axpy                    f32 / f64 at n = 2^28 against the HBM peak, the same kernel under two placements
+                          of x and y (same offset inside a 4 KiB block; y 3 KiB further in), and the CPU
+                          baseline for every AXPY size;
+  configs                 every GEMM and AXPY benchmark configuration (512^3; 1024..8192^3 x NN/NT/TN/TT;
+                          1000^3 and 4097x4095x4093 x 4; f64 4096^3 and 8192x256x8192; int32 2048^3; AXPY
+                          2^20 / 2^24 / 2^28 x f32 / f64), each with its own roofline fraction;
+  mlp_step                the MLP training step;
+  cpu_baseline            the reference-order CPU restatement (oracle/) timed on this box's host cores
+                          on the headline GEMM; `cpu_baselines` holds the other shapes it was timed on;
+  perf_floor              the two rates a regression must not pass unnoticed; the exit status is 3 when
+                          one is missed (the JSON line is printed either way; --no-floor disables it).
+The oracle is used here only as that timed baseline.
 """
 from __future__ import annotations
 
 import argparse
+import ctypes
 import json
 import os
 import sys
@@ -25,6 +37,8 @@ sys.path.insert(0, ROOT)
 
 F32_MATRIX_PEAK_TFLOPS = 157.3   # MI355X dense f32 matrix peak
 HBM_PEAK_GBS = 8000.0            # MI355X HBM3E
+FLOOR_GEMM_TFLOPS = 130.0        # f32 8192^3 NN (measured 139-144 across boxes)
+FLOOR_AXPY_GBS = 6600.0          # f32 n = 2^28 (measured 6820-6860 across boxes)
 
 
 def log(*a):
@@ -32,7 +46,8 @@ def log(*a):
 
 
 def read_traffic(name: str):
-    """HBM bytes per launch measured with rocprofv3 --pmc (FETCH_SIZE / WRITE_SIZE), if recorded."""
+    """HBM bytes per launch recorded from a rocprofv3 --pmc run (FETCH_SIZE / WRITE_SIZE) of this
+    command; not measured in this run."""
     path = os.path.join(ROOT, "profiles", "traffic.json")
     try:
         with open(path) as f:
@@ -74,7 +89,6 @@ def gemm_leg(wk, synth, n, steps, warmup):
     # recorded on the pipeline's own stream around the same launches give the kernel time.
     stream = wk._lib().wkz_context_stream(ctx._h, 0)
     device = wk._lib().wkz_context_device(ctx._h)
-    import ctypes
     e0, e1 = ctypes.c_void_p(), ctypes.c_void_p()
     wk._capi.check(lib.wk_event_create(device, ctypes.byref(e0)))
     wk._capi.check(lib.wk_event_create(device, ctypes.byref(e1)))
@@ -102,37 +116,72 @@ def gemm_leg(wk, synth, n, steps, warmup):
     }
 
 
-def axpy_leg(dev, raw, synth, dtype, log2n, steps, warmup):
+def axpy_placement_leg(dev, raw, dtype, log2n, steps, warmup):
+    """wk_axpy at n = 2^log2n on operands placed by hand inside two device blocks: x at the start of
+    a 4 KiB block, y once at the same offset inside its own (where two fresh device allocations put
+    them) and once 3 KiB further in (what the library's allocator gives neighbours in allocation
+    order).  Same kernel, same data; only the distance between the base addresses differs."""
     rd = raw.real_np_dtype(dtype)
     n = 1 << log2n
-    x = synth.uniform(synth.config_seed(2, 0), (n,), rd)
-    y = synth.uniform(synth.config_seed(2, 1), (n,), rd)
-    dx, dy = dev.upload(x), dev.upload(y)
+    nbytes = n * rd.itemsize
+    bx, by = dev.malloc(nbytes + 16384), dev.malloc(nbytes + 16384)
+    up = lambda p: (p + 4095) // 4096 * 4096
+    x0, y0 = up(bx.ptr.value), up(by.ptr.value)
+    did = raw.dtype_id(dtype)
+    s3 = (ctypes.c_uint64 * 3)(1, 1, n)
+    lo, span = raw.scalar_bytes(dtype, -1.0), raw.scalar_bytes(dtype, 2.0)
+    for seed, p in ((21, x0), (22, y0)):
+        raw.check(dev.lib.wk_random_uniform(dev.stream, did, (ctypes.c_uint64 * 3)(1, 1, n + 3072 // rd.itemsize),
+                                            ctypes.c_void_p(p), n + 3072 // rd.itemsize, n + 3072 // rd.itemsize, seed,
+                                            ctypes.cast(lo, ctypes.c_void_p), ctypes.cast(span, ctypes.c_void_p)),
+                  "wk_random_uniform")
+    alpha = raw.scalar_bytes(dtype, 0.75)
+    out = {}
+    for name, yp in (("same_offset_in_4KiB", y0), ("y_plus_3KiB", y0 + 3072)):
+        def step():
+            raw.check(dev.lib.wk_axpy(dev.stream, did, s3, ctypes.c_void_p(x0), n, n, ctypes.c_void_p(yp), n, n,
+                                      ctypes.cast(alpha, ctypes.c_void_p)), "wk_axpy")
+        for _ in range(warmup):
+            step()
+        dev.sync()
+        ms = dev.time_stream_ms(step, steps)
+        out[name] = 3.0 * nbytes / ms / 1e6
+    bx.free()
+    by.free()
+    return out
 
-    def step():
-        dev.axpy(dtype, (1, 1, n), dx, n, n, 0.75, dy, n, n)
 
-    for _ in range(warmup):
-        step()
-    dev.sync()
-    ms = dev.time_stream_ms(step, steps)
-    dx.free()
-    dy.free()
-    nbytes = 3.0 * n * rd.itemsize
-    return {"dtype": dtype, "n": n, "us": ms * 1e3, "gbs": nbytes / ms / 1e6, "bytes": nbytes}
-
-
-def cpu_baseline_leg(a, b, rows, threads):
-    """The reference CPU device's algorithm (packed path, block 16, 8 f32 lanes) on the first
-    `rows` rows of the same 8192^3 product, timed on this host."""
+def cpu_gemm_leg(dtype, M, N, K, alpha, beta, threads, a=None, b=None):
+    """The reference CPU device's algorithm (packed path, block 16, 8 lanes for f32) timed on this host."""
     import oracle
-    n = a.shape[1]
-    a_s = np.ascontiguousarray(a[:rows])
-    c_s = np.zeros((rows, n), dtype=np.float32)
+    from wekua_amd import synth
+    rd = oracle.real_np_dtype(dtype)
+    if a is None:
+        if rd.kind == "f":
+            a, b = synth.uniform(1, (M, K), rd), synth.uniform(2, (K, N), rd)
+        else:
+            a, b = synth.integers(1, (M, K), rd, -100, 100), synth.integers(2, (K, N), rd, -100, 100)
+    c = np.zeros((M, N), dtype=rd)
     t0 = time.perf_counter()
-    oracle.gemm("f32", 1.5, a_s, 0, b, 0, 0.5, c_s, vector_width=8, packed=True, threads=threads)
+    oracle.gemm(dtype, alpha, a, 0, b, 0, beta, c, vector_width=8, packed=True, threads=threads)
     dt = time.perf_counter() - t0
-    return {"seconds": dt, "tflops": 2.0 * rows * n * n / dt / 1e12}
+    return {"seconds": dt, "rate": 2.0 * M * N * K / dt / 1e12}
+
+
+def cpu_axpy_leg(dtype, log2n, threads, reps):
+    """axpy.cl's element-wise kernel with its work-items spread over the host threads, in place."""
+    import oracle
+    rd = oracle.real_np_dtype(dtype)
+    n = 1 << log2n
+    rng = np.random.default_rng(log2n)
+    x = rng.random(n, dtype=rd) * 2 - 1
+    y = rng.random(n, dtype=rd) * 2 - 1
+    oracle.axpy_inplace(dtype, x, 0.75, y, contract=True, threads=threads)   # first touch, thread start-up
+    t0 = time.perf_counter()
+    for _ in range(reps):
+        oracle.axpy_inplace(dtype, x, 0.75, y, contract=True, threads=threads)
+    dt = (time.perf_counter() - t0) / reps
+    return {"seconds": dt, "gbs": 3.0 * n * rd.itemsize / dt / 1e9}
 
 
 def main():
@@ -144,7 +193,9 @@ def main():
     ap.add_argument("--axpy-log2n", type=int, default=28)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-rows", type=int, default=8192)
-    ap.add_argument("--no-mlp", action="store_true", help="skip the MLP training step leg (BASELINE configuration 5)")
+    ap.add_argument("--no-mlp", action="store_true", help="skip the MLP training step leg (benchmark configuration 5)")
+    ap.add_argument("--no-configs", action="store_true", help="skip the sweep over the other benchmark configurations")
+    ap.add_argument("--no-floor", action="store_true", help="do not turn a missed performance floor into exit status 3")
     ap.add_argument("--calibrate", action="store_true",
                     help="also launch the plain 1 GiB copy kernel a few times, so that a profiler run of this "
                          "command holds a kernel of known HBM traffic to scale byte counters against")
@@ -155,7 +206,7 @@ def main():
         sys.exit(2)
 
     import wekua_amd as wk                # fails loudly if the native libraries are missing
-    from wekua_amd import raw, synth
+    from wekua_amd import benchmark, raw, synth
 
     g = gemm_leg(wk, synth, args.n, args.steps, args.warmup)
     dev = raw.Device(0)
@@ -164,10 +215,10 @@ def main():
     log(f"[bench] gemm f32 {args.n}^3 [{g['variant']}]: {g['kernel_ms']:.3f} ms/launch (events), "
         f"{g['wall_ms']:.3f} ms/step (wall) -> {g['tflops_kernel']:.1f} TFLOP/s")
 
-    ax = axpy_leg(dev, raw, synth, "f32", args.axpy_log2n, max(args.steps, 20), args.warmup)
-    ax64 = axpy_leg(dev, raw, synth, "f64", args.axpy_log2n, max(args.steps, 20), args.warmup)
-    log(f"[bench] axpy f32 2^{args.axpy_log2n}: {ax['us']:.1f} us -> {ax['gbs']:.0f} GB/s; "
-        f"f64: {ax64['us']:.1f} us -> {ax64['gbs']:.0f} GB/s")
+    place = {dt: axpy_placement_leg(dev, raw, dt, args.axpy_log2n, max(args.steps, 20), args.warmup) for dt in ("f32", "f64")}
+    for dt in ("f32", "f64"):
+        log(f"[bench] axpy {dt} 2^{args.axpy_log2n} by placement of y against x: same offset inside a 4 KiB block "
+            f"{place[dt]['same_offset_in_4KiB']:.0f} GB/s, 3 KiB further in {place[dt]['y_plus_3KiB']:.0f} GB/s")
     if args.calibrate:
         nbytes = 1 << 30
         src, dst = dev.malloc(nbytes), dev.malloc(nbytes)
@@ -179,46 +230,77 @@ def main():
         dst.free()
     dev.close()
 
+    # every benchmark configuration through the reference-shaped API (tensors from Tensor.alloc, so with
+    # the library's own pitches and placement), operands drawn on the device
+    configs = None
+    if not args.no_configs:
+        ses = benchmark.Session()
+        try:
+            configs = benchmark.run_baseline_configs(ses, log=lambda m: log("[bench] " + m))
+        finally:
+            ses.close()
+    ax_key = f"2_axpy_f32_2p{args.axpy_log2n}"
+    if configs and ax_key in configs:
+        ax_gbs, ax_us = configs[ax_key]["value"], configs[ax_key]["ms"] * 1e3
+        ax64 = configs[f"2_axpy_f64_2p{args.axpy_log2n}"]
+    else:   # the sweep was skipped: the coloured placement stands for the tensors' own
+        ax_gbs = place["f32"]["y_plus_3KiB"]
+        ax_us = 3.0 * 4 * (1 << args.axpy_log2n) / ax_gbs / 1e3
+        ax64 = {"value": place["f64"]["y_plus_3KiB"], "ms": 3.0 * 8 * (1 << args.axpy_log2n) / place["f64"]["y_plus_3KiB"] / 1e6}
+
     mlp = None
     if not args.no_mlp:
-        from wekua_amd import benchmark
         m = benchmark.time_mlp_step(steps=max(args.steps, 10), warmup=args.warmup)
         log(f"[bench] mlp step 1024-4096-4096-1024 f32 batch 2048 adam: {m['stream_ms']:.3f} ms/step "
             f"-> {m['tflops']:.1f} TFLOP/s over its GEMM flops")
         mlp = {"workload": "MLP training step 1024-4096-4096-1024, f32, batch 2048, tanh/tanh/sigmoid, MSE, Adam lr=1e-3 "
-                           "(BASELINE config 5): forward + loss + backward + update",
+                           "(benchmark configuration 5): forward + loss + backward + update",
                "ms_per_step": m["stream_ms"], "wall_ms_per_step": m["wall_ms"], "gemm_flops_per_step": m["flops"],
-               "value": m["tflops"], "unit": "TFLOP/s", "frac_of_f32_matrix_peak": m["tflops"] / F32_MATRIX_PEAK_TFLOPS}
-
-    other = None
-    if not args.no_mlp:   # the remaining benchmark configurations, a few launches each
-        from wekua_amd import benchmark
-        ses = benchmark.Session()
-        try:
-            other = {}
-            for key, dtype, (M, N, K), alpha, beta, unit in (("f64_gemm_4096", "f64", (4096, 4096, 4096), 1.0, 1.0, "TFLOP/s"),
-                                                             ("f64_gemm_8192x256x8192", "f64", (8192, 256, 8192), 1.0, 1.0, "TFLOP/s"),
-                                                             ("i32_gemm_2048", "i32", (2048, 2048, 2048), 3, -2, "TOP/s"),
-                                                             ("f32_gemm_1000", "f32", (1000, 1000, 1000), 1.5, 0.5, "TFLOP/s"),
-                                                             ("f32_gemm_4097x4095x4093", "f32", (4097, 4095, 4093), 1.5, 0.5, "TFLOP/s")):
-                ms, variant = benchmark.time_gemm(ses, dtype, M, N, K, 0, 0, alpha, beta)
-                other[key] = {"ms": ms, "value": 2.0 * M * N * K / ms / 1e9, "unit": unit, "kernel": variant}
-                log(f"[bench] {key}: {ms:.4f} ms -> {other[key]['value']:.1f} {unit} [{variant}]")
-        finally:
-            ses.close()
+               "value": m["tflops"], "unit": "TFLOP/s",
+               "roofline": {"bound": "mfma", "achieved": m["tflops"], "peak": F32_MATRIX_PEAK_TFLOPS, "unit": "TFLOP/s",
+                            "frac": m["tflops"] / F32_MATRIX_PEAK_TFLOPS}}
 
     cpu = None
+    cpu_all = None
+    axpy_cpu = None
     if not args.no_cpu_baseline:
         cores = min(os.cpu_count() or 1, int(os.environ.get("OMP_NUM_THREADS", "16") or 16), 16)
         rows = min(args.cpu_rows, args.n)
         log(f"[bench] cpu baseline: reference-order restatement, {rows} of {args.n} rows, {cores} threads ...")
-        c = cpu_baseline_leg(g["a"], g["b"], rows, cores)
-        log(f"[bench] cpu baseline: {c['seconds']:.1f}s -> {c['tflops'] * 1e3:.1f} GFLOP/s")
+        c = cpu_gemm_leg("f32", rows, args.n, args.n, 1.5, 0.5, cores, np.ascontiguousarray(g["a"][:rows]), g["b"])
+        log(f"[bench] cpu baseline: {c['seconds']:.1f}s -> {c['rate'] * 1e3:.1f} GFLOP/s")
+        kind = "reference CPU-device algorithm (packed path, block 16, 8 lanes), one call"
         cpu = {
-            "value": c["tflops"], "unit": "TFLOP/s", "cores": cores, "kind": "port",
-            "sample": f"rows 0..{rows - 1} of the same {args.n}^3 f32 GEMM ({rows}x{args.n}x{args.n}), "
-                      "reference CPU-device algorithm (packed path, block 16, 8 lanes), one call",
+            "value": c["rate"], "unit": "TFLOP/s", "cores": cores, "kind": "port",
+            "sample": f"rows 0..{rows - 1} of the same {args.n}^3 f32 GEMM ({rows}x{args.n}x{args.n}), {kind}",
         }
+        cpu_all = {}
+        for key, dtype, (M, N, K), alpha, beta, unit in (("1_f32_gemm_512_NN", "f32", (512, 512, 512), 1.0, 0.0, "TFLOP/s"),
+                                                         ("3_f32_gemm_1024_NN", "f32", (1024, 1024, 1024), 1.5, 0.5, "TFLOP/s"),
+                                                         ("3_f32_gemm_2048_NN", "f32", (2048, 2048, 2048), 1.5, 0.5, "TFLOP/s"),
+                                                         ("4_i32_gemm_2048_NN", "i32", (2048, 2048, 2048), 3, -2, "TOP/s")):
+            cpu_gemm_leg(dtype, 256, 256, 256, alpha, beta, cores)   # thread start-up outside the timed call
+            r = cpu_gemm_leg(dtype, M, N, K, alpha, beta, cores)
+            cpu_all[key] = {"value": r["rate"], "unit": unit, "cores": cores, "kind": "port", "seconds": r["seconds"],
+                            "sample": f"the whole {M}x{N}x{K} {dtype} GEMM, {kind}"}
+            log(f"[bench] cpu baseline {key}: {r['seconds'] * 1e3:.1f} ms -> {r['rate'] * 1e3:.1f} G{unit[1:]}")
+        axpy_cpu = {}
+        for dt in ("f32", "f64"):
+            for lg in (20, 24, args.axpy_log2n):
+                r = cpu_axpy_leg(dt, lg, cores, 20 if lg <= 24 else 3)
+                axpy_cpu[f"2_axpy_{dt}_2p{lg}"] = {"value": r["gbs"], "unit": "GB/s", "cores": cores, "kind": "port",
+                                                   "sample": f"the whole n=2^{lg} {dt} AXPY in place, axpy.cl's element-wise kernel "
+                                                             "spread over the host threads"}
+                log(f"[bench] cpu baseline axpy {dt} 2^{lg}: {r['seconds'] * 1e3:.2f} ms -> {r['gbs']:.1f} GB/s")
+        if configs:
+            for k, v in list(cpu_all.items()) + list(axpy_cpu.items()):
+                if k in configs:
+                    configs[k]["cpu_baseline"] = v
+
+    floor = {"gemm_f32_8192_NN_TFLOPs": {"floor": FLOOR_GEMM_TFLOPS, "value": g["tflops_kernel"]},
+             "axpy_f32_2p28_GBs": {"floor": FLOOR_AXPY_GBS, "value": ax_gbs}}
+    floor_ok = all(v["value"] >= v["floor"] for v in floor.values()) or args.n != 8192 or args.axpy_log2n != 28
+    floor["ok"] = bool(floor_ok)
 
     flops = 2.0 * args.n ** 3
     out = {
@@ -228,22 +310,30 @@ def main():
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "f32", "data": "synthetic",
         "config": {"workload": f"f32 GEMM C=1.5*A*B+0.5*C, M=N=K={args.n}, no transposes, uniform[-1,1) seeded "
-                               f"(BASELINE config 3 headline shape); plus AXPY y=0.75*x+y n=2^{args.axpy_log2n}",
+                               f"(benchmark configuration 3, headline shape); plus AXPY y=0.75*x+y n=2^{args.axpy_log2n}",
                    "kernel": g["variant"]},
         "roofline": {"bound": "mfma", "achieved": g["tflops_kernel"], "peak": F32_MATRIX_PEAK_TFLOPS,
                      "unit": "TFLOP/s", "frac": g["tflops_kernel"] / F32_MATRIX_PEAK_TFLOPS,
-                     "traffic": read_traffic("gemm_f32_8192"), "flops_per_launch": flops,
-                     "kernel_ms": g["kernel_ms"]},
-        "axpy": {"value": ax["gbs"], "unit": "GB/s", "dtype": "f32", "n": ax["n"], "us_per_call": ax["us"],
-                 "roofline": {"bound": "hbm", "achieved": ax["gbs"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                              "frac": ax["gbs"] / HBM_PEAK_GBS, "traffic": read_traffic("axpy_f32_2p28"),
-                              "bytes_per_launch": ax["bytes"]},
-                 "f64": {"value": ax64["gbs"], "us_per_call": ax64["us"], "frac": ax64["gbs"] / HBM_PEAK_GBS}},
+                     "traffic": read_traffic("gemm_f32_8192"), "traffic_source": "recorded from profiles/traffic.json, not measured in this run",
+                     "flops_per_launch": flops, "kernel_ms": g["kernel_ms"]},
+        "axpy": {"value": ax_gbs, "unit": "GB/s", "dtype": "f32", "n": 1 << args.axpy_log2n, "us_per_call": ax_us,
+                 "roofline": {"bound": "hbm", "achieved": ax_gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                              "frac": ax_gbs / HBM_PEAK_GBS, "traffic": read_traffic("axpy_f32_2p28"),
+                              "traffic_source": "recorded from profiles/traffic.json, not measured in this run",
+                              "bytes_per_launch": 3.0 * 4 * (1 << args.axpy_log2n)},
+                 "f64": {"value": ax64["value"], "us_per_call": ax64["ms"] * 1e3, "frac": ax64["value"] / HBM_PEAK_GBS},
+                 "placement_GBs": place,
+                 "cpu_baseline": (axpy_cpu or {}).get(f"2_axpy_f32_2p{args.axpy_log2n}")},
         "mlp_step": mlp,
-        "configs": other,
+        "configs": configs,
         "cpu_baseline": cpu,
+        "cpu_baselines": cpu_all,
+        "perf_floor": floor,
     }
     print(json.dumps(out), flush=True)
+    if not floor_ok and not args.no_floor:
+        log(f"[bench] below the performance floor: {floor}")
+        sys.exit(3)
 
 
 if __name__ == "__main__":

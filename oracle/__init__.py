@@ -70,6 +70,7 @@ def lib():
         L.wko_default_block_cpu.argtypes = [u64, u64, u64, ctypes.c_size_t]
         L.wko_get_algorithm.argtypes = [ci, u64]
         L.wko_axpy.argtypes = [ci, ctypes.POINTER(u64), vp, u64, u64, vp, u64, u64, vp, ci]
+        L.wko_axpy_threads.argtypes = [ci, ctypes.POINTER(u64), vp, u64, u64, vp, u64, u64, vp, ci, ci]
         L.wko_gemm.argtypes = [ci, ci, ci, u64, u64, u64, vp, vp, u64, vp, u64, vp, vp, u64,
                                u64, ci, ci, ci, ci]
         L.wko_gemm_block.argtypes = [ci, ci, ci, u64, u64, u64, u64, ci]
@@ -142,6 +143,24 @@ def axpy(dtype: str, x: np.ndarray, alpha, y: np.ndarray, contract: bool = False
     if rc:
         raise RuntimeError(f"wko_axpy failed: {rc}")
     return out
+
+
+def axpy_inplace(dtype: str, x: np.ndarray, alpha, y: np.ndarray, contract: bool = False, threads: int = 0) -> None:
+    """y = alpha*x + y in place on contiguous arrays, the elements spread over `threads` host threads
+    (0: all).  What a timed CPU baseline calls: no copy of y, one pass."""
+    _check(x, dtype); _check(y, dtype)
+    if x.shape != y.shape or not (x.flags.c_contiguous and y.flags.c_contiguous):
+        raise ValueError("UnqualTensorsShape")
+    shape = x.shape[:-1] if is_complex(dtype) else x.shape
+    cols = shape[-1]
+    rows = shape[-2] if len(shape) >= 2 else 1
+    depth = int(np.prod(shape[:-2], dtype=np.uint64)) if len(shape) >= 3 else 1
+    s3 = (ctypes.c_uint64 * 3)(depth, rows, cols)
+    _keep, ap = _scalar_buf(dtype, alpha)
+    rc = lib().wko_axpy_threads(dtype_id(dtype), s3, x.ctypes.data, cols, rows * cols,
+                                y.ctypes.data, cols, rows * cols, ap, int(contract), threads)
+    if rc:
+        raise RuntimeError(f"wko_axpy_threads failed: {rc}")
 
 
 def _mat_dims(a: np.ndarray, dtype: str):

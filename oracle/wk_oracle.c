@@ -303,6 +303,17 @@ int wko_axpy(int dtype, const uint64_t shape3[3],
     return 0;
 }
 
+int wko_axpy_threads(int dtype, const uint64_t shape3[3],
+                     const void *x, uint64_t xrp, uint64_t xsp,
+                     void *y, uint64_t yrp, uint64_t ysp, const void *alpha, int contract, int threads) {
+    if (threads <= 0) threads = omp_get_max_threads();
+#define CALL(tag) CAT(axpy_mt, tag)(shape3, (const CAT(elem, tag) *)x, xrp, xsp, (CAT(elem, tag) *)y, yrp, ysp, \
+                                    (const CAT(elem, tag) *)alpha, contract, threads)
+    DISPATCH(dtype, CALL)
+#undef CALL
+    return 0;
+}
+
 /* ---- pack ------------------------------------------------------------------------ */
 
 int wko_pack(int dtype, const void *src, uint64_t src_rows, uint64_t src_cols, uint64_t src_pitch,

@@ -69,6 +69,12 @@ int wko_axpy(int dtype, const uint64_t shape3[3],
              const void *x, uint64_t x_row_pitch, uint64_t x_slice_pitch,
              void *y, uint64_t y_row_pitch, uint64_t y_slice_pitch,
              const void *alpha, int contract);
+/* The same with the elements spread over `threads` host threads (<= 0: all), the way an OpenCL CPU
+ * device spreads its work-items over the cores; every element is computed as by wko_axpy. */
+int wko_axpy_threads(int dtype, const uint64_t shape3[3],
+                     const void *x, uint64_t x_row_pitch, uint64_t x_slice_pitch,
+                     void *y, uint64_t y_row_pitch, uint64_t y_slice_pitch,
+                     const void *alpha, int contract, int threads);
 
 /* C = alpha*op(A)*op(B) + beta*C exactly as the reference's CPU device computes it.
  *  - A, B, C are dense row-major host arrays with leading dimensions lda/ldb/ldc

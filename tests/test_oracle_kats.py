@@ -195,3 +195,21 @@ def test_axpy_float_fused_and_unfused_differ_by_at_most_one_rounding():
 def test_axpy_shape_mismatch_raises():
     with pytest.raises(ValueError):
         oracle.axpy("f32", np.zeros((2, 3), np.float32), 2.0, np.zeros((2, 4), np.float32))
+
+
+@pytest.mark.parametrize("dtype", ["f32", "f64", "i16", "cf32", "cu8"])
+def test_threaded_axpy_is_the_same_element_for_element(dtype):
+    """The in-place, threaded form (what the CPU baseline times) against the pinned one, over a length
+    that is not a multiple of the per-thread chunk and over 3-D shapes."""
+    from helpers import make_operand
+    for shape in [(3 * 65536 + 77,), (5, 9, 1031), (1,)]:
+        for alpha in ([None, (2, 1), (-1, 0)] if oracle.is_complex(dtype) else [None, 3, -1]):
+            if alpha is not None and oracle.real_np_dtype(dtype).kind == "u" and (alpha == -1 or alpha == (-1, 0)):
+                continue
+            x = make_operand(dtype, shape, 51)
+            y = make_operand(dtype, shape, 52)
+            want = oracle.axpy(dtype, x, alpha, y, contract=True)
+            for threads in (1, 3, 0):
+                got = y.copy()
+                oracle.axpy_inplace(dtype, x, alpha, got, contract=True, threads=threads)
+                assert np.array_equal(got, want), f"{dtype} {shape} alpha={alpha} threads={threads}"

@@ -60,6 +60,16 @@ class Session:
         self.wk.memory.readFromBuffer(self.pipeline, t, host)
         return t
 
+    def tensor_on_device(self, dtype, shape, seed):
+        """A tensor filled on the device by random.uniform (floats in [-1, 1), integers in [-100, 100]):
+        the same value ranges as `tensor` of a seeded host array, without the host generation and the upload."""
+        t = self.wk.Tensor.alloc(dtype, self.ctx, self.pipeline, shape)
+        if raw.real_np_dtype(dtype).kind == "f":
+            self.wk.random.uniform(self.pipeline, t, seed, -1.0, 1.0)
+        else:
+            self.wk.random.uniform(self.pipeline, t, seed, -100, 100)
+        return t
+
     def time_ms(self, call, iters, warm_seconds=0.15):
         """ms per call from events on the stream, after keeping the device busy for `warm_seconds`
         (short kernels measured right after an upload see the clocks still ramping)."""
@@ -82,14 +92,20 @@ class Session:
         return ms.value / iters
 
 
-def time_gemm(ses, dtype, M, N, K, op_a, op_b, alpha, beta, iters=10):
-    """blas.gemm on tensors created by Tensor.alloc (so with the library's own row pitches)."""
+def time_gemm(ses, dtype, M, N, K, op_a, op_b, alpha, beta, iters=10, device_fill=False):
+    """blas.gemm on tensors created by Tensor.alloc (so with the library's own row pitches).
+    device_fill: operands drawn on the device instead of generated on the host and uploaded."""
     rd = raw.real_np_dtype(dtype)
     wk = ses.wk
     tail = (2,) if dtype.startswith("c") else ()
-    A = ses.tensor(dtype, _operand(rd, ((K, M) if op_a else (M, K)) + tail, 1))
-    B = ses.tensor(dtype, _operand(rd, ((N, K) if op_b else (K, N)) + tail, 2))
-    C = ses.tensor(dtype, _operand(rd, (M, N) + tail, 3))
+    if device_fill:
+        A = ses.tensor_on_device(dtype, (K, M) if op_a else (M, K), 1)
+        B = ses.tensor_on_device(dtype, (N, K) if op_b else (K, N), 2)
+        C = ses.tensor_on_device(dtype, (M, N), 3)
+    else:
+        A = ses.tensor(dtype, _operand(rd, ((K, M) if op_a else (M, K)) + tail, 1))
+        B = ses.tensor(dtype, _operand(rd, ((N, K) if op_b else (K, N)) + tail, 2))
+        C = ses.tensor(dtype, _operand(rd, (M, N) + tail, 3))
     # as benchmark/gemm.zig:186-196 does: one GemmPackedTensors for the run, passed to every call
     packed = wk.GemmPackedTensors.init(ses.pipeline, C, K, True)
     ses.pipeline.waitAndCleanup()
@@ -103,12 +119,15 @@ def time_gemm(ses, dtype, M, N, K, op_a, op_b, alpha, beta, iters=10):
     return ms, variant
 
 
-def time_axpy(ses, dtype, n, iters=50):
+def time_axpy(ses, dtype, n, iters=50, device_fill=False):
     """n: element count of a 1-D tensor, or a shape tuple (2-D / 3-D tensors have pitched rows)."""
     rd = raw.real_np_dtype(dtype)
     wk = ses.wk
     shape = n if isinstance(n, tuple) else (n,)
-    x, y = ses.tensor(dtype, _operand(rd, shape, 1)), ses.tensor(dtype, _operand(rd, shape, 2))
+    if device_fill:
+        x, y = ses.tensor_on_device(dtype, shape, 1), ses.tensor_on_device(dtype, shape, 2)
+    else:
+        x, y = ses.tensor(dtype, _operand(rd, shape, 1)), ses.tensor(dtype, _operand(rd, shape, 2))
     ses.pipeline.waitAndCleanup()
     alpha = 0.75 if rd.kind == "f" else 3
     ms = ses.time_ms(lambda: wk.blas.axpy(ses.pipeline, x, alpha, y), iters)
@@ -144,31 +163,60 @@ def cmd_axpy(ses, args):
         print(f"{args.dtype:5s} {'x'.join(map(str, shape)):>10s} {ms * 1e3:9.2f} {nbytes / ms / 1e6:8.0f}", flush=True)
 
 
-def cmd_configs(ses, args):
-    rows = []
-    ms, v = time_gemm(ses, "f32", 512, 512, 512, 0, 0, 1.0, 0.0)
-    rows.append(("1 f32 512^3 NN a=1 b=0", ms, 2 * 512 ** 3 / ms / 1e9, "TFLOP/s", v))
-    for dt in ("f32", "f64"):
-        for lg in (20, 24, 28):
-            ms = time_axpy(ses, dt, 1 << lg)
-            rows.append((f"2 axpy {dt} n=2^{lg}", ms, 3 * (1 << lg) * raw.elem_size(dt) / ms / 1e6, "GB/s", "axpy_stream"))
+# Published MI355X peaks the rates are held against.  32-bit integer products run as ten int8 digit
+# products on the matrix cores, so their rate in int8 operations is ten times the 32-bit one.
+PEAK = {"f32": (157.3, "TFLOP/s", "mfma", 1.0), "f64": (78.6, "TFLOP/s", "mfma", 1.0), "i32": (5000.0, "TOP/s", "mfma", 10.0)}
+HBM_PEAK_GBS = 8000.0
+
+
+def baseline_gemm_cases():
+    """(key, dtype, M, N, K, op_a, op_b, alpha, beta) for every GEMM of the benchmark configurations, in the
+    sweep order of benchmark/gemm.zig:240-283 (size outermost, the four op pairs inside)."""
+    cases = [("1_f32_gemm_512_NN", "f32", 512, 512, 512, 0, 0, 1.0, 0.0)]
     for n in (1024, 2048, 4096, 8192):
         for op_a, op_b, name in OPS:
-            ms, v = time_gemm(ses, "f32", n, n, n, op_a, op_b, 1.5, 0.5)
-            rows.append((f"3 f32 {n}^3 {name}", ms, 2.0 * n ** 3 / ms / 1e9, "TFLOP/s", v))
+            cases.append((f"3_f32_gemm_{n}_{name}", "f32", n, n, n, op_a, op_b, 1.5, 0.5))
     for (M, N, K) in ((1000, 1000, 1000), (4097, 4095, 4093)):
         for op_a, op_b, name in OPS:
-            ms, v = time_gemm(ses, "f32", M, N, K, op_a, op_b, 1.5, 0.5)
-            rows.append((f"3 f32 {M}x{N}x{K} {name}", ms, 2.0 * M * N * K / ms / 1e9, "TFLOP/s", v))
-    ms, v = time_gemm(ses, "f64", 4096, 4096, 4096, 0, 0, 1.0, 1.0)
-    rows.append(("4 f64 4096^3 NN", ms, 2.0 * 4096 ** 3 / ms / 1e9, "TFLOP/s", v))
-    ms, v = time_gemm(ses, "f64", 8192, 256, 8192, 0, 0, 1.0, 1.0)
-    rows.append(("4 f64 8192x256x8192 NN", ms, 2.0 * 8192 * 256 * 8192 / ms / 1e9, "TFLOP/s", v))
-    ms, v = time_gemm(ses, "i32", 2048, 2048, 2048, 0, 0, 3, -2)
-    rows.append(("4 i32 2048^3 NN", ms, 2.0 * 2048 ** 3 / ms / 1e9, "TOP/s", v))
-    print(f"{'config':34s} {'ms':>9s} {'rate':>9s} unit     kernel")
-    for name, ms, rate, unit, v in rows:
-        print(f"{name:34s} {ms:9.4f} {rate:9.2f} {unit:8s} {v}")
+            cases.append((f"3_f32_gemm_{M}x{N}x{K}_{name}", "f32", M, N, K, op_a, op_b, 1.5, 0.5))
+    cases.append(("4_f64_gemm_4096_NN", "f64", 4096, 4096, 4096, 0, 0, 1.0, 1.0))
+    cases.append(("4_f64_gemm_8192x256x8192_NN", "f64", 8192, 256, 8192, 0, 0, 1.0, 1.0))
+    cases.append(("4_i32_gemm_2048_NN", "i32", 2048, 2048, 2048, 0, 0, 3, -2))
+    return cases
+
+
+def run_baseline_configs(ses, log=None, device_fill=True):
+    """Every GEMM and AXPY benchmark configuration, each with its own roofline figures.  Returns a dict
+    key -> {ms, value, unit, kernel, roofline}."""
+    out = {}
+    for key, dtype, M, N, K, op_a, op_b, alpha, beta in baseline_gemm_cases():
+        ms, variant = time_gemm(ses, dtype, M, N, K, op_a, op_b, alpha, beta, device_fill=device_fill)
+        peak, unit, bound, scale = PEAK[dtype]
+        rate = 2.0 * M * N * K / ms / 1e9
+        out[key] = {"ms": ms, "value": rate, "unit": unit, "kernel": variant,
+                    "roofline": {"bound": bound, "achieved": rate * scale, "peak": peak, "unit": unit,
+                                 "frac": rate * scale / peak}}
+        if log:
+            log(f"{key}: {ms:.4f} ms -> {rate:.1f} {unit} = {100 * rate * scale / peak:.1f} % of peak [{variant}]")
+    for dt in ("f32", "f64"):
+        for lg in (20, 24, 28):
+            ms = time_axpy(ses, dt, 1 << lg, device_fill=device_fill)
+            nbytes = 3.0 * (1 << lg) * raw.elem_size(dt)
+            rate = nbytes / ms / 1e6
+            key = f"2_axpy_{dt}_2p{lg}"
+            out[key] = {"ms": ms, "value": rate, "unit": "GB/s", "kernel": "axpy_stream", "bytes_per_launch": nbytes,
+                        "roofline": {"bound": "hbm", "achieved": rate, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                                     "frac": rate / HBM_PEAK_GBS}}
+            if log:
+                log(f"{key}: {ms * 1e3:.1f} us -> {rate:.0f} GB/s = {100 * rate / HBM_PEAK_GBS:.1f} % of HBM peak")
+    return out
+
+
+def cmd_configs(ses, args):
+    rows = run_baseline_configs(ses, device_fill=False)
+    print(f"{'config':38s} {'ms':>9s} {'rate':>9s} unit     % peak  kernel")
+    for name, r in rows.items():
+        print(f"{name:38s} {r['ms']:9.4f} {r['value']:9.2f} {r['unit']:8s} {100 * r['roofline']['frac']:6.1f}  {r['kernel']}")
 
 
 def cmd_tensor(ses, args):
