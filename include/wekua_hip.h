@@ -197,6 +197,16 @@ const char *wk_gemm_variant_with_workspace(int dtype, int op_a, int op_b, uint64
                                            uint64_t lda, uint64_t ldb, uint64_t ldc, const void *A, const void *B,
                                            const void *C, size_t workspace_bytes);
 
+/* Host arithmetic only, for tests and benchmarks: how a wk_gemm call on a stream lays out a product
+ * whose k is split over work-groups (few tiles of C, long k: every tile goes to `shares` work-groups
+ * that each sum `klen` values of k -- the last one what is left -- into partial tiles of
+ * `scratch_bytes` bytes in the stream's own scratch memory; the last work-group to arrive at a tile
+ * adds them in the order of the shares, so results are the same bits on every run).  variant NULL:
+ * the automatic choice (shares = 1 when it does not split); a split variant's name ("mfma_f32_64x64z",
+ * "mfma_f64_64x64z"): the plan that variant runs when forced.  No counterpart in the reference. */
+int wk_gemm_split_plan(int dtype, int op_a, int op_b, uint64_t M, uint64_t N, uint64_t K, const char *variant,
+                       uint32_t *shares, uint32_t *klen, uint64_t *tiles, size_t *scratch_bytes);
+
 /* Test and benchmark knob only, not for product code: force a gemm variant by name ("auto" restores
  * selection).  Process-wide, read by every wk_gemm call on every stream; changing it while a
  * PackedTensors keeps B invalidates what that handle remembers.  A forced variant whose kernel
@@ -242,6 +252,13 @@ int  wk_bias_step(wk_stream *s, int dtype, uint64_t rows, uint64_t cols, const v
  * that overlap on one device -- on different streams or from different threads -- race. */
 #define WK_BIAS_STEP_STATIC_SCRATCH_BYTES (1u << 20)
 int  wk_bias_step_static(wk_stream *s, int dtype, uint64_t rows, uint64_t cols, const void *sens, uint64_t pitch, void *bias_grad);
+/* Linear.backward's element-wise half in one pass over the layer's output (src/nn/layer/linear.zig:606-640:
+ * act.getDerivative, math.dot, getBiasSensitivity): dev = act'(out), sens *= dev, bias_grad[c] = sum_r sens[r][c]
+ * of the new sens (skipped when bias_grad is NULL).  The same values, bit for bit, as wk_activation_dev,
+ * wk_hadamard and wk_bias_step one after the other, with half the memory traffic.  kind WK_ACT_NONE: dev is
+ * read as it is (the reference multiplies by its cached derivative tensor whatever it holds) and out may be NULL. */
+int  wk_sensitivity_step(wk_stream *s, int dtype, int kind, uint64_t rows, uint64_t cols, const void *out, uint64_t out_pitch,
+                         void *sens, uint64_t sens_pitch, void *dev, uint64_t dev_pitch, void *bias_grad);
 /* loss.mse kernel: err = expected - output; error = err^2; dev = -2*err when dev != NULL
  * (src/nn/loss/kernels/mse.cl:3-35, src/nn/loss/mse.zig:63-132) */
 int  wk_mse(wk_stream *s, int dtype, const uint64_t shape3[3], const void *output, uint64_t out_row_pitch, uint64_t out_slice_pitch,
@@ -259,6 +276,18 @@ int  wk_sum(wk_stream *s, int dtype, const uint64_t shape3[3], const void *x, ui
 int  wk_adam_step(wk_stream *s, int dtype, const uint64_t shape3[3], void *w, uint64_t w_row_pitch, uint64_t w_slice_pitch,
                   const void *g, uint64_t g_row_pitch, uint64_t g_slice_pitch, void *m, void *v, uint64_t mv_row_pitch,
                   uint64_t mv_slice_pitch, double lr, double beta1, double beta2, double eps, uint64_t step);
+/* The same update of `count` parameter tensors (host array, read before the call returns) in one launch
+ * per eight tensors instead of one per tensor; every element gets exactly the arithmetic of wk_adam_step.
+ * Tensors that do not allow 16-byte accesses make the call fall back to one wk_adam_step each. */
+typedef struct wk_adam_tensor {
+    void       *w;
+    const void *g;
+    void       *m, *v;
+    uint64_t    shape3[3];
+    uint64_t    w_row_pitch, w_slice_pitch, g_row_pitch, g_slice_pitch, mv_row_pitch, mv_slice_pitch;
+} wk_adam_tensor;
+int  wk_adam_step_multi(wk_stream *s, int dtype, uint32_t count, const wk_adam_tensor *host_tensors, double lr, double beta1,
+                        double beta2, double eps, uint64_t step);
 
 /* ---- tensor support operations (src/tensor) --------------------------------------------------- */
 #define WK_MAX_DIMS 8

@@ -77,7 +77,7 @@ def test_float_small_shapes(dev, dtype, op_a, op_b, alpha, beta):
 
 
 @pytest.mark.parametrize("variant", ["tile64", "mfma_f32_64x64", "mfma_f32_64x64s2", "mfma_f32_64x64s4", "mfma_f32_32x32s4",
-                                     "mfma_f32_128x128", "mfma_f32_128x128s2", "mfma_f32_256x128"])
+                                     "mfma_f32_64x64z", "mfma_f32_128x128", "mfma_f32_128x128s2", "mfma_f32_256x128"])
 @pytest.mark.parametrize("op_a,op_b", OPS)
 def test_f32_every_variant(dev, variant, op_a, op_b):
     import ctypes
@@ -89,8 +89,8 @@ def test_f32_every_variant(dev, variant, op_a, op_b):
         dev.lib.wk_gemm_force_variant(b"auto")
 
 
-@pytest.mark.parametrize("variant", ["tile64", "mfma_f64_64x64", "mfma_f64_64x64s2", "mfma_f64_32x32s4", "mfma_f64_128x64",
-                                     "mfma_f64_128x128"])
+@pytest.mark.parametrize("variant", ["tile64", "mfma_f64_64x64", "mfma_f64_64x64s2", "mfma_f64_32x32s4", "mfma_f64_64x64z",
+                                     "mfma_f64_128x64", "mfma_f64_128x128"])
 @pytest.mark.parametrize("op_a,op_b", OPS)
 def test_f64_every_variant(dev, variant, op_a, op_b):
     assert dev.lib.wk_gemm_force_variant(variant.encode()) == 0
@@ -260,7 +260,8 @@ def test_invalid_arguments(dev):
                                            ("f32", "mfma_f32_32x32s4"), ("f32", "mfma_f32_128x128"), ("f32", "mfma_f32_128x128s2"),
                                            ("f32", "mfma_f32_256x128"),
                                            ("f64", "mfma_f64_64x64"), ("f64", "mfma_f64_64x64s2"), ("f64", "mfma_f64_32x32s4"),
-                                           ("f64", "mfma_f64_128x64"), ("f64", "mfma_f64_128x128")])
+                                           ("f64", "mfma_f64_128x64"), ("f64", "mfma_f64_128x128"),
+                                           ("f32", "mfma_f32_64x64z"), ("f64", "mfma_f64_64x64z")])
 def test_every_k_around_the_slab_boundaries(dev, dtype, variant):
     """Every K from 1 to 100 on a ragged tile and on a tile-aligned shape: the bounds-checked kernels
     choose per-flavour loops from the number of complete slabs (k-slab 16 or 32, one or two slabs of
@@ -305,6 +306,57 @@ def test_one_round_launches_take_the_k_split_tiles(dev):
             check(dev, dtype, 1024, 960, 300, op_a, op_b, 1.5, 0.5, seed=93)
             check(dev, dtype, 1000, 1000, 257, op_a, op_b, None, None, seed=94)
             check(dev, dtype, 500, 333, 129, op_a, op_b, 2.0, None, seed=95)
+
+
+@pytest.mark.parametrize("dtype", ["f32", "f64"])
+def test_k_split_over_work_groups(dev, dtype):
+    """Few tiles of C and a long k: every tile goes to several work-groups, whose partial tiles meet in
+    the stream's scratch and are added in a fixed order.  The automatic choice is checked by name and by
+    its plan; results against the oracle on all four layouts, aligned and ragged, and twice in a row
+    for the same bits (the order of the additions does not depend on which work-group arrives last;
+    the arrival counters are back at zero after every launch)."""
+    import ctypes
+    from wekua_amd import raw
+    lib = dev.lib
+    did = raw.dtype_id(dtype)
+    z = f"mfma_{dtype}_64x64z".encode()
+    assert lib.wk_gemm_variant(did, 0, 0, 512, 512, 8192, 8192, 512, 512, None, None, None) == z
+    assert lib.wk_gemm_variant(did, 0, 0, 512, 512, 512, 512, 512, 512, None, None, None) != z      # k too short to split
+    assert lib.wk_gemm_variant(did, 0, 0, 2048, 2048, 8192, 8192, 2048, 2048, None, None, None) != z  # enough tiles
+    shares, klen, tiles, nbytes = ctypes.c_uint32(), ctypes.c_uint32(), ctypes.c_uint64(), ctypes.c_size_t()
+    assert lib.wk_gemm_split_plan(did, 0, 0, 512, 512, 8192, None, shares, klen, tiles, nbytes) == 0
+    # 64 tiles on 256 compute units: shares until four (f32) / two (f64) work-groups sit on every unit
+    assert (shares.value, klen.value, tiles.value) == ((16, 512, 64) if dtype == "f32" else (8, 1024, 64))
+    for op_a, op_b in OPS:
+        check(dev, dtype, 512, 512, 4096, op_a, op_b, 1.5, 0.5, seed=71)           # automatic, aligned
+        check(dev, dtype, 300, 200, 4500, op_a, op_b, None, None, seed=72)         # automatic, ragged (k tail in the last share)
+        check(dev, dtype, 128, 64, 16500, op_a, op_b, 2.0, None, seed=76)          # two tiles, 64 shares
+    assert lib.wk_gemm_force_variant(z) == 0
+    try:
+        for op_a, op_b in OPS:
+            check(dev, dtype, 192, 128, 160, op_a, op_b, 2.0, None, seed=73)       # shares of one or two slabs
+            check(dev, dtype, 70, 45, 97, op_a, op_b, 1.5, 0.5, seed=74)           # the last share holds one element of k
+            check(dev, dtype, 130, 257, 333, op_a, op_b, None, -0.25, seed=75,
+                  lda=(130 if op_a else 333) + 1, ldb=(333 if op_b else 257) + 3, ldc=257 + 5)
+        # the same call several times: bit-identical, whoever arrives last
+        from helpers import make_operand
+        rd = np.float32 if dtype == "f32" else np.float64
+        M, N, K = 256, 192, 1024
+        a = make_operand(dtype, (M, K), 81)
+        b = make_operand(dtype, (K, N), 82)
+        dA, dB = dev.upload(a), dev.upload(b)
+        outs = []
+        for _ in range(4):
+            dC = dev.upload(np.zeros((M, N), dtype=rd))
+            dev.gemm(dtype, 0, 0, M, N, K, None, dA, K, dB, N, None, dC, N)
+            dev.sync()
+            outs.append(dC.download(rd, (M, N)))
+            dC.free()
+        for o in outs[1:]:
+            assert np.array_equal(o, outs[0])
+        dA.free(); dB.free()
+    finally:
+        lib.wk_gemm_force_variant(b"auto")
 
 
 @pytest.mark.parametrize("variant", ["mfma_i32_64x128", "mfma_i32_128x128", "mfma_i32_packed"])

@@ -419,3 +419,114 @@ def test_config5_mlp_training_step_full_size(env):
     seq.deinit(pipeline)
     x.release(pipeline)
     y.release(pipeline)
+
+
+# ---- the fused passes against the separate ones (raw C ABI) ---------------------------------------
+
+@pytest.mark.parametrize("dtype", ["f32", "f64"])
+@pytest.mark.parametrize("rows,cols,pad", [(1, 1, 0), (5, 3, 0), (19, 11, 1), (64, 256, 0), (33, 65, 3), (300, 1000, 8),
+                                           (2048, 1024, 128), (1000, 4100, 4)])
+def test_sensitivity_step_equals_the_three_passes(dev, dtype, rows, cols, pad):
+    """wk_sensitivity_step = wk_activation_dev + wk_hadamard + wk_bias_step, bit for bit (same
+    arithmetic per element, same order of additions per column), for sigmoid, tanh and no activation,
+    aligned and unaligned pitches, with and without a bias gradient; gaps between rows keep their
+    poison.  The separate passes are in turn held to the restatement by the tests above."""
+    import ctypes
+    from wekua_amd import raw
+    dt = NP[dtype]
+    did = raw.dtype_id(dtype)
+    lib = dev.lib
+    pitch = cols + pad
+    s3 = (ctypes.c_uint64 * 3)(1, rows, cols)
+
+    def padded(host, poison):
+        full = np.full((rows, pitch), poison, dtype=dt)
+        full[:, :cols] = host
+        return full
+
+    out_h = synth.uniform(61, (rows, cols), dt, 0.05, 0.95)     # a sigmoid / tanh output
+    sens_h = synth.uniform(62, (rows, cols), dt, -2.0, 2.0)
+    dev_h = synth.uniform(63, (rows, cols), dt, -1.0, 1.0)      # what a layer without activation multiplies by
+    for kind in (0, 1, -1):
+        for with_bias in (True, False):
+            # separate passes
+            d_out = dev.upload(padded(out_h, 7))
+            d_sens = dev.upload(padded(sens_h, 8))
+            d_dev = dev.upload(padded(dev_h, 9))
+            d_bg = dev.upload(np.full(cols + 4, -3, dtype=dt))
+            if kind >= 0:
+                assert lib.wk_activation_dev(dev.stream, did, kind, s3, d_out.ptr, pitch, 0, d_dev.ptr, pitch, 0) == 0
+            assert lib.wk_hadamard(dev.stream, did, s3, d_sens.ptr, pitch, 0, d_dev.ptr, pitch, 0) == 0
+            if with_bias:
+                assert lib.wk_bias_step(dev.stream, did, rows, cols, d_sens.ptr, pitch, d_bg.ptr) == 0
+            dev.sync()
+            want = [d.download(dt, (rows, pitch)) for d in (d_sens, d_dev, d_out)] + [d_bg.download(dt, (cols + 4,))]
+            for d in (d_out, d_sens, d_dev, d_bg):
+                d.free()
+            # one pass
+            f_out = dev.upload(padded(out_h, 7))
+            f_sens = dev.upload(padded(sens_h, 8))
+            f_dev = dev.upload(padded(dev_h, 9))
+            f_bg = dev.upload(np.full(cols + 4, -3, dtype=dt))
+            assert lib.wk_sensitivity_step(dev.stream, did, kind, rows, cols, f_out.ptr if kind >= 0 else None, pitch, f_sens.ptr, pitch,
+                                           f_dev.ptr, pitch, f_bg.ptr if with_bias else None) == 0
+            dev.sync()
+            got = [d.download(dt, (rows, pitch)) for d in (f_sens, f_dev, f_out)] + [f_bg.download(dt, (cols + 4,))]
+            for d in (f_out, f_sens, f_dev, f_bg):
+                d.free()
+            for name, g, w in zip(("sensitivity", "derivative", "output", "bias gradient"), got, want):
+                assert np.array_equal(g, w), f"{name} kind={kind} bias={with_bias} {rows}x{cols}+{pad}"
+            assert np.array_equal(got[2][:, :cols], out_h)     # the layer's output is read only
+    buf = dev.malloc(4096)
+    p = buf.ptr
+    assert lib.wk_sensitivity_step(dev.stream, did, 2, 4, 4, p, 4, p, 4, p, 4, None) == 1       # unknown activation
+    assert lib.wk_sensitivity_step(dev.stream, did, 0, 4, 4, None, 4, p, 4, p, 4, None) == 1    # sigmoid needs the output
+    assert lib.wk_sensitivity_step(dev.stream, did, 0, 4, 8, p, 8, p, 4, p, 8, None) == 1       # pitch < cols
+    assert lib.wk_sensitivity_step(dev.stream, raw.dtype_id("i32"), 0, 4, 4, p, 4, p, 4, p, 4, None) == 9
+    buf.free()
+
+
+@pytest.mark.parametrize("dtype", ["f32", "f64"])
+def test_adam_step_multi_equals_one_launch_per_tensor(dev, dtype):
+    """wk_adam_step_multi over a list of parameter tensors (more than one launch's worth, ragged
+    widths, pitched rows) against wk_adam_step on copies of the same tensors: the same bits in the
+    weights and both moments after three steps; an unaligned tensor in the list takes the per-tensor
+    route and still agrees."""
+    import ctypes
+    from wekua_amd import raw
+    from wekua_amd._capi import WkAdamTensor
+    dt = NP[dtype]
+    did = raw.dtype_id(dtype)
+    lib = dev.lib
+    for shapes in ([(1, 1, 5, 5), (1, 64, 256, 256), (1, 33, 65, 68), (2, 7, 12, 12), (1, 1, 4096, 4096), (1, 300, 1000, 1000),
+                    (1, 1, 1, 4), (1, 128, 512, 520), (1, 17, 130, 132), (1, 1, 70, 72)],
+                   [(1, 19, 11, 13), (1, 64, 64, 64)]):                       # (depth, rows, cols, pitch); 13 is not 16-byte aligned
+        sets = []
+        for which in range(2):
+            bufs = []
+            for i, (d, r, c, p) in enumerate(shapes):
+                arrs = [synth.uniform(100 + 4 * i + j, (d, r, p), dt, 0.0 if j == 3 else -1.0, 1.0) for j in range(4)]
+                bufs.append([dev.upload(a) for a in arrs])                        # w, g, m, v (v >= 0)
+            sets.append(bufs)
+        lr, b1, b2, eps = 1e-3, 0.9, 0.999, float(np.finfo(dt).eps)
+        for step in (1, 2, 3):
+            for (d, r, c, p), (w, g, m, v) in zip(shapes, sets[0]):
+                s3 = (ctypes.c_uint64 * 3)(d, r, c)
+                assert lib.wk_adam_step(dev.stream, did, s3, w.ptr, p, r * p, g.ptr, p, r * p, m.ptr, v.ptr, p, r * p, lr, b1, b2, eps, step) == 0
+            lst = (WkAdamTensor * len(shapes))()
+            for t, (d, r, c, p), (w, g, m, v) in zip(lst, shapes, sets[1]):
+                t.w, t.g, t.m, t.v = w.ptr.value, g.ptr.value, m.ptr.value, v.ptr.value
+                t.shape3[0], t.shape3[1], t.shape3[2] = d, r, c
+                t.w_row_pitch = t.g_row_pitch = t.mv_row_pitch = p
+                t.w_slice_pitch = t.g_slice_pitch = t.mv_slice_pitch = r * p
+            assert lib.wk_adam_step_multi(dev.stream, did, len(shapes), lst, lr, b1, b2, eps, step) == 0
+        dev.sync()
+        for (d, r, c, p), one, many in zip(shapes, sets[0], sets[1]):
+            for name, a, b in zip("wgmv", one, many):
+                assert np.array_equal(a.download(dt, (d, r, p)), b.download(dt, (d, r, p))), f"{name} of {(d, r, c, p)}"
+        for bufs in sets:
+            for quad in bufs:
+                for b in quad:
+                    b.free()
+    assert lib.wk_adam_step_multi(dev.stream, did, 0, None, 1e-3, 0.9, 0.999, 1e-8, 1) == 0
+    assert lib.wk_adam_step_multi(dev.stream, did, 1, None, 1e-3, 0.9, 0.999, 1e-8, 1) == 1

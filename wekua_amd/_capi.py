@@ -33,6 +33,14 @@ class WkProps(ctypes.Structure):
     ]
 
 
+class WkAdamTensor(ctypes.Structure):
+    """wk_adam_tensor of include/wekua_hip.h"""
+    _fields_ = [("w", ctypes.c_void_p), ("g", ctypes.c_void_p), ("m", ctypes.c_void_p), ("v", ctypes.c_void_p),
+                ("shape3", ctypes.c_uint64 * 3), ("w_row_pitch", ctypes.c_uint64), ("w_slice_pitch", ctypes.c_uint64),
+                ("g_row_pitch", ctypes.c_uint64), ("g_slice_pitch", ctypes.c_uint64), ("mv_row_pitch", ctypes.c_uint64),
+                ("mv_slice_pitch", ctypes.c_uint64)]
+
+
 # name -> (restype, argtypes); one entry per declaration in include/wekua_hip.h
 SIGNATURES = {
     "wk_strerror": (ctypes.c_char_p, [ci]),
@@ -67,6 +75,8 @@ SIGNATURES = {
     "wk_gemm_variant": (ctypes.c_char_p, [ci, ci, ci, u64, u64, u64, u64, u64, u64, vp, vp, vp]),
     "wk_gemm_variant_with_workspace": (ctypes.c_char_p, [ci, ci, ci, u64, u64, u64, u64, u64, u64, vp, vp, vp, sz]),
     "wk_gemm_force_variant": (ci, [ctypes.c_char_p]),
+    "wk_gemm_split_plan": (ci, [ci, ci, ci, u64, u64, u64, ctypes.c_char_p, ctypes.POINTER(ctypes.c_uint32),
+                                ctypes.POINTER(ctypes.c_uint32), ctypes.POINTER(u64), ctypes.POINTER(ctypes.c_size_t)]),
     "wk_copy_kernel": (ci, [vp, vp, vp, sz]),
     "wk_hadamard": (ci, [vp, ci, u64p, vp, u64, u64, vp, u64, u64]),
     "wk_activation": (ci, [vp, ci, ci, u64p, vp, u64, u64]),
@@ -75,6 +85,8 @@ SIGNATURES = {
     "wk_gemm_bias_activation": (ci, [vp, ci, ci, ci, u64, u64, u64, vp, u64, vp, u64, vp, u64, vp, ci]),
     "wk_bias_step": (ci, [vp, ci, u64, u64, vp, u64, vp]),
     "wk_bias_step_static": (ci, [vp, ci, u64, u64, vp, u64, vp]),
+    "wk_sensitivity_step": (ci, [vp, ci, ci, u64, u64, vp, u64, vp, u64, vp, u64, vp]),
+    "wk_adam_step_multi": (ci, [vp, ci, ctypes.c_uint32, vp, ctypes.c_double, ctypes.c_double, ctypes.c_double, ctypes.c_double, u64]),
     "wk_mse": (ci, [vp, ci, u64p, vp, u64, u64, vp, u64, u64, vp, u64, u64, vp, u64, u64]),
     "wk_sum_workspace_bytes": (sz, [ci]),
     "wk_sum": (ci, [vp, ci, u64p, vp, u64, u64, vp, vp, ctypes.c_double]),

@@ -2,7 +2,7 @@
 HIP path: a table of GEMM times over square sizes and the four transpose pairs, and of AXPY
 times over 1-D sizes, on GPU 0.
 
-    python -m wekua_amd.benchmark gemm [--dtype f32] [--sizes 1024 2048 ...] [--variant NAME]
+    python -m wekua_amd.benchmark gemm [--dtype f32] [--sizes 1024 2048 ...] [--shapes 8192x256x8192 ...] [--ops NN TN] [--variant NAME]
     python -m wekua_amd.benchmark axpy [--dtype f32]
     python -m wekua_amd.benchmark configs        # every BASELINE GEMM / AXPY configuration, one line each
     python -m wekua_amd.benchmark tensor         # transpose / copy / random.uniform / toComplex streaming rates
@@ -144,10 +144,14 @@ def cmd_gemm(ses, args):
     if cplx:
         alpha, beta = (alpha, 0.5 if is_float else 1), (beta, 0.25 if is_float else -1)
     ops = 8.0 if cplx else 2.0   # a complex multiply-add counted as four real ones
-    for n in args.sizes:
+    shapes = [(n, n, n) for n in args.sizes] if not args.shapes else [tuple(int(v) for v in sh.split("x")) for sh in args.shapes]
+    for M, N, K in shapes:
         for op_a, op_b, name in OPS:
-            ms, variant = time_gemm(ses, args.dtype, n, n, n, op_a, op_b, alpha, beta)
-            print(f"{args.dtype:5s} {n:6d} {name:2s} {ms:9.4f} {ops * n ** 3 / ms / 1e9:9.2f}  {variant}", flush=True)
+            if args.ops and name not in args.ops:
+                continue
+            ms, variant = time_gemm(ses, args.dtype, M, N, K, op_a, op_b, alpha, beta, device_fill=True)
+            label = str(M) if M == N == K else f"{M}x{N}x{K}"
+            print(f"{args.dtype:5s} {label:>6s} {name:2s} {ms:9.4f} {ops * M * N * K / ms / 1e9:9.2f}  {variant}", flush=True)
 
 
 def cmd_axpy(ses, args):
@@ -346,6 +350,8 @@ def main(argv=None):
     g.add_argument("--dtype", default="f32")
     g.add_argument("--sizes", type=int, nargs="+", default=[4 << i for i in range(4, 12)])
     g.add_argument("--variant", default="auto")
+    g.add_argument("--shapes", nargs="+", default=None, help="MxNxK ... instead of the square --sizes")
+    g.add_argument("--ops", nargs="+", default=None, choices=["NN", "NT", "TN", "TT"], help="only these operand layouts")
     a = sub.add_parser("axpy")
     a.add_argument("--dtype", default="f32")
     sub.add_parser("tensor")

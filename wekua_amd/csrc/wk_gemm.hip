@@ -117,6 +117,10 @@ static int gemm_entry(wk_stream *s, int dtype, int op_a, int op_b, uint64_t M, u
     if (rc) return rc;
     p.num_cus = (uint32_t)s->dev->props.multiProcessorCount;
     p.reuse_b = reuse_b;
+    p.scratch = s->scratch;
+    p.scratch_bytes = s->scratch_bytes;
+    p.counters = s->gemm_counters;
+    p.num_counters = WK_GEMM_COUNTERS;
     if (has_packed_path(dtype)) {
         const int forced = g_forced.load(std::memory_order_relaxed);
         const size_t need = gemm_int_packed_workspace_bytes(dtype, M, N, K);
@@ -174,6 +178,10 @@ int wk_gemm_bias_activation(wk_stream *s, int dtype, int op_a, int op_b, uint64_
     rc = build_problem(p, dtype, op_a, op_b, M, N, K, nullptr, A, lda, B, ldb, nullptr, C, ldc);
     if (rc) return rc;
     p.num_cus = (uint32_t)s->dev->props.multiProcessorCount;
+    p.scratch = s->scratch;
+    p.scratch_bytes = s->scratch_bytes;
+    p.counters = s->gemm_counters;
+    p.num_counters = WK_GEMM_COUNTERS;
     const int v = choose(p);
     if (v >= 0 && gemm_mfma_fuses(p, v) && (bias || kind != WK_ACT_NONE)) {
         p.ext = true;
@@ -195,6 +203,13 @@ const char *wk_gemm_variant(int dtype, int op_a, int op_b, uint64_t M, uint64_t 
     if (build_problem(p, dtype, op_a, op_b, M, N, K, nullptr, A ? A : dummy, lda, B ? B : dummy, ldb, nullptr,
                       C ? const_cast<void *>(C) : dummy, ldc))
         return "invalid";
+    // what a stream brings along (scratch for partial tiles, arrival counters), so that the answer is
+    // the kernel a wk_gemm call on a stream would launch
+    alignas(4) static uint32_t dummy_counter;
+    p.scratch = dummy;
+    p.scratch_bytes = WK_STREAM_SCRATCH_BYTES;
+    p.counters = &dummy_counter;
+    p.num_counters = WK_GEMM_COUNTERS;
     const int v = choose(p);
     return v >= 0 ? gemm_mfma_variant_name(v) : k_generic_name;
 }
@@ -221,6 +236,41 @@ const char *wk_gemm_variant_with_workspace(int dtype, int op_a, int op_b, uint64
     p.dtype = dtype; p.M = M; p.N = N; p.K = K;
     if (forced == -3) return fits ? k_packed_names[dtype] : "invalid";
     return fits && forced == -2 && packed_pays(p) ? k_packed_names[dtype] : plain;
+}
+
+int wk_gemm_split_plan(int dtype, int op_a, int op_b, uint64_t M, uint64_t N, uint64_t K, const char *variant, uint32_t *shares,
+                       uint32_t *klen, uint64_t *tiles, size_t *scratch_bytes) {
+    if (!shares || !klen || !tiles || !scratch_bytes) return WK_E_INVALID_VALUE;
+    *shares = 1;
+    *klen = 0;
+    *tiles = 0;
+    *scratch_bytes = 0;
+    GemmProblem p;
+    alignas(16) static unsigned char dummy[16];
+    alignas(4) static uint32_t dummy_counter;
+    const uint64_t lda = op_a ? M : K, ldb = op_b ? K : N;
+    int rc = build_problem(p, dtype, op_a, op_b, M, N, K, nullptr, dummy, lda, dummy, ldb, nullptr, dummy, N);
+    if (rc) return rc;
+    p.scratch = dummy;
+    p.scratch_bytes = WK_STREAM_SCRATCH_BYTES;
+    p.counters = &dummy_counter;
+    p.num_counters = WK_GEMM_COUNTERS;
+    int v = -1;
+    if (variant) {
+        for (int i = 0; gemm_mfma_variant_name(i); ++i)
+            if (!std::strcmp(variant, gemm_mfma_variant_name(i))) v = i;
+        if (v < 0 || gemm_mfma_variant_dtype(v) != dtype) return WK_E_INVALID_VALUE;
+    } else {
+        v = gemm_mfma_pick(p);
+    }
+    GemmSplitPlan plan;
+    if (v >= 0 && gemm_mfma_split_plan(p, v, variant != nullptr, plan)) {
+        *shares = plan.shares;
+        *klen = plan.klen;
+        *tiles = plan.tiles;
+        *scratch_bytes = plan.bytes;
+    }
+    return WK_OK;
 }
 
 int wk_gemm_force_variant(const char *name) {

@@ -59,6 +59,13 @@ template <typename T> struct MArgs {
     // epilogue extension (kernels instantiated with EXT): C = act(acc + bias[col]); bias may be null
     const T *bias;
     int act;
+    // k split over work-groups (kernels instantiated with SPLIT): blockIdx.y takes k values
+    // [blockIdx.y * klen, min(K, (blockIdx.y + 1) * klen)) of the sum, the partial tiles meet in
+    // `partials` ([share][tile][BM * BN]) and the work-group that arrives last at counters[tile] adds
+    // them up.  Unused (klen 0, null pointers) by every other kernel.
+    uint32_t klen;
+    T *partials;
+    uint32_t *counters;
 };
 
 // Work-groups that share a CU start in lock step (the whole first wave of work-groups is
@@ -111,9 +118,11 @@ template <int ROWS, int BK, bool KCONTIG> struct Slab {
 // KS * BK values between them (group kg multiplies the k values kg * BK .. kg * BK + BK - 1 of the
 // slab); their accumulators are added through LDS before the epilogue.  For launches that put a
 // single small work-group on a CU this doubles the wavefronts a SIMD can switch between.
-template <int BM, int BN, int BK, int WAVES_M, int WAVES_N, int OCC, bool A_K, bool B_K, bool EDGE, bool EXT = false, int KS = 1, int LSEL = -1>
+template <int BM, int BN, int BK, int WAVES_M, int WAVES_N, int OCC, bool A_K, bool B_K, bool EDGE, bool EXT = false, int KS = 1, int LSEL = -1,
+          bool SPLIT = false>
 __global__ __launch_bounds__(WAVES_M *WAVES_N * 64 * KS) __attribute__((amdgpu_waves_per_eu(OCC)))
 void gemm_f32_mfma_kernel(MArgs<float> g) {
+    static_assert(!SPLIT || KS == 1, "k is split over work-groups or inside one, not both");
     constexpr int NT = WAVES_M * WAVES_N * 64 * KS;
     constexpr int BKT = BK * KS; // k values per LDS slab
     constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N;
@@ -136,6 +145,13 @@ void gemm_f32_mfma_kernel(MArgs<float> g) {
     uint32_t tile_m, tile_n;
     tile_coords(g.tiles_m, g.tiles_n, tile_m, tile_n, g.xcd_remap);
     const uint32_t m0 = tile_m * BM, n0 = tile_n * BN;
+    if constexpr (SPLIT) { // this work-group's share of k; from here on the kernel sees a shorter product
+        const uint32_t k_begin = blockIdx.y * g.klen;
+        const uint32_t k_end = min(g.K, k_begin + g.klen);
+        g.A += A_K ? (size_t)k_begin : (size_t)k_begin * g.lda;
+        g.B += B_K ? (size_t)k_begin : (size_t)k_begin * g.ldb;
+        g.K = k_end - k_begin;
+    }
     // one solo iteration = FM*FN*BK/2 matrix instructions of 64 clocks = FM*FN*BK/4 sleep units
     startup_stagger(g.num_cus, OCC, FM * FN * BK / 4);
 
@@ -551,6 +567,61 @@ void gemm_f32_mfma_kernel(MArgs<float> g) {
         }
     }
 
+    if constexpr (SPLIT) {
+        // The shares' partial tiles meet in memory in accumulator-register order (register q of thread
+        // t at q * NT + t: coalesced).  The work-group that arrives last at the tile's counter adds
+        // them up, always in the order of the shares and its own read back like the others, so the
+        // result does not depend on which one that is; it leaves the counter at zero for the next
+        // launch.
+        // Work-groups of one tile may sit on different XCDs, behind different L2s.  The partial tiles
+        // are therefore written and read with device-scope accesses (relaxed atomics: they go through
+        // to the memory side and are read from there), a wavefront waits for its stores to be
+        // acknowledged before the barrier in front of the count, and the count itself is a
+        // device-scope atomic.  This orders everything that matters without release / acquire fences,
+        // which on this part write back and invalidate a whole L2 per work-group (measured: with
+        // fences the split launch was no faster than the unsplit one).
+        __shared__ uint32_t s_last;
+        constexpr int Q = FM * FN * 16;
+        constexpr size_t TILE = (size_t)BM * BN;
+        float *mine = g.partials + ((size_t)blockIdx.y * gridDim.x + blockIdx.x) * TILE + tid;
+#pragma unroll
+        for (int i = 0; i < FM; ++i)
+#pragma unroll
+            for (int j = 0; j < FN; ++j)
+#pragma unroll
+                for (int r = 0; r < 16; ++r)
+                    __hip_atomic_store(mine + (size_t)((i * FN + j) * 16 + r) * NT, acc[i][j][r], __ATOMIC_RELAXED,
+                                       __HIP_MEMORY_SCOPE_AGENT);
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        __syncthreads();
+        if (tid == 0) {
+            const uint32_t before = __hip_atomic_fetch_add(&g.counters[blockIdx.x], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            const uint32_t last = before == gridDim.y - 1 ? 1u : 0u;
+            if (last) __hip_atomic_store(&g.counters[blockIdx.x], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            s_last = last;
+        }
+        __syncthreads();
+        if (!s_last) return;
+#pragma unroll
+        for (int i = 0; i < FM; ++i)
+#pragma unroll
+            for (int j = 0; j < FN; ++j)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+        for (uint32_t z = 0; z < gridDim.y; ++z) {
+            const float *part = g.partials + ((size_t)z * gridDim.x + blockIdx.x) * TILE + tid;
+            float v[Q];
+#pragma unroll
+            for (int q = 0; q < Q; ++q) v[q] = __hip_atomic_load(part + (size_t)q * NT, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+#pragma unroll
+            for (int i = 0; i < FM; ++i)
+#pragma unroll
+                for (int j = 0; j < FN; ++j)
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) acc[i][j][r] += v[(i * FN + j) * 16 + r];
+        }
+    }
+
     // ---- epilogue: acc register r of lane l is C[8*(r/4) + 4*(l/32) + r%4][l%32] of its 32x32 block.
     // The reads of C_old (beta given) are issued for a whole 32x32 block before any is used; in the
     // bounds-checked instantiation their addresses are clamped into C instead of being skipped, so
@@ -600,9 +671,11 @@ template <int ROWS, int BK, bool KCONTIG> struct SlabD {
     static constexpr int SIZE = KCONTIG ? ROWS * LD : BK * LD;
 };
 
-template <int BM, int BN, int BK, int WAVES_M, int WAVES_N, int OCC, bool A_K, bool B_K, bool EDGE, bool EXT = false, int KS = 1>
+template <int BM, int BN, int BK, int WAVES_M, int WAVES_N, int OCC, bool A_K, bool B_K, bool EDGE, bool EXT = false, int KS = 1,
+          bool SPLIT = false>
 __global__ __launch_bounds__(WAVES_M *WAVES_N * 64 * KS) __attribute__((amdgpu_waves_per_eu(OCC)))
 void gemm_f64_mfma_kernel(MArgs<double> g) {
+    static_assert(!SPLIT || KS == 1, "k is split over work-groups or inside one, not both");
     constexpr int NT = WAVES_M * WAVES_N * 64 * KS; // KS groups of wavefronts split each slab, as in the f32 kernel
     constexpr int BKT = BK * KS;
     constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N;
@@ -625,6 +698,13 @@ void gemm_f64_mfma_kernel(MArgs<double> g) {
     uint32_t tile_m, tile_n;
     tile_coords(g.tiles_m, g.tiles_n, tile_m, tile_n, g.xcd_remap);
     const uint32_t m0 = tile_m * BM, n0 = tile_n * BN;
+    if constexpr (SPLIT) { // this work-group's share of k, as in the f32 kernel
+        const uint32_t k_begin = blockIdx.y * g.klen;
+        const uint32_t k_end = min(g.K, k_begin + g.klen);
+        g.A += A_K ? (size_t)k_begin : (size_t)k_begin * g.lda;
+        g.B += B_K ? (size_t)k_begin : (size_t)k_begin * g.ldb;
+        g.K = k_end - k_begin;
+    }
     // one solo iteration = FM*FN*BK/4 matrix instructions of 64 clocks = FM*FN*BK/8 sleep units
     startup_stagger(g.num_cus, OCC, FM * FN * BK / 8 > 0 ? FM * FN * BK / 8 : 1);
 
@@ -926,6 +1006,51 @@ void gemm_f64_mfma_kernel(MArgs<double> g) {
         }
     }
 
+    if constexpr (SPLIT) {
+        // partial tiles of the shares through memory, added by the last arrival in the order of the
+        // shares; device-scope accesses and a wait for the stores instead of fences (see the f32 kernel)
+        __shared__ uint32_t s_last;
+        constexpr int Q = FM * FN * 4;
+        constexpr size_t TILE = (size_t)BM * BN;
+        double *mine = g.partials + ((size_t)blockIdx.y * gridDim.x + blockIdx.x) * TILE + tid;
+#pragma unroll
+        for (int i = 0; i < FM; ++i)
+#pragma unroll
+            for (int j = 0; j < FN; ++j)
+#pragma unroll
+                for (int r = 0; r < 4; ++r)
+                    __hip_atomic_store(mine + (size_t)((i * FN + j) * 4 + r) * NT, acc[i][j][r], __ATOMIC_RELAXED,
+                                       __HIP_MEMORY_SCOPE_AGENT);
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        __syncthreads();
+        if (tid == 0) {
+            const uint32_t before = __hip_atomic_fetch_add(&g.counters[blockIdx.x], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            const uint32_t last = before == gridDim.y - 1 ? 1u : 0u;
+            if (last) __hip_atomic_store(&g.counters[blockIdx.x], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            s_last = last;
+        }
+        __syncthreads();
+        if (!s_last) return;
+#pragma unroll
+        for (int i = 0; i < FM; ++i)
+#pragma unroll
+            for (int j = 0; j < FN; ++j)
+#pragma unroll
+                for (int r = 0; r < 4; ++r) acc[i][j][r] = 0.0;
+        for (uint32_t z = 0; z < gridDim.y; ++z) {
+            const double *part = g.partials + ((size_t)z * gridDim.x + blockIdx.x) * TILE + tid;
+            double v[Q];
+#pragma unroll
+            for (int q = 0; q < Q; ++q) v[q] = __hip_atomic_load(part + (size_t)q * NT, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+#pragma unroll
+            for (int i = 0; i < FM; ++i)
+#pragma unroll
+                for (int j = 0; j < FN; ++j)
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) acc[i][j][r] += v[(i * FN + j) * 4 + r];
+        }
+    }
+
     const double alpha = g.alpha, beta = g.beta;
 #pragma unroll
     for (int i = 0; i < FM; ++i)
@@ -964,7 +1089,7 @@ void gemm_f64_mfma_kernel(MArgs<double> g) {
 // ------------------------------------------------------------------------------ dispatch ---
 
 template <typename T> MArgs<T> make_args(const GemmProblem &p, int bm, int bn) {
-    MArgs<T> g;
+    MArgs<T> g{}; // every field starts at zero / null; a split launch fills klen, partials and counters itself
     g.A = static_cast<const T *>(p.A);
     g.B = static_cast<const T *>(p.B);
     g.C = static_cast<T *>(p.C);
@@ -995,14 +1120,38 @@ template <typename K> int set_lds(K kernel, size_t bytes) {
     return WK_OK;
 }
 
-template <int BM, int BN, int BK, int WMS, int WNS, int OCC, bool AK, bool BKC, bool EDGE, bool EXT = false, int KS = 1, int LSEL = -1>
-int launch_f32_one(hipStream_t st, const GemmProblem &p) {
+// Fills the split-k fields of the kernel arguments from a plan and checks, on the host, everything the
+// kernel takes for granted: memory for the partial tiles and a counter for every tile.
+template <typename T> int apply_split(MArgs<T> &g, const GemmProblem &p, const GemmSplitPlan &plan, int bm, int bn) {
+    if (plan.shares < 2 || plan.klen == 0) return WK_E_INVALID_VALUE;
+    if (!p.scratch || !p.counters) return WK_E_INVALID_VALUE;
+    if (plan.tiles != (uint64_t)g.tiles_m * g.tiles_n || plan.tiles > p.num_counters) return WK_E_INVALID_VALUE;
+    if ((uint64_t)plan.shares * plan.tiles * bm * bn * sizeof(T) > p.scratch_bytes) return WK_E_INVALID_VALUE;
+    if ((uint64_t)plan.klen * (plan.shares - 1) >= p.K || (uint64_t)plan.klen * plan.shares < p.K) return WK_E_INVALID_VALUE;
+    if (plan.shares > 65535) return WK_E_INVALID_VALUE;
+    g.klen = plan.klen;
+    g.partials = static_cast<T *>(p.scratch);
+    g.counters = p.counters;
+    g.xcd_remap = 0; // blockIdx.x is the tile's number, its counter's index and its place among the partial tiles
+    return WK_OK;
+}
+
+template <int BM, int BN, int BK, int WMS, int WNS, int OCC, bool AK, bool BKC, bool EDGE, bool EXT = false, int KS = 1, int LSEL = -1,
+          bool SPLIT = false>
+int launch_f32_one(hipStream_t st, const GemmProblem &p, const GemmSplitPlan *plan = nullptr) {
     constexpr size_t lds = 2 * (Slab<BM, BK * KS, AK>::SIZE + Slab<BN, BK * KS, BKC>::SIZE) * sizeof(float);
-    auto kern = gemm_f32_mfma_kernel<BM, BN, BK, WMS, WNS, OCC, AK, BKC, EDGE, EXT, KS, LSEL>;
+    auto kern = gemm_f32_mfma_kernel<BM, BN, BK, WMS, WNS, OCC, AK, BKC, EDGE, EXT, KS, LSEL, SPLIT>;
     static int attr_rc = set_lds(kern, lds);
     if (attr_rc) return attr_rc;
     MArgs<float> g = make_args<float>(p, BM, BN);
-    hipLaunchKernelGGL(kern, dim3(g.tiles_m * g.tiles_n), dim3(WMS * WNS * 64 * KS), lds, st, g);
+    unsigned shares = 1;
+    if constexpr (SPLIT) {
+        if (!plan) return WK_E_INVALID_VALUE;
+        const int rc = apply_split(g, p, *plan, BM, BN);
+        if (rc) return rc;
+        shares = plan->shares;
+    }
+    hipLaunchKernelGGL(kern, dim3(g.tiles_m * g.tiles_n, shares), dim3(WMS * WNS * 64 * KS), lds, st, g);
     return launch_status();
 }
 
@@ -1027,14 +1176,22 @@ int launch_f32(hipStream_t st, const GemmProblem &p, bool edge) {
 #undef WK_CASE
 }
 
-template <int BM, int BN, int BK, int WMS, int WNS, int OCC, bool AK, bool BKC, bool EDGE, bool EXT = false, int KS = 1>
-int launch_f64_one(hipStream_t st, const GemmProblem &p) {
+template <int BM, int BN, int BK, int WMS, int WNS, int OCC, bool AK, bool BKC, bool EDGE, bool EXT = false, int KS = 1,
+          bool SPLIT = false>
+int launch_f64_one(hipStream_t st, const GemmProblem &p, const GemmSplitPlan *plan = nullptr) {
     constexpr size_t lds = 2 * (SlabD<BM, BK * KS, AK>::SIZE + SlabD<BN, BK * KS, BKC>::SIZE) * sizeof(double);
-    auto kern = gemm_f64_mfma_kernel<BM, BN, BK, WMS, WNS, OCC, AK, BKC, EDGE, EXT, KS>;
+    auto kern = gemm_f64_mfma_kernel<BM, BN, BK, WMS, WNS, OCC, AK, BKC, EDGE, EXT, KS, SPLIT>;
     static int attr_rc = set_lds(kern, lds);
     if (attr_rc) return attr_rc;
     MArgs<double> g = make_args<double>(p, BM, BN);
-    hipLaunchKernelGGL(kern, dim3(g.tiles_m * g.tiles_n), dim3(WMS * WNS * 64 * KS), lds, st, g);
+    unsigned shares = 1;
+    if constexpr (SPLIT) {
+        if (!plan) return WK_E_INVALID_VALUE;
+        const int rc = apply_split(g, p, *plan, BM, BN);
+        if (rc) return rc;
+        shares = plan->shares;
+    }
+    hipLaunchKernelGGL(kern, dim3(g.tiles_m * g.tiles_n, shares), dim3(WMS * WNS * 64 * KS), lds, st, g);
     return launch_status();
 }
 
@@ -1058,6 +1215,77 @@ int launch_f64(hipStream_t st, const GemmProblem &p, bool edge) {
 #undef WK_CASE
 }
 
+// ---- k split over work-groups ------------------------------------------------------------------
+// A product with few tiles of C and a long k leaves most compute units without work (512 x 512 x 8192
+// is 64 tiles of 64 x 64 on 256 units).  These variants give every tile to `shares` work-groups, each
+// summing a contiguous range of k; the partial tiles meet in the stream's scratch memory and the
+// work-group that arrives last at the tile's counter adds them in the order of the shares, so the
+// result is the same bits on every run.
+//   relaxed (a forced variant, tests): split whenever k holds two slabs, up to four shares.
+//   otherwise: only when the tiles leave at least half the compute units idle, as many shares as put
+//   four (f64: two) work-groups on every unit (a power of two, at most 64), each share at least eight
+//   slabs long.
+bool plan_split(const GemmProblem &p, int bm, int bn, int bkt, size_t elem, bool relaxed, GemmSplitPlan &plan) {
+    plan = GemmSplitPlan{};
+    plan.tiles = ((p.M + bm - 1) / bm) * ((p.N + bn - 1) / bn);
+    const uint64_t slabs = (p.K + bkt - 1) / bkt;
+    uint64_t shares = 1;
+    if (relaxed) {
+        shares = slabs >= 4 ? 4 : slabs;
+    } else {
+        // up to `occ` work-groups per compute unit (what the tile's registers and LDS allow): co-resident
+        // work-groups are what hides the slab hand-overs of one another
+        const uint64_t cus = p.num_cus ? p.num_cus : 256;
+        const uint64_t occ = elem == 8 ? 2 : 4;
+        if (plan.tiles * 2 > cus) return false;
+        while (shares < 64 && plan.tiles * shares * 2 <= cus * occ && slabs / (shares * 2) >= 8) shares *= 2;
+    }
+    if (shares < 2) return false;
+    const uint64_t klen = (slabs + shares - 1) / shares * bkt; // whole slabs per share
+    shares = (p.K + klen - 1) / klen;                           // the last share may have vanished
+    if (shares < 2) return false;
+    plan.shares = (uint32_t)shares;
+    plan.klen = (uint32_t)klen;
+    plan.bytes = (size_t)(shares * plan.tiles * bm * bn * elem);
+    return p.scratch && p.counters && plan.bytes <= p.scratch_bytes && plan.tiles <= p.num_counters;
+}
+
+// The 64 x 64 tiles with k split over work-groups; without a feasible plan (short k, no scratch, the
+// fused epilogue) the plain tile runs.
+int launch_f32_split64(hipStream_t st, const GemmProblem &p, bool edge) {
+    constexpr int BM = 64, BN = 64, BK = 32;
+    GemmSplitPlan plan;
+    if (p.ext || !plan_split(p, BM, BN, BK, sizeof(float), true, plan)) return launch_f32<BM, BN, BK, 2, 2, 4>(st, p, edge);
+    const int sel = (p.op_a ? 0 : 2) | (p.op_b ? 1 : 0);
+#define WK_CASE(AK, BKC)                                                                                                \
+    return edge ? launch_f32_one<BM, BN, BK, 2, 2, 4, AK, BKC, true, false, 1, -1, true>(st, p, &plan)                    \
+                : launch_f32_one<BM, BN, BK, 2, 2, 4, AK, BKC, false, false, 1, -1, true>(st, p, &plan)
+    switch (sel) {
+    case 0: WK_CASE(false, false);
+    case 1: WK_CASE(false, true);
+    case 2: WK_CASE(true, false);
+    default: WK_CASE(true, true);
+    }
+#undef WK_CASE
+}
+
+int launch_f64_split64(hipStream_t st, const GemmProblem &p, bool edge) {
+    constexpr int BM = 64, BN = 64, BK = 32;
+    GemmSplitPlan plan;
+    if (p.ext || !plan_split(p, BM, BN, BK, sizeof(double), true, plan)) return launch_f64<BM, BN, BK, 2, 2, 2>(st, p, edge);
+    const int sel = (p.op_a ? 0 : 2) | (p.op_b ? 1 : 0);
+#define WK_CASE(AK, BKC)                                                                                                \
+    return edge ? launch_f64_one<BM, BN, BK, 2, 2, 2, AK, BKC, true, false, 1, true>(st, p, &plan)                        \
+                : launch_f64_one<BM, BN, BK, 2, 2, 2, AK, BKC, false, false, 1, true>(st, p, &plan)
+    switch (sel) {
+    case 0: WK_CASE(false, false);
+    case 1: WK_CASE(false, true);
+    case 2: WK_CASE(true, false);
+    default: WK_CASE(true, true);
+    }
+#undef WK_CASE
+}
+
 struct VariantDesc {
     const char *name;
     int dtype, bm, bn, bk; // bk: k values per LDS slab
@@ -1070,6 +1298,8 @@ struct VariantDesc {
     // and the quarter-size tile (one wavefront's 32x32, k split over four of them) for launches
     // whose tiles of this size would leave a quarter of the CUs or more without work
     const char *sparse = nullptr;
+    // and the same tile with k split over work-groups, for few tiles and a long k (plan_split)
+    const char *split = nullptr;
 };
 
 const VariantDesc k_variants[] = {
@@ -1077,13 +1307,15 @@ const VariantDesc k_variants[] = {
     {"mfma_f32_128x128", WK_F32, 128, 128, 16, 0.885, 0.25, &launch_f32<128, 128, 16, 2, 2, 3>},
     {"mfma_f32_128x128s2", WK_F32, 128, 128, 32, 0.0, 0.25, &launch_f32<128, 128, 16, 2, 2, 2, 2>}, // 2 groups x 16 k, see pick
     {"mfma_f32_64x64", WK_F32, 64, 64, 32, 0.780, 0.10, &launch_f32<64, 64, 32, 2, 2, 4>, "mfma_f32_64x64s4", "mfma_f32_64x64s2",
-     "mfma_f32_32x32s4"},
+     "mfma_f32_32x32s4", "mfma_f32_64x64z"},
+    {"mfma_f32_64x64z", WK_F32, 64, 64, 32, 0.0, 0.10, &launch_f32_split64}, // k split over work-groups
     {"mfma_f32_64x64s2", WK_F32, 64, 64, 32, 0.0, 0.10, &launch_f32<64, 64, 16, 2, 2, 4, 2>}, // 2 groups x 16 k
     {"mfma_f32_64x64s4", WK_F32, 64, 64, 64, 0.0, 0.10, &launch_f32<64, 64, 16, 2, 2, 4, 4>}, // 4 groups x 16 k
     {"mfma_f32_32x32s4", WK_F32, 32, 32, 64, 0.0, 0.10, &launch_f32<32, 32, 16, 1, 1, 4, 4>}, // one wavefront's tile, 4 groups
     {"mfma_f64_128x128", WK_F64, 128, 128, 16, 0.908, 0.20, &launch_f64<128, 128, 16, 2, 2, 2>},
     {"mfma_f64_64x64", WK_F64, 64, 64, 32, 0.840, 0.05, &launch_f64<64, 64, 32, 2, 2, 2>, "mfma_f64_64x64s2", nullptr,
-     "mfma_f64_32x32s4"},
+     "mfma_f64_32x32s4", "mfma_f64_64x64z"},
+    {"mfma_f64_64x64z", WK_F64, 64, 64, 32, 0.0, 0.05, &launch_f64_split64}, // k split over work-groups
     {"mfma_f64_64x64s2", WK_F64, 64, 64, 64, 0.0, 0.05, &launch_f64<64, 64, 32, 2, 2, 2, 2>}, // 2 groups x 32 k
     // (two wavefronts per SIMD: with a 128-register budget its staging sets and fragments spill and it
     // runs several times slower than the 64x64 tile)
@@ -1144,6 +1376,25 @@ int wk::gemm_mfma_variant_dtype(int variant) {
 // is shorter than the latency of the global loads behind it, and the deeper slab halves the number
 // of such waits (f32 1024^3: 76 -> 84 TFLOP/s, 2048x1024x4096: 116 -> 130; f64 8192x256x8192:
 // 56 -> 60); the larger tiles measured no better with it.
+bool wk::gemm_mfma_split_plan(const GemmProblem &p, int variant, bool forced, GemmSplitPlan &plan) {
+    plan = GemmSplitPlan{};
+    if (variant < 0 || variant >= k_num_variants || p.ext) return false;
+    const VariantDesc &v = k_variants[variant];
+    if (v.launch != &launch_f32_split64 && v.launch != &launch_f64_split64) return false;
+    return plan_split(p, v.bm, v.bn, v.bk, v.dtype == WK_F64 ? 8 : 4, forced, plan);
+}
+
+namespace {
+// Splitting k costs a write and a read of every partial tile and one more pass of additions.  Measured
+// on MI355X against the quarter-size tile with k split inside the work-group, the next best choice for
+// few tiles: f32 512 x 512 x 8192 57 -> 52 us, 256 x 256 x 8192 54 -> 45, 1024 x 512 x 4096 43.5 -> 42,
+// but 512 x 512 x 2048 14.4 -> 18.6; f64 512 x 512 x 8192 111 -> 89 us, 256 x 256 x 8192 111 -> 89,
+// 512 x 512 x 2048 32 -> 30.
+bool split_pays(const GemmProblem &p, const GemmSplitPlan &plan) {
+    return plan.shares >= 2 && p.K >= (p.dtype == WK_F64 ? 2048u : 4096u);
+}
+} // namespace
+
 int wk::gemm_mfma_pick(const GemmProblem &p) {
     if (p.dtype != WK_F32 && p.dtype != WK_F64 && p.dtype != WK_I32 && p.dtype != WK_U32) return -1;
     if (p.M > 0x7fffffffull || p.N > 0x7fffffffull || p.K > 0x7fffffffull || p.lda > 0x7fffffffull ||
@@ -1184,7 +1435,11 @@ int wk::gemm_mfma_pick(const GemmProblem &p) {
         const VariantDesc &d = k_variants[best];
         const double tiles = (double)((p.M + d.bm - 1) / d.bm) * (double)((p.N + d.bn - 1) / d.bn);
         const char *twin = nullptr;
-        if (tiles <= 0.75 * cus && d.sparse) twin = d.sparse; // (f64 512^3: 21.5 -> 10.3 us, 512x512x2048: 74 -> 32 us)
+        GemmSplitPlan plan;
+        if (d.split && !p.ext && plan_split(p, d.bm, d.bn, d.bk, p.dtype == WK_F64 ? 8 : 4, false, plan) &&
+            split_pays(p, plan))
+            twin = d.split;
+        else if (tiles <= 0.75 * cus && d.sparse) twin = d.sparse; // (f64 512^3: 21.5 -> 10.3 us, 512x512x2048: 74 -> 32 us)
         else if (p.K >= 256) twin = tiles <= cus ? d.one_round : (tiles <= 2.0 * cus ? d.two_rounds : nullptr);
         for (int v = 0; twin && v < k_num_variants; ++v)
             if (!std::strcmp(k_variants[v].name, twin)) return v;

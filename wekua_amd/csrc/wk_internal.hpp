@@ -20,9 +20,16 @@ struct wk_stream {
     // stream is in order, so consecutive users never overlap).  Allocated with the stream.
     void *scratch;
     size_t scratch_bytes;
+    // Arrival counters of the GEMM that splits k over work-groups: one per tile of C, zero between
+    // launches (the work-group that arrives last at its tile's counter puts it back to zero).
+    uint32_t *gemm_counters;
 };
 
-constexpr size_t WK_STREAM_SCRATCH_BYTES = 1u << 20;
+constexpr size_t WK_STREAM_SCRATCH_BYTES = 16u << 20;
+constexpr size_t WK_GEMM_COUNTERS = 4096;
+// what wk_bias_step uses of the scratch: the number of row bands, and with it the order of the
+// additions, follows from this size, so it stays what it was when the scratch was this small
+constexpr size_t WK_BIAS_STEP_SCRATCH_BYTES = 1u << 20;
 
 struct wk_event {
     wk_device *dev;
@@ -170,7 +177,26 @@ struct GemmProblem {
     int ext_act = -1;                 // WK_ACT_*
     // the workspace still holds op(B)'s packed form from the previous call (wk_gemm_packed_b_kept)
     bool reuse_b = false;
+    // for kernels that split k over work-groups: device memory for the partial tiles and the tiles'
+    // arrival counters (the stream's; null: such kernels are not chosen, and refuse when forced)
+    void *scratch = nullptr;
+    size_t scratch_bytes = 0;
+    uint32_t *counters = nullptr;
+    size_t num_counters = 0;
 };
+
+// How a launch that splits k over work-groups is laid out; host arithmetic only.
+struct GemmSplitPlan {
+    uint32_t shares = 1;   // work-groups per tile of C (grid y); 1: no split
+    uint32_t klen = 0;     // k values per share, a multiple of the kernel's k-slab; the last share takes what is left
+    uint64_t tiles = 0;    // tiles of C (grid x) = arrival counters used
+    size_t bytes = 0;      // partial tiles: shares * tiles * tile area * element size
+};
+// Plan for `variant` (a split-k variant) on p.  forced: split whenever k holds two slabs, whatever the
+// number of tiles (tests); otherwise only when the tiles leave half the compute units idle and every
+// share keeps a few slabs.  Returns false when the variant does not split or the plan does not fit
+// p.scratch_bytes / p.num_counters (a null p.scratch or p.counters also fails).
+bool gemm_mfma_split_plan(const GemmProblem &p, int variant, bool forced, GemmSplitPlan &plan);
 
 // generic LDS-tiled VALU kernel, every dtype and shape (wk_gemm_generic.hip)
 int gemm_generic_launch(hipStream_t st, const GemmProblem &p);

@@ -147,6 +147,136 @@ __global__ __launch_bounds__(256) void colsum_bands_kernel(const T *__restrict__
         partial[blockIdx.y * cols + c] = (part[0][threadIdx.x] + part[1][threadIdx.x]) + (part[2][threadIdx.x] + part[3][threadIdx.x]);
 }
 
+// ---- Linear.backward's element-wise half in one pass (linear.zig:606-640: getDerivative, math.dot,
+// getBiasSensitivity): dev = act'(out), sens *= dev, and the band partials of the column sums of the
+// new sens.  Same block shape and the same order of additions per column as colsum_bands_kernel
+// (rows r0 + ty, r0 + ty + 4, ... per thread row ty, then (p0 + p1) + (p2 + p3)), so the bias gradient
+// comes out bit for bit as from the separate passes; every lane moves VE consecutive columns.
+// kind WK_ACT_NONE: dev is read, not written (the reference multiplies by the cached tensor as it is).
+template <typename T, bool VEC>
+__global__ __launch_bounds__(256) void sens_step_kernel(int kind, const T *__restrict__ out, uint64_t out_pitch, T *__restrict__ sens,
+                                                        uint64_t sens_pitch, T *__restrict__ dev, uint64_t dev_pitch, uint64_t rows,
+                                                        uint64_t cols, uint64_t band_rows, T *__restrict__ partial) {
+    constexpr int VE = VEC ? 16 / sizeof(T) : 1;
+    __shared__ T part[4][64][VE];
+    const uint64_t c = (blockIdx.x * 64ull + threadIdx.x) * VE;
+    const uint64_t r0 = blockIdx.y * band_rows;
+    const uint64_t r1 = r0 + band_rows < rows ? r0 + band_rows : rows;
+    T acc[VE];
+#pragma unroll
+    for (int e = 0; e < VE; ++e) acc[e] = T(0);
+    if (c < cols) {
+        const bool whole = VEC && c + VE <= cols;
+        for (uint64_t r = r0 + threadIdx.y; r < r1; r += 4) {
+            T *sp = sens + r * sens_pitch + c;
+            T *dp = dev + r * dev_pitch + c;
+            const T *op = out + r * out_pitch + c;
+            T sv[VE], dv[VE], ov[VE];
+            if (whole) {
+                __builtin_memcpy(sv, sp, sizeof sv);
+                if (kind == WK_ACT_NONE) __builtin_memcpy(dv, dp, sizeof dv);
+                else __builtin_memcpy(ov, op, sizeof ov);
+            } else {
+                for (int e = 0; e < VE; ++e) {
+                    const bool ok = c + e < cols;
+                    sv[e] = ok ? sp[e] : T(0);
+                    dv[e] = ok && kind == WK_ACT_NONE ? dp[e] : T(0);
+                    ov[e] = ok && kind != WK_ACT_NONE ? op[e] : T(0);
+                }
+            }
+#pragma unroll
+            for (int e = 0; e < VE; ++e) {
+                if (kind != WK_ACT_NONE) dv[e] = act_derivative<T>(kind, ov[e]);
+                {
+                    // the product is rounded before it is added (no fused multiply-add): the sum must be
+                    // over the values that are stored, as in the separate passes
+#pragma clang fp contract(off)
+                    sv[e] = sv[e] * dv[e];
+                    acc[e] = acc[e] + sv[e];
+                }
+            }
+            if (whole) {
+                if (kind != WK_ACT_NONE) __builtin_memcpy(dp, dv, sizeof dv);
+                __builtin_memcpy(sp, sv, sizeof sv);
+            } else {
+                for (int e = 0; e < VE; ++e)
+                    if (c + e < cols) {
+                        if (kind != WK_ACT_NONE) dp[e] = dv[e];
+                        sp[e] = sv[e];
+                    }
+            }
+        }
+    }
+    if (!partial) return;
+#pragma unroll
+    for (int e = 0; e < VE; ++e) part[threadIdx.y][threadIdx.x][e] = acc[e];
+    __syncthreads();
+    if (threadIdx.y == 0 && c < cols)
+#pragma unroll
+        for (int e = 0; e < VE; ++e)
+            if (c + e < cols)
+                partial[blockIdx.y * cols + c + e] =
+                    (part[0][threadIdx.x][e] + part[1][threadIdx.x][e]) + (part[2][threadIdx.x][e] + part[3][threadIdx.x][e]);
+}
+
+// One element of the Adam update.  Every product is rounded before it is added (no fused
+// multiply-add), so the one-tensor and the several-tensor kernels give the same bits whatever the
+// compiler makes of their surroundings.
+template <typename T>
+__device__ __forceinline__ void adam_update(T &w, T &m, T &v, T g, T b1, T ib1, T b2, T ib2, T step_size, T inv_sqrt_bc2, T eps) {
+#pragma clang fp contract(off)
+    m = b1 * m + ib1 * g;
+    v = b2 * v + (ib2 * g) * g;
+    w = w - step_size * m / (sqrt(v) * inv_sqrt_bc2 + eps);
+}
+
+// ---- Adam over several parameter tensors in one launch.  Blocks are dealt to the tensors in
+// proportion to their size; inside its tensor a block walks 16-byte vectors with a grid stride.
+constexpr int ADAM_MULTI_MAX = 8;
+template <typename T> struct AdamMultiArgs {
+    T *w[ADAM_MULTI_MAX], *m[ADAM_MULTI_MAX], *v[ADAM_MULTI_MAX];
+    const T *g[ADAM_MULTI_MAX];
+    uint64_t rows[ADAM_MULTI_MAX], cols[ADAM_MULTI_MAX]; // depth folded into rows (slices are back to back)
+    uint64_t wrp[ADAM_MULTI_MAX], grp[ADAM_MULTI_MAX], mrp[ADAM_MULTI_MAX];
+    uint32_t first_block[ADAM_MULTI_MAX + 1];
+    int count;
+    T b1, b2, ib1, ib2, step_size, inv_sqrt_bc2, eps;
+};
+
+template <typename T>
+__global__ __launch_bounds__(EW_BLOCK) void adam_multi_kernel(AdamMultiArgs<T> a) {
+    constexpr int VE = 16 / sizeof(T);
+    int t = 0;
+    while (t + 1 < a.count && blockIdx.x >= a.first_block[t + 1]) ++t;
+    const uint64_t nblocks = a.first_block[t + 1] - a.first_block[t];
+    const uint64_t cols_v = (a.cols[t] + VE - 1) / VE;
+    const uint64_t total = a.rows[t] * cols_v;
+    for (uint64_t idx = (blockIdx.x - a.first_block[t]) * (uint64_t)EW_BLOCK + threadIdx.x; idx < total; idx += nblocks * EW_BLOCK) {
+        const uint64_t r = idx / cols_v, c = (idx % cols_v) * VE;
+        T *wp = a.w[t] + r * a.wrp[t] + c, *mp = a.m[t] + r * a.mrp[t] + c, *vp = a.v[t] + r * a.mrp[t] + c;
+        const T *gp = a.g[t] + r * a.grp[t] + c;
+        const bool whole = c + VE <= a.cols[t];
+        T wv[VE], mv[VE], vv[VE], gv[VE];
+        if (whole) {
+            __builtin_memcpy(wv, wp, 16); __builtin_memcpy(mv, mp, 16); __builtin_memcpy(vv, vp, 16); __builtin_memcpy(gv, gp, 16);
+        } else {
+            for (int e = 0; e < VE; ++e) {
+                const bool ok = c + e < a.cols[t];
+                wv[e] = ok ? wp[e] : T(0); mv[e] = ok ? mp[e] : T(0); vv[e] = ok ? vp[e] : T(1); gv[e] = ok ? gp[e] : T(0);
+            }
+        }
+#pragma unroll
+        for (int e = 0; e < VE; ++e)
+            adam_update<T>(wv[e], mv[e], vv[e], gv[e], a.b1, a.ib1, a.b2, a.ib2, a.step_size, a.inv_sqrt_bc2, a.eps);
+        if (whole) {
+            __builtin_memcpy(wp, wv, 16); __builtin_memcpy(mp, mv, 16); __builtin_memcpy(vp, vv, 16);
+        } else {
+            for (int e = 0; e < VE; ++e)
+                if (c + e < a.cols[t]) { wp[e] = wv[e]; mp[e] = mv[e]; vp[e] = vv[e]; }
+        }
+    }
+}
+
 // ---- whole-tensor sum (math.sum + host finish, src/math/basic.zig:128-203): two fixed-shape
 // passes so that the result does not depend on scheduling. ------------------------------------
 constexpr int SUM_PARTIALS = 1024;
@@ -208,16 +338,22 @@ namespace {
 // Column sums of a rows x cols matrix in two launches of colsum_bands_kernel: bands of rows into
 // `partial_buf`, then the bands.  The number of bands depends only on (rows, cols, partial_bytes),
 // so two callers with equally sized buffers add in the same order and get the same bits.
+// How the rows are cut into bands: depends only on (rows, cols, element size, partial_bytes).
+inline void colsum_plan(uint64_t rows, uint64_t cols, size_t esize, size_t partial_bytes, uint64_t &bands, uint64_t &band_rows) {
+    bands = (rows + COLSUM_ROWS_PER_BAND - 1) / COLSUM_ROWS_PER_BAND;
+    if (bands > COLSUM_MAX_BANDS) bands = COLSUM_MAX_BANDS;
+    const uint64_t fit = partial_bytes / (cols * esize);
+    if (bands > fit) bands = fit;
+    if (bands < 2) bands = 1; // one band writes the result directly
+    band_rows = (rows + bands - 1) / bands;
+    bands = (rows + band_rows - 1) / band_rows;
+}
+
 template <typename T>
 int colsum_two_pass(wk_stream *s, uint64_t rows, uint64_t cols, const T *sens, uint64_t pitch, T *bias_grad,
                     void *partial_buf, size_t partial_bytes) {
-    uint64_t bands = (rows + COLSUM_ROWS_PER_BAND - 1) / COLSUM_ROWS_PER_BAND;
-    if (bands > COLSUM_MAX_BANDS) bands = COLSUM_MAX_BANDS;
-    const uint64_t fit = partial_bytes / (cols * sizeof(T));
-    if (bands > fit) bands = fit;
-    if (bands < 2) bands = 1; // one band writes the result directly
-    const uint64_t band_rows = (rows + bands - 1) / bands;
-    bands = (rows + band_rows - 1) / band_rows;
+    uint64_t bands, band_rows;
+    colsum_plan(rows, cols, sizeof(T), partial_bytes, bands, band_rows);
     T *partial = bands > 1 ? static_cast<T *>(partial_buf) : bias_grad;
     hipLaunchKernelGGL((colsum_bands_kernel<T>), dim3((unsigned)((cols + 63) / 64), (unsigned)bands), dim3(64, 4), 0,
                        s->stream, sens, rows, cols, pitch, band_rows, partial);
@@ -296,9 +432,9 @@ int wk_bias_step(wk_stream *s, int dtype, uint64_t rows, uint64_t cols, const vo
     if (!rows || !cols || !sens || !bias_grad || pitch < cols) return WK_E_INVALID_VALUE;
     if ((cols + 63) / 64 > 0x7fffffffull) return WK_E_INVALID_VALUE;
     return dispatch_float(dtype, [&]<typename T>() -> int {
-        // as many bands as the stream's scratch holds partials for
+        // as many bands as its share of the stream's scratch holds partials for
         return colsum_two_pass<T>(s, rows, cols, static_cast<const T *>(sens), pitch, static_cast<T *>(bias_grad), s->scratch,
-                                  s->scratch_bytes);
+                                  s->scratch_bytes < WK_BIAS_STEP_SCRATCH_BYTES ? s->scratch_bytes : WK_BIAS_STEP_SCRATCH_BYTES);
     });
 }
 
@@ -317,6 +453,104 @@ int wk_bias_step_static(wk_stream *s, int dtype, uint64_t rows, uint64_t cols, c
     return dispatch_float(dtype, [&]<typename T>() -> int {
         return colsum_two_pass<T>(s, rows, cols, static_cast<const T *>(sens), pitch, static_cast<T *>(bias_grad), ptr,
                                   STATIC_SCRATCH_BYTES);
+    });
+}
+
+int wk_sensitivity_step(wk_stream *s, int dtype, int kind, uint64_t rows, uint64_t cols, const void *out, uint64_t out_pitch,
+                        void *sens, uint64_t sens_pitch, void *dev, uint64_t dev_pitch, void *bias_grad) {
+    int rc = bind(s);
+    if (rc) return rc;
+    if (kind != WK_ACT_NONE && kind != WK_ACT_SIGMOID && kind != WK_ACT_TANH) return WK_E_INVALID_VALUE;
+    if (dtype != WK_F32 && dtype != WK_F64) return WK_E_TYPE_NOT_SUPPORTED;
+    if (!rows || !cols || !sens || !dev || sens_pitch < cols || dev_pitch < cols) return WK_E_INVALID_VALUE;
+    if (kind != WK_ACT_NONE && (!out || out_pitch < cols)) return WK_E_INVALID_VALUE;
+    return dispatch_float(dtype, [&]<typename T>() -> int {
+        constexpr uint64_t VE = 16 / sizeof(T);
+        const auto aligned = [&](const void *p, uint64_t pitch) { return !p || ((reinterpret_cast<uintptr_t>(p) & 15u) == 0 && pitch % VE == 0); };
+        const bool vec = aligned(kind != WK_ACT_NONE ? out : nullptr, out_pitch) && aligned(sens, sens_pitch) && aligned(dev, dev_pitch);
+        const uint64_t per_block = 64 * (vec ? VE : 1);
+        if ((cols + per_block - 1) / per_block > 0x7fffffffull) return WK_E_INVALID_VALUE;
+        // the bands of wk_bias_step, so that the bias gradient is the same bits as from that call
+        uint64_t bands, band_rows;
+        colsum_plan(rows, cols, sizeof(T), s->scratch_bytes < WK_BIAS_STEP_SCRATCH_BYTES ? s->scratch_bytes : WK_BIAS_STEP_SCRATCH_BYTES,
+                    bands, band_rows);
+        T *bg = static_cast<T *>(bias_grad);
+        T *partial = !bg ? nullptr : bands > 1 ? static_cast<T *>(s->scratch) : bg;
+        const dim3 grid((unsigned)((cols + per_block - 1) / per_block), (unsigned)bands), block(64, 4);
+        if (vec)
+            hipLaunchKernelGGL((sens_step_kernel<T, true>), grid, block, 0, s->stream, kind, static_cast<const T *>(out), out_pitch,
+                               static_cast<T *>(sens), sens_pitch, static_cast<T *>(dev), dev_pitch, rows, cols, band_rows, partial);
+        else
+            hipLaunchKernelGGL((sens_step_kernel<T, false>), grid, block, 0, s->stream, kind, static_cast<const T *>(out), out_pitch,
+                               static_cast<T *>(sens), sens_pitch, static_cast<T *>(dev), dev_pitch, rows, cols, band_rows, partial);
+        int lrc = launch_status();
+        if (lrc || !bg || bands == 1) return lrc;
+        hipLaunchKernelGGL((colsum_bands_kernel<T>), dim3((unsigned)((cols + 63) / 64), 1), dim3(64, 4), 0, s->stream,
+                           static_cast<const T *>(partial), bands, cols, cols, bands, bg);
+        return launch_status();
+    });
+}
+
+int wk_adam_step_multi(wk_stream *s, int dtype, uint32_t count, const wk_adam_tensor *host_tensors, double lr, double beta1,
+                       double beta2, double eps, uint64_t step) {
+    int rc = bind(s);
+    if (rc) return rc;
+    if (!count) return WK_OK;
+    if (!host_tensors || step == 0) return WK_E_INVALID_VALUE;
+    if (dtype != WK_F32 && dtype != WK_F64) return WK_E_TYPE_NOT_SUPPORTED;
+    const double bc1 = 1.0 - std::pow(beta1, (double)step), bc2 = 1.0 - std::pow(beta2, (double)step);
+    return dispatch_float(dtype, [&]<typename T>() -> int {
+        constexpr uint64_t VE = 16 / sizeof(T);
+        // every tensor is validated before anything is launched
+        bool vec = true;
+        for (uint32_t i = 0; i < count; ++i) {
+            const wk_adam_tensor &t = host_tensors[i];
+            Region rg;
+            if (check_region(t.shape3, rg)) return WK_E_INVALID_VALUE;
+            if (check_opnd<T>(rg, t.w, t.w_row_pitch, t.w_slice_pitch) || check_opnd<T>(rg, t.g, t.g_row_pitch, t.g_slice_pitch) ||
+                check_opnd<T>(rg, t.m, t.mv_row_pitch, t.mv_slice_pitch) || check_opnd<T>(rg, t.v, t.mv_row_pitch, t.mv_slice_pitch))
+                return WK_E_INVALID_VALUE;
+            // the one-launch kernel wants 16-byte rows and slices that follow one another at the row pitch
+            const auto ok = [&](const void *p, uint64_t rp, uint64_t sp) {
+                return (reinterpret_cast<uintptr_t>(p) & 15u) == 0 && (rg.rows * rg.depth == 1 || rp % VE == 0) &&
+                       (rg.depth == 1 || sp == rg.rows * rp);
+            };
+            vec = vec && ok(t.w, t.w_row_pitch, t.w_slice_pitch) && ok(t.g, t.g_row_pitch, t.g_slice_pitch) &&
+                  ok(t.m, t.mv_row_pitch, t.mv_slice_pitch) && ok(t.v, t.mv_row_pitch, t.mv_slice_pitch);
+        }
+        if (!vec || count == 1) { // the same update, one launch per tensor
+            for (uint32_t i = 0; i < count; ++i) {
+                const wk_adam_tensor &t = host_tensors[i];
+                const int r = wk_adam_step(s, dtype, t.shape3, t.w, t.w_row_pitch, t.w_slice_pitch, t.g, t.g_row_pitch, t.g_slice_pitch,
+                                           t.m, t.v, t.mv_row_pitch, t.mv_slice_pitch, lr, beta1, beta2, eps, step);
+                if (r) return r;
+            }
+            return WK_OK;
+        }
+        for (uint32_t first = 0; first < count; first += ADAM_MULTI_MAX) {
+            AdamMultiArgs<T> a{};
+            a.count = (int)(count - first < (uint32_t)ADAM_MULTI_MAX ? count - first : ADAM_MULTI_MAX);
+            a.b1 = (T)beta1; a.b2 = (T)beta2; a.ib1 = (T)(1.0 - beta1); a.ib2 = (T)(1.0 - beta2);
+            a.step_size = (T)(lr / bc1); a.inv_sqrt_bc2 = (T)(1.0 / std::sqrt(bc2)); a.eps = (T)eps;
+            uint64_t blocks = 0;
+            for (int i = 0; i < a.count; ++i) {
+                const wk_adam_tensor &t = host_tensors[first + i];
+                a.w[i] = static_cast<T *>(t.w); a.g[i] = static_cast<const T *>(t.g);
+                a.m[i] = static_cast<T *>(t.m); a.v[i] = static_cast<T *>(t.v);
+                a.rows[i] = t.shape3[0] * t.shape3[1]; a.cols[i] = t.shape3[2];
+                a.wrp[i] = t.w_row_pitch; a.grp[i] = t.g_row_pitch; a.mrp[i] = t.mv_row_pitch;
+                const uint64_t vecs = a.rows[i] * ((a.cols[i] + VE - 1) / VE);
+                uint64_t want = (vecs + EW_BLOCK - 1) / EW_BLOCK;
+                if (want > 16384) want = 16384; // grid stride beyond that
+                a.first_block[i] = (uint32_t)blocks;
+                blocks += want ? want : 1;
+            }
+            a.first_block[a.count] = (uint32_t)blocks;
+            hipLaunchKernelGGL((adam_multi_kernel<T>), dim3((unsigned)blocks), dim3(EW_BLOCK), 0, s->stream, a);
+            const int lrc = launch_status();
+            if (lrc) return lrc;
+        }
+        return WK_OK;
     });
 }
 
@@ -388,9 +622,7 @@ int wk_adam_step(wk_stream *s, int dtype, const uint64_t shape3[3], void *w, uin
         return ew_launch<T, 4, 7>(s, rg, Opnd<T>{(T *)w, wrp, wsp}, Opnd<T>{(T *)m, mrp, msp}, Opnd<T>{(T *)v, mrp, msp},
                                Opnd<T>{(T *)g, grp, gsp},
                                [=] __device__(uint64_t, T &wv, T &mv, T &vv, T &gv) {
-                                   mv = b1 * mv + ib1 * gv;
-                                   vv = b2 * vv + ib2 * gv * gv;
-                                   wv -= step_size * mv / (sqrt(vv) * inv_sqrt_bc2 + e);
+                                   adam_update<T>(wv, mv, vv, gv, b1, ib1, b2, ib2, step_size, inv_sqrt_bc2, e);
                                });
     });
 }

@@ -109,6 +109,7 @@ int wk_stream_create(wk_device *dev, wk_stream **out) {
     s->dev = dev;
     s->scratch = nullptr;
     s->scratch_bytes = 0;
+    s->gemm_counters = nullptr;
     hipError_t e = hipStreamCreateWithFlags(&s->stream, hipStreamNonBlocking);
     if (e != hipSuccess) {
         (void)hipGetLastError();
@@ -123,6 +124,18 @@ int wk_stream_create(wk_device *dev, wk_stream **out) {
         return hip_code(e);
     }
     s->scratch_bytes = WK_STREAM_SCRATCH_BYTES;
+    // arrival counters: zero from here on, every kernel that counts on them leaves them at zero
+    e = hipMalloc(reinterpret_cast<void **>(&s->gemm_counters), WK_GEMM_COUNTERS * sizeof(uint32_t));
+    // cleared on the stream itself, so that every later launch on it is ordered behind the clear
+    if (e == hipSuccess) e = hipMemsetAsync(s->gemm_counters, 0, WK_GEMM_COUNTERS * sizeof(uint32_t), s->stream);
+    if (e != hipSuccess) {
+        (void)hipGetLastError();
+        if (s->gemm_counters) (void)hipFree(s->gemm_counters);
+        (void)hipFree(s->scratch);
+        (void)hipStreamDestroy(s->stream);
+        delete s;
+        return hip_code(e);
+    }
     *out = s;
     return WK_OK;
 }
@@ -133,6 +146,7 @@ void wk_stream_destroy(wk_stream *s) {
         (void)hipStreamSynchronize(s->stream);
         (void)hipStreamDestroy(s->stream);
         if (s->scratch) (void)hipFree(s->scratch);
+        if (s->gemm_counters) (void)hipFree(s->gemm_counters);
     }
     (void)hipGetLastError();
     delete s;

@@ -246,17 +246,20 @@ template <typename T> struct Linear : Layer<T> {
         LinearCache *c = static_cast<LinearCache *>(cache);
         TensorT *sens = c->sensitivities.back();
         for (size_t i = weights.size(); i-- > 0;) {
-            if (activation) activation->getDerivative(pipeline, c->outputs[i], c->acti_derivatives[i]);
-            math::dot<T>(pipeline, sens, c->acti_derivatives[i]);
             TensorT *prev_output = i >= 1 ? c->outputs[i - 1] : input;
+            // activation derivative from the cached output, Hadamard product into the sensitivity and the
+            // bias gradient (column sums of the new sensitivity) in one pass over the layer's output
+            TensorT *dev = c->acti_derivatives[i];
+            helpers::eqlTensorsShape<T>(sens, dev);
+            helpers::eqlTensorsShape<T>(sens, c->outputs[i]);
+            check(wk_sensitivity_step(pipeline->command_queue->stream, core::getTypeIndex<T>(),
+                                      activation ? activation->kind : WK_ACT_NONE, sens->rows(), sens->cols(), c->outputs[i]->buffer,
+                                      c->outputs[i]->memory_layout.row_pitch, sens->buffer, sens->memory_layout.row_pitch, dev->buffer,
+                                      dev->memory_layout.row_pitch, bias_enabled ? c->bias_gradients[i]->buffer : nullptr));
+            pipeline->append(1);
             // weight gradient: sens^T [O,B] * prev_output [B,I]
             blas::gemm<T>(pipeline, std::nullopt, sens, blas::Operation::transpose, prev_output, blas::Operation::no_transpose,
                           std::nullopt, c->gradients[i], nullptr);
-            if (bias_enabled) {
-                check(wk_bias_step(pipeline->command_queue->stream, core::getTypeIndex<T>(), sens->rows(), sens->cols(),
-                                   sens->buffer, sens->memory_layout.row_pitch, c->bias_gradients[i]->buffer));
-                pipeline->append(1);
-            }
             TensorT *next = i >= 1 ? c->sensitivities[i - 1] : input_sensitivity;
             if (!next) return;
             // sensitivity of what feeds this matrix: sens [B,O] * W [O,I]
@@ -461,7 +464,8 @@ template <typename T> struct Adam : Optimizer<T> {
         o->eps = eps >= 0.0 ? eps : (double)std::numeric_limits<T>::epsilon(); // the siblings' +FLT_EPSILON (rmsprop.cl:54)
         return o;
     }
-    void update(Pipeline *pipeline, size_t &index, Tensor<T> *w, Tensor<T> *g) {
+    // one parameter tensor's entry of the step's update list (its moments are created on first sight)
+    void collect(Pipeline *pipeline, size_t &index, Tensor<T> *w, Tensor<T> *g, std::vector<wk_adam_tensor> &list) {
         if (index == state.size()) {
             Tensor<T> *m = Tensor<T>::alloc(w->context, pipeline, w->dimensions.shape);
             Tensor<T> *v = nullptr;
@@ -476,25 +480,31 @@ template <typename T> struct Adam : Optimizer<T> {
         Tensor<T> *m = state[index].first, *v = state[index].second;
         helpers::eqlTensorsShape<T>(w, g);
         helpers::eqlTensorsShape<T>(w, m);
-        const uint64_t shape3[3] = {w->depth(), w->rows(), w->cols()};
-        check(wk_adam_step(pipeline->command_queue->stream, core::getTypeIndex<T>(), shape3, w->buffer, w->memory_layout.row_pitch,
-                           w->memory_layout.slice_pitch, g->buffer, g->memory_layout.row_pitch, g->memory_layout.slice_pitch,
-                           m->buffer, v->buffer, m->memory_layout.row_pitch, m->memory_layout.slice_pitch, lr, beta1, beta2, eps, t));
-        pipeline->append(1);
+        wk_adam_tensor t{};
+        t.w = w->buffer; t.g = g->buffer; t.m = m->buffer; t.v = v->buffer;
+        t.shape3[0] = w->depth(); t.shape3[1] = w->rows(); t.shape3[2] = w->cols();
+        t.w_row_pitch = w->memory_layout.row_pitch; t.w_slice_pitch = w->memory_layout.slice_pitch;
+        t.g_row_pitch = g->memory_layout.row_pitch; t.g_slice_pitch = g->memory_layout.slice_pitch;
+        t.mv_row_pitch = m->memory_layout.row_pitch; t.mv_slice_pitch = m->memory_layout.slice_pitch;
+        list.push_back(t);
         ++index;
     }
     void step(Pipeline *pipeline, const Cache<T> *cache) override {
         ++t;
         size_t index = 0;
+        std::vector<wk_adam_tensor> list;
         for (const auto &slot : cache->slots) {
             auto w = slot.layer->getWeights();
             auto g = slot.layer->getGradients(slot.cache);
-            for (size_t i = 0; i < w.size(); ++i) update(pipeline, index, w[i], g[i]);
+            for (size_t i = 0; i < w.size(); ++i) collect(pipeline, index, w[i], g[i], list);
             auto b = slot.layer->getBias();
             auto bg = slot.layer->getBiasGradients(slot.cache);
             for (size_t i = 0; i < b.size(); ++i)
-                if (b[i] && bg[i]) update(pipeline, index, b[i], bg[i]);
+                if (b[i] && bg[i]) collect(pipeline, index, b[i], bg[i], list);
         }
+        check(wk_adam_step_multi(pipeline->command_queue->stream, core::getTypeIndex<T>(), (uint32_t)list.size(), list.data(), lr, beta1,
+                                 beta2, eps, t));
+        pipeline->append(1);
     }
     void zero(Pipeline *pipeline) override {
         for (auto &mv : state) {
