@@ -198,14 +198,18 @@ const char *wk_gemm_variant_with_workspace(int dtype, int op_a, int op_b, uint64
                                            const void *C, size_t workspace_bytes);
 
 /* Host arithmetic only, for tests and benchmarks: how a wk_gemm call on a stream lays out a product
- * whose k is split over work-groups (few tiles of C, long k: every tile goes to `shares` work-groups
- * that each sum `klen` values of k -- the last one what is left -- into partial tiles of
- * `scratch_bytes` bytes in the stream's own scratch memory; the last work-group to arrive at a tile
- * adds them in the order of the shares, so results are the same bits on every run).  variant NULL:
- * the automatic choice (shares = 1 when it does not split); a split variant's name ("mfma_f32_64x64z",
- * "mfma_f64_64x64z"): the plan that variant runs when forced.  No counterpart in the reference. */
+ * whose k is split over work-groups.  Two cases: few tiles of C and a long k (every tile is split:
+ * first_tile = 0), and a launch whose tiles do not fill whole rounds of the compute units (the whole
+ * rounds, tiles 0 .. first_tile - 1, run as they are; the `tiles` left-over ones follow as a second
+ * launch with k split).  A split tile goes to `shares` work-groups that each sum `klen` values of k
+ * -- the last one what is left -- into partial tiles of `scratch_bytes` bytes in the stream's own
+ * scratch memory; the last work-group to arrive at a tile adds them in the order of the shares, so
+ * results are the same bits on every run.  variant NULL: the automatic choice (shares = 1 when it
+ * does not split); a splitting variant's name ("mfma_f32_64x64z", "mfma_f64_64x64z",
+ * "mfma_f32_256x128t", "mfma_f32_128x128t"): the plan that variant runs when forced.  No counterpart
+ * in the reference. */
 int wk_gemm_split_plan(int dtype, int op_a, int op_b, uint64_t M, uint64_t N, uint64_t K, const char *variant,
-                       uint32_t *shares, uint32_t *klen, uint64_t *tiles, size_t *scratch_bytes);
+                       uint32_t *shares, uint32_t *klen, uint64_t *first_tile, uint64_t *tiles, size_t *scratch_bytes);
 
 /* Test and benchmark knob only, not for product code: force a gemm variant by name ("auto" restores
  * selection).  Process-wide, read by every wk_gemm call on every stream; changing it while a

@@ -42,7 +42,7 @@ def test_binding_covers_every_declared_symbol():
 def test_k_split_plans_fit_the_scratch_and_the_counters():
     """Host arithmetic of the GEMM that splits k over work-groups: whatever the shape, a plan that
     splits covers k exactly with whole slabs per share, and its partial tiles and arrival counters
-    fit what every stream owns (16 MiB, 4096 counters) -- the kernel takes both for granted."""
+    fit what every stream owns (64 MiB, 4096 counters) -- the kernel takes both for granted."""
     from wekua_amd import _capi
     lib = _capi.load()
     u32, u64, sz = ctypes.c_uint32, ctypes.c_uint64, ctypes.c_size_t
@@ -52,8 +52,8 @@ def test_k_split_plans_fit_the_scratch_and_the_counters():
             for (M, N, K) in [(512, 512, 8192), (512, 512, 512), (64, 64, 100000), (300, 200, 2500), (70, 45, 97), (1, 1, 1),
                               (1, 1, 64), (64, 64, 33), (2048, 2048, 8192), (8192, 256, 8192), (4096, 4096, 65), (1024, 64, 4096),
                               (100000, 64, 4096), (64, 262144, 4096), (768, 768, 3000), (5000, 3000, 128)]:
-                shares, klen, tiles, nbytes = u32(), u32(), u64(), sz()
-                assert lib.wk_gemm_split_plan(dtype, 0, 1, M, N, K, forced, shares, klen, tiles, nbytes) == 0
+                shares, klen, first, tiles, nbytes = u32(), u32(), u64(), u64(), sz()
+                assert lib.wk_gemm_split_plan(dtype, 0, 1, M, N, K, forced, shares, klen, first, tiles, nbytes) == 0
                 if shares.value == 1:
                     assert (klen.value, tiles.value, nbytes.value) == (0, 0, 0)
                     continue
@@ -61,15 +61,29 @@ def test_k_split_plans_fit_the_scratch_and_the_counters():
                 assert klen.value % 32 == 0 and klen.value > 0
                 assert klen.value * (shares.value - 1) < K <= klen.value * shares.value    # every share holds some of k
                 assert tiles.value == ((M + 63) // 64) * ((N + 63) // 64) <= 4096
-                assert nbytes.value == shares.value * tiles.value * 64 * 64 * es <= 16 << 20
+                assert nbytes.value == shares.value * tiles.value * 64 * 64 * es <= 64 << 20
+                assert first.value == 0                                                    # every tile is split
                 if forced is None:      # the automatic choice splits only few tiles with a long k
                     assert tiles.value <= 128 and tiles.value * shares.value <= (1024 if es == 4 else 512)
                     assert K >= (4096 if es == 4 else 2048) and klen.value >= 8 * 32
     assert seen_split >= 10
-    shares, klen, tiles, nbytes = u32(), u32(), u64(), sz()
-    assert lib.wk_gemm_split_plan(8, 0, 0, 512, 512, 8192, b"mfma_f64_64x64z", shares, klen, tiles, nbytes) == 1   # wrong dtype
-    assert lib.wk_gemm_split_plan(8, 0, 0, 512, 512, 8192, b"nope", shares, klen, tiles, nbytes) == 1
-    assert lib.wk_gemm_split_plan(8, 0, 0, 0, 512, 8192, None, shares, klen, tiles, nbytes) == 1
+    # left-over tiles as a tail: whole rounds (a round = the tiles resident at once: 256 units x 2 or 3
+    # work-groups) stay unsplit, the rest is split; the automatic plan needs a whole round in the body
+    for name, (bm, bn, occ) in ((b"mfma_f32_256x128t", (256, 128, 2)), (b"mfma_f32_128x128t", (128, 128, 3))):
+        for (M, N, K) in [(4097, 4095, 4093), (8191, 8193, 8190), (5000, 5000, 5000), (4096, 4096, 4096), (300, 200, 100),
+                          (7168, 7168, 7168), (3000, 3000, 64), (100000, 128, 4096)]:
+            shares, klen, first, tiles, nbytes = u32(), u32(), u64(), u64(), sz()
+            assert lib.wk_gemm_split_plan(8, 0, 0, M, N, K, name, shares, klen, first, tiles, nbytes) == 0
+            total = ((M + bm - 1) // bm) * ((N + bn - 1) // bn)
+            if shares.value == 1:
+                continue
+            assert first.value % (256 * occ) == 0 and first.value + tiles.value == total and 0 < tiles.value < 256 * occ
+            assert klen.value % 16 == 0 and klen.value * (shares.value - 1) < K <= klen.value * shares.value
+            assert nbytes.value == shares.value * tiles.value * bm * bn * 4 <= 64 << 20 and tiles.value <= 4096
+    shares, klen, first, tiles, nbytes = u32(), u32(), u64(), u64(), sz()
+    assert lib.wk_gemm_split_plan(8, 0, 0, 512, 512, 8192, b"mfma_f64_64x64z", shares, klen, first, tiles, nbytes) == 1   # wrong dtype
+    assert lib.wk_gemm_split_plan(8, 0, 0, 512, 512, 8192, b"nope", shares, klen, first, tiles, nbytes) == 1
+    assert lib.wk_gemm_split_plan(8, 0, 0, 0, 512, 8192, None, shares, klen, first, tiles, nbytes) == 1
 
 
 def _split_args(arglist):

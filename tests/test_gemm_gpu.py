@@ -77,7 +77,8 @@ def test_float_small_shapes(dev, dtype, op_a, op_b, alpha, beta):
 
 
 @pytest.mark.parametrize("variant", ["tile64", "mfma_f32_64x64", "mfma_f32_64x64s2", "mfma_f32_64x64s4", "mfma_f32_32x32s4",
-                                     "mfma_f32_64x64z", "mfma_f32_128x128", "mfma_f32_128x128s2", "mfma_f32_256x128"])
+                                     "mfma_f32_64x64z", "mfma_f32_128x128", "mfma_f32_128x128s2", "mfma_f32_256x128",
+                                     "mfma_f32_128x128t", "mfma_f32_256x128t"])
 @pytest.mark.parametrize("op_a,op_b", OPS)
 def test_f32_every_variant(dev, variant, op_a, op_b):
     import ctypes
@@ -261,7 +262,8 @@ def test_invalid_arguments(dev):
                                            ("f32", "mfma_f32_256x128"),
                                            ("f64", "mfma_f64_64x64"), ("f64", "mfma_f64_64x64s2"), ("f64", "mfma_f64_32x32s4"),
                                            ("f64", "mfma_f64_128x64"), ("f64", "mfma_f64_128x128"),
-                                           ("f32", "mfma_f32_64x64z"), ("f64", "mfma_f64_64x64z")])
+                                           ("f32", "mfma_f32_64x64z"), ("f64", "mfma_f64_64x64z"),
+                                           ("f32", "mfma_f32_128x128t"), ("f32", "mfma_f32_256x128t")])
 def test_every_k_around_the_slab_boundaries(dev, dtype, variant):
     """Every K from 1 to 100 on a ragged tile and on a tile-aligned shape: the bounds-checked kernels
     choose per-flavour loops from the number of complete slabs (k-slab 16 or 32, one or two slabs of
@@ -323,8 +325,8 @@ def test_k_split_over_work_groups(dev, dtype):
     assert lib.wk_gemm_variant(did, 0, 0, 512, 512, 8192, 8192, 512, 512, None, None, None) == z
     assert lib.wk_gemm_variant(did, 0, 0, 512, 512, 512, 512, 512, 512, None, None, None) != z      # k too short to split
     assert lib.wk_gemm_variant(did, 0, 0, 2048, 2048, 8192, 8192, 2048, 2048, None, None, None) != z  # enough tiles
-    shares, klen, tiles, nbytes = ctypes.c_uint32(), ctypes.c_uint32(), ctypes.c_uint64(), ctypes.c_size_t()
-    assert lib.wk_gemm_split_plan(did, 0, 0, 512, 512, 8192, None, shares, klen, tiles, nbytes) == 0
+    shares, klen, first, tiles, nbytes = ctypes.c_uint32(), ctypes.c_uint32(), ctypes.c_uint64(), ctypes.c_uint64(), ctypes.c_size_t()
+    assert lib.wk_gemm_split_plan(did, 0, 0, 512, 512, 8192, None, shares, klen, first, tiles, nbytes) == 0
     # 64 tiles on 256 compute units: shares until four (f32) / two (f64) work-groups sit on every unit
     assert (shares.value, klen.value, tiles.value) == ((16, 512, 64) if dtype == "f32" else (8, 1024, 64))
     for op_a, op_b in OPS:
@@ -357,6 +359,47 @@ def test_k_split_over_work_groups(dev, dtype):
         dA.free(); dB.free()
     finally:
         lib.wk_gemm_force_variant(b"auto")
+
+
+def test_left_over_tiles_run_as_a_k_split_tail(dev):
+    """A launch whose tiles do not fill whole rounds of the compute units: the whole rounds run as they
+    are, the left-over tiles as a second launch with k split over work-groups.  Checked: the plan of the
+    automatic choice for the ragged benchmark shape, results against the oracle for body + tail (forced
+    on shapes of a few hundred tiles, all layouts, aligned and ragged), and the same bits on every run."""
+    import ctypes
+    from helpers import make_operand
+    from wekua_amd import raw
+    lib = dev.lib
+    did = raw.dtype_id("f32")
+    shares, klen, first, tiles, nbytes = ctypes.c_uint32(), ctypes.c_uint32(), ctypes.c_uint64(), ctypes.c_uint64(), ctypes.c_size_t()
+    # 4097 x 4095 in tiles of 256 x 128: 17 x 32 = 544 = two rounds of 256 and 32 left over
+    assert lib.wk_gemm_split_plan(did, 0, 0, 4097, 4095, 4093, b"mfma_f32_256x128t", shares, klen, first, tiles, nbytes) == 0
+    assert (first.value, tiles.value) == (512, 32) and shares.value >= 2 and klen.value % 16 == 0
+    assert nbytes.value == shares.value * 32 * 256 * 128 * 4 <= 64 << 20
+    # a product of whole rounds has no tail; the variant then runs the plain tile
+    assert lib.wk_gemm_split_plan(did, 0, 0, 4096, 4096, 4096, b"mfma_f32_256x128t", shares, klen, first, tiles, nbytes) == 0
+    assert shares.value == 1
+    for variant, (M, N) in ((b"mfma_f32_128x128t", (2100, 2000)), (b"mfma_f32_256x128t", (4097, 2047))):
+        assert lib.wk_gemm_force_variant(variant) == 0
+        try:
+            for op_a, op_b in OPS:
+                check(dev, "f32", M, N, 160, op_a, op_b, 1.5, 0.5, seed=83)         # 272 tiles: one round + 16
+                check(dev, "f32", M, N - 5, 67, op_a, op_b, None, None, seed=84)    # k tail inside the last share
+            check(dev, "f32", 300, 200, 100, 0, 1, 2.0, None, seed=85)              # less than a round: all tail
+            a = make_operand("f32", (2100, 192), 86)
+            b = make_operand("f32", (192, 2000), 87)
+            dA, dB = dev.upload(a), dev.upload(b)
+            outs = []
+            for _ in range(3):
+                dC = dev.upload(np.zeros((2100, 2000), dtype=np.float32))
+                dev.gemm("f32", 0, 0, 2100, 2000, 192, None, dA, 192, dB, 2000, None, dC, 2000)
+                dev.sync()
+                outs.append(dC.download(np.float32, (2100, 2000)))
+                dC.free()
+            assert np.array_equal(outs[1], outs[0]) and np.array_equal(outs[2], outs[0])
+            dA.free(); dB.free()
+        finally:
+            lib.wk_gemm_force_variant(b"auto")
 
 
 @pytest.mark.parametrize("variant", ["mfma_i32_64x128", "mfma_i32_128x128", "mfma_i32_packed"])

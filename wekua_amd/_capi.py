@@ -76,7 +76,8 @@ SIGNATURES = {
     "wk_gemm_variant_with_workspace": (ctypes.c_char_p, [ci, ci, ci, u64, u64, u64, u64, u64, u64, vp, vp, vp, sz]),
     "wk_gemm_force_variant": (ci, [ctypes.c_char_p]),
     "wk_gemm_split_plan": (ci, [ci, ci, ci, u64, u64, u64, ctypes.c_char_p, ctypes.POINTER(ctypes.c_uint32),
-                                ctypes.POINTER(ctypes.c_uint32), ctypes.POINTER(u64), ctypes.POINTER(ctypes.c_size_t)]),
+                                ctypes.POINTER(ctypes.c_uint32), ctypes.POINTER(u64), ctypes.POINTER(u64),
+                                ctypes.POINTER(ctypes.c_size_t)]),
     "wk_copy_kernel": (ci, [vp, vp, vp, sz]),
     "wk_hadamard": (ci, [vp, ci, u64p, vp, u64, u64, vp, u64, u64]),
     "wk_activation": (ci, [vp, ci, ci, u64p, vp, u64, u64]),

@@ -239,10 +239,11 @@ const char *wk_gemm_variant_with_workspace(int dtype, int op_a, int op_b, uint64
 }
 
 int wk_gemm_split_plan(int dtype, int op_a, int op_b, uint64_t M, uint64_t N, uint64_t K, const char *variant, uint32_t *shares,
-                       uint32_t *klen, uint64_t *tiles, size_t *scratch_bytes) {
-    if (!shares || !klen || !tiles || !scratch_bytes) return WK_E_INVALID_VALUE;
+                       uint32_t *klen, uint64_t *first_tile, uint64_t *tiles, size_t *scratch_bytes) {
+    if (!shares || !klen || !first_tile || !tiles || !scratch_bytes) return WK_E_INVALID_VALUE;
     *shares = 1;
     *klen = 0;
+    *first_tile = 0;
     *tiles = 0;
     *scratch_bytes = 0;
     GemmProblem p;
@@ -267,6 +268,7 @@ int wk_gemm_split_plan(int dtype, int op_a, int op_b, uint64_t M, uint64_t N, ui
     if (v >= 0 && gemm_mfma_split_plan(p, v, variant != nullptr, plan)) {
         *shares = plan.shares;
         *klen = plan.klen;
+        *first_tile = plan.first_tile;
         *tiles = plan.tiles;
         *scratch_bytes = plan.bytes;
     }

@@ -66,6 +66,9 @@ template <typename T> struct MArgs {
     uint32_t klen;
     T *partials;
     uint32_t *counters;
+    // first tile number of this launch (a product may be launched as a body of whole rounds of tiles
+    // and a tail whose k is split; the tail's tile numbers follow the body's)
+    uint32_t pid_offset;
 };
 
 // Work-groups that share a CU start in lock step (the whole first wave of work-groups is
@@ -94,9 +97,11 @@ __device__ __forceinline__ void startup_stagger(uint32_t num_cus, uint32_t occup
 // compact 4 x 8 block of tiles per XCD inside each round of 8 x 32 tiles, which on paper halves the
 // L2 misses, runs at the same speed and misses 18 % MORE: the work-groups of an XCD are not close
 // enough in k for the 4 MB L2 to hold what they would share.)
-__device__ __forceinline__ void tile_coords(uint32_t tiles_m, uint32_t tiles_n, uint32_t &tm, uint32_t &tn, uint32_t remap = 0) {
+__device__ __forceinline__ void tile_coords(uint32_t tiles_m, uint32_t tiles_n, uint32_t &tm, uint32_t &tn, uint32_t remap = 0,
+                                            uint32_t pid_offset = 0) {
     uint32_t pid = blockIdx.x;
     if (remap && (gridDim.x % 8) == 0) pid = (pid % 8) * (gridDim.x / 8) + pid / 8;
+    pid += pid_offset;
     const uint32_t group_size = GROUP_M * tiles_n;
     const uint32_t group = pid / group_size;
     const uint32_t first_m = group * GROUP_M;
@@ -143,7 +148,7 @@ void gemm_f32_mfma_kernel(MArgs<float> g) {
     const int l32 = lane & 31, lhi = lane >> 5;
 
     uint32_t tile_m, tile_n;
-    tile_coords(g.tiles_m, g.tiles_n, tile_m, tile_n, g.xcd_remap);
+    tile_coords(g.tiles_m, g.tiles_n, tile_m, tile_n, g.xcd_remap, g.pid_offset);
     const uint32_t m0 = tile_m * BM, n0 = tile_n * BN;
     if constexpr (SPLIT) { // this work-group's share of k; from here on the kernel sees a shorter product
         const uint32_t k_begin = blockIdx.y * g.klen;
@@ -168,7 +173,7 @@ void gemm_f32_mfma_kernel(MArgs<float> g) {
     // Staging registers, global -> LDS: one set.  (LOOP 2 on the small tile keeps two and requests
     // slab kt+2 while slab kt is computed: with one or two 64x64 tiles on a CU a slab's matrix work is
     // shorter than the latency of a global load.  LOOP 3 gets the same lead from one set.)
-    constexpr int LOOP_WANTED = LSEL >= 0 ? LSEL : (BM * BN <= 128 * 128) ? 3 : B_K ? 3 : (A_K ? 0 : 5);
+    constexpr int LOOP_WANTED = LSEL >= 0 ? LSEL : (BM * BN <= 128 * 128) ? 3 : A_K ? 4 : B_K ? 3 : 5;
     constexpr int LOOP = (EDGE && LOOP_WANTED < 2) ? 2 : LOOP_WANTED;
     constexpr int PF = (BM * BN <= 64 * 64 && LOOP == 2) ? 2 : 1;
     f32x4 ra[PF][A_V4], rb[PF][B_V4];
@@ -380,18 +385,20 @@ void gemm_f32_mfma_kernel(MArgs<float> g) {
     // interleave on a CU depends on the instruction order the compiler derives from the spelling,
     // and the rate moves by up to 10 % with it; each tile (for 256x128: each operand layout) uses the one that measured fastest on
     // MI355X (same box, same process, f32, alpha and beta given):
-    //   LOOP 0  `if (more)` around the hand-over, written out      256x128: NN 142.0, NT 133.4, TN 129.4
-    //   LOOP 1  the same inside a lambda                            256x128: NN 129.3, NT 131.6, TN 128.6;
-    //                                                               128x128 at 2048x4096x4096: 136.4 (LOOP 0: 127.3, LOOP 2: 125.3)
-    //   LOOP 2  last slab peeled, hand-over fenced                  256x128: NN 133.4, NT 134.3, TN 131.1;
-    //           (sched_barrier) so that matrix instructions         64x64 at 1024^3: 90.8 (LOOP 1: 88.7), 2048^3: 122.8 (115-120)
+    //   LOOP 0  `if (more)` around the hand-over, written out      256x128: NN 132.6, NT 132.0, TN 132.3, TT 131.3
+    //   LOOP 1  the same inside a lambda                            256x128: NN 128.3, NT 134.1, TN 131.2, TT 128.3
+    //   LOOP 2  last slab peeled, hand-over fenced                  256x128: NN 134.2, NT 135.0, TN 132.7, TT 132.6
+    //           (sched_barrier) so that matrix instructions
     //           are not hoisted above the barrier
-    //   LOOP 3  LOOP 2 with an early store: slab kt+1, requested    256x128: NT 143.3, TT 141.2, NN 132.7, TN 127.2;
-    //           a whole iteration ago, goes to the free LDS        128x128: faster than LOOP 1 on every layout and shape tried
-    //           buffer at the top of iteration kt and slab kt+2     (4096^3 NT 109 -> 141, 2048x4096x4096 NN 126 -> 133);
-    //           is requested into the same registers               64x64: +1..3 % over LOOP 2 with two staging sets
-    //   LOOP 4 / 5  LOOP 3 for A only / for B only, the other     256x128 TN: LOOP 5 136.1 (LOOP 2: 133.3, LOOP 4: 132.7);
-    //           operand stored late as in LOOP 2                    NN: 140.2 / 135.9, TT: 136.2 / 138.6 -- behind their own
+    //   LOOP 3  LOOP 2 with an early store: slab kt+1, requested    256x128: NN 133.6, NT 142.0, TN 129.2, TT 142.2;
+    //           a whole iteration ago, goes to the free LDS        the loop of the 128x128 and 64x64 tiles
+    //           buffer at the top of iteration kt and slab kt+2
+    //           is requested into the same registers
+    //   LOOP 4 / 5  LOOP 3 for A only / for B only, the other     256x128: LOOP 4 NN 139.2, NT 144.0, TN 132.1, TT 135.5;
+    //           operand stored late as in LOOP 2                    LOOP 5 NN 135.5, NT 142.4, TN 136.1, TT 138.0
+    // (8192^3, alpha and beta given, TFLOP/s, one process on one box.  The ranking is not stable under
+    // changes elsewhere in the kernel: before the kernel arguments grew by the split-k fields LOOP 0 gave
+    // N,N 142.0 and LOOP 4 140.2.  bench.py holds a floor under the headline rate for that reason.)
     // (the bounds-checked instantiation takes LOOP 2 and up, whose iterations exist per flavour)
     f32x4 af[2][FM], bf[2][FN];
     read_frags(0, 0, af[0], bf[0]);
@@ -581,7 +588,6 @@ void gemm_f32_mfma_kernel(MArgs<float> g) {
         // which on this part write back and invalidate a whole L2 per work-group (measured: with
         // fences the split launch was no faster than the unsplit one).
         __shared__ uint32_t s_last;
-        constexpr int Q = FM * FN * 16;
         constexpr size_t TILE = (size_t)BM * BN;
         float *mine = g.partials + ((size_t)blockIdx.y * gridDim.x + blockIdx.x) * TILE + tid;
 #pragma unroll
@@ -610,15 +616,17 @@ void gemm_f32_mfma_kernel(MArgs<float> g) {
                 for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
         for (uint32_t z = 0; z < gridDim.y; ++z) {
             const float *part = g.partials + ((size_t)z * gridDim.x + blockIdx.x) * TILE + tid;
-            float v[Q];
-#pragma unroll
-            for (int q = 0; q < Q; ++q) v[q] = __hip_atomic_load(part + (size_t)q * NT, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 #pragma unroll
             for (int i = 0; i < FM; ++i)
 #pragma unroll
-                for (int j = 0; j < FN; ++j)
+                for (int j = 0; j < FN; ++j) {
+                    float v[16]; // one 32x32 block's worth of loads in flight
 #pragma unroll
-                    for (int r = 0; r < 16; ++r) acc[i][j][r] += v[(i * FN + j) * 16 + r];
+                    for (int r = 0; r < 16; ++r)
+                        v[r] = __hip_atomic_load(part + (size_t)((i * FN + j) * 16 + r) * NT, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) acc[i][j][r] += v[r];
+                }
         }
     }
 
@@ -696,7 +704,7 @@ void gemm_f64_mfma_kernel(MArgs<double> g) {
     const int l16 = lane & 15, lq = lane >> 4; // lq = 0..3
 
     uint32_t tile_m, tile_n;
-    tile_coords(g.tiles_m, g.tiles_n, tile_m, tile_n, g.xcd_remap);
+    tile_coords(g.tiles_m, g.tiles_n, tile_m, tile_n, g.xcd_remap, g.pid_offset);
     const uint32_t m0 = tile_m * BM, n0 = tile_n * BN;
     if constexpr (SPLIT) { // this work-group's share of k, as in the f32 kernel
         const uint32_t k_begin = blockIdx.y * g.klen;
@@ -1125,14 +1133,17 @@ template <typename K> int set_lds(K kernel, size_t bytes) {
 template <typename T> int apply_split(MArgs<T> &g, const GemmProblem &p, const GemmSplitPlan &plan, int bm, int bn) {
     if (plan.shares < 2 || plan.klen == 0) return WK_E_INVALID_VALUE;
     if (!p.scratch || !p.counters) return WK_E_INVALID_VALUE;
-    if (plan.tiles != (uint64_t)g.tiles_m * g.tiles_n || plan.tiles > p.num_counters) return WK_E_INVALID_VALUE;
+    // the launch covers tiles first_tile .. first_tile + tiles - 1 of C
+    if (plan.tiles == 0 || plan.first_tile + plan.tiles != (uint64_t)g.tiles_m * g.tiles_n || plan.tiles > p.num_counters)
+        return WK_E_INVALID_VALUE;
     if ((uint64_t)plan.shares * plan.tiles * bm * bn * sizeof(T) > p.scratch_bytes) return WK_E_INVALID_VALUE;
     if ((uint64_t)plan.klen * (plan.shares - 1) >= p.K || (uint64_t)plan.klen * plan.shares < p.K) return WK_E_INVALID_VALUE;
     if (plan.shares > 65535) return WK_E_INVALID_VALUE;
     g.klen = plan.klen;
     g.partials = static_cast<T *>(p.scratch);
     g.counters = p.counters;
-    g.xcd_remap = 0; // blockIdx.x is the tile's number, its counter's index and its place among the partial tiles
+    g.pid_offset = (uint32_t)plan.first_tile;
+    g.xcd_remap = 0; // blockIdx.x is the tile's counter index and its place among the partial tiles
     return WK_OK;
 }
 
@@ -1151,7 +1162,14 @@ int launch_f32_one(hipStream_t st, const GemmProblem &p, const GemmSplitPlan *pl
         if (rc) return rc;
         shares = plan->shares;
     }
-    hipLaunchKernelGGL(kern, dim3(g.tiles_m * g.tiles_n, shares), dim3(WMS * WNS * 64 * KS), lds, st, g);
+    uint32_t grid_x = g.tiles_m * g.tiles_n;
+    if constexpr (SPLIT) grid_x = (uint32_t)plan->tiles;
+    else if (plan) { // the body of a product whose tail is launched separately: the first tiles only
+        if (plan->first_tile == 0 || plan->first_tile >= grid_x) return WK_E_INVALID_VALUE;
+        grid_x = (uint32_t)plan->first_tile;
+        g.xcd_remap = 0;
+    }
+    hipLaunchKernelGGL(kern, dim3(grid_x, shares), dim3(WMS * WNS * 64 * KS), lds, st, g);
     return launch_status();
 }
 
@@ -1191,7 +1209,14 @@ int launch_f64_one(hipStream_t st, const GemmProblem &p, const GemmSplitPlan *pl
         if (rc) return rc;
         shares = plan->shares;
     }
-    hipLaunchKernelGGL(kern, dim3(g.tiles_m * g.tiles_n, shares), dim3(WMS * WNS * 64 * KS), lds, st, g);
+    uint32_t grid_x = g.tiles_m * g.tiles_n;
+    if constexpr (SPLIT) grid_x = (uint32_t)plan->tiles;
+    else if (plan) {
+        if (plan->first_tile == 0 || plan->first_tile >= grid_x) return WK_E_INVALID_VALUE;
+        grid_x = (uint32_t)plan->first_tile;
+        g.xcd_remap = 0;
+    }
+    hipLaunchKernelGGL(kern, dim3(grid_x, shares), dim3(WMS * WNS * 64 * KS), lds, st, g);
     return launch_status();
 }
 
@@ -1286,6 +1311,82 @@ int launch_f64_split64(hipStream_t st, const GemmProblem &p, bool edge) {
 #undef WK_CASE
 }
 
+// forced tail variants plan relaxed (tests reach the tail path on small shapes); WK_TAIL_STRICT=1 in the
+// environment makes them plan like the automatic choice (benchmarks of the choice itself)
+const bool g_tail_relaxed = [] {
+    const char *v = std::getenv("WK_TAIL_STRICT");
+    return !(v && v[0] == '1');
+}();
+
+// ---- a tail of tiles with k split --------------------------------------------------------------
+// A launch whose tiles do not fill whole rounds ends with a few compute units finishing the
+// left-over tiles while the rest idle (4097 x 4095 is 544 tiles of 256 x 128 on 256 units: two
+// rounds and 32 tiles more, which take as long as a third round).  These variants launch the whole
+// rounds as they are and the left-over tiles as a second launch with k split over work-groups, so
+// that the tail occupies every unit for a fraction of a tile's time.
+//   relaxed (forced variant, tests): every left-over tile is a tail tile, up to four shares; a product
+//   of less than one round is all tail.
+//   otherwise: at least one whole round in the body, a tail of at most half a round, as many shares
+//   as fill the units once (a power of two, at most 64), each at least eight slabs long.
+bool plan_tail(const GemmProblem &p, int bm, int bn, int bkt, size_t elem, int occ, bool relaxed, GemmSplitPlan &plan) {
+    plan = GemmSplitPlan{};
+    const uint64_t tiles = ((p.M + bm - 1) / bm) * ((p.N + bn - 1) / bn);
+    // a round = as many tiles as are resident at once: `occ` work-groups on every compute unit
+    const uint64_t round = (p.num_cus ? p.num_cus : 256) * (uint64_t)(occ > 0 ? occ : 1);
+    const uint64_t rem = tiles % round, body = tiles - rem;
+    const uint64_t slabs = (p.K + bkt - 1) / bkt;
+    if (rem == 0) return false;
+    uint64_t shares = 1;
+    if (relaxed) {
+        shares = slabs >= 4 ? 4 : slabs;
+    } else {
+        if (body == 0) return false;
+        while (shares < 64 && rem * shares * 2 <= round && slabs / (shares * 2) >= 8) shares *= 2;
+    }
+    if (shares < 2) return false;
+    const uint64_t klen = (slabs + shares - 1) / shares * bkt;
+    shares = (p.K + klen - 1) / klen;
+    if (shares < 2) return false;
+    plan.shares = (uint32_t)shares;
+    plan.klen = (uint32_t)klen;
+    plan.tiles = rem;
+    plan.first_tile = body;
+    plan.bytes = (size_t)(shares * rem * bm * bn * elem);
+    return p.scratch && p.counters && plan.bytes <= p.scratch_bytes && plan.tiles <= p.num_counters;
+}
+
+template <int BM, int BN, int BK, int WMS, int WNS, int OCC>
+int launch_f32_tail(hipStream_t st, const GemmProblem &p, bool edge) {
+    GemmSplitPlan plan;
+    if (p.ext || !plan_tail(p, BM, BN, BK, sizeof(float), OCC, g_tail_relaxed, plan)) return launch_f32<BM, BN, BK, WMS, WNS, OCC>(st, p, edge);
+    const int sel = (p.op_a ? 0 : 2) | (p.op_b ? 1 : 0);
+    int rc = WK_OK;
+    if (plan.first_tile > 0) { // the whole rounds, as the plain variant would run them
+#define WK_CASE(AK, BKC)                                                                                                \
+    rc = edge ? launch_f32_one<BM, BN, BK, WMS, WNS, OCC, AK, BKC, true>(st, p, &plan)                                   \
+              : launch_f32_one<BM, BN, BK, WMS, WNS, OCC, AK, BKC, false>(st, p, &plan);                                 \
+    break
+        switch (sel) {
+        case 0: WK_CASE(false, false);
+        case 1: WK_CASE(false, true);
+        case 2: WK_CASE(true, false);
+        default: WK_CASE(true, true);
+        }
+#undef WK_CASE
+        if (rc) return rc;
+    }
+#define WK_CASE(AK, BKC)                                                                                                \
+    return edge ? launch_f32_one<BM, BN, BK, WMS, WNS, OCC, AK, BKC, true, false, 1, -1, true>(st, p, &plan)              \
+                : launch_f32_one<BM, BN, BK, WMS, WNS, OCC, AK, BKC, false, false, 1, -1, true>(st, p, &plan)
+    switch (sel) {
+    case 0: WK_CASE(false, false);
+    case 1: WK_CASE(false, true);
+    case 2: WK_CASE(true, false);
+    default: WK_CASE(true, true);
+    }
+#undef WK_CASE
+}
+
 struct VariantDesc {
     const char *name;
     int dtype, bm, bn, bk; // bk: k values per LDS slab
@@ -1300,13 +1401,27 @@ struct VariantDesc {
     const char *sparse = nullptr;
     // and the same tile with k split over work-groups, for few tiles and a long k (plan_split)
     const char *split = nullptr;
+    // and the same tile with its left-over tiles launched as a tail with k split (plan_tail)
+    const char *tail = nullptr;
+    int occ = 0; // work-groups of this tile that share a compute unit (0: not needed)
 };
+enum { SPLIT_NONE = 0, SPLIT_ALL = 1, SPLIT_TAIL = 2 };
+int split_kind_of(const char *name) { // by the name's suffix: ...z splits every tile's k, ...t the tail's
+    const size_t n = std::strlen(name);
+    return n && name[n - 1] == 'z' ? SPLIT_ALL : n && name[n - 1] == 't' ? SPLIT_TAIL : SPLIT_NONE;
+}
 
 const VariantDesc k_variants[] = {
-    {"mfma_f32_256x128", WK_F32, 256, 128, 16, 0.943, 0.25, &launch_f32<256, 128, 16, 2, 2, 2>},
-    {"mfma_f32_128x128", WK_F32, 128, 128, 16, 0.885, 0.25, &launch_f32<128, 128, 16, 2, 2, 3>},
+    {"mfma_f32_256x128", WK_F32, 256, 128, 16, 0.940, 0.19, &launch_f32<256, 128, 16, 2, 2, 2>, nullptr, nullptr, nullptr, nullptr,
+     "mfma_f32_256x128t", 2},
+    {"mfma_f32_256x128t", WK_F32, 256, 128, 16, 0.0, 0.25, &launch_f32_tail<256, 128, 16, 2, 2, 2>, nullptr, nullptr, nullptr, nullptr,
+     nullptr, 2}, // whole rounds + a k-split tail
+    {"mfma_f32_128x128", WK_F32, 128, 128, 16, 0.897, 0.19, &launch_f32<128, 128, 16, 2, 2, 3>, nullptr, nullptr, nullptr, nullptr,
+     "mfma_f32_128x128t", 3},
+    {"mfma_f32_128x128t", WK_F32, 128, 128, 16, 0.0, 0.25, &launch_f32_tail<128, 128, 16, 2, 2, 3>, nullptr, nullptr, nullptr, nullptr,
+     nullptr, 3},
     {"mfma_f32_128x128s2", WK_F32, 128, 128, 32, 0.0, 0.25, &launch_f32<128, 128, 16, 2, 2, 2, 2>}, // 2 groups x 16 k, see pick
-    {"mfma_f32_64x64", WK_F32, 64, 64, 32, 0.780, 0.10, &launch_f32<64, 64, 32, 2, 2, 4>, "mfma_f32_64x64s4", "mfma_f32_64x64s2",
+    {"mfma_f32_64x64", WK_F32, 64, 64, 32, 0.813, 0.13, &launch_f32<64, 64, 32, 2, 2, 4>, "mfma_f32_64x64s4", "mfma_f32_64x64s2",
      "mfma_f32_32x32s4", "mfma_f32_64x64z"},
     {"mfma_f32_64x64z", WK_F32, 64, 64, 32, 0.0, 0.10, &launch_f32_split64}, // k split over work-groups
     {"mfma_f32_64x64s2", WK_F32, 64, 64, 32, 0.0, 0.10, &launch_f32<64, 64, 16, 2, 2, 4, 2>}, // 2 groups x 16 k
@@ -1380,8 +1495,12 @@ bool wk::gemm_mfma_split_plan(const GemmProblem &p, int variant, bool forced, Ge
     plan = GemmSplitPlan{};
     if (variant < 0 || variant >= k_num_variants || p.ext) return false;
     const VariantDesc &v = k_variants[variant];
-    if (v.launch != &launch_f32_split64 && v.launch != &launch_f64_split64) return false;
-    return plan_split(p, v.bm, v.bn, v.bk, v.dtype == WK_F64 ? 8 : 4, forced, plan);
+    const size_t elem = v.dtype == WK_F64 ? 8 : 4;
+    switch (split_kind_of(v.name)) {
+    case SPLIT_ALL: return plan_split(p, v.bm, v.bn, v.bk, elem, forced, plan);
+    case SPLIT_TAIL: return plan_tail(p, v.bm, v.bn, v.bk, elem, v.occ, forced && g_tail_relaxed, plan);
+    default: return false;
+    }
 }
 
 namespace {
@@ -1393,6 +1512,12 @@ namespace {
 bool split_pays(const GemmProblem &p, const GemmSplitPlan &plan) {
     return plan.shares >= 2 && p.K >= (p.dtype == WK_F64 ? 2048u : 4096u);
 }
+} // namespace
+
+namespace {
+// cost of a k-split tail in rounds of its tile: launch gap, hand-overs without a co-resident
+// work-group and the addition of the partial tiles (fixed part), plus the tile's time over the shares
+constexpr double TAIL_FIXED = 0.06, TAIL_PER_SHARE = 1.52;
 } // namespace
 
 int wk::gemm_mfma_pick(const GemmProblem &p) {
@@ -1407,11 +1532,31 @@ int wk::gemm_mfma_pick(const GemmProblem &p) {
         const VariantDesc &d = k_variants[v];
         if (d.dtype != p.dtype || d.efficiency <= 0.0) continue;
         const double tiles = (double)((p.M + d.bm - 1) / d.bm) * (double)((p.N + d.bn - 1) / d.bn);
-        const double rounds = (double)(uint64_t)((tiles + cus - 1.0) / cus);
-        const double cost = (rounds + d.fill) * d.bm * d.bn / d.efficiency;
+        // Whole rounds: the big tiles (two or three work-groups per unit) pay for a started round in
+        // full, the small tile (four per unit, short) for about two thirds of it.
+        const double whole = (double)(uint64_t)((tiles + cus - 1.0) / cus);
+        const double rounds = tiles / cus + (d.bm <= 64 ? 0.65 : 1.0) * (whole - tiles / cus);
+        // the bounds-checked instantiation runs slower than the interior one (8191 x 8193 x 8190 against
+        // 8192^3 on the 256 x 128 tile: 126 against 142 TFLOP/s with the tail split off)
+        const double eff = d.efficiency * (needs_edge(p, d) ? (d.bm >= 256 ? 0.86 : d.bm >= 128 ? 0.944 : 0.93) : 1.0);
+        const double cost = (rounds + d.fill) * d.bm * d.bn / eff;
         if (best < 0 || cost < best_cost) {
             best = v;
             best_cost = cost;
+        }
+        // the same tile with its left-over tiles as a k-split tail: the whole rounds, then a second
+        // launch that keeps every unit busy for a fraction of a tile's time (tail_rounds fitted to
+        // measured launches)
+        GemmSplitPlan tp;
+        if (d.tail && !p.ext && plan_tail(p, d.bm, d.bn, d.bk, 4, d.occ, false, tp)) {
+            const double tail_rounds = TAIL_FIXED + TAIL_PER_SHARE / tp.shares;
+            const double tcost = ((double)tp.first_tile / cus + d.fill + tail_rounds * tp.tiles * tp.shares / cus) * d.bm * d.bn / eff;
+            if (tcost < best_cost)
+                for (int w = 0; w < k_num_variants; ++w)
+                    if (!std::strcmp(k_variants[w].name, d.tail)) {
+                        best = w;
+                        best_cost = tcost;
+                    }
         }
     }
     // f32 problems that are one nearly full round of 128x128 tiles: that tile with two k-groups (eight

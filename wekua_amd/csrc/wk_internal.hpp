@@ -25,7 +25,7 @@ struct wk_stream {
     uint32_t *gemm_counters;
 };
 
-constexpr size_t WK_STREAM_SCRATCH_BYTES = 16u << 20;
+constexpr size_t WK_STREAM_SCRATCH_BYTES = 64u << 20;
 constexpr size_t WK_GEMM_COUNTERS = 4096;
 // what wk_bias_step uses of the scratch: the number of row bands, and with it the order of the
 // additions, follows from this size, so it stays what it was when the scratch was this small
@@ -189,7 +189,8 @@ struct GemmProblem {
 struct GemmSplitPlan {
     uint32_t shares = 1;   // work-groups per tile of C (grid y); 1: no split
     uint32_t klen = 0;     // k values per share, a multiple of the kernel's k-slab; the last share takes what is left
-    uint64_t tiles = 0;    // tiles of C (grid x) = arrival counters used
+    uint64_t tiles = 0;    // tiles of C whose k is split (grid x) = arrival counters used
+    uint64_t first_tile = 0; // their first tile number: the tiles before it are launched unsplit (0: every tile is split)
     size_t bytes = 0;      // partial tiles: shares * tiles * tile area * element size
 };
 // Plan for `variant` (a split-k variant) on p.  forced: split whenever k holds two slabs, whatever the
