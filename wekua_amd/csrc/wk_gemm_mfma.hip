@@ -148,7 +148,7 @@ void gemm_f32_mfma_kernel(MArgs<float> g) {
     const int l32 = lane & 31, lhi = lane >> 5;
 
     uint32_t tile_m, tile_n;
-    tile_coords(g.tiles_m, g.tiles_n, tile_m, tile_n, g.xcd_remap, g.pid_offset);
+    tile_coords(g.tiles_m, g.tiles_n, tile_m, tile_n, g.xcd_remap, SPLIT ? g.pid_offset : 0u); // only a split tail starts past tile 0
     const uint32_t m0 = tile_m * BM, n0 = tile_n * BN;
     if constexpr (SPLIT) { // this work-group's share of k; from here on the kernel sees a shorter product
         const uint32_t k_begin = blockIdx.y * g.klen;
@@ -173,7 +173,7 @@ void gemm_f32_mfma_kernel(MArgs<float> g) {
     // Staging registers, global -> LDS: one set.  (LOOP 2 on the small tile keeps two and requests
     // slab kt+2 while slab kt is computed: with one or two 64x64 tiles on a CU a slab's matrix work is
     // shorter than the latency of a global load.  LOOP 3 gets the same lead from one set.)
-    constexpr int LOOP_WANTED = LSEL >= 0 ? LSEL : (BM * BN <= 128 * 128) ? 3 : A_K ? 4 : B_K ? 3 : 5;
+    constexpr int LOOP_WANTED = LSEL >= 0 ? LSEL : (BM * BN <= 128 * 128) ? 3 : B_K ? 3 : (A_K ? 0 : 5);
     constexpr int LOOP = (EDGE && LOOP_WANTED < 2) ? 2 : LOOP_WANTED;
     constexpr int PF = (BM * BN <= 64 * 64 && LOOP == 2) ? 2 : 1;
     f32x4 ra[PF][A_V4], rb[PF][B_V4];
@@ -385,20 +385,22 @@ void gemm_f32_mfma_kernel(MArgs<float> g) {
     // interleave on a CU depends on the instruction order the compiler derives from the spelling,
     // and the rate moves by up to 10 % with it; each tile (for 256x128: each operand layout) uses the one that measured fastest on
     // MI355X (same box, same process, f32, alpha and beta given):
-    //   LOOP 0  `if (more)` around the hand-over, written out      256x128: NN 132.6, NT 132.0, TN 132.3, TT 131.3
-    //   LOOP 1  the same inside a lambda                            256x128: NN 128.3, NT 134.1, TN 131.2, TT 128.3
-    //   LOOP 2  last slab peeled, hand-over fenced                  256x128: NN 134.2, NT 135.0, TN 132.7, TT 132.6
+    //   LOOP 0  `if (more)` around the hand-over, written out      256x128: NN 143.0, NT 133.7, TN 130.6, TT 131.7
+    //   LOOP 1  the same inside a lambda                            256x128: NN 129.3, NT 131.6, TN 128.6
+    //   LOOP 2  last slab peeled, hand-over fenced                  256x128: NN 134.7, NT 135.2, TN 133.3, TT 133.0
     //           (sched_barrier) so that matrix instructions
     //           are not hoisted above the barrier
-    //   LOOP 3  LOOP 2 with an early store: slab kt+1, requested    256x128: NN 133.6, NT 142.0, TN 129.2, TT 142.2;
+    //   LOOP 3  LOOP 2 with an early store: slab kt+1, requested    256x128: NN 133.6, NT 144.0, TN 128.6, TT 142.3;
     //           a whole iteration ago, goes to the free LDS        the loop of the 128x128 and 64x64 tiles
     //           buffer at the top of iteration kt and slab kt+2
     //           is requested into the same registers
-    //   LOOP 4 / 5  LOOP 3 for A only / for B only, the other     256x128: LOOP 4 NN 139.2, NT 144.0, TN 132.1, TT 135.5;
-    //           operand stored late as in LOOP 2                    LOOP 5 NN 135.5, NT 142.4, TN 136.1, TT 138.0
-    // (8192^3, alpha and beta given, TFLOP/s, one process on one box.  The ranking is not stable under
-    // changes elsewhere in the kernel: before the kernel arguments grew by the split-k fields LOOP 0 gave
-    // N,N 142.0 and LOOP 4 140.2.  bench.py holds a floor under the headline rate for that reason.)
+    //   LOOP 4 / 5  LOOP 3 for A only / for B only, the other     256x128: LOOP 4 NN 139.7, NT 143.3, TN 132.6, TT 135.9;
+    //           operand stored late as in LOOP 2                    LOOP 5 NN 135.9, NT 143.9, TN 136.1, TT 138.5
+    // (8192^3, alpha and beta given, TFLOP/s, one process on one box.)  The ranking is not stable under
+    // changes elsewhere in the kernel: one more scalar kernel argument read by every instantiation (a
+    // tile-number offset) took N,N under LOOP 0 from 143 to 132.6 while LOOP 4 stayed at 139 -- the offset
+    // is therefore read by the split-k instantiations only, and bench.py holds a floor under the headline
+    // rate.
     // (the bounds-checked instantiation takes LOOP 2 and up, whose iterations exist per flavour)
     f32x4 af[2][FM], bf[2][FN];
     read_frags(0, 0, af[0], bf[0]);
@@ -704,7 +706,7 @@ void gemm_f64_mfma_kernel(MArgs<double> g) {
     const int l16 = lane & 15, lq = lane >> 4; // lq = 0..3
 
     uint32_t tile_m, tile_n;
-    tile_coords(g.tiles_m, g.tiles_n, tile_m, tile_n, g.xcd_remap, g.pid_offset);
+    tile_coords(g.tiles_m, g.tiles_n, tile_m, tile_n, g.xcd_remap, SPLIT ? g.pid_offset : 0u); // only a split tail starts past tile 0
     const uint32_t m0 = tile_m * BM, n0 = tile_n * BN;
     if constexpr (SPLIT) { // this work-group's share of k, as in the f32 kernel
         const uint32_t k_begin = blockIdx.y * g.klen;
