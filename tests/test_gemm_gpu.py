@@ -78,7 +78,7 @@ def test_float_small_shapes(dev, dtype, op_a, op_b, alpha, beta):
 
 @pytest.mark.parametrize("variant", ["tile64", "mfma_f32_64x64", "mfma_f32_64x64s2", "mfma_f32_64x64s4", "mfma_f32_32x32s4",
                                      "mfma_f32_64x64z", "mfma_f32_128x128", "mfma_f32_128x128s2", "mfma_f32_256x128",
-                                     "mfma_f32_128x128t", "mfma_f32_256x128t"])
+                                     "mfma_f32_128x128t", "mfma_f32_256x128t", "mfma_f32_256x128d"])
 @pytest.mark.parametrize("op_a,op_b", OPS)
 def test_f32_every_variant(dev, variant, op_a, op_b):
     import ctypes
@@ -359,6 +359,26 @@ def test_k_split_over_work_groups(dev, dtype):
         dA.free(); dB.free()
     finally:
         lib.wk_gemm_force_variant(b"auto")
+
+
+@pytest.mark.parametrize("op_a,op_b", OPS)
+def test_slabs_straight_into_lds(dev, op_a, op_b):
+    """The 256 x 128 kernel that brings its k-slabs from global memory straight into LDS (three stages,
+    swizzled layouts): every count of slabs from one to a handful (the pipeline's prologue and its last
+    two iterations are special), several tiles, every epilogue, leading dimensions with gaps; against
+    the oracle.  Shapes it does not take (ragged, unaligned) fall back to the register-staged tile."""
+    assert dev.lib.wk_gemm_force_variant(b"mfma_f32_256x128d") == 0
+    try:
+        for K in (16, 32, 48, 64, 80, 96, 112, 128, 256, 1040):
+            check(dev, "f32", 256, 128, K, op_a, op_b, 1.5, 0.5, seed=200 + K)
+        check(dev, "f32", 512, 384, 320, op_a, op_b, None, None, seed=231)
+        check(dev, "f32", 768, 256, 64, op_a, op_b, 2.0, None, seed=232)
+        check(dev, "f32", 2304, 1152, 176, op_a, op_b, None, -0.25, seed=233)            # 81 tiles, more than one group of tile rows
+        check(dev, "f32", 512, 256, 96, op_a, op_b, 1.5, 0.5, seed=234,
+              lda=(512 if op_a else 96) + 8, ldb=(96 if op_b else 256) + 12, ldc=256 + 5)  # gaps between rows, 16-byte aligned
+        check(dev, "f32", 300, 200, 100, op_a, op_b, 1.5, 0.5, seed=235)                  # ragged: the staged tile runs
+    finally:
+        dev.lib.wk_gemm_force_variant(b"auto")
 
 
 def test_left_over_tiles_run_as_a_k_split_tail(dev):

@@ -1,0 +1,338 @@
+// f32 GEMM on the CDNA4 matrix cores with k-slabs brought from global memory straight into LDS
+// (gfx950's 16-byte-per-lane global_load_lds), three slabs deep.
+//
+// Same tiling and matrix-instruction mapping as the 256 x 128 kernel of wk_gemm_mfma.hip
+// (v_mfma_f32_32x32x2_f32, 2 x 2 wavefronts, wave tile 128 x 64, k-slab 16), for the interior case
+// only: M % 256 == N % 128 == K % 16 == 0 and 16-byte aligned rows.  What differs is how a slab
+// gets into LDS and how the work-group hands over from one slab to the next:
+//   * no staging registers and no LDS stores: every lane names 16 bytes of global memory and the
+//     load unit writes them to LDS at (wave-uniform base) + 16 * lane.  The lane -> address map is
+//     free, the LDS side is not, so padding is replaced by swizzling: the lane that fills LDS
+//     chunk p of a row fetches the chunk that belongs there;
+//   * unpadded slabs are 24 KB (A 16 KB + B 8 KB), so three of them fit twice on a compute unit
+//     (144 of 160 KB).  Slab kt+2 is requested at the top of iteration kt, a whole iteration and a
+//     half before it is read, and the only thing between the matrix instructions of two slabs is
+//     one barrier (every wavefront first waits for its own share of slab kt+1 to have landed).
+//
+// LDS layouts (floats):
+//   k-contiguous operand (A for op_a = N, B for op_b = T): [row][16], four 16-byte chunks per row,
+//     chunk c of row r stored at chunk position c ^ ((r >> 2) & 3).  A fragment is one 16-byte read
+//     per lane (row = lane % 32, k = 8 s + 4 (lane / 32) + 0..3); sixteen consecutive rows at one
+//     logical chunk cover all 64 banks once.
+//   m/n-contiguous operand (A for op_a = T, B for op_b = N): [k][ROWS], element (k, m) stored at
+//     m ^ (32 * ((k >> 2) & 1)).  Fragments are 4-byte reads; the two half-wavefronts read rows k
+//     and k + 4, which the swizzle puts on disjoint banks.
+//
+// The loads are issued through inline assembly: the compiler's wait-count pass treats a direct-to-LDS
+// load it knows about as a store that any later LDS read may alias and would wait for all of them in
+// front of every fragment read, which serialises exactly what this kernel overlaps.  The waits that
+// are needed are written out instead (vmcnt before the barrier that publishes a slab).
+#include "wk_internal.hpp"
+
+#include <cstring>
+
+using namespace wk;
+
+namespace {
+
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+
+constexpr int GROUP_M = 8;
+
+struct DArgs {
+    const float *A, *B;
+    float *C;
+    uint32_t M, N, K;
+    uint32_t lda, ldb, ldc;
+    uint32_t tiles_m, tiles_n;
+    uint32_t num_cus;
+    int epi;
+    float alpha, beta;
+};
+
+// 16 bytes per lane from global memory (scalar base + 32-bit byte offset per lane) to LDS at
+// lds_base + 16 * lane; lds_base is a byte address, the same in every lane.
+__device__ __forceinline__ void dma16(const float *base, uint32_t byte_offset, uint32_t lds_base) {
+    asm volatile("s_mov_b32 m0, %2\n\t"
+                 "s_nop 0\n\t"
+                 "global_load_lds_dwordx4 %0, %1"
+                 :
+                 : "v"(byte_offset), "s"(base), "s"(lds_base)
+                 : "memory");
+}
+
+template <int N> __device__ __forceinline__ void wait_vm() { asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory"); }
+__device__ __forceinline__ void wait_lgkm0() { asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); }
+
+template <bool A_K, bool B_K>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2)))
+void gemm_f32_dma_kernel(DArgs g) {
+    constexpr int BM = 256, BN = 128, BK = 16, WM = 128, WN = 64, FM = 4, FN = 2;
+    constexpr int A_FLOATS = BM * BK, B_FLOATS = BN * BK, STAGE = A_FLOATS + B_FLOATS; // 4096 + 2048
+    constexpr int A_LOADS = 4, B_LOADS = 2; // per thread per slab
+
+    extern __shared__ __align__(16) float lds[]; // [3][STAGE]: A then B
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6); // the same in every lane: kept in a scalar register
+    const int wm = wave >> 1, wn = wave & 1;
+    const int l32 = lane & 31, lhi = lane >> 5;
+
+    // tile walk: groups of GROUP_M tile rows, as in wk_gemm_mfma.hip (every XCD sweeps the same panel of B)
+    uint32_t tile_m, tile_n;
+    {
+        const uint32_t pid = blockIdx.x;
+        const uint32_t group_size = GROUP_M * g.tiles_n;
+        const uint32_t group = pid / group_size;
+        const uint32_t first_m = group * GROUP_M;
+        const uint32_t gsz = min(g.tiles_m - first_m, (uint32_t)GROUP_M);
+        const uint32_t in_group = pid - group * group_size;
+        tile_m = first_m + in_group % gsz;
+        tile_n = in_group / gsz;
+    }
+    const uint32_t m0 = tile_m * BM, n0 = tile_n * BN;
+    // the second co-resident work-group of the first dispatch wave starts one solo iteration late, so
+    // that the two do not hand over at the same time
+    if (g.num_cus && blockIdx.x / g.num_cus == 1)
+        for (int i = 0; i < FM * FN * BK / 4; ++i) __builtin_amdgcn_s_sleep(2);
+
+    // ---- global side: scalar bases (advance by one slab per iteration) and per-lane byte offsets ----
+    const float *a_base = A_K ? g.A + (size_t)m0 * g.lda : g.A + m0;
+    const float *b_base = B_K ? g.B + (size_t)n0 * g.ldb : g.B + n0;
+    const size_t a_step = A_K ? (size_t)BK : (size_t)BK * g.lda; // floats per slab
+    const size_t b_step = B_K ? (size_t)BK : (size_t)BK * g.ldb;
+    uint32_t a_off[A_LOADS], b_off[B_LOADS];
+#pragma unroll
+    for (int i = 0; i < A_LOADS; ++i) {
+        const int grp = i * 4 + wave; // which 1 KB of the A slab this wavefront fills with load i
+        if constexpr (A_K) {
+            const uint32_t row = grp * 16 + (lane >> 2);
+            const uint32_t chunk = (lane & 3) ^ ((row >> 2) & 3);
+            a_off[i] = (row * g.lda + 4 * chunk) * 4u;
+        } else {
+            const uint32_t k = grp; // one row of k per load
+            const uint32_t chunk = lane ^ (((k >> 2) & 1) * 8);
+            a_off[i] = (k * g.lda + 4 * chunk) * 4u;
+        }
+    }
+#pragma unroll
+    for (int i = 0; i < B_LOADS; ++i) {
+        const int grp = i * 4 + wave; // which 1 KB of the B slab
+        if constexpr (B_K) {
+            const uint32_t row = grp * 16 + (lane >> 2);
+            const uint32_t chunk = (lane & 3) ^ ((row >> 2) & 3);
+            b_off[i] = (row * g.ldb + 4 * chunk) * 4u;
+        } else {
+            const uint32_t k = grp * 2 + (lane >> 5); // two rows of k per load
+            const uint32_t chunk = (lane & 31) ^ (((k >> 2) & 1) * 8);
+            b_off[i] = (k * g.ldb + 4 * chunk) * 4u;
+        }
+    }
+    const uint32_t lds0 =
+        __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)(__attribute__((address_space(3))) float *)lds); // byte address of the array
+
+    // the next slab of both operands into the stage at byte offset `stage_bytes`; the bases then point at
+    // the slab after it
+    auto issue = [&](uint32_t stage_bytes) {
+        const uint32_t sbase = lds0 + stage_bytes + (uint32_t)wave * 1024u;
+#pragma unroll
+        for (int i = 0; i < A_LOADS; ++i) dma16(a_base, a_off[i], sbase + (uint32_t)i * 4096u);
+#pragma unroll
+        for (int i = 0; i < B_LOADS; ++i) dma16(b_base, b_off[i], sbase + A_FLOATS * 4u + (uint32_t)i * 4096u);
+        a_base += a_step;
+        b_base += b_step;
+    };
+
+    // ---- LDS side: per-lane fragment addresses (floats from the start of a stage's A or B part) ----
+    // k-contiguous: row * 16 + 4 * (chunk ^ swz); chunk = 2 s + lhi, swz = (l32 >> 2) & 3 (row offsets are multiples of 32)
+    // m-contiguous: k * ROWS + (m ^ 32 lhi); k = 8 s + 4 lhi + t; m = wave offset + 32 i + l32
+    // (32-float blocks i of a half-wavefront: 32 (i ^ lhi) = 32 i + 32 lhi for even i, 32 i - 32 lhi for odd i,
+    // hence one base for the even blocks and one for the odd ones, the rest are immediates)
+    const int sw4 = 4 * (lhi ^ ((l32 >> 2) & 3));
+    const int a_frag_e = A_K ? (wm * WM + l32) * 16 + sw4 : 4 * lhi * BM + wm * WM + l32 + 32 * lhi;
+    const int a_frag_o = A_K ? a_frag_e : 4 * lhi * BM + wm * WM + l32 - 32 * lhi;
+    const int b_frag_e = B_K ? (wn * WN + l32) * 16 + sw4 : 4 * lhi * BN + wn * WN + l32 + 32 * lhi;
+    const int b_frag_o = B_K ? b_frag_e : 4 * lhi * BN + wn * WN + l32 - 32 * lhi;
+
+    auto read_frags = [&](uint32_t stage_bytes, int s, f32x4 *af, f32x4 *bf) {
+        const float *as = lds + stage_bytes / 4;
+        const float *bs = as + A_FLOATS;
+#pragma unroll
+        for (int i = 0; i < FM; ++i) {
+            if constexpr (A_K) {
+                // chunk 2 s + lhi: the second step's chunk is the first one's with bit 1 flipped
+                af[i] = *reinterpret_cast<const f32x4 *>(as + ((a_frag_e ^ (s ? 8 : 0)) + i * 32 * 16));
+            } else {
+                const int base = (i & 1) ? a_frag_o : a_frag_e;
+#pragma unroll
+                for (int t = 0; t < 4; ++t) af[i][t] = as[base + (8 * s + t) * BM + 32 * i];
+            }
+        }
+#pragma unroll
+        for (int j = 0; j < FN; ++j) {
+            if constexpr (B_K) {
+                bf[j] = *reinterpret_cast<const f32x4 *>(bs + ((b_frag_e ^ (s ? 8 : 0)) + j * 32 * 16));
+            } else {
+                const int base = (j & 1) ? b_frag_o : b_frag_e;
+#pragma unroll
+                for (int t = 0; t < 4; ++t) bf[j][t] = bs[base + (8 * s + t) * BN + 32 * j];
+            }
+        }
+    };
+
+    f32x16 acc[FM][FN];
+#pragma unroll
+    for (int i = 0; i < FM; ++i)
+#pragma unroll
+        for (int j = 0; j < FN; ++j)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+
+    f32x4 af[2][FM], bf[2][FN];
+    auto mfma_step = [&](int s) {
+#pragma unroll
+        for (int t = 0; t < 4; ++t)
+#pragma unroll
+            for (int i = 0; i < FM; ++i)
+#pragma unroll
+                for (int j = 0; j < FN; ++j)
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(af[s & 1][i][t], bf[s & 1][j][t], acc[i][j], 0, 0, 0);
+    };
+
+    const uint32_t ktiles = g.K / BK;
+
+    // The three stages rotate: the slab being multiplied, the next one, and the one after it (byte offsets).
+    constexpr uint32_t STAGE_BYTES = STAGE * 4u;
+    uint32_t st_cur = 0, st_next = STAGE_BYTES, st_after = 2 * STAGE_BYTES;
+
+    // prologue: slabs 0 and 1 on their way, slab 0 landed everywhere, first fragments read
+    issue(st_cur);
+    if (ktiles > 1) {
+        issue(st_next);
+        wait_vm<A_LOADS + B_LOADS>();
+    } else {
+        wait_vm<0>();
+    }
+    __builtin_amdgcn_s_barrier();
+    read_frags(st_cur, 0, af[0], bf[0]);
+
+    // One iteration on the slab in stage st_cur.  MORE2: slab kt+2 exists and is requested into the stage
+    // that slab kt-1 left (every wavefront is past the barrier of iteration kt-1, in front of which it
+    // waited for its last reads of that stage).  MORE1: slab kt+1 exists; before the last step's matrix
+    // instructions this wavefront waits for its own loads of slab kt+1 (those of slab kt+2 may stay in
+    // flight) and for its LDS reads, joins the barrier and reads the first fragments of slab kt+1.
+    auto iteration = [&](auto more2_tag, auto more1_tag) __attribute__((always_inline)) {
+        constexpr bool MORE2 = decltype(more2_tag)::value, MORE1 = decltype(more1_tag)::value;
+        if constexpr (MORE2) issue(st_after);
+        read_frags(st_cur, 1, af[1], bf[1]);
+        mfma_step(0);
+        if constexpr (MORE1) {
+            __builtin_amdgcn_sched_barrier(0);
+            if constexpr (MORE2) wait_vm<A_LOADS + B_LOADS>();
+            else wait_vm<0>();
+            wait_lgkm0();
+            __builtin_amdgcn_s_barrier();
+            read_frags(st_next, 0, af[0], bf[0]);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        mfma_step(1);
+        const uint32_t t = st_cur;
+        st_cur = st_next;
+        st_next = st_after;
+        st_after = t;
+    };
+    using T_ = std::true_type;
+    using F_ = std::false_type;
+    uint32_t kt = 0;
+    for (; kt + 2 < ktiles; ++kt) iteration(T_{}, T_{}); // steady state: both following slabs exist
+    if (kt + 1 < ktiles) iteration(F_{}, T_{});          // the last but one
+    iteration(F_{}, F_{});                               // the last
+
+    // ---- epilogue: acc register r of lane l is C[8*(r/4) + 4*(l/32) + r%4][l%32] of its 32x32 block;
+    // option semantics of src/blas/gemm.zig:500-501,591-602 (C_old is read and multiplied whenever beta
+    // is given); the reads of C_old of a block are issued as one batch
+    const float alpha = g.alpha, beta = g.beta;
+#pragma unroll
+    for (int i = 0; i < FM; ++i)
+#pragma unroll
+        for (int j = 0; j < FN; ++j) {
+            const uint32_t col = n0 + wn * WN + j * 32 + l32;
+            float old[16];
+            if (g.epi == EPI_ALPHA_BETA) {
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    const uint32_t row = m0 + wm * WM + i * 32 + 8 * (r / 4) + 4 * lhi + (r % 4);
+                    old[r] = g.C[(size_t)row * g.ldc + col];
+                }
+            }
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const uint32_t row = m0 + wm * WM + i * 32 + 8 * (r / 4) + 4 * lhi + (r % 4);
+                float v = acc[i][j][r];
+                if (g.epi == EPI_ALPHA) v = alpha * v;
+                else if (g.epi == EPI_ALPHA_BETA) v = alpha * v + beta * old[r];
+                g.C[(size_t)row * g.ldc + col] = v;
+            }
+        }
+}
+
+// first_tiles: launch only that many tiles, in tile-walk order (0: all of them)
+template <bool A_K, bool B_K> int launch_one(hipStream_t st, const DArgs &g, uint64_t first_tiles) {
+    constexpr size_t lds_bytes = 3 * (256 * 16 + 128 * 16) * sizeof(float); // 72 KB
+    auto kern = gemm_f32_dma_kernel<A_K, B_K>;
+    static const int attr_rc = [&] {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                           (int)lds_bytes);
+        if (e != hipSuccess) {
+            (void)hipGetLastError();
+            return hip_code(e);
+        }
+        return (int)WK_OK;
+    }();
+    if (attr_rc) return attr_rc;
+    const unsigned grid = first_tiles ? (unsigned)first_tiles : g.tiles_m * g.tiles_n;
+    hipLaunchKernelGGL(kern, dim3(grid), dim3(256), lds_bytes, st, g);
+    return launch_status();
+}
+
+} // namespace
+
+// What the kernel takes for granted, checked on the host: whole tiles, whole k-slabs, 16-byte aligned
+// rows, and every per-lane byte offset inside 32 bits.
+bool wk::gemm_f32_dma_applies(const GemmProblem &p) {
+    if (p.dtype != WK_F32 || p.ext) return false;
+    if (p.M % 256 || p.N % 128 || p.K % 16) return false;
+    if (p.lda % 4 || p.ldb % 4) return false;
+    if ((reinterpret_cast<uintptr_t>(p.A) | reinterpret_cast<uintptr_t>(p.B)) & 15u) return false;
+    if (p.M > 0x7fffffffull || p.N > 0x7fffffffull || p.K > 0x7fffffffull || p.ldc > 0x7fffffffull) return false;
+    // offsets reach 255 rows (k-contiguous) or 15 rows of k (m-contiguous) past the tile's origin
+    if (p.lda > (1ull << 21) || p.ldb > (1ull << 21)) return false;
+    if ((p.M / 256) * (p.N / 128) > 0x7fffffffull) return false;
+    return true;
+}
+
+int wk::gemm_f32_dma_launch(hipStream_t st, const GemmProblem &p, uint64_t first_tiles) {
+    if (!gemm_f32_dma_applies(p)) return WK_E_INVALID_VALUE;
+    if (first_tiles > (p.M / 256) * (p.N / 128)) return WK_E_INVALID_VALUE;
+    DArgs g{};
+    g.A = static_cast<const float *>(p.A);
+    g.B = static_cast<const float *>(p.B);
+    g.C = static_cast<float *>(p.C);
+    g.M = (uint32_t)p.M; g.N = (uint32_t)p.N; g.K = (uint32_t)p.K;
+    g.lda = (uint32_t)p.lda; g.ldb = (uint32_t)p.ldb; g.ldc = (uint32_t)p.ldc;
+    g.tiles_m = (uint32_t)(p.M / 256);
+    g.tiles_n = (uint32_t)(p.N / 128);
+    g.num_cus = p.num_cus;
+    g.epi = p.epi;
+    std::memcpy(&g.alpha, p.alpha, sizeof(float));
+    std::memcpy(&g.beta, p.beta, sizeof(float));
+    const int sel = (p.op_a ? 0 : 2) | (p.op_b ? 1 : 0); // bit 1: A k-contiguous, bit 0: B k-contiguous
+    switch (sel) {
+    case 0: return launch_one<false, false>(st, g, first_tiles);
+    case 1: return launch_one<false, true>(st, g, first_tiles);
+    case 2: return launch_one<true, false>(st, g, first_tiles);
+    default: return launch_one<true, true>(st, g, first_tiles);
+    }
+}

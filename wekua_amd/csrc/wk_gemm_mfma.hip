@@ -1363,7 +1363,10 @@ int launch_f32_tail(hipStream_t st, const GemmProblem &p, bool edge) {
     if (p.ext || !plan_tail(p, BM, BN, BK, sizeof(float), OCC, g_tail_relaxed, plan)) return launch_f32<BM, BN, BK, WMS, WNS, OCC>(st, p, edge);
     const int sel = (p.op_a ? 0 : 2) | (p.op_b ? 1 : 0);
     int rc = WK_OK;
-    if (plan.first_tile > 0) { // the whole rounds, as the plain variant would run them
+    if (plan.first_tile > 0 && BM == 256 && BN == 128 && !edge && gemm_f32_dma_applies(p)) {
+        rc = gemm_f32_dma_launch(st, p, plan.first_tile); // the whole rounds on the direct-to-LDS kernel
+        if (rc) return rc;
+    } else if (plan.first_tile > 0) { // the whole rounds, as the plain variant would run them
 #define WK_CASE(AK, BKC)                                                                                                \
     rc = edge ? launch_f32_one<BM, BN, BK, WMS, WNS, OCC, AK, BKC, true>(st, p, &plan)                                   \
               : launch_f32_one<BM, BN, BK, WMS, WNS, OCC, AK, BKC, false>(st, p, &plan);                                 \
@@ -1387,6 +1390,12 @@ int launch_f32_tail(hipStream_t st, const GemmProblem &p, bool edge) {
     default: WK_CASE(true, true);
     }
 #undef WK_CASE
+}
+
+// the direct-to-LDS kernel where it applies, the register-staged 256 x 128 tile elsewhere
+int launch_f32_dma(hipStream_t st, const GemmProblem &p, bool edge) {
+    if (!edge && gemm_f32_dma_applies(p)) return gemm_f32_dma_launch(st, p);
+    return launch_f32<256, 128, 16, 2, 2, 2>(st, p, edge);
 }
 
 struct VariantDesc {
@@ -1416,6 +1425,9 @@ int split_kind_of(const char *name) { // by the name's suffix: ...z splits every
 const VariantDesc k_variants[] = {
     {"mfma_f32_256x128", WK_F32, 256, 128, 16, 0.940, 0.19, &launch_f32<256, 128, 16, 2, 2, 2>, nullptr, nullptr, nullptr, nullptr,
      "mfma_f32_256x128t", 2},
+    // slabs straight into LDS, three deep; interior shapes only (the cost loop skips it elsewhere):
+    // 147.5 against 142.5 TFLOP/s at 8192^3, T,N 145.5 against 136
+    {"mfma_f32_256x128d", WK_F32, 256, 128, 16, 0.973, 0.19, &launch_f32_dma, nullptr, nullptr, nullptr, nullptr, "mfma_f32_256x128t", 2},
     {"mfma_f32_256x128t", WK_F32, 256, 128, 16, 0.0, 0.25, &launch_f32_tail<256, 128, 16, 2, 2, 2>, nullptr, nullptr, nullptr, nullptr,
      nullptr, 2}, // whole rounds + a k-split tail
     {"mfma_f32_128x128", WK_F32, 128, 128, 16, 0.897, 0.19, &launch_f32<128, 128, 16, 2, 2, 3>, nullptr, nullptr, nullptr, nullptr,
@@ -1533,6 +1545,7 @@ int wk::gemm_mfma_pick(const GemmProblem &p) {
     for (int v = 0; v < k_num_variants; ++v) {
         const VariantDesc &d = k_variants[v];
         if (d.dtype != p.dtype || d.efficiency <= 0.0) continue;
+        if (d.launch == &launch_f32_dma && (p.ext || !gemm_f32_dma_applies(p))) continue;
         const double tiles = (double)((p.M + d.bm - 1) / d.bm) * (double)((p.N + d.bn - 1) / d.bn);
         // Whole rounds: the big tiles (two or three work-groups per unit) pay for a started round in
         // full, the small tile (four per unit, short) for about two thirds of it.
