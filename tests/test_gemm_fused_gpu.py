@@ -48,13 +48,15 @@ def both(dev, dtype, M, N, K, op_a, op_b, kind, with_bias, seed, ld_extra=0):
 @pytest.mark.parametrize("dtype,variant", [("f32", "auto"), ("f32", "mfma_f32_64x64"), ("f32", "mfma_f32_64x64s2"),
                                            ("f32", "mfma_f32_64x64s4"), ("f32", "mfma_f32_32x32s4"), ("f32", "mfma_f32_128x128s2"), ("f64", "mfma_f64_64x64s2"), ("f64", "mfma_f64_32x32s4"), ("f32", "mfma_f32_128x128"),
                                            ("f32", "mfma_f32_256x128"), ("f64", "auto"), ("f64", "mfma_f64_64x64"),
-                                           ("f64", "mfma_f64_128x64"), ("f64", "mfma_f64_128x128"), ("f32", "tile64")])
+                                           ("f64", "mfma_f64_128x64"), ("f64", "mfma_f64_128x128"), ("f32", "tile64"),
+                                           ("f32", "mfma_f32_256x128d"), ("f32", "mfma_f32_128x128d"), ("f32", "mfma_f32_64x64d")])
 @pytest.mark.parametrize("kind", ["none", "sigmoid", "tanh"])
 def test_fused_equals_two_calls(dev, dtype, variant, kind):
     assert dev.lib.wk_gemm_force_variant(variant.encode()) == 0
     try:
         seed = 0
-        for (M, N, K, extra) in [(256, 256, 64, 0), (128, 384, 100, 0), (70, 45, 33, 0), (257, 129, 17, 3), (300, 200, 96, 4)]:
+        for (M, N, K, extra) in [(256, 256, 64, 0), (128, 384, 100, 0), (70, 45, 33, 0), (257, 129, 17, 3), (300, 200, 96, 4),
+                                 (512, 256, 48, 4), (256, 128, 16, 0), (768, 384, 160, 8)]:
             for with_bias in (True, False):
                 seed += 1
                 fused, two, A, B, bias = both(dev, dtype, M, N, K, 0, 1, kind, with_bias, seed, extra)

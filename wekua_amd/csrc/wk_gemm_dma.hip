@@ -1,16 +1,16 @@
 // f32 GEMM on the CDNA4 matrix cores with k-slabs brought from global memory straight into LDS
 // (gfx950's 16-byte-per-lane global_load_lds), three slabs deep.
 //
-// Same tiling and matrix-instruction mapping as the 256 x 128 kernel of wk_gemm_mfma.hip
-// (v_mfma_f32_32x32x2_f32, 2 x 2 wavefronts, wave tile 128 x 64, k-slab 16), for the interior case
-// only: M % 256 == N % 128 == K % 16 == 0 and 16-byte aligned rows.  What differs is how a slab
+// Same tiling and matrix-instruction mapping as the kernels of wk_gemm_mfma.hip
+// (v_mfma_f32_32x32x2_f32, 2 x 2 wavefronts, macro tiles 256 x 128, 128 x 128 and 64 x 64, k-slab 16),
+// for the interior case only: M % BM == N % BN == K % 16 == 0 and 16-byte aligned rows.  What differs is how a slab
 // gets into LDS and how the work-group hands over from one slab to the next:
 //   * no staging registers and no LDS stores: every lane names 16 bytes of global memory and the
 //     load unit writes them to LDS at (wave-uniform base) + 16 * lane.  The lane -> address map is
 //     free, the LDS side is not, so padding is replaced by swizzling: the lane that fills LDS
 //     chunk p of a row fetches the chunk that belongs there;
-//   * unpadded slabs are 24 KB (A 16 KB + B 8 KB), so three of them fit twice on a compute unit
-//     (144 of 160 KB).  Slab kt+2 is requested at the top of iteration kt, a whole iteration and a
+//   * unpadded slabs of the 256 x 128 tile are 24 KB (A 16 KB + B 8 KB), so three of them fit twice
+//     on a compute unit (144 of 160 KB; 128 x 128: 3 x 16 KB three times; 64 x 64: 3 x 8 KB four times).  Slab kt+2 is requested at the top of iteration kt, a whole iteration and a
 //     half before it is read, and the only thing between the matrix instructions of two slabs is
 //     one barrier (every wavefront first waits for its own share of slab kt+1 to have landed).
 //
@@ -49,6 +49,8 @@ struct DArgs {
     uint32_t num_cus;
     int epi;
     float alpha, beta;
+    const float *bias; // kernels instantiated with EXT: C = act(acc + bias[col]); bias may be null
+    int act;
 };
 
 // 16 bytes per lane from global memory (scalar base + 32-bit byte offset per lane) to LDS at
@@ -65,12 +67,13 @@ __device__ __forceinline__ void dma16(const float *base, uint32_t byte_offset, u
 template <int N> __device__ __forceinline__ void wait_vm() { asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory"); }
 __device__ __forceinline__ void wait_lgkm0() { asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); }
 
-template <bool A_K, bool B_K>
-__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2)))
+template <int BM, int BN, int OCC, bool A_K, bool B_K, bool EXT>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(OCC)))
 void gemm_f32_dma_kernel(DArgs g) {
-    constexpr int BM = 256, BN = 128, BK = 16, WM = 128, WN = 64, FM = 4, FN = 2;
-    constexpr int A_FLOATS = BM * BK, B_FLOATS = BN * BK, STAGE = A_FLOATS + B_FLOATS; // 4096 + 2048
-    constexpr int A_LOADS = 4, B_LOADS = 2; // per thread per slab
+    constexpr int BK = 16, WM = BM / 2, WN = BN / 2, FM = WM / 32, FN = WN / 32;
+    constexpr int A_FLOATS = BM * BK, B_FLOATS = BN * BK, STAGE = A_FLOATS + B_FLOATS;
+    constexpr int A_LOADS = BM / 64, B_LOADS = BN / 64; // 1 KB per wavefront and load, four wavefronts
+    static_assert(BM % 64 == 0 && BN % 64 == 0, "tile shape");
 
     extern __shared__ __align__(16) float lds[]; // [3][STAGE]: A then B
 
@@ -95,8 +98,11 @@ void gemm_f32_dma_kernel(DArgs g) {
     const uint32_t m0 = tile_m * BM, n0 = tile_n * BN;
     // the second co-resident work-group of the first dispatch wave starts one solo iteration late, so
     // that the two do not hand over at the same time
-    if (g.num_cus && blockIdx.x / g.num_cus == 1)
-        for (int i = 0; i < FM * FN * BK / 4; ++i) __builtin_amdgcn_s_sleep(2);
+    if (g.num_cus) {
+        const uint32_t slot = blockIdx.x / g.num_cus;
+        if (slot >= 1 && slot < (uint32_t)OCC)
+            for (uint32_t i = 0; i < slot * (FM * FN * BK / 4); ++i) __builtin_amdgcn_s_sleep(2);
+    }
 
     // ---- global side: scalar bases (advance by one slab per iteration) and per-lane byte offsets ----
     const float *a_base = A_K ? g.A + (size_t)m0 * g.lda : g.A + m0;
@@ -104,32 +110,27 @@ void gemm_f32_dma_kernel(DArgs g) {
     const size_t a_step = A_K ? (size_t)BK : (size_t)BK * g.lda; // floats per slab
     const size_t b_step = B_K ? (size_t)BK : (size_t)BK * g.ldb;
     uint32_t a_off[A_LOADS], b_off[B_LOADS];
-#pragma unroll
-    for (int i = 0; i < A_LOADS; ++i) {
-        const int grp = i * 4 + wave; // which 1 KB of the A slab this wavefront fills with load i
-        if constexpr (A_K) {
+    // load i of this wavefront fills the 1 KB group i * 4 + wave of the operand's slab: sixteen rows of a
+    // k-contiguous operand, 256 / ROWS rows of k of an m-contiguous one
+    auto lane_offset = [&](int grp, uint32_t ld, auto kc_tag, auto rows_tag) -> uint32_t {
+        constexpr bool KC = decltype(kc_tag)::value;
+        constexpr int ROWS = decltype(rows_tag)::value;
+        if constexpr (KC) {
             const uint32_t row = grp * 16 + (lane >> 2);
             const uint32_t chunk = (lane & 3) ^ ((row >> 2) & 3);
-            a_off[i] = (row * g.lda + 4 * chunk) * 4u;
+            return (row * ld + 4 * chunk) * 4u;
         } else {
-            const uint32_t k = grp; // one row of k per load
-            const uint32_t chunk = lane ^ (((k >> 2) & 1) * 8);
-            a_off[i] = (k * g.lda + 4 * chunk) * 4u;
+            constexpr int PER_ROW = ROWS / 4; // 16-byte chunks per row of k
+            const uint32_t k = grp * (64 / PER_ROW) + lane / PER_ROW;
+            const uint32_t chunk = (lane % PER_ROW) ^ (((k >> 2) & 1) * 8);
+            return (k * ld + 4 * chunk) * 4u;
         }
-    }
+    };
+    using std::integral_constant;
 #pragma unroll
-    for (int i = 0; i < B_LOADS; ++i) {
-        const int grp = i * 4 + wave; // which 1 KB of the B slab
-        if constexpr (B_K) {
-            const uint32_t row = grp * 16 + (lane >> 2);
-            const uint32_t chunk = (lane & 3) ^ ((row >> 2) & 3);
-            b_off[i] = (row * g.ldb + 4 * chunk) * 4u;
-        } else {
-            const uint32_t k = grp * 2 + (lane >> 5); // two rows of k per load
-            const uint32_t chunk = (lane & 31) ^ (((k >> 2) & 1) * 8);
-            b_off[i] = (k * g.ldb + 4 * chunk) * 4u;
-        }
-    }
+    for (int i = 0; i < A_LOADS; ++i) a_off[i] = lane_offset(i * 4 + wave, g.lda, integral_constant<bool, A_K>{}, integral_constant<int, BM>{});
+#pragma unroll
+    for (int i = 0; i < B_LOADS; ++i) b_off[i] = lane_offset(i * 4 + wave, g.ldb, integral_constant<bool, B_K>{}, integral_constant<int, BN>{});
     const uint32_t lds0 =
         __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)(__attribute__((address_space(3))) float *)lds); // byte address of the array
 
@@ -148,13 +149,14 @@ void gemm_f32_dma_kernel(DArgs g) {
     // ---- LDS side: per-lane fragment addresses (floats from the start of a stage's A or B part) ----
     // k-contiguous: row * 16 + 4 * (chunk ^ swz); chunk = 2 s + lhi, swz = (l32 >> 2) & 3 (row offsets are multiples of 32)
     // m-contiguous: k * ROWS + (m ^ 32 lhi); k = 8 s + 4 lhi + t; m = wave offset + 32 i + l32
-    // (32-float blocks i of a half-wavefront: 32 (i ^ lhi) = 32 i + 32 lhi for even i, 32 i - 32 lhi for odd i,
-    // hence one base for the even blocks and one for the odd ones, the rest are immediates)
     const int sw4 = 4 * (lhi ^ ((l32 >> 2) & 3));
-    const int a_frag_e = A_K ? (wm * WM + l32) * 16 + sw4 : 4 * lhi * BM + wm * WM + l32 + 32 * lhi;
-    const int a_frag_o = A_K ? a_frag_e : 4 * lhi * BM + wm * WM + l32 - 32 * lhi;
-    const int b_frag_e = B_K ? (wn * WN + l32) * 16 + sw4 : 4 * lhi * BN + wn * WN + l32 + 32 * lhi;
-    const int b_frag_o = B_K ? b_frag_e : 4 * lhi * BN + wn * WN + l32 - 32 * lhi;
+    int a_frag[FM], b_frag[FN]; // k-contiguous: one base (block i is an immediate away); m-contiguous: block i's column
+#pragma unroll
+    for (int i = 0; i < FM; ++i)
+        a_frag[i] = A_K ? (wm * WM + l32) * 16 + sw4 : 4 * lhi * BM + (((wm * WM + 32 * i) ^ (32 * lhi)) + l32);
+#pragma unroll
+    for (int j = 0; j < FN; ++j)
+        b_frag[j] = B_K ? (wn * WN + l32) * 16 + sw4 : 4 * lhi * BN + (((wn * WN + 32 * j) ^ (32 * lhi)) + l32);
 
     auto read_frags = [&](uint32_t stage_bytes, int s, f32x4 *af, f32x4 *bf) {
         const float *as = lds + stage_bytes / 4;
@@ -163,21 +165,19 @@ void gemm_f32_dma_kernel(DArgs g) {
         for (int i = 0; i < FM; ++i) {
             if constexpr (A_K) {
                 // chunk 2 s + lhi: the second step's chunk is the first one's with bit 1 flipped
-                af[i] = *reinterpret_cast<const f32x4 *>(as + ((a_frag_e ^ (s ? 8 : 0)) + i * 32 * 16));
+                af[i] = *reinterpret_cast<const f32x4 *>(as + ((a_frag[i] ^ (s ? 8 : 0)) + i * 32 * 16));
             } else {
-                const int base = (i & 1) ? a_frag_o : a_frag_e;
 #pragma unroll
-                for (int t = 0; t < 4; ++t) af[i][t] = as[base + (8 * s + t) * BM + 32 * i];
+                for (int t = 0; t < 4; ++t) af[i][t] = as[a_frag[i] + (8 * s + t) * BM];
             }
         }
 #pragma unroll
         for (int j = 0; j < FN; ++j) {
             if constexpr (B_K) {
-                bf[j] = *reinterpret_cast<const f32x4 *>(bs + ((b_frag_e ^ (s ? 8 : 0)) + j * 32 * 16));
+                bf[j] = *reinterpret_cast<const f32x4 *>(bs + ((b_frag[j] ^ (s ? 8 : 0)) + j * 32 * 16));
             } else {
-                const int base = (j & 1) ? b_frag_o : b_frag_e;
 #pragma unroll
-                for (int t = 0; t < 4; ++t) bf[j][t] = bs[base + (8 * s + t) * BN + 32 * j];
+                for (int t = 0; t < 4; ++t) bf[j][t] = bs[b_frag[j] + (8 * s + t) * BN];
             }
         }
     };
@@ -259,6 +259,10 @@ void gemm_f32_dma_kernel(DArgs g) {
 #pragma unroll
         for (int j = 0; j < FN; ++j) {
             const uint32_t col = n0 + wn * WN + j * 32 + l32;
+            float bias_v = 0.f;
+            if constexpr (EXT) {
+                if (g.bias) bias_v = g.bias[col];
+            }
             float old[16];
             if (g.epi == EPI_ALPHA_BETA) {
 #pragma unroll
@@ -273,15 +277,19 @@ void gemm_f32_dma_kernel(DArgs g) {
                 float v = acc[i][j][r];
                 if (g.epi == EPI_ALPHA) v = alpha * v;
                 else if (g.epi == EPI_ALPHA_BETA) v = alpha * v + beta * old[r];
+                if constexpr (EXT) { // the fused epilogue of Linear.forward, as in wk_gemm_mfma.hip
+                    if (g.bias) v += bias_v;
+                    v = act_forward<float>(g.act, v);
+                }
                 g.C[(size_t)row * g.ldc + col] = v;
             }
         }
 }
 
 // first_tiles: launch only that many tiles, in tile-walk order (0: all of them)
-template <bool A_K, bool B_K> int launch_one(hipStream_t st, const DArgs &g, uint64_t first_tiles) {
-    constexpr size_t lds_bytes = 3 * (256 * 16 + 128 * 16) * sizeof(float); // 72 KB
-    auto kern = gemm_f32_dma_kernel<A_K, B_K>;
+template <int BM, int BN, int OCC, bool A_K, bool B_K, bool EXT> int launch_one(hipStream_t st, const DArgs &g, uint64_t first_tiles) {
+    constexpr size_t lds_bytes = 3 * (BM * 16 + BN * 16) * sizeof(float); // 72 / 48 / 24 KB
+    auto kern = gemm_f32_dma_kernel<BM, BN, OCC, A_K, B_K, EXT>;
     static const int attr_rc = [&] {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
                                            (int)lds_bytes);
@@ -297,42 +305,54 @@ template <bool A_K, bool B_K> int launch_one(hipStream_t st, const DArgs &g, uin
     return launch_status();
 }
 
-} // namespace
-
-// What the kernel takes for granted, checked on the host: whole tiles, whole k-slabs, 16-byte aligned
-// rows, and every per-lane byte offset inside 32 bits.
-bool wk::gemm_f32_dma_applies(const GemmProblem &p) {
-    if (p.dtype != WK_F32 || p.ext) return false;
-    if (p.M % 256 || p.N % 128 || p.K % 16) return false;
-    if (p.lda % 4 || p.ldb % 4) return false;
-    if ((reinterpret_cast<uintptr_t>(p.A) | reinterpret_cast<uintptr_t>(p.B)) & 15u) return false;
-    if (p.M > 0x7fffffffull || p.N > 0x7fffffffull || p.K > 0x7fffffffull || p.ldc > 0x7fffffffull) return false;
-    // offsets reach 255 rows (k-contiguous) or 15 rows of k (m-contiguous) past the tile's origin
-    if (p.lda > (1ull << 21) || p.ldb > (1ull << 21)) return false;
-    if ((p.M / 256) * (p.N / 128) > 0x7fffffffull) return false;
-    return true;
-}
-
-int wk::gemm_f32_dma_launch(hipStream_t st, const GemmProblem &p, uint64_t first_tiles) {
-    if (!gemm_f32_dma_applies(p)) return WK_E_INVALID_VALUE;
-    if (first_tiles > (p.M / 256) * (p.N / 128)) return WK_E_INVALID_VALUE;
+template <int BM, int BN, int OCC> int launch_tile(hipStream_t st, const GemmProblem &p, uint64_t first_tiles) {
+    if (first_tiles > (p.M / BM) * (p.N / BN)) return WK_E_INVALID_VALUE;
     DArgs g{};
     g.A = static_cast<const float *>(p.A);
     g.B = static_cast<const float *>(p.B);
     g.C = static_cast<float *>(p.C);
     g.M = (uint32_t)p.M; g.N = (uint32_t)p.N; g.K = (uint32_t)p.K;
     g.lda = (uint32_t)p.lda; g.ldb = (uint32_t)p.ldb; g.ldc = (uint32_t)p.ldc;
-    g.tiles_m = (uint32_t)(p.M / 256);
-    g.tiles_n = (uint32_t)(p.N / 128);
+    g.tiles_m = (uint32_t)(p.M / BM);
+    g.tiles_n = (uint32_t)(p.N / BN);
     g.num_cus = p.num_cus;
     g.epi = p.epi;
     std::memcpy(&g.alpha, p.alpha, sizeof(float));
     std::memcpy(&g.beta, p.beta, sizeof(float));
+    g.bias = static_cast<const float *>(p.ext_bias);
+    g.act = p.ext_act;
     const int sel = (p.op_a ? 0 : 2) | (p.op_b ? 1 : 0); // bit 1: A k-contiguous, bit 0: B k-contiguous
+    if (p.ext) // instantiated for op N, T only (what Linear.forward runs)
+        return sel == 3 ? launch_one<BM, BN, OCC, true, true, true>(st, g, first_tiles) : (int)WK_E_INVALID_VALUE;
     switch (sel) {
-    case 0: return launch_one<false, false>(st, g, first_tiles);
-    case 1: return launch_one<false, true>(st, g, first_tiles);
-    case 2: return launch_one<true, false>(st, g, first_tiles);
-    default: return launch_one<true, true>(st, g, first_tiles);
+    case 0: return launch_one<BM, BN, OCC, false, false, false>(st, g, first_tiles);
+    case 1: return launch_one<BM, BN, OCC, false, true, false>(st, g, first_tiles);
+    case 2: return launch_one<BM, BN, OCC, true, false, false>(st, g, first_tiles);
+    default: return launch_one<BM, BN, OCC, true, true, false>(st, g, first_tiles);
     }
+}
+
+} // namespace
+
+// What the kernels take for granted, checked on the host: whole tiles, whole k-slabs, 16-byte aligned
+// rows, every per-lane byte offset inside 32 bits, and for the fused epilogue the one layout it exists for.
+bool wk::gemm_f32_dma_applies(const GemmProblem &p, int bm, int bn) {
+    if (p.dtype != WK_F32) return false;
+    if (!((bm == 256 && bn == 128) || (bm == 128 && bn == 128) || (bm == 64 && bn == 64))) return false;
+    if (p.ext && (p.op_a || !p.op_b)) return false;
+    if (p.M % bm || p.N % bn || p.K % 16) return false;
+    if (p.lda % 4 || p.ldb % 4) return false;
+    if ((reinterpret_cast<uintptr_t>(p.A) | reinterpret_cast<uintptr_t>(p.B)) & 15u) return false;
+    if (p.M > 0x7fffffffull || p.N > 0x7fffffffull || p.K > 0x7fffffffull || p.ldc > 0x7fffffffull) return false;
+    // offsets reach 255 rows (k-contiguous) or 15 rows of k (m-contiguous) past the tile's origin
+    if (p.lda > (1ull << 21) || p.ldb > (1ull << 21)) return false;
+    if ((p.M / bm) * (p.N / bn) > 0x7fffffffull) return false;
+    return true;
+}
+
+int wk::gemm_f32_dma_launch(hipStream_t st, const GemmProblem &p, int bm, int bn, uint64_t first_tiles) {
+    if (!gemm_f32_dma_applies(p, bm, bn)) return WK_E_INVALID_VALUE;
+    if (bm == 256) return launch_tile<256, 128, 2>(st, p, first_tiles);
+    if (bm == 128) return launch_tile<128, 128, 3>(st, p, first_tiles);
+    return launch_tile<64, 64, 4>(st, p, first_tiles);
 }

@@ -1363,8 +1363,8 @@ int launch_f32_tail(hipStream_t st, const GemmProblem &p, bool edge) {
     if (p.ext || !plan_tail(p, BM, BN, BK, sizeof(float), OCC, g_tail_relaxed, plan)) return launch_f32<BM, BN, BK, WMS, WNS, OCC>(st, p, edge);
     const int sel = (p.op_a ? 0 : 2) | (p.op_b ? 1 : 0);
     int rc = WK_OK;
-    if (plan.first_tile > 0 && BM == 256 && BN == 128 && !edge && gemm_f32_dma_applies(p)) {
-        rc = gemm_f32_dma_launch(st, p, plan.first_tile); // the whole rounds on the direct-to-LDS kernel
+    if (plan.first_tile > 0 && !edge && gemm_f32_dma_applies(p, BM, BN)) {
+        rc = gemm_f32_dma_launch(st, p, BM, BN, plan.first_tile); // the whole rounds on the direct-to-LDS kernel
         if (rc) return rc;
     } else if (plan.first_tile > 0) { // the whole rounds, as the plain variant would run them
 #define WK_CASE(AK, BKC)                                                                                                \
@@ -1392,10 +1392,10 @@ int launch_f32_tail(hipStream_t st, const GemmProblem &p, bool edge) {
 #undef WK_CASE
 }
 
-// the direct-to-LDS kernel where it applies, the register-staged 256 x 128 tile elsewhere
-int launch_f32_dma(hipStream_t st, const GemmProblem &p, bool edge) {
-    if (!edge && gemm_f32_dma_applies(p)) return gemm_f32_dma_launch(st, p);
-    return launch_f32<256, 128, 16, 2, 2, 2>(st, p, edge);
+// the direct-to-LDS kernels where they apply, the register-staged tile of the same size elsewhere
+template <int BM, int BN, int BK, int OCC> int launch_f32_dma(hipStream_t st, const GemmProblem &p, bool edge) {
+    if (gemm_f32_dma_applies(p, BM, BN)) return gemm_f32_dma_launch(st, p, BM, BN); // (checks everything it needs itself)
+    return launch_f32<BM, BN, BK, 2, 2, OCC>(st, p, edge);
 }
 
 struct VariantDesc {
@@ -1416,6 +1416,10 @@ struct VariantDesc {
     const char *tail = nullptr;
     int occ = 0; // work-groups of this tile that share a compute unit (0: not needed)
 };
+bool is_dma_variant(const char *name) { // ...d: k-slabs straight into LDS
+    const size_t n = std::strlen(name);
+    return n && name[n - 1] == 'd';
+}
 enum { SPLIT_NONE = 0, SPLIT_ALL = 1, SPLIT_TAIL = 2 };
 int split_kind_of(const char *name) { // by the name's suffix: ...z splits every tile's k, ...t the tail's
     const size_t n = std::strlen(name);
@@ -1427,7 +1431,14 @@ const VariantDesc k_variants[] = {
      "mfma_f32_256x128t", 2},
     // slabs straight into LDS, three deep; interior shapes only (the cost loop skips it elsewhere):
     // 147.5 against 142.5 TFLOP/s at 8192^3, T,N 145.5 against 136
-    {"mfma_f32_256x128d", WK_F32, 256, 128, 16, 0.973, 0.19, &launch_f32_dma, nullptr, nullptr, nullptr, nullptr, "mfma_f32_256x128t", 2},
+    {"mfma_f32_256x128d", WK_F32, 256, 128, 16, 0.943, 0.08, &launch_f32_dma<256, 128, 16, 2>, nullptr, nullptr, nullptr, nullptr,
+     "mfma_f32_256x128t", 2},
+    // 2048 x 4096 x 4096: N,T 143.0 (staged 139.6), N,N 141.8 (132.0); 4096^3 144
+    {"mfma_f32_128x128d", WK_F32, 128, 128, 16, 0.922, 0.08, &launch_f32_dma<128, 128, 16, 3>, nullptr, nullptr, nullptr, nullptr,
+     "mfma_f32_128x128t", 3},
+    // 3072^3 129.7 (staged 120.4), 2048 x 1024 x 4096 132 (126), 1024^3 103.7 (101.5 with four k-groups)
+    {"mfma_f32_64x64d", WK_F32, 64, 64, 32, 0.84, 0.10, &launch_f32_dma<64, 64, 32, 4>, nullptr, nullptr, "mfma_f32_32x32s4",
+     "mfma_f32_64x64z"},
     {"mfma_f32_256x128t", WK_F32, 256, 128, 16, 0.0, 0.25, &launch_f32_tail<256, 128, 16, 2, 2, 2>, nullptr, nullptr, nullptr, nullptr,
      nullptr, 2}, // whole rounds + a k-split tail
     {"mfma_f32_128x128", WK_F32, 128, 128, 16, 0.897, 0.19, &launch_f32<128, 128, 16, 2, 2, 3>, nullptr, nullptr, nullptr, nullptr,
@@ -1545,7 +1556,7 @@ int wk::gemm_mfma_pick(const GemmProblem &p) {
     for (int v = 0; v < k_num_variants; ++v) {
         const VariantDesc &d = k_variants[v];
         if (d.dtype != p.dtype || d.efficiency <= 0.0) continue;
-        if (d.launch == &launch_f32_dma && (p.ext || !gemm_f32_dma_applies(p))) continue;
+        if (is_dma_variant(d.name) && !gemm_f32_dma_applies(p, d.bm, d.bn)) continue;
         const double tiles = (double)((p.M + d.bm - 1) / d.bm) * (double)((p.N + d.bn - 1) / d.bn);
         // Whole rounds: the big tiles (two or three work-groups per unit) pay for a started round in
         // full, the small tile (four per unit, short) for about two thirds of it.
@@ -1580,9 +1591,12 @@ int wk::gemm_mfma_pick(const GemmProblem &p) {
     // fewer tiles (1536^3) or more than one round (3072^3) the 64x64 tile wins.
     if (p.dtype == WK_F32 && p.K >= 512) {
         const double tiles128 = (double)((p.M + 127) / 128) * (double)((p.N + 127) / 128);
-        if (tiles128 <= cus && tiles128 >= 0.85 * cus)
+        if (tiles128 <= cus && tiles128 >= 0.85 * cus) {
+            // (the direct-to-LDS kernel of that tile where it applies: 2048^3 N,N 131 against 128.5)
+            const char *want = gemm_f32_dma_applies(p, 128, 128) ? "mfma_f32_128x128d" : "mfma_f32_128x128s2";
             for (int v = 0; v < k_num_variants; ++v)
-                if (!std::strcmp(k_variants[v].name, "mfma_f32_128x128s2")) return v;
+                if (!std::strcmp(k_variants[v].name, want)) return v;
+        }
     }
     // A launch of one round (f32: up to two) of the small tile leaves each SIMD one or two wavefronts,
     // which stall together at every hand-over: the k-split twin of the tile gives it two to four.

@@ -217,11 +217,12 @@ int gemm_complex_packed_prepare(hipStream_t st, const GemmProblem &p, void *work
                                 int (*transpose)(void *ctx, int dtype, uint64_t rows, uint64_t cols, const void *src, uint64_t ld,
                                                  void *dst),
                                 void *ctx, GemmProblem &real, void **rest, size_t *rest_bytes);
-// f32, interior shapes only: k-slabs brought straight from global memory into LDS, three deep (wk_gemm_dma.hip)
-bool gemm_f32_dma_applies(const GemmProblem &p);
-// first_tiles: launch only the first so many tiles of the tile walk (0: all), for a product whose other
-// tiles run as a k-split tail
-int gemm_f32_dma_launch(hipStream_t st, const GemmProblem &p, uint64_t first_tiles = 0);
+// f32, interior shapes only: k-slabs brought straight from global memory into LDS, three deep
+// (wk_gemm_dma.hip); macro tiles 256 x 128, 128 x 128 and 64 x 64; the fused bias + activation epilogue
+// (p.ext) for op N, T.  first_tiles: launch only the first so many tiles of the tile walk (0: all), for
+// a product whose other tiles run as a k-split tail.
+bool gemm_f32_dma_applies(const GemmProblem &p, int bm, int bn);
+int gemm_f32_dma_launch(hipStream_t st, const GemmProblem &p, int bm, int bn, uint64_t first_tiles = 0);
 bool gemm_mfma_fuses(const GemmProblem &p, int variant); // variant can run p with the fused bias + activation epilogue
 int gemm_mfma_pick(const GemmProblem &p);        // -1: not applicable
 const char *gemm_mfma_variant_name(int variant); // nullptr past the end
