@@ -49,7 +49,8 @@ def both(dev, dtype, M, N, K, op_a, op_b, kind, with_bias, seed, ld_extra=0):
                                            ("f32", "mfma_f32_64x64s4"), ("f32", "mfma_f32_32x32s4"), ("f32", "mfma_f32_128x128s2"), ("f64", "mfma_f64_64x64s2"), ("f64", "mfma_f64_32x32s4"), ("f32", "mfma_f32_128x128"),
                                            ("f32", "mfma_f32_256x128"), ("f64", "auto"), ("f64", "mfma_f64_64x64"),
                                            ("f64", "mfma_f64_128x64"), ("f64", "mfma_f64_128x128"), ("f32", "tile64"),
-                                           ("f32", "mfma_f32_256x128d"), ("f32", "mfma_f32_128x128d"), ("f32", "mfma_f32_64x64d")])
+                                           ("f32", "mfma_f32_256x128d"), ("f32", "mfma_f32_128x128d"), ("f32", "mfma_f32_64x64d"),
+                                           ("f64", "mfma_f64_128x128d"), ("f64", "mfma_f64_64x64d")])
 @pytest.mark.parametrize("kind", ["none", "sigmoid", "tanh"])
 def test_fused_equals_two_calls(dev, dtype, variant, kind):
     assert dev.lib.wk_gemm_force_variant(variant.encode()) == 0

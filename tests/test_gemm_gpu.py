@@ -91,7 +91,7 @@ def test_f32_every_variant(dev, variant, op_a, op_b):
 
 
 @pytest.mark.parametrize("variant", ["tile64", "mfma_f64_64x64", "mfma_f64_64x64s2", "mfma_f64_32x32s4", "mfma_f64_64x64z",
-                                     "mfma_f64_128x64", "mfma_f64_128x128"])
+                                     "mfma_f64_128x64", "mfma_f64_128x128", "mfma_f64_128x128d", "mfma_f64_64x64d"])
 @pytest.mark.parametrize("op_a,op_b", OPS)
 def test_f64_every_variant(dev, variant, op_a, op_b):
     assert dev.lib.wk_gemm_force_variant(variant.encode()) == 0
@@ -308,8 +308,10 @@ def test_one_round_launches_take_the_k_split_tiles(dev):
     assert name("f32", 2040, 2040, 2040) == b"mfma_f32_128x128s2"
     assert name("f32", 512, 512, 512) == b"mfma_f32_32x32s4"       # 64 tiles of 64x64 would leave most CUs idle
     assert name("f32", 768, 768, 768) == b"mfma_f32_32x32s4"
-    assert name("f64", 1024, 1024, 1024) == b"mfma_f64_64x64s2"
-    assert name("f64", 2048, 2048, 2048) != b"mfma_f64_64x64s2"
+    assert name("f64", 1024, 1024, 1024) == b"mfma_f64_64x64d"
+    assert name("f64", 1000, 1000, 1000) == b"mfma_f64_64x64s2"
+    assert name("f64", 2048, 2048, 2048) == b"mfma_f64_64x64d"
+    assert name("f64", 4096, 4096, 4096) == b"mfma_f64_128x128d"
     assert name("f64", 512, 512, 512) == b"mfma_f64_32x32s4"
     for dtype in ("f32", "f64"):
         for op_a, op_b in OPS:
@@ -369,23 +371,25 @@ def test_k_split_over_work_groups(dev, dtype):
         lib.wk_gemm_force_variant(b"auto")
 
 
-@pytest.mark.parametrize("variant,bm,bn", [("mfma_f32_256x128d", 256, 128), ("mfma_f32_128x128d", 128, 128), ("mfma_f32_64x64d", 64, 64)])
+@pytest.mark.parametrize("variant,bm,bn", [("mfma_f32_256x128d", 256, 128), ("mfma_f32_128x128d", 128, 128), ("mfma_f32_64x64d", 64, 64),
+                                           ("mfma_f64_128x128d", 128, 128), ("mfma_f64_64x64d", 64, 64)])
 @pytest.mark.parametrize("op_a,op_b", OPS)
 def test_slabs_straight_into_lds(dev, variant, bm, bn, op_a, op_b):
     """The kernels that bring their k-slabs from global memory straight into LDS (three stages, swizzled
     layouts): every count of slabs from one to a handful (the pipeline's prologue and its last two
     iterations are special), several tiles, every epilogue, leading dimensions with gaps; against the
     oracle.  Shapes they do not take (ragged, unaligned) fall back to the register-staged tile."""
+    dtype = variant[5:8]
     assert dev.lib.wk_gemm_force_variant(variant.encode()) == 0
     try:
         for K in (16, 32, 48, 64, 80, 96, 112, 128, 256, 1040):
-            check(dev, "f32", bm, bn, K, op_a, op_b, 1.5, 0.5, seed=200 + K)
-        check(dev, "f32", 2 * bm, 3 * bn, 320, op_a, op_b, None, None, seed=231)
-        check(dev, "f32", 3 * bm, 2 * bn, 64, op_a, op_b, 2.0, None, seed=232)
-        check(dev, "f32", 9 * bm, 9 * bn, 176, op_a, op_b, None, -0.25, seed=233)          # 81 tiles, more than one group of tile rows
-        check(dev, "f32", 2 * bm, 2 * bn, 96, op_a, op_b, 1.5, 0.5, seed=234,
+            check(dev, dtype, bm, bn, K, op_a, op_b, 1.5, 0.5, seed=200 + K)
+        check(dev, dtype, 2 * bm, 3 * bn, 320, op_a, op_b, None, None, seed=231)
+        check(dev, dtype, 3 * bm, 2 * bn, 64, op_a, op_b, 2.0, None, seed=232)
+        check(dev, dtype, 9 * bm, 9 * bn, 176, op_a, op_b, None, -0.25, seed=233)          # 81 tiles, more than one group of tile rows
+        check(dev, dtype, 2 * bm, 2 * bn, 96, op_a, op_b, 1.5, 0.5, seed=234,
               lda=(2 * bm if op_a else 96) + 8, ldb=(96 if op_b else 2 * bn) + 12, ldc=2 * bn + 5)  # gaps between rows, 16-byte aligned
-        check(dev, "f32", 300, 200, 100, op_a, op_b, 1.5, 0.5, seed=235)                  # ragged: the staged tile runs
+        check(dev, dtype, 300, 200, 100, op_a, op_b, 1.5, 0.5, seed=235)                  # ragged: the staged tile runs
     finally:
         dev.lib.wk_gemm_force_variant(b"auto")
 

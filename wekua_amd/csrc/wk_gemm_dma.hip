@@ -286,6 +286,320 @@ void gemm_f32_dma_kernel(DArgs g) {
         }
 }
 
+// ------------------------------------------------------------------------------------ f64 ---
+// The same pipeline with v_mfma_f64_16x16x4_f64 (lane l supplies A[l % 16][l / 16] and B[l / 16][l % 16];
+// result register r of lane l is C[4 r + l / 16][l % 16] of its 16 x 16 block).  A 16-byte chunk is two
+// doubles.  Macro tiles 128 x 128 with k-slabs of 8 (three stages of 16 KB, three work-groups per unit)
+// and 64 x 64 with k-slabs of 16 (the same 16 KB).
+//   k-contiguous operand: [row][BK], BK / 2 chunks per row, chunk c of row r at position
+//     c ^ ((r >> 2) & 3) (BK = 8) or c ^ ((r >> 1) & 7) (BK = 16); a fragment is one 16-byte read
+//     (k = 8 s + 2 (lane / 16) + 0..1), sixteen consecutive rows at one logical chunk cover all banks once.
+//   m/n-contiguous operand: [k][ROWS], element (k, m) at m ^ (16 * ((k >> 1) & 1)); fragments are 8-byte
+//     reads, the four quarter-wavefronts read rows k, k + 2, k + 4, k + 6 and the swizzle puts
+//     neighbouring quarters on disjoint banks.
+typedef double f64x2 __attribute__((ext_vector_type(2)));
+typedef double f64x4 __attribute__((ext_vector_type(4)));
+
+struct DArgsD {
+    const double *A, *B;
+    double *C;
+    uint32_t M, N, K;
+    uint32_t lda, ldb, ldc;
+    uint32_t tiles_m, tiles_n;
+    uint32_t num_cus;
+    int epi;
+    double alpha, beta;
+    const double *bias;
+    int act;
+};
+
+__device__ __forceinline__ void dma16d(const double *base, uint32_t byte_offset, uint32_t lds_base) {
+    asm volatile("s_mov_b32 m0, %2\n\t"
+                 "s_nop 0\n\t"
+                 "global_load_lds_dwordx4 %0, %1"
+                 :
+                 : "v"(byte_offset), "s"(base), "s"(lds_base)
+                 : "memory");
+}
+
+template <int BM, int BN, int BK, int OCC, bool A_K, bool B_K, bool EXT>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(OCC)))
+void gemm_f64_dma_kernel(DArgsD g) {
+    constexpr int WM = BM / 2, WN = BN / 2, FM = WM / 16, FN = WN / 16;
+    constexpr int S = BK / 8;     // fragment steps per slab (8 values of k each, two matrix instructions per block)
+    constexpr int CPR = BK / 2;   // 16-byte chunks per row of a k-contiguous slab
+    constexpr int A_DOUBLES = BM * BK, B_DOUBLES = BN * BK, STAGE = A_DOUBLES + B_DOUBLES;
+    constexpr int A_LOADS = BM * BK / 512, B_LOADS = BN * BK / 512; // 1 KB = 128 doubles per wavefront and load
+    static_assert((BK == 8 || BK == 16) && BM % 32 == 0 && BN % 32 == 0 && A_LOADS >= 1 && B_LOADS >= 1, "tile shape");
+
+    extern __shared__ __align__(16) float lds_f[];
+    double *lds = reinterpret_cast<double *>(lds_f); // [3][STAGE]: A then B
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wm = wave >> 1, wn = wave & 1;
+    const int l16 = lane & 15, lq = lane >> 4;
+
+    uint32_t tile_m, tile_n;
+    {
+        const uint32_t pid = blockIdx.x;
+        const uint32_t group_size = GROUP_M * g.tiles_n;
+        const uint32_t group = pid / group_size;
+        const uint32_t first_m = group * GROUP_M;
+        const uint32_t gsz = min(g.tiles_m - first_m, (uint32_t)GROUP_M);
+        const uint32_t in_group = pid - group * group_size;
+        tile_m = first_m + in_group % gsz;
+        tile_n = in_group / gsz;
+    }
+    const uint32_t m0 = tile_m * BM, n0 = tile_n * BN;
+    if (g.num_cus) { // co-resident work-groups of the first dispatch wave start one solo iteration apart
+        const uint32_t slot = blockIdx.x / g.num_cus;
+        if (slot >= 1 && slot < (uint32_t)OCC)
+            for (uint32_t i = 0; i < slot * (FM * FN * BK / 8); ++i) __builtin_amdgcn_s_sleep(2);
+    }
+
+    // ---- global side ----
+    const double *a_base = A_K ? g.A + (size_t)m0 * g.lda : g.A + m0;
+    const double *b_base = B_K ? g.B + (size_t)n0 * g.ldb : g.B + n0;
+    const size_t a_step = A_K ? (size_t)BK : (size_t)BK * g.lda;
+    const size_t b_step = B_K ? (size_t)BK : (size_t)BK * g.ldb;
+    uint32_t a_off[A_LOADS], b_off[B_LOADS];
+    auto lane_offset = [&](int grp, uint32_t ld, auto kc_tag, auto rows_tag) -> uint32_t {
+        constexpr bool KC = decltype(kc_tag)::value;
+        constexpr int ROWS = decltype(rows_tag)::value;
+        if constexpr (KC) {
+            constexpr int RPL = 64 / CPR; // rows per load
+            const uint32_t row = grp * RPL + lane / CPR;
+            const uint32_t swz = CPR == 4 ? (row >> 2) & 3 : (row >> 1) & 7;
+            const uint32_t chunk = (lane % CPR) ^ swz;
+            return (row * ld + 2 * chunk) * 8u;
+        } else {
+            constexpr int PER_ROW = ROWS / 2; // chunks per row of k
+            static_assert(PER_ROW <= 64, "a row of k is at most one load");
+            const uint32_t k = grp * (64 / PER_ROW) + lane / PER_ROW;
+            const uint32_t chunk = (lane % PER_ROW) ^ (((k >> 1) & 1) * 8);
+            return (k * ld + 2 * chunk) * 8u;
+        }
+    };
+    using std::integral_constant;
+#pragma unroll
+    for (int i = 0; i < A_LOADS; ++i) a_off[i] = lane_offset(i * 4 + wave, g.lda, integral_constant<bool, A_K>{}, integral_constant<int, BM>{});
+#pragma unroll
+    for (int i = 0; i < B_LOADS; ++i) b_off[i] = lane_offset(i * 4 + wave, g.ldb, integral_constant<bool, B_K>{}, integral_constant<int, BN>{});
+    const uint32_t lds0 =
+        __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)(__attribute__((address_space(3))) float *)lds_f);
+
+    auto issue = [&](uint32_t stage_bytes) {
+        const uint32_t sbase = lds0 + stage_bytes + (uint32_t)wave * 1024u;
+#pragma unroll
+        for (int i = 0; i < A_LOADS; ++i) dma16d(a_base, a_off[i], sbase + (uint32_t)i * 4096u);
+#pragma unroll
+        for (int i = 0; i < B_LOADS; ++i) dma16d(b_base, b_off[i], sbase + A_DOUBLES * 8u + (uint32_t)i * 4096u);
+        a_base += a_step;
+        b_base += b_step;
+    };
+
+    // ---- LDS side: per-lane fragment addresses in doubles from the start of a stage's A or B part ----
+    // k-contiguous: row * BK + 2 * ((4 s + lq) ^ swz(row)); row = wave offset + 16 i + l16, so swz depends on l16 only
+    const int swz_l = CPR == 4 ? (l16 >> 2) & 3 : (l16 >> 1) & 7;
+    int a_frag[FM], b_frag[FN];
+#pragma unroll
+    for (int i = 0; i < FM; ++i)
+        a_frag[i] = A_K ? (wm * WM + 16 * i + l16) * BK + 2 * (lq ^ swz_l) : 2 * lq * BM + (((wm * WM + 16 * i) ^ (16 * (lq & 1))) + l16);
+#pragma unroll
+    for (int j = 0; j < FN; ++j)
+        b_frag[j] = B_K ? (wn * WN + 16 * j + l16) * BK + 2 * (lq ^ swz_l) : 2 * lq * BN + (((wn * WN + 16 * j) ^ (16 * (lq & 1))) + l16);
+
+    auto read_frags = [&](uint32_t stage_bytes, int s, f64x2 *af, f64x2 *bf) {
+        const double *as = lds + stage_bytes / 8;
+        const double *bs = as + A_DOUBLES;
+#pragma unroll
+        for (int i = 0; i < FM; ++i) {
+            if constexpr (A_K) {
+                // chunk 4 s + lq: the second step's chunk has bit 2 flipped (BK = 16 only)
+                af[i] = *reinterpret_cast<const f64x2 *>(as + (a_frag[i] ^ (s ? 8 : 0)));
+            } else {
+#pragma unroll
+                for (int t = 0; t < 2; ++t) af[i][t] = as[a_frag[i] + (8 * s + t) * BM];
+            }
+        }
+#pragma unroll
+        for (int j = 0; j < FN; ++j) {
+            if constexpr (B_K) {
+                bf[j] = *reinterpret_cast<const f64x2 *>(bs + (b_frag[j] ^ (s ? 8 : 0)));
+            } else {
+#pragma unroll
+                for (int t = 0; t < 2; ++t) bf[j][t] = bs[b_frag[j] + (8 * s + t) * BN];
+            }
+        }
+    };
+
+    f64x4 acc[FM][FN];
+#pragma unroll
+    for (int i = 0; i < FM; ++i)
+#pragma unroll
+        for (int j = 0; j < FN; ++j)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) acc[i][j][r] = 0.0;
+
+    // fragment sets alternate from step to step: step number n (counted over the whole product) uses set n % 2
+    f64x2 af[2][FM], bf[2][FN];
+    auto mfma_step = [&](int set) {
+#pragma unroll
+        for (int t = 0; t < 2; ++t)
+#pragma unroll
+            for (int i = 0; i < FM; ++i)
+#pragma unroll
+                for (int j = 0; j < FN; ++j)
+                    acc[i][j] = __builtin_amdgcn_mfma_f64_16x16x4f64(af[set][i][t], bf[set][j][t], acc[i][j], 0, 0, 0);
+    };
+
+    const uint32_t ktiles = g.K / BK;
+    constexpr uint32_t STAGE_BYTES = STAGE * 8u;
+    uint32_t st_cur = 0, st_next = STAGE_BYTES, st_after = 2 * STAGE_BYTES;
+
+    issue(st_cur);
+    if (ktiles > 1) {
+        issue(st_next);
+        wait_vm<A_LOADS + B_LOADS>();
+    } else {
+        wait_vm<0>();
+    }
+    __builtin_amdgcn_s_barrier();
+    read_frags(st_cur, 0, af[0], bf[0]);
+
+    // One iteration on the slab in st_cur; P: which fragment set holds its first step (a compile-time
+    // constant: with one step per slab the sets swap every iteration).  The hand-over to slab kt+1 (wait
+    // for this wavefront's own loads of it, barrier, first fragments) sits in front of the last step's
+    // matrix instructions, as in the f32 kernel.
+    auto iteration = [&](auto parity_tag, auto more2_tag, auto more1_tag) __attribute__((always_inline)) {
+        constexpr int P = decltype(parity_tag)::value;
+        constexpr bool MORE2 = decltype(more2_tag)::value, MORE1 = decltype(more1_tag)::value;
+        if constexpr (MORE2) issue(st_after);
+#pragma unroll
+        for (int s = 0; s < S; ++s) {
+            const int set = (P + s) & 1;
+            if (s + 1 < S) {
+                read_frags(st_cur, s + 1, af[set ^ 1], bf[set ^ 1]);
+            } else if constexpr (MORE1) {
+                __builtin_amdgcn_sched_barrier(0);
+                if constexpr (MORE2) wait_vm<A_LOADS + B_LOADS>();
+                else wait_vm<0>();
+                wait_lgkm0();
+                __builtin_amdgcn_s_barrier();
+                read_frags(st_next, 0, af[set ^ 1], bf[set ^ 1]);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+            mfma_step(set);
+        }
+        const uint32_t t = st_cur;
+        st_cur = st_next;
+        st_next = st_after;
+        st_after = t;
+    };
+    using T_ = std::true_type;
+    using F_ = std::false_type;
+    using P0 = integral_constant<int, 0>;
+    using P1 = integral_constant<int, 1>;
+    uint32_t kt = 0;
+    if constexpr (S % 2 == 0) { // the first step of every slab uses set 0
+        for (; kt + 2 < ktiles; ++kt) iteration(P0{}, T_{}, T_{});
+        if (kt + 1 < ktiles) iteration(P0{}, F_{}, T_{});
+        iteration(P0{}, F_{}, F_{});
+    } else { // sets alternate with the slabs: two iterations per trip, then the last one or two by parity
+        for (; kt + 3 < ktiles; kt += 2) {
+            iteration(P0{}, T_{}, T_{});
+            iteration(P1{}, T_{}, T_{});
+        }
+        // here kt is even and 1 <= ktiles - kt <= 3
+        if (kt + 2 < ktiles) { // three left
+            iteration(P0{}, T_{}, T_{});
+            iteration(P1{}, F_{}, T_{});
+            iteration(P0{}, F_{}, F_{});
+        } else if (kt + 1 < ktiles) { // two left
+            iteration(P0{}, F_{}, T_{});
+            iteration(P1{}, F_{}, F_{});
+        } else {
+            iteration(P0{}, F_{}, F_{});
+        }
+    }
+
+    const double alpha = g.alpha, beta = g.beta;
+#pragma unroll
+    for (int i = 0; i < FM; ++i)
+#pragma unroll
+        for (int j = 0; j < FN; ++j) {
+            const uint32_t col = n0 + wn * WN + j * 16 + l16;
+            double bias_v = 0.;
+            if constexpr (EXT) {
+                if (g.bias) bias_v = g.bias[col];
+            }
+            double old[4];
+            if (g.epi == EPI_ALPHA_BETA) {
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    const uint32_t row = m0 + wm * WM + i * 16 + 4 * r + lq;
+                    old[r] = g.C[(size_t)row * g.ldc + col];
+                }
+            }
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const uint32_t row = m0 + wm * WM + i * 16 + 4 * r + lq;
+                double v = acc[i][j][r];
+                if (g.epi == EPI_ALPHA) v = alpha * v;
+                else if (g.epi == EPI_ALPHA_BETA) v = alpha * v + beta * old[r];
+                if constexpr (EXT) {
+                    if (g.bias) v += bias_v;
+                    v = act_forward<double>(g.act, v);
+                }
+                g.C[(size_t)row * g.ldc + col] = v;
+            }
+        }
+}
+
+template <int BM, int BN, int BK, int OCC, bool A_K, bool B_K, bool EXT> int launch_one_d(hipStream_t st, const DArgsD &g) {
+    constexpr size_t lds_bytes = 3 * (BM * BK + BN * BK) * sizeof(double);
+    auto kern = gemm_f64_dma_kernel<BM, BN, BK, OCC, A_K, B_K, EXT>;
+    static const int attr_rc = [&] {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                           (int)lds_bytes);
+        if (e != hipSuccess) {
+            (void)hipGetLastError();
+            return hip_code(e);
+        }
+        return (int)WK_OK;
+    }();
+    if (attr_rc) return attr_rc;
+    hipLaunchKernelGGL(kern, dim3(g.tiles_m * g.tiles_n), dim3(256), lds_bytes, st, g);
+    return launch_status();
+}
+
+template <int BM, int BN, int BK, int OCC> int launch_tile_d(hipStream_t st, const GemmProblem &p) {
+    DArgsD g{};
+    g.A = static_cast<const double *>(p.A);
+    g.B = static_cast<const double *>(p.B);
+    g.C = static_cast<double *>(p.C);
+    g.M = (uint32_t)p.M; g.N = (uint32_t)p.N; g.K = (uint32_t)p.K;
+    g.lda = (uint32_t)p.lda; g.ldb = (uint32_t)p.ldb; g.ldc = (uint32_t)p.ldc;
+    g.tiles_m = (uint32_t)(p.M / BM);
+    g.tiles_n = (uint32_t)(p.N / BN);
+    g.num_cus = p.num_cus;
+    g.epi = p.epi;
+    std::memcpy(&g.alpha, p.alpha, sizeof(double));
+    std::memcpy(&g.beta, p.beta, sizeof(double));
+    g.bias = static_cast<const double *>(p.ext_bias);
+    g.act = p.ext_act;
+    const int sel = (p.op_a ? 0 : 2) | (p.op_b ? 1 : 0);
+    if (p.ext) return sel == 3 ? launch_one_d<BM, BN, BK, OCC, true, true, true>(st, g) : (int)WK_E_INVALID_VALUE;
+    switch (sel) {
+    case 0: return launch_one_d<BM, BN, BK, OCC, false, false, false>(st, g);
+    case 1: return launch_one_d<BM, BN, BK, OCC, false, true, false>(st, g);
+    case 2: return launch_one_d<BM, BN, BK, OCC, true, false, false>(st, g);
+    default: return launch_one_d<BM, BN, BK, OCC, true, true, false>(st, g);
+    }
+}
+
 // first_tiles: launch only that many tiles, in tile-walk order (0: all of them)
 template <int BM, int BN, int OCC, bool A_K, bool B_K, bool EXT> int launch_one(hipStream_t st, const DArgs &g, uint64_t first_tiles) {
     constexpr size_t lds_bytes = 3 * (BM * 16 + BN * 16) * sizeof(float); // 72 / 48 / 24 KB
@@ -348,6 +662,25 @@ bool wk::gemm_f32_dma_applies(const GemmProblem &p, int bm, int bn) {
     if (p.lda > (1ull << 21) || p.ldb > (1ull << 21)) return false;
     if ((p.M / bm) * (p.N / bn) > 0x7fffffffull) return false;
     return true;
+}
+
+bool wk::gemm_f64_dma_applies(const GemmProblem &p, int bm, int bn) {
+    if (p.dtype != WK_F64) return false;
+    if (!((bm == 128 && bn == 128) || (bm == 64 && bn == 64))) return false;
+    if (p.ext && (p.op_a || !p.op_b)) return false;
+    if (p.M % bm || p.N % bn || p.K % 16) return false;
+    if (p.lda % 2 || p.ldb % 2) return false;
+    if ((reinterpret_cast<uintptr_t>(p.A) | reinterpret_cast<uintptr_t>(p.B)) & 15u) return false;
+    if (p.M > 0x7fffffffull || p.N > 0x7fffffffull || p.K > 0x7fffffffull || p.ldc > 0x7fffffffull) return false;
+    if (p.lda > (1ull << 20) || p.ldb > (1ull << 20)) return false; // 127 rows * ld * 8 bytes inside 32 bits
+    if ((p.M / bm) * (p.N / bn) > 0x7fffffffull) return false;
+    return true;
+}
+
+int wk::gemm_f64_dma_launch(hipStream_t st, const GemmProblem &p, int bm, int bn) {
+    if (!gemm_f64_dma_applies(p, bm, bn)) return WK_E_INVALID_VALUE;
+    if (bm == 128) return launch_tile_d<128, 128, 8, 2>(st, p); // (128 accumulator + 64 fragment registers: two per SIMD)
+    return launch_tile_d<64, 64, 16, 3>(st, p);
 }
 
 int wk::gemm_f32_dma_launch(hipStream_t st, const GemmProblem &p, int bm, int bn, uint64_t first_tiles) {

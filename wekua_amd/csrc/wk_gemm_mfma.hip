@@ -1398,6 +1398,11 @@ template <int BM, int BN, int BK, int OCC> int launch_f32_dma(hipStream_t st, co
     return launch_f32<BM, BN, BK, 2, 2, OCC>(st, p, edge);
 }
 
+template <int BM, int BN, int BK, int OCC> int launch_f64_dma(hipStream_t st, const GemmProblem &p, bool edge) {
+    if (gemm_f64_dma_applies(p, BM, BN)) return gemm_f64_dma_launch(st, p, BM, BN);
+    return launch_f64<BM, BN, BK, 2, 2, OCC>(st, p, edge);
+}
+
 struct VariantDesc {
     const char *name;
     int dtype, bm, bn, bk; // bk: k values per LDS slab
@@ -1455,6 +1460,10 @@ const VariantDesc k_variants[] = {
     {"mfma_f64_128x128", WK_F64, 128, 128, 16, 0.908, 0.20, &launch_f64<128, 128, 16, 2, 2, 2>},
     {"mfma_f64_64x64", WK_F64, 64, 64, 32, 0.840, 0.05, &launch_f64<64, 64, 32, 2, 2, 2>, "mfma_f64_64x64s2", nullptr,
      "mfma_f64_32x32s4", "mfma_f64_64x64z"},
+    // slabs straight into LDS, three deep (wk_gemm_dma.hip), interior shapes: 4096^3 70.2 against 68.5 TFLOP/s
+    {"mfma_f64_128x128d", WK_F64, 128, 128, 16, 0.91, 0.10, &launch_f64_dma<128, 128, 16, 2>},
+    // 8192 x 256 x 8192 69.6 (staged 62.2), 2048^3 68 (61.7), 4096^3 69-70.5
+    {"mfma_f64_64x64d", WK_F64, 64, 64, 32, 0.89, 0.05, &launch_f64_dma<64, 64, 32, 2>, nullptr, nullptr, "mfma_f64_32x32s4", "mfma_f64_64x64z"},
     {"mfma_f64_64x64z", WK_F64, 64, 64, 32, 0.0, 0.05, &launch_f64_split64}, // k split over work-groups
     {"mfma_f64_64x64s2", WK_F64, 64, 64, 64, 0.0, 0.05, &launch_f64<64, 64, 32, 2, 2, 2, 2>}, // 2 groups x 32 k
     // (two wavefronts per SIMD: with a 128-register budget its staging sets and fragments spill and it
@@ -1556,7 +1565,8 @@ int wk::gemm_mfma_pick(const GemmProblem &p) {
     for (int v = 0; v < k_num_variants; ++v) {
         const VariantDesc &d = k_variants[v];
         if (d.dtype != p.dtype || d.efficiency <= 0.0) continue;
-        if (is_dma_variant(d.name) && !gemm_f32_dma_applies(p, d.bm, d.bn)) continue;
+        if (is_dma_variant(d.name) && !(d.dtype == WK_F64 ? gemm_f64_dma_applies(p, d.bm, d.bn) : gemm_f32_dma_applies(p, d.bm, d.bn)))
+            continue;
         const double tiles = (double)((p.M + d.bm - 1) / d.bm) * (double)((p.N + d.bn - 1) / d.bn);
         // Whole rounds: the big tiles (two or three work-groups per unit) pay for a started round in
         // full, the small tile (four per unit, short) for about two thirds of it.

@@ -223,6 +223,9 @@ int gemm_complex_packed_prepare(hipStream_t st, const GemmProblem &p, void *work
 // a product whose other tiles run as a k-split tail.
 bool gemm_f32_dma_applies(const GemmProblem &p, int bm, int bn);
 int gemm_f32_dma_launch(hipStream_t st, const GemmProblem &p, int bm, int bn, uint64_t first_tiles = 0);
+// the same for f64: macro tiles 128 x 128 (k-slabs of 8) and 64 x 64 (k-slabs of 16)
+bool gemm_f64_dma_applies(const GemmProblem &p, int bm, int bn);
+int gemm_f64_dma_launch(hipStream_t st, const GemmProblem &p, int bm, int bn);
 bool gemm_mfma_fuses(const GemmProblem &p, int variant); // variant can run p with the fused bias + activation epilogue
 int gemm_mfma_pick(const GemmProblem &p);        // -1: not applicable
 const char *gemm_mfma_variant_name(int variant); // nullptr past the end
