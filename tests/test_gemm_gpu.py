@@ -394,6 +394,21 @@ def test_slabs_straight_into_lds(dev, variant, bm, bn, op_a, op_b):
         dev.lib.wk_gemm_force_variant(b"auto")
 
 
+@pytest.mark.parametrize("variant,bm,bn", [("mfma_f32_256x128d", 256, 128), ("mfma_f32_128x128d", 128, 128), ("mfma_f32_64x64d", 64, 64)])
+def test_tile_walk_in_patches_covers_every_tile_once(dev, variant, bm, bn):
+    """The f32 direct-to-LDS kernels number their tiles in XCD-local patches (4 x 8, 4 x 4, 2 x 8 or 2 x 4
+    tiles, eight patches at a time) when the tile grid divides into them and in groups of tile rows
+    otherwise: one tile grid per patch shape and one that takes none, whole result against the oracle
+    (a tile visited twice or not at all leaves entries of C wrong)."""
+    assert dev.lib.wk_gemm_force_variant(variant.encode()) == 0
+    try:
+        for tiles_m, tiles_n in ((8, 32), (8, 16), (2, 64), (2, 32), (16, 16), (6, 10)):
+            for op_a, op_b in ((0, 0), (1, 1)):
+                check(dev, "f32", tiles_m * bm, tiles_n * bn, 48, op_a, op_b, None, None, seed=300 + tiles_m + tiles_n)
+    finally:
+        dev.lib.wk_gemm_force_variant(b"auto")
+
+
 def test_left_over_tiles_run_as_a_k_split_tail(dev):
     """A launch whose tiles do not fill whole rounds of the compute units: the whole rounds run as they
     are, the left-over tiles as a second launch with k split over work-groups.  Checked: the plan of the

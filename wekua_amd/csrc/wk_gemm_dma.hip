@@ -29,6 +29,7 @@
 // are needed are written out instead (vmcnt before the barrier that publishes a slab).
 #include "wk_internal.hpp"
 
+#include <cstdlib>
 #include <cstring>
 
 using namespace wk;
@@ -51,6 +52,7 @@ struct DArgs {
     float alpha, beta;
     const float *bias; // kernels instantiated with EXT: C = act(acc + bias[col]); bias may be null
     int act;
+    uint32_t patch_m, patch_n; // tile walk in XCD-local patches of patch_m x patch_n tiles (0: rows of groups)
 };
 
 // 16 bytes per lane from global memory (scalar base + 32-bit byte offset per lane) to LDS at
@@ -85,7 +87,17 @@ void gemm_f32_dma_kernel(DArgs g) {
 
     // tile walk: groups of GROUP_M tile rows, as in wk_gemm_mfma.hip (every XCD sweeps the same panel of B)
     uint32_t tile_m, tile_n;
-    {
+    if (g.patch_m) {
+        // work-group b runs on XCD b % 8: the j-th work-group of an XCD takes tile j % (patch) of that
+        // XCD's patch j / (patch), so the tiles that share an L2 at one time share rows of A and columns of B
+        const uint32_t pid = blockIdx.x;
+        const uint32_t x = pid & 7u, j = pid >> 3;
+        const uint32_t per_patch = g.patch_m * g.patch_n;
+        const uint32_t patch = (j / per_patch) * 8u + x, q = j % per_patch;
+        const uint32_t patches_n = g.tiles_n / g.patch_n;
+        tile_m = (patch / patches_n) * g.patch_m + q % g.patch_m;
+        tile_n = (patch % patches_n) * g.patch_n + q / g.patch_m;
+    } else {
         const uint32_t pid = blockIdx.x;
         const uint32_t group_size = GROUP_M * g.tiles_n;
         const uint32_t group = pid / group_size;
@@ -289,8 +301,9 @@ void gemm_f32_dma_kernel(DArgs g) {
 // ------------------------------------------------------------------------------------ f64 ---
 // The same pipeline with v_mfma_f64_16x16x4_f64 (lane l supplies A[l % 16][l / 16] and B[l / 16][l % 16];
 // result register r of lane l is C[4 r + l / 16][l % 16] of its 16 x 16 block).  A 16-byte chunk is two
-// doubles.  Macro tiles 128 x 128 with k-slabs of 8 (three stages of 16 KB, three work-groups per unit)
-// and 64 x 64 with k-slabs of 16 (the same 16 KB).
+// doubles.  Macro tiles 128 x 128 with k-slabs of 8 (three stages of 16 KB; two work-groups per unit: 128
+// accumulator and 64 fragment registers do not fit the 168 of three) and 64 x 64 with k-slabs of 16 (the
+// same 16 KB, three work-groups per unit).
 //   k-contiguous operand: [row][BK], BK / 2 chunks per row, chunk c of row r at position
 //     c ^ ((r >> 2) & 3) (BK = 8) or c ^ ((r >> 1) & 7) (BK = 16); a fragment is one 16-byte read
 //     (k = 8 s + 2 (lane / 16) + 0..1), sixteen consecutive rows at one logical chunk cover all banks once.
@@ -635,6 +648,21 @@ template <int BM, int BN, int OCC> int launch_tile(hipStream_t st, const GemmPro
     std::memcpy(&g.beta, p.beta, sizeof(float));
     g.bias = static_cast<const float *>(p.ext_bias);
     g.act = p.ext_act;
+    // XCD-local patches where the tile grid divides into them, eight patches at a time (one per XCD);
+    // the k-split tail numbers its tiles in the row-group order, so a body launch keeps that order
+    static const bool row_walk = [] {
+        const char *e = std::getenv("WK_GEMM_WALK");
+        return e && std::strcmp(e, "rows") == 0;
+    }();
+    if (!first_tiles && !row_walk) {
+        static const unsigned shapes[][2] = {{4, 8}, {4, 4}, {2, 8}, {2, 4}};
+        for (const auto &sh : shapes)
+            if (g.tiles_m % sh[0] == 0 && g.tiles_n % sh[1] == 0 && ((g.tiles_m / sh[0]) * (g.tiles_n / sh[1])) % 8 == 0) {
+                g.patch_m = sh[0];
+                g.patch_n = sh[1];
+                break;
+            }
+    }
     const int sel = (p.op_a ? 0 : 2) | (p.op_b ? 1 : 0); // bit 1: A k-contiguous, bit 0: B k-contiguous
     if (p.ext) // instantiated for op N, T only (what Linear.forward runs)
         return sel == 3 ? launch_one<BM, BN, OCC, true, true, true>(st, g, first_tiles) : (int)WK_E_INVALID_VALUE;
