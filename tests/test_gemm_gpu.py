@@ -293,19 +293,21 @@ def test_one_round_launches_take_the_k_split_tiles(dev):
     def name(dtype, M, N, K):
         return dev.lib.wk_gemm_variant(raw.dtype_id(dtype), 0, 0, M, N, K, K, N, N, None, None, None)
     # (the name query assumes 256 compute units and 16-byte aligned operands)
-    # interior f32 shapes take the kernels that bring their slabs straight into LDS, whose three stages
-    # already give a lone work-group something to overlap with ...
+    # f32 operands whose rows start on 16-byte boundaries take the kernels that bring their slabs straight
+    # into LDS, whose three stages already give a lone work-group something to overlap with ...
     assert name("f32", 1024, 1024, 1024) == b"mfma_f32_64x64d"
     assert name("f32", 2048, 1024, 1024) == b"mfma_f32_64x64d"
     assert name("f32", 1024, 1024, 128) == b"mfma_f32_64x64d"
     assert name("f32", 896, 896, 896) == b"mfma_f32_64x64d"
     assert name("f32", 2048, 2048, 2048) == b"mfma_f32_128x128d"   # one full round of 128x128 tiles
     assert name("f32", 1536, 1536, 1536) == b"mfma_f32_64x64d"
-    # ... ragged ones the register-staged tile and its k-split twins
-    assert name("f32", 1000, 1000, 1000) == b"mfma_f32_64x64s4"
-    assert name("f32", 2040, 1000, 1000) == b"mfma_f32_64x64s2"
-    assert name("f32", 1000, 1000, 100) == b"mfma_f32_64x64"
-    assert name("f32", 2040, 2040, 2040) == b"mfma_f32_128x128s2"
+    assert name("f32", 1000, 1000, 1000) == b"mfma_f32_64x64d"     # ragged, rows of 4000 bytes
+    assert name("f32", 2040, 2040, 2040) == b"mfma_f32_128x128d"
+    # ... any other leading dimension the register-staged tile and its k-split twins
+    assert name("f32", 1001, 1001, 1001) == b"mfma_f32_64x64s4"
+    assert name("f32", 2041, 1001, 1001) == b"mfma_f32_64x64s2"
+    assert name("f32", 1001, 1001, 101) == b"mfma_f32_64x64"
+    assert name("f32", 2042, 2042, 2042) == b"mfma_f32_128x128s2"
     assert name("f32", 512, 512, 512) == b"mfma_f32_32x32s4"       # 64 tiles of 64x64 would leave most CUs idle
     assert name("f32", 768, 768, 768) == b"mfma_f32_32x32s4"
     assert name("f64", 1024, 1024, 1024) == b"mfma_f64_64x64d"
@@ -317,6 +319,7 @@ def test_one_round_launches_take_the_k_split_tiles(dev):
         for op_a, op_b in OPS:
             check(dev, dtype, 1024, 960, 300, op_a, op_b, 1.5, 0.5, seed=93)
             check(dev, dtype, 1000, 1000, 257, op_a, op_b, None, None, seed=94)
+            check(dev, dtype, 1001, 999, 257, op_a, op_b, 1.5, 0.5, seed=96)
             check(dev, dtype, 500, 333, 129, op_a, op_b, 2.0, None, seed=95)
 
 
@@ -389,7 +392,18 @@ def test_slabs_straight_into_lds(dev, variant, bm, bn, op_a, op_b):
         check(dev, dtype, 9 * bm, 9 * bn, 176, op_a, op_b, None, -0.25, seed=233)          # 81 tiles, more than one group of tile rows
         check(dev, dtype, 2 * bm, 2 * bn, 96, op_a, op_b, 1.5, 0.5, seed=234,
               lda=(2 * bm if op_a else 96) + 8, ldb=(96 if op_b else 2 * bn) + 12, ldc=2 * bn + 5)  # gaps between rows, 16-byte aligned
-        check(dev, dtype, 300, 200, 100, op_a, op_b, 1.5, 0.5, seed=235)                  # ragged: the staged tile runs
+        check(dev, dtype, 300, 200, 100, op_a, op_b, 1.5, 0.5, seed=235)                  # ragged (f64: the staged tile runs)
+        if dtype == "f32":
+            # ragged in every dimension: border tiles fetch clamped rows and skip stores, the last slab is
+            # zero-filled in LDS beyond K; K below, at and around the slab size, one to three slabs and many
+            for K in (1, 3, 4, 15, 17, 31, 33, 47, 50, 100, 1001):
+                check(dev, dtype, bm + 1, 2 * bn - 3, K, op_a, op_b, 1.5, 0.5, seed=240 + K)
+            check(dev, dtype, 2 * bm + 7, bn + 5, 61, op_a, op_b, None, None, seed=251)
+            check(dev, dtype, 3, 5, 37, op_a, op_b, 2.0, None, seed=252)                  # smaller than one 16-byte chunk
+            check(dev, dtype, bm - 1, bn - 1, 16, op_a, op_b, None, -0.25, seed=253)
+            # rows that do not start on 16-byte boundaries: not this kernel's, the staged tile runs
+            check(dev, dtype, 2 * bm, bn, 40, op_a, op_b, 1.5, 0.5, seed=254,
+                  lda=(2 * bm if op_a else 40) + 3, ldb=(40 if op_b else bn) + 1, ldc=bn + 2)
     finally:
         dev.lib.wk_gemm_force_variant(b"auto")
 

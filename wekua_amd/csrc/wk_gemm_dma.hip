@@ -3,8 +3,9 @@
 //
 // Same tiling and matrix-instruction mapping as the kernels of wk_gemm_mfma.hip
 // (v_mfma_f32_32x32x2_f32, 2 x 2 wavefronts, macro tiles 256 x 128, 128 x 128 and 64 x 64, k-slab 16),
-// for the interior case only: M % BM == N % BN == K % 16 == 0 and 16-byte aligned rows.  What differs is how a slab
-// gets into LDS and how the work-group hands over from one slab to the next:
+// for operands whose rows start on 16-byte boundaries (f32: any M, N, K; f64: whole tiles and whole
+// k-slabs only).  What differs is how a slab gets into LDS and how the work-group hands over from one
+// slab to the next:
 //   * no staging registers and no LDS stores: every lane names 16 bytes of global memory and the
 //     load unit writes them to LDS at (wave-uniform base) + 16 * lane.  The lane -> address map is
 //     free, the LDS side is not, so padding is replaced by swizzling: the lane that fills LDS
@@ -124,25 +125,30 @@ void gemm_f32_dma_kernel(DArgs g) {
     uint32_t a_off[A_LOADS], b_off[B_LOADS];
     // load i of this wavefront fills the 1 KB group i * 4 + wave of the operand's slab: sixteen rows of a
     // k-contiguous operand, 256 / ROWS rows of k of an m-contiguous one
-    auto lane_offset = [&](int grp, uint32_t ld, auto kc_tag, auto rows_tag) -> uint32_t {
+    // Rows (columns) of the tile beyond the matrix are fetched from its last row (column): they only feed
+    // entries of C that are never stored.  A 16-byte chunk whose first float exists is fetched as it is:
+    // bases and leading dimensions are multiples of 16 bytes, so the chunk cannot leave the page of
+    // that float.  `last` = index of the last existing row (column) counted from the tile's origin.
+    auto lane_offset = [&](int grp, uint32_t ld, uint32_t last, auto kc_tag, auto rows_tag) -> uint32_t {
         constexpr bool KC = decltype(kc_tag)::value;
         constexpr int ROWS = decltype(rows_tag)::value;
         if constexpr (KC) {
             const uint32_t row = grp * 16 + (lane >> 2);
             const uint32_t chunk = (lane & 3) ^ ((row >> 2) & 3);
-            return (row * ld + 4 * chunk) * 4u;
+            return (min(row, last) * ld + 4 * chunk) * 4u;
         } else {
             constexpr int PER_ROW = ROWS / 4; // 16-byte chunks per row of k
             const uint32_t k = grp * (64 / PER_ROW) + lane / PER_ROW;
             const uint32_t chunk = (lane % PER_ROW) ^ (((k >> 2) & 1) * 8);
-            return (k * ld + 4 * chunk) * 4u;
+            return (k * ld + 4 * min(chunk, last >> 2)) * 4u;
         }
     };
     using std::integral_constant;
+    const uint32_t m_last = g.M - 1 - m0, n_last = g.N - 1 - n0;
 #pragma unroll
-    for (int i = 0; i < A_LOADS; ++i) a_off[i] = lane_offset(i * 4 + wave, g.lda, integral_constant<bool, A_K>{}, integral_constant<int, BM>{});
+    for (int i = 0; i < A_LOADS; ++i) a_off[i] = lane_offset(i * 4 + wave, g.lda, m_last, integral_constant<bool, A_K>{}, integral_constant<int, BM>{});
 #pragma unroll
-    for (int i = 0; i < B_LOADS; ++i) b_off[i] = lane_offset(i * 4 + wave, g.ldb, integral_constant<bool, B_K>{}, integral_constant<int, BN>{});
+    for (int i = 0; i < B_LOADS; ++i) b_off[i] = lane_offset(i * 4 + wave, g.ldb, n_last, integral_constant<bool, B_K>{}, integral_constant<int, BN>{});
     const uint32_t lds0 =
         __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)(__attribute__((address_space(3))) float *)lds); // byte address of the array
 
@@ -156,6 +162,53 @@ void gemm_f32_dma_kernel(DArgs g) {
         for (int i = 0; i < B_LOADS; ++i) dma16(b_base, b_off[i], sbase + A_FLOATS * 4u + (uint32_t)i * 4096u);
         a_base += a_step;
         b_base += b_step;
+    };
+
+    // ---- the last slab when K is not a multiple of 16: krem = K % 16 of its k values exist ----
+    // Chunks (k-contiguous operand) or rows of k (m-contiguous) that lie wholly beyond K are fetched from
+    // the last existing one instead; once a wavefront's own loads of that slab have landed it writes
+    // zeros over every float of its share whose k does not exist (products with them must vanish).
+    const uint32_t krem = g.K & 15u;
+    auto tail_offset = [&](uint32_t off, int grp, uint32_t ld, auto kc_tag, auto rows_tag) -> uint32_t {
+        constexpr bool KC = decltype(kc_tag)::value;
+        constexpr int ROWS = decltype(rows_tag)::value;
+        if constexpr (KC) {
+            const uint32_t row = grp * 16 + (lane >> 2);
+            const uint32_t chunk = (lane & 3) ^ ((row >> 2) & 3);
+            return 4 * chunk >= krem ? off - 16u * chunk : off; // chunk 0 of the row always has a float (krem >= 1)
+        } else {
+            constexpr int PER_ROW = ROWS / 4;
+            const uint32_t k = grp * (64 / PER_ROW) + lane / PER_ROW;
+            return k >= krem ? off - (k - (krem - 1)) * ld * 4u : off;
+        }
+    };
+    auto tail_offsets = [&]() {
+#pragma unroll
+        for (int i = 0; i < A_LOADS; ++i) a_off[i] = tail_offset(a_off[i], i * 4 + wave, g.lda, integral_constant<bool, A_K>{}, integral_constant<int, BM>{});
+#pragma unroll
+        for (int i = 0; i < B_LOADS; ++i) b_off[i] = tail_offset(b_off[i], i * 4 + wave, g.ldb, integral_constant<bool, B_K>{}, integral_constant<int, BN>{});
+    };
+    auto tail_zero = [&](float *dst, int grp, auto kc_tag, auto rows_tag) { // dst: this lane's 16 bytes of the load
+        constexpr bool KC = decltype(kc_tag)::value;
+        constexpr int ROWS = decltype(rows_tag)::value;
+        if constexpr (KC) {
+            const uint32_t row = grp * 16 + (lane >> 2);
+            const uint32_t chunk = (lane & 3) ^ ((row >> 2) & 3);
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+                if (4 * chunk + e >= krem) dst[e] = 0.f;
+        } else {
+            constexpr int PER_ROW = ROWS / 4;
+            const uint32_t k = grp * (64 / PER_ROW) + lane / PER_ROW;
+            if (k >= krem) *reinterpret_cast<f32x4 *>(dst) = f32x4{0.f, 0.f, 0.f, 0.f};
+        }
+    };
+    auto tail_zeros = [&](uint32_t stage_bytes) {
+        float *base = lds + stage_bytes / 4 + wave * 256 + lane * 4;
+#pragma unroll
+        for (int i = 0; i < A_LOADS; ++i) tail_zero(base + i * 1024, i * 4 + wave, integral_constant<bool, A_K>{}, integral_constant<int, BM>{});
+#pragma unroll
+        for (int i = 0; i < B_LOADS; ++i) tail_zero(base + A_FLOATS + i * 1024, i * 4 + wave, integral_constant<bool, B_K>{}, integral_constant<int, BN>{});
     };
 
     // ---- LDS side: per-lane fragment addresses (floats from the start of a stage's A or B part) ----
@@ -213,19 +266,25 @@ void gemm_f32_dma_kernel(DArgs g) {
                     acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(af[s & 1][i][t], bf[s & 1][j][t], acc[i][j], 0, 0, 0);
     };
 
-    const uint32_t ktiles = g.K / BK;
+    const uint32_t ktiles = (g.K + BK - 1) / BK;
 
     // The three stages rotate: the slab being multiplied, the next one, and the one after it (byte offsets).
     constexpr uint32_t STAGE_BYTES = STAGE * 4u;
     uint32_t st_cur = 0, st_next = STAGE_BYTES, st_after = 2 * STAGE_BYTES;
 
     // prologue: slabs 0 and 1 on their way, slab 0 landed everywhere, first fragments read
+    if (ktiles == 1 && krem) tail_offsets();
     issue(st_cur);
     if (ktiles > 1) {
+        if (ktiles == 2 && krem) tail_offsets();
         issue(st_next);
         wait_vm<A_LOADS + B_LOADS>();
     } else {
         wait_vm<0>();
+        if (krem) {
+            tail_zeros(st_cur);
+            wait_lgkm0();
+        }
     }
     __builtin_amdgcn_s_barrier();
     read_frags(st_cur, 0, af[0], bf[0]);
@@ -242,8 +301,12 @@ void gemm_f32_dma_kernel(DArgs g) {
         mfma_step(0);
         if constexpr (MORE1) {
             __builtin_amdgcn_sched_barrier(0);
-            if constexpr (MORE2) wait_vm<A_LOADS + B_LOADS>();
-            else wait_vm<0>();
+            if constexpr (MORE2) {
+                wait_vm<A_LOADS + B_LOADS>();
+            } else {
+                wait_vm<0>();
+                if (krem) tail_zeros(st_next); // slab kt+1 is the last one
+            }
             wait_lgkm0();
             __builtin_amdgcn_s_barrier();
             read_frags(st_next, 0, af[0], bf[0]);
@@ -258,44 +321,56 @@ void gemm_f32_dma_kernel(DArgs g) {
     using T_ = std::true_type;
     using F_ = std::false_type;
     uint32_t kt = 0;
-    for (; kt + 2 < ktiles; ++kt) iteration(T_{}, T_{}); // steady state: both following slabs exist
+    for (; kt + 3 < ktiles; ++kt) iteration(T_{}, T_{}); // steady state: both following slabs exist
+    if (kt + 2 < ktiles) {                               // the iteration that requests the last slab
+        if (krem) tail_offsets();
+        iteration(T_{}, T_{});
+        ++kt;
+    }
     if (kt + 1 < ktiles) iteration(F_{}, T_{});          // the last but one
     iteration(F_{}, F_{});                               // the last
 
     // ---- epilogue: acc register r of lane l is C[8*(r/4) + 4*(l/32) + r%4][l%32] of its 32x32 block;
     // option semantics of src/blas/gemm.zig:500-501,591-602 (C_old is read and multiplied whenever beta
     // is given); the reads of C_old of a block are issued as one batch
+    // Tiles that reach beyond C clamp the addresses of C_old and the bias and skip the stores there.
     const float alpha = g.alpha, beta = g.beta;
+    auto epilogue = [&](auto checked_tag) {
+        constexpr bool CHECKED = decltype(checked_tag)::value;
 #pragma unroll
-    for (int i = 0; i < FM; ++i)
+        for (int i = 0; i < FM; ++i)
 #pragma unroll
-        for (int j = 0; j < FN; ++j) {
-            const uint32_t col = n0 + wn * WN + j * 32 + l32;
-            float bias_v = 0.f;
-            if constexpr (EXT) {
-                if (g.bias) bias_v = g.bias[col];
-            }
-            float old[16];
-            if (g.epi == EPI_ALPHA_BETA) {
+            for (int j = 0; j < FN; ++j) {
+                const uint32_t col = n0 + wn * WN + j * 32 + l32;
+                const uint32_t colc = CHECKED ? min(col, g.N - 1) : col;
+                float bias_v = 0.f;
+                if constexpr (EXT) {
+                    if (g.bias) bias_v = g.bias[colc];
+                }
+                float old[16];
+                if (g.epi == EPI_ALPHA_BETA) {
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) {
+                        const uint32_t row = m0 + wm * WM + i * 32 + 8 * (r / 4) + 4 * lhi + (r % 4);
+                        old[r] = g.C[(size_t)(CHECKED ? min(row, g.M - 1) : row) * g.ldc + colc];
+                    }
+                }
 #pragma unroll
                 for (int r = 0; r < 16; ++r) {
                     const uint32_t row = m0 + wm * WM + i * 32 + 8 * (r / 4) + 4 * lhi + (r % 4);
-                    old[r] = g.C[(size_t)row * g.ldc + col];
+                    float v = acc[i][j][r];
+                    if (g.epi == EPI_ALPHA) v = alpha * v;
+                    else if (g.epi == EPI_ALPHA_BETA) v = alpha * v + beta * old[r];
+                    if constexpr (EXT) { // the fused epilogue of Linear.forward, as in wk_gemm_mfma.hip
+                        if (g.bias) v += bias_v;
+                        v = act_forward<float>(g.act, v);
+                    }
+                    if (!CHECKED || (row < g.M && col < g.N)) g.C[(size_t)row * g.ldc + col] = v;
                 }
             }
-#pragma unroll
-            for (int r = 0; r < 16; ++r) {
-                const uint32_t row = m0 + wm * WM + i * 32 + 8 * (r / 4) + 4 * lhi + (r % 4);
-                float v = acc[i][j][r];
-                if (g.epi == EPI_ALPHA) v = alpha * v;
-                else if (g.epi == EPI_ALPHA_BETA) v = alpha * v + beta * old[r];
-                if constexpr (EXT) { // the fused epilogue of Linear.forward, as in wk_gemm_mfma.hip
-                    if (g.bias) v += bias_v;
-                    v = act_forward<float>(g.act, v);
-                }
-                g.C[(size_t)row * g.ldc + col] = v;
-            }
-        }
+    };
+    if (m0 + BM <= g.M && n0 + BN <= g.N) epilogue(std::false_type{});
+    else epilogue(std::true_type{});
 }
 
 // ------------------------------------------------------------------------------------ f64 ---
@@ -306,7 +381,10 @@ void gemm_f32_dma_kernel(DArgs g) {
 // same 16 KB, three work-groups per unit).
 //   k-contiguous operand: [row][BK], BK / 2 chunks per row, chunk c of row r at position
 //     c ^ ((r >> 2) & 3) (BK = 8) or c ^ ((r >> 1) & 7) (BK = 16); a fragment is one 16-byte read
-//     (k = 8 s + 2 (lane / 16) + 0..1), sixteen consecutive rows at one logical chunk cover all banks once.
+//     (row = lane % 16, k = 8 s + 2 (lane / 16) + 0..1), sixteen consecutive rows at one logical chunk cover
+//     all banks once.  (For BK = 8 the bank-conflict counter still shows four cycles per such read, also
+//     with bits 2 and 3 of r exchanged in the swizzle; for BK = 16 and in the f32 kernels it shows none.
+//     That is 1.4 % of the kernel's clocks.)
 //   m/n-contiguous operand: [k][ROWS], element (k, m) at m ^ (16 * ((k >> 1) & 1)); fragments are 8-byte
 //     reads, the four quarter-wavefronts read rows k, k + 2, k + 4, k + 6 and the swizzle puts
 //     neighbouring quarters on disjoint banks.
@@ -633,15 +711,15 @@ template <int BM, int BN, int OCC, bool A_K, bool B_K, bool EXT> int launch_one(
 }
 
 template <int BM, int BN, int OCC> int launch_tile(hipStream_t st, const GemmProblem &p, uint64_t first_tiles) {
-    if (first_tiles > (p.M / BM) * (p.N / BN)) return WK_E_INVALID_VALUE;
+    if (first_tiles > ((p.M + BM - 1) / BM) * ((p.N + BN - 1) / BN)) return WK_E_INVALID_VALUE;
     DArgs g{};
     g.A = static_cast<const float *>(p.A);
     g.B = static_cast<const float *>(p.B);
     g.C = static_cast<float *>(p.C);
     g.M = (uint32_t)p.M; g.N = (uint32_t)p.N; g.K = (uint32_t)p.K;
     g.lda = (uint32_t)p.lda; g.ldb = (uint32_t)p.ldb; g.ldc = (uint32_t)p.ldc;
-    g.tiles_m = (uint32_t)(p.M / BM);
-    g.tiles_n = (uint32_t)(p.N / BN);
+    g.tiles_m = (uint32_t)((p.M + BM - 1) / BM);
+    g.tiles_n = (uint32_t)((p.N + BN - 1) / BN);
     g.num_cus = p.num_cus;
     g.epi = p.epi;
     std::memcpy(&g.alpha, p.alpha, sizeof(float));
@@ -676,19 +754,20 @@ template <int BM, int BN, int OCC> int launch_tile(hipStream_t st, const GemmPro
 
 } // namespace
 
-// What the kernels take for granted, checked on the host: whole tiles, whole k-slabs, 16-byte aligned
-// rows, every per-lane byte offset inside 32 bits, and for the fused epilogue the one layout it exists for.
+// What the kernels take for granted, checked on the host: 16-byte aligned rows (f64: also whole tiles and
+// whole k-slabs), every per-lane byte offset inside 32 bits, and for the fused epilogue the one layout it
+// exists for.
 bool wk::gemm_f32_dma_applies(const GemmProblem &p, int bm, int bn) {
     if (p.dtype != WK_F32) return false;
     if (!((bm == 256 && bn == 128) || (bm == 128 && bn == 128) || (bm == 64 && bn == 64))) return false;
     if (p.ext && (p.op_a || !p.op_b)) return false;
-    if (p.M % bm || p.N % bn || p.K % 16) return false;
+    if (!p.M || !p.N || !p.K) return false;
     if (p.lda % 4 || p.ldb % 4) return false;
     if ((reinterpret_cast<uintptr_t>(p.A) | reinterpret_cast<uintptr_t>(p.B)) & 15u) return false;
     if (p.M > 0x7fffffffull || p.N > 0x7fffffffull || p.K > 0x7fffffffull || p.ldc > 0x7fffffffull) return false;
     // offsets reach 255 rows (k-contiguous) or 15 rows of k (m-contiguous) past the tile's origin
     if (p.lda > (1ull << 21) || p.ldb > (1ull << 21)) return false;
-    if ((p.M / bm) * (p.N / bn) > 0x7fffffffull) return false;
+    if (((p.M + bm - 1) / bm) * ((p.N + bn - 1) / bn) > 0x7fffffffull) return false;
     return true;
 }
 

@@ -1363,7 +1363,7 @@ int launch_f32_tail(hipStream_t st, const GemmProblem &p, bool edge) {
     if (p.ext || !plan_tail(p, BM, BN, BK, sizeof(float), OCC, g_tail_relaxed, plan)) return launch_f32<BM, BN, BK, WMS, WNS, OCC>(st, p, edge);
     const int sel = (p.op_a ? 0 : 2) | (p.op_b ? 1 : 0);
     int rc = WK_OK;
-    if (plan.first_tile > 0 && !edge && gemm_f32_dma_applies(p, BM, BN)) {
+    if (plan.first_tile > 0 && gemm_f32_dma_applies(p, BM, BN)) {
         rc = gemm_f32_dma_launch(st, p, BM, BN, plan.first_tile); // the whole rounds on the direct-to-LDS kernel
         if (rc) return rc;
     } else if (plan.first_tile > 0) { // the whole rounds, as the plain variant would run them
@@ -1434,7 +1434,7 @@ int split_kind_of(const char *name) { // by the name's suffix: ...z splits every
 const VariantDesc k_variants[] = {
     {"mfma_f32_256x128", WK_F32, 256, 128, 16, 0.940, 0.19, &launch_f32<256, 128, 16, 2, 2, 2>, nullptr, nullptr, nullptr, nullptr,
      "mfma_f32_256x128t", 2},
-    // slabs straight into LDS, three deep; interior shapes only (the cost loop skips it elsewhere):
+    // slabs straight into LDS, three deep; 16-byte aligned rows only (the cost loop skips it elsewhere):
     // 147.5 against 142.5 TFLOP/s at 8192^3, T,N 145.5 against 136
     {"mfma_f32_256x128d", WK_F32, 256, 128, 16, 0.943, 0.08, &launch_f32_dma<256, 128, 16, 2>, nullptr, nullptr, nullptr, nullptr,
      "mfma_f32_256x128t", 2},
@@ -1574,7 +1574,9 @@ int wk::gemm_mfma_pick(const GemmProblem &p) {
         const double rounds = tiles / cus + (d.bm <= 64 ? 0.65 : 1.0) * (whole - tiles / cus);
         // the bounds-checked instantiation runs slower than the interior one (8191 x 8193 x 8190 against
         // 8192^3 on the 256 x 128 tile: 126 against 142 TFLOP/s with the tail split off)
-        const double eff = d.efficiency * (needs_edge(p, d) ? (d.bm >= 256 ? 0.86 : d.bm >= 128 ? 0.944 : 0.93) : 1.0);
+        // (the direct-to-LDS kernels run ragged shapes in the same loop: their cost is in the tile count)
+        const bool slower_edge = needs_edge(p, d) && !(is_dma_variant(d.name) && d.dtype == WK_F32);
+        const double eff = d.efficiency * (slower_edge ? (d.bm >= 256 ? 0.86 : d.bm >= 128 ? 0.944 : 0.93) : 1.0);
         const double cost = (rounds + d.fill) * d.bm * d.bn / eff;
         if (best < 0 || cost < best_cost) {
             best = v;
