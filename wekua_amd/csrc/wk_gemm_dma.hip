@@ -2,7 +2,7 @@
 // (gfx950's 16-byte-per-lane global_load_lds), three slabs deep.
 //
 // Same tiling and matrix-instruction mapping as the kernels of wk_gemm_mfma.hip
-// (v_mfma_f32_32x32x2_f32, 2 x 2 wavefronts, macro tiles 256 x 128, 128 x 128 and 64 x 64, k-slab 16),
+// (v_mfma_f32_32x32x2_f32, 2 x 2 wavefronts, macro tiles 256 x 128 and 128 x 128 with k-slabs of 16, 64 x 64 with 32),
 // for operands whose rows start on 16-byte boundaries (f32: any M, N, K; f64: whole tiles and whole
 // k-slabs only).  What differs is how a slab gets into LDS and how the work-group hands over from one
 // slab to the next:
@@ -11,7 +11,7 @@
 //     free, the LDS side is not, so padding is replaced by swizzling: the lane that fills LDS
 //     chunk p of a row fetches the chunk that belongs there;
 //   * unpadded slabs of the 256 x 128 tile are 24 KB (A 16 KB + B 8 KB), so three of them fit twice
-//     on a compute unit (144 of 160 KB; 128 x 128: 3 x 16 KB three times; 64 x 64: 3 x 8 KB four times).  Slab kt+2 is requested at the top of iteration kt, a whole iteration and a
+//     on a compute unit (144 of 160 KB; 128 x 128: 3 x 16 KB three times; 64 x 64 with k-slabs of 32: 3 x 16 KB three times).  Slab kt+2 is requested at the top of iteration kt, a whole iteration and a
 //     half before it is read, and the only thing between the matrix instructions of two slabs is
 //     one barrier (every wavefront first waits for its own share of slab kt+1 to have landed).
 //
@@ -68,17 +68,35 @@ __device__ __forceinline__ void dma16(const float *base, uint32_t byte_offset, u
 }
 
 template <int N> __device__ __forceinline__ void wait_vm() { asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory"); }
+// wait until at most min(later, MAXN) slabs' loads of this wavefront (PER loads each) are still in flight
+template <int PER, int MAXN> __device__ __forceinline__ void wait_vm_slabs(uint32_t later) {
+    if constexpr (MAXN <= 0) {
+        wait_vm<0>();
+    } else {
+        if (later >= (uint32_t)MAXN) wait_vm<MAXN * PER>();
+        else wait_vm_slabs<PER, MAXN - 1>(later);
+    }
+}
+// f(integral_constant<int, A>) for A = FROM, FROM - 1, ..., 0
+template <int FROM, typename F> __device__ __forceinline__ void drain(F &&f) {
+    if constexpr (FROM >= 0) {
+        f(std::integral_constant<int, FROM>{});
+        drain<FROM - 1>(f);
+    }
+}
 __device__ __forceinline__ void wait_lgkm0() { asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); }
 
-template <int BM, int BN, int OCC, bool A_K, bool B_K, bool EXT>
+template <int BM, int BN, int BK, int NS, int OCC, bool A_K, bool B_K, bool EXT>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(OCC)))
 void gemm_f32_dma_kernel(DArgs g) {
-    constexpr int BK = 16, WM = BM / 2, WN = BN / 2, FM = WM / 32, FN = WN / 32;
+    constexpr int WM = BM / 2, WN = BN / 2, FM = WM / 32, FN = WN / 32;
+    constexpr int S = BK / 8;   // fragment steps per slab (8 values of k each: four matrix instructions per block)
+    constexpr int CPR = BK / 4; // 16-byte chunks per row of a k-contiguous slab
     constexpr int A_FLOATS = BM * BK, B_FLOATS = BN * BK, STAGE = A_FLOATS + B_FLOATS;
-    constexpr int A_LOADS = BM / 64, B_LOADS = BN / 64; // 1 KB per wavefront and load, four wavefronts
-    static_assert(BM % 64 == 0 && BN % 64 == 0, "tile shape");
+    constexpr int A_LOADS = BM * BK / 1024, B_LOADS = BN * BK / 1024; // 1 KB per wavefront and load, four wavefronts
+    static_assert(BM % 64 == 0 && BN % 64 == 0 && (BK == 16 || BK == 32) && NS >= 3, "tile shape");
 
-    extern __shared__ __align__(16) float lds[]; // [3][STAGE]: A then B
+    extern __shared__ __align__(16) float lds[]; // [NS][STAGE]: A then B
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -117,6 +135,9 @@ void gemm_f32_dma_kernel(DArgs g) {
             for (uint32_t i = 0; i < slot * (FM * FN * BK / 4); ++i) __builtin_amdgcn_s_sleep(2);
     }
 
+    // position of a 16-byte chunk inside its row of a k-contiguous slab: chunk number ^ swizzle(row)
+    auto swizzle = [](uint32_t row) -> uint32_t { return CPR == 4 ? (row >> 2) & 3u : (row >> 1) & 7u; };
+
     // ---- global side: scalar bases (advance by one slab per iteration) and per-lane byte offsets ----
     const float *a_base = A_K ? g.A + (size_t)m0 * g.lda : g.A + m0;
     const float *b_base = B_K ? g.B + (size_t)n0 * g.ldb : g.B + n0;
@@ -133,8 +154,8 @@ void gemm_f32_dma_kernel(DArgs g) {
         constexpr bool KC = decltype(kc_tag)::value;
         constexpr int ROWS = decltype(rows_tag)::value;
         if constexpr (KC) {
-            const uint32_t row = grp * 16 + (lane >> 2);
-            const uint32_t chunk = (lane & 3) ^ ((row >> 2) & 3);
+            const uint32_t row = grp * (64 / CPR) + lane / CPR;
+            const uint32_t chunk = (lane % CPR) ^ swizzle(row);
             return (min(row, last) * ld + 4 * chunk) * 4u;
         } else {
             constexpr int PER_ROW = ROWS / 4; // 16-byte chunks per row of k
@@ -168,13 +189,13 @@ void gemm_f32_dma_kernel(DArgs g) {
     // Chunks (k-contiguous operand) or rows of k (m-contiguous) that lie wholly beyond K are fetched from
     // the last existing one instead; once a wavefront's own loads of that slab have landed it writes
     // zeros over every float of its share whose k does not exist (products with them must vanish).
-    const uint32_t krem = g.K & 15u;
+    const uint32_t krem = g.K % BK;
     auto tail_offset = [&](uint32_t off, int grp, uint32_t ld, auto kc_tag, auto rows_tag) -> uint32_t {
         constexpr bool KC = decltype(kc_tag)::value;
         constexpr int ROWS = decltype(rows_tag)::value;
         if constexpr (KC) {
-            const uint32_t row = grp * 16 + (lane >> 2);
-            const uint32_t chunk = (lane & 3) ^ ((row >> 2) & 3);
+            const uint32_t row = grp * (64 / CPR) + lane / CPR;
+            const uint32_t chunk = (lane % CPR) ^ swizzle(row);
             return 4 * chunk >= krem ? off - 16u * chunk : off; // chunk 0 of the row always has a float (krem >= 1)
         } else {
             constexpr int PER_ROW = ROWS / 4;
@@ -192,8 +213,8 @@ void gemm_f32_dma_kernel(DArgs g) {
         constexpr bool KC = decltype(kc_tag)::value;
         constexpr int ROWS = decltype(rows_tag)::value;
         if constexpr (KC) {
-            const uint32_t row = grp * 16 + (lane >> 2);
-            const uint32_t chunk = (lane & 3) ^ ((row >> 2) & 3);
+            const uint32_t row = grp * (64 / CPR) + lane / CPR;
+            const uint32_t chunk = (lane % CPR) ^ swizzle(row);
 #pragma unroll
             for (int e = 0; e < 4; ++e)
                 if (4 * chunk + e >= krem) dst[e] = 0.f;
@@ -212,16 +233,16 @@ void gemm_f32_dma_kernel(DArgs g) {
     };
 
     // ---- LDS side: per-lane fragment addresses (floats from the start of a stage's A or B part) ----
-    // k-contiguous: row * 16 + 4 * (chunk ^ swz); chunk = 2 s + lhi, swz = (l32 >> 2) & 3 (row offsets are multiples of 32)
+    // k-contiguous: row * BK + 4 * (chunk ^ swz); chunk = 2 s + lhi, swz from l32 alone (row offsets are multiples of 32)
     // m-contiguous: k * ROWS + (m ^ 32 lhi); k = 8 s + 4 lhi + t; m = wave offset + 32 i + l32
-    const int sw4 = 4 * (lhi ^ ((l32 >> 2) & 3));
+    const int sw4 = 4 * (lhi ^ (int)swizzle((uint32_t)l32));
     int a_frag[FM], b_frag[FN]; // k-contiguous: one base (block i is an immediate away); m-contiguous: block i's column
 #pragma unroll
     for (int i = 0; i < FM; ++i)
-        a_frag[i] = A_K ? (wm * WM + l32) * 16 + sw4 : 4 * lhi * BM + (((wm * WM + 32 * i) ^ (32 * lhi)) + l32);
+        a_frag[i] = A_K ? (wm * WM + l32) * BK + sw4 : 4 * lhi * BM + (((wm * WM + 32 * i) ^ (32 * lhi)) + l32);
 #pragma unroll
     for (int j = 0; j < FN; ++j)
-        b_frag[j] = B_K ? (wn * WN + l32) * 16 + sw4 : 4 * lhi * BN + (((wn * WN + 32 * j) ^ (32 * lhi)) + l32);
+        b_frag[j] = B_K ? (wn * WN + l32) * BK + sw4 : 4 * lhi * BN + (((wn * WN + 32 * j) ^ (32 * lhi)) + l32);
 
     auto read_frags = [&](uint32_t stage_bytes, int s, f32x4 *af, f32x4 *bf) {
         const float *as = lds + stage_bytes / 4;
@@ -229,8 +250,8 @@ void gemm_f32_dma_kernel(DArgs g) {
 #pragma unroll
         for (int i = 0; i < FM; ++i) {
             if constexpr (A_K) {
-                // chunk 2 s + lhi: the second step's chunk is the first one's with bit 1 flipped
-                af[i] = *reinterpret_cast<const f32x4 *>(as + ((a_frag[i] ^ (s ? 8 : 0)) + i * 32 * 16));
+                // chunk 2 s + lhi: step s flips the bits of 2 s in the chunk number
+                af[i] = *reinterpret_cast<const f32x4 *>(as + ((a_frag[i] ^ (8 * s)) + i * 32 * BK));
             } else {
 #pragma unroll
                 for (int t = 0; t < 4; ++t) af[i][t] = as[a_frag[i] + (8 * s + t) * BM];
@@ -239,7 +260,7 @@ void gemm_f32_dma_kernel(DArgs g) {
 #pragma unroll
         for (int j = 0; j < FN; ++j) {
             if constexpr (B_K) {
-                bf[j] = *reinterpret_cast<const f32x4 *>(bs + ((b_frag[j] ^ (s ? 8 : 0)) + j * 32 * 16));
+                bf[j] = *reinterpret_cast<const f32x4 *>(bs + ((b_frag[j] ^ (8 * s)) + j * 32 * BK));
             } else {
 #pragma unroll
                 for (int t = 0; t < 4; ++t) bf[j][t] = bs[b_frag[j] + (8 * s + t) * BN];
@@ -268,67 +289,95 @@ void gemm_f32_dma_kernel(DArgs g) {
 
     const uint32_t ktiles = (g.K + BK - 1) / BK;
 
-    // The three stages rotate: the slab being multiplied, the next one, and the one after it (byte offsets).
+    // The NS stages rotate (byte offsets): st[0] holds the slab being multiplied, st[1] the next one, ...,
+    // st[NS - 1] is the stage the slab before left, into which slab kt + NS - 1 is requested.
     constexpr uint32_t STAGE_BYTES = STAGE * 4u;
-    uint32_t st_cur = 0, st_next = STAGE_BYTES, st_after = 2 * STAGE_BYTES;
+    constexpr int LOADS = A_LOADS + B_LOADS; // per wavefront and slab
+    uint32_t st[NS];
+#pragma unroll
+    for (int n = 0; n < NS; ++n) st[n] = n * STAGE_BYTES;
 
-    // prologue: slabs 0 and 1 on their way, slab 0 landed everywhere, first fragments read
-    if (ktiles == 1 && krem) tail_offsets();
-    issue(st_cur);
-    if (ktiles > 1) {
-        if (ktiles == 2 && krem) tail_offsets();
-        issue(st_next);
-        wait_vm<A_LOADS + B_LOADS>();
-    } else {
-        wait_vm<0>();
-        if (krem) {
-            tail_zeros(st_cur);
-            wait_lgkm0();
+    // The one-block-per-wavefront tile fetches C_old ahead of everything else (16 registers): its launches
+    // are short and the latency of that read at the end of a tile is a visible share of them.  These loads
+    // are older than every slab load, so the counted waits below cover them as well.
+    constexpr bool PRELOAD_C = FM * FN == 1;
+    float c_old[PRELOAD_C ? 16 : 1];
+    if constexpr (PRELOAD_C) {
+        if (g.epi == EPI_ALPHA_BETA) {
+            const uint32_t colc = min(n0 + wn * WN + l32, g.N - 1);
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const uint32_t row = m0 + wm * WM + 8 * (r / 4) + 4 * lhi + (r % 4);
+                c_old[r] = g.C[(size_t)min(row, g.M - 1) * g.ldc + colc];
+            }
         }
     }
-    __builtin_amdgcn_s_barrier();
-    read_frags(st_cur, 0, af[0], bf[0]);
 
-    // One iteration on the slab in stage st_cur.  MORE2: slab kt+2 exists and is requested into the stage
-    // that slab kt-1 left (every wavefront is past the barrier of iteration kt-1, in front of which it
-    // waited for its last reads of that stage).  MORE1: slab kt+1 exists; before the last step's matrix
-    // instructions this wavefront waits for its own loads of slab kt+1 (those of slab kt+2 may stay in
-    // flight) and for its LDS reads, joins the barrier and reads the first fragments of slab kt+1.
-    auto iteration = [&](auto more2_tag, auto more1_tag) __attribute__((always_inline)) {
-        constexpr bool MORE2 = decltype(more2_tag)::value, MORE1 = decltype(more1_tag)::value;
-        if constexpr (MORE2) issue(st_after);
-        read_frags(st_cur, 1, af[1], bf[1]);
-        mfma_step(0);
-        if constexpr (MORE1) {
+    // prologue: the first NS - 1 slabs on their way, slab 0 landed everywhere, first fragments read
+#pragma unroll
+    for (int n = 0; n < NS - 1; ++n)
+        if ((uint32_t)n < ktiles) {
+            if ((uint32_t)n + 1 == ktiles && krem) tail_offsets();
+            issue(st[n]);
+        }
+    wait_vm_slabs<LOADS, NS - 2>(ktiles - 1); // all but the slabs after the first
+    if (ktiles == 1 && krem) {
+        tail_zeros(st[0]);
+        wait_lgkm0();
+    }
+    __builtin_amdgcn_s_barrier();
+    read_frags(st[0], 0, af[0], bf[0]);
+
+    // One iteration on the slab in stage st[0].  ISSUE: slab kt + NS - 1 exists and is requested into the
+    // stage that slab kt - 1 left (every wavefront is past the barrier of iteration kt - 1, in front of
+    // which it waited for its last reads of that stage).  AHEAD >= 0: slab kt + 1 exists and AHEAD slabs
+    // after it have been requested; before the last step's matrix instructions this wavefront waits for
+    // its own loads of slab kt + 1 (the AHEAD later ones may stay in flight) and for its LDS reads, joins
+    // the barrier and reads the first fragments of slab kt + 1.  AHEAD < 0: the last slab.
+    auto iteration = [&](auto issue_tag, auto ahead_tag) __attribute__((always_inline)) {
+        constexpr bool ISSUE = decltype(issue_tag)::value;
+        constexpr int AHEAD = decltype(ahead_tag)::value;
+        if constexpr (ISSUE) issue(st[NS - 1]);
+#pragma unroll
+        for (int s = 0; s + 1 < S; ++s) {
+            read_frags(st[0], s + 1, af[(s + 1) & 1], bf[(s + 1) & 1]);
+            mfma_step(s);
+        }
+        if constexpr (AHEAD >= 0) {
             __builtin_amdgcn_sched_barrier(0);
-            if constexpr (MORE2) {
-                wait_vm<A_LOADS + B_LOADS>();
-            } else {
-                wait_vm<0>();
-                if (krem) tail_zeros(st_next); // slab kt+1 is the last one
+            wait_vm<AHEAD * LOADS>();
+            if constexpr (AHEAD == 0) {
+                if (krem) tail_zeros(st[1]); // slab kt + 1 is the last one
             }
             wait_lgkm0();
             __builtin_amdgcn_s_barrier();
-            read_frags(st_next, 0, af[0], bf[0]);
+            read_frags(st[1], 0, af[0], bf[0]);
             __builtin_amdgcn_sched_barrier(0);
         }
-        mfma_step(1);
-        const uint32_t t = st_cur;
-        st_cur = st_next;
-        st_next = st_after;
-        st_after = t;
+        mfma_step(S - 1);
+        const uint32_t t = st[0];
+#pragma unroll
+        for (int n = 0; n + 1 < NS; ++n) st[n] = st[n + 1];
+        st[NS - 1] = t;
     };
+    using std::integral_constant;
     using T_ = std::true_type;
     using F_ = std::false_type;
     uint32_t kt = 0;
-    for (; kt + 3 < ktiles; ++kt) iteration(T_{}, T_{}); // steady state: both following slabs exist
-    if (kt + 2 < ktiles) {                               // the iteration that requests the last slab
+    for (; kt + NS < ktiles; ++kt) iteration(T_{}, integral_constant<int, NS - 2>{}); // steady state
+    if (kt + NS - 1 < ktiles) { // the iteration that requests the last slab
         if (krem) tail_offsets();
-        iteration(T_{}, T_{});
+        iteration(T_{}, integral_constant<int, NS - 2>{});
         ++kt;
     }
-    if (kt + 1 < ktiles) iteration(F_{}, T_{});          // the last but one
-    iteration(F_{}, F_{});                               // the last
+    // the pipeline drains: ktiles - 2 - kt slabs are in flight beyond the next one
+    drain<NS - 3>([&](auto ahead_tag) {
+        if (kt + 2 + decltype(ahead_tag)::value == ktiles) {
+            iteration(F_{}, ahead_tag);
+            ++kt;
+        }
+    });
+    iteration(F_{}, integral_constant<int, -1>{}); // the last
 
     // ---- epilogue: acc register r of lane l is C[8*(r/4) + 4*(l/32) + r%4][l%32] of its 32x32 block;
     // option semantics of src/blas/gemm.zig:500-501,591-602 (C_old is read and multiplied whenever beta
@@ -352,7 +401,8 @@ void gemm_f32_dma_kernel(DArgs g) {
 #pragma unroll
                     for (int r = 0; r < 16; ++r) {
                         const uint32_t row = m0 + wm * WM + i * 32 + 8 * (r / 4) + 4 * lhi + (r % 4);
-                        old[r] = g.C[(size_t)(CHECKED ? min(row, g.M - 1) : row) * g.ldc + colc];
+                        if constexpr (PRELOAD_C) old[r] = c_old[r];
+                        else old[r] = g.C[(size_t)(CHECKED ? min(row, g.M - 1) : row) * g.ldc + colc];
                     }
                 }
 #pragma unroll
@@ -692,9 +742,9 @@ template <int BM, int BN, int BK, int OCC> int launch_tile_d(hipStream_t st, con
 }
 
 // first_tiles: launch only that many tiles, in tile-walk order (0: all of them)
-template <int BM, int BN, int OCC, bool A_K, bool B_K, bool EXT> int launch_one(hipStream_t st, const DArgs &g, uint64_t first_tiles) {
-    constexpr size_t lds_bytes = 3 * (BM * 16 + BN * 16) * sizeof(float); // 72 / 48 / 24 KB
-    auto kern = gemm_f32_dma_kernel<BM, BN, OCC, A_K, B_K, EXT>;
+template <int BM, int BN, int BK, int NS, int OCC, bool A_K, bool B_K, bool EXT> int launch_one(hipStream_t st, const DArgs &g, uint64_t first_tiles) {
+    constexpr size_t lds_bytes = NS * (BM * BK + BN * BK) * sizeof(float); // 3 x 24 KB / 3 x 16 KB / 4 x 16 KB
+    auto kern = gemm_f32_dma_kernel<BM, BN, BK, NS, OCC, A_K, B_K, EXT>;
     static const int attr_rc = [&] {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
                                            (int)lds_bytes);
@@ -710,7 +760,7 @@ template <int BM, int BN, int OCC, bool A_K, bool B_K, bool EXT> int launch_one(
     return launch_status();
 }
 
-template <int BM, int BN, int OCC> int launch_tile(hipStream_t st, const GemmProblem &p, uint64_t first_tiles) {
+template <int BM, int BN, int BK, int NS, int OCC> int launch_tile(hipStream_t st, const GemmProblem &p, uint64_t first_tiles) {
     if (first_tiles > ((p.M + BM - 1) / BM) * ((p.N + BN - 1) / BN)) return WK_E_INVALID_VALUE;
     DArgs g{};
     g.A = static_cast<const float *>(p.A);
@@ -743,12 +793,12 @@ template <int BM, int BN, int OCC> int launch_tile(hipStream_t st, const GemmPro
     }
     const int sel = (p.op_a ? 0 : 2) | (p.op_b ? 1 : 0); // bit 1: A k-contiguous, bit 0: B k-contiguous
     if (p.ext) // instantiated for op N, T only (what Linear.forward runs)
-        return sel == 3 ? launch_one<BM, BN, OCC, true, true, true>(st, g, first_tiles) : (int)WK_E_INVALID_VALUE;
+        return sel == 3 ? launch_one<BM, BN, BK, NS, OCC, true, true, true>(st, g, first_tiles) : (int)WK_E_INVALID_VALUE;
     switch (sel) {
-    case 0: return launch_one<BM, BN, OCC, false, false, false>(st, g, first_tiles);
-    case 1: return launch_one<BM, BN, OCC, false, true, false>(st, g, first_tiles);
-    case 2: return launch_one<BM, BN, OCC, true, false, false>(st, g, first_tiles);
-    default: return launch_one<BM, BN, OCC, true, true, false>(st, g, first_tiles);
+    case 0: return launch_one<BM, BN, BK, NS, OCC, false, false, false>(st, g, first_tiles);
+    case 1: return launch_one<BM, BN, BK, NS, OCC, false, true, false>(st, g, first_tiles);
+    case 2: return launch_one<BM, BN, BK, NS, OCC, true, false, false>(st, g, first_tiles);
+    default: return launch_one<BM, BN, BK, NS, OCC, true, true, false>(st, g, first_tiles);
     }
 }
 
@@ -792,7 +842,11 @@ int wk::gemm_f64_dma_launch(hipStream_t st, const GemmProblem &p, int bm, int bn
 
 int wk::gemm_f32_dma_launch(hipStream_t st, const GemmProblem &p, int bm, int bn, uint64_t first_tiles) {
     if (!gemm_f32_dma_applies(p, bm, bn)) return WK_E_INVALID_VALUE;
-    if (bm == 256) return launch_tile<256, 128, 2>(st, p, first_tiles);
-    if (bm == 128) return launch_tile<128, 128, 3>(st, p, first_tiles);
-    return launch_tile<64, 64, 4>(st, p, first_tiles);
+    if (bm == 256) return launch_tile<256, 128, 16, 3, 2>(st, p, first_tiles);
+    if (bm == 128) return launch_tile<128, 128, 16, 3, 3>(st, p, first_tiles);
+    // (k-slabs of 32, three work-groups per unit; with slabs of 16 and four: 1024^3 101 against 103.5 TFLOP/s,
+    // 3000^3 118 against 125, 2049 x 2047 x 2050 108 against 106.5)
+    // Deeper pipelines were measured for this tile and gave nothing: four stages (two work-groups per unit)
+    // and five (one) 1024^3 101-104 TFLOP/s like three, 1536^3 95 against 98; six stages of 16: 90-100.
+    return launch_tile<64, 64, 32, 3, 3>(st, p, first_tiles);
 }
