@@ -167,13 +167,15 @@ def test_config4_int32_overflow_forcing(dev):
     assert np.array_equal(oracle.gemm("i32", 65537, a, 0, b, 0, -3, c), want)
 
 
+@pytest.mark.parametrize("shape", [(4096, 4096, 2048), (2048, 2048, 2048), (2125, 1541, 1090)])
 @pytest.mark.parametrize("op_a,op_b", OPS)
-def test_config4_int32_large_with_packed_tensors(op_a, op_b):
+def test_config4_int32_large_with_packed_tensors(op_a, op_b, shape):
     """The int32 product the way benchmark/gemm.zig drives it: through blas.gemm with a
-    GemmPackedTensors, at a size where the library takes its pack pass + packed kernel."""
+    GemmPackedTensors, at sizes where the library takes its pack pass + packed kernel: configuration 4's
+    own 2048^3, a larger one, and a ragged one whose 35 k-slabs are padded to an even count."""
     import wekua_amd as wk
     from wekua_amd import raw
-    M, N, K = 4096, 4096, 2048
+    M, N, K = shape
     a = synth.integers(synth.config_seed(4, 6), (K, M) if op_a else (M, K), np.int32, -100, 100)
     b = synth.integers(synth.config_seed(4, 7), (N, K) if op_b else (K, N), np.int32, -100, 100)
     c = synth.integers(synth.config_seed(4, 8), (M, N), np.int32, -100, 100)

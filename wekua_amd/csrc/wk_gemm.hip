@@ -43,12 +43,13 @@ int transpose_for_gemm(void *ctx, int dtype, uint64_t rows, uint64_t cols, const
 bool is_int32(int dtype) { return dtype == WK_I32 || dtype == WK_U32; }
 bool has_packed_path(int dtype) { return dtype >= WK_I8 && dtype <= WK_U32; }
 // The pack pass reads A and B once more and writes as much.  32-bit, measured against the fused
-// matrix-core kernel on MI355X (all four layouts): 1024^3 -8 %, 2048^3 equal, 4096^3 +9..10 %,
-// 8192^3 +13..18 %.  8- and 16-bit integers have only the vector-ALU kernel (36-45 TOP/s) beside it:
-// the two launches of the packed path take 16-20 us up to 1024^3, which that kernel beats below ~700^3.
+// matrix-core kernels on MI355X (N,N / T,N, microseconds, fused best of its two tiles -> packed): 1024^3
+// 34 / 43 -> 39, 1536^3 61 / 63 -> 48, 2048^3 86 -> 77, 1024 x 1024 x 4096 117 / 154 -> 96, 2048 x 2048 x 512
+// 28 -> 33; 4096^3 +15 %, 8192^3 +25 %.  8- and 16-bit integers have only the vector-ALU kernel (36-45 TOP/s)
+// beside it: the two launches of the packed path take 16-20 us up to 1024^3, which that kernel beats below ~700^3.
 bool packed_pays(const GemmProblem &p) {
     const double work = (double)p.M * (double)p.N * (double)p.K;
-    if (is_int32(p.dtype)) return p.M >= 1024 && p.N >= 1024 && work >= 3.0e10;
+    if (is_int32(p.dtype)) return p.M >= 1024 && p.N >= 1024 && work >= 3.0e9;
     return p.M >= 256 && p.N >= 256 && work >= 4.0e8;
 }
 

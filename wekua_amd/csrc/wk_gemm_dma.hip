@@ -29,11 +29,13 @@
 // front of every fragment read, which serialises exactly what this kernel overlaps.  The waits that
 // are needed are written out instead (vmcnt before the barrier that publishes a slab).
 #include "wk_internal.hpp"
+#include "wk_lds_dma.hpp"
 
 #include <cstdlib>
 #include <cstring>
 
 using namespace wk;
+using namespace wk::lds_dma;
 
 namespace {
 
@@ -55,36 +57,6 @@ struct DArgs {
     int act;
     uint32_t patch_m, patch_n; // tile walk in XCD-local patches of patch_m x patch_n tiles (0: rows of groups)
 };
-
-// 16 bytes per lane from global memory (scalar base + 32-bit byte offset per lane) to LDS at
-// lds_base + 16 * lane; lds_base is a byte address, the same in every lane.
-__device__ __forceinline__ void dma16(const float *base, uint32_t byte_offset, uint32_t lds_base) {
-    asm volatile("s_mov_b32 m0, %2\n\t"
-                 "s_nop 0\n\t"
-                 "global_load_lds_dwordx4 %0, %1"
-                 :
-                 : "v"(byte_offset), "s"(base), "s"(lds_base)
-                 : "memory");
-}
-
-template <int N> __device__ __forceinline__ void wait_vm() { asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory"); }
-// wait until at most min(later, MAXN) slabs' loads of this wavefront (PER loads each) are still in flight
-template <int PER, int MAXN> __device__ __forceinline__ void wait_vm_slabs(uint32_t later) {
-    if constexpr (MAXN <= 0) {
-        wait_vm<0>();
-    } else {
-        if (later >= (uint32_t)MAXN) wait_vm<MAXN * PER>();
-        else wait_vm_slabs<PER, MAXN - 1>(later);
-    }
-}
-// f(integral_constant<int, A>) for A = FROM, FROM - 1, ..., 0
-template <int FROM, typename F> __device__ __forceinline__ void drain(F &&f) {
-    if constexpr (FROM >= 0) {
-        f(std::integral_constant<int, FROM>{});
-        drain<FROM - 1>(f);
-    }
-}
-__device__ __forceinline__ void wait_lgkm0() { asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); }
 
 template <int BM, int BN, int BK, int NS, int OCC, bool A_K, bool B_K, bool EXT>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(OCC)))
@@ -454,14 +426,6 @@ struct DArgsD {
     int act;
 };
 
-__device__ __forceinline__ void dma16d(const double *base, uint32_t byte_offset, uint32_t lds_base) {
-    asm volatile("s_mov_b32 m0, %2\n\t"
-                 "s_nop 0\n\t"
-                 "global_load_lds_dwordx4 %0, %1"
-                 :
-                 : "v"(byte_offset), "s"(base), "s"(lds_base)
-                 : "memory");
-}
 
 template <int BM, int BN, int BK, int OCC, bool A_K, bool B_K, bool EXT>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(OCC)))
@@ -534,9 +498,9 @@ void gemm_f64_dma_kernel(DArgsD g) {
     auto issue = [&](uint32_t stage_bytes) {
         const uint32_t sbase = lds0 + stage_bytes + (uint32_t)wave * 1024u;
 #pragma unroll
-        for (int i = 0; i < A_LOADS; ++i) dma16d(a_base, a_off[i], sbase + (uint32_t)i * 4096u);
+        for (int i = 0; i < A_LOADS; ++i) dma16(a_base, a_off[i], sbase + (uint32_t)i * 4096u);
 #pragma unroll
-        for (int i = 0; i < B_LOADS; ++i) dma16d(b_base, b_off[i], sbase + A_DOUBLES * 8u + (uint32_t)i * 4096u);
+        for (int i = 0; i < B_LOADS; ++i) dma16(b_base, b_off[i], sbase + A_DOUBLES * 8u + (uint32_t)i * 4096u);
         a_base += a_step;
         b_base += b_step;
     };

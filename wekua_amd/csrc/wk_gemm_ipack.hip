@@ -27,6 +27,7 @@
 // of 32, so that it is 4 KiB per 32 rows whatever the width, and the matrix work per slab is 4 x 1 or
 // 2 x 3 instructions per 32 x 32 block instead of 10.  Their only other kernel is the vector-ALU one.
 #include "wk_internal.hpp"
+#include "wk_lds_dma.hpp"
 
 #include <cstring>
 #include <type_traits>
@@ -61,7 +62,9 @@ Layout make_layout(int digits, uint64_t M, uint64_t N, uint64_t K) {
     w.Mp = (M + m_tile - 1) / m_tile * m_tile;
     const uint64_t n_tile = digits == 1 ? 256 : TILE; // 8-bit: also the 256-column tile
     w.Np = (N + n_tile - 1) / n_tile * n_tile;
-    w.KB = ((K + BK - 1) / BK + per_slab - 1) / per_slab * per_slab;
+    // (32-bit types: an even number of slabs, for the two-slab loop of the direct-to-LDS kernel)
+    const uint64_t kb_round = digits == 4 ? 2 : per_slab;
+    w.KB = ((K + BK - 1) / BK + kb_round - 1) / kb_round * kb_round;
     w.slabs = w.KB / per_slab;
     // enough work-groups in the pack launch to fill the chip: (Mp + Np) / 32 row blocks x ksplit
     uint64_t ks = 2048 / ((w.Mp + w.Np) / 32);
@@ -220,6 +223,7 @@ struct PArgs {
     uint32_t M, N, K, slabs, Mp, Np, ksplit, ldc, tiles_m, tiles_n;
     int epi;
     uint32_t alpha, beta;
+    uint32_t patch_m, patch_n; // the direct-to-LDS kernel's tile walk (0: groups of tile rows)
 };
 
 // BM x 128 tile, BM / 32 x 2 waves.  BM = 128 (one 8-wave work-group per CU) is what is launched.
@@ -271,8 +275,13 @@ void gemm_int_packed_kernel(PArgs g) {
     if (tid < BM + BN) {
         const uint32_t *src = tid < BM ? g.sums_a + m0 + tid : g.sums_b + n0 + (tid - BM);
         const uint32_t stride = tid < BM ? g.Mp : g.Np;
+        // (all partial sums requested at once: one after the other they cost a memory latency each)
+        uint32_t part[MAX_KSPLIT];
+#pragma unroll
+        for (uint32_t i = 0; i < MAX_KSPLIT; ++i) part[i] = i < g.ksplit ? src[(size_t)i * stride] : 0u;
         uint32_t s = 0;
-        for (uint32_t i = 0; i < g.ksplit; ++i) s += src[(size_t)i * stride];
+#pragma unroll
+        for (uint32_t i = 0; i < MAX_KSPLIT; ++i) s += part[i];
         row_sum[tid] = s; // col_sum follows row_sum
     }
 
@@ -439,6 +448,265 @@ template <typename E, int BM, bool EDGE, int WMF = 1, int BN = TILE> int launch_
     return launch_status();
 }
 
+// ---- 32-bit product kernel with the slabs brought straight into LDS ------------------------------
+// The packed planes are already in the order the matrix instruction eats them (1 KiB per block, lane l
+// owning bytes 16 l .. 16 l + 15), which is also the order in which a direct global -> LDS load lays a
+// wavefront's 64 x 16 bytes down.  So a slab of the 128 x 128 tile (four row groups of A, four column
+// groups of B, 32 KiB) is 32 such loads, eight per wavefront, NS stages deep, with no staging registers
+// and no LDS stores.  The registers go to the tile instead: four wavefronts of 64 x 64 (one per SIMD,
+// 256 accumulator registers: 2 x 2 blocks x four shift sets) with two sets of the slab's sixteen
+// fragments, so that a wavefront reads 16 KiB from LDS per 40 matrix instructions (the 8-wavefront
+// kernel above: 12 KiB per 20) and the fragments of slab kt + 1 are on their way while slab kt is
+// multiplied.  Per iteration: request slab kt + NS - 1, half of the matrix instructions, wait for the
+// own loads of slab kt + 1, barrier, read its fragments into the other set, the other half.
+struct PackedDmaTile {
+    static constexpr int BM = TILE, BN = TILE, GROUPS = 8, STAGE_BYTES = GROUPS * GROUP_BYTES;
+    static constexpr size_t lds_bytes(int ns) { return (size_t)ns * STAGE_BYTES + (BM + BN) * sizeof(uint32_t); }
+};
+
+template <bool EDGE, int NS>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1)))
+void gemm_i32_packed_dma_kernel(PArgs g) {
+    using namespace wk::lds_dma;
+    using TL = PackedDmaTile;
+    constexpr int BM = TL::BM, BN = TL::BN, STAGE_BYTES = TL::STAGE_BYTES;
+    constexpr uint32_t CBIAS = 0x80808080u;
+    extern __shared__ __align__(16) unsigned char lds_raw[];
+    uint32_t *row_sum = reinterpret_cast<uint32_t *>(lds_raw + NS * STAGE_BYTES); // [BM], then col_sum [BN]
+    uint32_t *col_sum = row_sum + BM;
+
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wm = wave >> 1, wn = wave & 1, l32 = lane & 31, lhi = lane >> 5;
+    uint32_t tile_m, tile_n;
+    if (g.patch_m) { // XCD-local patches: work-group b runs on XCD b % 8 (see wk_gemm_dma.hip)
+        const uint32_t pid = blockIdx.x, x = pid & 7u, j = pid >> 3;
+        const uint32_t per_patch = g.patch_m * g.patch_n, patch = (j / per_patch) * 8u + x, q = j % per_patch;
+        const uint32_t patches_n = g.tiles_n / g.patch_n;
+        tile_m = (patch / patches_n) * g.patch_m + q % g.patch_m;
+        tile_n = (patch % patches_n) * g.patch_n + q / g.patch_m;
+    } else {
+        const uint32_t pid = blockIdx.x, group_size = 8 * g.tiles_n, group = pid / group_size, first_m = group * 8;
+        const uint32_t gsz = min(g.tiles_m - first_m, 8u), in_group = pid - group * group_size;
+        tile_m = first_m + in_group % gsz;
+        tile_n = in_group / gsz;
+    }
+    const uint32_t m0 = tile_m * BM, n0 = tile_n * BN;
+
+    {
+        const uint32_t *src = tid < BM ? g.sums_a + m0 + tid : g.sums_b + n0 + (tid - BM);
+        const uint32_t stride = tid < BM ? g.Mp : g.Np;
+        uint32_t part[MAX_KSPLIT]; // all partial sums requested at once
+#pragma unroll
+        for (uint32_t i = 0; i < MAX_KSPLIT; ++i) part[i] = i < g.ksplit ? src[(size_t)i * stride] : 0u;
+        uint32_t s = 0;
+#pragma unroll
+        for (uint32_t i = 0; i < MAX_KSPLIT; ++i) s += part[i];
+        row_sum[tid] = s; // col_sum follows row_sum; published by the first barrier below
+    }
+    // these loads are older than every slab load: wait for them here, so that the counted waits below
+    // count slab loads only
+    wait_vm<0>();
+
+    // wavefront w brings groups 2 w and 2 w + 1 of every slab: A's row groups 0..3, then B's column groups
+    const unsigned char *src_g[2];
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+        const int gi = 2 * wave + h;
+        src_g[h] = gi < 4 ? g.planes_a + (size_t)(tile_m * 4 + gi) * g.slabs * GROUP_BYTES
+                          : g.planes_b + (size_t)(tile_n * 4 + gi - 4) * g.slabs * GROUP_BYTES;
+    }
+    uint32_t voff[4];
+#pragma unroll
+    for (int d = 0; d < 4; ++d) voff[d] = lane * 16 + d * BLOCK_BYTES;
+    const uint32_t lds0 = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)(__attribute__((address_space(3))) unsigned char *)lds_raw);
+    auto issue = [&](uint32_t stage_bytes) {
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+#pragma unroll
+            for (int d = 0; d < 4; ++d)
+                dma16(src_g[h], voff[d], lds0 + stage_bytes + (uint32_t)(2 * wave + h) * GROUP_BYTES + d * BLOCK_BYTES);
+            src_g[h] += GROUP_BYTES;
+        }
+    };
+    constexpr int LOADS = 8;
+
+    i32x16 acc[4][2][2]; // [shift i + j][row block][column block]
+#pragma unroll
+    for (int s = 0; s < 4; ++s)
+#pragma unroll
+        for (int am = 0; am < 2; ++am)
+#pragma unroll
+            for (int b = 0; b < 2; ++b)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) acc[s][am][b][r] = 0;
+
+    // Fragment reads and matrix instructions are written as inline assembly, in the order they are to be
+    // issued.  (1) The accumulators: the compiler keeps all sixteen in the 256 accumulation registers,
+    // needs a few of those for itself and then spills accumulators inside the loop; here shifts 0..2
+    // (twelve accumulators) are pinned to accumulation registers and shift 3 (four) to vector registers
+    // beside the fragments.  (2) The order: a wavefront is alone on its SIMD, so whatever holds up its
+    // instruction stream idles the matrix pipe.  Sixteen 16-byte LDS reads in a row do (four wavefronts'
+    // reads of a slab keep the LDS busy for 512 clocks and the read queue is short), so each read follows
+    // one matrix instruction, and the slab requests are spread over the first half in the same way.
+    // What the compiler cannot see in inline assembly are the latencies: LDS reads are waited for by hand
+    // (lgkmcnt at the top of the iteration that uses them), two matrix instructions on one accumulator
+    // are at least four instructions apart, and in front of the epilogue, which reads the accumulators
+    // with vector instructions, the wait is written out.
+    i32x4 fa[2][2][4], fb[2][2][4]; // [set][block][digit]
+    const uint32_t frag_a = lds0 + lane * 16 + (wm * 2) * GROUP_BYTES, frag_b = lds0 + lane * 16 + (4 + wn * 2) * GROUP_BYTES;
+    // fragment number f of a slab: 0..7 A (block f / 4, digit f % 4), 8..15 B
+    auto read_frag = [&](uint32_t stage_bytes, auto set_tag, auto f_tag) __attribute__((always_inline)) {
+        constexpr int SET = decltype(set_tag)::value, F = decltype(f_tag)::value;
+        constexpr int BLK = (F & 7) / 4, DIG = F & 3, IMM = BLK * GROUP_BYTES + DIG * BLOCK_BYTES;
+        // (operands of inline assembly do not capture by themselves inside a generic lambda)
+        i32x4 &dst = F < 8 ? fa[SET][BLK][DIG] : fb[SET][BLK][DIG];
+        const uint32_t addr = (F < 8 ? frag_a : frag_b) + stage_bytes;
+        asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(dst) : "v"(addr), "n"(IMM));
+    };
+    // matrix instruction number n of a slab (0..39): digit pair n / 4 in the order (0,0) (0,1) (1,0) (0,2) (1,1)
+    // (2,0) (0,3) (1,2) (2,1) (3,0), row block (n / 2) % 2, column block n % 2
+    auto mfma_n = [&](auto set_tag, auto n_tag) __attribute__((always_inline)) {
+        constexpr int SET = decltype(set_tag)::value, N = decltype(n_tag)::value;
+        constexpr int PAIR = N / 4, AM = (N / 2) & 1, B = N & 1;
+        constexpr int SH = PAIR < 1 ? 0 : PAIR < 3 ? 1 : PAIR < 6 ? 2 : 3;
+        constexpr int I = PAIR - (SH == 0 ? 0 : SH == 1 ? 1 : SH == 2 ? 3 : 6);
+        i32x16 &c = acc[SH][AM][B];
+        const i32x4 &a = fa[SET][AM][I], &b = fb[SET][B][SH - I];
+        if constexpr (SH == 3) asm volatile("v_mfma_i32_32x32x32_i8 %0, %1, %2, %0" : "+v"(c) : "v"(a), "v"(b));
+        else asm volatile("v_mfma_i32_32x32x32_i8 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
+    };
+    // one of the eight slab requests of this wavefront (group h = R / 4 of its two, digit block R % 4)
+    auto issue_one = [&](uint32_t stage_bytes, auto r_tag) __attribute__((always_inline)) {
+        constexpr int R = decltype(r_tag)::value, H = R / 4, DIG = R & 3;
+        dma16(src_g[H], voff[DIG], lds0 + stage_bytes + (uint32_t)(2 * wave + H) * GROUP_BYTES + DIG * BLOCK_BYTES);
+        if constexpr (DIG == 3) src_g[H] += GROUP_BYTES;
+    };
+
+    const uint32_t ktiles = g.slabs;
+    uint32_t st[NS];
+#pragma unroll
+    for (int n = 0; n < NS; ++n) st[n] = n * STAGE_BYTES;
+
+    using std::integral_constant;
+#pragma unroll
+    for (int n = 0; n < NS - 1; ++n)
+        if ((uint32_t)n < ktiles) issue(st[n]);
+    wait_vm_slabs<LOADS, NS - 2>(ktiles - 1);
+    wait_lgkm0(); // (the row and column sums are in LDS before anyone passes the barrier)
+    __builtin_amdgcn_s_barrier();
+    static_for<16>([&](auto f_tag) { read_frag(st[0], integral_constant<int, 0>{}, f_tag); });
+
+    // P: the fragment set that holds slab kt.  ISSUE / AHEAD as in the f32 kernel of wk_gemm_dma.hip.
+    auto iteration = [&](auto parity_tag, auto issue_tag, auto ahead_tag) __attribute__((always_inline)) {
+        constexpr int P = decltype(parity_tag)::value;
+        constexpr bool ISSUE = decltype(issue_tag)::value;
+        constexpr int AHEAD = decltype(ahead_tag)::value;
+        wait_lgkm0(); // the fragments of this slab
+        static_for<20>([&](auto n_tag) {
+            constexpr int N = decltype(n_tag)::value;
+            mfma_n(integral_constant<int, P>{}, n_tag);
+            if constexpr (ISSUE && N % 2 == 0 && N < 16) issue_one(st[NS - 1], integral_constant<int, N / 2>{});
+        });
+        if constexpr (AHEAD >= 0) {
+            wait_vm<AHEAD * LOADS>();
+            __builtin_amdgcn_s_barrier();
+        }
+        static_for<20>([&](auto n_tag) {
+            constexpr int N = decltype(n_tag)::value;
+            mfma_n(integral_constant<int, P>{}, integral_constant<int, 20 + N>{});
+            if constexpr (AHEAD >= 0 && N < 16) read_frag(st[1], integral_constant<int, P ^ 1>{}, n_tag);
+        });
+        const uint32_t t = st[0];
+#pragma unroll
+        for (int n = 0; n + 1 < NS; ++n) st[n] = st[n + 1];
+        st[NS - 1] = t;
+    };
+    using std::integral_constant;
+    using T_ = std::true_type;
+    using F_ = std::false_type;
+    using P0 = integral_constant<int, 0>;
+    using P1 = integral_constant<int, 1>;
+    using STEADY = integral_constant<int, NS - 2>;
+    static_assert(NS == 3 || NS == 4, "the drain below is written out for these depths");
+    // The fragment sets swap with the slabs, so the loop runs two slabs per trip; the pack pass pads the
+    // planes of the 32-bit types to an even number of slabs (zero digits), which keeps the drain below to
+    // one fixed sequence per pipeline depth.
+    uint32_t kt = 0;
+    for (; kt + NS < ktiles; kt += 2) {
+        iteration(P0{}, T_{}, STEADY{});
+        iteration(P1{}, T_{}, STEADY{});
+    }
+    if constexpr (NS == 4) {
+        if (kt + 4 == ktiles) { // four left: the last slab is still to be requested
+            iteration(P0{}, T_{}, integral_constant<int, 2>{});
+            iteration(P1{}, F_{}, integral_constant<int, 1>{});
+        }
+    }
+    iteration(P0{}, F_{}, integral_constant<int, 0>{}); // two left
+    iteration(P1{}, F_{}, integral_constant<int, -1>{});
+
+    // the last matrix instructions' results are not back yet (eight passes of four clocks and change)
+    asm volatile("s_nop 15\n\ts_nop 15\n\ts_nop 15" ::: "memory");
+
+    // epilogue, as in the kernel above; the C_old values of all four blocks are requested before any is
+    // used (the fragment registers are free by now): a one-round launch pays every memory latency here in full
+    const uint32_t kc2 = g.K * (CBIAS * CBIAS);
+    uint32_t *C = static_cast<uint32_t *>(g.C);
+    uint32_t old[2][2][16];
+    if (g.epi == EPI_ALPHA_BETA) {
+#pragma unroll
+        for (int am = 0; am < 2; ++am)
+#pragma unroll
+            for (int blk = 0; blk < 2; ++blk) {
+                const uint32_t col = n0 + wn * 64 + blk * 32 + l32, colc = EDGE ? min(col, g.N - 1) : col;
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    const uint32_t row = m0 + (wm * 2 + am) * 32 + 8 * (r / 4) + 4 * lhi + (r % 4);
+                    old[am][blk][r] = C[(size_t)(EDGE ? min(row, g.M - 1) : row) * g.ldc + colc];
+                }
+            }
+    }
+#pragma unroll
+    for (int am = 0; am < 2; ++am)
+#pragma unroll
+        for (int blk = 0; blk < 2; ++blk) {
+            const uint32_t lcol = wn * 64 + blk * 32 + l32, col = n0 + lcol;
+            const uint32_t csum = col_sum[lcol];
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const uint32_t lrow = (wm * 2 + am) * 32 + 8 * (r / 4) + 4 * lhi + (r % 4), row = m0 + lrow;
+                uint32_t v = 0;
+#pragma unroll
+                for (int s = 0; s < 4; ++s) v += (uint32_t)acc[s][am][blk][r] << (8 * s);
+                v += CBIAS * (row_sum[lrow] + csum) - kc2;
+                if (g.epi == EPI_ALPHA) v = g.alpha * v;
+                else if (g.epi == EPI_ALPHA_BETA) v = g.alpha * v + g.beta * old[am][blk][r];
+                if (!EDGE || ((row < g.M) & (col < g.N))) C[(size_t)row * g.ldc + col] = v;
+            }
+        }
+}
+
+template <bool EDGE, int NS> int launch_packed_dma(hipStream_t st, PArgs g) {
+    constexpr size_t lds = PackedDmaTile::lds_bytes(NS);
+    auto kern = gemm_i32_packed_dma_kernel<EDGE, NS>;
+    static const hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
+                                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    if (attr != hipSuccess) { (void)hipGetLastError(); return hip_code(attr); }
+    g.tiles_m = (g.M + TILE - 1) / TILE;
+    g.tiles_n = (g.N + TILE - 1) / TILE;
+    g.patch_m = g.patch_n = 0;
+    static const unsigned shapes[][2] = {{4, 8}, {4, 4}, {2, 8}, {2, 4}};
+    for (const auto &sh : shapes)
+        if (g.tiles_m % sh[0] == 0 && g.tiles_n % sh[1] == 0 && ((g.tiles_m / sh[0]) * (g.tiles_n / sh[1])) % 8 == 0) {
+            g.patch_m = sh[0];
+            g.patch_n = sh[1];
+            break;
+        }
+    hipLaunchKernelGGL(kern, dim3(g.tiles_m * g.tiles_n), dim3(256), lds, st, g);
+    return launch_status();
+}
+
 int digits_of(int dtype) {
     switch (dtype) {
     case WK_I8: case WK_U8: return 1;
@@ -511,7 +779,13 @@ template <typename E> int launch_typed(hipStream_t st, const GemmProblem &p, uns
         }
     }
     const bool edge = p.M % TILE != 0 || p.N % TILE != 0;
-    return edge ? launch_packed<E, 128, true>(st, g) : launch_packed<E, 128, false>(st, g);
+    if constexpr (D == 4) {
+        // 32 bits: the direct-to-LDS kernel, four stages (three measured 1-2 % slower; the 8-wavefront kernel
+        // above: 8192^3 222-226 against 274-280 TOP/s, 4096^3 212-226 against 249-257, 2048^3 187-190 against 218-225)
+        return edge ? launch_packed_dma<true, 4>(st, g) : launch_packed_dma<false, 4>(st, g);
+    } else {
+        return edge ? launch_packed<E, 128, true>(st, g) : launch_packed<E, 128, false>(st, g);
+    }
 }
 
 } // namespace
