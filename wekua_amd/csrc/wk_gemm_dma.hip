@@ -612,22 +612,13 @@ void gemm_f64_dma_kernel(DArgsD g) {
         for (; kt + 2 < ktiles; ++kt) iteration(P0{}, T_{}, T_{});
         if (kt + 1 < ktiles) iteration(P0{}, F_{}, T_{});
         iteration(P0{}, F_{}, F_{});
-    } else { // sets alternate with the slabs: two iterations per trip, then the last one or two by parity
+    } else { // sets alternate with the slabs: two iterations per trip; K % 16 == 0 makes the slab count even
         for (; kt + 3 < ktiles; kt += 2) {
             iteration(P0{}, T_{}, T_{});
             iteration(P1{}, T_{}, T_{});
         }
-        // here kt is even and 1 <= ktiles - kt <= 3
-        if (kt + 2 < ktiles) { // three left
-            iteration(P0{}, T_{}, T_{});
-            iteration(P1{}, F_{}, T_{});
-            iteration(P0{}, F_{}, F_{});
-        } else if (kt + 1 < ktiles) { // two left
-            iteration(P0{}, F_{}, T_{});
-            iteration(P1{}, F_{}, F_{});
-        } else {
-            iteration(P0{}, F_{}, F_{});
-        }
+        iteration(P0{}, F_{}, T_{}); // two left
+        iteration(P1{}, F_{}, F_{});
     }
 
     const double alpha = g.alpha, beta = g.beta;
