@@ -78,7 +78,8 @@ def test_float_small_shapes(dev, dtype, op_a, op_b, alpha, beta):
 
 @pytest.mark.parametrize("variant", ["tile64", "mfma_f32_64x64", "mfma_f32_64x64s2", "mfma_f32_64x64s4", "mfma_f32_32x32s4",
                                      "mfma_f32_64x64z", "mfma_f32_128x128", "mfma_f32_128x128s2", "mfma_f32_256x128",
-                                     "mfma_f32_128x128t", "mfma_f32_256x128t", "mfma_f32_256x128d", "mfma_f32_128x128d", "mfma_f32_64x64d"])
+                                     "mfma_f32_128x128t", "mfma_f32_256x128t", "mfma_f32_256x128d", "mfma_f32_128x128d", "mfma_f32_64x64d",
+                                     "mfma_f32_128x128d2", "mfma_f32_64x64d2"])
 @pytest.mark.parametrize("op_a,op_b", OPS)
 def test_f32_every_variant(dev, variant, op_a, op_b):
     import ctypes
@@ -295,14 +296,15 @@ def test_one_round_launches_take_the_k_split_tiles(dev):
     # (the name query assumes 256 compute units and 16-byte aligned operands)
     # f32 operands whose rows start on 16-byte boundaries take the kernels that bring their slabs straight
     # into LDS, whose three stages already give a lone work-group something to overlap with ...
-    assert name("f32", 1024, 1024, 1024) == b"mfma_f32_64x64d"
-    assert name("f32", 2048, 1024, 1024) == b"mfma_f32_64x64d"
-    assert name("f32", 1024, 1024, 128) == b"mfma_f32_64x64d"
-    assert name("f32", 896, 896, 896) == b"mfma_f32_64x64d"
-    assert name("f32", 2048, 2048, 2048) == b"mfma_f32_128x128d"   # one full round of 128x128 tiles
+    assert name("f32", 1024, 1024, 1024) == b"mfma_f32_64x64d2"    # one round: two groups of wavefronts per tile
+    assert name("f32", 1000, 1000, 1000) == b"mfma_f32_64x64d2"    # ragged, rows of 4000 bytes
+    assert name("f32", 2048, 1024, 1024) == b"mfma_f32_64x64d"     # two rounds
+    assert name("f32", 1024, 1024, 128) == b"mfma_f32_64x64d"      # short k
     assert name("f32", 1536, 1536, 1536) == b"mfma_f32_64x64d"
-    assert name("f32", 1000, 1000, 1000) == b"mfma_f32_64x64d"     # ragged, rows of 4000 bytes
-    assert name("f32", 2040, 2040, 2040) == b"mfma_f32_128x128d"
+    assert name("f32", 2048, 2048, 2048) == b"mfma_f32_128x128d2"  # one full round of 128x128 tiles
+    assert name("f32", 2040, 2040, 2040) == b"mfma_f32_128x128d2"
+    assert name("f32", 2048, 2048, 512) == b"mfma_f32_128x128d"
+    assert dev.lib.wk_gemm_variant(raw.dtype_id("f32"), 1, 0, 1024, 1024, 1024, 1024, 1024, 1024, None, None, None) == b"mfma_f32_64x64d"  # T,N
     # ... any other leading dimension the register-staged tile and its k-split twins
     assert name("f32", 1001, 1001, 1001) == b"mfma_f32_64x64s4"
     assert name("f32", 2041, 1001, 1001) == b"mfma_f32_64x64s2"
@@ -375,6 +377,7 @@ def test_k_split_over_work_groups(dev, dtype):
 
 
 @pytest.mark.parametrize("variant,bm,bn", [("mfma_f32_256x128d", 256, 128), ("mfma_f32_128x128d", 128, 128), ("mfma_f32_64x64d", 64, 64),
+                                           ("mfma_f32_128x128d2", 128, 128), ("mfma_f32_64x64d2", 64, 64),
                                            ("mfma_f64_128x128d", 128, 128), ("mfma_f64_64x64d", 64, 64)])
 @pytest.mark.parametrize("op_a,op_b", OPS)
 def test_slabs_straight_into_lds(dev, variant, bm, bn, op_a, op_b):
@@ -408,7 +411,8 @@ def test_slabs_straight_into_lds(dev, variant, bm, bn, op_a, op_b):
         dev.lib.wk_gemm_force_variant(b"auto")
 
 
-@pytest.mark.parametrize("variant,bm,bn", [("mfma_f32_256x128d", 256, 128), ("mfma_f32_128x128d", 128, 128), ("mfma_f32_64x64d", 64, 64)])
+@pytest.mark.parametrize("variant,bm,bn", [("mfma_f32_256x128d", 256, 128), ("mfma_f32_128x128d", 128, 128), ("mfma_f32_64x64d", 64, 64),
+                                           ("mfma_f32_64x64d2", 64, 64)])
 def test_tile_walk_in_patches_covers_every_tile_once(dev, variant, bm, bn):
     """The f32 direct-to-LDS kernels number their tiles in XCD-local patches (4 x 8, 4 x 4, 2 x 8 or 2 x 4
     tiles, eight patches at a time) when the tile grid divides into them and in groups of tile rows

@@ -58,22 +58,30 @@ struct DArgs {
     uint32_t patch_m, patch_n; // tile walk in XCD-local patches of patch_m x patch_n tiles (0: rows of groups)
 };
 
-template <int BM, int BN, int BK, int NS, int OCC, bool A_K, bool B_K, bool EXT>
-__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(OCC)))
+// KS: groups of 2 x 2 wavefronts on the same tile (1 or 2).  A launch of one round of tiles leaves every SIMD
+// a single wavefront, which stands still at every wait; with KS = 2 all eight wavefronts bring the slabs
+// in, group kg multiplies steps kg * S / KS ... of every slab, and the two partial tiles are added
+// through LDS (the stages, free by then) before group 0 runs the epilogue.
+template <int BM, int BN, int BK, int NS, int OCC, bool A_K, bool B_K, bool EXT, int KS = 1>
+__global__ __launch_bounds__(256 * KS) __attribute__((amdgpu_waves_per_eu(OCC)))
 void gemm_f32_dma_kernel(DArgs g) {
     constexpr int WM = BM / 2, WN = BN / 2, FM = WM / 32, FN = WN / 32;
     constexpr int S = BK / 8;   // fragment steps per slab (8 values of k each: four matrix instructions per block)
     constexpr int CPR = BK / 4; // 16-byte chunks per row of a k-contiguous slab
     constexpr int A_FLOATS = BM * BK, B_FLOATS = BN * BK, STAGE = A_FLOATS + B_FLOATS;
-    constexpr int A_LOADS = BM * BK / 1024, B_LOADS = BN * BK / 1024; // 1 KB per wavefront and load, four wavefronts
+    constexpr int WAVES = 4 * KS;
+    constexpr int SG = S / KS; // steps of a slab per group of wavefronts
+    constexpr int A_LOADS = BM * BK / (256 * WAVES), B_LOADS = BN * BK / (256 * WAVES); // 1 KB per wavefront and load
     static_assert(BM % 64 == 0 && BN % 64 == 0 && (BK == 16 || BK == 32) && NS >= 3, "tile shape");
+    static_assert((KS == 1 || KS == 2) && SG >= 2 && SG % 2 == 0 && A_LOADS >= 1 && B_LOADS >= 1, "k-groups");
 
     extern __shared__ __align__(16) float lds[]; // [NS][STAGE]: A then B
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6); // the same in every lane: kept in a scalar register
-    const int wm = wave >> 1, wn = wave & 1;
+    const int kg = wave >> 2;                                  // k-group of this wavefront
+    const int wm = (wave >> 1) & 1, wn = wave & 1;
     const int l32 = lane & 31, lhi = lane >> 5;
 
     // tile walk: groups of GROUP_M tile rows, as in wk_gemm_mfma.hip (every XCD sweeps the same panel of B)
@@ -139,9 +147,9 @@ void gemm_f32_dma_kernel(DArgs g) {
     using std::integral_constant;
     const uint32_t m_last = g.M - 1 - m0, n_last = g.N - 1 - n0;
 #pragma unroll
-    for (int i = 0; i < A_LOADS; ++i) a_off[i] = lane_offset(i * 4 + wave, g.lda, m_last, integral_constant<bool, A_K>{}, integral_constant<int, BM>{});
+    for (int i = 0; i < A_LOADS; ++i) a_off[i] = lane_offset(i * WAVES + wave, g.lda, m_last, integral_constant<bool, A_K>{}, integral_constant<int, BM>{});
 #pragma unroll
-    for (int i = 0; i < B_LOADS; ++i) b_off[i] = lane_offset(i * 4 + wave, g.ldb, n_last, integral_constant<bool, B_K>{}, integral_constant<int, BN>{});
+    for (int i = 0; i < B_LOADS; ++i) b_off[i] = lane_offset(i * WAVES + wave, g.ldb, n_last, integral_constant<bool, B_K>{}, integral_constant<int, BN>{});
     const uint32_t lds0 =
         __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)(__attribute__((address_space(3))) float *)lds); // byte address of the array
 
@@ -150,9 +158,9 @@ void gemm_f32_dma_kernel(DArgs g) {
     auto issue = [&](uint32_t stage_bytes) {
         const uint32_t sbase = lds0 + stage_bytes + (uint32_t)wave * 1024u;
 #pragma unroll
-        for (int i = 0; i < A_LOADS; ++i) dma16(a_base, a_off[i], sbase + (uint32_t)i * 4096u);
+        for (int i = 0; i < A_LOADS; ++i) dma16(a_base, a_off[i], sbase + (uint32_t)i * (WAVES * 1024u));
 #pragma unroll
-        for (int i = 0; i < B_LOADS; ++i) dma16(b_base, b_off[i], sbase + A_FLOATS * 4u + (uint32_t)i * 4096u);
+        for (int i = 0; i < B_LOADS; ++i) dma16(b_base, b_off[i], sbase + A_FLOATS * 4u + (uint32_t)i * (WAVES * 1024u));
         a_base += a_step;
         b_base += b_step;
     };
@@ -177,9 +185,9 @@ void gemm_f32_dma_kernel(DArgs g) {
     };
     auto tail_offsets = [&]() {
 #pragma unroll
-        for (int i = 0; i < A_LOADS; ++i) a_off[i] = tail_offset(a_off[i], i * 4 + wave, g.lda, integral_constant<bool, A_K>{}, integral_constant<int, BM>{});
+        for (int i = 0; i < A_LOADS; ++i) a_off[i] = tail_offset(a_off[i], i * WAVES + wave, g.lda, integral_constant<bool, A_K>{}, integral_constant<int, BM>{});
 #pragma unroll
-        for (int i = 0; i < B_LOADS; ++i) b_off[i] = tail_offset(b_off[i], i * 4 + wave, g.ldb, integral_constant<bool, B_K>{}, integral_constant<int, BN>{});
+        for (int i = 0; i < B_LOADS; ++i) b_off[i] = tail_offset(b_off[i], i * WAVES + wave, g.ldb, integral_constant<bool, B_K>{}, integral_constant<int, BN>{});
     };
     auto tail_zero = [&](float *dst, int grp, auto kc_tag, auto rows_tag) { // dst: this lane's 16 bytes of the load
         constexpr bool KC = decltype(kc_tag)::value;
@@ -199,9 +207,9 @@ void gemm_f32_dma_kernel(DArgs g) {
     auto tail_zeros = [&](uint32_t stage_bytes) {
         float *base = lds + stage_bytes / 4 + wave * 256 + lane * 4;
 #pragma unroll
-        for (int i = 0; i < A_LOADS; ++i) tail_zero(base + i * 1024, i * 4 + wave, integral_constant<bool, A_K>{}, integral_constant<int, BM>{});
+        for (int i = 0; i < A_LOADS; ++i) tail_zero(base + i * (WAVES * 256), i * WAVES + wave, integral_constant<bool, A_K>{}, integral_constant<int, BM>{});
 #pragma unroll
-        for (int i = 0; i < B_LOADS; ++i) tail_zero(base + A_FLOATS + i * 1024, i * 4 + wave, integral_constant<bool, B_K>{}, integral_constant<int, BN>{});
+        for (int i = 0; i < B_LOADS; ++i) tail_zero(base + A_FLOATS + i * (WAVES * 256), i * WAVES + wave, integral_constant<bool, B_K>{}, integral_constant<int, BN>{});
     };
 
     // ---- LDS side: per-lane fragment addresses (floats from the start of a stage's A or B part) ----
@@ -215,6 +223,12 @@ void gemm_f32_dma_kernel(DArgs g) {
 #pragma unroll
     for (int j = 0; j < FN; ++j)
         b_frag[j] = B_K ? (wn * WN + l32) * BK + sw4 : 4 * lhi * BN + (((wn * WN + 32 * j) ^ (32 * lhi)) + l32);
+    if constexpr (KS > 1) { // group kg starts at step kg * SG of every slab (SG a power of two: the bits do not meet)
+#pragma unroll
+        for (int i = 0; i < FM; ++i) a_frag[i] = A_K ? a_frag[i] ^ (8 * SG * kg) : a_frag[i] + 8 * SG * kg * BM;
+#pragma unroll
+        for (int j = 0; j < FN; ++j) b_frag[j] = B_K ? b_frag[j] ^ (8 * SG * kg) : b_frag[j] + 8 * SG * kg * BN;
+    }
 
     auto read_frags = [&](uint32_t stage_bytes, int s, f32x4 *af, f32x4 *bf) {
         const float *as = lds + stage_bytes / 4;
@@ -275,7 +289,7 @@ void gemm_f32_dma_kernel(DArgs g) {
     constexpr bool PRELOAD_C = FM * FN == 1;
     float c_old[PRELOAD_C ? 16 : 1];
     if constexpr (PRELOAD_C) {
-        if (g.epi == EPI_ALPHA_BETA) {
+        if (g.epi == EPI_ALPHA_BETA && (KS == 1 || kg == 0)) {
             const uint32_t colc = min(n0 + wn * WN + l32, g.N - 1);
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
@@ -311,7 +325,7 @@ void gemm_f32_dma_kernel(DArgs g) {
         constexpr int AHEAD = decltype(ahead_tag)::value;
         if constexpr (ISSUE) issue(st[NS - 1]);
 #pragma unroll
-        for (int s = 0; s + 1 < S; ++s) {
+        for (int s = 0; s + 1 < SG; ++s) {
             read_frags(st[0], s + 1, af[(s + 1) & 1], bf[(s + 1) & 1]);
             mfma_step(s);
         }
@@ -326,7 +340,7 @@ void gemm_f32_dma_kernel(DArgs g) {
             read_frags(st[1], 0, af[0], bf[0]);
             __builtin_amdgcn_sched_barrier(0);
         }
-        mfma_step(S - 1);
+        mfma_step(SG - 1);
         const uint32_t t = st[0];
 #pragma unroll
         for (int n = 0; n + 1 < NS; ++n) st[n] = st[n + 1];
@@ -354,6 +368,29 @@ void gemm_f32_dma_kernel(DArgs g) {
     // ---- epilogue: acc register r of lane l is C[8*(r/4) + 4*(l/32) + r%4][l%32] of its 32x32 block;
     // option semantics of src/blas/gemm.zig:500-501,591-602 (C_old is read and multiplied whenever beta
     // is given); the reads of C_old of a block are issued as one batch
+    if constexpr (KS > 1) {
+        // the partial tile of group 1 goes through LDS to group 0: register r of block (i, j) of wavefront
+        // (wm, wn) at float ((4 wm + 2 wn ... ) below, consecutive lanes on consecutive floats
+        static_assert(4 * FM * FN * 16 * 64 <= NS * STAGE, "the partial tile fits the stages");
+        __builtin_amdgcn_s_barrier(); // every wavefront is done with the stages (its last reads were waited for)
+        float *part = lds + ((wave & 3) * FM * FN) * 16 * 64 + lane;
+        if (kg == 1) {
+#pragma unroll
+            for (int i = 0; i < FM; ++i)
+#pragma unroll
+                for (int j = 0; j < FN; ++j)
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) part[((i * FN + j) * 16 + r) * 64] = acc[i][j][r];
+        }
+        __syncthreads();
+        if (kg == 1) return;
+#pragma unroll
+        for (int i = 0; i < FM; ++i)
+#pragma unroll
+            for (int j = 0; j < FN; ++j)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) acc[i][j][r] += part[((i * FN + j) * 16 + r) * 64];
+    }
     // Tiles that reach beyond C clamp the addresses of C_old and the bias and skip the stores there.
     const float alpha = g.alpha, beta = g.beta;
     auto epilogue = [&](auto checked_tag) {
@@ -697,9 +734,9 @@ template <int BM, int BN, int BK, int OCC> int launch_tile_d(hipStream_t st, con
 }
 
 // first_tiles: launch only that many tiles, in tile-walk order (0: all of them)
-template <int BM, int BN, int BK, int NS, int OCC, bool A_K, bool B_K, bool EXT> int launch_one(hipStream_t st, const DArgs &g, uint64_t first_tiles) {
-    constexpr size_t lds_bytes = NS * (BM * BK + BN * BK) * sizeof(float); // 3 x 24 KB / 3 x 16 KB / 4 x 16 KB
-    auto kern = gemm_f32_dma_kernel<BM, BN, BK, NS, OCC, A_K, B_K, EXT>;
+template <int BM, int BN, int BK, int NS, int OCC, bool A_K, bool B_K, bool EXT, int KS = 1> int launch_one(hipStream_t st, const DArgs &g, uint64_t first_tiles) {
+    constexpr size_t lds_bytes = NS * (BM * BK + BN * BK) * sizeof(float); // 3 x 24 KB / 3 x 16 KB / 3 x 32 KB
+    auto kern = gemm_f32_dma_kernel<BM, BN, BK, NS, OCC, A_K, B_K, EXT, KS>;
     static const int attr_rc = [&] {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
                                            (int)lds_bytes);
@@ -711,11 +748,11 @@ template <int BM, int BN, int BK, int NS, int OCC, bool A_K, bool B_K, bool EXT>
     }();
     if (attr_rc) return attr_rc;
     const unsigned grid = first_tiles ? (unsigned)first_tiles : g.tiles_m * g.tiles_n;
-    hipLaunchKernelGGL(kern, dim3(grid), dim3(256), lds_bytes, st, g);
+    hipLaunchKernelGGL(kern, dim3(grid), dim3(256 * KS), lds_bytes, st, g);
     return launch_status();
 }
 
-template <int BM, int BN, int BK, int NS, int OCC> int launch_tile(hipStream_t st, const GemmProblem &p, uint64_t first_tiles) {
+template <int BM, int BN, int BK, int NS, int OCC, int KS = 1> int launch_tile(hipStream_t st, const GemmProblem &p, uint64_t first_tiles) {
     if (first_tiles > ((p.M + BM - 1) / BM) * ((p.N + BN - 1) / BN)) return WK_E_INVALID_VALUE;
     DArgs g{};
     g.A = static_cast<const float *>(p.A);
@@ -747,13 +784,17 @@ template <int BM, int BN, int BK, int NS, int OCC> int launch_tile(hipStream_t s
             }
     }
     const int sel = (p.op_a ? 0 : 2) | (p.op_b ? 1 : 0); // bit 1: A k-contiguous, bit 0: B k-contiguous
-    if (p.ext) // instantiated for op N, T only (what Linear.forward runs)
-        return sel == 3 ? launch_one<BM, BN, BK, NS, OCC, true, true, true>(st, g, first_tiles) : (int)WK_E_INVALID_VALUE;
+    if (p.ext) { // instantiated for op N, T only (what Linear.forward runs), one group of wavefronts
+        if constexpr (KS == 1)
+            return sel == 3 ? launch_one<BM, BN, BK, NS, OCC, true, true, true>(st, g, first_tiles) : (int)WK_E_INVALID_VALUE;
+        else
+            return WK_E_INVALID_VALUE;
+    }
     switch (sel) {
-    case 0: return launch_one<BM, BN, BK, NS, OCC, false, false, false>(st, g, first_tiles);
-    case 1: return launch_one<BM, BN, BK, NS, OCC, false, true, false>(st, g, first_tiles);
-    case 2: return launch_one<BM, BN, BK, NS, OCC, true, false, false>(st, g, first_tiles);
-    default: return launch_one<BM, BN, BK, NS, OCC, true, true, false>(st, g, first_tiles);
+    case 0: return launch_one<BM, BN, BK, NS, OCC, false, false, false, KS>(st, g, first_tiles);
+    case 1: return launch_one<BM, BN, BK, NS, OCC, false, true, false, KS>(st, g, first_tiles);
+    case 2: return launch_one<BM, BN, BK, NS, OCC, true, false, false, KS>(st, g, first_tiles);
+    default: return launch_one<BM, BN, BK, NS, OCC, true, true, false, KS>(st, g, first_tiles);
     }
 }
 
@@ -795,8 +836,13 @@ int wk::gemm_f64_dma_launch(hipStream_t st, const GemmProblem &p, int bm, int bn
     return launch_tile_d<64, 64, 16, 3>(st, p);
 }
 
-int wk::gemm_f32_dma_launch(hipStream_t st, const GemmProblem &p, int bm, int bn, uint64_t first_tiles) {
+int wk::gemm_f32_dma_launch(hipStream_t st, const GemmProblem &p, int bm, int bn, uint64_t first_tiles, int k_groups) {
     if (!gemm_f32_dma_applies(p, bm, bn)) return WK_E_INVALID_VALUE;
+    if (k_groups == 2) { // eight wavefronts per tile, k-slabs of 32 (128 x 128: one work-group per unit, 96 KB of stages)
+        if (p.ext || first_tiles || bm == 256) return WK_E_INVALID_VALUE;
+        if (bm == 128) return launch_tile<128, 128, 32, 3, 2, 2>(st, p, 0);
+        return launch_tile<64, 64, 32, 3, 4, 2>(st, p, 0);
+    }
     if (bm == 256) return launch_tile<256, 128, 16, 3, 2>(st, p, first_tiles);
     if (bm == 128) return launch_tile<128, 128, 16, 3, 3>(st, p, first_tiles);
     // (k-slabs of 32, three work-groups per unit; with slabs of 16 and four: 1024^3 101 against 103.5 TFLOP/s,

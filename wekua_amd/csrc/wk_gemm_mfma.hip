@@ -1398,6 +1398,13 @@ template <int BM, int BN, int BK, int OCC> int launch_f32_dma(hipStream_t st, co
     return launch_f32<BM, BN, BK, 2, 2, OCC>(st, p, edge);
 }
 
+// two groups of wavefronts per tile on the direct-to-LDS kernel; elsewhere the k-split twin of the staged tile
+template <int BM, int BN> int launch_f32_dma2(hipStream_t st, const GemmProblem &p, bool edge) {
+    if (!p.ext && gemm_f32_dma_applies(p, BM, BN)) return gemm_f32_dma_launch(st, p, BM, BN, 0, 2);
+    if (BM == 128) return launch_f32<128, 128, 16, 2, 2, 2, 2>(st, p, edge);
+    return launch_f32<64, 64, 16, 2, 2, 4, 4>(st, p, edge);
+}
+
 template <int BM, int BN, int BK, int OCC> int launch_f64_dma(hipStream_t st, const GemmProblem &p, bool edge) {
     if (gemm_f64_dma_applies(p, BM, BN)) return gemm_f64_dma_launch(st, p, BM, BN);
     return launch_f64<BM, BN, BK, 2, 2, OCC>(st, p, edge);
@@ -1439,11 +1446,17 @@ const VariantDesc k_variants[] = {
     {"mfma_f32_256x128d", WK_F32, 256, 128, 16, 0.943, 0.08, &launch_f32_dma<256, 128, 16, 2>, nullptr, nullptr, nullptr, nullptr,
      "mfma_f32_256x128t", 2},
     // 2048 x 4096 x 4096: N,T 143.0 (staged 139.6), N,N 141.8 (132.0); 4096^3 144
-    {"mfma_f32_128x128d", WK_F32, 128, 128, 16, 0.922, 0.08, &launch_f32_dma<128, 128, 16, 3>, nullptr, nullptr, nullptr, nullptr,
+    {"mfma_f32_128x128d", WK_F32, 128, 128, 16, 0.922, 0.08, &launch_f32_dma<128, 128, 16, 3>, "mfma_f32_128x128d2", nullptr, nullptr, nullptr,
      "mfma_f32_128x128t", 3},
     // 3072^3 129.7 (staged 120.4), 2048 x 1024 x 4096 132 (126), 1024^3 103.7 (101.5 with four k-groups)
-    {"mfma_f32_64x64d", WK_F32, 64, 64, 32, 0.84, 0.10, &launch_f32_dma<64, 64, 32, 4>, nullptr, nullptr, "mfma_f32_32x32s4",
+    {"mfma_f32_64x64d", WK_F32, 64, 64, 32, 0.84, 0.10, &launch_f32_dma<64, 64, 32, 4>, "mfma_f32_64x64d2", nullptr, "mfma_f32_32x32s4",
      "mfma_f32_64x64z"},
+    // eight wavefronts per tile in two k-groups, for launches of one round (see gemm_f32_dma_kernel).  Measured
+    // against the one-group kernels (N,N / N,T / T,N / T,T, TFLOP/s): 2048^3 129.5 / 132.6 / 122.9 / 129.7 ->
+    // 133.7 / 137.2 / 129.1 / 133.2, 1024 x 4096 x 2048 T,N 123.9 -> 128.0; 64 x 64: 1024^3 102 / 101 / 105 / 102 ->
+    // 105 / 106 / 97 / 103, 1024 x 1024 x 4096 121 / 120 / 124 / 119 -> 124 / 127 / 120 / 123: not for T,N there
+    {"mfma_f32_128x128d2", WK_F32, 128, 128, 32, 0.0, 0.08, &launch_f32_dma2<128, 128>},
+    {"mfma_f32_64x64d2", WK_F32, 64, 64, 32, 0.0, 0.10, &launch_f32_dma2<64, 64>},
     {"mfma_f32_256x128t", WK_F32, 256, 128, 16, 0.0, 0.25, &launch_f32_tail<256, 128, 16, 2, 2, 2>, nullptr, nullptr, nullptr, nullptr,
      nullptr, 2}, // whole rounds + a k-split tail
     {"mfma_f32_128x128", WK_F32, 128, 128, 16, 0.897, 0.19, &launch_f32<128, 128, 16, 2, 2, 3>, nullptr, nullptr, nullptr, nullptr,
@@ -1605,7 +1618,9 @@ int wk::gemm_mfma_pick(const GemmProblem &p) {
         const double tiles128 = (double)((p.M + 127) / 128) * (double)((p.N + 127) / 128);
         if (tiles128 <= cus && tiles128 >= 0.85 * cus) {
             // (the direct-to-LDS kernel of that tile where it applies: 2048^3 N,N 131 against 128.5)
-            const char *want = gemm_f32_dma_applies(p, 128, 128) ? "mfma_f32_128x128d" : "mfma_f32_128x128s2";
+            const char *want = !gemm_f32_dma_applies(p, 128, 128) ? "mfma_f32_128x128s2"
+                               : (p.K >= 1024 && !p.ext)           ? "mfma_f32_128x128d2"
+                                                                   : "mfma_f32_128x128d";
             for (int v = 0; v < k_num_variants; ++v)
                 if (!std::strcmp(k_variants[v].name, want)) return v;
         }
@@ -1627,6 +1642,10 @@ int wk::gemm_mfma_pick(const GemmProblem &p) {
             twin = d.split;
         else if (tiles <= 0.75 * cus && d.sparse) twin = d.sparse; // (f64 512^3: 21.5 -> 10.3 us, 512x512x2048: 74 -> 32 us)
         else if (p.K >= 256) twin = tiles <= cus ? d.one_round : (tiles <= 2.0 * cus ? d.two_rounds : nullptr);
+        if (twin && twin == d.one_round && is_dma_variant(d.name)) { // the two-group direct-to-LDS kernels: not fused
+            if (p.ext || p.K < (d.bm == 64 ? 512u : 1024u)) twin = nullptr; // (below: equal)
+            else if (d.bm == 64 && p.op_a && !p.op_b) twin = nullptr;       // 64 x 64, T,N: the one-group kernel is faster
+        }
         for (int v = 0; twin && v < k_num_variants; ++v)
             if (!std::strcmp(k_variants[v].name, twin)) return v;
     }
