@@ -839,6 +839,8 @@ int wk::gemm_f64_dma_launch(hipStream_t st, const GemmProblem &p, int bm, int bn
 int wk::gemm_f32_dma_launch(hipStream_t st, const GemmProblem &p, int bm, int bn, uint64_t first_tiles, int k_groups) {
     if (!gemm_f32_dma_applies(p, bm, bn)) return WK_E_INVALID_VALUE;
     if (k_groups == 2) { // eight wavefronts per tile, k-slabs of 32 (128 x 128: one work-group per unit, 96 KB of stages)
+        // (the 256 x 128 tile with two groups, 144 KB of stages, measured no better than two work-groups of the
+        // 128 x 128 tile where it would apply: 2048 x 4096 x 4096 143 against 143 TFLOP/s, 4096 x 2048 x 2048 138 against 139)
         if (p.ext || first_tiles || bm == 256) return WK_E_INVALID_VALUE;
         if (bm == 128) return launch_tile<128, 128, 32, 3, 2, 2>(st, p, 0);
         return launch_tile<64, 64, 32, 3, 4, 2>(st, p, 0);
