@@ -153,7 +153,7 @@ def test_axpy_pitched_regions(dev, dtype):
 @pytest.mark.parametrize("dtype", ["f32", "f64"])
 @pytest.mark.parametrize("n", [2 ** 20, 2 ** 24])
 def test_axpy_config_sizes(dev, dtype, n):
-    """BASELINE config 2 at the sizes the oracle finishes in seconds (2^28: see the property test)."""
+    """Benchmark configuration 2 at the sizes the oracle finishes in seconds (2^28: see the property test)."""
     x = make_operand(dtype, (n,), 0x5EED0020)
     y = make_operand(dtype, (n,), 0x5EED0021)
     got = run_axpy(dev, dtype, x, 0.75, y)

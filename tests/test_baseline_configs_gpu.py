@@ -1,4 +1,4 @@
-"""GPU: the benchmark configurations (BASELINE.json `configs`) at their real sizes.
+"""GPU: the benchmark configurations at their real sizes.
 
 Shapes the oracle finishes in seconds are compared entry by entry with it.  The large ones
 (>= 4096^3) are checked through properties that do not need a second full product:

@@ -375,7 +375,7 @@ def test_xor_example_trains(env):
 
 
 def test_config5_mlp_training_step_full_size(env):
-    """BASELINE configuration 5: 1024-4096-4096-1024, f32, batch 2048, tanh hidden / sigmoid output,
+    """Benchmark configuration 5: 1024-4096-4096-1024, f32, batch 2048, tanh hidden / sigmoid output,
     MSE against uniform[0,1) targets, Adam lr = 1e-3, N(0,1) inputs, Xavier-uniform weights."""
     context, pipeline = env
     sizes, acts, batch = [1024, 4096, 4096, 1024], [onn.TANH, onn.TANH, onn.SIGMOID], 2048

@@ -4,7 +4,7 @@ times over 1-D sizes, on GPU 0.
 
     python -m wekua_amd.benchmark gemm [--dtype f32] [--sizes 1024 2048 ...] [--shapes 8192x256x8192 ...] [--ops NN TN] [--variant NAME]
     python -m wekua_amd.benchmark axpy [--dtype f32]
-    python -m wekua_amd.benchmark configs        # every BASELINE GEMM / AXPY configuration, one line each
+    python -m wekua_amd.benchmark configs        # every GEMM / AXPY benchmark configuration, one line each
     python -m wekua_amd.benchmark tensor         # transpose / copy / random.uniform / toComplex streaming rates
     python -m wekua_amd.benchmark mlp [--dtype f32] [--sizes 1024 4096 4096 1024] [--batch 2048] [--optimizer adam]
 
@@ -269,7 +269,7 @@ def mlp_flops(sizes, batch):
 
 def time_mlp_step(dtype="f32", sizes=(1024, 4096, 4096, 1024), batch=2048, optimizer="adam", lr=1e-3, steps=20, warmup=3,
                   seed=None):
-    """One training step of BASELINE configuration 5 through the reference-shaped API: Sequential of
+    """One training step of benchmark configuration 5 through the reference-shaped API: Sequential of
     Linear layers (tanh hidden, sigmoid output), loss.mse with derivative, backward, optimizer step.
     Returns ms per step from events on the pipeline's stream and from the wall clock."""
     import ctypes
