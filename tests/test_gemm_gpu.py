@@ -427,6 +427,27 @@ def test_tile_walk_in_patches_covers_every_tile_once(dev, variant, bm, bn):
         dev.lib.wk_gemm_force_variant(b"auto")
 
 
+@pytest.mark.parametrize("variant", ["mfma_f32_256x128d", "mfma_f32_128x128d", "mfma_f32_64x64d", "mfma_f32_128x128d2", "mfma_f32_64x64d2"])
+def test_direct_to_lds_on_seeded_random_shapes(dev, variant):
+    """Twenty-four shapes drawn from a fixed seed (1 <= M, N <= 700, 1 <= K <= 900), leading dimensions a
+    multiple of four with or without a gap, every layout and option combination in turn: the f32 kernels
+    that bring their slabs straight into LDS against the oracle, border tiles and k tails included."""
+    rng = np.random.default_rng(20240611)
+    options = [(None, None), (2.0, None), (1.5, 0.5), (None, -0.25)]
+    assert dev.lib.wk_gemm_force_variant(variant.encode()) == 0
+    try:
+        for n in range(24):
+            M, N, K = int(rng.integers(1, 701)), int(rng.integers(1, 701)), int(rng.integers(1, 901))
+            op_a, op_b = OPS[n % 4]
+            alpha, beta = options[(n // 4) % 4]
+            cols_a, cols_b = (M if op_a else K), (K if op_b else N)
+            pad = 4 * int(rng.integers(0, 3))
+            check(dev, "f32", M, N, K, op_a, op_b, alpha, beta, seed=400 + n,
+                  lda=(cols_a + 3) // 4 * 4 + pad, ldb=(cols_b + 3) // 4 * 4 + pad, ldc=N + int(rng.integers(0, 4)))
+    finally:
+        dev.lib.wk_gemm_force_variant(b"auto")
+
+
 def test_left_over_tiles_run_as_a_k_split_tail(dev):
     """A launch whose tiles do not fill whole rounds of the compute units: the whole rounds run as they
     are, the left-over tiles as a second launch with k split over work-groups.  Checked: the plan of the
