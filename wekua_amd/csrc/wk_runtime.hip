@@ -279,16 +279,17 @@ int wk_memset_async(wk_stream *s, void *dptr, int byte, size_t bytes) {
 }
 
 // Device-to-device copy of a pitched region, one 16-byte vector per lane: blockIdx.y walks the
-// rows (all slices), blockIdx.x the 16-byte columns, so no lane divides anything per element.
-__global__ __launch_bounds__(256) void rect_copy16_kernel(char *__restrict__ dst, size_t drp, size_t dsp,
-                                                          const char *__restrict__ src, size_t srp, size_t ssp, size_t width16,
-                                                          size_t rows, size_t total_rows) {
+// rows (all slices), blockIdx.x the 16-byte columns, so no lane divides anything per element.  One
+// wavefront per work-group, like the AXPY kernels: latency is hidden by the number of work-groups in flight.
+__global__ __launch_bounds__(64) void rect_copy16_kernel(char *__restrict__ dst, size_t drp, size_t dsp,
+                                                         const char *__restrict__ src, size_t srp, size_t ssp, size_t width16,
+                                                         size_t rows, size_t total_rows) {
     for (size_t row = blockIdx.y; row < total_rows; row += gridDim.y) {
         const size_t z = row / rows, r = row % rows;
         typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
         const u32x4 *sp = reinterpret_cast<const u32x4 *>(src + z * ssp + r * srp);
         u32x4 *dp = reinterpret_cast<u32x4 *>(dst + z * dsp + r * drp);
-        for (size_t c = blockIdx.x * 256ull + threadIdx.x; c < width16; c += (size_t)gridDim.x * 256ull)
+        for (size_t c = blockIdx.x * 64ull + threadIdx.x; c < width16; c += (size_t)gridDim.x * 64ull)
             __builtin_nontemporal_store(__builtin_nontemporal_load(&sp[c]), &dp[c]);
     }
 }
@@ -312,11 +313,10 @@ static int rect_copy(wk_stream *s, void *dst, size_t drp, size_t dsp, const void
             d_rp = s_rp = w16 * 16;
         }
         const size_t total_rows = nrows * nslices;
-        const size_t gx = (w16 + 255) / 256;
-        const unsigned grid_x = (unsigned)(gx < 1 ? 1 : (gx > 8192 ? 8192 : gx));
-        const size_t want_y = grid_x >= 8192 ? 1 : (8192 + grid_x - 1) / grid_x;
-        const unsigned grid_y = (unsigned)(total_rows < want_y ? total_rows : (want_y > 65535 ? 65535 : want_y));
-        hipLaunchKernelGGL(rect_copy16_kernel, dim3(grid_x, grid_y ? grid_y : 1), dim3(256), 0, s->stream, static_cast<char *>(dst),
+        const size_t gx = (w16 + 63) / 64;
+        const unsigned grid_x = (unsigned)(gx < 1 ? 1 : (gx > (1u << 22) ? (1u << 22) : gx));
+        const unsigned grid_y = (unsigned)(total_rows > 65535 ? 65535 : total_rows);
+        hipLaunchKernelGGL(rect_copy16_kernel, dim3(grid_x, grid_y ? grid_y : 1), dim3(64), 0, s->stream, static_cast<char *>(dst),
                            d_rp, dsp, static_cast<const char *>(src), s_rp, ssp, w16, nrows, total_rows);
         return launch_status();
     }
