@@ -61,8 +61,13 @@ __global__ __launch_bounds__(256) void transpose_tiled_kernel(const E *__restric
         if (r0 + r >= a.rows) continue;
         const E *p = src + so + (r0 + r) * a.src_row_pitch + c0 + c;
         if (VEC && c0 + c + VE <= a.cols) {
+            typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+            // streamed (read once, written once) for elements of up to four bytes: f32 8192^2 104 -> 95 us, u8
+            // 16384^2 110 -> 103; the 8- and 16-byte types measured 4 % slower with it
+            const u32x4 raw = sizeof(E) <= 4 ? __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(p))
+                                             : *reinterpret_cast<const u32x4 *>(p);
             E tmp[VE];
-            __builtin_memcpy(tmp, __builtin_assume_aligned(p, 16), 16);
+            __builtin_memcpy(tmp, &raw, 16);
 #pragma unroll
             for (int e = 0; e < VE; ++e) tile[r][c + e] = tmp[e];
         } else {
@@ -81,7 +86,11 @@ __global__ __launch_bounds__(256) void transpose_tiled_kernel(const E *__restric
             E tmp[VE];
 #pragma unroll
             for (int e = 0; e < VE; ++e) tmp[e] = tile[r + e][c];
-            __builtin_memcpy(__builtin_assume_aligned(p, 16), tmp, 16);
+            typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+            u32x4 raw;
+            __builtin_memcpy(&raw, tmp, 16);
+            if (sizeof(E) <= 4) __builtin_nontemporal_store(raw, reinterpret_cast<u32x4 *>(p));
+            else *reinterpret_cast<u32x4 *>(p) = raw;
         } else {
             for (int e = 0; e < VE; ++e)
                 if (r0 + r + e < a.rows) p[e] = tile[r + e][c];
