@@ -216,10 +216,16 @@ void gemm_f32_dma_kernel(DArgs g) {
     // k-contiguous: row * BK + 4 * (chunk ^ swz); chunk = 2 s + lhi, swz from l32 alone (row offsets are multiples of 32)
     // m-contiguous: k * ROWS + (m ^ 32 lhi); k = 8 s + 4 lhi + t; m = wave offset + 32 i + l32
     const int sw4 = 4 * (lhi ^ (int)swizzle((uint32_t)l32));
+    // A_PERM (m-contiguous A, four blocks per wavefront): lane l32 of block i stands for tile row 4 l32 + i
+    // instead of 32 i + l32, so that one 16-byte read (four consecutive m at one k) serves all four blocks;
+    // the epilogue maps the rows back.  (16 four-byte reads per step otherwise: T,N and T,T were the slow layouts.)
+    constexpr bool A_PERM = !A_K && FM == 4;
     int a_frag[FM], b_frag[FN]; // k-contiguous: one base (block i is an immediate away); m-contiguous: block i's column
 #pragma unroll
     for (int i = 0; i < FM; ++i)
-        a_frag[i] = A_K ? (wm * WM + l32) * BK + sw4 : 4 * lhi * BM + (((wm * WM + 32 * i) ^ (32 * lhi)) + l32);
+        a_frag[i] = A_K      ? (wm * WM + l32) * BK + sw4
+                    : A_PERM ? 4 * lhi * BM + ((wm * WM + 4 * l32) ^ (32 * lhi))
+                             : 4 * lhi * BM + (((wm * WM + 32 * i) ^ (32 * lhi)) + l32);
 #pragma unroll
     for (int j = 0; j < FN; ++j)
         b_frag[j] = B_K ? (wn * WN + l32) * BK + sw4 : 4 * lhi * BN + (((wn * WN + 32 * j) ^ (32 * lhi)) + l32);
@@ -233,14 +239,23 @@ void gemm_f32_dma_kernel(DArgs g) {
     auto read_frags = [&](uint32_t stage_bytes, int s, f32x4 *af, f32x4 *bf) {
         const float *as = lds + stage_bytes / 4;
         const float *bs = as + A_FLOATS;
+        if constexpr (A_PERM) {
 #pragma unroll
-        for (int i = 0; i < FM; ++i) {
-            if constexpr (A_K) {
-                // chunk 2 s + lhi: step s flips the bits of 2 s in the chunk number
-                af[i] = *reinterpret_cast<const f32x4 *>(as + ((a_frag[i] ^ (8 * s)) + i * 32 * BK));
-            } else {
+            for (int t = 0; t < 4; ++t) {
+                const f32x4 v = *reinterpret_cast<const f32x4 *>(as + a_frag[0] + (8 * s + t) * BM);
 #pragma unroll
-                for (int t = 0; t < 4; ++t) af[i][t] = as[a_frag[i] + (8 * s + t) * BM];
+                for (int i = 0; i < FM; ++i) af[i][t] = v[i];
+            }
+        } else {
+#pragma unroll
+            for (int i = 0; i < FM; ++i) {
+                if constexpr (A_K) {
+                    // chunk 2 s + lhi: step s flips the bits of 2 s in the chunk number
+                    af[i] = *reinterpret_cast<const f32x4 *>(as + ((a_frag[i] ^ (8 * s)) + i * 32 * BK));
+                } else {
+#pragma unroll
+                    for (int t = 0; t < 4; ++t) af[i][t] = as[a_frag[i] + (8 * s + t) * BM];
+                }
             }
         }
 #pragma unroll
@@ -391,6 +406,8 @@ void gemm_f32_dma_kernel(DArgs g) {
 #pragma unroll
                 for (int r = 0; r < 16; ++r) acc[i][j][r] += part[((i * FN + j) * 16 + r) * 64];
     }
+    // row of the wavefront's tile that output row `rho` of block i holds
+    auto tile_row = [](int i, int rho) -> uint32_t { return A_PERM ? (uint32_t)(4 * rho + i) : (uint32_t)(32 * i + rho); };
     // Tiles that reach beyond C clamp the addresses of C_old and the bias and skip the stores there.
     const float alpha = g.alpha, beta = g.beta;
     auto epilogue = [&](auto checked_tag) {
@@ -409,14 +426,14 @@ void gemm_f32_dma_kernel(DArgs g) {
                 if (g.epi == EPI_ALPHA_BETA) {
 #pragma unroll
                     for (int r = 0; r < 16; ++r) {
-                        const uint32_t row = m0 + wm * WM + i * 32 + 8 * (r / 4) + 4 * lhi + (r % 4);
+                        const uint32_t row = m0 + wm * WM + tile_row(i, 8 * (r / 4) + 4 * lhi + (r % 4));
                         if constexpr (PRELOAD_C) old[r] = c_old[r];
                         else old[r] = g.C[(size_t)(CHECKED ? min(row, g.M - 1) : row) * g.ldc + colc];
                     }
                 }
 #pragma unroll
                 for (int r = 0; r < 16; ++r) {
-                    const uint32_t row = m0 + wm * WM + i * 32 + 8 * (r / 4) + 4 * lhi + (r % 4);
+                    const uint32_t row = m0 + wm * WM + tile_row(i, 8 * (r / 4) + 4 * lhi + (r % 4));
                     float v = acc[i][j][r];
                     if (g.epi == EPI_ALPHA) v = alpha * v;
                     else if (g.epi == EPI_ALPHA_BETA) v = alpha * v + beta * old[r];
