@@ -452,15 +452,15 @@ void gemm_f32_dma_kernel(DArgs g) {
 // ------------------------------------------------------------------------------------ f64 ---
 // The same pipeline with v_mfma_f64_16x16x4_f64 (lane l supplies A[l % 16][l / 16] and B[l / 16][l % 16];
 // result register r of lane l is C[4 r + l / 16][l % 16] of its 16 x 16 block).  A 16-byte chunk is two
-// doubles.  Macro tiles 128 x 128 with k-slabs of 8 (three stages of 16 KB; two work-groups per unit: 128
-// accumulator and 64 fragment registers do not fit the 168 of three) and 64 x 64 with k-slabs of 16 (the
-// same 16 KB, three work-groups per unit).
-//   k-contiguous operand: [row][BK], BK / 2 chunks per row, chunk c of row r at position
-//     c ^ ((r >> 2) & 3) (BK = 8) or c ^ ((r >> 1) & 7) (BK = 16); a fragment is one 16-byte read
-//     (row = lane % 16, k = 8 s + 2 (lane / 16) + 0..1), sixteen consecutive rows at one logical chunk cover
-//     all banks once.  (For BK = 8 the bank-conflict counter still shows four cycles per such read, also
-//     with bits 2 and 3 of r exchanged in the swizzle; for BK = 16 and in the f32 kernels it shows none.
-//     That is 1.4 % of the kernel's clocks.)
+// doubles.  k-slabs of 16 (two fragment steps).  Macro tiles 64 x 64 (three stages of 16 KB, three
+// work-groups per unit) and 128 x 128 (two work-groups per unit: 128 accumulator and 64 fragment registers
+// do not fit the 168 of three; two stages of 32 KB, the next slab requested at the top of an iteration into
+// the stage the hand-over before it set free -- one iteration of 64 matrix instructions of 64 clocks, beside
+// the other work-group's, is time enough for it to arrive.  With slabs of 8 in three stages the hand-over came
+// twice as often: 4096^3 70.7 against 72.3 TFLOP/s, 8192^3 72.0 against 74.2).
+//   k-contiguous operand: [row][16], 8 chunks per row, chunk c of row r at position c ^ ((r >> 1) & 7); a
+//     fragment is one 16-byte read (row = lane % 16, k = 8 s + 2 (lane / 16) + 0..1), sixteen consecutive rows
+//     at one logical chunk cover all banks once.
 //   m/n-contiguous operand: [k][ROWS], element (k, m) at m ^ (16 * ((k >> 1) & 1)); fragments are 8-byte
 //     reads, the four quarter-wavefronts read rows k, k + 2, k + 4, k + 6 and the swizzle puts
 //     neighbouring quarters on disjoint banks.
@@ -478,21 +478,23 @@ struct DArgsD {
     double alpha, beta;
     const double *bias;
     int act;
+    uint32_t patch_m, patch_n; // as in DArgs
 };
 
 
-template <int BM, int BN, int BK, int OCC, bool A_K, bool B_K, bool EXT>
+template <int BM, int BN, int BK, int NS, int OCC, bool A_K, bool B_K, bool EXT>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(OCC)))
 void gemm_f64_dma_kernel(DArgsD g) {
+    static_assert(NS == 2 || NS == 3, "stages");
     constexpr int WM = BM / 2, WN = BN / 2, FM = WM / 16, FN = WN / 16;
     constexpr int S = BK / 8;     // fragment steps per slab (8 values of k each, two matrix instructions per block)
     constexpr int CPR = BK / 2;   // 16-byte chunks per row of a k-contiguous slab
     constexpr int A_DOUBLES = BM * BK, B_DOUBLES = BN * BK, STAGE = A_DOUBLES + B_DOUBLES;
     constexpr int A_LOADS = BM * BK / 512, B_LOADS = BN * BK / 512; // 1 KB = 128 doubles per wavefront and load
-    static_assert((BK == 8 || BK == 16) && BM % 32 == 0 && BN % 32 == 0 && A_LOADS >= 1 && B_LOADS >= 1, "tile shape");
+    static_assert(BK == 16 && BM % 32 == 0 && BN % 32 == 0 && A_LOADS >= 1 && B_LOADS >= 1, "tile shape");
 
     extern __shared__ __align__(16) float lds_f[];
-    double *lds = reinterpret_cast<double *>(lds_f); // [3][STAGE]: A then B
+    double *lds = reinterpret_cast<double *>(lds_f); // [NS][STAGE]: A then B
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -501,7 +503,15 @@ void gemm_f64_dma_kernel(DArgsD g) {
     const int l16 = lane & 15, lq = lane >> 4;
 
     uint32_t tile_m, tile_n;
-    {
+    if (g.patch_m) { // XCD-local patches, as in the f32 kernel
+        const uint32_t pid = blockIdx.x;
+        const uint32_t x = pid & 7u, j = pid >> 3;
+        const uint32_t per_patch = g.patch_m * g.patch_n;
+        const uint32_t patch = (j / per_patch) * 8u + x, q = j % per_patch;
+        const uint32_t patches_n = g.tiles_n / g.patch_n;
+        tile_m = (patch / patches_n) * g.patch_m + q % g.patch_m;
+        tile_n = (patch % patches_n) * g.patch_n + q / g.patch_m;
+    } else {
         const uint32_t pid = blockIdx.x;
         const uint32_t group_size = GROUP_M * g.tiles_n;
         const uint32_t group = pid / group_size;
@@ -530,7 +540,7 @@ void gemm_f64_dma_kernel(DArgsD g) {
         if constexpr (KC) {
             constexpr int RPL = 64 / CPR; // rows per load
             const uint32_t row = grp * RPL + lane / CPR;
-            const uint32_t swz = CPR == 4 ? (row >> 2) & 3 : (row >> 1) & 7;
+            const uint32_t swz = (row >> 1) & 7;
             const uint32_t chunk = (lane % CPR) ^ swz;
             return (row * ld + 2 * chunk) * 8u;
         } else {
@@ -561,7 +571,7 @@ void gemm_f64_dma_kernel(DArgsD g) {
 
     // ---- LDS side: per-lane fragment addresses in doubles from the start of a stage's A or B part ----
     // k-contiguous: row * BK + 2 * ((4 s + lq) ^ swz(row)); row = wave offset + 16 i + l16, so swz depends on l16 only
-    const int swz_l = CPR == 4 ? (l16 >> 2) & 3 : (l16 >> 1) & 7;
+    const int swz_l = (l16 >> 1) & 7;
     int a_frag[FM], b_frag[FN];
 #pragma unroll
     for (int i = 0; i < FM; ++i)
@@ -576,8 +586,8 @@ void gemm_f64_dma_kernel(DArgsD g) {
 #pragma unroll
         for (int i = 0; i < FM; ++i) {
             if constexpr (A_K) {
-                // chunk 4 s + lq: the second step's chunk has bit 2 flipped (BK = 16 only)
-                af[i] = *reinterpret_cast<const f64x2 *>(as + (a_frag[i] ^ (s ? 8 : 0)));
+                // chunk 4 s + lq: the second step's chunk has bit 2 flipped
+                af[i] = *reinterpret_cast<const f64x2 *>(as + (a_frag[i] ^ (8 * s)));
             } else {
 #pragma unroll
                 for (int t = 0; t < 2; ++t) af[i][t] = as[a_frag[i] + (8 * s + t) * BM];
@@ -586,7 +596,7 @@ void gemm_f64_dma_kernel(DArgsD g) {
 #pragma unroll
         for (int j = 0; j < FN; ++j) {
             if constexpr (B_K) {
-                bf[j] = *reinterpret_cast<const f64x2 *>(bs + (b_frag[j] ^ (s ? 8 : 0)));
+                bf[j] = *reinterpret_cast<const f64x2 *>(bs + (b_frag[j] ^ (8 * s)));
             } else {
 #pragma unroll
                 for (int t = 0; t < 2; ++t) bf[j][t] = bs[b_frag[j] + (8 * s + t) * BN];
@@ -619,7 +629,7 @@ void gemm_f64_dma_kernel(DArgsD g) {
     uint32_t st_cur = 0, st_next = STAGE_BYTES, st_after = 2 * STAGE_BYTES;
 
     issue(st_cur);
-    if (ktiles > 1) {
+    if (NS == 3 && ktiles > 1) {
         issue(st_next);
         wait_vm<A_LOADS + B_LOADS>();
     } else {
@@ -628,22 +638,22 @@ void gemm_f64_dma_kernel(DArgsD g) {
     __builtin_amdgcn_s_barrier();
     read_frags(st_cur, 0, af[0], bf[0]);
 
-    // One iteration on the slab in st_cur; P: which fragment set holds its first step (a compile-time
-    // constant: with one step per slab the sets swap every iteration).  The hand-over to slab kt+1 (wait
-    // for this wavefront's own loads of it, barrier, first fragments) sits in front of the last step's
-    // matrix instructions, as in the f32 kernel.
-    auto iteration = [&](auto parity_tag, auto more2_tag, auto more1_tag) __attribute__((always_inline)) {
-        constexpr int P = decltype(parity_tag)::value;
+    // One iteration on the slab in st_cur (its first step's fragments are in set 0).  The hand-over to slab
+    // kt+1 (wait for this wavefront's own loads of it, barrier, first fragments) sits in front of the last
+    // step's matrix instructions, as in the f32 kernel.
+    auto iteration = [&](auto more2_tag, auto more1_tag) __attribute__((always_inline)) {
         constexpr bool MORE2 = decltype(more2_tag)::value, MORE1 = decltype(more1_tag)::value;
-        if constexpr (MORE2) issue(st_after);
+        // two stages: the stage of the slab before this one is free (every wavefront's last reads of it had
+        // landed before the barrier of its hand-over), and slab kt+1 has this iteration's length to arrive
+        if constexpr (NS == 3 ? MORE2 : MORE1) issue(NS == 3 ? st_after : st_next);
 #pragma unroll
         for (int s = 0; s < S; ++s) {
-            const int set = (P + s) & 1;
+            const int set = s & 1;
             if (s + 1 < S) {
                 read_frags(st_cur, s + 1, af[set ^ 1], bf[set ^ 1]);
             } else if constexpr (MORE1) {
                 __builtin_amdgcn_sched_barrier(0);
-                if constexpr (MORE2) wait_vm<A_LOADS + B_LOADS>();
+                if constexpr (NS == 3 && MORE2) wait_vm<A_LOADS + B_LOADS>();
                 else wait_vm<0>();
                 wait_lgkm0();
                 __builtin_amdgcn_s_barrier();
@@ -654,26 +664,19 @@ void gemm_f64_dma_kernel(DArgsD g) {
         }
         const uint32_t t = st_cur;
         st_cur = st_next;
-        st_next = st_after;
-        st_after = t;
+        if constexpr (NS == 3) {
+            st_next = st_after;
+            st_after = t;
+        } else {
+            st_next = t;
+        }
     };
     using T_ = std::true_type;
     using F_ = std::false_type;
-    using P0 = integral_constant<int, 0>;
-    using P1 = integral_constant<int, 1>;
     uint32_t kt = 0;
-    if constexpr (S % 2 == 0) { // the first step of every slab uses set 0
-        for (; kt + 2 < ktiles; ++kt) iteration(P0{}, T_{}, T_{});
-        if (kt + 1 < ktiles) iteration(P0{}, F_{}, T_{});
-        iteration(P0{}, F_{}, F_{});
-    } else { // sets alternate with the slabs: two iterations per trip; K % 16 == 0 makes the slab count even
-        for (; kt + 3 < ktiles; kt += 2) {
-            iteration(P0{}, T_{}, T_{});
-            iteration(P1{}, T_{}, T_{});
-        }
-        iteration(P0{}, F_{}, T_{}); // two left
-        iteration(P1{}, F_{}, F_{});
-    }
+    for (; kt + 2 < ktiles; ++kt) iteration(T_{}, T_{});
+    if (kt + 1 < ktiles) iteration(F_{}, T_{});
+    iteration(F_{}, F_{});
 
     const double alpha = g.alpha, beta = g.beta;
 #pragma unroll
@@ -708,9 +711,9 @@ void gemm_f64_dma_kernel(DArgsD g) {
         }
 }
 
-template <int BM, int BN, int BK, int OCC, bool A_K, bool B_K, bool EXT> int launch_one_d(hipStream_t st, const DArgsD &g) {
-    constexpr size_t lds_bytes = 3 * (BM * BK + BN * BK) * sizeof(double);
-    auto kern = gemm_f64_dma_kernel<BM, BN, BK, OCC, A_K, B_K, EXT>;
+template <int BM, int BN, int BK, int NS, int OCC, bool A_K, bool B_K, bool EXT> int launch_one_d(hipStream_t st, const DArgsD &g) {
+    constexpr size_t lds_bytes = NS * (BM * BK + BN * BK) * sizeof(double);
+    auto kern = gemm_f64_dma_kernel<BM, BN, BK, NS, OCC, A_K, B_K, EXT>;
     static const int attr_rc = [&] {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
                                            (int)lds_bytes);
@@ -725,7 +728,7 @@ template <int BM, int BN, int BK, int OCC, bool A_K, bool B_K, bool EXT> int lau
     return launch_status();
 }
 
-template <int BM, int BN, int BK, int OCC> int launch_tile_d(hipStream_t st, const GemmProblem &p) {
+template <int BM, int BN, int BK, int NS, int OCC> int launch_tile_d(hipStream_t st, const GemmProblem &p) {
     DArgsD g{};
     g.A = static_cast<const double *>(p.A);
     g.B = static_cast<const double *>(p.B);
@@ -740,13 +743,26 @@ template <int BM, int BN, int BK, int OCC> int launch_tile_d(hipStream_t st, con
     std::memcpy(&g.beta, p.beta, sizeof(double));
     g.bias = static_cast<const double *>(p.ext_bias);
     g.act = p.ext_act;
+    static const bool row_walk = [] {
+        const char *e = std::getenv("WK_GEMM_WALK");
+        return e && std::strcmp(e, "rows") == 0;
+    }();
+    if (!row_walk) {
+        static const unsigned shapes[][2] = {{4, 8}, {4, 4}, {2, 8}, {2, 4}};
+        for (const auto &sh : shapes)
+            if (g.tiles_m % sh[0] == 0 && g.tiles_n % sh[1] == 0 && ((g.tiles_m / sh[0]) * (g.tiles_n / sh[1])) % 8 == 0) {
+                g.patch_m = sh[0];
+                g.patch_n = sh[1];
+                break;
+            }
+    }
     const int sel = (p.op_a ? 0 : 2) | (p.op_b ? 1 : 0);
-    if (p.ext) return sel == 3 ? launch_one_d<BM, BN, BK, OCC, true, true, true>(st, g) : (int)WK_E_INVALID_VALUE;
+    if (p.ext) return sel == 3 ? launch_one_d<BM, BN, BK, NS, OCC, true, true, true>(st, g) : (int)WK_E_INVALID_VALUE;
     switch (sel) {
-    case 0: return launch_one_d<BM, BN, BK, OCC, false, false, false>(st, g);
-    case 1: return launch_one_d<BM, BN, BK, OCC, false, true, false>(st, g);
-    case 2: return launch_one_d<BM, BN, BK, OCC, true, false, false>(st, g);
-    default: return launch_one_d<BM, BN, BK, OCC, true, true, false>(st, g);
+    case 0: return launch_one_d<BM, BN, BK, NS, OCC, false, false, false>(st, g);
+    case 1: return launch_one_d<BM, BN, BK, NS, OCC, false, true, false>(st, g);
+    case 2: return launch_one_d<BM, BN, BK, NS, OCC, true, false, false>(st, g);
+    default: return launch_one_d<BM, BN, BK, NS, OCC, true, true, false>(st, g);
     }
 }
 
@@ -849,8 +865,10 @@ bool wk::gemm_f64_dma_applies(const GemmProblem &p, int bm, int bn) {
 
 int wk::gemm_f64_dma_launch(hipStream_t st, const GemmProblem &p, int bm, int bn) {
     if (!gemm_f64_dma_applies(p, bm, bn)) return WK_E_INVALID_VALUE;
-    if (bm == 128) return launch_tile_d<128, 128, 8, 2>(st, p); // (128 accumulator + 64 fragment registers: two per SIMD)
-    return launch_tile_d<64, 64, 16, 3>(st, p);
+    if (bm == 128) return launch_tile_d<128, 128, 16, 2, 2>(st, p);
+    // (64 x 64 with k-slabs of 32 in two stages, two work-groups per unit, measured the same within the run-to-run
+    // spread: 8192 x 256 x 8192 67.4-68.6 against 68.0-68.2 TFLOP/s, 2048^3 68-69 against 66-68, 3072^3 70-71 both)
+    return launch_tile_d<64, 64, 16, 3, 3>(st, p);
 }
 
 int wk::gemm_f32_dma_launch(hipStream_t st, const GemmProblem &p, int bm, int bn, uint64_t first_tiles, int k_groups) {

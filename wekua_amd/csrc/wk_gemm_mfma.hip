@@ -1474,7 +1474,7 @@ const VariantDesc k_variants[] = {
     {"mfma_f64_64x64", WK_F64, 64, 64, 32, 0.840, 0.05, &launch_f64<64, 64, 32, 2, 2, 2>, "mfma_f64_64x64s2", nullptr,
      "mfma_f64_32x32s4", "mfma_f64_64x64z"},
     // slabs straight into LDS, three deep (wk_gemm_dma.hip), interior shapes: 4096^3 70.2 against 68.5 TFLOP/s
-    {"mfma_f64_128x128d", WK_F64, 128, 128, 16, 0.91, 0.10, &launch_f64_dma<128, 128, 16, 2>},
+    {"mfma_f64_128x128d", WK_F64, 128, 128, 16, 0.94, 0.10, &launch_f64_dma<128, 128, 16, 2>},
     // 8192 x 256 x 8192 69.6 (staged 62.2), 2048^3 68 (61.7), 4096^3 69-70.5
     {"mfma_f64_64x64d", WK_F64, 64, 64, 32, 0.89, 0.05, &launch_f64_dma<64, 64, 32, 2>, nullptr, nullptr, "mfma_f64_32x32s4", "mfma_f64_64x64z"},
     {"mfma_f64_64x64z", WK_F64, 64, 64, 32, 0.0, 0.05, &launch_f64_split64}, // k split over work-groups
