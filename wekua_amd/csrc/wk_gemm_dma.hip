@@ -72,7 +72,7 @@ void gemm_f32_dma_kernel(DArgs g) {
     constexpr int WAVES = 4 * KS;
     constexpr int SG = S / KS; // steps of a slab per group of wavefronts
     constexpr int A_LOADS = BM * BK / (256 * WAVES), B_LOADS = BN * BK / (256 * WAVES); // 1 KB per wavefront and load
-    static_assert(BM % 64 == 0 && BN % 64 == 0 && (BK == 16 || BK == 32) && NS >= 3, "tile shape");
+    static_assert(BM % 64 == 0 && BN % 64 == 0 && (BK == 16 || BK == 32) && NS >= 2, "tile shape");
     static_assert((KS == 1 || KS == 2) && SG >= 2 && SG % 2 == 0 && A_LOADS >= 1 && B_LOADS >= 1, "k-groups");
 
     extern __shared__ __align__(16) float lds[]; // [NS][STAGE]: A then B
@@ -334,10 +334,13 @@ void gemm_f32_dma_kernel(DArgs g) {
     // which it waited for its last reads of that stage).  AHEAD >= 0: slab kt + 1 exists and AHEAD slabs
     // after it have been requested; before the last step's matrix instructions this wavefront waits for
     // its own loads of slab kt + 1 (the AHEAD later ones may stay in flight) and for its LDS reads, joins
-    // the barrier and reads the first fragments of slab kt + 1.  AHEAD < 0: the last slab.
-    auto iteration = [&](auto issue_tag, auto ahead_tag) __attribute__((always_inline)) {
+    // the barrier and reads the first fragments of slab kt + 1.  AHEAD < 0: the last slab.  LAST_NEXT: slab
+    // kt + 1 is the last one (its k values beyond K are overwritten with zeros once it has landed).
+    auto iteration = [&](auto issue_tag, auto ahead_tag, auto last_next_tag) __attribute__((always_inline)) {
         constexpr bool ISSUE = decltype(issue_tag)::value;
         constexpr int AHEAD = decltype(ahead_tag)::value;
+        constexpr bool LAST_NEXT = decltype(last_next_tag)::value;
+        static_assert(!LAST_NEXT || AHEAD == 0, "nothing is requested beyond the last slab");
         if constexpr (ISSUE) issue(st[NS - 1]);
 #pragma unroll
         for (int s = 0; s + 1 < SG; ++s) {
@@ -347,8 +350,8 @@ void gemm_f32_dma_kernel(DArgs g) {
         if constexpr (AHEAD >= 0) {
             __builtin_amdgcn_sched_barrier(0);
             wait_vm<AHEAD * LOADS>();
-            if constexpr (AHEAD == 0) {
-                if (krem) tail_zeros(st[1]); // slab kt + 1 is the last one
+            if constexpr (LAST_NEXT) {
+                if (krem) tail_zeros(st[1]);
             }
             wait_lgkm0();
             __builtin_amdgcn_s_barrier();
@@ -365,20 +368,20 @@ void gemm_f32_dma_kernel(DArgs g) {
     using T_ = std::true_type;
     using F_ = std::false_type;
     uint32_t kt = 0;
-    for (; kt + NS < ktiles; ++kt) iteration(T_{}, integral_constant<int, NS - 2>{}); // steady state
-    if (kt + NS - 1 < ktiles) { // the iteration that requests the last slab
+    for (; kt + NS < ktiles; ++kt) iteration(T_{}, integral_constant<int, NS - 2>{}, F_{}); // steady state
+    if (kt + NS - 1 < ktiles) { // the iteration that requests the last slab (with two stages: and hands over to it)
         if (krem) tail_offsets();
-        iteration(T_{}, integral_constant<int, NS - 2>{});
+        iteration(T_{}, integral_constant<int, NS - 2>{}, integral_constant<bool, NS == 2>{});
         ++kt;
     }
     // the pipeline drains: ktiles - 2 - kt slabs are in flight beyond the next one
     drain<NS - 3>([&](auto ahead_tag) {
         if (kt + 2 + decltype(ahead_tag)::value == ktiles) {
-            iteration(F_{}, ahead_tag);
+            iteration(F_{}, ahead_tag, integral_constant<bool, decltype(ahead_tag)::value == 0>{});
             ++kt;
         }
     });
-    iteration(F_{}, integral_constant<int, -1>{}); // the last
+    iteration(F_{}, integral_constant<int, -1>{}, F_{}); // the last
 
     // ---- epilogue: acc register r of lane l is C[8*(r/4) + 4*(l/32) + r%4][l%32] of its 32x32 block;
     // option semantics of src/blas/gemm.zig:500-501,591-602 (C_old is read and multiplied whenever beta
@@ -881,6 +884,10 @@ int wk::gemm_f32_dma_launch(hipStream_t st, const GemmProblem &p, int bm, int bn
         return launch_tile<64, 64, 32, 3, 4, 2>(st, p, 0);
     }
     if (bm == 256) return launch_tile<256, 128, 16, 3, 2>(st, p, first_tiles);
+    // 128 x 128 with both operands m/n-contiguous (T,N): k-slabs of 32 in two stages, two work-groups per unit
+    // (half as many hand-overs; 2048 x 4096 x 4096 139 -> 143 TFLOP/s, 4096 x 2048 x 2048 135 -> 140, 2048 x 2048 x
+    // 8192 129 -> 138; the other layouts measured the same or up to 2 % less that way and keep three stages of 16)
+    if (bm == 128 && p.op_a && !p.op_b) return launch_tile<128, 128, 32, 2, 2>(st, p, first_tiles);
     if (bm == 128) return launch_tile<128, 128, 16, 3, 3>(st, p, first_tiles);
     // (k-slabs of 32, three work-groups per unit; with slabs of 16 and four: 1024^3 101 against 103.5 TFLOP/s,
     // 3000^3 118 against 125, 2049 x 2047 x 2050 108 against 106.5)
