@@ -313,7 +313,8 @@ def test_one_round_launches_take_the_k_split_tiles(dev):
     assert name("f32", 512, 512, 512) == b"mfma_f32_32x32s4"       # 64 tiles of 64x64 would leave most CUs idle
     assert name("f32", 768, 768, 768) == b"mfma_f32_32x32s4"
     assert name("f64", 1024, 1024, 1024) == b"mfma_f64_64x64d"
-    assert name("f64", 1000, 1000, 1000) == b"mfma_f64_64x64s2"
+    assert name("f64", 1000, 1000, 1000) == b"mfma_f64_64x64d"
+    assert name("f64", 1001, 1001, 1001) == b"mfma_f64_64x64s2"   # rows of 8008 bytes: the register-staged tile
     assert name("f64", 2048, 2048, 2048) == b"mfma_f64_64x64d"
     assert name("f64", 4096, 4096, 4096) == b"mfma_f64_128x128d"
     assert name("f64", 512, 512, 512) == b"mfma_f64_32x32s4"
@@ -384,8 +385,14 @@ def test_slabs_straight_into_lds(dev, variant, bm, bn, op_a, op_b):
     """The kernels that bring their k-slabs from global memory straight into LDS (three stages, swizzled
     layouts): every count of slabs from one to a handful (the pipeline's prologue and its last two
     iterations are special), several tiles, every epilogue, leading dimensions with gaps; against the
-    oracle.  Shapes they do not take (ragged, unaligned) fall back to the register-staged tile."""
+    oracle.  Operands whose rows do not start on 16-byte boundaries fall back to the register-staged tile."""
     dtype = variant[5:8]
+    per = 4 if dtype == "f32" else 2                 # elements in 16 bytes
+
+    def ragged(M, N, K, alpha, beta, seed):          # rows padded to 16-byte boundaries: these kernels run
+        cols_a, cols_b = (M if op_a else K), (K if op_b else N)
+        check(dev, dtype, M, N, K, op_a, op_b, alpha, beta, seed=seed,
+              lda=-(-cols_a // per) * per, ldb=-(-cols_b // per) * per)
     assert dev.lib.wk_gemm_force_variant(variant.encode()) == 0
     try:
         for K in (16, 32, 48, 64, 80, 96, 112, 128, 256, 1040):
@@ -395,26 +402,27 @@ def test_slabs_straight_into_lds(dev, variant, bm, bn, op_a, op_b):
         check(dev, dtype, 9 * bm, 9 * bn, 176, op_a, op_b, None, -0.25, seed=233)          # 81 tiles, more than one group of tile rows
         check(dev, dtype, 2 * bm, 2 * bn, 96, op_a, op_b, 1.5, 0.5, seed=234,
               lda=(2 * bm if op_a else 96) + 8, ldb=(96 if op_b else 2 * bn) + 12, ldc=2 * bn + 5)  # gaps between rows, 16-byte aligned
-        check(dev, dtype, 300, 200, 100, op_a, op_b, 1.5, 0.5, seed=235)                  # ragged (f64: the staged tile runs)
-        if dtype == "f32":
-            # ragged in every dimension: border tiles fetch clamped rows and skip stores, the last slab is
-            # zero-filled in LDS beyond K; K below, at and around the slab size, one to three slabs and many
-            for K in (1, 3, 4, 15, 17, 31, 33, 47, 50, 100, 1001):
-                check(dev, dtype, bm + 1, 2 * bn - 3, K, op_a, op_b, 1.5, 0.5, seed=240 + K)
-            check(dev, dtype, 2 * bm + 7, bn + 5, 61, op_a, op_b, None, None, seed=251)
-            check(dev, dtype, 3, 5, 37, op_a, op_b, 2.0, None, seed=252)                  # smaller than one 16-byte chunk
-            check(dev, dtype, bm - 1, bn - 1, 16, op_a, op_b, None, -0.25, seed=253)
-            # rows that do not start on 16-byte boundaries: not this kernel's, the staged tile runs
-            check(dev, dtype, 2 * bm, bn, 40, op_a, op_b, 1.5, 0.5, seed=254,
-                  lda=(2 * bm if op_a else 40) + 3, ldb=(40 if op_b else bn) + 1, ldc=bn + 2)
+        check(dev, dtype, 300, 200, 100, op_a, op_b, 1.5, 0.5, seed=235)                  # ragged, dense rows
+        # ragged in every dimension: border tiles fetch clamped rows and skip stores, the last slab is
+        # zero-filled in LDS beyond K; K below, at and around the slab size, one to three slabs and many
+        for K in (1, 3, 4, 15, 17, 31, 33, 47, 50, 100, 1001):
+            ragged(bm + 1, 2 * bn - 3, K, 1.5, 0.5, 240 + K)
+            check(dev, dtype, bm + 1, 2 * bn - 3, K, op_a, op_b, 1.5, 0.5, seed=240 + K)  # dense rows: whichever kernel takes them
+        ragged(2 * bm + 7, bn + 5, 61, None, None, 251)
+        ragged(3, 5, 37, 2.0, None, 252)                                                  # smaller than one 16-byte chunk
+        ragged(1, 1, 1, 1.5, 0.5, 255)
+        ragged(bm - 1, bn - 1, 16, None, -0.25, 253)
+        # rows that do not start on 16-byte boundaries: not this kernel's, the staged tile runs
+        check(dev, dtype, 2 * bm, bn, 40, op_a, op_b, 1.5, 0.5, seed=254,
+              lda=(2 * bm if op_a else 40) + 3, ldb=(40 if op_b else bn) + 1, ldc=bn + 2)
     finally:
         dev.lib.wk_gemm_force_variant(b"auto")
 
 
 @pytest.mark.parametrize("variant,bm,bn", [("mfma_f32_256x128d", 256, 128), ("mfma_f32_128x128d", 128, 128), ("mfma_f32_64x64d", 64, 64),
-                                           ("mfma_f32_64x64d2", 64, 64)])
+                                           ("mfma_f32_64x64d2", 64, 64), ("mfma_f64_128x128d", 128, 128), ("mfma_f64_64x64d", 64, 64)])
 def test_tile_walk_in_patches_covers_every_tile_once(dev, variant, bm, bn):
-    """The f32 direct-to-LDS kernels number their tiles in XCD-local patches (4 x 8, 4 x 4, 2 x 8 or 2 x 4
+    """The direct-to-LDS kernels number their tiles in XCD-local patches (4 x 8, 4 x 4, 2 x 8 or 2 x 4
     tiles, eight patches at a time) when the tile grid divides into them and in groups of tile rows
     otherwise: one tile grid per patch shape and one that takes none, whole result against the oracle
     (a tile visited twice or not at all leaves entries of C wrong)."""
@@ -422,17 +430,20 @@ def test_tile_walk_in_patches_covers_every_tile_once(dev, variant, bm, bn):
     try:
         for tiles_m, tiles_n in ((8, 32), (8, 16), (2, 64), (2, 32), (16, 16), (6, 10)):
             for op_a, op_b in ((0, 0), (1, 1)):
-                check(dev, "f32", tiles_m * bm, tiles_n * bn, 48, op_a, op_b, None, None, seed=300 + tiles_m + tiles_n)
+                check(dev, variant[5:8], tiles_m * bm, tiles_n * bn, 48, op_a, op_b, None, None, seed=300 + tiles_m + tiles_n)
     finally:
         dev.lib.wk_gemm_force_variant(b"auto")
 
 
-@pytest.mark.parametrize("variant", ["mfma_f32_256x128d", "mfma_f32_128x128d", "mfma_f32_64x64d", "mfma_f32_128x128d2", "mfma_f32_64x64d2"])
+@pytest.mark.parametrize("variant", ["mfma_f32_256x128d", "mfma_f32_128x128d", "mfma_f32_64x64d", "mfma_f32_128x128d2", "mfma_f32_64x64d2",
+                                     "mfma_f64_128x128d", "mfma_f64_64x64d"])
 def test_direct_to_lds_on_seeded_random_shapes(dev, variant):
-    """Twenty-four shapes drawn from a fixed seed (1 <= M, N <= 700, 1 <= K <= 900), leading dimensions a
-    multiple of four with or without a gap, every layout and option combination in turn: the f32 kernels
-    that bring their slabs straight into LDS against the oracle, border tiles and k tails included."""
+    """Twenty-four shapes drawn from a fixed seed (1 <= M, N <= 700, 1 <= K <= 900), rows of 16-byte multiples
+    with or without a gap, every layout and option combination in turn: the kernels that bring their slabs
+    straight into LDS against the oracle, border tiles and k tails included."""
     rng = np.random.default_rng(20240611)
+    dtype = variant[5:8]
+    per = 4 if dtype == "f32" else 2
     options = [(None, None), (2.0, None), (1.5, 0.5), (None, -0.25)]
     assert dev.lib.wk_gemm_force_variant(variant.encode()) == 0
     try:
@@ -441,9 +452,9 @@ def test_direct_to_lds_on_seeded_random_shapes(dev, variant):
             op_a, op_b = OPS[n % 4]
             alpha, beta = options[(n // 4) % 4]
             cols_a, cols_b = (M if op_a else K), (K if op_b else N)
-            pad = 4 * int(rng.integers(0, 3))
-            check(dev, "f32", M, N, K, op_a, op_b, alpha, beta, seed=400 + n,
-                  lda=(cols_a + 3) // 4 * 4 + pad, ldb=(cols_b + 3) // 4 * 4 + pad, ldc=N + int(rng.integers(0, 4)))
+            pad = per * int(rng.integers(0, 3))
+            check(dev, dtype, M, N, K, op_a, op_b, alpha, beta, seed=400 + n,
+                  lda=-(-cols_a // per) * per + pad, ldb=-(-cols_b // per) * per + pad, ldc=N + int(rng.integers(0, 4)))
     finally:
         dev.lib.wk_gemm_force_variant(b"auto")
 

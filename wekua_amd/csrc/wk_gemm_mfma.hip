@@ -1588,7 +1588,7 @@ int wk::gemm_mfma_pick(const GemmProblem &p) {
         // the bounds-checked instantiation runs slower than the interior one (8191 x 8193 x 8190 against
         // 8192^3 on the 256 x 128 tile: 126 against 142 TFLOP/s with the tail split off)
         // (the direct-to-LDS kernels run ragged shapes in the same loop: their cost is in the tile count)
-        const bool slower_edge = needs_edge(p, d) && !(is_dma_variant(d.name) && d.dtype == WK_F32);
+        const bool slower_edge = needs_edge(p, d) && !is_dma_variant(d.name);
         const double eff = d.efficiency * (slower_edge ? (d.bm >= 256 ? 0.86 : d.bm >= 128 ? 0.944 : 0.93) : 1.0);
         const double cost = (rounds + d.fill) * d.bm * d.bn / eff;
         if (best < 0 || cost < best_cost) {
