@@ -25,9 +25,12 @@ from . import raw, synth
 OPS = [(0, 0, "NN"), (0, 1, "NT"), (1, 0, "TN"), (1, 1, "TT")]
 
 
-def _operand(rd, shape, seed):
+def _operand(rd, shape, seed, full_range=False):
     if rd.kind == "f":
         return synth.uniform(seed, shape, rd)
+    if full_range:
+        info = np.iinfo(rd)
+        return synth.integers(seed, shape, rd, int(info.min), int(info.max))
     return synth.integers(seed, shape, rd, -100, 100)
 
 
@@ -60,12 +63,15 @@ class Session:
         self.wk.memory.readFromBuffer(self.pipeline, t, host)
         return t
 
-    def tensor_on_device(self, dtype, shape, seed):
-        """A tensor filled on the device by random.uniform (floats in [-1, 1), integers in [-100, 100]):
-        the same value ranges as `tensor` of a seeded host array, without the host generation and the upload."""
+    def tensor_on_device(self, dtype, shape, seed, full_range=False):
+        """A tensor filled on the device by random.uniform (floats in [-1, 1), integers in [-100, 100] or,
+        with full_range, over the whole type): the same value ranges as `tensor` of a seeded host array,
+        without the host generation and the upload."""
         t = self.wk.Tensor.alloc(dtype, self.ctx, self.pipeline, shape)
         if raw.real_np_dtype(dtype).kind == "f":
             self.wk.random.uniform(self.pipeline, t, seed, -1.0, 1.0)
+        elif full_range:
+            self.wk.random.uniform(self.pipeline, t, seed)
         else:
             self.wk.random.uniform(self.pipeline, t, seed, -100, 100)
         return t
@@ -92,20 +98,23 @@ class Session:
         return ms.value / iters
 
 
-def time_gemm(ses, dtype, M, N, K, op_a, op_b, alpha, beta, iters=10, device_fill=False):
+def time_gemm(ses, dtype, M, N, K, op_a, op_b, alpha, beta, iters=10, device_fill=False, full_range=False):
     """blas.gemm on tensors created by Tensor.alloc (so with the library's own row pitches).
-    device_fill: operands drawn on the device instead of generated on the host and uploaded."""
+    device_fill: operands drawn on the device instead of generated on the host and uploaded.
+    full_range: integer entries over the whole type instead of [-100, 100] (the integer kernels are exact
+    either way, but the clock the part holds under the int8 matrix instruction depends on how many
+    operand bits toggle, and entries of small magnitude have zero upper digits)."""
     rd = raw.real_np_dtype(dtype)
     wk = ses.wk
     tail = (2,) if dtype.startswith("c") else ()
     if device_fill:
-        A = ses.tensor_on_device(dtype, (K, M) if op_a else (M, K), 1)
-        B = ses.tensor_on_device(dtype, (N, K) if op_b else (K, N), 2)
-        C = ses.tensor_on_device(dtype, (M, N), 3)
+        A = ses.tensor_on_device(dtype, (K, M) if op_a else (M, K), 1, full_range)
+        B = ses.tensor_on_device(dtype, (N, K) if op_b else (K, N), 2, full_range)
+        C = ses.tensor_on_device(dtype, (M, N), 3, full_range)
     else:
-        A = ses.tensor(dtype, _operand(rd, ((K, M) if op_a else (M, K)) + tail, 1))
-        B = ses.tensor(dtype, _operand(rd, ((N, K) if op_b else (K, N)) + tail, 2))
-        C = ses.tensor(dtype, _operand(rd, (M, N) + tail, 3))
+        A = ses.tensor(dtype, _operand(rd, ((K, M) if op_a else (M, K)) + tail, 1, full_range))
+        B = ses.tensor(dtype, _operand(rd, ((N, K) if op_b else (K, N)) + tail, 2, full_range))
+        C = ses.tensor(dtype, _operand(rd, (M, N) + tail, 3, full_range))
     # as benchmark/gemm.zig:186-196 does: one GemmPackedTensors for the run, passed to every call
     packed = wk.GemmPackedTensors.init(ses.pipeline, C, K, True)
     ses.pipeline.waitAndCleanup()
@@ -149,7 +158,7 @@ def cmd_gemm(ses, args):
         for op_a, op_b, name in OPS:
             if args.ops and name not in args.ops:
                 continue
-            ms, variant = time_gemm(ses, args.dtype, M, N, K, op_a, op_b, alpha, beta, device_fill=True)
+            ms, variant = time_gemm(ses, args.dtype, M, N, K, op_a, op_b, alpha, beta, device_fill=True, full_range=args.full_range)
             label = str(M) if M == N == K else f"{M}x{N}x{K}"
             print(f"{args.dtype:5s} {label:>6s} {name:2s} {ms:9.4f} {ops * M * N * K / ms / 1e9:9.2f}  {variant}", flush=True)
 
@@ -175,7 +184,8 @@ HBM_PEAK_GBS = 8000.0
 
 def baseline_gemm_cases():
     """(key, dtype, M, N, K, op_a, op_b, alpha, beta) for every GEMM of the benchmark configurations, in the
-    sweep order of benchmark/gemm.zig:240-283 (size outermost, the four op pairs inside)."""
+    sweep order of benchmark/gemm.zig:240-283 (size outermost, the four op pairs inside).  A key that ends in
+    `_full_range` draws its integer entries over the whole type instead of [-100, 100]."""
     cases = [("1_f32_gemm_512_NN", "f32", 512, 512, 512, 0, 0, 1.0, 0.0)]
     for n in (1024, 2048, 4096, 8192):
         for op_a, op_b, name in OPS:
@@ -186,6 +196,7 @@ def baseline_gemm_cases():
     cases.append(("4_f64_gemm_4096_NN", "f64", 4096, 4096, 4096, 0, 0, 1.0, 1.0))
     cases.append(("4_f64_gemm_8192x256x8192_NN", "f64", 8192, 256, 8192, 0, 0, 1.0, 1.0))
     cases.append(("4_i32_gemm_2048_NN", "i32", 2048, 2048, 2048, 0, 0, 3, -2))
+    cases.append(("4_i32_gemm_2048_NN_full_range", "i32", 2048, 2048, 2048, 0, 0, 3, -2))
     return cases
 
 
@@ -194,12 +205,15 @@ def run_baseline_configs(ses, log=None, device_fill=True):
     key -> {ms, value, unit, kernel, roofline}."""
     out = {}
     for key, dtype, M, N, K, op_a, op_b, alpha, beta in baseline_gemm_cases():
-        ms, variant = time_gemm(ses, dtype, M, N, K, op_a, op_b, alpha, beta, device_fill=device_fill)
+        ms, variant = time_gemm(ses, dtype, M, N, K, op_a, op_b, alpha, beta, device_fill=device_fill,
+                                full_range=key.endswith("_full_range"))
         peak, unit, bound, scale = PEAK[dtype]
         rate = 2.0 * M * N * K / ms / 1e9
         out[key] = {"ms": ms, "value": rate, "unit": unit, "kernel": variant,
                     "roofline": {"bound": bound, "achieved": rate * scale, "peak": peak, "unit": unit,
                                  "frac": rate * scale / peak}}
+        if raw.real_np_dtype(dtype).kind != "f":
+            out[key]["entries"] = "uniform over the whole type" if key.endswith("_full_range") else "uniform in [-100, 100]"
         if log:
             log(f"{key}: {ms:.4f} ms -> {rate:.1f} {unit} = {100 * rate * scale / peak:.1f} % of peak [{variant}]")
     for dt in ("f32", "f64"):
@@ -352,6 +366,7 @@ def main(argv=None):
     g.add_argument("--variant", default="auto")
     g.add_argument("--shapes", nargs="+", default=None, help="MxNxK ... instead of the square --sizes")
     g.add_argument("--ops", nargs="+", default=None, choices=["NN", "NT", "TN", "TT"], help="only these operand layouts")
+    g.add_argument("--full-range", action="store_true", help="integer entries over the whole type instead of [-100, 100]")
     a = sub.add_parser("axpy")
     a.add_argument("--dtype", default="f32")
     sub.add_parser("tensor")

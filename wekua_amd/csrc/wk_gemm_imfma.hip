@@ -4,14 +4,18 @@
 // C = alpha*op(A)*op(B) + beta*C in the element width, i.e. modulo 2^32 for i32/u32.  There is no
 // 32-bit integer matrix instruction, but the ring identity lets the int8 one do the work:
 //
-//   write every element as  a = S(a) + c,  c = 0x80808080,  where the four bytes of a ^ c, read as
-//   SIGNED bytes s_0..s_3, give  S(a) = sum_i 256^i s_i  (each unsigned byte u is s + 128).  Then
-//       sum_k a*b = sum_k S(a)S(b) + c*sum_k a + c*sum_k b - K*c*c            (mod 2^32)
-//   and   sum_k S(a)S(b) = sum_{i+j<=3} 256^(i+j) * sum_k s_i(a) s_j(b)       (mod 2^32)
+//   write every element in balanced digits,  a = sum_i 256^i s_i  (mod 2^32)  with s_i in [-128, 127]:
+//   with c = 0x80808080 and t = a + c (carries and all, modulo 2^32), a = t - c = sum_i 256^i (t_i - 128)
+//   over the unsigned bytes t_i of t, and t_i - 128 read as a signed byte is t_i ^ 0x80.  Then
+//       sum_k a*b = sum_{i+j<=3} 256^(i+j) * sum_k s_i(a) s_j(b)              (mod 2^32)
 //   (digit pairs with i+j >= 4 are multiples of 2^32).  The ten digit-pair sums are int8 x int8
 //   products accumulated in int32 -- exactly v_mfma_i32_32x32x32_i8 -- and wraparound of those
-//   accumulators is harmless because everything is taken modulo 2^32 anyway.  The row sums of A
-//   and column sums of B are collected from the elements as they pass through the loader.
+//   accumulators is harmless because everything is taken modulo 2^32 anyway.  Elements of small
+//   magnitude have zero upper digits, and zero padding is zero digits.  (The plain bytes of a with
+//   0x80 taken off each -- no carries -- also work, with row and column sums of the elements as
+//   correction terms; but then every small element has upper digits of -128 or 127, and with
+//   operands that toggle all their bits the part holds a lower clock under the int8 matrix
+//   instruction: 2048^3 with entries in [-100, 100] 81 against 61 us, 4096^3 536 against 390.)
 //
 // So one 32-bit product costs ten int8 matrix products; against the vector ALU (a 32-bit
 // multiply-add per lane and clock at best) that is still several times faster.
@@ -56,7 +60,7 @@ struct IArgs {
 
 // 4x4 byte transpose: e[t] = element at k+t (bytes = digits 0..3); p[d] = digit d of k+0..k+3
 __device__ __forceinline__ void digit_planes(const uint32_t e[4], uint32_t p[4]) {
-    const uint32_t a = e[0] ^ CBIAS, b = e[1] ^ CBIAS, c = e[2] ^ CBIAS, d = e[3] ^ CBIAS;
+    const uint32_t a = (e[0] + CBIAS) ^ CBIAS, b = (e[1] + CBIAS) ^ CBIAS, c = (e[2] + CBIAS) ^ CBIAS, d = (e[3] + CBIAS) ^ CBIAS;
     const uint32_t ab_lo = __builtin_amdgcn_perm(b, a, 0x05010400u); // a0 b0 a1 b1
     const uint32_t ab_hi = __builtin_amdgcn_perm(b, a, 0x07030602u); // a2 b2 a3 b3
     const uint32_t cd_lo = __builtin_amdgcn_perm(d, c, 0x05010400u);
@@ -77,8 +81,6 @@ void gemm_i32_mfma_kernel(IArgs g) {
     constexpr int PLANE_A = plane_bytes(BM), PLANE_B = plane_bytes(BN), SLAB_BYTES = slab_bytes(BM);
     extern __shared__ __align__(16) unsigned char lds_raw[];
     unsigned char *slabs = lds_raw;                                               // [2][SLAB_BYTES]
-    uint32_t *row_sum = reinterpret_cast<uint32_t *>(lds_raw + 2 * SLAB_BYTES);   // [BM]
-    uint32_t *col_sum = row_sum + BM;                                             // [BN]
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wm = wave >> 1, wn = wave & 1, l32 = lane & 31, lhi = lane >> 5;
@@ -91,8 +93,6 @@ void gemm_i32_mfma_kernel(IArgs g) {
         tile_n = in_group / gsz;
     }
     const uint32_t m0 = tile_m * BM, n0 = tile_n * BN;
-
-    if (tid < BM + BN) row_sum[tid] = 0; // row_sum and col_sum are adjacent
 
     i32x16 acc[4][2];
 #pragma unroll
@@ -109,7 +109,6 @@ void gemm_i32_mfma_kernel(IArgs g) {
     // two patch-loaded operands land on different threads.
     constexpr int A_NV = A_K ? BM * 8 / NT : 4, B_NV = B_K ? BN * 8 / NT : 4;
     u32x4 ra[A_NV], rb[B_NV];
-    uint32_t sum_a[4] = {0, 0, 0, 0}, sum_b[4] = {0, 0, 0, 0}; // KC: one per vector (its row); else one per patch column
 
     auto load_vec = [&](const uint32_t *base, uint32_t ld, uint32_t r, uint32_t r_lim, uint32_t c, uint32_t c_lim) -> u32x4 {
         const uint32_t *p = base + (size_t)r * ld + c;
@@ -149,8 +148,8 @@ void gemm_i32_mfma_kernel(IArgs g) {
             }
         }
     };
-    // registers -> digit planes in LDS; also adds the raw elements into the running sums
-    auto sstore = [&](unsigned char *planes, const u32x4 *src, uint32_t *sums, auto kc_tag, auto rows_tag, auto first_tag) {
+    // registers -> digit planes in LDS
+    auto sstore = [&](unsigned char *planes, const u32x4 *src, auto kc_tag, auto rows_tag, auto first_tag) {
         constexpr bool KC = decltype(kc_tag)::value;
         constexpr int ROWS = decltype(rows_tag)::value;
         constexpr int T0 = decltype(first_tag)::value;
@@ -162,7 +161,6 @@ void gemm_i32_mfma_kernel(IArgs g) {
                 const uint32_t e[4] = {src[i][0], src[i][1], src[i][2], src[i][3]};
                 uint32_t p[4];
                 digit_planes(e, p);
-                sums[i] += e[0] + e[1] + e[2] + e[3];
                 const int off = slot<P>(q / 8) * LDB + 4 * (q % 8);
 #pragma unroll
                 for (int d = 0; d < 4; ++d) *reinterpret_cast<uint32_t *>(planes + d * plane_bytes + off) = p[d];
@@ -176,7 +174,6 @@ void gemm_i32_mfma_kernel(IArgs g) {
                     const uint32_t e[4] = {src[0][c], src[1][c], src[2][c], src[3][c]};
                     uint32_t p[4];
                     digit_planes(e, p);
-                    sums[c] += e[0] + e[1] + e[2] + e[3];
                     const int off = slot<P>(row + c) * LDB + koff;
 #pragma unroll
                     for (int d = 0; d < 4; ++d) *reinterpret_cast<uint32_t *>(planes + d * plane_bytes + off) = p[d];
@@ -192,8 +189,8 @@ void gemm_i32_mfma_kernel(IArgs g) {
     };
     auto store_ab = [&](int buf) {
         unsigned char *s = slabs + buf * SLAB_BYTES;
-        sstore(s, ra, sum_a, integral_constant<bool, A_K>{}, integral_constant<int, BM>{}, integral_constant<int, T0_A>{});
-        sstore(s + 4 * PLANE_A, rb, sum_b, integral_constant<bool, B_K>{}, integral_constant<int, BN>{}, integral_constant<int, T0_B>{});
+        sstore(s, ra, integral_constant<bool, A_K>{}, integral_constant<int, BM>{}, integral_constant<int, T0_A>{});
+        sstore(s + 4 * PLANE_A, rb, integral_constant<bool, B_K>{}, integral_constant<int, BN>{}, integral_constant<int, T0_B>{});
     };
 
     // ---- matrix work of one slab ----------------------------------------------------------------
@@ -242,33 +239,10 @@ void gemm_i32_mfma_kernel(IArgs g) {
         }
     }
 
-    // ---- row / column sums of the raw elements ------------------------------------------------------
-    if constexpr (A_K) {
-#pragma unroll
-        for (int i = 0; i < BM * 8 / NT; ++i) atomicAdd(&row_sum[(tid + i * NT) / 8], sum_a[i]);
-    } else {
-        const int pq = tid - T0_A;
-        if (pq >= 0 && pq < BM * 2)
-#pragma unroll
-            for (int c = 0; c < 4; ++c) atomicAdd(&row_sum[4 * (pq % (BM / 4)) + c], sum_a[c]);
-    }
-    if constexpr (B_K) {
-#pragma unroll
-        for (int i = 0; i < BN * 8 / NT; ++i) atomicAdd(&col_sum[(tid + i * NT) / 8], sum_b[i]);
-    } else {
-        const int pq = tid - T0_B;
-        if (pq >= 0 && pq < BN * 2)
-#pragma unroll
-            for (int c = 0; c < 4; ++c) atomicAdd(&col_sum[4 * (pq % (BN / 4)) + c], sum_b[c]);
-    }
-    __syncthreads();
-
     // ---- epilogue: register r of lane l is C[8*(r/4) + 4*(l/32) + r%4][l%32] of its 32x32 block -----
-    const uint32_t kc2 = ktiles * BK * (CBIAS * CBIAS); // every k of the (zero-padded) slabs took part
 #pragma unroll
     for (int blk = 0; blk < 2; ++blk) {
-        const uint32_t lcol = wn * 64 + blk * 32 + l32, col = n0 + lcol;
-        const uint32_t csum = col_sum[lcol];
+        const uint32_t col = n0 + wn * 64 + blk * 32 + l32;
         uint32_t old[16];
         if (g.epi == EPI_ALPHA_BETA) {
 #pragma unroll
@@ -280,10 +254,9 @@ void gemm_i32_mfma_kernel(IArgs g) {
         }
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
-            const uint32_t lrow = wm * 32 + 8 * (r / 4) + 4 * lhi + (r % 4), row = m0 + lrow;
+            const uint32_t row = m0 + wm * 32 + 8 * (r / 4) + 4 * lhi + (r % 4);
             uint32_t v = (uint32_t)acc[0][blk][r] + ((uint32_t)acc[1][blk][r] << 8) + ((uint32_t)acc[2][blk][r] << 16) +
                          ((uint32_t)acc[3][blk][r] << 24);
-            v += CBIAS * (row_sum[lrow] + csum) - kc2;
             if (g.epi == EPI_ALPHA) v = g.alpha * v;
             else if (g.epi == EPI_ALPHA_BETA) v = g.alpha * v + g.beta * old[r];
             if (!EDGE || ((row < g.M) & (col < g.N))) g.C[(size_t)row * g.ldc + col] = v;
@@ -293,7 +266,7 @@ void gemm_i32_mfma_kernel(IArgs g) {
 
 template <int BM, bool AK, bool BKC, bool EDGE> int launch_one(hipStream_t st, const GemmProblem &p) {
     constexpr int NT = 4 * BM;
-    constexpr size_t lds = 2 * slab_bytes(BM) + (BM + BN) * sizeof(uint32_t);
+    constexpr size_t lds = 2 * slab_bytes(BM);
     auto kern = gemm_i32_mfma_kernel<BM, AK, BKC, EDGE>;
     static const hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
                                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);

@@ -3,15 +3,14 @@
 // reference's PackedTensors brings packed_a / packed_b and runs its pack kernel before every
 // product: src/blas/gemm.zig:272-357, 705-720).
 //
-// The arithmetic is the same ring identity (a = S(a) + c with c = 0x80808080, ten signed-digit
-// products, row and column sums; see wk_gemm_imfma.hip).  What changes is where the digits are made:
+// The arithmetic is the same ring identity (a = sum_i 256^i s_i with balanced signed digits s_i, ten
+// signed-digit products; see wk_gemm_imfma.hip).  What changes is where the digits are made:
 //
 //   pass 1  ipack_kernel      reads op(A) and op(B) once, whatever their layout, and writes their
 //                             signed-digit planes in the order the matrix instruction eats them:
 //                             1 KiB blocks, one per (32 rows, 32 k, digit), lane l of a wavefront
 //                             owning bytes 16 l .. 16 l + 15 = row l % 32, k 16 (l / 32) .. + 15.
-//                             Rows and k beyond the matrix are zero digits.  It also leaves the row
-//                             sums of the raw elements, one partial per k-range of the launch.
+//                             Rows and k beyond the matrix are zero digits.
 //   pass 2  gemm_i32_packed_kernel   128 x 128 tile, 8 waves, k-slab 32: 32 KiB of blocks per slab
 //                             go global -> registers -> LDS as plain 16-byte copies, fragments come
 //                             back with one conflict-free 16-byte LDS read each, and the loop is
@@ -19,8 +18,7 @@
 //                             arithmetic, no edge cases (the planes are padded to the tile), one
 //                             set of staging registers that fits beside the 128 accumulators.
 //
-// Workspace: 128 bytes per (padded row, 32 k) of each operand + the partial sums; for 2048^3 that
-// is 2 x 16 MiB.  The pack pass costs what reading A and B once and writing as much costs.
+// Workspace: 128 bytes per (padded row, 32 k) of each operand; for 2048^3 that is 2 x 16 MiB.  The pack pass costs what reading A and B once and writing as much costs.
 //
 // 8- and 16-bit integers take the same two passes with one or two digits per element (modulo 2^8 only
 // the pair (0,0) survives, modulo 2^16 the pairs with i + j <= 1): a slab is then four or two k-blocks
@@ -42,17 +40,16 @@ typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
 struct __attribute__((packed, aligned(4))) u32x4_u { u32x4 v; };
 
 constexpr int TILE = 128, BK = 32, BLOCK_BYTES = 1024, GROUP_BYTES = 4 * BLOCK_BYTES; // one slab of 32 rows: 4 blocks
-// element of D bytes = D digits; c = 0x80 in every byte; a slab holds 4 / D k-blocks of D digit blocks
+// element of D bytes = D digits; a slab holds 4 / D k-blocks of D digit blocks
 template <typename E> struct Digits {
     static constexpr int D = sizeof(E), KB_PER_SLAB = 4 / D;
-    static constexpr uint32_t CBIAS = D == 1 ? 0x80u : D == 2 ? 0x8080u : 0x80808080u;
 };
 constexpr int PACK_THREADS = 256;
 constexpr uint32_t MAX_KSPLIT = 16;
 
 struct Layout {
-    uint64_t Mp, Np, KB, slabs, ksplit; // KB: k-blocks of 32, padded to whole slabs
-    size_t planes_a, planes_b, sums_a, sums_b, total; // byte offsets into the workspace
+    uint64_t Mp, Np, KB, slabs, ksplit; // KB: k-blocks of 32, padded to whole slabs; ksplit: k-ranges of the pack launch
+    size_t planes_a, planes_b, total;   // byte offsets into the workspace
 };
 
 Layout make_layout(int digits, uint64_t M, uint64_t N, uint64_t K) {
@@ -73,16 +70,16 @@ Layout make_layout(int digits, uint64_t M, uint64_t N, uint64_t K) {
     w.ksplit = ks;
     w.planes_a = 0;
     w.planes_b = w.planes_a + (size_t)w.Mp / 32 * w.slabs * GROUP_BYTES;
-    w.sums_a = w.planes_b + (size_t)w.Np / 32 * w.slabs * GROUP_BYTES;
-    w.sums_b = w.sums_a + (size_t)w.ksplit * w.Mp * 4;
-    w.total = w.sums_b + (size_t)w.ksplit * w.Np * 4;
+    w.total = w.planes_b + (size_t)w.Np / 32 * w.slabs * GROUP_BYTES;
     return w;
 }
 
-// 4x4 byte transpose: e[t] = element at k+t (bytes = digits 0..3) -> p[d] = digit d of k+0..k+3, signed form
+// Balanced digits: with c = 0x80 in every byte, the bytes t_i of t = a + c (carries and all, modulo 2^32) give
+// a = t - c = sum_i 256^i (t_i - 128), and t_i - 128 as a signed byte is t_i ^ 0x80.  Small |a| have zero upper digits.
+// 4x4 byte transpose: e[t] = element at k+t -> p[d] = digit d of k+0..k+3
 __device__ __forceinline__ void digit_planes(const uint32_t e[4], uint32_t p[4]) {
     constexpr uint32_t CBIAS = 0x80808080u;
-    const uint32_t a = e[0] ^ CBIAS, b = e[1] ^ CBIAS, c = e[2] ^ CBIAS, d = e[3] ^ CBIAS;
+    const uint32_t a = (e[0] + CBIAS) ^ CBIAS, b = (e[1] + CBIAS) ^ CBIAS, c = (e[2] + CBIAS) ^ CBIAS, d = (e[3] + CBIAS) ^ CBIAS;
     const uint32_t ab_lo = __builtin_amdgcn_perm(b, a, 0x05010400u), ab_hi = __builtin_amdgcn_perm(b, a, 0x07030602u);
     const uint32_t cd_lo = __builtin_amdgcn_perm(d, c, 0x05010400u), cd_hi = __builtin_amdgcn_perm(d, c, 0x07030602u);
     p[0] = __builtin_amdgcn_perm(cd_lo, ab_lo, 0x05040100u);
@@ -91,10 +88,10 @@ __device__ __forceinline__ void digit_planes(const uint32_t e[4], uint32_t p[4])
     p[3] = __builtin_amdgcn_perm(cd_hi, ab_hi, 0x07060302u);
 }
 
-// the same for D = 1 or 2 digits: p[d] = byte d of the four (zero-extended) elements, signed form
+// the same for D = 1 or 2 digits of the four (zero-extended) elements (one digit: the byte itself, read as signed)
 template <int D> __device__ __forceinline__ void digit_planes_narrow(const uint32_t e[4], uint32_t p[D]) {
-    constexpr uint32_t c = D == 1 ? 0x80u : 0x8080u;
-    const uint32_t a = e[0] ^ c, b = e[1] ^ c, cc = e[2] ^ c, d = e[3] ^ c;
+    constexpr uint32_t c = D == 1 ? 0u : 0x8080u;
+    const uint32_t a = (e[0] + c) ^ c, b = (e[1] + c) ^ c, cc = (e[2] + c) ^ c, d = (e[3] + c) ^ c;
 #pragma unroll
     for (int i = 0; i < D; ++i)
         p[i] = ((a >> (8 * i)) & 0xffu) | (((b >> (8 * i)) & 0xffu) << 8) | (((cc >> (8 * i)) & 0xffu) << 16) |
@@ -105,7 +102,6 @@ struct PackOperand {
     const void *src;       // element (r, k) at src[r * ld + k] (k-contiguous) or src[k * ld + r]
     uint32_t ld, rows, row_blocks; // true rows; padded rows / 32
     unsigned char *planes;
-    uint32_t *sums;        // [ksplit][row_blocks * 32]
     uint32_t k_contiguous, vector_ok; // vector_ok: 16-byte loads along the contiguous direction are aligned
 };
 struct PackArgs {
@@ -118,8 +114,6 @@ struct PackArgs {
 template <typename E>
 __global__ __launch_bounds__(PACK_THREADS) void ipack_kernel(PackArgs g) {
     constexpr int D = Digits<E>::D;
-    constexpr uint32_t CBIAS = Digits<E>::CBIAS;
-    __shared__ uint32_t partial[PACK_THREADS];
     __shared__ __align__(16) unsigned char gather_tile[(PACK_THREADS / 64) * 32 * (32 * (D < 4 ? D : 1) + 4)];
     const int which = blockIdx.x >= g.op[0].row_blocks;
     const PackOperand &o = g.op[which];
@@ -129,7 +123,6 @@ __global__ __launch_bounds__(PACK_THREADS) void ipack_kernel(PackArgs g) {
     const uint32_t row = rb * 32 + l32;
     const bool row_ok = row < o.rows;
     const uint32_t kb_begin = blockIdx.y * g.kb_per_split, kb_end = min(g.KB, kb_begin + g.kb_per_split);
-    uint32_t sum = 0;
     for (uint32_t kb = kb_begin + wave; kb < kb_end; kb += PACK_THREADS / 64) {
         const uint32_t k0 = kb * BK + 16 * half;
         uint32_t e[16];
@@ -142,18 +135,10 @@ __global__ __launch_bounds__(PACK_THREADS) void ipack_kernel(PackArgs g) {
                 E raw[16];
                 __builtin_memcpy(raw, vec, 16 * D);
 #pragma unroll
-                for (int j = 0; j < 16; ++j) {
-                    e[j] = raw[j];
-                    sum += e[j];
-                }
+                for (int j = 0; j < 16; ++j) e[j] = raw[j];
             } else {
 #pragma unroll
-                for (int j = 0; j < 16; ++j) {
-                    const bool ok = row_ok && k0 + j < g.K;
-                    const uint32_t v = ok ? (uint32_t)p[j] : 0u;
-                    sum += v;
-                    e[j] = ok ? v : CBIAS; // CBIAS has all-zero signed digits
-                }
+                for (int j = 0; j < 16; ++j) e[j] = row_ok && k0 + j < g.K ? (uint32_t)p[j] : 0u;
             }
         } else if (D < 4 && o.vector_ok && rb * 32 + 32 <= o.rows && kb * BK + BK <= g.K) {
             // Row-contiguous storage of a narrow type, block inside the operand: a lane gathering its
@@ -177,20 +162,12 @@ __global__ __launch_bounds__(PACK_THREADS) void ipack_kernel(PackArgs g) {
             __builtin_amdgcn_wave_barrier();
             __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 #pragma unroll
-            for (int j = 0; j < 16; ++j) {
-                e[j] = *reinterpret_cast<const E *>(tile + (16 * half + j) * PITCH + l32 * D);
-                sum += e[j];
-            }
+            for (int j = 0; j < 16; ++j) e[j] = *reinterpret_cast<const E *>(tile + (16 * half + j) * PITCH + l32 * D);
             __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
             __builtin_amdgcn_wave_barrier(); // the tile is overwritten by the next block
         } else {
 #pragma unroll
-            for (int j = 0; j < 16; ++j) {
-                const bool ok = row_ok && k0 + j < g.K;
-                const uint32_t v = ok ? (uint32_t)src[(size_t)(k0 + j) * o.ld + row] : 0u;
-                sum += v;
-                e[j] = ok ? v : CBIAS;
-            }
+            for (int j = 0; j < 16; ++j) e[j] = row_ok && k0 + j < g.K ? (uint32_t)src[(size_t)(k0 + j) * o.ld + row] : 0u;
         }
         u32x4 out[D];
 #pragma unroll
@@ -206,21 +183,12 @@ __global__ __launch_bounds__(PACK_THREADS) void ipack_kernel(PackArgs g) {
 #pragma unroll
         for (int d = 0; d < D; ++d) *reinterpret_cast<u32x4 *>(dst + d * BLOCK_BYTES) = out[d];
     }
-    partial[tid] = sum;
-    __syncthreads();
-    if (tid < 32) {
-        uint32_t s = 0;
-#pragma unroll
-        for (int i = 0; i < PACK_THREADS / 32; ++i) s += partial[tid + 32 * i];
-        o.sums[(size_t)blockIdx.y * o.row_blocks * 32 + rb * 32 + tid] = s;
-    }
 }
 
 struct PArgs {
     const unsigned char *planes_a, *planes_b;
-    const uint32_t *sums_a, *sums_b;
     void *C;
-    uint32_t M, N, K, slabs, Mp, Np, ksplit, ldc, tiles_m, tiles_n;
+    uint32_t M, N, K, slabs, Mp, Np, ldc, tiles_m, tiles_n;
     int epi;
     uint32_t alpha, beta;
     uint32_t patch_m, patch_n; // the direct-to-LDS kernel's tile walk (0: groups of tile rows)
@@ -243,7 +211,7 @@ template <int BM, int WMF = 1, int BN = TILE> struct PackedTile {
     static constexpr int STAGE_BYTES = GROUPS * GROUP_BYTES;
     static constexpr int GROUPS_PER_PASS = NT * 16 / GROUP_BYTES; // 1 or 2
     static constexpr int PASSES = GROUPS / GROUPS_PER_PASS;
-    static constexpr size_t LDS_BYTES = 2 * STAGE_BYTES + (BM + BN) * sizeof(uint32_t);
+    static constexpr size_t LDS_BYTES = 2 * STAGE_BYTES;
 };
 
 template <typename E, int BM, bool EDGE, int WMF = 1, int BN = TILE>
@@ -252,14 +220,11 @@ void gemm_int_packed_kernel(PArgs g) {
     using TL = PackedTile<BM, WMF, BN>;
     constexpr int WNF = BN / 64;        // 32-column blocks of B per wavefront
     constexpr bool ONE_SET = BN > TILE; // the 256 x 256 tile has registers for one staging set only
-    static_assert(BM + BN <= TL::NT && TL::GROUPS % TL::GROUPS_PER_PASS == 0, "tile shape");
+    static_assert(TL::GROUPS % TL::GROUPS_PER_PASS == 0, "tile shape");
     constexpr int D = Digits<E>::D, KB_PER_SLAB = Digits<E>::KB_PER_SLAB;
-    constexpr uint32_t CBIAS = Digits<E>::CBIAS;
     constexpr int STAGE_BYTES = TL::STAGE_BYTES, PASSES = TL::PASSES, A_GROUPS = BM / 32;
     extern __shared__ __align__(16) unsigned char lds_raw[];
     unsigned char *stages = lds_raw;                                              // [2][STAGE_BYTES]
-    uint32_t *row_sum = reinterpret_cast<uint32_t *>(lds_raw + 2 * STAGE_BYTES);  // [BM]
-    uint32_t *col_sum = row_sum + BM;                                             // [BN]
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wm = wave >> 1, wn = wave & 1, l32 = lane & 31, lhi = lane >> 5;
@@ -271,19 +236,6 @@ void gemm_int_packed_kernel(PArgs g) {
         tile_n = in_group / gsz;
     }
     const uint32_t m0 = tile_m * BM, n0 = tile_n * BN;
-
-    if (tid < BM + BN) {
-        const uint32_t *src = tid < BM ? g.sums_a + m0 + tid : g.sums_b + n0 + (tid - BM);
-        const uint32_t stride = tid < BM ? g.Mp : g.Np;
-        // (all partial sums requested at once: one after the other they cost a memory latency each)
-        uint32_t part[MAX_KSPLIT];
-#pragma unroll
-        for (uint32_t i = 0; i < MAX_KSPLIT; ++i) part[i] = i < g.ksplit ? src[(size_t)i * stride] : 0u;
-        uint32_t s = 0;
-#pragma unroll
-        for (uint32_t i = 0; i < MAX_KSPLIT; ++i) s += part[i];
-        row_sum[tid] = s; // col_sum follows row_sum
-    }
 
     i32x16 acc[D][WMF][WNF]; // one set per shift i + j
 #pragma unroll
@@ -405,14 +357,12 @@ void gemm_int_packed_kernel(PArgs g) {
 
     // epilogue: register r of lane l is C[8*(r/4) + 4*(l/32) + r%4][l%32] of its 32x32 block
     // (all of it modulo 2^32; the store keeps the low 8 * D bits, which is the product modulo 2^(8 D))
-    const uint32_t kc2 = g.K * (CBIAS * CBIAS);
     E *C = static_cast<E *>(g.C);
 #pragma unroll
     for (int am = 0; am < WMF; ++am)
 #pragma unroll
     for (int blk = 0; blk < WNF; ++blk) {
-        const uint32_t lcol = wn * (BN / 2) + blk * 32 + l32, col = n0 + lcol;
-        const uint32_t csum = col_sum[lcol];
+        const uint32_t col = n0 + wn * (BN / 2) + blk * 32 + l32;
         uint32_t old[16];
         if (g.epi == EPI_ALPHA_BETA) {
 #pragma unroll
@@ -424,11 +374,10 @@ void gemm_int_packed_kernel(PArgs g) {
         }
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
-            const uint32_t lrow = (wm * WMF + am) * 32 + 8 * (r / 4) + 4 * lhi + (r % 4), row = m0 + lrow;
+            const uint32_t row = m0 + (wm * WMF + am) * 32 + 8 * (r / 4) + 4 * lhi + (r % 4);
             uint32_t v = 0;
 #pragma unroll
             for (int s = 0; s < D; ++s) v += (uint32_t)acc[s][am][blk][r] << (8 * s);
-            v += CBIAS * (row_sum[lrow] + csum) - kc2;
             if (g.epi == EPI_ALPHA) v = g.alpha * v;
             else if (g.epi == EPI_ALPHA_BETA) v = g.alpha * v + g.beta * old[r];
             if (!EDGE || ((row < g.M) & (col < g.N))) C[(size_t)row * g.ldc + col] = (E)v;
@@ -461,7 +410,7 @@ template <typename E, int BM, bool EDGE, int WMF = 1, int BN = TILE> int launch_
 // own loads of slab kt + 1, barrier, read its fragments into the other set, the other half.
 struct PackedDmaTile {
     static constexpr int BM = TILE, BN = TILE, GROUPS = 8, STAGE_BYTES = GROUPS * GROUP_BYTES;
-    static constexpr size_t lds_bytes(int ns) { return (size_t)ns * STAGE_BYTES + (BM + BN) * sizeof(uint32_t); }
+    static constexpr size_t lds_bytes(int ns) { return (size_t)ns * STAGE_BYTES; }
 };
 
 template <bool EDGE, int NS>
@@ -470,10 +419,7 @@ void gemm_i32_packed_dma_kernel(PArgs g) {
     using namespace wk::lds_dma;
     using TL = PackedDmaTile;
     constexpr int BM = TL::BM, BN = TL::BN, STAGE_BYTES = TL::STAGE_BYTES;
-    constexpr uint32_t CBIAS = 0x80808080u;
     extern __shared__ __align__(16) unsigned char lds_raw[];
-    uint32_t *row_sum = reinterpret_cast<uint32_t *>(lds_raw + NS * STAGE_BYTES); // [BM], then col_sum [BN]
-    uint32_t *col_sum = row_sum + BM;
 
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -492,21 +438,6 @@ void gemm_i32_packed_dma_kernel(PArgs g) {
         tile_n = in_group / gsz;
     }
     const uint32_t m0 = tile_m * BM, n0 = tile_n * BN;
-
-    {
-        const uint32_t *src = tid < BM ? g.sums_a + m0 + tid : g.sums_b + n0 + (tid - BM);
-        const uint32_t stride = tid < BM ? g.Mp : g.Np;
-        uint32_t part[MAX_KSPLIT]; // all partial sums requested at once
-#pragma unroll
-        for (uint32_t i = 0; i < MAX_KSPLIT; ++i) part[i] = i < g.ksplit ? src[(size_t)i * stride] : 0u;
-        uint32_t s = 0;
-#pragma unroll
-        for (uint32_t i = 0; i < MAX_KSPLIT; ++i) s += part[i];
-        row_sum[tid] = s; // col_sum follows row_sum; published by the first barrier below
-    }
-    // these loads are older than every slab load: wait for them here, so that the counted waits below
-    // count slab loads only
-    wait_vm<0>();
 
     // wavefront w brings groups 2 w and 2 w + 1 of every slab: A's row groups 0..3, then B's column groups
     const unsigned char *src_g[2];
@@ -593,7 +524,6 @@ void gemm_i32_packed_dma_kernel(PArgs g) {
     for (int n = 0; n < NS - 1; ++n)
         if ((uint32_t)n < ktiles) issue(st[n]);
     wait_vm_slabs<LOADS, NS - 2>(ktiles - 1);
-    wait_lgkm0(); // (the row and column sums are in LDS before anyone passes the barrier)
     __builtin_amdgcn_s_barrier();
     static_for<16>([&](auto f_tag) { read_frag(st[0], integral_constant<int, 0>{}, f_tag); });
 
@@ -651,7 +581,6 @@ void gemm_i32_packed_dma_kernel(PArgs g) {
 
     // epilogue, as in the kernel above; the C_old values of all four blocks are requested before any is
     // used (the fragment registers are free by now): a one-round launch pays every memory latency here in full
-    const uint32_t kc2 = g.K * (CBIAS * CBIAS);
     uint32_t *C = static_cast<uint32_t *>(g.C);
     uint32_t old[2][2][16];
     if (g.epi == EPI_ALPHA_BETA) {
@@ -671,15 +600,13 @@ void gemm_i32_packed_dma_kernel(PArgs g) {
     for (int am = 0; am < 2; ++am)
 #pragma unroll
         for (int blk = 0; blk < 2; ++blk) {
-            const uint32_t lcol = wn * 64 + blk * 32 + l32, col = n0 + lcol;
-            const uint32_t csum = col_sum[lcol];
+            const uint32_t col = n0 + wn * 64 + blk * 32 + l32;
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
-                const uint32_t lrow = (wm * 2 + am) * 32 + 8 * (r / 4) + 4 * lhi + (r % 4), row = m0 + lrow;
+                const uint32_t row = m0 + (wm * 2 + am) * 32 + 8 * (r / 4) + 4 * lhi + (r % 4);
                 uint32_t v = 0;
 #pragma unroll
                 for (int s = 0; s < 4; ++s) v += (uint32_t)acc[s][am][blk][r] << (8 * s);
-                v += CBIAS * (row_sum[lrow] + csum) - kc2;
                 if (g.epi == EPI_ALPHA) v = g.alpha * v;
                 else if (g.epi == EPI_ALPHA_BETA) v = g.alpha * v + g.beta * old[am][blk][r];
                 if (!EDGE || ((row < g.M) & (col < g.N))) C[(size_t)row * g.ldc + col] = v;
@@ -719,25 +646,22 @@ int digits_of(int dtype) {
 template <typename E> int launch_typed(hipStream_t st, const GemmProblem &p, unsigned char *ws, const Layout &w) {
     constexpr int D = Digits<E>::D;
     PackArgs pa;
-    auto operand = [&](PackOperand &o, const void *src, uint64_t ld, uint64_t rows, uint64_t rows_p, bool kc, size_t planes,
-                       size_t sums) {
+    auto operand = [&](PackOperand &o, const void *src, uint64_t ld, uint64_t rows, uint64_t rows_p, bool kc, size_t planes) {
         o.src = src;
         o.ld = (uint32_t)ld;
         o.rows = (uint32_t)rows;
         o.row_blocks = (uint32_t)(rows_p / 32);
         o.planes = ws + planes;
-        o.sums = reinterpret_cast<uint32_t *>(ws + sums);
         o.k_contiguous = kc;
         // 16-byte loads along the contiguous direction (k, or for the narrow types also the rows) are aligned
         o.vector_ok = (kc || D < 4) && (ld * D) % 16 == 0 && (reinterpret_cast<uintptr_t>(src) & 15u) == 0;
     };
-    operand(pa.op[0], p.A, p.lda, p.M, w.Mp, !p.op_a, w.planes_a, w.sums_a); // A is k-contiguous for op N
-    operand(pa.op[1], p.B, p.ldb, p.N, w.Np, p.op_b != 0, w.planes_b, w.sums_b); // B for op T
+    operand(pa.op[0], p.A, p.lda, p.M, w.Mp, !p.op_a, w.planes_a); // A is k-contiguous for op N
+    operand(pa.op[1], p.B, p.ldb, p.N, w.Np, p.op_b != 0, w.planes_b); // B for op T
     pa.K = (uint32_t)p.K;
     pa.KB = (uint32_t)w.KB;
     pa.kb_per_split = (uint32_t)((w.KB + w.ksplit - 1) / w.ksplit);
-    // A's row blocks come first in the grid: with B's planes and column sums kept from the previous
-    // call only those are launched
+    // A's row blocks come first in the grid: with B's planes kept from the previous call only those are launched
     const uint64_t row_blocks = (p.reuse_b ? w.Mp : w.Mp + w.Np) / 32;
     hipLaunchKernelGGL(ipack_kernel<E>, dim3((unsigned)row_blocks, (unsigned)w.ksplit), dim3(PACK_THREADS), 0, st, pa);
     int rc = launch_status();
@@ -746,11 +670,9 @@ template <typename E> int launch_typed(hipStream_t st, const GemmProblem &p, uns
     PArgs g;
     g.planes_a = ws + w.planes_a;
     g.planes_b = ws + w.planes_b;
-    g.sums_a = reinterpret_cast<const uint32_t *>(ws + w.sums_a);
-    g.sums_b = reinterpret_cast<const uint32_t *>(ws + w.sums_b);
     g.C = p.C;
     g.M = (uint32_t)p.M; g.N = (uint32_t)p.N; g.K = (uint32_t)p.K;
-    g.slabs = (uint32_t)w.slabs; g.Mp = (uint32_t)w.Mp; g.Np = (uint32_t)w.Np; g.ksplit = (uint32_t)w.ksplit;
+    g.slabs = (uint32_t)w.slabs; g.Mp = (uint32_t)w.Mp; g.Np = (uint32_t)w.Np;
     g.ldc = (uint32_t)p.ldc;
     g.tiles_m = (uint32_t)(w.Mp / TILE);
     g.tiles_n = (uint32_t)(w.Np / TILE);
