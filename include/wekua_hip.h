@@ -175,7 +175,7 @@ int    wk_gemm(wk_stream *s, int dtype, int op_a, int op_b, uint64_t M, uint64_t
 size_t wk_gemm_workspace_bytes(int dtype, int op_a, int op_b, uint64_t M, uint64_t N, uint64_t K);
 
 /* wk_gemm for a caller whose op(B) has not changed since the previous call: the workspace still
- * holds B's packed form (digit planes and column sums of an integer B; the real 2K x 2N form of a
+ * holds B's packed form (digit planes of an integer B; the real 2K x 2N form of a
  * complex B, which has alpha folded in), so only A is packed again.  The reference packs both
  * operands before every product (gemm.zig:713-719) although its callers' B is usually a weight
  * matrix that changes once per step; this is the entry point behind blas.PackedTensors.keepB.

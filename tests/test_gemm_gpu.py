@@ -155,12 +155,13 @@ def test_int32_packed_needs_its_workspace(dev):
 
 
 def test_int32_matrix_core_extremes(dev):
-    """Inputs built from the byte values that stress the signed-digit split: 0x00, 0x7f, 0x80, 0xff in
-    every byte position, so that every digit pair hits -128 * -128 and the row / column sum
-    corrections wrap many times."""
+    """Inputs built from the byte values that stress the split into balanced signed digits: 0x00, 0x7f,
+    0x80, 0xff in every byte position, values whose digits are all -128 or all 127 (every digit pair then
+    hits -128 * -128), and values one off a carry into the next digit (0x..7f / 0x..80 at each byte)."""
     import oracle
     vals = np.array([0x00000000, 0x7f7f7f7f, 0x80808080, 0xffffffff, 0x80000000, 0x7fffffff, 0x00800080, 0xff00ff00,
-                     0x01010101, 0x807f807f], dtype=np.uint32)
+                     0x01010101, 0x807f807f, 0x7f7f7f80, 0x0000007f, 0x00000080, 0x00007f80, 0x007f8000, 0x7f800000,
+                     0xffffff80, 0xffffff7f, 0xffff8000, 0x80007fff], dtype=np.uint32)
     M, N, K = 128, 128, 320
     rng = np.random.default_rng(77)
     a = vals[rng.integers(0, len(vals), (M, K))].view(np.int32)
