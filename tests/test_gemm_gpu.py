@@ -460,6 +460,31 @@ def test_direct_to_lds_on_seeded_random_shapes(dev, variant):
         dev.lib.wk_gemm_force_variant(b"auto")
 
 
+@pytest.mark.parametrize("dtype,M,N,K,split", [("f32", 4097, 4095, 1024, True),    # one row beyond sixteen tiles of 256
+                                                ("f32", 2050, 4097, 1536, True),    # two rows and one column beyond
+                                                ("f32", 4096, 4100, 1024, True),    # four columns beyond
+                                                ("f32", 4097, 4095, 64, False),     # short k: a launch more costs more than it saves
+                                                ("f32", 4160, 4096, 1024, True),    # 64 rows beyond: a quarter of the tile, still thin
+                                                ("f32", 4225, 4096, 1024, True),    # one row beyond 33 tiles of 128
+                                                ("f32", 4200, 4096, 1024, False),   # 104 rows beyond: a tile row of its own
+                                                ("f32", 1025, 1024, 1024, False),   # the body is too small to carry a strip's launch
+                                                ("f64", 2049, 2050, 1024, True)])
+def test_thin_strips_beyond_whole_tiles_are_products_of_their_own(dev, dtype, M, N, K, split):
+    """A matrix a few rows or columns larger than whole large tiles is multiplied in parts (the body of whole
+    tiles, then the thin strips beyond it, each with its own kernel) when k is long and the body large enough
+    to carry the extra launches; the name query marks it.  Every entry of C against the oracle, all four layouts, rows of 16-byte
+    multiples (which is what tensors have), C with a gap between rows whose poison must survive."""
+    from wekua_amd import raw
+    per = 4 if dtype == "f32" else 2
+    up = lambda n: -(-n // per) * per
+    for op_a, op_b in OPS:
+        lda, ldb = up(M if op_a else K), up(K if op_b else N)
+        name = dev.lib.wk_gemm_variant(raw.dtype_id(dtype), op_a, op_b, M, N, K, lda, ldb, N + 3, None, None, None).decode()
+        assert name.endswith("+strips") == split, (name, op_a, op_b)
+        check(dev, dtype, M, N, K, op_a, op_b, 1.5, 0.5, seed=500 + op_a * 2 + op_b, lda=lda, ldb=ldb, ldc=N + 3)
+    check(dev, dtype, M, N, K, 0, 1, None, None, seed=505, lda=up(K), ldb=up(K))
+
+
 def test_left_over_tiles_run_as_a_k_split_tail(dev):
     """A launch whose tiles do not fill whole rounds of the compute units: the whole rounds run as they
     are, the left-over tiles as a second launch with k split over work-groups.  Checked: the plan of the

@@ -3,8 +3,11 @@
 // per-tensor work-item tables).
 #include "wk_internal.hpp"
 
+#include <array>
 #include <atomic>
+#include <cstdlib>
 #include <cstring>
+#include <string>
 
 using namespace wk;
 
@@ -89,6 +92,55 @@ int build_problem(GemmProblem &p, int dtype, int op_a, int op_b, uint64_t M, uin
     return WK_OK;
 }
 
+// A matrix that is a few rows or columns more than whole large tiles (4097 x 4095: one row beyond 16 tiles of
+// 256) makes every large tile pay for a started round and sends the whole product to the small tile.  Such
+// a product is launched in parts instead: the body of whole tiles, and the thin strip(s) beyond it as
+// products of their own (same K, disjoint parts of C, the same arithmetic per entry), each with the kernel the
+// cost model picks for it.  A strip of one row still reads the whole other operand, so this wants a body
+// that is large beside it and a k long enough for a launch more not to matter.  Measured (N,N, TFLOP/s):
+// f32 4097 x 4095 x 4093 125-129 -> 137-139, 4097^3 120 -> 130, 8191 x 8193 x 8190 136-141 -> 142-143,
+// 6145 x 6144 x 6144 136 -> 141, 3073 x 3072 x 3072 121 -> 127, 2049 x 2047 x 2050 103 -> 111 (T,N: 102 -> 99);
+// f64 4097 x 4095 x 4093 61-64 -> 69.6, 4100^3 60-63 -> 67, 2049 x 2047 x 2050 55 -> 58.5.
+struct StripPlan {
+    int parts = 0;
+    GemmProblem part[3]; // body, rows beyond it (over all of N), columns beyond it (over the body's rows)
+};
+bool plan_strips(const GemmProblem &p, StripPlan &out) {
+    if ((p.dtype != WK_F32 && p.dtype != WK_F64) || p.ext) return false;
+    if (!(p.dtype == WK_F32 ? gemm_f32_dma_applies(p, 128, 128) : gemm_f64_dma_applies(p, 128, 128))) return false;
+    // thin: at most a quarter of the tile's rows (256 or 128 of them: the large tiles) or of its 128 columns
+    const uint64_t bn = 128;
+    uint64_t bm = p.dtype == WK_F32 ? 256 : 128;
+    if (bm == 256 && (p.M % 256 == 0 || p.M % 256 > 64)) bm = 128;
+    const uint64_t m_rem = p.M % bm, n_rem = p.N % bn;
+    const bool thin_m = m_rem && m_rem <= bm / 4 && p.M > bm, thin_n = n_rem && n_rem <= bn / 4 && p.N > bn;
+    if (!thin_m && !thin_n) return false;
+    if (p.K < 512 || (thin_m ? p.M - m_rem : p.M) * (thin_n ? p.N - n_rem : p.N) < (1ull << 21)) return false;
+    const size_t es = wk_dtype_size(p.dtype);
+    const uint64_t Mb = thin_m ? p.M - m_rem : p.M, Nb = thin_n ? p.N - n_rem : p.N;
+    out.parts = 0;
+    GemmProblem &body = out.part[out.parts++];
+    body = p;
+    body.M = Mb;
+    body.N = Nb;
+    if (thin_m) {
+        GemmProblem &q = out.part[out.parts++];
+        q = p;
+        q.M = m_rem;
+        q.A = static_cast<const unsigned char *>(p.A) + (p.op_a ? Mb : Mb * p.lda) * es;
+        q.C = static_cast<unsigned char *>(p.C) + Mb * p.ldc * es;
+    }
+    if (thin_n) {
+        GemmProblem &q = out.part[out.parts++];
+        q = p;
+        q.M = Mb;
+        q.N = n_rem;
+        q.B = static_cast<const unsigned char *>(p.B) + (p.op_b ? Nb * p.ldb : Nb) * es;
+        q.C = static_cast<unsigned char *>(p.C) + Nb * es;
+    }
+    return true;
+}
+
 int choose(const GemmProblem &p) {
     const int forced = g_forced.load(std::memory_order_relaxed);
     if (forced == -1) return -1;
@@ -148,6 +200,17 @@ static int gemm_entry(wk_stream *s, int dtype, int op_a, int op_b, uint64_t M, u
                 return gemm_int_packed_launch(s->stream, real, rest, rest_bytes);
             const int rv = gemm_mfma_pick(real);
             return rv >= 0 ? gemm_mfma_launch(s->stream, real, rv) : gemm_generic_launch(s->stream, real);
+        }
+    }
+    if (g_forced.load(std::memory_order_relaxed) == -2) {
+        StripPlan sp;
+        if (plan_strips(p, sp)) {
+            for (int i = 0; i < sp.parts; ++i) {
+                const int pv = gemm_mfma_pick(sp.part[i]);
+                rc = pv >= 0 ? gemm_mfma_launch(s->stream, sp.part[i], pv) : gemm_generic_launch(s->stream, sp.part[i]);
+                if (rc) return rc;
+            }
+            return WK_OK;
         }
     }
     const int v = choose(p);
@@ -211,6 +274,18 @@ const char *wk_gemm_variant(int dtype, int op_a, int op_b, uint64_t M, uint64_t 
     p.scratch_bytes = WK_STREAM_SCRATCH_BYTES;
     p.counters = &dummy_counter;
     p.num_counters = WK_GEMM_COUNTERS;
+    if (g_forced.load(std::memory_order_relaxed) == -2) {
+        StripPlan sp;
+        if (plan_strips(p, sp)) { // the body's kernel, marked: the strips beyond it are launches of their own
+            const int bv = gemm_mfma_pick(sp.part[0]);
+            static const std::array<std::string, 64> marked = [] {
+                std::array<std::string, 64> names;
+                for (int i = 0; i < 64 && gemm_mfma_variant_name(i); ++i) names[i] = std::string(gemm_mfma_variant_name(i)) + "+strips";
+                return names;
+            }();
+            if (bv >= 0 && bv < 64) return marked[bv].c_str();
+        }
+    }
     const int v = choose(p);
     return v >= 0 ? gemm_mfma_variant_name(v) : k_generic_name;
 }

@@ -1557,7 +1557,10 @@ namespace {
 // but 512 x 512 x 2048 14.4 -> 18.6; f64 512 x 512 x 8192 111 -> 89 us, 256 x 256 x 8192 111 -> 89,
 // 512 x 512 x 2048 32 -> 30.
 bool split_pays(const GemmProblem &p, const GemmSplitPlan &plan) {
-    return plan.shares >= 2 && p.K >= (p.dtype == WK_F64 ? 2048u : 4096u);
+    // (a thin strip -- a handful of rows or columns -- reads the whole other operand whatever the tile: there the
+    // shares pay from half that length on, 1 x 4095 x 4093 47.5 -> 35.6 us, 4096 x 1 x 4093 76 -> 51)
+    const bool strip = p.dtype == WK_F32 && (p.M <= 64 || p.N <= 64);
+    return plan.shares >= 2 && p.K >= (p.dtype == WK_F64 || strip ? 2048u : 4096u);
 }
 } // namespace
 
