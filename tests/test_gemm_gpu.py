@@ -466,8 +466,9 @@ def test_direct_to_lds_on_seeded_random_shapes(dev, variant):
                                                 ("f32", 4097, 4095, 64, False),     # short k: a launch more costs more than it saves
                                                 ("f32", 4160, 4096, 1024, True),    # 64 rows beyond: a quarter of the tile, still thin
                                                 ("f32", 4225, 4096, 1024, True),    # one row beyond 33 tiles of 128
-                                                ("f32", 4200, 4096, 1024, False),   # 104 rows beyond: a tile row of its own
-                                                ("f32", 1025, 1024, 1024, False),   # the body is too small to carry a strip's launch
+                                                ("f32", 4200, 4096, 1024, True),    # 104 rows beyond: split off because the cost model says so
+                                                ("f32", 3000, 3000, 1024, False),   # ... and here it does not: the body would fill half a round
+                                                ("f32", 2049, 2047, 1024, False),   # the body is too small to carry a strip's launch
                                                 ("f64", 2049, 2050, 1024, True)])
 def test_thin_strips_beyond_whole_tiles_are_products_of_their_own(dev, dtype, M, N, K, split):
     """A matrix a few rows or columns larger than whole large tiles is multiplied in parts (the body of whole

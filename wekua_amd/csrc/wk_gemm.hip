@@ -99,46 +99,87 @@ int build_problem(GemmProblem &p, int dtype, int op_a, int op_b, uint64_t M, uin
 // cost model picks for it.  A strip of one row still reads the whole other operand, so this wants a body
 // that is large beside it and a k long enough for a launch more not to matter.  Measured (N,N, TFLOP/s):
 // f32 4097 x 4095 x 4093 125-129 -> 137-139, 4097^3 120 -> 130, 8191 x 8193 x 8190 136-141 -> 142-143,
-// 6145 x 6144 x 6144 136 -> 141, 3073 x 3072 x 3072 121 -> 127, 2049 x 2047 x 2050 103 -> 111 (T,N: 102 -> 99);
-// f64 4097 x 4095 x 4093 61-64 -> 69.6, 4100^3 60-63 -> 67, 2049 x 2047 x 2050 55 -> 58.5.
+// 6145 x 6144 x 6144 136 -> 141, 3073 x 3072 x 3072 121 -> 127;
+// f64 4097 x 4095 x 4093 61-64 -> 69.6, 4100^3 60-63 -> 67.  Wider remainders
+// are split off only where the cost model says so (second half of plan_strips).
 struct StripPlan {
     int parts = 0;
     GemmProblem part[3]; // body, rows beyond it (over all of N), columns beyond it (over the body's rows)
 };
-bool plan_strips(const GemmProblem &p, StripPlan &out) {
-    if ((p.dtype != WK_F32 && p.dtype != WK_F64) || p.ext) return false;
-    if (!(p.dtype == WK_F32 ? gemm_f32_dma_applies(p, 128, 128) : gemm_f64_dma_applies(p, 128, 128))) return false;
-    // thin: at most a quarter of the tile's rows (256 or 128 of them: the large tiles) or of its 128 columns
-    const uint64_t bn = 128;
-    uint64_t bm = p.dtype == WK_F32 ? 256 : 128;
-    if (bm == 256 && (p.M % 256 == 0 || p.M % 256 > 64)) bm = 128;
-    const uint64_t m_rem = p.M % bm, n_rem = p.N % bn;
-    const bool thin_m = m_rem && m_rem <= bm / 4 && p.M > bm, thin_n = n_rem && n_rem <= bn / 4 && p.N > bn;
-    if (!thin_m && !thin_n) return false;
-    if (p.K < 512 || (thin_m ? p.M - m_rem : p.M) * (thin_n ? p.N - n_rem : p.N) < (1ull << 21)) return false;
+// the product in parts: rows [0, Mb) x columns [0, Nb), then the rows beyond Mb over all of N, then the
+// columns beyond Nb over the body's rows (Mb = M / Nb = N: no such strip)
+void make_parts(const GemmProblem &p, uint64_t Mb, uint64_t Nb, StripPlan &out) {
     const size_t es = wk_dtype_size(p.dtype);
-    const uint64_t Mb = thin_m ? p.M - m_rem : p.M, Nb = thin_n ? p.N - n_rem : p.N;
     out.parts = 0;
     GemmProblem &body = out.part[out.parts++];
     body = p;
     body.M = Mb;
     body.N = Nb;
-    if (thin_m) {
+    if (Mb < p.M) {
         GemmProblem &q = out.part[out.parts++];
         q = p;
-        q.M = m_rem;
+        q.M = p.M - Mb;
         q.A = static_cast<const unsigned char *>(p.A) + (p.op_a ? Mb : Mb * p.lda) * es;
         q.C = static_cast<unsigned char *>(p.C) + Mb * p.ldc * es;
     }
-    if (thin_n) {
+    if (Nb < p.N) {
         GemmProblem &q = out.part[out.parts++];
         q = p;
         q.M = Mb;
-        q.N = n_rem;
+        q.N = p.N - Nb;
         q.B = static_cast<const unsigned char *>(p.B) + (p.op_b ? Nb * p.ldb : Nb) * es;
         q.C = static_cast<unsigned char *>(p.C) + Nb * es;
     }
-    return true;
+}
+
+bool plan_strips(const GemmProblem &p, StripPlan &out) {
+    if ((p.dtype != WK_F32 && p.dtype != WK_F64) || p.ext || p.K < 512) return false;
+    if (!(p.dtype == WK_F32 ? gemm_f32_dma_applies(p, 128, 128) : gemm_f64_dma_applies(p, 128, 128))) return false;
+    const uint64_t bn = 128, big = p.dtype == WK_F32 ? 256 : 128;
+    // (1) thin strips -- at most a quarter of the tile's rows (256 or 128 of them: the large tiles) or of its 128
+    // columns: always, when the body is large enough to carry the extra launches
+    {
+        uint64_t bm = big;
+        if (bm == 256 && (p.M % 256 == 0 || p.M % 256 > 64)) bm = 128;
+        const uint64_t m_rem = p.M % bm, n_rem = p.N % bn;
+        const bool thin_m = m_rem && m_rem <= bm / 4 && p.M > bm, thin_n = n_rem && n_rem <= bn / 4 && p.N > bn;
+        const uint64_t Mb = thin_m ? p.M - m_rem : p.M, Nb = thin_n ? p.N - n_rem : p.N;
+        if ((thin_m || thin_n) && Mb * Nb >= (1ull << 22)) { // (2048 x 2047 and below: N,N gains 7 %, T,N loses as much)
+            make_parts(p, Mb, Nb, out);
+            return true;
+        }
+    }
+    // (2) any remainder beyond whole large tiles, where the cost model puts the parts, with a launch each, well
+    // below the whole (4296 x 4096 x 4096: 127 -> 142 TFLOP/s, 4096 x 4160 x 4096 123 -> 143, 8292 x 8192 x 4096
+    // 141 -> 146, 4200^3 126 -> 135; 3000^3, 2500^3, 6000^3: the whole stays cheaper, by the model and measured)
+    double whole = 0.0;
+    if (gemm_mfma_pick(p, &whole) < 0) return false;
+    // a launch more: about 4 us in the model's unit (cost x k / 3.05e5 = microseconds in f32, half that rate in f64)
+    const double launch = 4.0 * (p.dtype == WK_F32 ? 3.05e5 : 1.525e5) / (double)p.K;
+    const uint64_t m_rem = p.M > big ? p.M % big : 0, n_rem = p.N > bn ? p.N % bn : 0;
+    double best = 0.95 * whole;
+    bool found = false;
+    for (int cand = 1; cand < 4; ++cand) {
+        const bool sm = cand & 1, sn = cand & 2;
+        if ((sm && !m_rem) || (sn && !n_rem)) continue;
+        const uint64_t Mb = sm ? p.M - m_rem : p.M, Nb = sn ? p.N - n_rem : p.N;
+        if (Mb * Nb < (1ull << 21)) continue;
+        StripPlan trial;
+        make_parts(p, Mb, Nb, trial);
+        double sum = 0.0;
+        bool ok = true;
+        for (int i = 0; i < trial.parts && ok; ++i) {
+            double c = 0.0;
+            ok = gemm_mfma_pick(trial.part[i], &c) >= 0;
+            sum += c + (i ? launch : 0.0);
+        }
+        if (ok && sum < best) {
+            best = sum;
+            out = trial;
+            found = true;
+        }
+    }
+    return found;
 }
 
 int choose(const GemmProblem &p) {

@@ -29,6 +29,7 @@
 #include "wk_internal.hpp"
 
 #include <cstdlib>
+#include <algorithm>
 #include <cstring>
 
 using namespace wk;
@@ -1566,11 +1567,14 @@ bool split_pays(const GemmProblem &p, const GemmSplitPlan &plan) {
 
 namespace {
 // cost of a k-split tail in rounds of its tile: launch gap, hand-overs without a co-resident
-// work-group and the addition of the partial tiles (fixed part), plus the tile's time over the shares
-constexpr double TAIL_FIXED = 0.06, TAIL_PER_SHARE = 1.52;
+// work-group and the addition of the partial tiles (fixed part), plus the tile's time over the shares.
+// Measured with the direct-to-LDS body (time of the whole launch minus the body's rounds, in tile times): 0.34
+// at 4 shares (8292 x 8192 x 4096), 0.39 at 5 (4200^3) and at 8 (8191 x 8193 x 8190), 0.35 at 16 (4096 x 4160 x
+// 4096): from five shares on it does not shrink any further (TAIL_FLOOR).
+constexpr double TAIL_FIXED = 0.06, TAIL_PER_SHARE = 1.52, TAIL_FLOOR = 0.36;
 } // namespace
 
-int wk::gemm_mfma_pick(const GemmProblem &p) {
+int wk::gemm_mfma_pick(const GemmProblem &p, double *cost_out) {
     if (p.dtype != WK_F32 && p.dtype != WK_F64 && p.dtype != WK_I32 && p.dtype != WK_U32) return -1;
     if (p.M > 0x7fffffffull || p.N > 0x7fffffffull || p.K > 0x7fffffffull || p.lda > 0x7fffffffull ||
         p.ldb > 0x7fffffffull || p.ldc > 0x7fffffffull)
@@ -1603,7 +1607,7 @@ int wk::gemm_mfma_pick(const GemmProblem &p) {
         // measured launches)
         GemmSplitPlan tp;
         if (d.tail && !p.ext && plan_tail(p, d.bm, d.bn, d.bk, 4, d.occ, false, tp)) {
-            const double tail_rounds = TAIL_FIXED + TAIL_PER_SHARE / tp.shares;
+            const double tail_rounds = std::max(TAIL_FIXED + TAIL_PER_SHARE / tp.shares, TAIL_FLOOR);
             const double tcost = ((double)tp.first_tile / cus + d.fill + tail_rounds * tp.tiles * tp.shares / cus) * d.bm * d.bn / eff;
             if (tcost < best_cost)
                 for (int w = 0; w < k_num_variants; ++w)
@@ -1613,6 +1617,7 @@ int wk::gemm_mfma_pick(const GemmProblem &p) {
                     }
         }
     }
+    if (cost_out) *cost_out = best_cost;
     // f32 problems that are one nearly full round of 128x128 tiles: that tile with two k-groups (eight
     // wavefronts per CU) beats the four rounds of 64x64 the cost model would take -- 2048^3 126 / 132 /
     // 120 / 126 -> 130 / 136 / 126 / 131 TFLOP/s (NN / NT / TN / TT), 2048x2048x4096 128 -> 134.  With
