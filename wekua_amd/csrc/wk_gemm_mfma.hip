@@ -1249,10 +1249,11 @@ int launch_f64(hipStream_t st, const GemmProblem &p, bool edge) {
 // summing a contiguous range of k; the partial tiles meet in the stream's scratch memory and the
 // work-group that arrives last at the tile's counter adds them in the order of the shares, so the
 // result is the same bits on every run.
-//   relaxed (a forced variant, tests): split whenever k holds two slabs, up to four shares.
-//   otherwise: only when the tiles leave at least half the compute units idle, as many shares as put
+//   The plan: only when the tiles leave at least half the compute units idle, as many shares as put
 //   four (f64: two) work-groups on every unit (a power of two, at most 64), each share at least eight
-//   slabs long.
+//   slabs long.  Where that gives none, a forced variant (tests) falls back to the relaxed plan: split
+//   whenever k holds two slabs, up to four shares.  (Launches used to take the relaxed plan always:
+//   512 x 512 x 8192 52 -> 47 us, 256 x 256 x 8192 51 -> 31, 128 x 128 x 16384 94 -> 38, f64 256 x 256 x 8192 89 -> 50.)
 bool plan_split(const GemmProblem &p, int bm, int bn, int bkt, size_t elem, bool relaxed, GemmSplitPlan &plan) {
     plan = GemmSplitPlan{};
     plan.tiles = ((p.M + bm - 1) / bm) * ((p.N + bn - 1) / bn);
@@ -1283,7 +1284,9 @@ bool plan_split(const GemmProblem &p, int bm, int bn, int bkt, size_t elem, bool
 int launch_f32_split64(hipStream_t st, const GemmProblem &p, bool edge) {
     constexpr int BM = 64, BN = 64, BK = 32;
     GemmSplitPlan plan;
-    if (p.ext || !plan_split(p, BM, BN, BK, sizeof(float), true, plan)) return launch_f32<BM, BN, BK, 2, 2, 4>(st, p, edge);
+    // the plan of the automatic choice where it exists (as many shares as fill the units), else the forced variant's
+    if (p.ext || !(plan_split(p, BM, BN, BK, sizeof(float), false, plan) || plan_split(p, BM, BN, BK, sizeof(float), true, plan)))
+        return launch_f32<BM, BN, BK, 2, 2, 4>(st, p, edge);
     const int sel = (p.op_a ? 0 : 2) | (p.op_b ? 1 : 0);
 #define WK_CASE(AK, BKC)                                                                                                \
     return edge ? launch_f32_one<BM, BN, BK, 2, 2, 4, AK, BKC, true, false, 1, -1, true>(st, p, &plan)                    \
@@ -1300,7 +1303,8 @@ int launch_f32_split64(hipStream_t st, const GemmProblem &p, bool edge) {
 int launch_f64_split64(hipStream_t st, const GemmProblem &p, bool edge) {
     constexpr int BM = 64, BN = 64, BK = 32;
     GemmSplitPlan plan;
-    if (p.ext || !plan_split(p, BM, BN, BK, sizeof(double), true, plan)) return launch_f64<BM, BN, BK, 2, 2, 2>(st, p, edge);
+    if (p.ext || !(plan_split(p, BM, BN, BK, sizeof(double), false, plan) || plan_split(p, BM, BN, BK, sizeof(double), true, plan)))
+        return launch_f64<BM, BN, BK, 2, 2, 2>(st, p, edge);
     const int sel = (p.op_a ? 0 : 2) | (p.op_b ? 1 : 0);
 #define WK_CASE(AK, BKC)                                                                                                \
     return edge ? launch_f64_one<BM, BN, BK, 2, 2, 2, AK, BKC, true, false, 1, true>(st, p, &plan)                        \
@@ -1545,7 +1549,7 @@ bool wk::gemm_mfma_split_plan(const GemmProblem &p, int variant, bool forced, Ge
     const VariantDesc &v = k_variants[variant];
     const size_t elem = v.dtype == WK_F64 ? 8 : 4;
     switch (split_kind_of(v.name)) {
-    case SPLIT_ALL: return plan_split(p, v.bm, v.bn, v.bk, elem, forced, plan);
+    case SPLIT_ALL: return plan_split(p, v.bm, v.bn, v.bk, elem, false, plan) || (forced && plan_split(p, v.bm, v.bn, v.bk, elem, true, plan));
     case SPLIT_TAIL: return plan_tail(p, v.bm, v.bn, v.bk, elem, v.occ, forced && g_tail_relaxed, plan);
     default: return false;
     }
