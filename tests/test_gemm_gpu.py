@@ -486,6 +486,34 @@ def test_thin_strips_beyond_whole_tiles_are_products_of_their_own(dev, dtype, M,
     check(dev, dtype, M, N, K, 0, 1, None, None, seed=505, lda=up(K), ldb=up(K))
 
 
+@pytest.mark.parametrize("dtype", ["f32", "f64"])
+@pytest.mark.parametrize("op_a,op_b", OPS)
+def test_thin_products(dev, dtype, op_a, op_b):
+    """At most four rows or four columns of C (matrix-vector products in all but name): the kernels that read
+    the long operand once along its storage order, one to four rows / columns, k below, at and beyond the
+    1024 values of the thin operand that LDS holds at a time, every epilogue, rows of 16-byte multiples and
+    not (the vector and the scalar loads), gaps between the rows of C whose poison must survive; against the
+    oracle.  The name query says which products take them."""
+    from wekua_amd import raw
+    per = 4 if dtype == "f32" else 2
+    up = lambda n: -(-n // per) * per
+    did = raw.dtype_id(dtype)
+
+    def name(M, N, K):
+        return dev.lib.wk_gemm_variant(did, op_a, op_b, M, N, K, M if op_a else K, K if op_b else N, N, None, None, None)
+    assert name(1, 4095, 4093) == b"thin" and name(4096, 1, 4093) == b"thin" and name(4, 512, 128) == b"thin"
+    assert name(5, 4095, 4093) != b"thin" and name(1, 500, 4093) != b"thin" and name(2, 3, 4093) != b"thin" and name(1, 4095, 100) != b"thin"
+    options = [(None, None), (2.0, None), (1.5, 0.5), (None, -0.25)]
+    n = 0
+    for (M, N, K) in [(1, 4095, 4093), (4096, 1, 4093), (3, 1000, 700), (700, 4, 1024), (2, 513, 129), (1031, 2, 2050),
+                      (4, 2048, 1025), (600, 3, 128)]:
+        alpha, beta = options[n % 4]
+        cols_a, cols_b = (M if op_a else K), (K if op_b else N)
+        check(dev, dtype, M, N, K, op_a, op_b, alpha, beta, seed=600 + n)                                   # dense rows
+        check(dev, dtype, M, N, K, op_a, op_b, alpha, beta, seed=620 + n, lda=up(cols_a) + per, ldb=up(cols_b), ldc=N + 3)
+        n += 1
+
+
 def test_left_over_tiles_run_as_a_k_split_tail(dev):
     """A launch whose tiles do not fill whole rounds of the compute units: the whole rounds run as they
     are, the left-over tiles as a second launch with k split over work-groups.  Checked: the plan of the

@@ -244,11 +244,17 @@ static int gemm_entry(wk_stream *s, int dtype, int op_a, int op_b, uint64_t M, u
         }
     }
     if (g_forced.load(std::memory_order_relaxed) == -2) {
+        if (gemm_thin_applies(p)) return gemm_thin_launch(s->stream, p);
         StripPlan sp;
         if (plan_strips(p, sp)) {
             for (int i = 0; i < sp.parts; ++i) {
-                const int pv = gemm_mfma_pick(sp.part[i]);
-                rc = pv >= 0 ? gemm_mfma_launch(s->stream, sp.part[i], pv) : gemm_generic_launch(s->stream, sp.part[i]);
+                const GemmProblem &q = sp.part[i];
+                if (gemm_thin_applies(q)) {
+                    rc = gemm_thin_launch(s->stream, q);
+                } else {
+                    const int pv = gemm_mfma_pick(q);
+                    rc = pv >= 0 ? gemm_mfma_launch(s->stream, q, pv) : gemm_generic_launch(s->stream, q);
+                }
                 if (rc) return rc;
             }
             return WK_OK;
@@ -316,6 +322,7 @@ const char *wk_gemm_variant(int dtype, int op_a, int op_b, uint64_t M, uint64_t 
     p.counters = &dummy_counter;
     p.num_counters = WK_GEMM_COUNTERS;
     if (g_forced.load(std::memory_order_relaxed) == -2) {
+        if (gemm_thin_applies(p)) return "thin";
         StripPlan sp;
         if (plan_strips(p, sp)) { // the body's kernel, marked: the strips beyond it are launches of their own
             const int bv = gemm_mfma_pick(sp.part[0]);

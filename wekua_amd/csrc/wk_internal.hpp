@@ -227,6 +227,9 @@ int gemm_f32_dma_launch(hipStream_t st, const GemmProblem &p, int bm, int bn, ui
 bool gemm_f64_dma_applies(const GemmProblem &p, int bm, int bn);
 int gemm_f64_dma_launch(hipStream_t st, const GemmProblem &p, int bm, int bn);
 bool gemm_mfma_fuses(const GemmProblem &p, int variant); // variant can run p with the fused bias + activation epilogue
+// f32 / f64 products with at most four rows or columns of C (wk_gemm_thin.hip)
+bool gemm_thin_applies(const GemmProblem &p);
+int gemm_thin_launch(hipStream_t st, const GemmProblem &p);
 int gemm_mfma_pick(const GemmProblem &p, double *cost = nullptr); // -1: not applicable; cost: the model's figure for
                                                               // the chosen tile (rounds x tile area / efficiency; times k
                                                               // proportional to the launch's time: 3.05e5 per us in f32)
