@@ -189,7 +189,7 @@ int    wk_gemm_packed_b_kept(wk_stream *s, int dtype, int op_a, int op_b, uint64
                              const void *host_beta, void *C, uint64_t ldc, void *workspace, size_t workspace_bytes);
 
 /* Name of the kernel variant wk_gemm() would launch for these arguments ("mfma_f32_256x128",
- * "tile64", ...).  A name that ends in "+strips" is the kernel of the body of whole tiles of a product
+ * "tile64", "thin" for a product of at most four rows or columns, ...).  A name that ends in "+strips" is the kernel of the body of whole tiles of a product
  * that wk_gemm launches in parts: the rows or columns beyond the body follow as products of their own.
  * For benchmarks and profiles; not part of the reference's surface. */
 const char *wk_gemm_variant(int dtype, int op_a, int op_b, uint64_t M, uint64_t N, uint64_t K,
