@@ -939,7 +939,8 @@ int wk::gemm_f64_dma_launch(hipStream_t st, const GemmProblem &p, int bm, int bn
     if (!gemm_f64_dma_applies(p, bm, bn)) return WK_E_INVALID_VALUE;
     if (bm == 128) return launch_tile_d<128, 128, 16, 2, 2>(st, p);
     // (64 x 64 with k-slabs of 32 in two stages, two work-groups per unit, measured the same within the run-to-run
-    // spread: 8192 x 256 x 8192 67.4-68.6 against 68.0-68.2 TFLOP/s, 2048^3 68-69 against 66-68, 3072^3 70-71 both)
+    // spread: 8192 x 256 x 8192 67.4-68.6 against 68.0-68.2 TFLOP/s, 2048^3 68-69 against 66-68, 3072^3 70-71 both;
+    // two stages of 16 with three or four per unit: 8192 x 256 x 8192 65.6 against 68.7, 1024^3 45 against 53-56)
     return launch_tile_d<64, 64, 16, 3, 3>(st, p);
 }
 
