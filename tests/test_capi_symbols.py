@@ -104,6 +104,35 @@ def _split_args(arglist):
     return out
 
 
+def test_thin_products_and_strips_by_name():
+    """Host arithmetic of the launch plan, through the name query (256 compute units and 16-byte aligned
+    operands assumed): which f32 / f64 products run as thin products, which are launched as a body of whole
+    tiles plus strips, and which stay whole."""
+    from wekua_amd import _capi
+    lib = _capi.load()
+
+    def name(dtype, M, N, K, op_a=0, op_b=0, lda=None, ldb=None):
+        lda = lda or (M if op_a else K)
+        ldb = ldb or (K if op_b else N)
+        return lib.wk_gemm_variant(dtype, op_a, op_b, M, N, K, lda, ldb, N, None, None, None).decode()
+    for dt in (8, 9):
+        per = 4 if dt == 8 else 2
+        for op_a, op_b in ((0, 0), (0, 1), (1, 0), (1, 1)):
+            # at most four rows or four columns, the other dimension and k long enough
+            assert name(dt, 1, 4096, 4096, op_a, op_b) == "thin" and name(dt, 4096, 4, 512, op_a, op_b) == "thin"
+            assert name(dt, 5, 4096, 4096, op_a, op_b) != "thin" and name(dt, 1, 256, 4096, op_a, op_b) != "thin"
+            assert name(dt, 4, 4, 4096, op_a, op_b) != "thin" and name(dt, 1, 4096, 64, op_a, op_b) != "thin"
+            # a row or a column beyond whole tiles, aligned rows: body + strips; unaligned rows: one launch
+            lda, ldb = (4100 if op_a else 4096), (4096 if op_b else 4100)
+            assert name(dt, 4097, 4097, 4096, op_a, op_b, lda, ldb).endswith("+strips")
+            assert not name(dt, 4097, 4097, 4095, op_a, op_b, 4097 if op_a else 4095, 4095 if op_b else 4097).endswith("+strips")
+            assert not name(dt, 4096, 4096, 4096, op_a, op_b).endswith("+strips")              # nothing beyond
+            assert not name(dt, 4097, 4096, 256, op_a, op_b, lda, 4096).endswith("+strips")     # short k
+            assert not name(dt, 1025, 1024, 4096, op_a, op_b, 1028 if op_a else 4096, 4096 if op_b else 1024).endswith("+strips")  # small body
+    assert name(4, 4097, 4097, 4096) in ("mfma_i32_128x128", "mfma_i32_64x128")            # integers: never in parts
+    assert name(8, 4200, 4096, 1024).endswith("+strips") and not name(8, 3000, 3000, 1024, lda=3000, ldb=3000).endswith("+strips")
+
+
 def test_zig_binding_in_the_integration_guide_matches_the_header():
     """The `extern fn` block a wekua maintainer would paste declares exactly the functions of the
     header, each with the header's number of parameters."""
