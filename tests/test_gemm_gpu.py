@@ -600,6 +600,9 @@ def test_narrow_integers_packed_large_tile(dev, dtype):
         if dtype == "u8":   # and from one 256 x 256 tile per compute unit up the 8-bit types run that one
             check(dev, dtype, 4096, 4096, 128, 0, 1, None, 5, seed=67, packed=True)
             check(dev, dtype, 4096 + 77, 4096 + 5, 96, 1, 0, 3, 7, seed=68, packed=True)
+            # (its pipeline runs stages of 64 k, a multiple of four of them: four, eight and twelve here)
+            check(dev, dtype, 4096, 4096, 300, 0, 0, 3, None, seed=69, packed=True)
+            check(dev, dtype, 4096 + 1, 4096 + 255, 520, 1, 1, None, None, seed=70, packed=True)
     finally:
         dev.lib.wk_gemm_force_variant(b"auto")
 

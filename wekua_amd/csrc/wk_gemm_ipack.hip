@@ -59,8 +59,8 @@ Layout make_layout(int digits, uint64_t M, uint64_t N, uint64_t K) {
     w.Mp = (M + m_tile - 1) / m_tile * m_tile;
     const uint64_t n_tile = digits == 1 ? 256 : TILE; // 8-bit: also the 256-column tile
     w.Np = (N + n_tile - 1) / n_tile * n_tile;
-    // (32-bit types: an even number of slabs, for the two-slab loop of the direct-to-LDS kernel)
-    const uint64_t kb_round = digits == 4 ? 2 : per_slab;
+    // (8- and 32-bit types: an even number of slabs, for the two-stage loop of the direct-to-LDS kernels)
+    const uint64_t kb_round = digits == 2 ? per_slab : 2 * per_slab;
     w.KB = ((K + BK - 1) / BK + kb_round - 1) / kb_round * kb_round;
     w.slabs = w.KB / per_slab;
     // enough work-groups in the pack launch to fill the chip: (Mp + Np) / 32 row blocks x ksplit
@@ -219,7 +219,6 @@ __global__ __launch_bounds__(BM / (32 * WMF) * 128) __attribute__((amdgpu_waves_
 void gemm_int_packed_kernel(PArgs g) {
     using TL = PackedTile<BM, WMF, BN>;
     constexpr int WNF = BN / 64;        // 32-column blocks of B per wavefront
-    constexpr bool ONE_SET = BN > TILE; // the 256 x 256 tile has registers for one staging set only
     static_assert(TL::GROUPS % TL::GROUPS_PER_PASS == 0, "tile shape");
     constexpr int D = Digits<E>::D, KB_PER_SLAB = Digits<E>::KB_PER_SLAB;
     constexpr int STAGE_BYTES = TL::STAGE_BYTES, PASSES = TL::PASSES, A_GROUPS = BM / 32;
@@ -266,7 +265,7 @@ void gemm_int_packed_kernel(PArgs g) {
     // used in step kb + 2, so a load has two slabs of matrix work to arrive.
     // (past the end the last slab is loaded again and dropped: no branch, so the loads stay where
     // they are written, ahead of the matrix work)
-    u32x4 staged[ONE_SET ? 1 : 2][PASSES];
+    u32x4 staged[2][PASSES];
     auto gload = [&](u32x4 *dst, uint32_t kb) {
         const int off = (int)(min(kb, g.slabs - 1) * GROUP_BYTES);
 #pragma unroll
@@ -281,24 +280,6 @@ void gemm_int_packed_kernel(PArgs g) {
     auto compute = [&](int buf) {
         const unsigned char *sa = stages + buf * STAGE_BYTES + wm * WMF * GROUP_BYTES + lane * 16;
         const unsigned char *sb = stages + buf * STAGE_BYTES + (A_GROUPS + wn * WNF) * GROUP_BYTES + lane * 16;
-        if constexpr (D == 1 && WNF > 2) {
-            // one digit, large tile: a k-block needs only its own fragments, so they are fetched per
-            // k-block instead of all sixteen of the slab at once (which would not fit the registers)
-#pragma unroll
-            for (int kbl = 0; kbl < KB_PER_SLAB; ++kbl) {
-                i32x4 a[WMF], b[WNF];
-#pragma unroll
-                for (int am = 0; am < WMF; ++am) a[am] = *reinterpret_cast<const i32x4 *>(sa + am * GROUP_BYTES + kbl * BLOCK_BYTES);
-#pragma unroll
-                for (int blk = 0; blk < WNF; ++blk) b[blk] = *reinterpret_cast<const i32x4 *>(sb + blk * GROUP_BYTES + kbl * BLOCK_BYTES);
-#pragma unroll
-                for (int am = 0; am < WMF; ++am)
-#pragma unroll
-                    for (int blk = 0; blk < WNF; ++blk)
-                        acc[0][am][blk] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a[am], b[blk], acc[0][am][blk], 0, 0, 0);
-            }
-            return;
-        }
         // the four blocks of a group: k-block f / D of the slab, digit f % D
         i32x4 a[WMF][4], b[WNF][4];
 #pragma unroll
@@ -324,31 +305,17 @@ void gemm_int_packed_kernel(PArgs g) {
     // one step: slab kb is in LDS stage `cur`, slab kb + 1 in flight in staged[other]
     auto step = [&](uint32_t kb, auto cur_tag) {
         constexpr int cur = decltype(cur_tag)::value;
-        if constexpr (ONE_SET) {
-            // one set: slab kb + 1, requested a step ago, goes to the free stage first and slab kb + 2
-            // is requested into the same registers (measured equal to the two-set order on the other tiles)
-            if (kb + 1 < g.slabs) sstore(staged[0], cur ^ 1);
-            gload(staged[0], kb + 2);
-            compute(cur);
-            if (kb + 1 < g.slabs) __syncthreads();
-        } else {
-            gload(staged[cur], kb + 2);
-            compute(cur);
-            if (kb + 1 < g.slabs) {
-                sstore(staged[cur ^ 1], cur ^ 1);
-                __syncthreads();
-            }
+        gload(staged[cur], kb + 2);
+        compute(cur);
+        if (kb + 1 < g.slabs) {
+            sstore(staged[cur ^ 1], cur ^ 1);
+            __syncthreads();
         }
     };
 
     gload(staged[0], 0);
-    if constexpr (ONE_SET) {
-        sstore(staged[0], 0);
-        gload(staged[0], 1);
-    } else {
-        gload(staged[1], 1);
-        sstore(staged[0], 0);
-    }
+    gload(staged[1], 1);
+    sstore(staged[0], 0);
     __syncthreads();
     for (uint32_t kb = 0; kb < g.slabs; kb += 2) {
         step(kb, std::integral_constant<int, 0>{});
@@ -634,6 +601,207 @@ template <bool EDGE, int NS> int launch_packed_dma(hipStream_t st, PArgs g) {
     return launch_status();
 }
 
+// ---- 8-bit product kernel with the slabs brought straight into LDS -------------------------------
+// One digit per element: the 256 x 256 tile (256 operations per byte fetched) with four wavefronts of 128 x 128
+// (one per SIMD: 4 x 4 blocks = 256 accumulator registers, twelve blocks pinned to accumulation registers and
+// four to vector registers as in the 32-bit kernel).  The unit of the pipeline is half a slab, two k-blocks
+// of 32: eight row groups of A and eight column groups of B at 2 KiB each = 32 KiB per stage, four stages;
+// a wavefront requests eight KiB of it, multiplies 2 x 16 blocks and reads sixteen fragments per stage.
+struct ByteDmaTile {
+    static constexpr int BM = 256, BN = 256, GROUPS = 16, HALF = GROUP_BYTES / 2, STAGE_BYTES = GROUPS * HALF;
+    static constexpr size_t lds_bytes(int ns) { return (size_t)ns * STAGE_BYTES; }
+};
+
+template <bool EDGE, int NS>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1)))
+void gemm_i8_packed_dma_kernel(PArgs g) {
+    using namespace wk::lds_dma;
+    using TL = ByteDmaTile;
+    constexpr int BM = TL::BM, BN = TL::BN, STAGE_BYTES = TL::STAGE_BYTES, HALF = TL::HALF;
+    static_assert(NS == 4, "the drain below is written out for four stages");
+    extern __shared__ __align__(16) unsigned char lds_raw[];
+
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wm = wave >> 1, wn = wave & 1, l32 = lane & 31, lhi = lane >> 5;
+    uint32_t tile_m, tile_n;
+    if (g.patch_m) { // XCD-local patches: work-group b runs on XCD b % 8 (see wk_gemm_dma.hip)
+        const uint32_t pid = blockIdx.x, x = pid & 7u, j = pid >> 3;
+        const uint32_t per_patch = g.patch_m * g.patch_n, patch = (j / per_patch) * 8u + x, q = j % per_patch;
+        const uint32_t patches_n = g.tiles_n / g.patch_n;
+        tile_m = (patch / patches_n) * g.patch_m + q % g.patch_m;
+        tile_n = (patch % patches_n) * g.patch_n + q / g.patch_m;
+    } else {
+        const uint32_t pid = blockIdx.x, group_size = 8 * g.tiles_n, group = pid / group_size, first_m = group * 8;
+        const uint32_t gsz = min(g.tiles_m - first_m, 8u), in_group = pid - group * group_size;
+        tile_m = first_m + in_group % gsz;
+        tile_n = in_group / gsz;
+    }
+    const uint32_t m0 = tile_m * BM, n0 = tile_n * BN;
+
+    // wavefront w brings groups 4 w .. 4 w + 3 of every stage: A's row groups 0..7, then B's column groups
+    const unsigned char *src_g[4];
+#pragma unroll
+    for (int h = 0; h < 4; ++h) {
+        const int gi = 4 * wave + h;
+        src_g[h] = gi < 8 ? g.planes_a + (size_t)(tile_m * 8 + gi) * g.slabs * GROUP_BYTES
+                          : g.planes_b + (size_t)(tile_n * 8 + gi - 8) * g.slabs * GROUP_BYTES;
+    }
+    uint32_t voff[2];
+#pragma unroll
+    for (int d = 0; d < 2; ++d) voff[d] = lane * 16 + d * BLOCK_BYTES;
+    const uint32_t lds0 = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)(__attribute__((address_space(3))) unsigned char *)lds_raw);
+    auto issue = [&](uint32_t stage_bytes) {
+#pragma unroll
+        for (int h = 0; h < 4; ++h) {
+#pragma unroll
+            for (int d = 0; d < 2; ++d)
+                dma16(src_g[h], voff[d], lds0 + stage_bytes + (uint32_t)(4 * wave + h) * HALF + d * BLOCK_BYTES);
+            src_g[h] += HALF;
+        }
+    };
+    constexpr int LOADS = 8;
+
+    i32x16 acc[4][4]; // [row block][column block]
+#pragma unroll
+    for (int am = 0; am < 4; ++am)
+#pragma unroll
+        for (int b = 0; b < 4; ++b)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[am][b][r] = 0;
+
+    i32x4 fa[2][4][2], fb[2][4][2]; // [set][block][k-block of the stage]
+    const uint32_t frag_a = lds0 + lane * 16 + (wm * 4) * HALF, frag_b = lds0 + lane * 16 + (8 + wn * 4) * HALF;
+    // fragment number f of a stage: 0..7 A (block f / 2, k-block f % 2), 8..15 B
+    auto read_frag = [&](uint32_t stage_bytes, auto set_tag, auto f_tag) __attribute__((always_inline)) {
+        constexpr int SET = decltype(set_tag)::value, F = decltype(f_tag)::value;
+        constexpr int BLK = (F & 7) / 2, Q = F & 1, IMM = BLK * HALF + Q * BLOCK_BYTES;
+        i32x4 &dst = F < 8 ? fa[SET][BLK][Q] : fb[SET][BLK][Q];
+        const uint32_t addr = (F < 8 ? frag_a : frag_b) + stage_bytes;
+        asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(dst) : "v"(addr), "n"(IMM));
+    };
+    // matrix instruction number n of a stage (0..31): k-block n / 16, row block (n / 4) % 4, column block n % 4;
+    // two on one accumulator are sixteen instructions apart
+    auto mfma_n = [&](auto set_tag, auto n_tag) __attribute__((always_inline)) {
+        constexpr int SET = decltype(set_tag)::value, N = decltype(n_tag)::value;
+        constexpr int Q = N / 16, AM = (N / 4) & 3, B = N & 3;
+        i32x16 &c = acc[AM][B];
+        const i32x4 &a = fa[SET][AM][Q], &b = fb[SET][B][Q];
+        if constexpr (AM == 3) asm volatile("v_mfma_i32_32x32x32_i8 %0, %1, %2, %0" : "+v"(c) : "v"(a), "v"(b));
+        else asm volatile("v_mfma_i32_32x32x32_i8 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
+    };
+    auto issue_one = [&](uint32_t stage_bytes, auto r_tag) __attribute__((always_inline)) {
+        constexpr int R = decltype(r_tag)::value, H = R / 2, Q = R & 1;
+        dma16(src_g[H], voff[Q], lds0 + stage_bytes + (uint32_t)(4 * wave + H) * HALF + Q * BLOCK_BYTES);
+        if constexpr (Q == 1) src_g[H] += HALF;
+    };
+
+    const uint32_t ktiles = g.slabs * 2; // stages of two k-blocks; a multiple of four (the pack pass pads the planes)
+    uint32_t st[NS];
+#pragma unroll
+    for (int n = 0; n < NS; ++n) st[n] = n * STAGE_BYTES;
+
+    using std::integral_constant;
+#pragma unroll
+    for (int n = 0; n < NS - 1; ++n)
+        if ((uint32_t)n < ktiles) issue(st[n]);
+    wait_vm_slabs<LOADS, NS - 2>(ktiles - 1);
+    __builtin_amdgcn_s_barrier();
+    static_for<16>([&](auto f_tag) { read_frag(st[0], integral_constant<int, 0>{}, f_tag); });
+
+    auto iteration = [&](auto parity_tag, auto issue_tag, auto ahead_tag) __attribute__((always_inline)) {
+        constexpr int P = decltype(parity_tag)::value;
+        constexpr bool ISSUE = decltype(issue_tag)::value;
+        constexpr int AHEAD = decltype(ahead_tag)::value;
+        wait_lgkm0(); // the fragments of this stage
+        static_for<16>([&](auto n_tag) {
+            constexpr int N = decltype(n_tag)::value;
+            mfma_n(integral_constant<int, P>{}, n_tag);
+            if constexpr (ISSUE && N % 2 == 0) issue_one(st[NS - 1], integral_constant<int, N / 2>{});
+        });
+        if constexpr (AHEAD >= 0) {
+            wait_vm<AHEAD * LOADS>();
+            __builtin_amdgcn_s_barrier();
+        }
+        static_for<16>([&](auto n_tag) {
+            mfma_n(integral_constant<int, P>{}, integral_constant<int, 16 + decltype(n_tag)::value>{});
+            if constexpr (AHEAD >= 0) read_frag(st[1], integral_constant<int, P ^ 1>{}, n_tag);
+        });
+        const uint32_t t = st[0];
+#pragma unroll
+        for (int n = 0; n + 1 < NS; ++n) st[n] = st[n + 1];
+        st[NS - 1] = t;
+    };
+    using T_ = std::true_type;
+    using F_ = std::false_type;
+    using P0 = integral_constant<int, 0>;
+    using P1 = integral_constant<int, 1>;
+    using STEADY = integral_constant<int, NS - 2>;
+    uint32_t kt = 0;
+    for (; kt + NS < ktiles; kt += 2) { // the fragment sets swap with the stages: two per trip
+        iteration(P0{}, T_{}, STEADY{});
+        iteration(P1{}, T_{}, STEADY{});
+    }
+    if (kt + 4 == ktiles) { // four left: the last stage is still to be requested
+        iteration(P0{}, T_{}, integral_constant<int, 2>{});
+        iteration(P1{}, F_{}, integral_constant<int, 1>{});
+    }
+    iteration(P0{}, F_{}, integral_constant<int, 0>{}); // two left
+    iteration(P1{}, F_{}, integral_constant<int, -1>{});
+
+    asm volatile("s_nop 15\n\ts_nop 15\n\ts_nop 15" ::: "memory"); // the last matrix instructions' results
+
+    // epilogue as in the kernels above, modulo 2^8 (the store keeps the low byte)
+    unsigned char *C = static_cast<unsigned char *>(g.C);
+#pragma unroll
+    for (int am = 0; am < 4; ++am) {
+        uint32_t old[4][16];
+        if (g.epi == EPI_ALPHA_BETA) {
+#pragma unroll
+            for (int blk = 0; blk < 4; ++blk) {
+                const uint32_t col = n0 + wn * 128 + blk * 32 + l32, colc = EDGE ? min(col, g.N - 1) : col;
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    const uint32_t row = m0 + (wm * 4 + am) * 32 + 8 * (r / 4) + 4 * lhi + (r % 4);
+                    old[blk][r] = C[(size_t)(EDGE ? min(row, g.M - 1) : row) * g.ldc + colc];
+                }
+            }
+        }
+#pragma unroll
+        for (int blk = 0; blk < 4; ++blk) {
+            const uint32_t col = n0 + wn * 128 + blk * 32 + l32;
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const uint32_t row = m0 + (wm * 4 + am) * 32 + 8 * (r / 4) + 4 * lhi + (r % 4);
+                uint32_t v = (uint32_t)acc[am][blk][r];
+                if (g.epi == EPI_ALPHA) v = g.alpha * v;
+                else if (g.epi == EPI_ALPHA_BETA) v = g.alpha * v + g.beta * old[blk][r];
+                if (!EDGE || ((row < g.M) & (col < g.N))) C[(size_t)row * g.ldc + col] = (unsigned char)v;
+            }
+        }
+    }
+}
+
+template <bool EDGE, int NS> int launch_i8_dma(hipStream_t st, PArgs g) {
+    constexpr size_t lds = ByteDmaTile::lds_bytes(NS);
+    auto kern = gemm_i8_packed_dma_kernel<EDGE, NS>;
+    static const hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
+                                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    if (attr != hipSuccess) { (void)hipGetLastError(); return hip_code(attr); }
+    g.tiles_m = (g.M + ByteDmaTile::BM - 1) / ByteDmaTile::BM;
+    g.tiles_n = (g.N + ByteDmaTile::BN - 1) / ByteDmaTile::BN;
+    g.patch_m = g.patch_n = 0;
+    static const unsigned shapes[][2] = {{4, 8}, {4, 4}, {2, 8}, {2, 4}};
+    for (const auto &sh : shapes)
+        if (g.tiles_m % sh[0] == 0 && g.tiles_n % sh[1] == 0 && ((g.tiles_m / sh[0]) * (g.tiles_n / sh[1])) % 8 == 0) {
+            g.patch_m = sh[0];
+            g.patch_n = sh[1];
+            break;
+        }
+    hipLaunchKernelGGL(kern, dim3(g.tiles_m * g.tiles_n), dim3(256), lds, st, g);
+    return launch_status();
+}
+
 int digits_of(int dtype) {
     switch (dtype) {
     case WK_I8: case WK_U8: return 1;
@@ -687,12 +855,14 @@ template <typename E> int launch_typed(hipStream_t st, const GemmProblem &p, uns
         // These products move one byte per 170 operations even so and are bound by what the L2 delivers.
         const uint64_t tiles256 = ((p.M + 255) / 256) * ((p.N + TILE - 1) / TILE);
         if constexpr (D == 1) {
-            // one digit: from one 256 x 256 tile per CU up that tile (64 x 128 per wavefront, 256 operations
-            // per byte fetched): i8 4096^3 1461 -> 1737 TOP/s, 8192^3 1736 -> 2034, 16384^3 1795 -> 2118
+            // one digit: from one 256 x 256 tile per CU up that tile, slabs straight into LDS (256 operations per
+            // byte fetched).  Against the 256 x 128 tile of the eight-wavefront kernel: i8 4096^3 1461 -> 1631-1814
+            // TOP/s by the layout, 8192^3 1736 -> 2170-2260, 16384^3 1795 -> 2470-2490 (the eight-wavefront kernel
+            // on the same 256 x 256 tile, which this one replaced: 1572-1743, 1911-2002, 2083-2106)
             const uint64_t tiles256x256 = ((p.M + 255) / 256) * ((p.N + 255) / 256);
             if (tiles256x256 >= (p.num_cus ? p.num_cus : 256u)) {
                 const bool edge = p.M % 256 != 0 || p.N % 256 != 0;
-                return edge ? launch_packed<E, 256, true, 2, 256>(st, g) : launch_packed<E, 256, false, 2, 256>(st, g);
+                return edge ? launch_i8_dma<true, 4>(st, g) : launch_i8_dma<false, 4>(st, g);
             }
         }
         if (tiles256 >= (p.num_cus ? p.num_cus : 256u)) {
