@@ -597,6 +597,9 @@ def test_narrow_integers_packed_large_tile(dev, dtype):
     try:
         check(dev, dtype, 4096, 2048, 128, 0, 1, None, None, seed=65, packed=True)
         check(dev, dtype, 4096 + 77, 2048 + 5, 96, 1, 0, 3, 7, seed=66, packed=True)
+        if dtype == "i16":  # (its pipeline runs stages of 32 k, a multiple of four of them: twelve and twenty here)
+            check(dev, dtype, 4096, 2048, 300, 0, 0, 3, None, seed=71, packed=True)
+            check(dev, dtype, 4096 + 1, 2048 + 127, 520, 1, 1, None, -2, seed=72, packed=True)
         if dtype == "u8":   # and from one 256 x 256 tile per compute unit up the 8-bit types run that one
             check(dev, dtype, 4096, 4096, 128, 0, 1, None, 5, seed=67, packed=True)
             check(dev, dtype, 4096 + 77, 4096 + 5, 96, 1, 0, 3, 7, seed=68, packed=True)

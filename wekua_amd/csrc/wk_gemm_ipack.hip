@@ -59,8 +59,8 @@ Layout make_layout(int digits, uint64_t M, uint64_t N, uint64_t K) {
     w.Mp = (M + m_tile - 1) / m_tile * m_tile;
     const uint64_t n_tile = digits == 1 ? 256 : TILE; // 8-bit: also the 256-column tile
     w.Np = (N + n_tile - 1) / n_tile * n_tile;
-    // (8- and 32-bit types: an even number of slabs, for the two-stage loop of the direct-to-LDS kernels)
-    const uint64_t kb_round = digits == 2 ? per_slab : 2 * per_slab;
+    // (an even number of slabs, for the two-stage loop of the direct-to-LDS kernels)
+    const uint64_t kb_round = 2 * per_slab;
     w.KB = ((K + BK - 1) / BK + kb_round - 1) / kb_round * kb_round;
     w.slabs = w.KB / per_slab;
     // enough work-groups in the pack launch to fill the chip: (Mp + Np) / 32 row blocks x ksplit
@@ -803,6 +803,210 @@ template <bool EDGE, int NS> int launch_i8_dma(hipStream_t st, PArgs g) {
     return launch_status();
 }
 
+// ---- 16-bit product kernel with the slabs brought straight into LDS ------------------------------
+// Two digits per element: the 256 x 128 tile with four wavefronts of 128 x 64 (one per SIMD: 4 x 2 blocks x two
+// shift sets = 256 accumulator registers, pinned as above).  The unit of the pipeline is one k-block of 32 with
+// its two digit blocks: eight row groups of A and four column groups of B at 2 KiB = 24 KiB per stage, four
+// stages; per stage a wavefront requests six KiB, runs the three digit products (0,0), (0,1), (1,0) on its
+// eight blocks and reads twelve fragments.
+struct WordDmaTile {
+    static constexpr int BM = 256, BN = TILE, GROUPS = 12, HALF = GROUP_BYTES / 2, STAGE_BYTES = GROUPS * HALF;
+    static constexpr size_t lds_bytes(int ns) { return (size_t)ns * STAGE_BYTES; }
+};
+
+template <bool EDGE, int NS>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1)))
+void gemm_i16_packed_dma_kernel(PArgs g) {
+    using namespace wk::lds_dma;
+    using TL = WordDmaTile;
+    constexpr int BM = TL::BM, BN = TL::BN, STAGE_BYTES = TL::STAGE_BYTES, HALF = TL::HALF;
+    static_assert(NS == 4, "the drain below is written out for four stages");
+    extern __shared__ __align__(16) unsigned char lds_raw[];
+
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wm = wave >> 1, wn = wave & 1, l32 = lane & 31, lhi = lane >> 5;
+    uint32_t tile_m, tile_n;
+    if (g.patch_m) { // XCD-local patches: work-group b runs on XCD b % 8 (see wk_gemm_dma.hip)
+        const uint32_t pid = blockIdx.x, x = pid & 7u, j = pid >> 3;
+        const uint32_t per_patch = g.patch_m * g.patch_n, patch = (j / per_patch) * 8u + x, q = j % per_patch;
+        const uint32_t patches_n = g.tiles_n / g.patch_n;
+        tile_m = (patch / patches_n) * g.patch_m + q % g.patch_m;
+        tile_n = (patch % patches_n) * g.patch_n + q / g.patch_m;
+    } else {
+        const uint32_t pid = blockIdx.x, group_size = 8 * g.tiles_n, group = pid / group_size, first_m = group * 8;
+        const uint32_t gsz = min(g.tiles_m - first_m, 8u), in_group = pid - group * group_size;
+        tile_m = first_m + in_group % gsz;
+        tile_n = in_group / gsz;
+    }
+    const uint32_t m0 = tile_m * BM, n0 = tile_n * BN;
+
+    // wavefront w brings groups 3 w .. 3 w + 2 of every stage: A's row groups 0..7, then B's column groups
+    const unsigned char *src_g[3];
+#pragma unroll
+    for (int h = 0; h < 3; ++h) {
+        const int gi = 3 * wave + h;
+        src_g[h] = gi < 8 ? g.planes_a + (size_t)(tile_m * 8 + gi) * g.slabs * GROUP_BYTES
+                          : g.planes_b + (size_t)(tile_n * 4 + gi - 8) * g.slabs * GROUP_BYTES;
+    }
+    uint32_t voff[2];
+#pragma unroll
+    for (int d = 0; d < 2; ++d) voff[d] = lane * 16 + d * BLOCK_BYTES;
+    const uint32_t lds0 = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)(__attribute__((address_space(3))) unsigned char *)lds_raw);
+    auto issue = [&](uint32_t stage_bytes) {
+#pragma unroll
+        for (int h = 0; h < 3; ++h) {
+#pragma unroll
+            for (int d = 0; d < 2; ++d)
+                dma16(src_g[h], voff[d], lds0 + stage_bytes + (uint32_t)(3 * wave + h) * HALF + d * BLOCK_BYTES);
+            src_g[h] += HALF;
+        }
+    };
+    constexpr int LOADS = 6;
+
+    i32x16 acc[2][4][2]; // [shift i + j][row block][column block]
+#pragma unroll
+    for (int s = 0; s < 2; ++s)
+#pragma unroll
+        for (int am = 0; am < 4; ++am)
+#pragma unroll
+            for (int b = 0; b < 2; ++b)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) acc[s][am][b][r] = 0;
+
+    i32x4 fa[2][4][2], fb[2][2][2]; // [set][block][digit]
+    const uint32_t frag_a = lds0 + lane * 16 + (wm * 4) * HALF, frag_b = lds0 + lane * 16 + (8 + wn * 2) * HALF;
+    // fragment number f of a stage: 0..7 A (block f / 2, digit f % 2), 8..11 B
+    auto read_frag = [&](uint32_t stage_bytes, auto set_tag, auto f_tag) __attribute__((always_inline)) {
+        constexpr int SET = decltype(set_tag)::value, F = decltype(f_tag)::value;
+        constexpr int BLK = (F & 7) / 2, DIG = F & 1, IMM = BLK * HALF + DIG * BLOCK_BYTES;
+        i32x4 &dst = F < 8 ? fa[SET][BLK][DIG] : fb[SET][BLK][DIG];
+        const uint32_t addr = (F < 8 ? frag_a : frag_b) + stage_bytes;
+        asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(dst) : "v"(addr), "n"(IMM));
+    };
+    // matrix instruction number n of a stage (0..23): digit pair n / 8 in the order (0,0) (0,1) (1,0), row block
+    // (n / 2) % 4, column block n % 2; two on one accumulator are eight instructions apart
+    auto mfma_n = [&](auto set_tag, auto n_tag) __attribute__((always_inline)) {
+        constexpr int SET = decltype(set_tag)::value, N = decltype(n_tag)::value;
+        constexpr int PAIR = N / 8, AM = (N / 2) & 3, B = N & 1;
+        constexpr int SH = PAIR == 0 ? 0 : 1, I = PAIR == 2 ? 1 : 0;
+        i32x16 &c = acc[SH][AM][B];
+        const i32x4 &a = fa[SET][AM][I], &b = fb[SET][B][SH - I];
+        if constexpr (SH == 1 && AM >= 2) asm volatile("v_mfma_i32_32x32x32_i8 %0, %1, %2, %0" : "+v"(c) : "v"(a), "v"(b));
+        else asm volatile("v_mfma_i32_32x32x32_i8 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
+    };
+    auto issue_one = [&](uint32_t stage_bytes, auto r_tag) __attribute__((always_inline)) {
+        constexpr int R = decltype(r_tag)::value, H = R / 2, DIG = R & 1;
+        dma16(src_g[H], voff[DIG], lds0 + stage_bytes + (uint32_t)(3 * wave + H) * HALF + DIG * BLOCK_BYTES);
+        if constexpr (DIG == 1) src_g[H] += HALF;
+    };
+
+    const uint32_t ktiles = g.slabs * 2; // stages of one k-block; a multiple of four (the pack pass pads the planes)
+    uint32_t st[NS];
+#pragma unroll
+    for (int n = 0; n < NS; ++n) st[n] = n * STAGE_BYTES;
+
+    using std::integral_constant;
+#pragma unroll
+    for (int n = 0; n < NS - 1; ++n)
+        if ((uint32_t)n < ktiles) issue(st[n]);
+    wait_vm_slabs<LOADS, NS - 2>(ktiles - 1);
+    __builtin_amdgcn_s_barrier();
+    static_for<12>([&](auto f_tag) { read_frag(st[0], integral_constant<int, 0>{}, f_tag); });
+
+    auto iteration = [&](auto parity_tag, auto issue_tag, auto ahead_tag) __attribute__((always_inline)) {
+        constexpr int P = decltype(parity_tag)::value;
+        constexpr bool ISSUE = decltype(issue_tag)::value;
+        constexpr int AHEAD = decltype(ahead_tag)::value;
+        wait_lgkm0(); // the fragments of this stage
+        static_for<12>([&](auto n_tag) {
+            constexpr int N = decltype(n_tag)::value;
+            mfma_n(integral_constant<int, P>{}, n_tag);
+            if constexpr (ISSUE && N % 2 == 0) issue_one(st[NS - 1], integral_constant<int, N / 2>{});
+        });
+        if constexpr (AHEAD >= 0) {
+            wait_vm<AHEAD * LOADS>();
+            __builtin_amdgcn_s_barrier();
+        }
+        static_for<12>([&](auto n_tag) {
+            mfma_n(integral_constant<int, P>{}, integral_constant<int, 12 + decltype(n_tag)::value>{});
+            if constexpr (AHEAD >= 0) read_frag(st[1], integral_constant<int, P ^ 1>{}, n_tag);
+        });
+        const uint32_t t = st[0];
+#pragma unroll
+        for (int n = 0; n + 1 < NS; ++n) st[n] = st[n + 1];
+        st[NS - 1] = t;
+    };
+    using T_ = std::true_type;
+    using F_ = std::false_type;
+    using P0 = integral_constant<int, 0>;
+    using P1 = integral_constant<int, 1>;
+    using STEADY = integral_constant<int, NS - 2>;
+    uint32_t kt = 0;
+    for (; kt + NS < ktiles; kt += 2) { // the fragment sets swap with the stages: two per trip
+        iteration(P0{}, T_{}, STEADY{});
+        iteration(P1{}, T_{}, STEADY{});
+    }
+    if (kt + 4 == ktiles) { // four left: the last stage is still to be requested
+        iteration(P0{}, T_{}, integral_constant<int, 2>{});
+        iteration(P1{}, F_{}, integral_constant<int, 1>{});
+    }
+    iteration(P0{}, F_{}, integral_constant<int, 0>{}); // two left
+    iteration(P1{}, F_{}, integral_constant<int, -1>{});
+
+    asm volatile("s_nop 15\n\ts_nop 15\n\ts_nop 15" ::: "memory"); // the last matrix instructions' results
+
+    // epilogue as in the kernels above, modulo 2^16 (the store keeps the low half)
+    unsigned short *C = static_cast<unsigned short *>(g.C);
+#pragma unroll
+    for (int am = 0; am < 4; ++am) {
+        uint32_t old[2][16];
+        if (g.epi == EPI_ALPHA_BETA) {
+#pragma unroll
+            for (int blk = 0; blk < 2; ++blk) {
+                const uint32_t col = n0 + wn * 64 + blk * 32 + l32, colc = EDGE ? min(col, g.N - 1) : col;
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    const uint32_t row = m0 + (wm * 4 + am) * 32 + 8 * (r / 4) + 4 * lhi + (r % 4);
+                    old[blk][r] = C[(size_t)(EDGE ? min(row, g.M - 1) : row) * g.ldc + colc];
+                }
+            }
+        }
+#pragma unroll
+        for (int blk = 0; blk < 2; ++blk) {
+            const uint32_t col = n0 + wn * 64 + blk * 32 + l32;
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const uint32_t row = m0 + (wm * 4 + am) * 32 + 8 * (r / 4) + 4 * lhi + (r % 4);
+                uint32_t v = (uint32_t)acc[0][am][blk][r] + ((uint32_t)acc[1][am][blk][r] << 8);
+                if (g.epi == EPI_ALPHA) v = g.alpha * v;
+                else if (g.epi == EPI_ALPHA_BETA) v = g.alpha * v + g.beta * old[blk][r];
+                if (!EDGE || ((row < g.M) & (col < g.N))) C[(size_t)row * g.ldc + col] = (unsigned short)v;
+            }
+        }
+    }
+}
+
+template <bool EDGE, int NS> int launch_i16_dma(hipStream_t st, PArgs g) {
+    constexpr size_t lds = WordDmaTile::lds_bytes(NS);
+    auto kern = gemm_i16_packed_dma_kernel<EDGE, NS>;
+    static const hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
+                                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    if (attr != hipSuccess) { (void)hipGetLastError(); return hip_code(attr); }
+    g.tiles_m = (g.M + WordDmaTile::BM - 1) / WordDmaTile::BM;
+    g.tiles_n = (g.N + WordDmaTile::BN - 1) / WordDmaTile::BN;
+    g.patch_m = g.patch_n = 0;
+    static const unsigned shapes[][2] = {{4, 8}, {4, 4}, {2, 8}, {2, 4}};
+    for (const auto &sh : shapes)
+        if (g.tiles_m % sh[0] == 0 && g.tiles_n % sh[1] == 0 && ((g.tiles_m / sh[0]) * (g.tiles_n / sh[1])) % 8 == 0) {
+            g.patch_m = sh[0];
+            g.patch_n = sh[1];
+            break;
+        }
+    hipLaunchKernelGGL(kern, dim3(g.tiles_m * g.tiles_n), dim3(256), lds, st, g);
+    return launch_status();
+}
+
 int digits_of(int dtype) {
     switch (dtype) {
     case WK_I8: case WK_U8: return 1;
@@ -868,6 +1072,9 @@ template <typename E> int launch_typed(hipStream_t st, const GemmProblem &p, uns
         }
         if (tiles256 >= (p.num_cus ? p.num_cus : 256u)) {
             const bool edge = p.M % 256 != 0 || p.N % TILE != 0;
+            // two digits: that tile with the slabs straight into LDS (four wavefronts of 128 x 64): u16 4096^3 727-737 ->
+            // 817-836 TOP/s, 8192^3 799-820 -> 969-975 (entries over the whole type 688 -> 793), ci16 4096^3 645 -> 709
+            if constexpr (D == 2) return edge ? launch_i16_dma<true, 4>(st, g) : launch_i16_dma<false, 4>(st, g);
             return edge ? launch_packed<E, 256, true, 2>(st, g) : launch_packed<E, 256, false, 2>(st, g);
         }
     }
