@@ -103,7 +103,7 @@ int  wk_event_elapsed_ms(wk_event *start, wk_event *stop, float *out_ms);
 /* ---- memory: cl.buffer.create/release (src/tensor/main.zig:229-234,253-263) -----------
  * Pointers from wk_malloc are at least 1 KiB aligned and must go back through wk_free (blocks of
  * 1 MiB and more start 0 / 3 / 6 / 9 KiB into their device allocation in turn, which spreads
- * streams that are walked in step over the memory channels; WK_ALLOC_COLOURS=0 disables it). */
+ * streams that are walked in step over the memory channels). */
 int  wk_malloc(wk_device *dev, size_t bytes, void **out_dptr);
 int  wk_free(wk_device *dev, void *dptr);
 int  wk_mem_info(wk_device *dev, size_t *free_bytes, size_t *total_bytes);
@@ -187,38 +187,6 @@ size_t wk_gemm_workspace_bytes(int dtype, int op_a, int op_b, uint64_t M, uint64
 int    wk_gemm_packed_b_kept(wk_stream *s, int dtype, int op_a, int op_b, uint64_t M, uint64_t N, uint64_t K,
                              const void *host_alpha, const void *A, uint64_t lda, const void *B, uint64_t ldb,
                              const void *host_beta, void *C, uint64_t ldc, void *workspace, size_t workspace_bytes);
-
-/* Name of the kernel variant wk_gemm() would launch for these arguments ("mfma_f32_256x128",
- * "tile64", "thin" for a product of at most four rows or columns, ...).  A name that ends in "+strips" is the kernel of the body of whole tiles of a product
- * that wk_gemm launches in parts: the rows or columns beyond the body follow as products of their own.
- * For benchmarks and profiles; not part of the reference's surface. */
-const char *wk_gemm_variant(int dtype, int op_a, int op_b, uint64_t M, uint64_t N, uint64_t K,
-                            uint64_t lda, uint64_t ldb, uint64_t ldc, const void *A, const void *B, const void *C);
-/* The same for a call that brings workspace_bytes bytes of workspace ("mfma_i32_packed", ...). */
-const char *wk_gemm_variant_with_workspace(int dtype, int op_a, int op_b, uint64_t M, uint64_t N, uint64_t K,
-                                           uint64_t lda, uint64_t ldb, uint64_t ldc, const void *A, const void *B,
-                                           const void *C, size_t workspace_bytes);
-
-/* Host arithmetic only, for tests and benchmarks: how a wk_gemm call on a stream lays out a product
- * whose k is split over work-groups.  Two cases: few tiles of C and a long k (every tile is split:
- * first_tile = 0), and a launch whose tiles do not fill whole rounds of the compute units (the whole
- * rounds, tiles 0 .. first_tile - 1, run as they are; the `tiles` left-over ones follow as a second
- * launch with k split).  A split tile goes to `shares` work-groups that each sum `klen` values of k
- * -- the last one what is left -- into partial tiles of `scratch_bytes` bytes in the stream's own
- * scratch memory; the last work-group to arrive at a tile adds them in the order of the shares, so
- * results are the same bits on every run.  variant NULL: the automatic choice (shares = 1 when it
- * does not split); a splitting variant's name ("mfma_f32_64x64z", "mfma_f64_64x64z",
- * "mfma_f32_256x128t", "mfma_f32_128x128t"): the plan that variant runs when forced.  No counterpart
- * in the reference. */
-int wk_gemm_split_plan(int dtype, int op_a, int op_b, uint64_t M, uint64_t N, uint64_t K, const char *variant,
-                       uint32_t *shares, uint32_t *klen, uint64_t *first_tile, uint64_t *tiles, size_t *scratch_bytes);
-
-/* Test and benchmark knob only, not for product code: force a gemm variant by name ("auto" restores
- * selection).  Process-wide, read by every wk_gemm call on every stream; changing it while a
- * PackedTensors keeps B invalidates what that handle remembers.  A forced variant whose kernel
- * cannot take the problem (a dimension or leading dimension of 2^31 or more) makes wk_gemm return
- * WK_E_INVALID_VALUE.  Returns WK_E_INVALID_VALUE for an unknown name. */
-int wk_gemm_force_variant(const char *name);
 
 /* ---- around the hot path: what one MLP training step needs besides gemm / axpy -----------------
  * (f32 and f64 only; every tensor is a logical {depth, rows, cols} region with its own pitches) */
@@ -320,10 +288,6 @@ int  wk_to_complex(wk_stream *s, int real_dtype, const uint64_t shape3[3], const
                    uint64_t src_slice_pitch, void *dst, uint64_t dst_row_pitch, uint64_t dst_slice_pitch, int space);
 int  wk_to_real(wk_stream *s, int real_dtype, const uint64_t shape3[3], const void *src, uint64_t src_row_pitch,
                 uint64_t src_slice_pitch, void *dst, uint64_t dst_row_pitch, uint64_t dst_slice_pitch, int space);
-
-/* A plain device-to-device streaming copy kernel of known size, used only to calibrate
- * profiler byte counters against a known amount of traffic. */
-int wk_copy_kernel(wk_stream *s, void *dst, const void *src, size_t bytes);
 
 #ifdef __cplusplus
 }

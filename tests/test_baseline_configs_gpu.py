@@ -1,9 +1,12 @@
 """GPU: the benchmark configurations at their real sizes.
 
-Shapes the oracle finishes in seconds are compared entry by entry with it.  The large ones
-(>= 4096^3) are checked through properties that do not need a second full product:
-  * 1024 sampled entries against float64 dot products (tolerance 1e-5*sqrt(K) / 1e-12*sqrt(K)
-    relative to sum|a||b|, as stated for the task);
+Every shape, 8192^3 included, is compared entry by entry with the oracle's reference-order product
+(threaded, it finishes 8192^3 in seconds), both through the mirrored API (the library's own pitches:
+what the benchmark figures are measured on) and through the C ABI with unpadded leading dimensions.
+A float64 second opinion that does not go through the C oracle is taken on one layout per shape:
+  * a lattice of entries -- one in every 32x32 block of C, walking through every position of a block,
+    plus the last row and column -- against float64 dot products (tolerance 1e-5*sqrt(K) /
+    1e-12*sqrt(K) relative to sum|a||b|, as stated for the task);
   * every entry, in aggregate: C @ 1 must equal alpha * A (B 1) + beta * C0 1 (linearity), an
     O(n^2) identity evaluated in float64.
 int32 is compared bit for bit: for |entries| <= 2^20 and K = 2048 every partial sum stays
@@ -13,7 +16,8 @@ import numpy as np
 import pytest
 
 import oracle
-from helpers import F32_TOL, F64_TOL, assert_gemm_close
+from helpers import (F32_TOL, F64_TOL, assert_every_entry, assert_gemm_close, gemm_bound_fast,
+                     lattice_errors)
 from wekua_amd import synth
 
 pytestmark = pytest.mark.gpu
@@ -39,6 +43,9 @@ def operands(rd, M, N, K, op_a, op_b, cfg):
 
 
 def check_by_properties(dtype, got, alpha, a, op_a, b, op_b, beta, c, K):
+    """A float64 second opinion that is independent of the C oracle: a lattice of entries (one in every 32x32
+    block of C, walking through every position of such a block, plus the whole last row and column) against
+    float64 dot products, and the row / column sums of all entries (linearity)."""
     tol = (F32_TOL if dtype == "f32" else F64_TOL) * np.sqrt(K)
     assert np.isfinite(got).all()
     A = a.T if op_a else a
@@ -46,16 +53,9 @@ def check_by_properties(dtype, got, alpha, a, op_a, b, op_b, beta, c, K):
     al = 1.0 if alpha is None else float(alpha)
     be = 0.0 if beta is None else float(beta)
     M, N = got.shape
-    # sampled entries
-    rng = np.random.default_rng(123)
-    ii = rng.integers(0, M, 1024)
-    jj = rng.integers(0, N, 1024)
-    Ar = A[ii].astype(np.float64)
-    Bc = B[:, jj].astype(np.float64).T
-    want = al * np.einsum("ik,ik->i", Ar, Bc) + be * c[ii, jj].astype(np.float64)
-    bound = abs(al) * np.einsum("ik,ik->i", np.abs(Ar), np.abs(Bc)) + abs(be) * np.abs(c[ii, jj]).astype(np.float64)
-    err = np.abs(got[ii, jj].astype(np.float64) - want) / bound
-    assert err.max() <= tol, f"sampled entries: {err.max():.3e} > {tol:.3e}"
+    ii, jj, err = lattice_errors(dtype, got, alpha, a, op_a, b, op_b, beta, c, K)
+    worst = int(err.argmax())
+    assert err[worst] <= 1.0, f"lattice entry ({ii[worst]}, {jj[worst]}): {err[worst]:.3g} x tolerance"
     # linearity over all entries: row sums
     ones = np.ones(N, dtype=np.float64)
     rhs = al * (A.astype(np.float64) @ (B.astype(np.float64) @ ones)) + be * (c.astype(np.float64) @ ones)
@@ -71,6 +71,51 @@ def check_by_properties(dtype, got, alpha, a, op_a, b, op_b, beta, c, K):
     assert cerr.max() <= tol, f"column sums: {cerr.max():.3e} > {tol:.3e}"
 
 
+@pytest.fixture(scope="module")
+def api():
+    """One context + pipeline of the mirrored API: the path bench.py times (the library's own row pitches)."""
+    import wekua_amd as wk
+    context = wk.Context.initFromDeviceType(wk.DeviceType.all)
+    pipeline = wk.Pipeline.init(context.command_queues[0])
+    yield wk, context, pipeline
+    pipeline.deinit()
+    context.deinit()
+
+
+def run_tensors(api, dtype, alpha, a, op_a, b, op_b, beta, c, expect_variant=None):
+    """blas.gemm on Tensor operands (padded, possibly skewed pitches: what the headline figures are measured
+    on).  Returns the product and the name of the kernel variant the library chose."""
+    from wekua_amd import raw
+    wk, context, pipeline = api
+    M, N = c.shape
+    K = a.shape[0] if op_a else a.shape[1]
+    tensors = []
+    for host in (a, b, c):
+        t = wk.Tensor.alloc(dtype, context, pipeline, host.shape)
+        wk.memory.readFromBuffer(pipeline, t, host)
+        tensors.append(t)
+    A, B, C = tensors
+    name = wk._capi.load().wk_gemm_variant(raw.dtype_id(dtype), op_a, op_b, M, N, K, A.row_pitch, B.row_pitch,
+                                               C.row_pitch, A.buffer, B.buffer, C.buffer).decode()
+    wk.blas.gemm(pipeline, alpha, A, op_a, B, op_b, beta, C, None)
+    got = np.empty_like(c)
+    wk.memory.writeToBuffer(pipeline, C, got)
+    pipeline.waitAndCleanup()
+    for t in tensors:
+        t.release(pipeline)
+    if expect_variant is not None:
+        assert expect_variant in name, f"expected a {expect_variant} kernel, the library chose {name}"
+    return got, name
+
+
+def check_whole_product(dtype, got, alpha, a, op_a, b, op_b, beta, c, K, what):
+    """Every entry against the oracle's reference-order product (the CPU device's packed path)."""
+    vw = 8 if dtype == "f32" else 4
+    want = oracle.gemm(dtype, alpha, a, op_a, b, op_b, beta, c, vector_width=vw, packed=True, threads=0)
+    bound = gemm_bound_fast(dtype, alpha, a, op_a, b, op_b, beta, c)
+    assert_every_entry(dtype, got, want, bound, K, what=what)
+
+
 def test_config1_f32_512(dev):
     """f32 C = 1.0*A*B + 0.0*C at 512^3 (C initially zero), also the reference CPU path's own case."""
     a, b, _ = operands(np.float32, 512, 512, 512, 0, 0, 1)
@@ -84,47 +129,80 @@ def test_config1_f32_512(dev):
 
 @pytest.mark.parametrize("n", [1024, 2048])
 @pytest.mark.parametrize("op_a,op_b", OPS)
-def test_config3_f32_square_vs_oracle(dev, n, op_a, op_b):
+def test_config3_f32_square_vs_oracle(dev, api, n, op_a, op_b):
     a, b, c = operands(np.float32, n, n, n, op_a, op_b, 3)
     got = run(dev, "f32", 1.5, a, op_a, b, op_b, 0.5, c)
     want = oracle.gemm("f32", 1.5, a, op_a, b, op_b, 0.5, c, vector_width=8, packed=True)
     assert_gemm_close("f32", got, want, 1.5, a, op_a, b, op_b, 0.5, c, n, what=f"config 3 n={n}")
+    got, name = run_tensors(api, "f32", 1.5, a, op_a, b, op_b, 0.5, c)
+    assert_gemm_close("f32", got, want, 1.5, a, op_a, b, op_b, 0.5, c, n, what=f"config 3 n={n} tensors ({name})")
 
 
 @pytest.mark.parametrize("n", [4096, 8192])
 @pytest.mark.parametrize("op_a,op_b", OPS)
-def test_config3_f32_square_large(dev, n, op_a, op_b):
+def test_config3_f32_square_large_every_entry(dev, api, n, op_a, op_b):
+    """4096^3 and 8192^3, all four layouts, every entry of C against the oracle: once through the mirrored API
+    (the kernel and the pitches of the headline figure) and once through the C ABI with unpadded leading
+    dimensions."""
+    print(f"f32 {n}^3 op=({op_a},{op_b})", flush=True)
     a, b, c = operands(np.float32, n, n, n, op_a, op_b, 3)
+    want = oracle.gemm("f32", 1.5, a, op_a, b, op_b, 0.5, c, vector_width=8, packed=True, threads=0)
+    bound = gemm_bound_fast("f32", 1.5, a, op_a, b, op_b, 0.5, c)
+    got, name = run_tensors(api, "f32", 1.5, a, op_a, b, op_b, 0.5, c, expect_variant="256x128d")
+    assert_every_entry("f32", got, want, bound, n, what=f"config 3 n={n} tensors ({name})")
+    if (op_a, op_b) == (0, 0):
+        check_by_properties("f32", got, 1.5, a, op_a, b, op_b, 0.5, c, n)      # float64, independent of the oracle
     got = run(dev, "f32", 1.5, a, op_a, b, op_b, 0.5, c)
-    check_by_properties("f32", got, 1.5, a, op_a, b, op_b, 0.5, c, n)
+    assert_every_entry("f32", got, want, bound, n, what=f"config 3 n={n} C ABI")
 
 
 @pytest.mark.parametrize("op_a,op_b", OPS)
-def test_config3_f32_ragged_1000(dev, op_a, op_b):
+def test_config3_f32_ragged_1000(dev, api, op_a, op_b):
     a, b, c = operands(np.float32, 1000, 1000, 1000, op_a, op_b, 3)
     got = run(dev, "f32", 1.5, a, op_a, b, op_b, 0.5, c)
     want = oracle.gemm("f32", 1.5, a, op_a, b, op_b, 0.5, c, vector_width=8, packed=True)
     assert_gemm_close("f32", got, want, 1.5, a, op_a, b, op_b, 0.5, c, 1000, what="config 3 1000^3")
+    got, name = run_tensors(api, "f32", 1.5, a, op_a, b, op_b, 0.5, c)
+    assert_gemm_close("f32", got, want, 1.5, a, op_a, b, op_b, 0.5, c, 1000, what=f"config 3 1000^3 tensors ({name})")
 
 
 @pytest.mark.parametrize("op_a,op_b", OPS)
-def test_config3_f32_ragged_4097x4095x4093(dev, op_a, op_b):
+def test_config3_f32_ragged_4097x4095x4093_every_entry(dev, api, op_a, op_b):
+    """The ragged configuration: every entry, through the mirrored API (body of whole tiles on the direct-to-LDS
+    kernel + the strip of one row as a product of its own) and through the C ABI with lda = K etc. (rows that
+    do not start on 16-byte boundaries)."""
     M, N, K = 4097, 4095, 4093
+    print(f"f32 {M}x{N}x{K} op=({op_a},{op_b})", flush=True)
     a, b, c = operands(np.float32, M, N, K, op_a, op_b, 3)
+    want = oracle.gemm("f32", 1.5, a, op_a, b, op_b, 0.5, c, vector_width=8, packed=True, threads=0)
+    bound = gemm_bound_fast("f32", 1.5, a, op_a, b, op_b, 0.5, c)
+    got, name = run_tensors(api, "f32", 1.5, a, op_a, b, op_b, 0.5, c)
+    assert_every_entry("f32", got, want, bound, K, what=f"4097x4095x4093 tensors ({name})")
+    if (op_a, op_b) == (1, 0):
+        check_by_properties("f32", got, 1.5, a, op_a, b, op_b, 0.5, c, K)
     got = run(dev, "f32", 1.5, a, op_a, b, op_b, 0.5, c)
-    check_by_properties("f32", got, 1.5, a, op_a, b, op_b, 0.5, c, K)
+    assert_every_entry("f32", got, want, bound, K, what="4097x4095x4093 C ABI")
 
 
-def test_config4_f64_4096(dev):
-    a, b, c = operands(np.float64, 4096, 4096, 4096, 0, 0, 4)
-    got = run(dev, "f64", 1.0, a, 0, b, 0, 1.0, c)
-    check_by_properties("f64", got, 1.0, a, 0, b, 0, 1.0, c, 4096)
+@pytest.mark.parametrize("op_a,op_b", OPS)
+def test_config4_f64_4096_every_entry(dev, api, op_a, op_b):
+    print(f"f64 4096^3 op=({op_a},{op_b})", flush=True)
+    a, b, c = operands(np.float64, 4096, 4096, 4096, op_a, op_b, 4)
+    got, name = run_tensors(api, "f64", 1.0, a, op_a, b, op_b, 1.0, c, expect_variant="128x128d")
+    check_whole_product("f64", got, 1.0, a, op_a, b, op_b, 1.0, c, 4096, f"f64 4096^3 tensors ({name})")
+    if (op_a, op_b) == (0, 0):
+        check_by_properties("f64", got, 1.0, a, 0, b, 0, 1.0, c, 4096)
+        got = run(dev, "f64", 1.0, a, 0, b, 0, 1.0, c)
+        check_whole_product("f64", got, 1.0, a, 0, b, 0, 1.0, c, 4096, "f64 4096^3 C ABI")
 
 
-def test_config4_f64_tall_skinny(dev):
+def test_config4_f64_tall_skinny_every_entry(dev, api):
     M, N, K = 8192, 256, 8192
     a, b, c = operands(np.float64, M, N, K, 0, 0, 4)
+    got, name = run_tensors(api, "f64", 1.0, a, 0, b, 0, 1.0, c)
+    check_whole_product("f64", got, 1.0, a, 0, b, 0, 1.0, c, K, f"f64 8192x256x8192 tensors ({name})")
     got = run(dev, "f64", 1.0, a, 0, b, 0, 1.0, c)
+    check_whole_product("f64", got, 1.0, a, 0, b, 0, 1.0, c, K, "f64 8192x256x8192 C ABI")
     check_by_properties("f64", got, 1.0, a, 0, b, 0, 1.0, c, K)
     # small enough for a full float64 reference as well (numpy's own BLAS, a third opinion)
     ref = a @ b + c

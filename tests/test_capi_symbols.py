@@ -10,12 +10,32 @@ import pytest
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 HEADER = os.path.join(ROOT, "include", "wekua_hip.h")
+TEST_HEADER = os.path.join(ROOT, "include", "wekua_hip_test.h")     # knobs for tests, benchmarks and profiles
+TEST_ONLY = {"wk_gemm_variant", "wk_gemm_variant_with_workspace", "wk_gemm_split_plan", "wk_gemm_force_variant",
+             "wk_test_option", "wk_copy_kernel"}
 
 
-def declared_functions():
-    text = open(HEADER).read()
-    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
-    return sorted(set(re.findall(r"\b(wk_[a-z0-9_]+)\s*\(", text)))
+def declared_functions(headers=(HEADER, TEST_HEADER)):
+    names = set()
+    for h in headers:
+        text = re.sub(r"/\*.*?\*/", "", open(h).read(), flags=re.S)
+        names |= set(re.findall(r"\b(wk_[a-z0-9_]+)\s*\(", text))
+    return sorted(names)
+
+
+def test_test_knobs_are_not_in_the_product_header():
+    """What exposes or overrides the library's own choices lives in wekua_hip_test.h, and the library reads
+    no switch from the environment."""
+    assert not TEST_ONLY & set(declared_functions((HEADER,)))
+    assert set(declared_functions((TEST_HEADER,))) == TEST_ONLY
+    csrc = os.path.join(ROOT, "wekua_amd", "csrc")
+    for f in os.listdir(csrc):
+        assert "getenv" not in open(os.path.join(csrc, f)).read(), f
+    from wekua_amd import _capi
+    lib = _capi.load()
+    assert lib.wk_test_option(b"no-such-switch", 1) == 1
+    for name, default in ((b"gemm_walk_rows", 0), (b"tail_strict", 0), (b"alloc_colours", 1)):
+        assert lib.wk_test_option(name, default) == 0
 
 
 def test_header_declares_the_hot_path():
@@ -29,7 +49,7 @@ def test_library_exports_every_declared_symbol():
     from wekua_amd import _capi
     lib = _capi.load()
     missing = [n for n in declared_functions() if not hasattr(lib, n)]
-    assert not missing, f"declared in wekua_hip.h but not exported: {missing}"
+    assert not missing, f"declared in the headers but not exported: {missing}"
 
 
 def test_binding_covers_every_declared_symbol():
@@ -142,7 +162,7 @@ def test_zig_binding_in_the_integration_guide_matches_the_header():
     doc = open(os.path.join(ROOT, "INTEGRATION.md")).read()
     zig = {m.group(1): len(_split_args(m.group(2)))
            for m in re.finditer(r"pub extern fn (wk_[a-z0-9_]+)\(([^;]*?)\)\s*[^;()]*;", doc, flags=re.S)}
-    assert set(header) == set(declared_functions())
+    assert set(header) == set(declared_functions((HEADER,)))
     assert set(zig) == set(header), f"not in the guide: {set(header) - set(zig)}; not in the header: {set(zig) - set(header)}"
     wrong = {n: (header[n], zig[n]) for n in header if header[n] != zig[n]}
     assert not wrong, f"parameter counts differ (header, guide): {wrong}"

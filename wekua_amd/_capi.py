@@ -41,7 +41,7 @@ class WkAdamTensor(ctypes.Structure):
                 ("mv_slice_pitch", ctypes.c_uint64)]
 
 
-# name -> (restype, argtypes); one entry per declaration in include/wekua_hip.h
+# name -> (restype, argtypes); one entry per declaration in include/wekua_hip.h and include/wekua_hip_test.h
 SIGNATURES = {
     "wk_strerror": (ctypes.c_char_p, [ci]),
     "wk_abi_version": (ci, []),
@@ -79,6 +79,7 @@ SIGNATURES = {
                                 ctypes.POINTER(ctypes.c_uint32), ctypes.POINTER(u64), ctypes.POINTER(u64),
                                 ctypes.POINTER(ctypes.c_size_t)]),
     "wk_copy_kernel": (ci, [vp, vp, vp, sz]),
+    "wk_test_option": (ci, [ctypes.c_char_p, ci]),
     "wk_hadamard": (ci, [vp, ci, u64p, vp, u64, u64, vp, u64, u64]),
     "wk_activation": (ci, [vp, ci, ci, u64p, vp, u64, u64]),
     "wk_activation_dev": (ci, [vp, ci, ci, u64p, vp, u64, u64, vp, u64, u64]),

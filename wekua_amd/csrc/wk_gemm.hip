@@ -265,18 +265,24 @@ static int gemm_entry(wk_stream *s, int dtype, int op_a, int op_b, uint64_t M, u
     return gemm_generic_launch(s->stream, p);
 }
 
+// a HIP error out of a launch may have cut a counting kernel short
+static int after_launch(wk_stream *s, int rc) {
+    if (rc >= WK_E_HIP_BASE) reset_gemm_counters(s);
+    return rc;
+}
+
 int wk_gemm(wk_stream *s, int dtype, int op_a, int op_b, uint64_t M, uint64_t N, uint64_t K, const void *host_alpha,
             const void *A, uint64_t lda, const void *B, uint64_t ldb, const void *host_beta, void *C, uint64_t ldc,
             void *workspace, size_t workspace_bytes) {
-    return gemm_entry(s, dtype, op_a, op_b, M, N, K, host_alpha, A, lda, B, ldb, host_beta, C, ldc, workspace, workspace_bytes,
-                      false);
+    return after_launch(s, gemm_entry(s, dtype, op_a, op_b, M, N, K, host_alpha, A, lda, B, ldb, host_beta, C, ldc, workspace,
+                                      workspace_bytes, false));
 }
 
 int wk_gemm_packed_b_kept(wk_stream *s, int dtype, int op_a, int op_b, uint64_t M, uint64_t N, uint64_t K,
                           const void *host_alpha, const void *A, uint64_t lda, const void *B, uint64_t ldb, const void *host_beta,
                           void *C, uint64_t ldc, void *workspace, size_t workspace_bytes) {
-    return gemm_entry(s, dtype, op_a, op_b, M, N, K, host_alpha, A, lda, B, ldb, host_beta, C, ldc, workspace, workspace_bytes,
-                      true);
+    return after_launch(s, gemm_entry(s, dtype, op_a, op_b, M, N, K, host_alpha, A, lda, B, ldb, host_beta, C, ldc, workspace,
+                                      workspace_bytes, true));
 }
 
 int wk_gemm_bias_activation(wk_stream *s, int dtype, int op_a, int op_b, uint64_t M, uint64_t N, uint64_t K, const void *A,

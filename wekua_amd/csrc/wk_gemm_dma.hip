@@ -815,10 +815,7 @@ template <int BM, int BN, int BK, int NS, int OCC> int launch_tile_d(hipStream_t
     std::memcpy(&g.beta, p.beta, sizeof(double));
     g.bias = static_cast<const double *>(p.ext_bias);
     g.act = p.ext_act;
-    static const bool row_walk = [] {
-        const char *e = std::getenv("WK_GEMM_WALK");
-        return e && std::strcmp(e, "rows") == 0;
-    }();
+    const bool row_walk = g_test_options.gemm_walk_rows != 0;
     if (!row_walk) {
         static const unsigned shapes[][2] = {{4, 8}, {4, 4}, {2, 8}, {2, 4}};
         for (const auto &sh : shapes)
@@ -875,10 +872,7 @@ template <int BM, int BN, int BK, int NS, int OCC, int KS = 1> int launch_tile(h
     g.act = p.ext_act;
     // XCD-local patches where the tile grid divides into them, eight patches at a time (one per XCD);
     // the k-split tail numbers its tiles in the row-group order, so a body launch keeps that order
-    static const bool row_walk = [] {
-        const char *e = std::getenv("WK_GEMM_WALK");
-        return e && std::strcmp(e, "rows") == 0;
-    }();
+    const bool row_walk = g_test_options.gemm_walk_rows != 0;
     if (!first_tiles && !row_walk) {
         static const unsigned shapes[][2] = {{4, 8}, {4, 4}, {2, 8}, {2, 4}};
         for (const auto &sh : shapes)

@@ -1318,12 +1318,9 @@ int launch_f64_split64(hipStream_t st, const GemmProblem &p, bool edge) {
 #undef WK_CASE
 }
 
-// forced tail variants plan relaxed (tests reach the tail path on small shapes); WK_TAIL_STRICT=1 in the
-// environment makes them plan like the automatic choice (benchmarks of the choice itself)
-const bool g_tail_relaxed = [] {
-    const char *v = std::getenv("WK_TAIL_STRICT");
-    return !(v && v[0] == '1');
-}();
+// forced tail variants plan relaxed (tests reach the tail path on small shapes); the test option
+// "tail_strict" makes them plan like the automatic choice (benchmarks of the choice itself)
+inline bool tail_relaxed() { return g_test_options.tail_strict == 0; }
 
 // ---- a tail of tiles with k split --------------------------------------------------------------
 // A launch whose tiles do not fill whole rounds ends with a few compute units finishing the
@@ -1365,7 +1362,7 @@ bool plan_tail(const GemmProblem &p, int bm, int bn, int bkt, size_t elem, int o
 template <int BM, int BN, int BK, int WMS, int WNS, int OCC>
 int launch_f32_tail(hipStream_t st, const GemmProblem &p, bool edge) {
     GemmSplitPlan plan;
-    if (p.ext || !plan_tail(p, BM, BN, BK, sizeof(float), OCC, g_tail_relaxed, plan)) return launch_f32<BM, BN, BK, WMS, WNS, OCC>(st, p, edge);
+    if (p.ext || !plan_tail(p, BM, BN, BK, sizeof(float), OCC, tail_relaxed(), plan)) return launch_f32<BM, BN, BK, WMS, WNS, OCC>(st, p, edge);
     const int sel = (p.op_a ? 0 : 2) | (p.op_b ? 1 : 0);
     int rc = WK_OK;
     if (plan.first_tile > 0 && gemm_f32_dma_applies(p, BM, BN)) {
@@ -1550,7 +1547,7 @@ bool wk::gemm_mfma_split_plan(const GemmProblem &p, int variant, bool forced, Ge
     const size_t elem = v.dtype == WK_F64 ? 8 : 4;
     switch (split_kind_of(v.name)) {
     case SPLIT_ALL: return plan_split(p, v.bm, v.bn, v.bk, elem, false, plan) || (forced && plan_split(p, v.bm, v.bn, v.bk, elem, true, plan));
-    case SPLIT_TAIL: return plan_tail(p, v.bm, v.bn, v.bk, elem, v.occ, forced && g_tail_relaxed, plan);
+    case SPLIT_TAIL: return plan_tail(p, v.bm, v.bn, v.bk, elem, v.occ, forced && tail_relaxed(), plan);
     default: return false;
     }
 }

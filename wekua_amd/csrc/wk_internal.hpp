@@ -7,6 +7,7 @@
 #include <cstdint>
 
 #include "wekua_hip.h"
+#include "wekua_hip_test.h"
 
 struct wk_device {
     int ordinal;
@@ -38,6 +39,14 @@ struct wk_event {
 
 namespace wk {
 
+// Switches of wk_test_option (wekua_hip_test.h): process-wide, set by tests and benchmarks only.
+struct TestOptions {
+    int gemm_walk_rows = 0; // 1: the direct-to-LDS kernels walk the tiles in groups of rows, not XCD-local patches
+    int tail_strict = 0;    // 1: forced k-split tail variants plan like the automatic choice
+    int alloc_colours = 1;  // 0: wk_malloc hands out blocks as hipMalloc returns them
+};
+extern TestOptions g_test_options;
+
 inline int hip_code(hipError_t e) {
     if (e == hipSuccess) return WK_OK;
     if (e == hipErrorOutOfMemory) return WK_E_OUT_OF_MEMORY;
@@ -59,6 +68,14 @@ inline int launch_status() { return hip_code(hipGetLastError()); }
 // Looks up this device's address of the static scratch array of wk_bias_step_static (wk_nn.hip);
 // wk_device_open calls it with the device current.
 int static_scratch_setup(int ordinal);
+
+// The arrival counters are only zero between launches when every counting kernel ran to its end; after
+// a launch or a wait on the stream has failed they are put back to zero.
+inline void reset_gemm_counters(wk_stream *s) {
+    if (!s || !s->gemm_counters) return;
+    (void)hipMemsetAsync(s->gemm_counters, 0, WK_GEMM_COUNTERS * sizeof(uint32_t), s->stream);
+    (void)hipGetLastError();
+}
 
 inline int bind(wk_stream *s) {
     if (!s || !s->dev) return WK_E_INVALID_VALUE;
