@@ -45,15 +45,19 @@ def log(*a):
     print(*a, file=sys.stderr, flush=True)
 
 
-def read_traffic(name: str):
+def read_traffic(name: str, kernel: str):
     """HBM bytes per launch recorded from a rocprofv3 --pmc run (FETCH_SIZE / WRITE_SIZE) of this
-    command; not measured in this run."""
+    command; not measured in this run.  Returns (bytes, stale): stale when the record was taken on
+    another kernel than the one this run launches."""
     path = os.path.join(ROOT, "profiles", "traffic.json")
     try:
         with open(path) as f:
-            return json.load(f).get(name)
+            rec = json.load(f).get(name)
     except (OSError, ValueError):
-        return None
+        return None, None
+    if not isinstance(rec, dict):
+        return None, None
+    return rec.get("bytes"), rec.get("kernel") != kernel
 
 
 def gemm_leg(wk, synth, n, steps, warmup):
@@ -151,6 +155,34 @@ def axpy_placement_leg(dev, raw, dtype, log2n, steps, warmup):
     return out
 
 
+def memory_ceilings(dev, raw, log2n):
+    """What the memory system gives simpler access patterns on this box in this run, for scale next to
+    the AXPY figure (2 read streams + 1 write stream): a plain copy kernel (1 read + 1 write stream) and
+    math.sum's reduction (1 read stream), both over n = 2^log2n f32 of random data; median of five
+    batches of ten launches."""
+    from wekua_amd._capi import check
+    n = 1 << log2n
+    nbytes = 4 * n
+    src, dst = dev.malloc(nbytes), dev.malloc(nbytes)
+    did = raw.dtype_id("f32")
+    s3 = (ctypes.c_uint64 * 3)(1, 1, n)
+    lo, span = raw.scalar_bytes("f32", -1.0), raw.scalar_bytes("f32", 2.0)
+    check(dev.lib.wk_random_uniform(dev.stream, did, s3, src.ptr, n, n, 5, ctypes.cast(lo, ctypes.c_void_p),
+                                    ctypes.cast(span, ctypes.c_void_p)), "wk_random_uniform")
+    ws = dev.malloc(max(int(dev.lib.wk_sum_workspace_bytes(did)), 16))
+    res = dev.malloc(16)
+    median = lambda call: sorted(dev.time_stream_ms(call, 10) for _ in range(5))[2]
+    for _ in range(3):
+        check(dev.lib.wk_copy_kernel(dev.stream, dst.ptr, src.ptr, nbytes), "copy")
+    dev.sync()
+    copy_ms = median(lambda: check(dev.lib.wk_copy_kernel(dev.stream, dst.ptr, src.ptr, nbytes), "copy"))
+    read_ms = median(lambda: check(dev.lib.wk_sum(dev.stream, did, s3, src.ptr, n, n, ws.ptr, res.ptr, 1.0), "sum"))
+    for b in (src, dst, ws, res):
+        b.free()
+    return {"copy_GBs": 2.0 * nbytes / copy_ms / 1e6, "read_GBs": nbytes / read_ms / 1e6, "n": n, "dtype": "f32",
+            "what": "plain copy kernel (bytes read + written) and math.sum (bytes read), median of 5 batches of 10 launches"}
+
+
 def cpu_gemm_leg(dtype, M, N, K, alpha, beta, threads, a=None, b=None):
     """The reference CPU device's algorithm (packed path, block 16, 8 lanes for f32) timed on this host."""
     import oracle
@@ -196,9 +228,6 @@ def main():
     ap.add_argument("--no-mlp", action="store_true", help="skip the MLP training step leg (benchmark configuration 5)")
     ap.add_argument("--no-configs", action="store_true", help="skip the sweep over the other benchmark configurations")
     ap.add_argument("--no-floor", action="store_true", help="do not turn a missed performance floor into exit status 3")
-    ap.add_argument("--calibrate", action="store_true",
-                    help="also launch the plain 1 GiB copy kernel a few times, so that a profiler run of this "
-                         "command holds a kernel of known HBM traffic to scale byte counters against")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build uses one GPU; --gpus N with N > 1 is not supported "
@@ -219,15 +248,9 @@ def main():
     for dt in ("f32", "f64"):
         log(f"[bench] axpy {dt} 2^{args.axpy_log2n} by placement of y against x: same offset inside a 4 KiB block "
             f"{place[dt]['same_offset_in_4KiB']:.0f} GB/s, 3 KiB further in {place[dt]['y_plus_3KiB']:.0f} GB/s")
-    if args.calibrate:
-        nbytes = 1 << 30
-        src, dst = dev.malloc(nbytes), dev.malloc(nbytes)
-        from wekua_amd._capi import check
-        check(dev.lib.wk_memset_async(dev.stream, src.ptr, 1, nbytes), "memset")
-        ms = dev.time_stream_ms(lambda: check(dev.lib.wk_copy_kernel(dev.stream, dst.ptr, src.ptr, nbytes), "copy"), 5)
-        log(f"[bench] calibration copy 1 GiB: {ms * 1e3:.1f} us -> {2 * nbytes / ms / 1e6:.0f} GB/s (read + write)")
-        src.free()
-        dst.free()
+    ceilings = memory_ceilings(dev, raw, args.axpy_log2n)
+    log(f"[bench] memory ceilings on this box, same buffers: copy (1 read + 1 write stream) {ceilings['copy_GBs']:.0f} GB/s, "
+        f"sum (1 read stream) {ceilings['read_GBs']:.0f} GB/s")
     dev.close()
 
     # every benchmark configuration through the reference-shaped API (tensors from Tensor.alloc, so with
@@ -303,6 +326,8 @@ def main():
     floor["ok"] = bool(floor_ok)
 
     flops = 2.0 * args.n ** 3
+    gemm_traffic, gemm_traffic_stale = read_traffic("gemm_f32_8192", g["variant"]) if args.n == 8192 else (None, None)
+    axpy_traffic, axpy_traffic_stale = read_traffic("axpy_f32_2p28", "axpy_stream") if args.axpy_log2n == 28 else (None, None)
     out = {
         "metric": "f32 GEMM TFLOP/s @8192^3 + AXPY HBM GB/s, each as % of MI355X roofline",
         "value": g["tflops_wall"], "unit": "TFLOP/s",
@@ -314,14 +339,18 @@ def main():
                    "kernel": g["variant"]},
         "roofline": {"bound": "mfma", "achieved": g["tflops_kernel"], "peak": F32_MATRIX_PEAK_TFLOPS,
                      "unit": "TFLOP/s", "frac": g["tflops_kernel"] / F32_MATRIX_PEAK_TFLOPS,
-                     "traffic": read_traffic("gemm_f32_8192"), "traffic_source": "recorded from profiles/traffic.json, not measured in this run",
+                     "traffic": gemm_traffic, "traffic_stale": gemm_traffic_stale,
+                     "traffic_source": "recorded from profiles/traffic.json, not measured in this run",
                      "flops_per_launch": flops, "kernel_ms": g["kernel_ms"]},
         "axpy": {"value": ax_gbs, "unit": "GB/s", "dtype": "f32", "n": 1 << args.axpy_log2n, "us_per_call": ax_us,
                  "roofline": {"bound": "hbm", "achieved": ax_gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                              "frac": ax_gbs / HBM_PEAK_GBS, "traffic": read_traffic("axpy_f32_2p28"),
+                              "frac": ax_gbs / HBM_PEAK_GBS, "traffic": axpy_traffic, "traffic_stale": axpy_traffic_stale,
                               "traffic_source": "recorded from profiles/traffic.json, not measured in this run",
                               "bytes_per_launch": 3.0 * 4 * (1 << args.axpy_log2n)},
                  "f64": {"value": ax64["value"], "us_per_call": ax64["ms"] * 1e3, "frac": ax64["value"] / HBM_PEAK_GBS},
+                 "over_batches": (configs or {}).get(ax_key, {}).get("over_batches"),
+                 "f64_over_batches": (configs or {}).get(f"2_axpy_f64_2p{args.axpy_log2n}", {}).get("over_batches"),
+                 "ceilings": ceilings,
                  "placement_GBs": place,
                  "cpu_baseline": (axpy_cpu or {}).get(f"2_axpy_f32_2p{args.axpy_log2n}")},
         "mlp_step": mlp,
