@@ -182,6 +182,76 @@ def test_int32_matrix_core_extremes(dev):
         dev.lib.wk_gemm_force_variant(b"auto")
 
 
+def _fast_exact_i32(alpha, A, B, beta, c):
+    """The exact product modulo 2^32 of int32 matrices through float64 products of 16-bit halves (each partial
+    product exact below 2^53 for k up to 2^20 or so).  A, B already in op() form."""
+    a = A.astype(np.int64)
+    b = B.astype(np.int64)
+    al, ah = (a & 0xFFFF).astype(np.float64), (a >> 16).astype(np.float64)     # a = ah * 2^16 + al, al unsigned
+    bl, bh = (b & 0xFFFF).astype(np.float64), (b >> 16).astype(np.float64)
+    ll = (al @ bl).astype(np.uint64)
+    mid = ((al @ bh) + (ah @ bl)).astype(np.int64).astype(np.uint64)             # two's complement, then modular
+    prod = (ll + (mid << np.uint64(16))) & np.uint64(0xFFFFFFFF)               # ah * bh * 2^32 vanishes
+    out = prod
+    if alpha is not None or beta is not None:
+        out = prod * np.uint64((1 if alpha is None else alpha) & 0xFFFFFFFF)
+    if beta is not None:
+        out = out + c.astype(np.int64).astype(np.uint64) * np.uint64(beta & 0xFFFFFFFF)
+    return (out & np.uint64(0xFFFFFFFF)).astype(np.uint32).view(np.int32)
+
+
+@pytest.mark.parametrize("case", ["small", "two_digits", "big_a_entry", "big_b_entry", "big_a_row", "zero_a", "zero_b",
+                                  "minus128", "plus128", "big_in_k_padding_neighbour"])
+@pytest.mark.parametrize("op_a,op_b", [(0, 0), (1, 1)])
+def test_int32_packed_skips_only_empty_digit_planes(dev, case, op_a, op_b):
+    """The packed 32-bit product leaves out digit products whose planes the pack pass found all zero, tile by
+    tile.  Whatever the magnitudes -- entries of one digit everywhere, of two, one large entry in A only, in B
+    only, one large row, an all-zero operand, the values on either side of the first digit's range -- the
+    result is the exact product modulo 2^32.  Ragged in every dimension, several tiles, k over several stages."""
+    M, N, K = 300, 260, 700
+    rng = np.random.default_rng(sum(map(ord, case)))
+    lo, hi = (-30000, 30000) if case == "two_digits" else (-100, 100)
+    A = rng.integers(lo, hi + 1, (M, K)).astype(np.int32)
+    B = rng.integers(lo, hi + 1, (K, N)).astype(np.int32)
+    if case == "big_a_entry":
+        A[170, 333] = -1234567890
+    elif case == "big_b_entry":
+        B[650, 259] = 2 ** 31 - 1
+    elif case == "big_a_row":
+        A[5, :] = rng.integers(-2 ** 31, 2 ** 31, K).astype(np.int32)
+    elif case == "zero_a":
+        A[:] = 0
+    elif case == "zero_b":
+        B[:] = 0
+    elif case == "minus128":
+        A[::7, ::5] = -128         # still one digit
+        B[::3, ::11] = -129        # two digits: -129 = 127 - 256
+    elif case == "plus128":
+        A[::7, ::5] = 127          # one digit
+        B[::3, ::11] = 128         # two digits: 128 = -128 + 256
+    elif case == "big_in_k_padding_neighbour":
+        A[:, K - 1] = 2 ** 24 + 3  # the last real k, next to the zero padding of the planes
+        B[K - 1, :] = -(2 ** 24)
+    c = rng.integers(-2 ** 31, 2 ** 31, (M, N)).astype(np.int32)
+    a = np.ascontiguousarray(A.T) if op_a else A
+    b = np.ascontiguousarray(B.T) if op_b else B
+    assert dev.lib.wk_gemm_force_variant(b"mfma_i32_packed") == 0
+    try:
+        for alpha, beta in ((None, None), (3, -2)):
+            got = run_gemm(dev, "i32", alpha, a, op_a, b, op_b, beta, c, packed=True)
+            want = _fast_exact_i32(alpha, A, B, beta, c)
+            bad = np.argwhere(got != want)
+            assert len(bad) == 0, f"{case}: {len(bad)} mismatches, first at {bad[0]}"
+    finally:
+        dev.lib.wk_gemm_force_variant(b"auto")
+
+
+def test_fast_exact_i32_agrees_with_the_semantic_oracle(dev):
+    a, b, c = gemm_operands("i32", 40, 30, 50, 0, 0, 9)
+    assert np.array_equal(_fast_exact_i32(-7, a, b, 5, c), oracle.semantic_gemm("i32", -7, a, 0, b, 0, 5, c))
+    assert np.array_equal(_fast_exact_i32(None, a, b, None, c), oracle.semantic_gemm("i32", None, a, 0, b, 0, None, c))
+
+
 @pytest.mark.parametrize("op_a,op_b", OPS)
 def test_int32_with_workspace_mid_size(dev, op_a, op_b):
     """Mid-size ragged problem with and without a workspace under the automatic choice (which takes

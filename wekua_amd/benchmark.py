@@ -98,12 +98,15 @@ class Session:
         return ms.value / iters
 
 
-def time_gemm(ses, dtype, M, N, K, op_a, op_b, alpha, beta, iters=10, device_fill=False, full_range=False):
+def time_gemm(ses, dtype, M, N, K, op_a, op_b, alpha, beta, iters=10, device_fill=False, full_range=False, keep_b=False):
     """blas.gemm on tensors created by Tensor.alloc (so with the library's own row pitches).
     device_fill: operands drawn on the device instead of generated on the host and uploaded.
     full_range: integer entries over the whole type instead of [-100, 100] (the integer kernels are exact
-    either way, but the clock the part holds under the int8 matrix instruction depends on how many
-    operand bits toggle, and entries of small magnitude have zero upper digits)."""
+    either way, but entries of small magnitude have zero upper digits: the packed 32-bit kernel leaves out
+    the digit products of empty planes, and the clock the part holds under the int8 matrix instruction
+    depends on how many operand bits toggle).
+    keep_b: GemmPackedTensors.keepB(True), i.e. B (the weights of a layer, say) stays packed across the
+    calls and only A goes through the pack pass."""
     rd = raw.real_np_dtype(dtype)
     wk = ses.wk
     tail = (2,) if dtype.startswith("c") else ()
@@ -117,6 +120,8 @@ def time_gemm(ses, dtype, M, N, K, op_a, op_b, alpha, beta, iters=10, device_fil
         C = ses.tensor(dtype, _operand(rd, (M, N) + tail, 3, full_range))
     # as benchmark/gemm.zig:186-196 does: one GemmPackedTensors for the run, passed to every call
     packed = wk.GemmPackedTensors.init(ses.pipeline, C, K, True)
+    if keep_b:
+        packed.keepB(True)
     ses.pipeline.waitAndCleanup()
     ms = ses.time_ms(lambda: wk.blas.gemm(ses.pipeline, alpha, A, op_a, B, op_b, beta, C, packed), iters)
     variant = ses.lib.wk_gemm_variant_with_workspace(raw.dtype_id(dtype), op_a, op_b, M, N, K, A.row_pitch, B.row_pitch,
@@ -189,7 +194,8 @@ HBM_PEAK_GBS = 8000.0
 def baseline_gemm_cases():
     """(key, dtype, M, N, K, op_a, op_b, alpha, beta) for every GEMM of the benchmark configurations, in the
     sweep order of benchmark/gemm.zig:240-283 (size outermost, the four op pairs inside).  A key that ends in
-    `_full_range` draws its integer entries over the whole type instead of [-100, 100]."""
+    `_full_range` draws its integer entries over the whole type instead of [-100, 100]; one that ends in
+    `_b_kept` keeps B packed across the calls (GemmPackedTensors.keepB), so that only A is packed per call."""
     cases = [("1_f32_gemm_512_NN", "f32", 512, 512, 512, 0, 0, 1.0, 0.0)]
     for n in (1024, 2048, 4096, 8192):
         for op_a, op_b, name in OPS:
@@ -201,6 +207,7 @@ def baseline_gemm_cases():
     cases.append(("4_f64_gemm_8192x256x8192_NN", "f64", 8192, 256, 8192, 0, 0, 1.0, 1.0))
     cases.append(("4_i32_gemm_2048_NN", "i32", 2048, 2048, 2048, 0, 0, 3, -2))
     cases.append(("4_i32_gemm_2048_NN_full_range", "i32", 2048, 2048, 2048, 0, 0, 3, -2))
+    cases.append(("4_i32_gemm_2048_NN_b_kept", "i32", 2048, 2048, 2048, 0, 0, 3, -2))
     return cases
 
 
@@ -210,12 +217,22 @@ def run_baseline_configs(ses, log=None, device_fill=True):
     out = {}
     for key, dtype, M, N, K, op_a, op_b, alpha, beta in baseline_gemm_cases():
         ms, variant = time_gemm(ses, dtype, M, N, K, op_a, op_b, alpha, beta, device_fill=device_fill,
-                                full_range=key.endswith("_full_range"))
+                                full_range=key.endswith("_full_range"), keep_b=key.endswith("_b_kept"))
         peak, unit, bound, scale = PEAK[dtype]
+        issued = None
+        if dtype == "i32":
+            # digit products the packed kernel issues per element product: all ten pairs (i, j), i + j <= 3, when
+            # the entries fill the type; the single pair (0, 0) when every entry is one balanced digit ([-128, 127])
+            issued = 10 if key.endswith("_full_range") else 1
+            scale = float(issued)
         rate = 2.0 * M * N * K / ms / 1e9
         out[key] = {"ms": ms, "value": rate, "unit": unit, "kernel": variant,
                     "roofline": {"bound": bound, "achieved": rate * scale, "peak": peak, "unit": unit,
                                  "frac": rate * scale / peak}}
+        if issued is not None:
+            out[key]["roofline"]["digit_products_issued"] = issued
+            out[key]["roofline"]["note"] = ("achieved = 32-bit operations x int8 digit products issued per element product, "
+                                            "against the int8 matrix peak; the pack pass is inside the time")
         if raw.real_np_dtype(dtype).kind != "f":
             out[key]["entries"] = "uniform over the whole type" if key.endswith("_full_range") else "uniform in [-100, 100]"
         if log:

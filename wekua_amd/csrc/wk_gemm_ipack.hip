@@ -49,7 +49,9 @@ constexpr uint32_t MAX_KSPLIT = 16;
 
 struct Layout {
     uint64_t Mp, Np, KB, slabs, ksplit; // KB: k-blocks of 32, padded to whole slabs; ksplit: k-ranges of the pack launch
-    size_t planes_a, planes_b, total;   // byte offsets into the workspace
+    size_t planes_a, planes_b;          // byte offsets into the workspace
+    size_t flags_a, flags_b;            // one byte per (row block, k-range of the pack launch): which digit planes hold a non-zero digit
+    size_t total;
 };
 
 Layout make_layout(int digits, uint64_t M, uint64_t N, uint64_t K) {
@@ -59,8 +61,9 @@ Layout make_layout(int digits, uint64_t M, uint64_t N, uint64_t K) {
     w.Mp = (M + m_tile - 1) / m_tile * m_tile;
     const uint64_t n_tile = digits == 1 ? 256 : TILE; // 8-bit: also the 256-column tile
     w.Np = (N + n_tile - 1) / n_tile * n_tile;
-    // (an even number of slabs, for the two-stage loop of the direct-to-LDS kernels)
-    const uint64_t kb_round = 2 * per_slab;
+    // (an even number of slabs, for the two-stage loop of the direct-to-LDS kernels; the 32-bit product kernel
+    // takes stages of up to four k-blocks when the upper digit planes are empty: eight k-blocks)
+    const uint64_t kb_round = digits == 4 ? 8 : 2 * per_slab;
     w.KB = ((K + BK - 1) / BK + kb_round - 1) / kb_round * kb_round;
     w.slabs = w.KB / per_slab;
     // enough work-groups in the pack launch to fill the chip: (Mp + Np) / 32 row blocks x ksplit
@@ -70,7 +73,9 @@ Layout make_layout(int digits, uint64_t M, uint64_t N, uint64_t K) {
     w.ksplit = ks;
     w.planes_a = 0;
     w.planes_b = w.planes_a + (size_t)w.Mp / 32 * w.slabs * GROUP_BYTES;
-    w.total = w.planes_b + (size_t)w.Np / 32 * w.slabs * GROUP_BYTES;
+    w.flags_a = w.planes_b + (size_t)w.Np / 32 * w.slabs * GROUP_BYTES;
+    w.flags_b = w.flags_a + (size_t)w.Mp / 32 * MAX_KSPLIT;
+    w.total = w.flags_b + (size_t)w.Np / 32 * MAX_KSPLIT;
     return w;
 }
 
@@ -102,6 +107,7 @@ struct PackOperand {
     const void *src;       // element (r, k) at src[r * ld + k] (k-contiguous) or src[k * ld + r]
     uint32_t ld, rows, row_blocks; // true rows; padded rows / 32
     unsigned char *planes;
+    unsigned char *flags;  // [row block][MAX_KSPLIT]: bit d set when digit plane d of that row block and k-range is not all zero
     uint32_t k_contiguous, vector_ok; // vector_ok: 16-byte loads along the contiguous direction are aligned
 };
 struct PackArgs {
@@ -117,12 +123,16 @@ __global__ __launch_bounds__(PACK_THREADS) void ipack_kernel(PackArgs g) {
     __shared__ __align__(16) unsigned char gather_tile[(PACK_THREADS / 64) * 32 * (32 * (D < 4 ? D : 1) + 4)];
     const int which = blockIdx.x >= g.op[0].row_blocks;
     const PackOperand &o = g.op[which];
-    const E *src = static_cast<const E *>(o.src);
+    const E *__restrict__ src = static_cast<const E *>(o.src);
+    unsigned char *__restrict__ planes = o.planes;
     const uint32_t rb = blockIdx.x - (which ? g.op[0].row_blocks : 0u);
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, l32 = lane & 31, half = lane >> 5;
     const uint32_t row = rb * 32 + l32;
     const bool row_ok = row < o.rows;
     const uint32_t kb_begin = blockIdx.y * g.kb_per_split, kb_end = min(g.KB, kb_begin + g.kb_per_split);
+    uint32_t nonzero[D];
+#pragma unroll
+    for (int d = 0; d < D; ++d) nonzero[d] = 0u;
     for (uint32_t kb = kb_begin + wave; kb < kb_end; kb += PACK_THREADS / 64) {
         const uint32_t k0 = kb * BK + 16 * half;
         uint32_t e[16];
@@ -179,16 +189,37 @@ __global__ __launch_bounds__(PACK_THREADS) void ipack_kernel(PackArgs g) {
             for (int d = 0; d < D; ++d) out[d][q] = pd[d];
         }
         // block (rb, kb, d) is the (kb * D + d)-th of its row block
-        unsigned char *dst = o.planes + ((size_t)rb * g.KB * D + (size_t)kb * D) * BLOCK_BYTES + lane * 16;
+        unsigned char *dst = planes + ((size_t)rb * g.KB * D + (size_t)kb * D) * BLOCK_BYTES + lane * 16;
 #pragma unroll
-        for (int d = 0; d < D; ++d) *reinterpret_cast<u32x4 *>(dst + d * BLOCK_BYTES) = out[d];
+        for (int d = 0; d < D; ++d) {
+            *reinterpret_cast<u32x4 *>(dst + d * BLOCK_BYTES) = out[d];
+            nonzero[d] |= out[d][0] | out[d][1] | out[d][2] | out[d][3];
+        }
+    }
+    // Which digit planes of this row block and k-range hold anything: elements of small magnitude have zero
+    // upper digits, and a product kernel that knows it multiplies only the digit pairs that can be non-zero.
+    // One byte per work-group, written by plain stores (every byte has exactly one writer, so nothing needs
+    // clearing beforehand).
+    __shared__ uint32_t wave_mask[PACK_THREADS / 64];
+    uint32_t mask = 0;
+#pragma unroll
+    for (int d = 0; d < D; ++d) mask |= __builtin_amdgcn_ballot_w64(nonzero[d] != 0u) ? 1u << d : 0u;
+    if (lane == 0) wave_mask[wave] = mask;
+    __syncthreads();
+    if (tid == 0) {
+        mask = 0;
+#pragma unroll
+        for (int w2 = 0; w2 < PACK_THREADS / 64; ++w2) mask |= wave_mask[w2];
+        o.flags[(size_t)rb * MAX_KSPLIT + blockIdx.y] = (unsigned char)mask;
     }
 }
 
 struct PArgs {
     const unsigned char *planes_a, *planes_b;
+    const unsigned char *flags_a, *flags_b; // the pack pass's digit-plane masks, [row block][MAX_KSPLIT]
     void *C;
-    uint32_t M, N, K, slabs, Mp, Np, ldc, tiles_m, tiles_n;
+    uint32_t M, N, K, slabs, Mp, Np, ldc, tiles_m, tiles_n; // slabs: what a row block's planes hold (their stride)
+    uint32_t kblocks, ksplit;  // k-blocks of 32 that hold any of k; k-ranges of the pack launch (valid flag bytes per row block)
     int epi;
     uint32_t alpha, beta;
     uint32_t patch_m, patch_n; // the direct-to-LDS kernel's tile walk (0: groups of tile rows)
@@ -406,179 +437,221 @@ void gemm_i32_packed_dma_kernel(PArgs g) {
     }
     const uint32_t m0 = tile_m * BM, n0 = tile_n * BN;
 
-    // wavefront w brings groups 2 w and 2 w + 1 of every slab: A's row groups 0..3, then B's column groups
-    const unsigned char *src_g[2];
-#pragma unroll
-    for (int h = 0; h < 2; ++h) {
-        const int gi = 2 * wave + h;
-        src_g[h] = gi < 4 ? g.planes_a + (size_t)(tile_m * 4 + gi) * g.slabs * GROUP_BYTES
-                          : g.planes_b + (size_t)(tile_n * 4 + gi - 4) * g.slabs * GROUP_BYTES;
-    }
-    uint32_t voff[4];
-#pragma unroll
-    for (int d = 0; d < 4; ++d) voff[d] = lane * 16 + d * BLOCK_BYTES;
     const uint32_t lds0 = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)(__attribute__((address_space(3))) unsigned char *)lds_raw);
-    auto issue = [&](uint32_t stage_bytes) {
-#pragma unroll
-        for (int h = 0; h < 2; ++h) {
-#pragma unroll
-            for (int d = 0; d < 4; ++d)
-                dma16(src_g[h], voff[d], lds0 + stage_bytes + (uint32_t)(2 * wave + h) * GROUP_BYTES + d * BLOCK_BYTES);
-            src_g[h] += GROUP_BYTES;
-        }
-    };
-    constexpr int LOADS = 8;
 
-    i32x16 acc[4][2][2]; // [shift i + j][row block][column block]
-#pragma unroll
-    for (int s = 0; s < 4; ++s)
-#pragma unroll
-        for (int am = 0; am < 2; ++am)
-#pragma unroll
-            for (int b = 0; b < 2; ++b)
-#pragma unroll
-                for (int r = 0; r < 16; ++r) acc[s][am][b][r] = 0;
+    // How many digit planes of this tile's operands hold anything (the pack pass's masks: one byte per row
+    // block and k-range, 4 x MAX_KSPLIT = 64 bytes per operand and tile, one per lane).  Planes that are all
+    // zero contribute nothing to any digit product, so leaving their products out changes no bit of the
+    // result.  ND = 1: only digit 0 anywhere (entries in [-128, 127]); 2: digits 0 and 1; else all four.
+    uint32_t nd;
+    {
+        static_assert(MAX_KSPLIT == 16, "one flag byte per lane: four row blocks x sixteen k-ranges");
+        const uint32_t blk = lane >> 4, range = lane & 15;
+        uint32_t m = 0;
+        if (range < g.ksplit)
+            m = (uint32_t)g.flags_a[(size_t)(tile_m * 4 + blk) * MAX_KSPLIT + range] |
+                (uint32_t)g.flags_b[(size_t)(tile_n * 4 + blk) * MAX_KSPLIT + range];
+        const bool upper = __builtin_amdgcn_ballot_w64((m & 0xCu) != 0u) != 0, second = __builtin_amdgcn_ballot_w64((m & 0x2u) != 0u) != 0;
+        nd = upper ? 4u : second ? 2u : 1u;
+    }
 
+    // The main loop for ND digit planes per operand.  A stage of the pipeline is always 32 KiB: for each of
+    // the tile's eight groups (A's four row groups, then B's four column groups) four 1 KiB blocks, which are
+    // the ND digit blocks of 4 / ND consecutive k-blocks (block slot s = k-block s / ND of the stage, digit
+    // s % ND).  ND = 4 is the whole product: ten digit pairs on one k-block, 40 matrix instructions per
+    // stage and wavefront; ND = 2 multiplies the four pairs of digits 0 and 1 on two k-blocks (32); ND = 1
+    // the pair (0, 0) on four k-blocks (16).  Wavefront w brings groups 2 w and 2 w + 1 of every stage.
+    //
     // Fragment reads and matrix instructions are written as inline assembly, in the order they are to be
     // issued.  (1) The accumulators: the compiler keeps all sixteen in the 256 accumulation registers,
     // needs a few of those for itself and then spills accumulators inside the loop; here shifts 0..2
     // (twelve accumulators) are pinned to accumulation registers and shift 3 (four) to vector registers
     // beside the fragments.  (2) The order: a wavefront is alone on its SIMD, so whatever holds up its
     // instruction stream idles the matrix pipe.  Sixteen 16-byte LDS reads in a row do (four wavefronts'
-    // reads of a slab keep the LDS busy for 512 clocks and the read queue is short), so each read follows
-    // one matrix instruction, and the slab requests are spread over the first half in the same way.
+    // reads of a slab keep the LDS busy for 512 clocks and the read queue is short), so the reads follow
+    // the matrix instructions one by one, and the slab requests are spread over the first half in the same way.
     // What the compiler cannot see in inline assembly are the latencies: LDS reads are waited for by hand
     // (lgkmcnt at the top of the iteration that uses them), two matrix instructions on one accumulator
     // are at least four instructions apart, and in front of the epilogue, which reads the accumulators
     // with vector instructions, the wait is written out.
-    i32x4 fa[2][2][4], fb[2][2][4]; // [set][block][digit]
-    const uint32_t frag_a = lds0 + lane * 16 + (wm * 2) * GROUP_BYTES, frag_b = lds0 + lane * 16 + (4 + wn * 2) * GROUP_BYTES;
-    // fragment number f of a slab: 0..7 A (block f / 4, digit f % 4), 8..15 B
-    auto read_frag = [&](uint32_t stage_bytes, auto set_tag, auto f_tag) __attribute__((always_inline)) {
-        constexpr int SET = decltype(set_tag)::value, F = decltype(f_tag)::value;
-        constexpr int BLK = (F & 7) / 4, DIG = F & 3, IMM = BLK * GROUP_BYTES + DIG * BLOCK_BYTES;
-        // (operands of inline assembly do not capture by themselves inside a generic lambda)
-        i32x4 &dst = F < 8 ? fa[SET][BLK][DIG] : fb[SET][BLK][DIG];
-        const uint32_t addr = (F < 8 ? frag_a : frag_b) + stage_bytes;
-        asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(dst) : "v"(addr), "n"(IMM));
-    };
-    // matrix instruction number n of a slab (0..39): digit pair n / 4 in the order (0,0) (0,1) (1,0) (0,2) (1,1)
-    // (2,0) (0,3) (1,2) (2,1) (3,0), row block (n / 2) % 2, column block n % 2
-    auto mfma_n = [&](auto set_tag, auto n_tag) __attribute__((always_inline)) {
-        constexpr int SET = decltype(set_tag)::value, N = decltype(n_tag)::value;
-        constexpr int PAIR = N / 4, AM = (N / 2) & 1, B = N & 1;
-        constexpr int SH = PAIR < 1 ? 0 : PAIR < 3 ? 1 : PAIR < 6 ? 2 : 3;
-        constexpr int I = PAIR - (SH == 0 ? 0 : SH == 1 ? 1 : SH == 2 ? 3 : 6);
-        i32x16 &c = acc[SH][AM][B];
-        const i32x4 &a = fa[SET][AM][I], &b = fb[SET][B][SH - I];
-        if constexpr (SH == 3) asm volatile("v_mfma_i32_32x32x32_i8 %0, %1, %2, %0" : "+v"(c) : "v"(a), "v"(b));
-        else asm volatile("v_mfma_i32_32x32x32_i8 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
-    };
-    // one of the eight slab requests of this wavefront (group h = R / 4 of its two, digit block R % 4)
-    auto issue_one = [&](uint32_t stage_bytes, auto r_tag) __attribute__((always_inline)) {
-        constexpr int R = decltype(r_tag)::value, H = R / 4, DIG = R & 3;
-        dma16(src_g[H], voff[DIG], lds0 + stage_bytes + (uint32_t)(2 * wave + H) * GROUP_BYTES + DIG * BLOCK_BYTES);
-        if constexpr (DIG == 3) src_g[H] += GROUP_BYTES;
-    };
-
-    const uint32_t ktiles = g.slabs;
-    uint32_t st[NS];
+    auto main_loop = [&](auto nd_tag) __attribute__((always_inline)) {
+        constexpr int ND = decltype(nd_tag)::value;
+        constexpr int KBS = 4 / ND;                                  // k-blocks per stage
+        constexpr int PAIRS = ND == 4 ? 10 : ND == 2 ? 4 : 1;        // digit pairs (i, j), i, j < ND, i + j <= 3
+        constexpr int NM = KBS * PAIRS * 4, HALF = NM / 2;           // matrix instructions per stage and wavefront
+        constexpr int SHIFTS = ND == 4 ? 4 : 2 * ND - 1;             // accumulator sets: one per shift i + j
+        constexpr int LOADS = 8;
+        i32x16 acc[SHIFTS][2][2]; // [shift i + j][row block][column block]
 #pragma unroll
-    for (int n = 0; n < NS; ++n) st[n] = n * STAGE_BYTES;
-
-    using std::integral_constant;
+        for (int s = 0; s < SHIFTS; ++s)
 #pragma unroll
-    for (int n = 0; n < NS - 1; ++n)
-        if ((uint32_t)n < ktiles) issue(st[n]);
-    wait_vm_slabs<LOADS, NS - 2>(ktiles - 1);
-    __builtin_amdgcn_s_barrier();
-    static_for<16>([&](auto f_tag) { read_frag(st[0], integral_constant<int, 0>{}, f_tag); });
-
-    // P: the fragment set that holds slab kt.  ISSUE / AHEAD as in the f32 kernel of wk_gemm_dma.hip.
-    auto iteration = [&](auto parity_tag, auto issue_tag, auto ahead_tag) __attribute__((always_inline)) {
-        constexpr int P = decltype(parity_tag)::value;
-        constexpr bool ISSUE = decltype(issue_tag)::value;
-        constexpr int AHEAD = decltype(ahead_tag)::value;
-        wait_lgkm0(); // the fragments of this slab
-        static_for<20>([&](auto n_tag) {
-            constexpr int N = decltype(n_tag)::value;
-            mfma_n(integral_constant<int, P>{}, n_tag);
-            if constexpr (ISSUE && N % 2 == 0 && N < 16) issue_one(st[NS - 1], integral_constant<int, N / 2>{});
-        });
-        if constexpr (AHEAD >= 0) {
-            wait_vm<AHEAD * LOADS>();
-            __builtin_amdgcn_s_barrier();
+            for (int am = 0; am < 2; ++am)
+#pragma unroll
+                for (int b = 0; b < 2; ++b)
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) acc[s][am][b][r] = 0;
+        // C_old (beta given) of all four blocks as one batch of loads.  With fewer than four accumulator sets
+        // the registers are there to request it ahead of the loop, so that a launch of one round does not
+        // pay that latency between its last matrix instruction and its stores; the whole product reads it
+        // after the loop (the fragment registers are free by then).
+        uint32_t *C = static_cast<uint32_t *>(g.C);
+        uint32_t old[2][2][16];
+        auto read_c_old = [&]() {
+            if (g.epi != EPI_ALPHA_BETA) return;
+#pragma unroll
+            for (int am = 0; am < 2; ++am)
+#pragma unroll
+                for (int blk = 0; blk < 2; ++blk) {
+                    const uint32_t col = n0 + wn * 64 + blk * 32 + l32, colc = EDGE ? min(col, g.N - 1) : col;
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) {
+                        const uint32_t row = m0 + (wm * 2 + am) * 32 + 8 * (r / 4) + 4 * lhi + (r % 4);
+                        old[am][blk][r] = C[(size_t)(EDGE ? min(row, g.M - 1) : row) * g.ldc + colc];
+                    }
+                }
+        };
+        if constexpr (ND < 4) read_c_old();
+        const unsigned char *src_g[2];
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+            const int gi = 2 * wave + h;
+            src_g[h] = gi < 4 ? g.planes_a + (size_t)(tile_m * 4 + gi) * g.slabs * GROUP_BYTES
+                              : g.planes_b + (size_t)(tile_n * 4 + gi - 4) * g.slabs * GROUP_BYTES;
         }
-        static_for<20>([&](auto n_tag) {
-            constexpr int N = decltype(n_tag)::value;
-            mfma_n(integral_constant<int, P>{}, integral_constant<int, 20 + N>{});
-            if constexpr (AHEAD >= 0 && N < 16) read_frag(st[1], integral_constant<int, P ^ 1>{}, n_tag);
-        });
-        const uint32_t t = st[0];
+        uint32_t voff[4]; // block slot s of a stage, relative to the stage's first k-block of the group
 #pragma unroll
-        for (int n = 0; n + 1 < NS; ++n) st[n] = st[n + 1];
-        st[NS - 1] = t;
-    };
-    using std::integral_constant;
-    using T_ = std::true_type;
-    using F_ = std::false_type;
-    using P0 = integral_constant<int, 0>;
-    using P1 = integral_constant<int, 1>;
-    using STEADY = integral_constant<int, NS - 2>;
-    static_assert(NS == 3 || NS == 4, "the drain below is written out for these depths");
-    // The fragment sets swap with the slabs, so the loop runs two slabs per trip; the pack pass pads the
-    // planes of the 32-bit types to an even number of slabs (zero digits), which keeps the drain below to
-    // one fixed sequence per pipeline depth.
-    uint32_t kt = 0;
-    for (; kt + NS < ktiles; kt += 2) {
-        iteration(P0{}, T_{}, STEADY{});
-        iteration(P1{}, T_{}, STEADY{});
-    }
-    if constexpr (NS == 4) {
-        if (kt + 4 == ktiles) { // four left: the last slab is still to be requested
-            iteration(P0{}, T_{}, integral_constant<int, 2>{});
-            iteration(P1{}, F_{}, integral_constant<int, 1>{});
+        for (int sl = 0; sl < 4; ++sl) voff[sl] = lane * 16 + (sl / ND) * GROUP_BYTES + (sl % ND) * BLOCK_BYTES;
+        // one of the eight requests of this wavefront per stage (group h = R / 4 of its two, block slot R % 4)
+        auto issue_one = [&](uint32_t stage_bytes, auto r_tag) __attribute__((always_inline)) {
+            constexpr int R = decltype(r_tag)::value, H = R / 4, SL = R & 3;
+            dma16(src_g[H], voff[SL], lds0 + stage_bytes + (uint32_t)(2 * wave + H) * GROUP_BYTES + SL * BLOCK_BYTES);
+            if constexpr (SL == 3) src_g[H] += KBS * GROUP_BYTES;
+        };
+        auto issue = [&](uint32_t stage_bytes) {
+            static_for<LOADS>([&](auto r_tag) { issue_one(stage_bytes, r_tag); });
+        };
+
+        i32x4 fa[2][2][4], fb[2][2][4]; // [set][block][block slot]
+        const uint32_t frag_a = lds0 + lane * 16 + (wm * 2) * GROUP_BYTES, frag_b = lds0 + lane * 16 + (4 + wn * 2) * GROUP_BYTES;
+        // fragment number f of a stage: 0..7 A (block f / 4, slot f % 4), 8..15 B
+        auto read_frag = [&](uint32_t stage_bytes, auto set_tag, auto f_tag) __attribute__((always_inline)) {
+            constexpr int SET = decltype(set_tag)::value, F = decltype(f_tag)::value;
+            constexpr int BLK = (F & 7) / 4, SL = F & 3, IMM = BLK * GROUP_BYTES + SL * BLOCK_BYTES;
+            // (operands of inline assembly do not capture by themselves inside a generic lambda)
+            i32x4 &dst = F < 8 ? fa[SET][BLK][SL] : fb[SET][BLK][SL];
+            const uint32_t addr = (F < 8 ? frag_a : frag_b) + stage_bytes;
+            asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(dst) : "v"(addr), "n"(IMM));
+        };
+        // matrix instruction number n of a stage: k-block n / (4 PAIRS), digit pair (n / 4) % PAIRS in the order
+        // (0,0) (0,1) (1,0) (0,2) (1,1) (2,0) (0,3) (1,2) (2,1) (3,0) -- for ND = 2: (0,0) (0,1) (1,0) (1,1) --
+        // row block (n / 2) % 2, column block n % 2
+        auto mfma_n = [&](auto set_tag, auto n_tag) __attribute__((always_inline)) {
+            constexpr int SET = decltype(set_tag)::value, N = decltype(n_tag)::value;
+            constexpr int Q = N / (4 * PAIRS), PAIR = (N / 4) % PAIRS, AM = (N / 2) & 1, B = N & 1;
+            constexpr int SH = ND == 2 ? (PAIR + 1) / 2 : PAIR < 1 ? 0 : PAIR < 3 ? 1 : PAIR < 6 ? 2 : 3;
+            constexpr int I = ND == 2 ? PAIR / 2 : PAIR - (SH == 0 ? 0 : SH == 1 ? 1 : SH == 2 ? 3 : 6);
+            static_assert(I < ND && SH - I < ND && SH - I >= 0, "digit pair");
+            i32x16 &c = acc[SH][AM][B];
+            const i32x4 &a = fa[SET][AM][Q * ND + I], &b = fb[SET][B][Q * ND + SH - I];
+            if constexpr (SH == 3) asm volatile("v_mfma_i32_32x32x32_i8 %0, %1, %2, %0" : "+v"(c) : "v"(a), "v"(b));
+            else asm volatile("v_mfma_i32_32x32x32_i8 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
+        };
+
+        // stages that hold any of k, rounded up to an even number (the planes are padded with zero digits
+        // to eight k-blocks)
+        const uint32_t ktiles = (g.kblocks + 2 * KBS - 1) / (2 * KBS) * 2;
+        uint32_t st[NS];
+#pragma unroll
+        for (int n = 0; n < NS; ++n) st[n] = n * STAGE_BYTES;
+
+        using std::integral_constant;
+#pragma unroll
+        for (int n = 0; n < NS - 1; ++n)
+            if ((uint32_t)n < ktiles) issue(st[n]);
+        wait_vm_slabs<LOADS, NS - 2>(ktiles - 1);
+        __builtin_amdgcn_s_barrier();
+        static_for<16>([&](auto f_tag) { read_frag(st[0], integral_constant<int, 0>{}, f_tag); });
+
+        // P: the fragment set that holds stage kt.  ISSUE / AHEAD as in the f32 kernel of wk_gemm_dma.hip.
+        // The eight requests go behind the first matrix instructions of the first half (every other one when
+        // there are at least sixteen), the sixteen fragment reads behind those of the second half.
+        auto iteration = [&](auto parity_tag, auto issue_tag, auto ahead_tag) __attribute__((always_inline)) {
+            constexpr int P = decltype(parity_tag)::value;
+            constexpr bool ISSUE = decltype(issue_tag)::value;
+            constexpr int AHEAD = decltype(ahead_tag)::value;
+            constexpr int ISTEP = HALF >= 16 ? 2 : 1, RPER = (16 + HALF - 1) / HALF; // reads per matrix instruction
+            wait_lgkm0(); // the fragments of this stage
+            static_for<HALF>([&](auto n_tag) {
+                constexpr int N = decltype(n_tag)::value;
+                mfma_n(integral_constant<int, P>{}, n_tag);
+                if constexpr (ISSUE && N % ISTEP == 0 && N / ISTEP < LOADS) issue_one(st[NS - 1], integral_constant<int, N / ISTEP>{});
+            });
+            if constexpr (AHEAD >= 0) {
+                wait_vm<AHEAD * LOADS>();
+                __builtin_amdgcn_s_barrier();
+            }
+            static_for<HALF>([&](auto n_tag) {
+                constexpr int N = decltype(n_tag)::value;
+                mfma_n(integral_constant<int, P>{}, integral_constant<int, HALF + N>{});
+                if constexpr (AHEAD >= 0)
+                    static_for<RPER>([&](auto r_tag) {
+                        constexpr int F = N * RPER + decltype(r_tag)::value;
+                        if constexpr (F < 16) read_frag(st[1], integral_constant<int, P ^ 1>{}, integral_constant<int, F>{});
+                    });
+            });
+            const uint32_t t = st[0];
+#pragma unroll
+            for (int n = 0; n + 1 < NS; ++n) st[n] = st[n + 1];
+            st[NS - 1] = t;
+        };
+        using T_ = std::true_type;
+        using F_ = std::false_type;
+        using P0 = integral_constant<int, 0>;
+        using P1 = integral_constant<int, 1>;
+        using STEADY = integral_constant<int, NS - 2>;
+        static_assert(NS == 3 || NS == 4, "the drain below is written out for these depths");
+        // The fragment sets swap with the stages, so the loop runs two stages per trip; the stage count is
+        // even (above), which keeps the drain below to one fixed sequence per pipeline depth.
+        uint32_t kt = 0;
+        for (; kt + NS < ktiles; kt += 2) {
+            iteration(P0{}, T_{}, STEADY{});
+            iteration(P1{}, T_{}, STEADY{});
         }
-    }
-    iteration(P0{}, F_{}, integral_constant<int, 0>{}); // two left
-    iteration(P1{}, F_{}, integral_constant<int, -1>{});
+        if constexpr (NS == 4) {
+            if (kt + 4 == ktiles) { // four left: the last stage is still to be requested
+                iteration(P0{}, T_{}, integral_constant<int, 2>{});
+                iteration(P1{}, F_{}, integral_constant<int, 1>{});
+            }
+        }
+        iteration(P0{}, F_{}, integral_constant<int, 0>{}); // two left
+        iteration(P1{}, F_{}, integral_constant<int, -1>{});
 
-    // the last matrix instructions' results are not back yet (eight passes of four clocks and change)
-    asm volatile("s_nop 15\n\ts_nop 15\n\ts_nop 15" ::: "memory");
+        // the last matrix instructions' results are not back yet (eight passes of four clocks and change)
+        asm volatile("s_nop 15\n\ts_nop 15\n\ts_nop 15" ::: "memory");
 
-    // epilogue, as in the kernel above; the C_old values of all four blocks are requested before any is
-    // used (the fragment registers are free by now): a one-round launch pays every memory latency here in full
-    uint32_t *C = static_cast<uint32_t *>(g.C);
-    uint32_t old[2][2][16];
-    if (g.epi == EPI_ALPHA_BETA) {
+        // epilogue: register r of lane l is C[8*(r/4) + 4*(l/32) + r%4][l%32] of its 32x32 block, all of it
+        // modulo 2^32
+        if constexpr (ND == 4) read_c_old();
 #pragma unroll
         for (int am = 0; am < 2; ++am)
 #pragma unroll
             for (int blk = 0; blk < 2; ++blk) {
-                const uint32_t col = n0 + wn * 64 + blk * 32 + l32, colc = EDGE ? min(col, g.N - 1) : col;
+                const uint32_t col = n0 + wn * 64 + blk * 32 + l32;
 #pragma unroll
                 for (int r = 0; r < 16; ++r) {
                     const uint32_t row = m0 + (wm * 2 + am) * 32 + 8 * (r / 4) + 4 * lhi + (r % 4);
-                    old[am][blk][r] = C[(size_t)(EDGE ? min(row, g.M - 1) : row) * g.ldc + colc];
+                    uint32_t v = 0;
+#pragma unroll
+                    for (int sh = 0; sh < SHIFTS; ++sh) v += (uint32_t)acc[sh][am][blk][r] << (8 * sh);
+                    if (g.epi == EPI_ALPHA) v = g.alpha * v;
+                    else if (g.epi == EPI_ALPHA_BETA) v = g.alpha * v + g.beta * old[am][blk][r];
+                    if (!EDGE || ((row < g.M) & (col < g.N))) C[(size_t)row * g.ldc + col] = v;
                 }
             }
-    }
-#pragma unroll
-    for (int am = 0; am < 2; ++am)
-#pragma unroll
-        for (int blk = 0; blk < 2; ++blk) {
-            const uint32_t col = n0 + wn * 64 + blk * 32 + l32;
-#pragma unroll
-            for (int r = 0; r < 16; ++r) {
-                const uint32_t row = m0 + (wm * 2 + am) * 32 + 8 * (r / 4) + 4 * lhi + (r % 4);
-                uint32_t v = 0;
-#pragma unroll
-                for (int s = 0; s < 4; ++s) v += (uint32_t)acc[s][am][blk][r] << (8 * s);
-                if (g.epi == EPI_ALPHA) v = g.alpha * v;
-                else if (g.epi == EPI_ALPHA_BETA) v = g.alpha * v + g.beta * old[am][blk][r];
-                if (!EDGE || ((row < g.M) & (col < g.N))) C[(size_t)row * g.ldc + col] = v;
-            }
-        }
+    };
+    if (nd == 1u) main_loop(std::integral_constant<int, 1>{});
+    else if (nd == 2u) main_loop(std::integral_constant<int, 2>{});
+    else main_loop(std::integral_constant<int, 4>{});
 }
 
 template <bool EDGE, int NS> int launch_packed_dma(hipStream_t st, PArgs g) {
@@ -1031,6 +1104,8 @@ template <typename E> int launch_typed(hipStream_t st, const GemmProblem &p, uns
     };
     operand(pa.op[0], p.A, p.lda, p.M, w.Mp, !p.op_a, w.planes_a); // A is k-contiguous for op N
     operand(pa.op[1], p.B, p.ldb, p.N, w.Np, p.op_b != 0, w.planes_b); // B for op T
+    pa.op[0].flags = ws + w.flags_a;
+    pa.op[1].flags = ws + w.flags_b;
     pa.K = (uint32_t)p.K;
     pa.KB = (uint32_t)w.KB;
     pa.kb_per_split = (uint32_t)((w.KB + w.ksplit - 1) / w.ksplit);
@@ -1043,6 +1118,10 @@ template <typename E> int launch_typed(hipStream_t st, const GemmProblem &p, uns
     PArgs g;
     g.planes_a = ws + w.planes_a;
     g.planes_b = ws + w.planes_b;
+    g.flags_a = ws + w.flags_a;
+    g.flags_b = ws + w.flags_b;
+    g.kblocks = (uint32_t)((p.K + BK - 1) / BK);
+    g.ksplit = (uint32_t)w.ksplit;
     g.C = p.C;
     g.M = (uint32_t)p.M; g.N = (uint32_t)p.N; g.K = (uint32_t)p.K;
     g.slabs = (uint32_t)w.slabs; g.Mp = (uint32_t)w.Mp; g.Np = (uint32_t)w.Np;

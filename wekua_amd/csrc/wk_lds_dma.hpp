@@ -16,15 +16,16 @@ namespace wk {
 namespace lds_dma {
 
 // 16 bytes per lane from global memory (scalar base + 32-bit byte offset per lane) to LDS at
-// lds_base + 16 * lane; lds_base is a byte address, the same in every lane.  M0 is named as clobbered so
-// that the compiler never keeps a value of its own (dynamic indexing, lane reads) live in it across the load.
+// lds_base + 16 * lane; lds_base is a byte address, the same in every lane.  The LDS base travels in M0,
+// which the register allocator writes itself (the "{m0}" operand): a value of its own that it keeps there
+// (lane indexing, messages) is then saved and restored around the load like around any other use.  The
+// s_nop covers the wait state between a write of M0 and an LDS-DMA instruction that reads it.
 __device__ __forceinline__ void dma16(const void *base, uint32_t byte_offset, uint32_t lds_base) {
-    asm volatile("s_mov_b32 m0, %2\n\t"
-                 "s_nop 0\n\t"
+    asm volatile("s_nop 0\n\t"
                  "global_load_lds_dwordx4 %0, %1"
                  :
-                 : "v"(byte_offset), "s"(base), "s"(lds_base)
-                 : "memory", "m0");
+                 : "v"(byte_offset), "s"(base), "{m0}"(lds_base)
+                 : "memory");
 }
 
 template <int N> __device__ __forceinline__ void wait_vm() { asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory"); }
