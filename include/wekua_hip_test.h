@@ -58,6 +58,12 @@ int wk_gemm_force_variant(const char *name);
  *                       blocks of 1 MiB and more start 0 / 3 / 6 / 9 KiB into their allocation in turn). */
 int wk_test_option(const char *name, int value);
 
+/* Launch-cost probes for profiles: a kernel with the grid, work-group size (a multiple of 64) and dynamic LDS
+ * claim of a GEMM launch that does nothing (kind 0), or only stores 16 floats per thread into dst (kind 1:
+ * what the C write-back of a tile costs; dst_bytes >= work_groups * threads * 64). */
+int wk_probe_launch(wk_stream *s, int kind, unsigned work_groups, unsigned threads, size_t lds_bytes, void *dst,
+                    size_t dst_bytes);
+
 /* A plain device-to-device streaming copy kernel of known size, used only to calibrate
  * profiler byte counters against a known amount of traffic. */
 int wk_copy_kernel(wk_stream *s, void *dst, const void *src, size_t bytes);

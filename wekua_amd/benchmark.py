@@ -6,6 +6,7 @@ times over 1-D sizes, on GPU 0.
     python -m wekua_amd.benchmark axpy [--dtype f32]
     python -m wekua_amd.benchmark configs        # every GEMM / AXPY benchmark configuration, one line each
     python -m wekua_amd.benchmark tensor         # transpose / copy / random.uniform / toComplex streaming rates
+    python -m wekua_amd.benchmark probe          # cost of an empty and of a store-only launch on the GEMM grids
     python -m wekua_amd.benchmark mlp [--dtype f32] [--sizes 1024 4096 4096 1024] [--batch 2048] [--optimizer adam]
 
 Everything goes through the reference-shaped API (Tensor.alloc, memory.readFromBuffer, blas.*).
@@ -380,6 +381,37 @@ def time_mlp_step(dtype="f32", sizes=(1024, 4096, 4096, 1024), batch=2048, optim
             "loss_after": float(loss[0])}
 
 
+def cmd_probe(ses, args):
+    """What a launch costs before any product is computed: an empty kernel and a kernel that only stores an
+    f32 tile per work-group, on the grids, work-group sizes and LDS claims of the small one-round GEMM launches;
+    per-call time on the stream (back-to-back launches, like the GEMM rows of this benchmark)."""
+    import ctypes
+    wk = ses.wk
+    dev = wk._lib().wkz_context_device(ses.ctx._h)
+    buf = ctypes.c_void_p()
+    nbytes = 64 << 20
+    wk._capi.check(ses.lib.wk_malloc(dev, nbytes, ctypes.byref(buf)))
+    print(f"{'probe':12s} {'work-groups':>11s} {'threads':>7s} {'LDS KiB':>7s} {'us':>7s}")
+    for wgs, threads, lds_kib in ((256, 256, 0), (256, 256, 48), (256, 512, 96), (256, 1024, 96), (64, 256, 48), (1024, 256, 48),
+                                  (2048, 256, 72)):
+        for kind, name in ((0, "empty"), (1, "store-only")):
+            check = wk._capi.check
+
+            def batch(iters):
+                check(ses.lib.wk_event_record(ses.e0, ses.stream))
+                for _ in range(iters):
+                    check(ses.lib.wk_probe_launch(ses.stream, kind, wgs, threads, lds_kib << 10, buf, nbytes))
+                check(ses.lib.wk_event_record(ses.e1, ses.stream))
+                check(ses.lib.wk_stream_sync(ses.stream))     # these launches do not go through the pipeline
+                t = ctypes.c_float()
+                check(ses.lib.wk_event_elapsed_ms(ses.e0, ses.e1, ctypes.byref(t)))
+                return t.value / iters
+            batch(200)
+            ms = min(batch(50) for _ in range(3))
+            print(f"{name:12s} {wgs:11d} {threads:7d} {lds_kib:7d} {ms * 1e3:7.2f}", flush=True)
+    wk._capi.check(ses.lib.wk_free(dev, buf))
+
+
 def cmd_mlp(args):
     r = time_mlp_step(args.dtype, tuple(args.sizes), args.batch, args.optimizer, args.lr, args.steps, args.warmup)
     print(f"mlp {'-'.join(map(str, args.sizes))} {args.dtype} batch {args.batch} {args.optimizer}: "
@@ -401,6 +433,7 @@ def main(argv=None):
     a = sub.add_parser("axpy")
     a.add_argument("--dtype", default="f32")
     sub.add_parser("tensor")
+    sub.add_parser("probe")
     c = sub.add_parser("configs")
     c.add_argument("--variant", default="auto")
     m = sub.add_parser("mlp")
@@ -419,7 +452,7 @@ def main(argv=None):
     try:
         if getattr(args, "variant", "auto") != "auto":
             raw.check(ses.lib.wk_gemm_force_variant(args.variant.encode()), "wk_gemm_force_variant")
-        {"gemm": cmd_gemm, "axpy": cmd_axpy, "configs": cmd_configs, "tensor": cmd_tensor}[args.cmd](ses, args)
+        {"gemm": cmd_gemm, "axpy": cmd_axpy, "configs": cmd_configs, "tensor": cmd_tensor, "probe": cmd_probe}[args.cmd](ses, args)
     finally:
         ses.close()
     return 0

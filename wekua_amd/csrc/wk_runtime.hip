@@ -439,6 +439,29 @@ __global__ __launch_bounds__(256) void copy16_kernel(uint4 *__restrict__ dst, co
         dst[i] = src[i];
 }
 
+// Launch-cost probes: the same grid, work-group size and LDS claim as a GEMM launch, with nothing (kind 0)
+// or only the stores of an f32 tile per work-group (kind 1: 16 floats per thread, rows of 64 floats) inside.
+extern "C" __global__ void wk_probe_kernel(int kind, float *dst, float value) {
+    extern __shared__ float probe_lds[];
+    if (kind == 0) return;
+    float *tile = dst + (size_t)blockIdx.x * blockDim.x * 16;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) tile[(size_t)r * blockDim.x + threadIdx.x] = value;
+}
+
+extern "C" int wk_probe_launch(wk_stream *s, int kind, unsigned work_groups, unsigned threads, size_t lds_bytes, void *dst,
+                               size_t dst_bytes) {
+    int rc = bind(s);
+    if (rc) return rc;
+    if (kind < 0 || kind > 1 || !work_groups || !threads || threads > 1024 || threads % 64 || lds_bytes > 160 * 1024) return WK_E_INVALID_VALUE;
+    if (kind == 1 && (!dst || dst_bytes < (size_t)work_groups * threads * 16 * sizeof(float))) return WK_E_INVALID_VALUE;
+    static hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void *>(wk_probe_kernel),
+                                                 hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+    if (attr != hipSuccess) { (void)hipGetLastError(); return hip_code(attr); }
+    hipLaunchKernelGGL(wk_probe_kernel, dim3(work_groups), dim3(threads), lds_bytes, s->stream, kind, static_cast<float *>(dst), 1.0f);
+    return launch_status();
+}
+
 extern "C" int wk_copy_kernel(wk_stream *s, void *dst, const void *src, size_t bytes) {
     int rc = bind(s);
     if (rc) return rc;
