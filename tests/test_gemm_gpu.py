@@ -252,6 +252,78 @@ def test_fast_exact_i32_agrees_with_the_semantic_oracle(dev):
     assert np.array_equal(_fast_exact_i32(None, a, b, None, c), oracle.semantic_gemm("i32", None, a, 0, b, 0, None, c))
 
 
+def _wrapping_u64_product(alpha, A, B, beta, c):
+    """alpha * A B + beta * C modulo 2^64 with numpy's wrapping unsigned arithmetic (A, B in op() form)."""
+    u = np.uint64
+    prod = A.view(u) @ B.view(u) if A.dtype.itemsize == 8 else A.astype(u) @ B.astype(u)
+    if alpha is None and beta is None:
+        out = prod
+    else:
+        out = prod * u((1 if alpha is None else alpha) & 0xFFFFFFFFFFFFFFFF)
+        if beta is not None:
+            out = out + c.view(u) * u(beta & 0xFFFFFFFFFFFFFFFF)
+    return out.view(c.dtype)
+
+
+@pytest.mark.parametrize("dtype", ["i64", "u64"])
+@pytest.mark.parametrize("op_a,op_b", OPS)
+def test_int64_packed_bit_exact(dev, dtype, op_a, op_b):
+    """64-bit integers on the int8 matrix cores (eight balanced digits, 36 digit products) against the exact
+    product modulo 2^64 on full-range entries: interior and ragged shapes, K not a multiple of the k-block,
+    every alpha / beta combination, unaligned leading dimensions."""
+    variant = f"mfma_{dtype}_packed"
+    assert dev.lib.wk_gemm_force_variant(variant.encode()) == 0
+    try:
+        for (M, N, K) in [(128, 64, 32), (128, 128, 64), (256, 192, 416), (1, 1, 1), (65, 129, 33), (200, 300, 77), (63, 127, 500)]:
+            for alpha, beta in [(None, None), (3, None), (-5 if dtype == "i64" else 2 ** 63 + 12345, 7), (None, 1)]:
+                check(dev, dtype, M, N, K, op_a, op_b, alpha, beta, seed=31, packed=True)
+        check(dev, dtype, 130, 70, 200, op_a, op_b, 3, 7, seed=32, packed=True,
+              lda=(130 if op_a else 200) + 3, ldb=(200 if op_b else 70) + 5, ldc=70 + 7)
+    finally:
+        dev.lib.wk_gemm_force_variant(b"auto")
+
+
+def test_int64_packed_digit_extremes_and_long_k(dev):
+    """Values that stress the split into eight balanced digits (0x00, 0x7f, 0x80, 0xff in every byte position,
+    all digits -128 or all 127, values one off a carry into the next digit), and a k longer than one launch
+    may sum exactly (16384): the product is then a chain of launches through C."""
+    pieces = np.array([0x00, 0x7f, 0x80, 0xff, 0x01, 0x81, 0x7e, 0xfe], dtype=np.uint64)
+    rng = np.random.default_rng(5)
+
+    def draw(shape):
+        out = np.zeros(shape, dtype=np.uint64)
+        for byte in range(8):
+            out |= pieces[rng.integers(0, len(pieces), shape)] << np.uint64(8 * byte)
+        return out.view(np.int64)
+    tiny_a, tiny_b, tiny_c = draw((9, 40)), draw((40, 7)), draw((9, 7))
+    assert np.array_equal(_wrapping_u64_product(-3, tiny_a, tiny_b, 5, tiny_c), oracle.semantic_gemm("i64", -3, tiny_a, 0, tiny_b, 0, 5, tiny_c))
+    assert dev.lib.wk_gemm_force_variant(b"mfma_i64_packed") == 0
+    try:
+        for (M, N, K) in [(128, 64, 320), (130, 70, 16384 + 16384 + 333)]:
+            a, b, c = draw((M, K)), draw((K, N)), draw((M, N))
+            for alpha, beta in [(None, None), (-3, 5), (7, None)]:
+                got = run_gemm(dev, "i64", alpha, a, 0, b, 0, beta, c, packed=True)
+                assert np.array_equal(got, _wrapping_u64_product(alpha, a, b, beta, c)), (M, N, K, alpha, beta)
+            at, bt = np.ascontiguousarray(a.T), np.ascontiguousarray(b.T)
+            got = run_gemm(dev, "i64", 2, at, 1, bt, 1, -1, c, packed=True)
+            assert np.array_equal(got, _wrapping_u64_product(2, a, b, -1, c))
+    finally:
+        dev.lib.wk_gemm_force_variant(b"auto")
+
+
+def test_int64_automatic_choice_with_workspace(dev):
+    """With a workspace the automatic choice takes the matrix-core path from mid sizes up and the vector-ALU
+    kernel below; both bit-exact, and the name query says which."""
+    from wekua_amd import raw
+    did = raw.dtype_id("u64")
+    name = lambda M, N, K: dev.lib.wk_gemm_variant_with_workspace(did, 0, 0, M, N, K, K, N, N, None, None, None, 1 << 40).decode()
+    assert name(512, 512, 512) == "mfma_u64_packed" and name(32, 32, 32) == "tile64"
+    for (M, N, K) in [(512, 384, 256), (32, 32, 32)]:
+        a, b, c = gemm_operands("u64", M, N, K, 0, 1, 41)
+        got = run_gemm(dev, "u64", 3, a, 0, b, 1, 2 ** 64 - 2, c, packed=True)
+        assert np.array_equal(got, _wrapping_u64_product(3, a, np.ascontiguousarray(b.T), 2 ** 64 - 2, c))
+
+
 @pytest.mark.parametrize("op_a,op_b", OPS)
 def test_int32_with_workspace_mid_size(dev, op_a, op_b):
     """Mid-size ragged problem with and without a workspace under the automatic choice (which takes
@@ -737,7 +809,7 @@ def test_seeded_random_problems(dev, dtype):
         check(dev, dtype, M, N, K, op_a, op_b, alpha, beta, seed=1000 + case, packed=integer and case % 2 == 0, **kw)
 
 
-@pytest.mark.parametrize("dtype", ["cf32", "cf64", "ci8", "cu8", "ci16", "cu16", "ci32", "cu32"])
+@pytest.mark.parametrize("dtype", ["cf32", "cf64", "ci8", "cu8", "ci16", "cu16", "ci32", "cu32", "ci64", "cu64"])
 @pytest.mark.parametrize("op_a,op_b", OPS)
 def test_complex_through_the_real_matrix_cores(dev, dtype, op_a, op_b):
     """Complex types with a workspace: B is expanded to its real 2K x 2N form (alpha folded in),
@@ -770,7 +842,7 @@ def test_complex_float_nan_in_c_propagates_with_beta(dev):
         dev.lib.wk_gemm_force_variant(b"auto")
 
 
-@pytest.mark.parametrize("dtype", ["i8", "u16", "i32", "cf32", "cf64", "ci16", "cu32"])
+@pytest.mark.parametrize("dtype", ["i8", "u16", "i32", "u64", "cf32", "cf64", "ci16", "cu32", "ci64"])
 @pytest.mark.parametrize("op_a,op_b", OPS)
 def test_packed_b_kept_across_calls(dev, dtype, op_a, op_b):
     """wk_gemm_packed_b_kept: after one wk_gemm with a workspace, later calls with a new A pack only A.

@@ -18,17 +18,17 @@ namespace {
 std::atomic<int> g_forced{-2};
 
 const char *k_generic_name = "tile64";
-// indexed by dtype (WK_I8 .. WK_U32)
-const char *k_packed_names[6] = {"mfma_i8_packed", "mfma_u8_packed", "mfma_i16_packed", "mfma_u16_packed",
-                                 "mfma_i32_packed", "mfma_u32_packed"};
-const char *k_complex_packed_names[8] = {"mfma_ci8_packed",  "mfma_cu8_packed",  "mfma_ci16_packed", "mfma_cu16_packed",
-                                         "mfma_ci32_packed", "mfma_cu32_packed", "mfma_cf32_packed", "mfma_cf64_packed"};
+// indexed by dtype (WK_I8 .. WK_U64)
+const char *k_packed_names[8] = {"mfma_i8_packed", "mfma_u8_packed", "mfma_i16_packed", "mfma_u16_packed",
+                                 "mfma_i32_packed", "mfma_u32_packed", "mfma_i64_packed", "mfma_u64_packed"};
+// indexed by dtype - WK_COMPLEX
+const char *k_complex_packed_names[10] = {"mfma_ci8_packed",  "mfma_cu8_packed",  "mfma_ci16_packed", "mfma_cu16_packed",
+                                          "mfma_ci32_packed", "mfma_cu32_packed", "mfma_ci64_packed", "mfma_cu64_packed",
+                                          "mfma_cf32_packed", "mfma_cf64_packed"};
 bool is_complex_float(int dtype) { return dtype == WK_CF32 || dtype == WK_CF64; }
-bool is_complex_small_int(int dtype) { return dtype >= WK_COMPLEX + WK_I8 && dtype <= WK_COMPLEX + WK_U32; }
+bool is_complex_small_int(int dtype) { return dtype >= WK_COMPLEX + WK_I8 && dtype <= WK_COMPLEX + WK_U64; }
 bool has_complex_packed_path(int dtype) { return is_complex_float(dtype) || is_complex_small_int(dtype); }
-const char *complex_packed_name(int dtype) {
-    return k_complex_packed_names[is_complex_float(dtype) ? 6 + (dtype == WK_CF64) : dtype - WK_COMPLEX];
-}
+const char *complex_packed_name(int dtype) { return k_complex_packed_names[dtype - WK_COMPLEX]; }
 // Two to four extra launches over the operands.  Measured against the generic kernel on MI355X: 512^3
 // 4x faster (cf32 0.137 -> 0.034 ms), 1024^3 3.7x, 4096^3 1.8x; the launches alone cost ~15 us.
 bool complex_packed_pays(const GemmProblem &p) {
@@ -44,7 +44,8 @@ int transpose_for_gemm(void *ctx, int dtype, uint64_t rows, uint64_t cols, const
 }
 
 bool is_int32(int dtype) { return dtype == WK_I32 || dtype == WK_U32; }
-bool has_packed_path(int dtype) { return dtype >= WK_I8 && dtype <= WK_U32; }
+bool is_int64(int dtype) { return dtype == WK_I64 || dtype == WK_U64; }
+bool has_packed_path(int dtype) { return dtype >= WK_I8 && dtype <= WK_U64; }
 // The pack pass reads A and B once more and writes as much.  32-bit, measured against the fused
 // matrix-core kernels on MI355X (N,N / T,N, microseconds, fused best of its two tiles -> packed): 1024^3
 // 34 / 43 -> 39, 1536^3 61 / 63 -> 48, 2048^3 86 -> 77, 1024 x 1024 x 4096 117 / 154 -> 96, 2048 x 2048 x 512
@@ -53,6 +54,8 @@ bool has_packed_path(int dtype) { return dtype >= WK_I8 && dtype <= WK_U32; }
 bool packed_pays(const GemmProblem &p) {
     const double work = (double)p.M * (double)p.N * (double)p.K;
     if (is_int32(p.dtype)) return p.M >= 1024 && p.N >= 1024 && work >= 3.0e9;
+    // 64 bits: the vector-ALU kernel (14-17 TOP/s) is the only other one (128^3: 36 us against 14, 512^3: 126 against 33)
+    if (is_int64(p.dtype)) return p.M >= 32 && p.N >= 32 && p.K >= 32 && work >= 262144.0;
     return p.M >= 256 && p.N >= 256 && work >= 4.0e8;
 }
 

@@ -1,4 +1,4 @@
-// Complex GEMM (float and 8/16/32-bit integer components) through the real matrix-core kernels, for callers that bring a workspace
+// Complex GEMM (float and integer components) through the real matrix-core kernels, for callers that bring a workspace
 // (blas.PackedTensors, the reference's pack pass: src/blas/gemm.zig:272-357, 705-720).
 //
 // With interleaved storage a complex M x K matrix IS a real M x 2K matrix, and
@@ -12,7 +12,7 @@
 // Rounding differs from the reference's three-multiplication complex product
 // (wekua_cl_lib.cl:648-653) only within the stated float tolerance.
 // For the complex integer types everything is arithmetic modulo 2^width, where the identity is exact:
-// the passes compute in unsigned 32-bit and truncate (signed and unsigned share the bits), and the real
+// the passes compute in unsigned 32-bit (64-bit components: 64-bit) and truncate (signed and unsigned share the bits), and the real
 // product is the packed int8 matrix-core path on (M, 2N, 2K) in the section of the workspace behind B~.
 #include "wk_internal.hpp"
 
@@ -26,7 +26,8 @@ namespace {
 constexpr int CP_BLOCK = 256;
 
 // the type the passes compute in: wraparound arithmetic for the integers without promotion to signed int
-template <typename R> using Wide = std::conditional_t<std::is_integral_v<R>, uint32_t, R>;
+template <typename R>
+using Wide = std::conditional_t<std::is_integral_v<R>, std::conditional_t<sizeof(R) == 8, uint64_t, uint32_t>, R>;
 
 // one thread per complex element of B (K x N, row pitch ldb complex elements)
 template <typename R>
@@ -95,7 +96,7 @@ int prepare(hipStream_t st, const GemmProblem &p, const void *b_src, uint64_t ld
 int real_of(int dtype) {
     if (dtype == WK_CF32) return WK_F32;
     if (dtype == WK_CF64) return WK_F64;
-    if (dtype >= WK_COMPLEX + WK_I8 && dtype <= WK_COMPLEX + WK_U32) return dtype - WK_COMPLEX;
+    if (dtype >= WK_COMPLEX + WK_I8 && dtype <= WK_COMPLEX + WK_U64) return dtype - WK_COMPLEX;
     return -1;
 }
 
@@ -156,7 +157,7 @@ int wk::gemm_complex_packed_prepare(hipStream_t st, const GemmProblem &p, void *
     case 2: rc = prepare<uint8_t>(st, p, b_src, ldb, bx); break;
     case 4: rc = prepare<uint16_t>(st, p, b_src, ldb, bx); break;
     case 8: rc = rd == WK_F32 ? prepare<float>(st, p, b_src, ldb, bx) : prepare<uint32_t>(st, p, b_src, ldb, bx); break;
-    default: rc = prepare<double>(st, p, b_src, ldb, bx); break;
+    default: rc = rd == WK_F64 ? prepare<double>(st, p, b_src, ldb, bx) : prepare<uint64_t>(st, p, b_src, ldb, bx); break;
     }
     if (rc) return rc;
 

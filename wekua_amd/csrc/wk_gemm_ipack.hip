@@ -1172,6 +1172,7 @@ template <typename E> int launch_typed(hipStream_t st, const GemmProblem &p, uns
 // 0: this problem cannot take the packed path (not an 8/16/32-bit integer type; a group stream of
 // slabs * 4 KiB must fit the 31-bit extent of a buffer resource, the dimensions 31 bits)
 size_t wk::gemm_int_packed_workspace_bytes(int dtype, uint64_t M, uint64_t N, uint64_t K) {
+    if (dtype == WK_I64 || dtype == WK_U64) return gemm_i64_packed_workspace_bytes(M, N, K);
     const int digits = digits_of(dtype);
     if (!digits || !M || !N || !K || M > 0x7fffffffull || N > 0x7fffffffull) return 0;
     if (K > (0x7fffffffull / GROUP_BYTES - 1) * BK * (4 / digits)) return 0;
@@ -1179,6 +1180,7 @@ size_t wk::gemm_int_packed_workspace_bytes(int dtype, uint64_t M, uint64_t N, ui
 }
 
 int wk::gemm_int_packed_launch(hipStream_t st, const GemmProblem &p, void *workspace, size_t workspace_bytes) {
+    if (p.dtype == WK_I64 || p.dtype == WK_U64) return gemm_i64_packed_launch(st, p, workspace, workspace_bytes);
     const size_t need = gemm_int_packed_workspace_bytes(p.dtype, p.M, p.N, p.K);
     if (!need || !workspace || workspace_bytes < need || (reinterpret_cast<uintptr_t>(workspace) & 15u)) return WK_E_INVALID_VALUE;
     // 32-bit extents and leading dimensions inside the pack pass and the product kernel

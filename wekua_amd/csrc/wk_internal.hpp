@@ -226,6 +226,9 @@ int gemm_i32_mfma_launch_128(hipStream_t st, const GemmProblem &p, bool edge); /
 // 8/16/32-bit integers with a pack pass into caller-provided workspace (wk_gemm_ipack.hip)
 size_t gemm_int_packed_workspace_bytes(int dtype, uint64_t M, uint64_t N, uint64_t K); // 0: not applicable
 int gemm_int_packed_launch(hipStream_t st, const GemmProblem &p, void *workspace, size_t workspace_bytes);
+// 64-bit integers the same way: eight digit planes, 36 digit products (wk_gemm_i64pack.hip)
+size_t gemm_i64_packed_workspace_bytes(uint64_t M, uint64_t N, uint64_t K); // 0: not applicable
+int gemm_i64_packed_launch(hipStream_t st, const GemmProblem &p, void *workspace, size_t workspace_bytes);
 constexpr int WK_CF32 = WK_COMPLEX + WK_F32, WK_CF64 = WK_COMPLEX + WK_F64;
 // cf32 / cf64 and the complex 8/16/32-bit integers through the real matrix-core kernels, operands
 // rebuilt in caller-provided workspace (wk_gemm_cpack.hip)
