@@ -91,6 +91,54 @@ def test_f32_every_variant(dev, variant, op_a, op_b):
         dev.lib.wk_gemm_force_variant(b"auto")
 
 
+@pytest.mark.parametrize("variant", ["mfma_f32_256x128d", "mfma_f32_128x128d", "mfma_f32_64x64d", "mfma_f64_128x128d", "mfma_f64_64x64d"])
+@pytest.mark.parametrize("op_a,op_b", OPS)
+def test_direct_to_lds_with_rows_that_start_anywhere(dev, variant, op_a, op_b):
+    """The direct-to-LDS kernels on operands whose rows do not start on 16-byte boundaries (leading dimensions
+    that are not multiples of 16 bytes, bases one to three elements into an allocation): four bytes per lane and
+    load instead of sixteen.  Several k-slabs with a ragged last one, ragged tiles, poisoned gaps between the rows
+    and around the operands, so that a float fetched from the wrong place or a write outside C shows."""
+    import ctypes
+    from wekua_amd import raw
+    dtype = variant[5:8]
+    rd = np.float32 if dtype == "f32" else np.float64
+    es = np.dtype(rd).itemsize
+    poison = rd(7.0e37)
+    assert dev.lib.wk_gemm_force_variant(variant.encode()) == 0
+    try:
+        for (M, N, K), (pa, pb), (sa, sb) in [((300, 200, 100), (1, 3), (1, 2)), ((257, 129, 77), (3, 2), (3, 0)),
+                                              ((512, 384, 256), (5, 7), (0, 1)), ((130, 70, 37), (0, 1), (2, 3))]:
+            a, b, c = gemm_operands(dtype, M, N, K, op_a, op_b, 91)
+            lda, ldb, ldc = a.shape[1] + pa, b.shape[1] + pb, N + 3
+
+            def device_copy(m, ld, shift):
+                # rows of ld floats, the whole thing `shift` floats into its allocation, everything else poisoned
+                flat = np.full(shift + m.shape[0] * ld + 8, poison, dtype=rd)
+                view = flat[shift:shift + m.shape[0] * ld].reshape(m.shape[0], ld)
+                view[:, :m.shape[1]] = m
+                return dev.upload(flat), flat
+
+            (dA, _), (dB, _), (dC, c_flat) = device_copy(a, lda, sa), device_copy(b, ldb, sb), device_copy(c, ldc, 1)
+            ptr = lambda buf, shift: ctypes.c_void_p(buf.ptr.value + es * shift)
+            name = dev.lib.wk_gemm_variant(raw.dtype_id(dtype), op_a, op_b, M, N, K, lda, ldb, ldc, ptr(dA, sa), ptr(dB, sb), ptr(dC, 1))
+            assert name == variant.encode()
+            alpha, beta = raw.scalar_bytes(dtype, 1.5), raw.scalar_bytes(dtype, 0.5)
+            raw.check(dev.lib.wk_gemm(dev.stream, raw.dtype_id(dtype), op_a, op_b, M, N, K, ctypes.cast(alpha, ctypes.c_void_p),
+                                      ptr(dA, sa), lda, ptr(dB, sb), ldb, ctypes.cast(beta, ctypes.c_void_p), ptr(dC, 1), ldc, None, 0),
+                      "wk_gemm")
+            dev.sync()
+            out = dC.download(rd, c_flat.shape)
+            got = out[1:1 + M * ldc].reshape(M, ldc)
+            assert (got[:, N:] == poison).all() and out[0] == poison and (out[1 + M * ldc:] == poison).all()
+            want = oracle.gemm(dtype, 1.5, a, op_a, b, op_b, 0.5, c)
+            assert_gemm_close(dtype, np.ascontiguousarray(got[:, :N]), want, 1.5, a, op_a, b, op_b, 0.5, c, K,
+                              what=f"{variant} {M}x{N}x{K} op=({op_a},{op_b}) lda={lda} ldb={ldb} shifts={sa},{sb}")
+            for d in (dA, dB, dC):
+                d.free()
+    finally:
+        dev.lib.wk_gemm_force_variant(b"auto")
+
+
 @pytest.mark.parametrize("variant", ["tile64", "mfma_f64_64x64", "mfma_f64_64x64s2", "mfma_f64_32x32s4", "mfma_f64_64x64z",
                                      "mfma_f64_128x64", "mfma_f64_128x128", "mfma_f64_128x128d", "mfma_f64_64x64d"])
 @pytest.mark.parametrize("op_a,op_b", OPS)
@@ -448,16 +496,16 @@ def test_one_round_launches_take_the_k_split_tiles(dev):
     assert name("f32", 2040, 2040, 2040) == b"mfma_f32_128x128d2"
     assert name("f32", 2048, 2048, 512) == b"mfma_f32_128x128d"
     assert dev.lib.wk_gemm_variant(raw.dtype_id("f32"), 1, 0, 1024, 1024, 1024, 1024, 1024, 1024, None, None, None) == b"mfma_f32_64x64d"  # T,N
-    # ... any other leading dimension the register-staged tile and its k-split twins
-    assert name("f32", 1001, 1001, 1001) == b"mfma_f32_64x64s4"
-    assert name("f32", 2041, 1001, 1001) == b"mfma_f32_64x64s2"
-    assert name("f32", 1001, 1001, 101) == b"mfma_f32_64x64"
-    assert name("f32", 2042, 2042, 2042) == b"mfma_f32_128x128s2"
+    # ... any other leading dimension the same kernels with four bytes per lane and load, one group of wavefronts
+    assert name("f32", 1001, 1001, 1001) == b"mfma_f32_64x64d"
+    assert name("f32", 2041, 1001, 1001) == b"mfma_f32_64x64d"
+    assert name("f32", 1001, 1001, 101) == b"mfma_f32_64x64d"
+    assert name("f32", 2042, 2042, 2042) == b"mfma_f32_128x128d"
     assert name("f32", 512, 512, 512) == b"mfma_f32_32x32s4"       # 64 tiles of 64x64 would leave most CUs idle
     assert name("f32", 768, 768, 768) == b"mfma_f32_32x32s4"
     assert name("f64", 1024, 1024, 1024) == b"mfma_f64_64x64d"
     assert name("f64", 1000, 1000, 1000) == b"mfma_f64_64x64d"
-    assert name("f64", 1001, 1001, 1001) == b"mfma_f64_64x64s2"   # rows of 8008 bytes: the register-staged tile
+    assert name("f64", 1001, 1001, 1001) == b"mfma_f64_64x64d"    # rows of 8008 bytes: four-byte loads
     assert name("f64", 2048, 2048, 2048) == b"mfma_f64_64x64d"
     assert name("f64", 4096, 4096, 4096) == b"mfma_f64_128x128d"
     assert name("f64", 512, 512, 512) == b"mfma_f64_32x32s4"
@@ -919,4 +967,4 @@ def test_seeded_random_mid_size_problems(dev, dtype):
         seen.add(dev.lib.wk_gemm_variant(raw.dtype_id(dtype), op_a, op_b, M, N, K, M if op_a else K, K if op_b else N, N, None, None,
                                          None))
         check(dev, dtype, M, N, K, op_a, op_b, alpha, beta, seed=700 + case)
-    assert len(seen) >= 3, seen
+    assert len(seen) >= 2, seen

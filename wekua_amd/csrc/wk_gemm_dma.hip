@@ -61,9 +61,14 @@ struct DArgs {
 // a single wavefront, which stands still at every wait; with KS = 2 all eight wavefronts bring the slabs
 // in, group kg multiplies steps kg * S / KS ... of every slab, and the two partial tiles are added
 // through LDS (the stages, free by then) before group 0 runs the epilogue.
-template <int BM, int BN, int BK, int NS, int OCC, bool A_K, bool B_K, bool EXT, int KS = 1>
+// VB: bytes per lane and load.  16 for operands whose rows start on 16-byte boundaries; 4 for any other (every
+// lane then fetches one float into the same place of the same LDS layout: SUB = 4 loads per KiB instead of one,
+// nothing read beyond the end of a row).
+template <int BM, int BN, int BK, int NS, int OCC, bool A_K, bool B_K, bool EXT, int KS = 1, int VB = 16>
 __global__ __launch_bounds__(256 * KS) __attribute__((amdgpu_waves_per_eu(OCC)))
 void gemm_f32_dma_kernel(DArgs g) {
+    static_assert(VB == 16 || VB == 4, "bytes per lane");
+    constexpr int SUB = 16 / VB;
     constexpr int WM = BM / 2, WN = BN / 2, FM = WM / 32, FN = WN / 32;
     constexpr int S = BK / 8;   // fragment steps per slab (8 values of k each: four matrix instructions per block)
     constexpr int CPR = BK / 4; // 16-byte chunks per row of a k-contiguous slab
@@ -122,33 +127,50 @@ void gemm_f32_dma_kernel(DArgs g) {
     const float *b_base = B_K ? g.B + (size_t)n0 * g.ldb : g.B + n0;
     const size_t a_step = A_K ? (size_t)BK : (size_t)BK * g.lda; // floats per slab
     const size_t b_step = B_K ? (size_t)BK : (size_t)BK * g.ldb;
-    uint32_t a_off[A_LOADS], b_off[B_LOADS];
-    // load i of this wavefront fills the 1 KB group i * 4 + wave of the operand's slab: sixteen rows of a
+    uint32_t a_off[A_LOADS * SUB], b_off[B_LOADS * SUB];
+    // loads i * SUB ... of this wavefront fill the 1 KB group i * 4 + wave of the operand's slab: sixteen rows of a
     // k-contiguous operand, 256 / ROWS rows of k of an m-contiguous one
     // Rows (columns) of the tile beyond the matrix are fetched from its last row (column): they only feed
     // entries of C that are never stored.  A 16-byte chunk whose first float exists is fetched as it is:
     // bases and leading dimensions are multiples of 16 bytes, so the chunk cannot leave the page of
     // that float.  `last` = index of the last existing row (column) counted from the tile's origin.
-    auto lane_offset = [&](int grp, uint32_t ld, uint32_t last, auto kc_tag, auto rows_tag) -> uint32_t {
+    // With one float per lane (VB = 4) lane l of load q of a group fetches the float that belongs at float
+    // 64 q + l of the group.
+    auto lane_offset = [&](int grp, int q, uint32_t ld, uint32_t last, auto kc_tag, auto rows_tag) -> uint32_t {
         constexpr bool KC = decltype(kc_tag)::value;
         constexpr int ROWS = decltype(rows_tag)::value;
-        if constexpr (KC) {
-            const uint32_t row = grp * (64 / CPR) + lane / CPR;
-            const uint32_t chunk = (lane % CPR) ^ swizzle(row);
-            return (min(row, last) * ld + 4 * chunk) * 4u;
+        if constexpr (VB == 16) {
+            if constexpr (KC) {
+                const uint32_t row = grp * (64 / CPR) + lane / CPR;
+                const uint32_t chunk = (lane % CPR) ^ swizzle(row);
+                return (min(row, last) * ld + 4 * chunk) * 4u;
+            } else {
+                constexpr int PER_ROW = ROWS / 4; // 16-byte chunks per row of k
+                const uint32_t k = grp * (64 / PER_ROW) + lane / PER_ROW;
+                const uint32_t chunk = (lane % PER_ROW) ^ (((k >> 2) & 1) * 8);
+                return (k * ld + 4 * min(chunk, last >> 2)) * 4u;
+            }
         } else {
-            constexpr int PER_ROW = ROWS / 4; // 16-byte chunks per row of k
-            const uint32_t k = grp * (64 / PER_ROW) + lane / PER_ROW;
-            const uint32_t chunk = (lane % PER_ROW) ^ (((k >> 2) & 1) * 8);
-            return (k * ld + 4 * min(chunk, last >> 2)) * 4u;
+            const uint32_t f = 64 * q + lane; // float of the group
+            if constexpr (KC) {
+                const uint32_t row = grp * (256 / BK) + f / BK, pos = f % BK;
+                const uint32_t chunk = (pos >> 2) ^ swizzle(row);
+                return (min(row, last) * ld + 4 * chunk + (pos & 3)) * 4u;
+            } else {
+                const uint32_t k = grp * (256 / ROWS) + f / ROWS;
+                const uint32_t m = (f % ROWS) ^ (((k >> 2) & 1) * 32);
+                return (k * ld + min(m, last)) * 4u;
+            }
         }
     };
     using std::integral_constant;
     const uint32_t m_last = g.M - 1 - m0, n_last = g.N - 1 - n0;
 #pragma unroll
-    for (int i = 0; i < A_LOADS; ++i) a_off[i] = lane_offset(i * WAVES + wave, g.lda, m_last, integral_constant<bool, A_K>{}, integral_constant<int, BM>{});
+    for (int i = 0; i < A_LOADS * SUB; ++i)
+        a_off[i] = lane_offset((i / SUB) * WAVES + wave, i % SUB, g.lda, m_last, integral_constant<bool, A_K>{}, integral_constant<int, BM>{});
 #pragma unroll
-    for (int i = 0; i < B_LOADS; ++i) b_off[i] = lane_offset(i * WAVES + wave, g.ldb, n_last, integral_constant<bool, B_K>{}, integral_constant<int, BN>{});
+    for (int i = 0; i < B_LOADS * SUB; ++i)
+        b_off[i] = lane_offset((i / SUB) * WAVES + wave, i % SUB, g.ldb, n_last, integral_constant<bool, B_K>{}, integral_constant<int, BN>{});
     const uint32_t lds0 =
         __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)(__attribute__((address_space(3))) float *)lds); // byte address of the array
 
@@ -156,10 +178,19 @@ void gemm_f32_dma_kernel(DArgs g) {
     // the slab after it
     auto issue = [&](uint32_t stage_bytes) {
         const uint32_t sbase = lds0 + stage_bytes + (uint32_t)wave * 1024u;
+        if constexpr (VB == 16) {
 #pragma unroll
-        for (int i = 0; i < A_LOADS; ++i) dma16(a_base, a_off[i], sbase + (uint32_t)i * (WAVES * 1024u));
+            for (int i = 0; i < A_LOADS; ++i) dma16(a_base, a_off[i], sbase + (uint32_t)i * (WAVES * 1024u));
 #pragma unroll
-        for (int i = 0; i < B_LOADS; ++i) dma16(b_base, b_off[i], sbase + A_FLOATS * 4u + (uint32_t)i * (WAVES * 1024u));
+            for (int i = 0; i < B_LOADS; ++i) dma16(b_base, b_off[i], sbase + A_FLOATS * 4u + (uint32_t)i * (WAVES * 1024u));
+        } else {
+#pragma unroll
+            for (int i = 0; i < A_LOADS * SUB; ++i)
+                dma4(a_base, a_off[i], sbase + (uint32_t)(i / SUB) * (WAVES * 1024u) + (uint32_t)(i % SUB) * 256u);
+#pragma unroll
+            for (int i = 0; i < B_LOADS * SUB; ++i)
+                dma4(b_base, b_off[i], sbase + A_FLOATS * 4u + (uint32_t)(i / SUB) * (WAVES * 1024u) + (uint32_t)(i % SUB) * 256u);
+        }
         a_base += a_step;
         b_base += b_step;
     };
@@ -169,10 +200,25 @@ void gemm_f32_dma_kernel(DArgs g) {
     // the last existing one instead; once a wavefront's own loads of that slab have landed it writes
     // zeros over every float of its share whose k does not exist (products with them must vanish).
     const uint32_t krem = g.K % BK;
-    auto tail_offset = [&](uint32_t off, int grp, uint32_t ld, auto kc_tag, auto rows_tag) -> uint32_t {
+    // k of the float that lane `lane` of load q of group grp fetches with one float per lane (VB = 4)
+    auto k_of_float = [&](int grp, int q, auto kc_tag, auto rows_tag) -> uint32_t {
         constexpr bool KC = decltype(kc_tag)::value;
         constexpr int ROWS = decltype(rows_tag)::value;
+        const uint32_t f = 64 * q + lane;
         if constexpr (KC) {
+            const uint32_t row = grp * (256 / BK) + f / BK, pos = f % BK;
+            return 4 * ((pos >> 2) ^ swizzle(row)) + (pos & 3);
+        } else {
+            return grp * (256 / ROWS) + f / ROWS;
+        }
+    };
+    auto tail_offset = [&](uint32_t off, int grp, int q, uint32_t ld, auto kc_tag, auto rows_tag) -> uint32_t {
+        constexpr bool KC = decltype(kc_tag)::value;
+        constexpr int ROWS = decltype(rows_tag)::value;
+        if constexpr (VB == 4) { // a float whose k does not exist: the last existing one of its row (column) instead
+            const uint32_t k = k_of_float(grp, q, kc_tag, rows_tag);
+            return k >= krem ? off - (k - (krem - 1)) * (KC ? 1u : ld) * 4u : off;
+        } else if constexpr (KC) {
             const uint32_t row = grp * (64 / CPR) + lane / CPR;
             const uint32_t chunk = (lane % CPR) ^ swizzle(row);
             return 4 * chunk >= krem ? off - 16u * chunk : off; // chunk 0 of the row always has a float (krem >= 1)
@@ -184,14 +230,18 @@ void gemm_f32_dma_kernel(DArgs g) {
     };
     auto tail_offsets = [&]() {
 #pragma unroll
-        for (int i = 0; i < A_LOADS; ++i) a_off[i] = tail_offset(a_off[i], i * WAVES + wave, g.lda, integral_constant<bool, A_K>{}, integral_constant<int, BM>{});
+        for (int i = 0; i < A_LOADS * SUB; ++i)
+            a_off[i] = tail_offset(a_off[i], (i / SUB) * WAVES + wave, i % SUB, g.lda, integral_constant<bool, A_K>{}, integral_constant<int, BM>{});
 #pragma unroll
-        for (int i = 0; i < B_LOADS; ++i) b_off[i] = tail_offset(b_off[i], i * WAVES + wave, g.ldb, integral_constant<bool, B_K>{}, integral_constant<int, BN>{});
+        for (int i = 0; i < B_LOADS * SUB; ++i)
+            b_off[i] = tail_offset(b_off[i], (i / SUB) * WAVES + wave, i % SUB, g.ldb, integral_constant<bool, B_K>{}, integral_constant<int, BN>{});
     };
-    auto tail_zero = [&](float *dst, int grp, auto kc_tag, auto rows_tag) { // dst: this lane's 16 bytes of the load
+    auto tail_zero = [&](float *dst, int grp, int q, auto kc_tag, auto rows_tag) { // dst: this lane's bytes of the load
         constexpr bool KC = decltype(kc_tag)::value;
         constexpr int ROWS = decltype(rows_tag)::value;
-        if constexpr (KC) {
+        if constexpr (VB == 4) {
+            if (k_of_float(grp, q, kc_tag, rows_tag) >= krem) dst[0] = 0.f;
+        } else if constexpr (KC) {
             const uint32_t row = grp * (64 / CPR) + lane / CPR;
             const uint32_t chunk = (lane % CPR) ^ swizzle(row);
 #pragma unroll
@@ -204,11 +254,15 @@ void gemm_f32_dma_kernel(DArgs g) {
         }
     };
     auto tail_zeros = [&](uint32_t stage_bytes) {
-        float *base = lds + stage_bytes / 4 + wave * 256 + lane * 4;
+        float *base = lds + stage_bytes / 4 + wave * 256 + lane * (VB / 4);
 #pragma unroll
-        for (int i = 0; i < A_LOADS; ++i) tail_zero(base + i * (WAVES * 256), i * WAVES + wave, integral_constant<bool, A_K>{}, integral_constant<int, BM>{});
+        for (int i = 0; i < A_LOADS * SUB; ++i)
+            tail_zero(base + (i / SUB) * (WAVES * 256) + (i % SUB) * 64, (i / SUB) * WAVES + wave, i % SUB, integral_constant<bool, A_K>{},
+                      integral_constant<int, BM>{});
 #pragma unroll
-        for (int i = 0; i < B_LOADS; ++i) tail_zero(base + A_FLOATS + i * (WAVES * 256), i * WAVES + wave, integral_constant<bool, B_K>{}, integral_constant<int, BN>{});
+        for (int i = 0; i < B_LOADS * SUB; ++i)
+            tail_zero(base + A_FLOATS + (i / SUB) * (WAVES * 256) + (i % SUB) * 64, (i / SUB) * WAVES + wave, i % SUB,
+                      integral_constant<bool, B_K>{}, integral_constant<int, BN>{});
     };
 
     // ---- LDS side: per-lane fragment addresses (floats from the start of a stage's A or B part) ----
@@ -292,7 +346,8 @@ void gemm_f32_dma_kernel(DArgs g) {
     // The NS stages rotate (byte offsets): st[0] holds the slab being multiplied, st[1] the next one, ...,
     // st[NS - 1] is the stage the slab before left, into which slab kt + NS - 1 is requested.
     constexpr uint32_t STAGE_BYTES = STAGE * 4u;
-    constexpr int LOADS = A_LOADS + B_LOADS; // per wavefront and slab
+    constexpr int LOADS = (A_LOADS + B_LOADS) * SUB; // per wavefront and slab
+    static_assert(LOADS * (NS - 1) <= 63 || VB == 4, "the wait counter holds 63 loads");
     uint32_t st[NS];
 #pragma unroll
     for (int n = 0; n < NS; ++n) st[n] = n * STAGE_BYTES;
@@ -484,10 +539,14 @@ struct DArgsD {
 };
 
 
-template <int BM, int BN, int BK, int NS, int OCC, bool A_K, bool B_K, bool EXT>
+// VB as in the f32 kernel: 16 bytes per lane and load for rows that start on 16-byte boundaries, 4 (half a
+// double) for any other.
+template <int BM, int BN, int BK, int NS, int OCC, bool A_K, bool B_K, bool EXT, int VB = 16>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(OCC)))
 void gemm_f64_dma_kernel(DArgsD g) {
     static_assert(NS == 2 || NS == 3, "stages");
+    static_assert(VB == 16 || VB == 4, "bytes per lane");
+    constexpr int SUB = 16 / VB;
     constexpr int WM = BM / 2, WN = BN / 2, FM = WM / 16, FN = WN / 16;
     constexpr int S = BK / 8;     // fragment steps per slab (8 values of k each, two matrix instructions per block)
     constexpr int CPR = BK / 2;   // 16-byte chunks per row of a k-contiguous slab
@@ -537,11 +596,30 @@ void gemm_f64_dma_kernel(DArgsD g) {
     const double *b_base = B_K ? g.B + (size_t)n0 * g.ldb : g.B + n0;
     const size_t a_step = A_K ? (size_t)BK : (size_t)BK * g.lda;
     const size_t b_step = B_K ? (size_t)BK : (size_t)BK * g.ldb;
-    uint32_t a_off[A_LOADS], b_off[B_LOADS];
-    auto lane_offset = [&](int grp, uint32_t ld, uint32_t last, auto kc_tag, auto rows_tag) -> uint32_t {
+    uint32_t a_off[A_LOADS * SUB], b_off[B_LOADS * SUB];
+    // (k, row or column) of the double that lane `lane` of load q of group grp fetches half of with four bytes
+    // per lane: the double that belongs at double 32 q + lane / 2 of the group
+    auto double_of = [&](int grp, int q, uint32_t &k, uint32_t &r, auto kc_tag, auto rows_tag) {
         constexpr bool KC = decltype(kc_tag)::value;
         constexpr int ROWS = decltype(rows_tag)::value;
+        const uint32_t f = 32 * q + (lane >> 1);
         if constexpr (KC) {
+            r = grp * (128 / BK) + f / BK;
+            const uint32_t pos = f % BK;
+            k = 2 * ((pos >> 1) ^ ((r >> 1) & 7)) + (pos & 1);
+        } else {
+            k = grp * (128 / ROWS) + f / ROWS;
+            r = (f % ROWS) ^ (((k >> 1) & 1) * 16);
+        }
+    };
+    auto lane_offset = [&](int grp, int q, uint32_t ld, uint32_t last, auto kc_tag, auto rows_tag) -> uint32_t {
+        constexpr bool KC = decltype(kc_tag)::value;
+        constexpr int ROWS = decltype(rows_tag)::value;
+        if constexpr (VB == 4) {
+            uint32_t k, r;
+            double_of(grp, q, k, r, kc_tag, rows_tag);
+            return (KC ? min(r, last) * ld + k : k * ld + min(r, last)) * 8u + 4u * (lane & 1);
+        } else if constexpr (KC) {
             constexpr int RPL = 64 / CPR; // rows per load
             const uint32_t row = grp * RPL + lane / CPR;
             const uint32_t swz = (row >> 1) & 7;
@@ -558,18 +636,28 @@ void gemm_f64_dma_kernel(DArgsD g) {
     using std::integral_constant;
     const uint32_t m_last = g.M - 1 - m0, n_last = g.N - 1 - n0;
 #pragma unroll
-    for (int i = 0; i < A_LOADS; ++i) a_off[i] = lane_offset(i * 4 + wave, g.lda, m_last, integral_constant<bool, A_K>{}, integral_constant<int, BM>{});
+    for (int i = 0; i < A_LOADS * SUB; ++i)
+        a_off[i] = lane_offset((i / SUB) * 4 + wave, i % SUB, g.lda, m_last, integral_constant<bool, A_K>{}, integral_constant<int, BM>{});
 #pragma unroll
-    for (int i = 0; i < B_LOADS; ++i) b_off[i] = lane_offset(i * 4 + wave, g.ldb, n_last, integral_constant<bool, B_K>{}, integral_constant<int, BN>{});
+    for (int i = 0; i < B_LOADS * SUB; ++i)
+        b_off[i] = lane_offset((i / SUB) * 4 + wave, i % SUB, g.ldb, n_last, integral_constant<bool, B_K>{}, integral_constant<int, BN>{});
     const uint32_t lds0 =
         __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)(__attribute__((address_space(3))) float *)lds_f);
 
     auto issue = [&](uint32_t stage_bytes) {
         const uint32_t sbase = lds0 + stage_bytes + (uint32_t)wave * 1024u;
+        if constexpr (VB == 16) {
 #pragma unroll
-        for (int i = 0; i < A_LOADS; ++i) dma16(a_base, a_off[i], sbase + (uint32_t)i * 4096u);
+            for (int i = 0; i < A_LOADS; ++i) dma16(a_base, a_off[i], sbase + (uint32_t)i * 4096u);
 #pragma unroll
-        for (int i = 0; i < B_LOADS; ++i) dma16(b_base, b_off[i], sbase + A_DOUBLES * 8u + (uint32_t)i * 4096u);
+            for (int i = 0; i < B_LOADS; ++i) dma16(b_base, b_off[i], sbase + A_DOUBLES * 8u + (uint32_t)i * 4096u);
+        } else {
+#pragma unroll
+            for (int i = 0; i < A_LOADS * SUB; ++i) dma4(a_base, a_off[i], sbase + (uint32_t)(i / SUB) * 4096u + (uint32_t)(i % SUB) * 256u);
+#pragma unroll
+            for (int i = 0; i < B_LOADS * SUB; ++i)
+                dma4(b_base, b_off[i], sbase + A_DOUBLES * 8u + (uint32_t)(i / SUB) * 4096u + (uint32_t)(i % SUB) * 256u);
+        }
         a_base += a_step;
         b_base += b_step;
     };
@@ -578,10 +666,14 @@ void gemm_f64_dma_kernel(DArgsD g) {
     // of k wholly beyond K are fetched from the last existing one, and the wavefront that loaded a share of
     // that slab writes zeros over its doubles whose k does not exist once the loads have landed ----
     const uint32_t krem = g.K % BK;
-    auto tail_offset = [&](uint32_t off, int grp, uint32_t ld, auto kc_tag, auto rows_tag) -> uint32_t {
+    auto tail_offset = [&](uint32_t off, int grp, int q, uint32_t ld, auto kc_tag, auto rows_tag) -> uint32_t {
         constexpr bool KC = decltype(kc_tag)::value;
         constexpr int ROWS = decltype(rows_tag)::value;
-        if constexpr (KC) {
+        if constexpr (VB == 4) { // a double whose k does not exist: the last existing one of its row (column) instead
+            uint32_t k, r;
+            double_of(grp, q, k, r, kc_tag, rows_tag);
+            return k >= krem ? off - (k - (krem - 1)) * (KC ? 1u : ld) * 8u : off;
+        } else if constexpr (KC) {
             const uint32_t row = grp * (64 / CPR) + lane / CPR;
             const uint32_t chunk = (lane % CPR) ^ ((row >> 1) & 7);
             return 2 * chunk >= krem ? off - 16u * chunk : off; // chunk 0 of the row always has a double (krem >= 1)
@@ -593,19 +685,25 @@ void gemm_f64_dma_kernel(DArgsD g) {
     };
     auto tail_offsets = [&]() {
 #pragma unroll
-        for (int i = 0; i < A_LOADS; ++i) a_off[i] = tail_offset(a_off[i], i * 4 + wave, g.lda, integral_constant<bool, A_K>{}, integral_constant<int, BM>{});
+        for (int i = 0; i < A_LOADS * SUB; ++i)
+            a_off[i] = tail_offset(a_off[i], (i / SUB) * 4 + wave, i % SUB, g.lda, integral_constant<bool, A_K>{}, integral_constant<int, BM>{});
 #pragma unroll
-        for (int i = 0; i < B_LOADS; ++i) b_off[i] = tail_offset(b_off[i], i * 4 + wave, g.ldb, integral_constant<bool, B_K>{}, integral_constant<int, BN>{});
+        for (int i = 0; i < B_LOADS * SUB; ++i)
+            b_off[i] = tail_offset(b_off[i], (i / SUB) * 4 + wave, i % SUB, g.ldb, integral_constant<bool, B_K>{}, integral_constant<int, BN>{});
     };
-    auto tail_zero = [&](double *dst, int grp, auto kc_tag, auto rows_tag) { // dst: this lane's 16 bytes of the load
+    auto tail_zero = [&](float *dst, int grp, int q, auto kc_tag, auto rows_tag) { // dst: this lane's bytes of the load
         constexpr bool KC = decltype(kc_tag)::value;
         constexpr int ROWS = decltype(rows_tag)::value;
-        if constexpr (KC) {
+        if constexpr (VB == 4) {
+            uint32_t k, r;
+            double_of(grp, q, k, r, kc_tag, rows_tag);
+            if (k >= krem) dst[0] = 0.f; // (its half of the double)
+        } else if constexpr (KC) {
             const uint32_t row = grp * (64 / CPR) + lane / CPR;
             const uint32_t chunk = (lane % CPR) ^ ((row >> 1) & 7);
 #pragma unroll
             for (int e = 0; e < 2; ++e)
-                if (2 * chunk + e >= krem) dst[e] = 0.0;
+                if (2 * chunk + e >= krem) reinterpret_cast<double *>(dst)[e] = 0.0;
         } else {
             constexpr int PER_ROW = ROWS / 2;
             const uint32_t k = grp * (64 / PER_ROW) + lane / PER_ROW;
@@ -613,11 +711,15 @@ void gemm_f64_dma_kernel(DArgsD g) {
         }
     };
     auto tail_zeros = [&](uint32_t stage_bytes) {
-        double *base = lds + stage_bytes / 8 + wave * 128 + lane * 2;
+        float *base = lds_f + stage_bytes / 4 + wave * 256 + lane * (VB / 4);
 #pragma unroll
-        for (int i = 0; i < A_LOADS; ++i) tail_zero(base + i * 512, i * 4 + wave, integral_constant<bool, A_K>{}, integral_constant<int, BM>{});
+        for (int i = 0; i < A_LOADS * SUB; ++i)
+            tail_zero(base + (i / SUB) * 1024 + (i % SUB) * 64, (i / SUB) * 4 + wave, i % SUB, integral_constant<bool, A_K>{},
+                      integral_constant<int, BM>{});
 #pragma unroll
-        for (int i = 0; i < B_LOADS; ++i) tail_zero(base + A_DOUBLES + i * 512, i * 4 + wave, integral_constant<bool, B_K>{}, integral_constant<int, BN>{});
+        for (int i = 0; i < B_LOADS * SUB; ++i)
+            tail_zero(base + A_DOUBLES * 2 + (i / SUB) * 1024 + (i % SUB) * 64, (i / SUB) * 4 + wave, i % SUB,
+                      integral_constant<bool, B_K>{}, integral_constant<int, BN>{});
     };
 
     // ---- LDS side: per-lane fragment addresses in doubles from the start of a stage's A or B part ----
@@ -679,7 +781,7 @@ void gemm_f64_dma_kernel(DArgsD g) {
     // (see there): st[0] holds the slab being multiplied, slab kt + NS - 1 goes into st[NS - 1].
     const uint32_t ktiles = (g.K + BK - 1) / BK;
     constexpr uint32_t STAGE_BYTES = STAGE * 8u;
-    constexpr int LOADS = A_LOADS + B_LOADS;
+    constexpr int LOADS = (A_LOADS + B_LOADS) * SUB;
     uint32_t st[NS];
 #pragma unroll
     for (int n = 0; n < NS; ++n) st[n] = n * STAGE_BYTES;
@@ -783,9 +885,9 @@ void gemm_f64_dma_kernel(DArgsD g) {
     else epilogue(std::true_type{});
 }
 
-template <int BM, int BN, int BK, int NS, int OCC, bool A_K, bool B_K, bool EXT> int launch_one_d(hipStream_t st, const DArgsD &g) {
+template <int BM, int BN, int BK, int NS, int OCC, bool A_K, bool B_K, bool EXT, int VB = 16> int launch_one_d(hipStream_t st, const DArgsD &g) {
     constexpr size_t lds_bytes = NS * (BM * BK + BN * BK) * sizeof(double);
-    auto kern = gemm_f64_dma_kernel<BM, BN, BK, NS, OCC, A_K, B_K, EXT>;
+    auto kern = gemm_f64_dma_kernel<BM, BN, BK, NS, OCC, A_K, B_K, EXT, VB>;
     static const int attr_rc = [&] {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
                                            (int)lds_bytes);
@@ -800,7 +902,7 @@ template <int BM, int BN, int BK, int NS, int OCC, bool A_K, bool B_K, bool EXT>
     return launch_status();
 }
 
-template <int BM, int BN, int BK, int NS, int OCC> int launch_tile_d(hipStream_t st, const GemmProblem &p) {
+template <int BM, int BN, int BK, int NS, int OCC, int VB = 16> int launch_tile_d(hipStream_t st, const GemmProblem &p) {
     DArgsD g{};
     g.A = static_cast<const double *>(p.A);
     g.B = static_cast<const double *>(p.B);
@@ -826,19 +928,27 @@ template <int BM, int BN, int BK, int NS, int OCC> int launch_tile_d(hipStream_t
             }
     }
     const int sel = (p.op_a ? 0 : 2) | (p.op_b ? 1 : 0);
-    if (p.ext) return sel == 3 ? launch_one_d<BM, BN, BK, NS, OCC, true, true, true>(st, g) : (int)WK_E_INVALID_VALUE;
+    if (p.ext) {
+        if constexpr (VB == 16) return sel == 3 ? launch_one_d<BM, BN, BK, NS, OCC, true, true, true>(st, g) : (int)WK_E_INVALID_VALUE;
+        else return WK_E_INVALID_VALUE;
+    }
     switch (sel) {
-    case 0: return launch_one_d<BM, BN, BK, NS, OCC, false, false, false>(st, g);
-    case 1: return launch_one_d<BM, BN, BK, NS, OCC, false, true, false>(st, g);
-    case 2: return launch_one_d<BM, BN, BK, NS, OCC, true, false, false>(st, g);
-    default: return launch_one_d<BM, BN, BK, NS, OCC, true, true, false>(st, g);
+    case 0: return launch_one_d<BM, BN, BK, NS, OCC, false, false, false, VB>(st, g);
+    case 1: return launch_one_d<BM, BN, BK, NS, OCC, false, true, false, VB>(st, g);
+    case 2: return launch_one_d<BM, BN, BK, NS, OCC, true, false, false, VB>(st, g);
+    default: return launch_one_d<BM, BN, BK, NS, OCC, true, true, false, VB>(st, g);
     }
 }
 
+bool f64_rows_aligned(const GemmProblem &p) {
+    return p.lda % 2 == 0 && p.ldb % 2 == 0 && ((reinterpret_cast<uintptr_t>(p.A) | reinterpret_cast<uintptr_t>(p.B)) & 15u) == 0;
+}
+
 // first_tiles: launch only that many tiles, in tile-walk order (0: all of them)
-template <int BM, int BN, int BK, int NS, int OCC, bool A_K, bool B_K, bool EXT, int KS = 1> int launch_one(hipStream_t st, const DArgs &g, uint64_t first_tiles) {
+template <int BM, int BN, int BK, int NS, int OCC, bool A_K, bool B_K, bool EXT, int KS = 1, int VB = 16>
+int launch_one(hipStream_t st, const DArgs &g, uint64_t first_tiles) {
     constexpr size_t lds_bytes = NS * (BM * BK + BN * BK) * sizeof(float); // 3 x 24 KB / 3 x 16 KB / 3 x 32 KB
-    auto kern = gemm_f32_dma_kernel<BM, BN, BK, NS, OCC, A_K, B_K, EXT, KS>;
+    auto kern = gemm_f32_dma_kernel<BM, BN, BK, NS, OCC, A_K, B_K, EXT, KS, VB>;
     static const int attr_rc = [&] {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
                                            (int)lds_bytes);
@@ -854,7 +964,7 @@ template <int BM, int BN, int BK, int NS, int OCC, bool A_K, bool B_K, bool EXT,
     return launch_status();
 }
 
-template <int BM, int BN, int BK, int NS, int OCC, int KS = 1> int launch_tile(hipStream_t st, const GemmProblem &p, uint64_t first_tiles) {
+template <int BM, int BN, int BK, int NS, int OCC, int KS = 1, int VB = 16> int launch_tile(hipStream_t st, const GemmProblem &p, uint64_t first_tiles) {
     if (first_tiles > ((p.M + BM - 1) / BM) * ((p.N + BN - 1) / BN)) return WK_E_INVALID_VALUE;
     DArgs g{};
     g.A = static_cast<const float *>(p.A);
@@ -883,32 +993,36 @@ template <int BM, int BN, int BK, int NS, int OCC, int KS = 1> int launch_tile(h
             }
     }
     const int sel = (p.op_a ? 0 : 2) | (p.op_b ? 1 : 0); // bit 1: A k-contiguous, bit 0: B k-contiguous
-    if (p.ext) { // instantiated for op N, T only (what Linear.forward runs), one group of wavefronts
-        if constexpr (KS == 1)
+    if (p.ext) { // instantiated for op N, T only (what Linear.forward runs), one group of wavefronts, aligned rows
+        if constexpr (KS == 1 && VB == 16)
             return sel == 3 ? launch_one<BM, BN, BK, NS, OCC, true, true, true>(st, g, first_tiles) : (int)WK_E_INVALID_VALUE;
         else
             return WK_E_INVALID_VALUE;
     }
     switch (sel) {
-    case 0: return launch_one<BM, BN, BK, NS, OCC, false, false, false, KS>(st, g, first_tiles);
-    case 1: return launch_one<BM, BN, BK, NS, OCC, false, true, false, KS>(st, g, first_tiles);
-    case 2: return launch_one<BM, BN, BK, NS, OCC, true, false, false, KS>(st, g, first_tiles);
-    default: return launch_one<BM, BN, BK, NS, OCC, true, true, false, KS>(st, g, first_tiles);
+    case 0: return launch_one<BM, BN, BK, NS, OCC, false, false, false, KS, VB>(st, g, first_tiles);
+    case 1: return launch_one<BM, BN, BK, NS, OCC, false, true, false, KS, VB>(st, g, first_tiles);
+    case 2: return launch_one<BM, BN, BK, NS, OCC, true, false, false, KS, VB>(st, g, first_tiles);
+    default: return launch_one<BM, BN, BK, NS, OCC, true, true, false, KS, VB>(st, g, first_tiles);
     }
+}
+
+// rows of both operands start on 16-byte boundaries: 16 bytes per lane and load; otherwise 4
+bool f32_rows_aligned(const GemmProblem &p) {
+    return p.lda % 4 == 0 && p.ldb % 4 == 0 && ((reinterpret_cast<uintptr_t>(p.A) | reinterpret_cast<uintptr_t>(p.B)) & 15u) == 0;
 }
 
 } // namespace
 
-// What the kernels take for granted, checked on the host: 16-byte aligned rows, every per-lane byte offset
-// inside 32 bits, and for the fused epilogue the one layout it
-// exists for.
+// What the kernels take for granted, checked on the host: element-aligned operands (rows that start on 16-byte
+// boundaries get 16-byte loads, any other 4-byte ones), every per-lane byte offset inside 32 bits, and for the
+// fused epilogue the one layout and the alignment it exists for.
 bool wk::gemm_f32_dma_applies(const GemmProblem &p, int bm, int bn) {
     if (p.dtype != WK_F32) return false;
     if (!((bm == 256 && bn == 128) || (bm == 128 && bn == 128) || (bm == 64 && bn == 64))) return false;
-    if (p.ext && (p.op_a || !p.op_b)) return false;
+    if (p.ext && (p.op_a || !p.op_b || !f32_rows_aligned(p))) return false;
     if (!p.M || !p.N || !p.K) return false;
-    if (p.lda % 4 || p.ldb % 4) return false;
-    if ((reinterpret_cast<uintptr_t>(p.A) | reinterpret_cast<uintptr_t>(p.B)) & 15u) return false;
+    if ((reinterpret_cast<uintptr_t>(p.A) | reinterpret_cast<uintptr_t>(p.B)) & 3u) return false;
     if (p.M > 0x7fffffffull || p.N > 0x7fffffffull || p.K > 0x7fffffffull || p.ldc > 0x7fffffffull) return false;
     // offsets reach 255 rows (k-contiguous) or 15 rows of k (m-contiguous) past the tile's origin
     if (p.lda > (1ull << 21) || p.ldb > (1ull << 21)) return false;
@@ -916,13 +1030,15 @@ bool wk::gemm_f32_dma_applies(const GemmProblem &p, int bm, int bn) {
     return true;
 }
 
+// rows of A and B start on 16-byte boundaries (16-byte loads; the two-group and fused kernels exist for these only)
+bool wk::gemm_dma_rows_aligned(const GemmProblem &p) { return p.dtype == WK_F64 ? f64_rows_aligned(p) : f32_rows_aligned(p); }
+
 bool wk::gemm_f64_dma_applies(const GemmProblem &p, int bm, int bn) {
     if (p.dtype != WK_F64) return false;
     if (!((bm == 128 && bn == 128) || (bm == 64 && bn == 64))) return false;
-    if (p.ext && (p.op_a || !p.op_b)) return false;
+    if (p.ext && (p.op_a || !p.op_b || !f64_rows_aligned(p))) return false;
     if (!p.M || !p.N || !p.K) return false;
-    if (p.lda % 2 || p.ldb % 2) return false;
-    if ((reinterpret_cast<uintptr_t>(p.A) | reinterpret_cast<uintptr_t>(p.B)) & 15u) return false;
+    if ((reinterpret_cast<uintptr_t>(p.A) | reinterpret_cast<uintptr_t>(p.B)) & 7u) return false;
     if (p.M > 0x7fffffffull || p.N > 0x7fffffffull || p.K > 0x7fffffffull || p.ldc > 0x7fffffffull) return false;
     if (p.lda > (1ull << 20) || p.ldb > (1ull << 20)) return false; // 127 rows * ld * 8 bytes inside 32 bits
     if (((p.M + bm - 1) / bm) * ((p.N + bn - 1) / bn) > 0x7fffffffull) return false;
@@ -931,6 +1047,8 @@ bool wk::gemm_f64_dma_applies(const GemmProblem &p, int bm, int bn) {
 
 int wk::gemm_f64_dma_launch(hipStream_t st, const GemmProblem &p, int bm, int bn) {
     if (!gemm_f64_dma_applies(p, bm, bn)) return WK_E_INVALID_VALUE;
+    if (!f64_rows_aligned(p)) // rows that start anywhere: four bytes per lane and load
+        return bm == 128 ? launch_tile_d<128, 128, 16, 2, 2, 4>(st, p) : launch_tile_d<64, 64, 16, 3, 3, 4>(st, p);
     if (bm == 128) return launch_tile_d<128, 128, 16, 2, 2>(st, p);
     // (64 x 64 with k-slabs of 32 in two stages, two work-groups per unit, measured the same within the run-to-run
     // spread: 8192 x 256 x 8192 67.4-68.6 against 68.0-68.2 TFLOP/s, 2048^3 68-69 against 66-68, 3072^3 70-71 both;
@@ -940,12 +1058,17 @@ int wk::gemm_f64_dma_launch(hipStream_t st, const GemmProblem &p, int bm, int bn
 
 int wk::gemm_f32_dma_launch(hipStream_t st, const GemmProblem &p, int bm, int bn, uint64_t first_tiles, int k_groups) {
     if (!gemm_f32_dma_applies(p, bm, bn)) return WK_E_INVALID_VALUE;
-    if (k_groups == 2) { // eight wavefronts per tile, k-slabs of 32 (128 x 128: one work-group per unit, 96 KB of stages)
+    if (k_groups == 2 && f32_rows_aligned(p)) { // eight wavefronts per tile, k-slabs of 32 (128 x 128: one work-group per unit, 96 KB of stages)
         // (the 256 x 128 tile with two groups, 144 KB of stages, measured no better than two work-groups of the
         // 128 x 128 tile where it would apply: 2048 x 4096 x 4096 143 against 143 TFLOP/s, 4096 x 2048 x 2048 138 against 139)
         if (p.ext || first_tiles || bm == 256) return WK_E_INVALID_VALUE;
         if (bm == 128) return launch_tile<128, 128, 32, 3, 2, 2>(st, p, 0);
         return launch_tile<64, 64, 32, 3, 4, 2>(st, p, 0);
+    }
+    if (!f32_rows_aligned(p)) { // one float per lane and load; one group of wavefronts
+        if (bm == 256) return launch_tile<256, 128, 16, 3, 2, 1, 4>(st, p, first_tiles);
+        if (bm == 128) return launch_tile<128, 128, 16, 3, 3, 1, 4>(st, p, first_tiles);
+        return launch_tile<64, 64, 32, 3, 3, 1, 4>(st, p, first_tiles);
     }
     if (bm == 256) return launch_tile<256, 128, 16, 3, 2>(st, p, first_tiles);
     // 128 x 128 with both operands m/n-contiguous (T,N): k-slabs of 32 in two stages, two work-groups per unit

@@ -1628,7 +1628,7 @@ int wk::gemm_mfma_pick(const GemmProblem &p, double *cost_out) {
         if (tiles128 <= cus && tiles128 >= 0.85 * cus) {
             // (the direct-to-LDS kernel of that tile where it applies: 2048^3 N,N 131 against 128.5)
             const char *want = !gemm_f32_dma_applies(p, 128, 128) ? "mfma_f32_128x128s2"
-                               : (p.K >= 1024 && !p.ext)           ? "mfma_f32_128x128d2"
+                               : (p.K >= 1024 && !p.ext && gemm_dma_rows_aligned(p)) ? "mfma_f32_128x128d2"
                                                                    : "mfma_f32_128x128d";
             for (int v = 0; v < k_num_variants; ++v)
                 if (!std::strcmp(k_variants[v].name, want)) return v;
@@ -1652,7 +1652,7 @@ int wk::gemm_mfma_pick(const GemmProblem &p, double *cost_out) {
         else if (tiles <= 0.75 * cus && d.sparse) twin = d.sparse; // (f64 512^3: 21.5 -> 10.3 us, 512x512x2048: 74 -> 32 us)
         else if (p.K >= 256) twin = tiles <= cus ? d.one_round : (tiles <= 2.0 * cus ? d.two_rounds : nullptr);
         if (twin && twin == d.one_round && is_dma_variant(d.name)) { // the two-group direct-to-LDS kernels: not fused
-            if (p.ext || p.K < (d.bm == 64 ? 512u : 1024u)) twin = nullptr; // (below: equal)
+            if (p.ext || !gemm_dma_rows_aligned(p) || p.K < (d.bm == 64 ? 512u : 1024u)) twin = nullptr; // (below: equal)
             else if (d.bm == 64 && p.op_a && !p.op_b) twin = nullptr;       // 64 x 64, T,N: the one-group kernel is faster
         }
         for (int v = 0; twin && v < k_num_variants; ++v)

@@ -242,6 +242,7 @@ int gemm_complex_packed_prepare(hipStream_t st, const GemmProblem &p, void *work
 // (p.ext) for op N, T.  first_tiles: launch only the first so many tiles of the tile walk (0: all), for
 // a product whose other tiles run as a k-split tail.
 bool gemm_f32_dma_applies(const GemmProblem &p, int bm, int bn);
+bool gemm_dma_rows_aligned(const GemmProblem &p); // 16-byte loads (else 4-byte ones: one group of wavefronts, no fused epilogue)
 int gemm_f32_dma_launch(hipStream_t st, const GemmProblem &p, int bm, int bn, uint64_t first_tiles = 0, int k_groups = 1);
 // the same for f64: macro tiles 128 x 128 (k-slabs of 8) and 64 x 64 (k-slabs of 16)
 bool gemm_f64_dma_applies(const GemmProblem &p, int bm, int bn);

@@ -28,6 +28,17 @@ __device__ __forceinline__ void dma16(const void *base, uint32_t byte_offset, ui
                  : "memory");
 }
 
+// The same with 4 bytes per lane: LDS at lds_base + 4 * lane.  For operands whose rows do not start on
+// 16-byte boundaries: every lane names exactly one existing element (or half of one), so nothing is
+// read beyond a row, at four times the instructions per byte.
+__device__ __forceinline__ void dma4(const void *base, uint32_t byte_offset, uint32_t lds_base) {
+    asm volatile("s_nop 0\n\t"
+                 "global_load_lds_dword %0, %1"
+                 :
+                 : "v"(byte_offset), "s"(base), "{m0}"(lds_base)
+                 : "memory");
+}
+
 template <int N> __device__ __forceinline__ void wait_vm() { asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory"); }
 // wait until at most min(later, MAXN) slabs' loads of this wavefront (PER loads each) are still in flight
 template <int PER, int MAXN> __device__ __forceinline__ void wait_vm_slabs(uint32_t later) {
