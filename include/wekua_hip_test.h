@@ -55,7 +55,9 @@ int wk_gemm_force_variant(const char *name);
  *                       which is what lets tests reach the tail path on small shapes (default 0);
  *                       wk_gemm_split_plan reports the plan of the mode in force;
  *   "alloc_colours"  0: wk_malloc returns blocks as the device allocator hands them out (default 1:
- *                       blocks of 1 MiB and more start 0 / 3 / 6 / 9 KiB into their allocation in turn). */
+ *                       blocks of 1 MiB and more start 0 / 3 / 6 / 9 KiB into their allocation in turn);
+ *   "stream_k"       0: the automatic choice never takes the kernels that deal their work by k-slabs
+ *                       ("...k") (default 1). */
 int wk_test_option(const char *name, int value);
 
 /* Launch-cost probes for profiles: a kernel with the grid, work-group size (a multiple of 64) and dynamic LDS

@@ -34,7 +34,7 @@ def test_test_knobs_are_not_in_the_product_header():
     from wekua_amd import _capi
     lib = _capi.load()
     assert lib.wk_test_option(b"no-such-switch", 1) == 1
-    for name, default in ((b"gemm_walk_rows", 0), (b"tail_strict", 0), (b"alloc_colours", 1)):
+    for name, default in ((b"gemm_walk_rows", 0), (b"tail_strict", 0), (b"alloc_colours", 1), (b"stream_k", 1)):
         assert lib.wk_test_option(name, default) == 0
 
 
@@ -62,7 +62,7 @@ def test_binding_covers_every_declared_symbol():
 def test_k_split_plans_fit_the_scratch_and_the_counters():
     """Host arithmetic of the GEMM that splits k over work-groups: whatever the shape, a plan that
     splits covers k exactly with whole slabs per share, and its partial tiles and arrival counters
-    fit what every stream owns (64 MiB, 4096 counters) -- the kernel takes both for granted."""
+    fit what every stream owns (128 MiB, 4096 counters) -- the kernel takes both for granted."""
     from wekua_amd import _capi
     lib = _capi.load()
     u32, u64, sz = ctypes.c_uint32, ctypes.c_uint64, ctypes.c_size_t
@@ -81,7 +81,7 @@ def test_k_split_plans_fit_the_scratch_and_the_counters():
                 assert klen.value % 32 == 0 and klen.value > 0
                 assert klen.value * (shares.value - 1) < K <= klen.value * shares.value    # every share holds some of k
                 assert tiles.value == ((M + 63) // 64) * ((N + 63) // 64) <= 4096
-                assert nbytes.value == shares.value * tiles.value * 64 * 64 * es <= 64 << 20
+                assert nbytes.value == shares.value * tiles.value * 64 * 64 * es <= 128 << 20
                 assert first.value == 0                                                    # every tile is split
                 if forced is None:      # the automatic choice splits only few tiles with a long k
                     assert tiles.value <= 128 and tiles.value * shares.value <= (1024 if es == 4 else 512)
@@ -99,7 +99,7 @@ def test_k_split_plans_fit_the_scratch_and_the_counters():
                 continue
             assert first.value % (256 * occ) == 0 and first.value + tiles.value == total and 0 < tiles.value < 256 * occ
             assert klen.value % 16 == 0 and klen.value * (shares.value - 1) < K <= klen.value * shares.value
-            assert nbytes.value == shares.value * tiles.value * bm * bn * 4 <= 64 << 20 and tiles.value <= 4096
+            assert nbytes.value == shares.value * tiles.value * bm * bn * 4 <= 128 << 20 and tiles.value <= 4096
     shares, klen, first, tiles, nbytes = u32(), u32(), u64(), u64(), sz()
     assert lib.wk_gemm_split_plan(8, 0, 0, 512, 512, 8192, b"mfma_f64_64x64z", shares, klen, first, tiles, nbytes) == 1   # wrong dtype
     assert lib.wk_gemm_split_plan(8, 0, 0, 512, 512, 8192, b"nope", shares, klen, first, tiles, nbytes) == 1

@@ -79,7 +79,7 @@ def test_float_small_shapes(dev, dtype, op_a, op_b, alpha, beta):
 @pytest.mark.parametrize("variant", ["tile64", "mfma_f32_64x64", "mfma_f32_64x64s2", "mfma_f32_64x64s4", "mfma_f32_32x32s4",
                                      "mfma_f32_64x64z", "mfma_f32_128x128", "mfma_f32_128x128s2", "mfma_f32_256x128",
                                      "mfma_f32_128x128t", "mfma_f32_256x128t", "mfma_f32_256x128d", "mfma_f32_128x128d", "mfma_f32_64x64d",
-                                     "mfma_f32_128x128d2", "mfma_f32_64x64d2"])
+                                     "mfma_f32_128x128d2", "mfma_f32_64x64d2", "mfma_f32_256x128k", "mfma_f32_128x128k"])
 @pytest.mark.parametrize("op_a,op_b", OPS)
 def test_f32_every_variant(dev, variant, op_a, op_b):
     import ctypes
@@ -515,6 +515,50 @@ def test_one_round_launches_take_the_k_split_tiles(dev):
             check(dev, dtype, 1000, 1000, 257, op_a, op_b, None, None, seed=94)
             check(dev, dtype, 1001, 999, 257, op_a, op_b, 1.5, 0.5, seed=96)
             check(dev, dtype, 500, 333, 129, op_a, op_b, 2.0, None, seed=95)
+
+
+@pytest.mark.parametrize("op_a,op_b", OPS)
+def test_work_dealt_by_k_slabs(dev, op_a, op_b):
+    """Products whose tiles do not fill whole rounds of the compute units have their work dealt by k-slabs
+    (mfma_f32_128x128k): tiles are split between work-groups at arbitrary slabs, the parts meet in the stream's
+    scratch and are added in the order of k.  The automatic choice by name, every entry against the oracle,
+    ragged in every dimension with a k tail, and the same bits on every run (the order of the additions does not
+    depend on which work-group arrives last)."""
+    from wekua_amd import raw
+    M, N, K = 2300, 2500, 2090
+    a, b, c = gemm_operands("f32", M, N, K, op_a, op_b, 97)
+    up = lambda v: (v + 3) // 4 * 4
+
+    def padded(m):
+        out = np.zeros((m.shape[0], up(m.shape[1])), dtype=m.dtype)
+        out[:, :m.shape[1]] = m
+        return out
+    ap, bp, cp = padded(a), padded(b), padded(c)
+    lda, ldb, ldc = ap.shape[1], bp.shape[1], cp.shape[1]
+    dA, dB = dev.upload(ap), dev.upload(bp)
+    name = dev.lib.wk_gemm_variant(raw.dtype_id("f32"), op_a, op_b, M, N, K, lda, ldb, ldc, dA.ptr, dB.ptr, dA.ptr)
+    assert name == b"mfma_f32_128x128k"
+    want = oracle.gemm("f32", 1.5, a, op_a, b, op_b, 0.5, c, threads=0)
+    first = None
+    for _ in range(6):
+        dC = dev.upload(cp)
+        dev.gemm("f32", op_a, op_b, M, N, K, 1.5, dA, lda, dB, ldb, 0.5, dC, ldc)
+        dev.sync()
+        got = np.ascontiguousarray(dC.download(np.float32, cp.shape)[:, :N])
+        dC.free()
+        if first is None:
+            first = got
+            assert_gemm_close("f32", got, want, 1.5, a, op_a, b, op_b, 0.5, c, K, what="work dealt by k-slabs")
+        else:
+            assert np.array_equal(got, first), "the bits depend on the run"
+    # the switch for A/B measurements takes the kernel away
+    assert dev.lib.wk_test_option(b"stream_k", 0) == 0
+    try:
+        assert dev.lib.wk_gemm_variant(raw.dtype_id("f32"), op_a, op_b, M, N, K, lda, ldb, ldc, dA.ptr, dB.ptr, dA.ptr) != b"mfma_f32_128x128k"
+    finally:
+        dev.lib.wk_test_option(b"stream_k", 1)
+    for d in (dA, dB):
+        d.free()
 
 
 @pytest.mark.parametrize("dtype", ["f32", "f64"])

@@ -149,6 +149,22 @@ bool plan_strips(const GemmProblem &p, StripPlan &out) {
         const uint64_t Mb = thin_m ? p.M - m_rem : p.M, Nb = thin_n ? p.N - n_rem : p.N;
         if ((thin_m || thin_n) && Mb * Nb >= (1ull << 22)) { // (2048 x 2047 and below: N,N gains 7 %, T,N loses as much)
             make_parts(p, Mb, Nb, out);
+            // ... unless the whole product would have its work dealt by k-slabs, which does not care about a started
+            // round, and the model puts that below the parts (2200^3: 113 TFLOP/s whole, 102 in parts)
+            double whole = 0.0;
+            const int wv = gemm_mfma_pick(p, &whole);
+            const char *wname = wv >= 0 ? gemm_mfma_variant_name(wv) : nullptr;
+            if (wname && wname[std::strlen(wname) - 1] == 'k') {
+                const double launch = 4.0 * 3.05e5 / (double)p.K;
+                double sum = 0.0;
+                for (int i = 0; i < out.parts; ++i) {
+                    double c = 0.0;
+                    if (gemm_thin_applies(out.part[i])) c = 5.0 * launch; // (a thin product reads the long operand once: 16-46 us)
+                    else if (gemm_mfma_pick(out.part[i], &c) < 0) return true;
+                    sum += c + (i ? launch : 0.0);
+                }
+                if (sum >= whole) return false;
+            }
             return true;
         }
     }

@@ -40,6 +40,7 @@ namespace {
 
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef unsigned int u32x4_t __attribute__((ext_vector_type(4)));
 
 constexpr int GROUP_M = 8;
 
@@ -55,6 +56,11 @@ struct DArgs {
     const float *bias; // kernels instantiated with EXT: C = act(acc + bias[col]); bias may be null
     int act;
     uint32_t patch_m, patch_n; // tile walk in XCD-local patches of patch_m x patch_n tiles (0: rows of groups)
+    // kernels instantiated with SK (work dealt by k-slabs, not by tiles): k-slabs per work-group, k-slabs in all
+    // (tiles x slabs per tile), memory for two partial tiles per work-group and one arrival counter per tile
+    uint32_t sk_units, sk_total;
+    float *partials;
+    uint32_t *counters;
 };
 
 // KS: groups of 2 x 2 wavefronts on the same tile (1 or 2).  A launch of one round of tiles leaves every SIMD
@@ -64,11 +70,23 @@ struct DArgs {
 // VB: bytes per lane and load.  16 for operands whose rows start on 16-byte boundaries; 4 for any other (every
 // lane then fetches one float into the same place of the same LDS layout: SUB = 4 loads per KiB instead of one,
 // nothing read beyond the end of a row).
-template <int BM, int BN, int BK, int NS, int OCC, bool A_K, bool B_K, bool EXT, int KS = 1, int VB = 16>
+// SK: the launch is as many work-groups as are resident at once (compute units x OCC), and the work is dealt to
+// them by k-slabs instead of by tiles: work-group b takes slabs [b' U, (b' + 1) U) of the tiles x slabs-per-tile
+// of the product in tile-walk order (b' numbers the work-groups of one XCD consecutively), so every unit is busy
+// for the same time whatever the number of tiles.  A range that holds a whole tile runs it as ever; a part of a
+// tile (at most two per work-group: the end of one tile at the start of its range, the start of another at its
+// end) goes to memory as a partial tile, and the work-group that arrives last at the tile's counter adds the
+// parts up in the order of k -- its own read back like the others, so the bits do not depend on who that is --
+// and runs the epilogue.  The same hand-over as the k-split kernels of wk_gemm_mfma.hip (device-scope stores and
+// loads, a wait for the stores in front of the count).
+template <int BM, int BN, int BK, int NS, int OCC, bool A_K, bool B_K, bool EXT, int KS = 1, int VB = 16, bool SK = false>
 __global__ __launch_bounds__(256 * KS) __attribute__((amdgpu_waves_per_eu(OCC)))
 void gemm_f32_dma_kernel(DArgs g) {
     static_assert(VB == 16 || VB == 4, "bytes per lane");
+    static_assert(!SK || KS == 1, "work dealt by k-slabs: one group of wavefronts");
     constexpr int SUB = 16 / VB;
+    __shared__ uint32_t s_last;
+    auto run = [&](const uint32_t pid, const uint32_t kb, const uint32_t ke, const uint32_t bq, const bool stagger) __attribute__((always_inline)) {
     constexpr int WM = BM / 2, WN = BN / 2, FM = WM / 32, FN = WN / 32;
     constexpr int S = BK / 8;   // fragment steps per slab (8 values of k each: four matrix instructions per block)
     constexpr int CPR = BK / 4; // 16-byte chunks per row of a k-contiguous slab
@@ -93,7 +111,6 @@ void gemm_f32_dma_kernel(DArgs g) {
     if (g.patch_m) {
         // work-group b runs on XCD b % 8: the j-th work-group of an XCD takes tile j % (patch) of that
         // XCD's patch j / (patch), so the tiles that share an L2 at one time share rows of A and columns of B
-        const uint32_t pid = blockIdx.x;
         const uint32_t x = pid & 7u, j = pid >> 3;
         const uint32_t per_patch = g.patch_m * g.patch_n;
         const uint32_t patch = (j / per_patch) * 8u + x, q = j % per_patch;
@@ -101,7 +118,6 @@ void gemm_f32_dma_kernel(DArgs g) {
         tile_m = (patch / patches_n) * g.patch_m + q % g.patch_m;
         tile_n = (patch % patches_n) * g.patch_n + q / g.patch_m;
     } else {
-        const uint32_t pid = blockIdx.x;
         const uint32_t group_size = GROUP_M * g.tiles_n;
         const uint32_t group = pid / group_size;
         const uint32_t first_m = group * GROUP_M;
@@ -113,7 +129,7 @@ void gemm_f32_dma_kernel(DArgs g) {
     const uint32_t m0 = tile_m * BM, n0 = tile_n * BN;
     // the second co-resident work-group of the first dispatch wave starts one solo iteration late, so
     // that the two do not hand over at the same time
-    if (g.num_cus) {
+    if (stagger && g.num_cus) {
         const uint32_t slot = blockIdx.x / g.num_cus;
         if (slot >= 1 && slot < (uint32_t)OCC)
             for (uint32_t i = 0; i < slot * (FM * FN * BK / 4); ++i) __builtin_amdgcn_s_sleep(2);
@@ -127,6 +143,10 @@ void gemm_f32_dma_kernel(DArgs g) {
     const float *b_base = B_K ? g.B + (size_t)n0 * g.ldb : g.B + n0;
     const size_t a_step = A_K ? (size_t)BK : (size_t)BK * g.lda; // floats per slab
     const size_t b_step = B_K ? (size_t)BK : (size_t)BK * g.ldb;
+    if constexpr (SK) { // this range starts at slab kb of the tile
+        a_base += kb * a_step;
+        b_base += kb * b_step;
+    }
     uint32_t a_off[A_LOADS * SUB], b_off[B_LOADS * SUB];
     // loads i * SUB ... of this wavefront fill the 1 KB group i * 4 + wave of the operand's slab: sixteen rows of a
     // k-contiguous operand, 256 / ROWS rows of k of an m-contiguous one
@@ -199,7 +219,7 @@ void gemm_f32_dma_kernel(DArgs g) {
     // Chunks (k-contiguous operand) or rows of k (m-contiguous) that lie wholly beyond K are fetched from
     // the last existing one instead; once a wavefront's own loads of that slab have landed it writes
     // zeros over every float of its share whose k does not exist (products with them must vanish).
-    const uint32_t krem = g.K % BK;
+    const uint32_t krem = !SK || ke * BK >= g.K ? g.K % BK : 0u; // (a range that ends inside the tile has whole slabs only)
     // k of the float that lane `lane` of load q of group grp fetches with one float per lane (VB = 4)
     auto k_of_float = [&](int grp, int q, auto kc_tag, auto rows_tag) -> uint32_t {
         constexpr bool KC = decltype(kc_tag)::value;
@@ -341,7 +361,7 @@ void gemm_f32_dma_kernel(DArgs g) {
                     acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(af[s & 1][i][t], bf[s & 1][j][t], acc[i][j], 0, 0, 0);
     };
 
-    const uint32_t ktiles = (g.K + BK - 1) / BK;
+    const uint32_t ktiles = SK ? ke - kb : (g.K + BK - 1) / BK;
 
     // The NS stages rotate (byte offsets): st[0] holds the slab being multiplied, st[1] the next one, ...,
     // st[NS - 1] is the stage the slab before left, into which slab kt + NS - 1 is requested.
@@ -463,6 +483,94 @@ void gemm_f32_dma_kernel(DArgs g) {
 #pragma unroll
                 for (int r = 0; r < 16; ++r) acc[i][j][r] += part[((i * FN + j) * 16 + r) * 64];
     }
+    if constexpr (SK) {
+        const uint32_t slabs_per_tile = (g.K + BK - 1) / BK;
+        if (!(kb == 0 && ke == slabs_per_tile)) {
+            // a part of the tile: to memory in accumulator-register order, 16 bytes per lane (registers 4 q .. 4 q + 3
+            // of thread t at (q * 256 + t) * 16 bytes: coalesced; the thread's part of the address in a register, the rest scalar); slot 2 b' holds the part that starts inside the
+            // tile, 2 b' + 1 the one that starts it.  Device-scope accesses (the sc1 cache policy, bit 4 of the
+            // buffer instructions' auxiliary operand): the parts of a tile come from different XCDs.
+            constexpr size_t TILE = (size_t)BM * BN;
+            constexpr int SC1 = 16;
+            const uint32_t U = g.sk_units, t0 = pid * slabs_per_tile;
+            const uint32_t b_first = t0 / U, b_last = (t0 + slabs_per_tile - 1) / U; // the work-groups that hold parts of it
+            const uint32_t nparts = b_last - b_first + 1;
+            // The part that starts the tile is the last of its work-group's range, so it is usually the last to be
+            // ready: when the counter says that all the others have arrived, it stays in the accumulators and the
+            // others are added to it in the order of k (no store, no read-back: 0 + p0 + p1 ... and p0 + p1 ... are
+            // the same bits).  Otherwise it goes to memory like any other part.
+            uint32_t first_part = 0;
+            if (kb == 0) {
+                if (tid == 0) {
+                    const uint32_t arrived = __hip_atomic_load(&g.counters[pid], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    if (arrived == nparts - 1) __hip_atomic_store(&g.counters[pid], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    s_last = arrived == nparts - 1 ? 1u : 0u;
+                }
+                __syncthreads();
+                first_part = s_last;
+                __syncthreads(); // (s_last is written again below)
+            }
+            if (first_part == 0) {
+                __amdgpu_buffer_rsrc_t mine = __builtin_amdgcn_make_buffer_rsrc(
+                    g.partials + (size_t)(2 * bq + (kb == 0 ? 1u : 0u)) * TILE, 0, (int)(TILE * sizeof(float)), 0x00020000);
+#pragma unroll
+                for (int i = 0; i < FM; ++i)
+#pragma unroll
+                    for (int j = 0; j < FN; ++j)
+#pragma unroll
+                        for (int q = 0; q < 4; ++q) {
+                            const f32x4 v = {acc[i][j][4 * q], acc[i][j][4 * q + 1], acc[i][j][4 * q + 2], acc[i][j][4 * q + 3]};
+                            __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4_t, v), mine, tid * 16, ((i * FN + j) * 4 + q) * 4096, SC1);
+                        }
+                asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+                __syncthreads();
+                if (tid == 0) {
+                    const uint32_t before = __hip_atomic_fetch_add(&g.counters[pid], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    const uint32_t last = before == nparts - 1 ? 1u : 0u;
+                    if (last) __hip_atomic_store(&g.counters[pid], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    s_last = last;
+                }
+                __syncthreads();
+                if (!s_last) return;
+                // the last to arrive adds the parts up in the order of k, its own read back like the others
+#pragma unroll
+                for (int i = 0; i < FM; ++i)
+#pragma unroll
+                    for (int j = 0; j < FN; ++j)
+#pragma unroll
+                        for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+            }
+            // Every round trip to memory costs a few microseconds whatever it carries, so the loads of four
+            // blocks of a part (64 registers) are in flight together.
+            constexpr int NB = FM * FN < 4 ? FM * FN : 4; // blocks per batch of loads
+            static_assert((FM * FN) % NB == 0, "blocks divide into batches");
+            for (uint32_t pp = first_part; pp < nparts; ++pp) {
+                const uint32_t b2 = b_first + pp;
+                __amdgpu_buffer_rsrc_t part = __builtin_amdgcn_make_buffer_rsrc(
+                    g.partials + (size_t)(2 * b2 + (pp == 0 ? 1u : 0u)) * TILE, 0, (int)(TILE * sizeof(float)), 0x00020000);
+#pragma unroll
+                for (int batch = 0; batch < FM * FN / NB; ++batch) {
+                    u32x4_t v[NB][4];
+#pragma unroll
+                    for (int n = 0; n < NB; ++n)
+#pragma unroll
+                        for (int q = 0; q < 4; ++q)
+                            v[n][q] = __builtin_amdgcn_raw_buffer_load_b128(part, tid * 16, ((batch * NB + n) * 4 + q) * 4096, SC1);
+#pragma unroll
+                    for (int n = 0; n < NB; ++n) {
+                        const int blk = batch * NB + n, i = blk / FN, j = blk % FN;
+#pragma unroll
+                        for (int q = 0; q < 4; ++q) {
+                            const f32x4 f = __builtin_bit_cast(f32x4, v[n][q]);
+#pragma unroll
+                            for (int e = 0; e < 4; ++e) acc[i][j][4 * q + e] += f[e];
+                        }
+                    }
+                    __builtin_amdgcn_sched_barrier(0); // (one batch of loads at a time)
+                }
+            }
+        }
+    }
     // row of the wavefront's tile that output row `rho` of block i holds
     auto tile_row = [](int i, int rho) -> uint32_t { return A_PERM ? (uint32_t)(4 * rho + i) : (uint32_t)(32 * i + rho); };
     // Tiles that reach beyond C clamp the addresses of C_old and the bias and skip the stores there.
@@ -504,6 +612,25 @@ void gemm_f32_dma_kernel(DArgs g) {
     };
     if (m0 + BM <= g.M && n0 + BN <= g.N) epilogue(std::false_type{});
     else epilogue(std::true_type{});
+    }; // run
+    if constexpr (!SK) {
+        run(blockIdx.x, 0u, 0u, 0u, true);
+    } else {
+        const uint32_t slabs_per_tile = (g.K + BK - 1) / BK;
+        // work-groups b, b + 8, ... share an XCD: they take consecutive ranges, and with them neighbouring tiles
+        const uint32_t bq = (blockIdx.x & 7u) * (gridDim.x >> 3) + (blockIdx.x >> 3);
+        uint32_t u = bq * g.sk_units;
+        const uint32_t u_end = min(u + g.sk_units, g.sk_total);
+        bool first = true;
+        while (u < u_end) {
+            const uint32_t pid = u / slabs_per_tile, kb = u - pid * slabs_per_tile;
+            const uint32_t ke = min(slabs_per_tile, kb + (u_end - u));
+            if (!first) __syncthreads(); // every wavefront is done with the stages of the range before
+            run(pid, kb, ke, bq, first);
+            first = false;
+            u += ke - kb;
+        }
+    }
 }
 
 // ------------------------------------------------------------------------------------ f64 ---
@@ -945,10 +1072,11 @@ bool f64_rows_aligned(const GemmProblem &p) {
 }
 
 // first_tiles: launch only that many tiles, in tile-walk order (0: all of them)
-template <int BM, int BN, int BK, int NS, int OCC, bool A_K, bool B_K, bool EXT, int KS = 1, int VB = 16>
-int launch_one(hipStream_t st, const DArgs &g, uint64_t first_tiles) {
+// sk_groups: work dealt by k-slabs to that many work-groups (0: one work-group per tile)
+template <int BM, int BN, int BK, int NS, int OCC, bool A_K, bool B_K, bool EXT, int KS = 1, int VB = 16, bool SK = false>
+int launch_one(hipStream_t st, const DArgs &g, uint64_t first_tiles, unsigned sk_groups = 0) {
     constexpr size_t lds_bytes = NS * (BM * BK + BN * BK) * sizeof(float); // 3 x 24 KB / 3 x 16 KB / 3 x 32 KB
-    auto kern = gemm_f32_dma_kernel<BM, BN, BK, NS, OCC, A_K, B_K, EXT, KS, VB>;
+    auto kern = gemm_f32_dma_kernel<BM, BN, BK, NS, OCC, A_K, B_K, EXT, KS, VB, SK>;
     static const int attr_rc = [&] {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
                                            (int)lds_bytes);
@@ -959,12 +1087,26 @@ int launch_one(hipStream_t st, const DArgs &g, uint64_t first_tiles) {
         return (int)WK_OK;
     }();
     if (attr_rc) return attr_rc;
-    const unsigned grid = first_tiles ? (unsigned)first_tiles : g.tiles_m * g.tiles_n;
+    const unsigned grid = SK ? sk_groups : first_tiles ? (unsigned)first_tiles : g.tiles_m * g.tiles_n;
     hipLaunchKernelGGL(kern, dim3(grid), dim3(256 * KS), lds_bytes, st, g);
     return launch_status();
 }
 
-template <int BM, int BN, int BK, int NS, int OCC, int KS = 1, int VB = 16> int launch_tile(hipStream_t st, const GemmProblem &p, uint64_t first_tiles) {
+// How the work-groups of a launch that deals its work by k-slabs share it: groups = compute units x occ (a
+// multiple of eight), units = ceil(tiles x slabs per tile / groups) slabs each.  false: the problem does not fit
+// (no scratch for two partial tiles per work-group, more tiles than counters, 32-bit slab numbers).
+bool stream_k_plan(const GemmProblem &p, int bm, int bn, int bk, int occ, unsigned &groups, uint32_t &units, uint32_t &total) {
+    const uint64_t tiles = ((p.M + bm - 1) / bm) * ((p.N + bn - 1) / bn), slabs = (p.K + bk - 1) / bk;
+    const uint64_t cus = p.num_cus ? p.num_cus : 256;
+    groups = (unsigned)(cus * occ);
+    if (groups % 8 || !p.scratch || !p.counters || tiles > p.num_counters || tiles * slabs > 0x7fffffffull) return false;
+    if ((uint64_t)2 * groups * bm * bn * sizeof(float) > p.scratch_bytes) return false;
+    total = (uint32_t)(tiles * slabs);
+    units = (uint32_t)((tiles * slabs + groups - 1) / groups);
+    return units >= 1;
+}
+
+template <int BM, int BN, int BK, int NS, int OCC, int KS = 1, int VB = 16, bool SK = false> int launch_tile(hipStream_t st, const GemmProblem &p, uint64_t first_tiles) {
     if (first_tiles > ((p.M + BM - 1) / BM) * ((p.N + BN - 1) / BN)) return WK_E_INVALID_VALUE;
     DArgs g{};
     g.A = static_cast<const float *>(p.A);
@@ -993,17 +1135,24 @@ template <int BM, int BN, int BK, int NS, int OCC, int KS = 1, int VB = 16> int 
             }
     }
     const int sel = (p.op_a ? 0 : 2) | (p.op_b ? 1 : 0); // bit 1: A k-contiguous, bit 0: B k-contiguous
+    unsigned sk_groups = 0;
+    if constexpr (SK) {
+        if (first_tiles || !stream_k_plan(p, BM, BN, BK, OCC, sk_groups, g.sk_units, g.sk_total)) return WK_E_INVALID_VALUE;
+        g.partials = static_cast<float *>(p.scratch);
+        g.counters = p.counters;
+        g.patch_m = g.patch_n = 0; // consecutive tile numbers are neighbours in the row-group walk
+    }
     if (p.ext) { // instantiated for op N, T only (what Linear.forward runs), one group of wavefronts, aligned rows
         if constexpr (KS == 1 && VB == 16)
-            return sel == 3 ? launch_one<BM, BN, BK, NS, OCC, true, true, true>(st, g, first_tiles) : (int)WK_E_INVALID_VALUE;
+            return sel == 3 ? launch_one<BM, BN, BK, NS, OCC, true, true, true, 1, 16, SK>(st, g, first_tiles, sk_groups) : (int)WK_E_INVALID_VALUE;
         else
             return WK_E_INVALID_VALUE;
     }
     switch (sel) {
-    case 0: return launch_one<BM, BN, BK, NS, OCC, false, false, false, KS, VB>(st, g, first_tiles);
-    case 1: return launch_one<BM, BN, BK, NS, OCC, false, true, false, KS, VB>(st, g, first_tiles);
-    case 2: return launch_one<BM, BN, BK, NS, OCC, true, false, false, KS, VB>(st, g, first_tiles);
-    default: return launch_one<BM, BN, BK, NS, OCC, true, true, false, KS, VB>(st, g, first_tiles);
+    case 0: return launch_one<BM, BN, BK, NS, OCC, false, false, false, KS, VB, SK>(st, g, first_tiles, sk_groups);
+    case 1: return launch_one<BM, BN, BK, NS, OCC, false, true, false, KS, VB, SK>(st, g, first_tiles, sk_groups);
+    case 2: return launch_one<BM, BN, BK, NS, OCC, true, false, false, KS, VB, SK>(st, g, first_tiles, sk_groups);
+    default: return launch_one<BM, BN, BK, NS, OCC, true, true, false, KS, VB, SK>(st, g, first_tiles, sk_groups);
     }
 }
 
@@ -1056,6 +1205,20 @@ int wk::gemm_f64_dma_launch(hipStream_t st, const GemmProblem &p, int bm, int bn
     return launch_tile_d<64, 64, 16, 3, 3>(st, p);
 }
 
+// work dealt by k-slabs (the 256 x 128 and 128 x 128 tiles, rows that start on 16-byte boundaries)
+bool wk::gemm_f32_dma_stream_k_applies(const GemmProblem &p, int bm, int bn) {
+    if (!(bn == 128 && (bm == 256 || bm == 128)) || !gemm_f32_dma_applies(p, bm, bn) || !f32_rows_aligned(p)) return false;
+    unsigned groups;
+    uint32_t units, total;
+    return stream_k_plan(p, bm, bn, 16, bm == 256 ? 2 : 3, groups, units, total);
+}
+
+int wk::gemm_f32_dma_stream_k_launch(hipStream_t st, const GemmProblem &p, int bm, int bn) {
+    if (!gemm_f32_dma_stream_k_applies(p, bm, bn)) return WK_E_INVALID_VALUE;
+    if (bm == 256) return launch_tile<256, 128, 16, 3, 2, 1, 16, true>(st, p, 0);
+    return launch_tile<128, 128, 16, 3, 3, 1, 16, true>(st, p, 0);
+}
+
 int wk::gemm_f32_dma_launch(hipStream_t st, const GemmProblem &p, int bm, int bn, uint64_t first_tiles, int k_groups) {
     if (!gemm_f32_dma_applies(p, bm, bn)) return WK_E_INVALID_VALUE;
     if (k_groups == 2 && f32_rows_aligned(p)) { // eight wavefronts per tile, k-slabs of 32 (128 x 128: one work-group per unit, 96 KB of stages)
@@ -1063,6 +1226,8 @@ int wk::gemm_f32_dma_launch(hipStream_t st, const GemmProblem &p, int bm, int bn
         // 128 x 128 tile where it would apply: 2048 x 4096 x 4096 143 against 143 TFLOP/s, 4096 x 2048 x 2048 138 against 139)
         if (p.ext || first_tiles || bm == 256) return WK_E_INVALID_VALUE;
         if (bm == 128) return launch_tile<128, 128, 32, 3, 2, 2>(st, p, 0);
+        // (four, six and eight stages instead of three, for a lone work-group per unit: 1024^3, 1000^3 and
+        // 1024 x 1024 x 4096 all within 1 % of three, every layout)
         return launch_tile<64, 64, 32, 3, 4, 2>(st, p, 0);
     }
     if (!f32_rows_aligned(p)) { // one float per lane and load; one group of wavefronts

@@ -28,6 +28,7 @@
 // M % BM == N % BN == K % BK == 0 and 16-byte aligned rows.
 #include "wk_internal.hpp"
 
+#include <cmath>
 #include <cstdlib>
 #include <algorithm>
 #include <cstring>
@@ -1407,6 +1408,12 @@ template <int BM, int BN> int launch_f32_dma2(hipStream_t st, const GemmProblem 
     return launch_f32<64, 64, 16, 2, 2, 4, 4>(st, p, edge);
 }
 
+// work dealt by k-slabs to as many work-groups as are resident at once; where that does not apply, by tiles
+template <int BM, int BN, int OCC> int launch_f32_stream_k(hipStream_t st, const GemmProblem &p, bool edge) {
+    if (gemm_f32_dma_stream_k_applies(p, BM, BN)) return gemm_f32_dma_stream_k_launch(st, p, BM, BN);
+    return launch_f32_dma<BM, BN, 16, OCC>(st, p, edge);
+}
+
 template <int BM, int BN, int BK, int OCC> int launch_f64_dma(hipStream_t st, const GemmProblem &p, bool edge) {
     if (gemm_f64_dma_applies(p, BM, BN)) return gemm_f64_dma_launch(st, p, BM, BN);
     return launch_f64<BM, BN, BK, 2, 2, OCC>(st, p, edge);
@@ -1459,6 +1466,9 @@ const VariantDesc k_variants[] = {
     // 105 / 106 / 97 / 103, 1024 x 1024 x 4096 121 / 120 / 124 / 119 -> 124 / 127 / 120 / 123: not for T,N there
     {"mfma_f32_128x128d2", WK_F32, 128, 128, 32, 0.0, 0.08, &launch_f32_dma2<128, 128>},
     {"mfma_f32_64x64d2", WK_F32, 64, 64, 32, 0.0, 0.10, &launch_f32_dma2<64, 64>},
+    // the same kernels with the work dealt by k-slabs (see gemm_f32_dma_kernel), for tiles that do not fill whole rounds
+    {"mfma_f32_256x128k", WK_F32, 256, 128, 16, 0.0, 0.08, &launch_f32_stream_k<256, 128, 2>, nullptr, nullptr, nullptr, nullptr, nullptr, 2},
+    {"mfma_f32_128x128k", WK_F32, 128, 128, 16, 0.0, 0.08, &launch_f32_stream_k<128, 128, 3>, nullptr, nullptr, nullptr, nullptr, nullptr, 3},
     {"mfma_f32_256x128t", WK_F32, 256, 128, 16, 0.0, 0.25, &launch_f32_tail<256, 128, 16, 2, 2, 2>, nullptr, nullptr, nullptr, nullptr,
      nullptr, 2}, // whole rounds + a k-split tail
     {"mfma_f32_128x128", WK_F32, 128, 128, 16, 0.897, 0.19, &launch_f32<128, 128, 16, 2, 2, 3>, nullptr, nullptr, nullptr, nullptr,
@@ -1615,6 +1625,30 @@ int wk::gemm_mfma_pick(const GemmProblem &p, double *cost_out) {
                     if (!std::strcmp(k_variants[w].name, d.tail)) {
                         best = w;
                         best_cost = tcost;
+                    }
+        }
+    }
+    // Tiles that do not fill whole rounds: the 128 x 128 kernel with the work dealt by k-slabs (every unit busy for
+    // the same time) where that beats what was found above by more than the model's error.  Its time is that of
+    // the tiles spread evenly over the units plus about 22 us per launch, whatever the shape: the parts of split
+    // tiles meet in memory and every work-group runs its epilogue at the same moment (this form reproduces the
+    // measured launches from 2200^3 to 4200^3 and 2048 x 4096 x 1024 to 3 %).  Measured against the choice without
+    // it, N,N, TFLOP/s: 2200^3 102 -> 113, 2300^3 115 -> 126, 2500^3 116 -> 122, 3000^3 125 -> 131, 3700^3 123 -> 133,
+    // 4000^3 129 -> 135, 3000 x 3000 x 8192 126 -> 135, 2500 x 3500 x 4096 121 -> 130, 5000 x 3000 x 2000 120 -> 128; no
+    // gain where whole rounds or split-off strips fit anyway (2816^3, 3200^3, 4200^3), a loss on 2048 x 4096 x 1024
+    // (121 against 134).  Beyond some 1100 tiles the work-groups of an XCD, each on its own run of tiles, no longer
+    // share their panels in the L2 (5000^3 131 against 135, 6500^3 120 against 142): not taken there.  The 256 x 128
+    // tile dealt the same way (mfma_f32_256x128k) wins nowhere by more than a percent.
+    if (p.dtype == WK_F32 && best >= 0 && p.K >= 1536 && g_test_options.stream_k) { // (k = 1024: 4200 x 4096 x 1024 128 against 131 in parts)
+        constexpr double SK_FIXED_US = 22.0, COST_PER_US = 3.05e5, SK_MAX_TILES = 1100.0;
+        const double tiles = (double)((p.M + 127) / 128) * (double)((p.N + 127) / 128);
+        if (tiles > cus && tiles <= SK_MAX_TILES && std::fmod(tiles, cus * 3.0) != 0.0 && gemm_f32_dma_stream_k_applies(p, 128, 128)) {
+            const double cost = tiles / cus * 128.0 * 128.0 / 0.922 + SK_FIXED_US * COST_PER_US / (double)p.K;
+            if (cost < 0.97 * best_cost)
+                for (int w = 0; w < k_num_variants; ++w)
+                    if (!std::strcmp(k_variants[w].name, "mfma_f32_128x128k")) {
+                        best = w;
+                        best_cost = cost;
                     }
         }
     }

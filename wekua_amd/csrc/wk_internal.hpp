@@ -26,7 +26,7 @@ struct wk_stream {
     uint32_t *gemm_counters;
 };
 
-constexpr size_t WK_STREAM_SCRATCH_BYTES = 64u << 20;
+constexpr size_t WK_STREAM_SCRATCH_BYTES = 128u << 20;
 constexpr size_t WK_GEMM_COUNTERS = 4096;
 // what wk_bias_step uses of the scratch: the number of row bands, and with it the order of the
 // additions, follows from this size, so it stays what it was when the scratch was this small
@@ -44,6 +44,7 @@ struct TestOptions {
     int gemm_walk_rows = 0; // 1: the direct-to-LDS kernels walk the tiles in groups of rows, not XCD-local patches
     int tail_strict = 0;    // 1: forced k-split tail variants plan like the automatic choice
     int alloc_colours = 1;  // 0: wk_malloc hands out blocks as hipMalloc returns them
+    int stream_k = 1;       // 0: the automatic choice never deals work by k-slabs
 };
 extern TestOptions g_test_options;
 
@@ -242,6 +243,10 @@ int gemm_complex_packed_prepare(hipStream_t st, const GemmProblem &p, void *work
 // (p.ext) for op N, T.  first_tiles: launch only the first so many tiles of the tile walk (0: all), for
 // a product whose other tiles run as a k-split tail.
 bool gemm_f32_dma_applies(const GemmProblem &p, int bm, int bn);
+// the same kernels with the work dealt to compute units x occ work-groups by k-slabs instead of by tiles
+// (parts of tiles meet in p.scratch, counted on p.counters): for products whose tiles do not fill whole rounds
+bool gemm_f32_dma_stream_k_applies(const GemmProblem &p, int bm, int bn);
+int gemm_f32_dma_stream_k_launch(hipStream_t st, const GemmProblem &p, int bm, int bn);
 bool gemm_dma_rows_aligned(const GemmProblem &p); // 16-byte loads (else 4-byte ones: one group of wavefronts, no fused epilogue)
 int gemm_f32_dma_launch(hipStream_t st, const GemmProblem &p, int bm, int bn, uint64_t first_tiles = 0, int k_groups = 1);
 // the same for f64: macro tiles 128 x 128 (k-slabs of 8) and 64 x 64 (k-slabs of 16)
