@@ -157,9 +157,11 @@ def axpy_placement_leg(dev, raw, dtype, log2n, steps, warmup):
 
 def memory_ceilings(dev, raw, log2n):
     """What the memory system gives simpler access patterns on this box in this run, for scale next to
-    the AXPY figure (2 read streams + 1 write stream): a plain copy kernel (1 read + 1 write stream) and
-    math.sum's reduction (1 read stream), both over n = 2^log2n f32 of random data; median of five
-    batches of ten launches."""
+    the AXPY figure (2 read streams + 1 write stream).  Three probes in the AXPY kernel's own shape (one
+    wavefront per work-group, one 16-byte vector per lane, non-temporal loads, streaming stores): a copy
+    (1 read + 1 write stream), one read stream and two read streams; and the plain grid-stride copy kernel
+    that calibrates the profiler's byte counters.  n = 2^log2n f32 of random data in [-1, 1); median of
+    five batches of ten launches each."""
     from wekua_amd._capi import check
     n = 1 << log2n
     nbytes = 4 * n
@@ -167,20 +169,26 @@ def memory_ceilings(dev, raw, log2n):
     did = raw.dtype_id("f32")
     s3 = (ctypes.c_uint64 * 3)(1, 1, n)
     lo, span = raw.scalar_bytes("f32", -1.0), raw.scalar_bytes("f32", 2.0)
-    check(dev.lib.wk_random_uniform(dev.stream, did, s3, src.ptr, n, n, 5, ctypes.cast(lo, ctypes.c_void_p),
-                                    ctypes.cast(span, ctypes.c_void_p)), "wk_random_uniform")
-    ws = dev.malloc(max(int(dev.lib.wk_sum_workspace_bytes(did)), 16))
-    res = dev.malloc(16)
+    for buf, seed in ((src, 5), (dst, 6)):
+        check(dev.lib.wk_random_uniform(dev.stream, did, s3, buf.ptr, n, n, seed, ctypes.cast(lo, ctypes.c_void_p),
+                                        ctypes.cast(span, ctypes.c_void_p)), "wk_random_uniform")
+    # 0x7fc01234 is a NaN as f32: neither a value in [-1, 1) nor, in all four words, the xor of two of them
+    sentinel = 0x7fc01234
     median = lambda call: sorted(dev.time_stream_ms(call, 10) for _ in range(5))[2]
-    for _ in range(3):
-        check(dev.lib.wk_copy_kernel(dev.stream, dst.ptr, src.ptr, nbytes), "copy")
+    probe = lambda kind: (lambda: check(dev.lib.wk_stream_probe(dev.stream, kind, dst.ptr, src.ptr, nbytes, sentinel), "probe"))
+    plain = lambda: check(dev.lib.wk_copy_kernel(dev.stream, dst.ptr, src.ptr, nbytes), "copy")
+    for call in (probe(0), probe(1), probe(2), plain):
+        call()
     dev.sync()
-    copy_ms = median(lambda: check(dev.lib.wk_copy_kernel(dev.stream, dst.ptr, src.ptr, nbytes), "copy"))
-    read_ms = median(lambda: check(dev.lib.wk_sum(dev.stream, did, s3, src.ptr, n, n, ws.ptr, res.ptr, 1.0), "sum"))
-    for b in (src, dst, ws, res):
+    ms = {"copy": median(probe(0)), "read": median(probe(1)), "read2": median(probe(2)), "plain": median(plain)}
+    for b in (src, dst):
         b.free()
-    return {"copy_GBs": 2.0 * nbytes / copy_ms / 1e6, "read_GBs": nbytes / read_ms / 1e6, "n": n, "dtype": "f32",
-            "what": "plain copy kernel (bytes read + written) and math.sum (bytes read), median of 5 batches of 10 launches"}
+    return {"copy_GBs": 2.0 * nbytes / ms["copy"] / 1e6, "read_GBs": nbytes / ms["read"] / 1e6,
+            "two_reads_GBs": 2.0 * nbytes / ms["read2"] / 1e6, "plain_copy_GBs": 2.0 * nbytes / ms["plain"] / 1e6,
+            "n": n, "dtype": "f32",
+            "what": "probes in the AXPY kernel's shape: copy (1 read + 1 write stream), read (1 read stream), two_reads "
+                    "(2 read streams); plain_copy is the grid-stride copy kernel that calibrates the byte counters; "
+                    "bytes moved / time, median of 5 batches of 10 launches"}
 
 
 def cpu_gemm_leg(dtype, M, N, K, alpha, beta, threads, a=None, b=None):
@@ -249,8 +257,9 @@ def main():
         log(f"[bench] axpy {dt} 2^{args.axpy_log2n} by placement of y against x: same offset inside a 4 KiB block "
             f"{place[dt]['same_offset_in_4KiB']:.0f} GB/s, 3 KiB further in {place[dt]['y_plus_3KiB']:.0f} GB/s")
     ceilings = memory_ceilings(dev, raw, args.axpy_log2n)
-    log(f"[bench] memory ceilings on this box, same buffers: copy (1 read + 1 write stream) {ceilings['copy_GBs']:.0f} GB/s, "
-        f"sum (1 read stream) {ceilings['read_GBs']:.0f} GB/s")
+    log(f"[bench] memory rates on this box in the AXPY kernel's shape: copy (1 read + 1 write stream) {ceilings['copy_GBs']:.0f} GB/s, "
+        f"1 read stream {ceilings['read_GBs']:.0f} GB/s, 2 read streams {ceilings['two_reads_GBs']:.0f} GB/s; "
+        f"plain grid-stride copy {ceilings['plain_copy_GBs']:.0f} GB/s")
     dev.close()
 
     # every benchmark configuration through the reference-shaped API (tensors from Tensor.alloc, so with

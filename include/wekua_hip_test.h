@@ -66,6 +66,13 @@ int wk_test_option(const char *name, int value);
 int wk_probe_launch(wk_stream *s, int kind, unsigned work_groups, unsigned threads, size_t lds_bytes, void *dst,
                     size_t dst_bytes);
 
+/* Memory-rate probes in the shape of the AXPY stream kernel (one wavefront per work-group, one 16-byte
+ * vector per lane, non-temporal loads, streaming stores): kind 0 copies src to dst, kind 1 only reads src,
+ * kind 2 reads src and dst.  The reading kinds write a vector to dst only where all four of its words (of
+ * src, or of src xor dst) equal `sentinel`: pass a value the data cannot hold.  They give the benchmark the
+ * rates this memory system reaches with fewer streams than AXPY's two reads and one write.  bytes % 16 == 0. */
+int wk_stream_probe(wk_stream *s, int kind, void *dst, const void *src, size_t bytes, unsigned sentinel);
+
 /* A plain device-to-device streaming copy kernel of known size, used only to calibrate
  * profiler byte counters against a known amount of traffic. */
 int wk_copy_kernel(wk_stream *s, void *dst, const void *src, size_t bytes);

@@ -12,7 +12,7 @@ ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 HEADER = os.path.join(ROOT, "include", "wekua_hip.h")
 TEST_HEADER = os.path.join(ROOT, "include", "wekua_hip_test.h")     # knobs for tests, benchmarks and profiles
 TEST_ONLY = {"wk_gemm_variant", "wk_gemm_variant_with_workspace", "wk_gemm_split_plan", "wk_gemm_force_variant",
-             "wk_test_option", "wk_copy_kernel", "wk_probe_launch"}
+             "wk_test_option", "wk_copy_kernel", "wk_probe_launch", "wk_stream_probe"}
 
 
 def declared_functions(headers=(HEADER, TEST_HEADER)):

@@ -79,6 +79,7 @@ SIGNATURES = {
                                 ctypes.POINTER(ctypes.c_uint32), ctypes.POINTER(u64), ctypes.POINTER(u64),
                                 ctypes.POINTER(ctypes.c_size_t)]),
     "wk_copy_kernel": (ci, [vp, vp, vp, sz]),
+    "wk_stream_probe": (ci, [vp, ctypes.c_int, vp, vp, sz, ctypes.c_uint]),
     "wk_test_option": (ci, [ctypes.c_char_p, ci]),
     "wk_probe_launch": (ci, [vp, ci, ctypes.c_uint, ctypes.c_uint, sz, vp, sz]),
     "wk_hadamard": (ci, [vp, ci, u64p, vp, u64, u64, vp, u64, u64]),

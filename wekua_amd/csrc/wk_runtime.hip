@@ -463,6 +463,41 @@ extern "C" int wk_probe_launch(wk_stream *s, int kind, unsigned work_groups, uns
     return launch_status();
 }
 
+// Memory-rate probes in the shape of the AXPY stream kernel: one wavefront per work-group, one 16-byte
+// vector per lane, non-temporal loads, streaming stores.  kind 0 copies src to dst (1 read + 1 write
+// stream), kind 1 only reads src (1 read stream), kind 2 reads src and dst (2 read streams).  The reading
+// kinds store a lane's vector only when all its words equal the sentinel the host passes, which the host
+// chooses so that it never happens; the loads stay because the compiler cannot know that.
+typedef unsigned u32x4_probe __attribute__((ext_vector_type(4)));
+__global__ __launch_bounds__(64) void stream_probe_kernel(int kind, u32x4_probe *__restrict__ dst, const u32x4_probe *__restrict__ src,
+                                                           size_t n16, unsigned sentinel) {
+    const size_t i = (size_t)blockIdx.x * 64 + threadIdx.x;
+    if (i >= n16) return;
+    u32x4_probe v = __builtin_nontemporal_load(src + i);
+    if (kind == 0) {
+        asm volatile("global_store_dwordx4 %0, %1, off nt sc0 sc1" ::"v"(dst + i), "v"(v) : "memory");
+        return;
+    }
+    if (kind == 2) {
+        const u32x4_probe w = __builtin_nontemporal_load(dst + i);
+        v ^= w;
+    }
+    if (v.x == sentinel && v.y == sentinel && v.z == sentinel && v.w == sentinel) dst[i] = v;
+}
+
+extern "C" int wk_stream_probe(wk_stream *s, int kind, void *dst, const void *src, size_t bytes, unsigned sentinel) {
+    int rc = bind(s);
+    if (rc) return rc;
+    if (kind < 0 || kind > 2 || !dst || !src || bytes % 16 || bytes / 16 / 64 >= 0x7fffffffull ||
+        (reinterpret_cast<uintptr_t>(dst) | reinterpret_cast<uintptr_t>(src)) % 16)
+        return WK_E_INVALID_VALUE;
+    if (!bytes) return WK_OK;
+    const size_t n16 = bytes / 16;
+    hipLaunchKernelGGL(stream_probe_kernel, dim3(static_cast<unsigned>((n16 + 63) / 64)), dim3(64), 0, s->stream, kind,
+                       static_cast<u32x4_probe *>(dst), static_cast<const u32x4_probe *>(src), n16, sentinel);
+    return launch_status();
+}
+
 extern "C" int wk_copy_kernel(wk_stream *s, void *dst, const void *src, size_t bytes) {
     int rc = bind(s);
     if (rc) return rc;
