@@ -610,6 +610,32 @@ def test_k_split_over_work_groups(dev, dtype):
         dA.free(); dB.free()
     finally:
         lib.wk_gemm_force_variant(b"auto")
+    # The hand-over of partial tiles between work-groups behind different L2s.  Nine tiles: the grid is
+    # (tiles, shares) and work-groups go to the eight XCDs in turn by linear number, tile + 9 * share, so
+    # the shares of one tile sit on XCDs tile + share (mod 8), eight neighbours on eight different ones.
+    # The same launch many times into a poisoned C, every result compared bit for bit with the first and
+    # the first with the oracle: a stale partial tile read by the adding work-group would show as a
+    # difference.  This is the test to run after a compiler or driver change.
+    M = N = 192
+    K = 8192
+    assert lib.wk_gemm_variant(did, 0, 1, M, N, K, K, K, N, None, None, None) == z
+    assert lib.wk_gemm_split_plan(did, 0, 1, M, N, K, None, shares, klen, first, tiles, nbytes) == 0
+    assert tiles.value == 9 and shares.value >= 8
+    check(dev, dtype, M, N, K, 0, 1, None, None, seed=91)
+    a = make_operand(dtype, (M, K), 92)
+    b = make_operand(dtype, (N, K), 93)
+    dA, dB = dev.upload(a), dev.upload(b)
+    dC = dev.upload(np.full((M, N), np.nan, dtype=rd))
+    first_bits = None
+    for launch in range(24):
+        dev.gemm(dtype, 0, 1, M, N, K, None, dA, K, dB, K, None, dC, N)
+        dev.sync()
+        got = dC.download(rd, (M, N))
+        if first_bits is None:
+            first_bits = got
+        assert np.array_equal(got, first_bits), f"launch {launch} differs from launch 0"
+        dC.write(np.full((M, N), np.nan, dtype=rd))
+    dA.free(); dB.free(); dC.free()
 
 
 @pytest.mark.parametrize("variant,bm,bn", [("mfma_f32_256x128d", 256, 128), ("mfma_f32_128x128d", 128, 128), ("mfma_f32_64x64d", 64, 64),

@@ -50,7 +50,6 @@ struct DArgs {
     uint32_t M, N, K;
     uint32_t lda, ldb, ldc;
     uint32_t tiles_m, tiles_n;
-    uint32_t num_cus;
     int epi;
     float alpha, beta;
     const float *bias; // kernels instantiated with EXT: C = act(acc + bias[col]); bias may be null
@@ -86,7 +85,7 @@ void gemm_f32_dma_kernel(DArgs g) {
     static_assert(!SK || KS == 1, "work dealt by k-slabs: one group of wavefronts");
     constexpr int SUB = 16 / VB;
     __shared__ uint32_t s_last;
-    auto run = [&](const uint32_t pid, const uint32_t kb, const uint32_t ke, const uint32_t bq, const bool stagger) __attribute__((always_inline)) {
+    auto run = [&](const uint32_t pid, const uint32_t kb, const uint32_t ke, const uint32_t bq) __attribute__((always_inline)) {
     constexpr int WM = BM / 2, WN = BN / 2, FM = WM / 32, FN = WN / 32;
     constexpr int S = BK / 8;   // fragment steps per slab (8 values of k each: four matrix instructions per block)
     constexpr int CPR = BK / 4; // 16-byte chunks per row of a k-contiguous slab
@@ -127,13 +126,6 @@ void gemm_f32_dma_kernel(DArgs g) {
         tile_n = in_group / gsz;
     }
     const uint32_t m0 = tile_m * BM, n0 = tile_n * BN;
-    // the second co-resident work-group of the first dispatch wave starts one solo iteration late, so
-    // that the two do not hand over at the same time
-    if (stagger && g.num_cus) {
-        const uint32_t slot = blockIdx.x / g.num_cus;
-        if (slot >= 1 && slot < (uint32_t)OCC)
-            for (uint32_t i = 0; i < slot * (FM * FN * BK / 4); ++i) __builtin_amdgcn_s_sleep(2);
-    }
 
     // position of a 16-byte chunk inside its row of a k-contiguous slab: chunk number ^ swizzle(row)
     auto swizzle = [](uint32_t row) -> uint32_t { return CPR == 4 ? (row >> 2) & 3u : (row >> 1) & 7u; };
@@ -614,7 +606,7 @@ void gemm_f32_dma_kernel(DArgs g) {
     else epilogue(std::true_type{});
     }; // run
     if constexpr (!SK) {
-        run(blockIdx.x, 0u, 0u, 0u, true);
+        run(blockIdx.x, 0u, 0u, 0u);
     } else {
         const uint32_t slabs_per_tile = (g.K + BK - 1) / BK;
         // work-groups b, b + 8, ... share an XCD: they take consecutive ranges, and with them neighbouring tiles
@@ -626,7 +618,7 @@ void gemm_f32_dma_kernel(DArgs g) {
             const uint32_t pid = u / slabs_per_tile, kb = u - pid * slabs_per_tile;
             const uint32_t ke = min(slabs_per_tile, kb + (u_end - u));
             if (!first) __syncthreads(); // every wavefront is done with the stages of the range before
-            run(pid, kb, ke, bq, first);
+            run(pid, kb, ke, bq);
             first = false;
             u += ke - kb;
         }
@@ -657,7 +649,6 @@ struct DArgsD {
     uint32_t M, N, K;
     uint32_t lda, ldb, ldc;
     uint32_t tiles_m, tiles_n;
-    uint32_t num_cus;
     int epi;
     double alpha, beta;
     const double *bias;
@@ -710,11 +701,6 @@ void gemm_f64_dma_kernel(DArgsD g) {
         tile_n = in_group / gsz;
     }
     const uint32_t m0 = tile_m * BM, n0 = tile_n * BN;
-    if (g.num_cus) { // co-resident work-groups of the first dispatch wave start one solo iteration apart
-        const uint32_t slot = blockIdx.x / g.num_cus;
-        if (slot >= 1 && slot < (uint32_t)OCC)
-            for (uint32_t i = 0; i < slot * (FM * FN * BK / 8); ++i) __builtin_amdgcn_s_sleep(2);
-    }
 
     // ---- global side ----
     // Ragged shapes as in the f32 kernel: rows (columns) beyond the matrix are fetched from its last one, a
@@ -1038,7 +1024,6 @@ template <int BM, int BN, int BK, int NS, int OCC, int VB = 16> int launch_tile_
     g.lda = (uint32_t)p.lda; g.ldb = (uint32_t)p.ldb; g.ldc = (uint32_t)p.ldc;
     g.tiles_m = (uint32_t)((p.M + BM - 1) / BM);
     g.tiles_n = (uint32_t)((p.N + BN - 1) / BN);
-    g.num_cus = p.num_cus;
     g.epi = p.epi;
     std::memcpy(&g.alpha, p.alpha, sizeof(double));
     std::memcpy(&g.beta, p.beta, sizeof(double));
@@ -1116,7 +1101,6 @@ template <int BM, int BN, int BK, int NS, int OCC, int KS = 1, int VB = 16, bool
     g.lda = (uint32_t)p.lda; g.ldb = (uint32_t)p.ldb; g.ldc = (uint32_t)p.ldc;
     g.tiles_m = (uint32_t)((p.M + BM - 1) / BM);
     g.tiles_n = (uint32_t)((p.N + BN - 1) / BN);
-    g.num_cus = p.num_cus;
     g.epi = p.epi;
     std::memcpy(&g.alpha, p.alpha, sizeof(float));
     std::memcpy(&g.beta, p.beta, sizeof(float));

@@ -54,7 +54,6 @@ template <typename T> struct MArgs {
     uint32_t M, N, K;
     uint32_t lda, ldb, ldc;
     uint32_t tiles_m, tiles_n;
-    uint32_t num_cus; // compute units of the device (0 disables the start-up stagger)
     uint32_t xcd_remap; // 1: renumber work-groups so that each XCD gets a contiguous run of tiles
     int epi;
     T alpha, beta;
@@ -72,21 +71,6 @@ template <typename T> struct MArgs {
     // and a tail whose k is split; the tail's tile numbers follow the body's)
     uint32_t pid_offset;
 };
-
-// Work-groups that share a CU start in lock step (the whole first wave of work-groups is
-// dispatched at once) and, doing identical work, stay in lock step: they reach the slab
-// hand-over (LDS store, barrier, fragment reload) at the same time and the matrix pipe idles.
-// Delaying the k-th co-resident work-group of the first dispatch wave by k solo-iterations
-// keeps one of them in its matrix phase while the other hands over.  Later work-groups
-// inherit the offset of the one whose slot they take.  Measured on MI355X at 8192^3 f32 with
-// the 256x128 tile: 132 -> 141 TFLOP/s.
-__device__ __forceinline__ void startup_stagger(uint32_t num_cus, uint32_t occupancy, uint32_t units_per_slot) {
-    if (num_cus == 0) return;
-    const uint32_t slot = blockIdx.x / num_cus;
-    if (slot == 0 || slot >= occupancy) return;
-    const uint32_t n = slot * units_per_slot;
-    for (uint32_t i = 0; i < n; ++i) __builtin_amdgcn_s_sleep(2); // 2 * 64 clocks
-}
 
 // blockIdx.x -> (tile_m, tile_n): grouped walk, GROUP_M tile rows at a time.
 // Work-groups are dealt to the 8 XCDs round-robin (work-group b runs on XCD b % 8; checked by
@@ -160,7 +144,6 @@ void gemm_f32_mfma_kernel(MArgs<float> g) {
         g.K = k_end - k_begin;
     }
     // one solo iteration = FM*FN*BK/2 matrix instructions of 64 clocks = FM*FN*BK/4 sleep units
-    startup_stagger(g.num_cus, OCC, FM * FN * BK / 4);
 
     f32x16 acc[FM][FN];
 #pragma unroll
@@ -718,7 +701,6 @@ void gemm_f64_mfma_kernel(MArgs<double> g) {
         g.K = k_end - k_begin;
     }
     // one solo iteration = FM*FN*BK/4 matrix instructions of 64 clocks = FM*FN*BK/8 sleep units
-    startup_stagger(g.num_cus, OCC, FM * FN * BK / 8 > 0 ? FM * FN * BK / 8 : 1);
 
     f64x4 acc[FM][FN];
 #pragma unroll
@@ -1109,7 +1091,6 @@ template <typename T> MArgs<T> make_args(const GemmProblem &p, int bm, int bn) {
     g.lda = (uint32_t)p.lda; g.ldb = (uint32_t)p.ldb; g.ldc = (uint32_t)p.ldc;
     g.tiles_m = (uint32_t)((p.M + bm - 1) / bm);
     g.tiles_n = (uint32_t)((p.N + bn - 1) / bn);
-    g.num_cus = p.num_cus;
     // Small launches (every tile resident at once) run out of the per-XCD L2: give each XCD a
     // compact run of tiles.  Large launches stream from the shared Infinity Cache: keep the XCDs on
     // the same B panel (see tile_coords).  Measured: 1024^3 f32 48 -> 62 TFLOP/s with the
