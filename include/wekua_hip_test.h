@@ -57,7 +57,11 @@ int wk_gemm_force_variant(const char *name);
  *   "alloc_colours"  0: wk_malloc returns blocks as the device allocator hands them out (default 1:
  *                       blocks of 1 MiB and more start 0 / 3 / 6 / 9 KiB into their allocation in turn);
  *   "stream_k"       0: the automatic choice never takes the kernels that deal their work by k-slabs
- *                       ("...k") (default 1). */
+ *                       ("...k") (default 1); 2: those kernels deal every tile's k-slabs instead of running the
+ *                       whole rounds of tiles whole;
+ *   "strips"         0: a product is never multiplied in parts (body of whole tiles + strips); 2: thin strips are
+ *                       split off whatever the cost model says (default 1: where the model puts the parts below
+ *                       the whole). */
 int wk_test_option(const char *name, int value);
 
 /* Launch-cost probes for profiles: a kernel with the grid, work-group size (a multiple of 64) and dynamic LDS

@@ -561,6 +561,45 @@ def test_work_dealt_by_k_slabs(dev, op_a, op_b):
         d.free()
 
 
+@pytest.mark.parametrize("variant,mode,M,N,K,ops", [
+    ("mfma_f32_128x128k", 1, 2300, 2500, 700, (0, 0)),    # 360 tiles: 256 run whole, the k-slabs of 104 dealt to 256 work-groups
+    ("mfma_f32_128x128k", 2, 2300, 2500, 700, (1, 0)),    # the same product with every tile dealt (768 work-groups)
+    ("mfma_f32_256x128k", 1, 4100, 4200, 300, (0, 1)),    # 561 tiles of 256 x 128: two whole rounds, 49 tiles dealt
+    ("mfma_f32_256x128k", 1, 2300, 2500, 700, (1, 1)),    # 180 tiles, fewer than compute units: all dealt
+    ("mfma_f32_128x128k", 1, 2048, 4096, 520, (0, 0)),    # 512 tiles, whole rounds: the last round dealt one tile each
+    ("mfma_f32_128x128k", 1, 1000, 900, 2000, (1, 0)),    # 64 tiles over 768 work-groups: a dozen parts per tile
+    ("mfma_f32_256x128k", 2, 4100, 4200, 300, (0, 0))])
+def test_work_dealt_by_k_slabs_in_every_form(dev, variant, mode, M, N, K, ops):
+    """The kernels that deal k-slabs, forced, in both of their plans (whole rounds of tiles run whole and the rest
+    dealt; every tile dealt) and on tile counts below, between and at whole rounds of the compute units: every
+    entry against the oracle and the same bits on three runs."""
+    op_a, op_b = ops
+    a, b, c = gemm_operands("f32", M, N, K, op_a, op_b, 131 + mode)
+    lda, ldb = a.shape[1], b.shape[1]
+    assert lda % 4 == 0 and ldb % 4 == 0, "these kernels take rows that start on 16-byte boundaries"
+    want = oracle.gemm("f32", 1.5, a, op_a, b, op_b, 0.5, c, threads=0)
+    dA, dB = dev.upload(a), dev.upload(b)
+    assert dev.lib.wk_gemm_force_variant(variant.encode()) == 0
+    assert dev.lib.wk_test_option(b"stream_k", mode) == 0
+    try:
+        first = None
+        for _ in range(3):
+            dC = dev.upload(c)
+            dev.gemm("f32", op_a, op_b, M, N, K, 1.5, dA, lda, dB, ldb, 0.5, dC, N)
+            dev.sync()
+            got = dC.download(np.float32, c.shape)
+            dC.free()
+            if first is None:
+                first = got
+                assert_gemm_close("f32", got, want, 1.5, a, op_a, b, op_b, 0.5, c, K, what=f"{variant}, plan {mode}")
+            else:
+                assert np.array_equal(got, first), "the bits depend on the run"
+    finally:
+        dev.lib.wk_test_option(b"stream_k", 1)
+        dev.lib.wk_gemm_force_variant(b"auto")
+        dA.free(); dB.free()
+
+
 @pytest.mark.parametrize("dtype", ["f32", "f64"])
 def test_k_split_over_work_groups(dev, dtype):
     """Few tiles of C and a long k: every tile goes to several work-groups, whose partial tiles meet in

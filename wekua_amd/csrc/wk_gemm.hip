@@ -136,11 +136,11 @@ void make_parts(const GemmProblem &p, uint64_t Mb, uint64_t Nb, StripPlan &out) 
 }
 
 bool plan_strips(const GemmProblem &p, StripPlan &out) {
-    if ((p.dtype != WK_F32 && p.dtype != WK_F64) || p.ext || p.K < 512) return false;
+    if ((p.dtype != WK_F32 && p.dtype != WK_F64) || p.ext || p.K < 512 || !g_test_options.strips) return false;
     if (!(p.dtype == WK_F32 ? gemm_f32_dma_applies(p, 128, 128) : gemm_f64_dma_applies(p, 128, 128))) return false;
     const uint64_t bn = 128, big = p.dtype == WK_F32 ? 256 : 128;
     // (1) thin strips -- at most a quarter of the tile's rows (256 or 128 of them: the large tiles) or of its 128
-    // columns: always, when the body is large enough to carry the extra launches
+    // columns: when the body is large enough to carry the extra launches and the model agrees
     {
         uint64_t bm = big;
         if (bm == 256 && (p.M % 256 == 0 || p.M % 256 > 64)) bm = 128;
@@ -149,23 +149,30 @@ bool plan_strips(const GemmProblem &p, StripPlan &out) {
         const uint64_t Mb = thin_m ? p.M - m_rem : p.M, Nb = thin_n ? p.N - n_rem : p.N;
         if ((thin_m || thin_n) && Mb * Nb >= (1ull << 22)) { // (2048 x 2047 and below: N,N gains 7 %, T,N loses as much)
             make_parts(p, Mb, Nb, out);
-            // ... unless the whole product would have its work dealt by k-slabs, which does not care about a started
-            // round, and the model puts that below the parts (2200^3: 113 TFLOP/s whole, 102 in parts)
+            if (g_test_options.strips == 2) return true;
+            // Strips of at most four rows or columns go to the thin-product kernels, which read the long operand once
+            // (16-46 us): split off as ever (4096 x 4100 x 1024: 128 TFLOP/s against 107 whole, 2050 x 4097 x 1536 125
+            // against 120, f64 2049 x 2050 x 1024 58 against 54), unless the whole product would have its work dealt
+            // by k-slabs -- such a launch does not pay for a started round -- and the model puts it below the parts.
+            // Wider strips are launches of tile kernels, 20 us and more each: the model decides (2200^3: 123 TFLOP/s
+            // whole against 106 in parts, 4000^3 138 against 130, 2312 x 2304 x 2304 127 against 120).
+            bool all_thin = true;
+            for (int i = 1; i < out.parts; ++i) all_thin = all_thin && gemm_thin_applies(out.part[i]);
             double whole = 0.0;
             const int wv = gemm_mfma_pick(p, &whole);
-            const char *wname = wv >= 0 ? gemm_mfma_variant_name(wv) : nullptr;
-            if (wname && wname[std::strlen(wname) - 1] == 'k') {
-                const double launch = 4.0 * 3.05e5 / (double)p.K;
-                double sum = 0.0;
-                for (int i = 0; i < out.parts; ++i) {
-                    double c = 0.0;
-                    if (gemm_thin_applies(out.part[i])) c = 5.0 * launch; // (a thin product reads the long operand once: 16-46 us)
-                    else if (gemm_mfma_pick(out.part[i], &c) < 0) return true;
-                    sum += c + (i ? launch : 0.0);
-                }
-                if (sum >= whole) return false;
+            if (wv < 0) return true;
+            const char *wname = gemm_mfma_variant_name(wv);
+            const bool whole_dealt = wname && wname[0] && wname[std::strlen(wname) - 1] == 'k';
+            if (all_thin && !whole_dealt) return true;
+            const double launch = 4.0 * (p.dtype == WK_F32 ? 3.05e5 : 1.525e5) / (double)p.K;
+            double sum = 0.0;
+            for (int i = 0; i < out.parts; ++i) {
+                double c = 0.0;
+                if (gemm_thin_applies(out.part[i])) c = 5.0 * launch; // (a thin product reads the long operand once)
+                else if (gemm_mfma_pick(out.part[i], &c) < 0) return true;
+                sum += c + (i ? launch : 0.0);
             }
-            return true;
+            return sum < whole;
         }
     }
     // (2) any remainder beyond whole large tiles, where the cost model puts the parts, with a launch each, well
@@ -176,7 +183,12 @@ bool plan_strips(const GemmProblem &p, StripPlan &out) {
     // a launch more: about 4 us in the model's unit (cost x k / 3.05e5 = microseconds in f32, half that rate in f64)
     const double launch = 4.0 * (p.dtype == WK_F32 ? 3.05e5 : 1.525e5) / (double)p.K;
     const uint64_t m_rem = p.M > big ? p.M % big : 0, n_rem = p.N > bn ? p.N % bn : 0;
-    double best = 0.95 * whole;
+    // (a whole whose work is dealt by k-slabs was already chosen with a margin of its own, and the model prices the
+    // parts a few per cent too high: 4296 x 4096 x 4096 142 TFLOP/s in parts against 139 dealt, 4096 x 4160 x 4096 143 / 139)
+    const int whole_v = gemm_mfma_pick(p, nullptr);
+    const char *whole_name = whole_v >= 0 ? gemm_mfma_variant_name(whole_v) : "";
+    const bool whole_dealt = whole_name[0] && whole_name[std::strlen(whole_name) - 1] == 'k';
+    double best = (whole_dealt ? 1.03 : 0.95) * whole;
     bool found = false;
     for (int cand = 1; cand < 4; ++cand) {
         const bool sm = cand & 1, sn = cand & 2;

@@ -57,7 +57,9 @@ struct DArgs {
     uint32_t patch_m, patch_n; // tile walk in XCD-local patches of patch_m x patch_n tiles (0: rows of groups)
     // kernels instantiated with SK (work dealt by k-slabs, not by tiles): k-slabs per work-group, k-slabs in all
     // (tiles x slabs per tile), memory for two partial tiles per work-group and one arrival counter per tile
-    uint32_t sk_units, sk_total;
+    // sk_first: the tiles before that one are run whole, one work-group each (work-groups sk_groups ... of the
+    // launch); the k-slabs of the tiles from it on are dealt to work-groups 0 ... sk_groups - 1
+    uint32_t sk_units, sk_total, sk_first, sk_groups;
     float *partials;
     uint32_t *counters;
 };
@@ -484,7 +486,7 @@ void gemm_f32_dma_kernel(DArgs g) {
             // buffer instructions' auxiliary operand): the parts of a tile come from different XCDs.
             constexpr size_t TILE = (size_t)BM * BN;
             constexpr int SC1 = 16;
-            const uint32_t U = g.sk_units, t0 = pid * slabs_per_tile;
+            const uint32_t U = g.sk_units, t0 = (pid - g.sk_first) * slabs_per_tile;
             const uint32_t b_first = t0 / U, b_last = (t0 + slabs_per_tile - 1) / U; // the work-groups that hold parts of it
             const uint32_t nparts = b_last - b_first + 1;
             // The part that starts the tile is the last of its work-group's range, so it is usually the last to be
@@ -609,16 +611,20 @@ void gemm_f32_dma_kernel(DArgs g) {
         run(blockIdx.x, 0u, 0u, 0u);
     } else {
         const uint32_t slabs_per_tile = (g.K + BK - 1) / BK;
+        if (blockIdx.x >= g.sk_groups) { // a whole tile
+            run(blockIdx.x - g.sk_groups, 0u, slabs_per_tile, 0u);
+            return;
+        }
         // work-groups b, b + 8, ... share an XCD: they take consecutive ranges, and with them neighbouring tiles
-        const uint32_t bq = (blockIdx.x & 7u) * (gridDim.x >> 3) + (blockIdx.x >> 3);
+        const uint32_t bq = (blockIdx.x & 7u) * (g.sk_groups >> 3) + (blockIdx.x >> 3);
         uint32_t u = bq * g.sk_units;
         const uint32_t u_end = min(u + g.sk_units, g.sk_total);
         bool first = true;
         while (u < u_end) {
-            const uint32_t pid = u / slabs_per_tile, kb = u - pid * slabs_per_tile;
+            const uint32_t t = u / slabs_per_tile, kb = u - t * slabs_per_tile;
             const uint32_t ke = min(slabs_per_tile, kb + (u_end - u));
             if (!first) __syncthreads(); // every wavefront is done with the stages of the range before
-            run(pid, kb, ke, bq);
+            run(g.sk_first + t, kb, ke, bq);
             first = false;
             u += ke - kb;
         }
@@ -1077,17 +1083,28 @@ int launch_one(hipStream_t st, const DArgs &g, uint64_t first_tiles, unsigned sk
     return launch_status();
 }
 
-// How the work-groups of a launch that deals its work by k-slabs share it: groups = compute units x occ (a
-// multiple of eight), units = ceil(tiles x slabs per tile / groups) slabs each.  false: the problem does not fit
-// (no scratch for two partial tiles per work-group, more tiles than counters, 32-bit slab numbers).
-bool stream_k_plan(const GemmProblem &p, int bm, int bn, int bk, int occ, unsigned &groups, uint32_t &units, uint32_t &total) {
+// How the work-groups of a launch that deals its work by k-slabs share it.  With at least as many tiles as
+// compute units, the whole rounds of tiles (one tile per unit and round) are run whole, one work-group each, and
+// only the k-slabs of the tiles that are left are dealt, to one work-group per unit: every unit then has the same
+// amount of matrix work, few tiles are split, and the dealt work-groups -- the first of the launch, so the first to
+// start -- are done and their parts added up while the whole tiles are still being multiplied.  With fewer tiles
+// than units (or with the test option "stream_k" at 2) all tiles are dealt, to as many work-groups as are
+// resident at once (units x occ).  groups: the work-groups that take dealt k-slabs (a multiple of eight), units
+// = ceil(dealt tiles x slabs per tile / groups) slabs each, first: the number of tiles run whole.  false: the
+// problem does not fit (no scratch for two partial tiles per dealt work-group, more tiles than counters,
+// 32-bit slab numbers).
+bool stream_k_plan(const GemmProblem &p, int bm, int bn, int bk, int occ, unsigned &groups, uint32_t &units, uint32_t &total,
+                   uint32_t &first) {
     const uint64_t tiles = ((p.M + bm - 1) / bm) * ((p.N + bn - 1) / bn), slabs = (p.K + bk - 1) / bk;
     const uint64_t cus = p.num_cus ? p.num_cus : 256;
-    groups = (unsigned)(cus * occ);
+    uint64_t whole = g_test_options.stream_k == 2 || tiles < cus ? 0 : tiles / cus * cus;
+    if (whole == tiles) whole -= cus; // (a launch of whole rounds has no use for this: deal the last round)
+    groups = (unsigned)(whole ? cus : cus * occ);
     if (groups % 8 || !p.scratch || !p.counters || tiles > p.num_counters || tiles * slabs > 0x7fffffffull) return false;
     if ((uint64_t)2 * groups * bm * bn * sizeof(float) > p.scratch_bytes) return false;
-    total = (uint32_t)(tiles * slabs);
-    units = (uint32_t)((tiles * slabs + groups - 1) / groups);
+    first = (uint32_t)whole;
+    total = (uint32_t)((tiles - whole) * slabs);
+    units = (uint32_t)(((tiles - whole) * slabs + groups - 1) / groups);
     return units >= 1;
 }
 
@@ -1121,7 +1138,9 @@ template <int BM, int BN, int BK, int NS, int OCC, int KS = 1, int VB = 16, bool
     const int sel = (p.op_a ? 0 : 2) | (p.op_b ? 1 : 0); // bit 1: A k-contiguous, bit 0: B k-contiguous
     unsigned sk_groups = 0;
     if constexpr (SK) {
-        if (first_tiles || !stream_k_plan(p, BM, BN, BK, OCC, sk_groups, g.sk_units, g.sk_total)) return WK_E_INVALID_VALUE;
+        if (first_tiles || !stream_k_plan(p, BM, BN, BK, OCC, sk_groups, g.sk_units, g.sk_total, g.sk_first)) return WK_E_INVALID_VALUE;
+        g.sk_groups = sk_groups;
+        sk_groups += g.sk_first; // the launch: the dealt work-groups, then one per whole tile
         g.partials = static_cast<float *>(p.scratch);
         g.counters = p.counters;
         g.patch_m = g.patch_n = 0; // consecutive tile numbers are neighbours in the row-group walk
@@ -1193,8 +1212,8 @@ int wk::gemm_f64_dma_launch(hipStream_t st, const GemmProblem &p, int bm, int bn
 bool wk::gemm_f32_dma_stream_k_applies(const GemmProblem &p, int bm, int bn) {
     if (!(bn == 128 && (bm == 256 || bm == 128)) || !gemm_f32_dma_applies(p, bm, bn) || !f32_rows_aligned(p)) return false;
     unsigned groups;
-    uint32_t units, total;
-    return stream_k_plan(p, bm, bn, 16, bm == 256 ? 2 : 3, groups, units, total);
+    uint32_t units, total, first;
+    return stream_k_plan(p, bm, bn, 16, bm == 256 ? 2 : 3, groups, units, total, first);
 }
 
 int wk::gemm_f32_dma_stream_k_launch(hipStream_t st, const GemmProblem &p, int bm, int bn) {

@@ -1609,25 +1609,29 @@ int wk::gemm_mfma_pick(const GemmProblem &p, double *cost_out) {
                     }
         }
     }
-    // Tiles that do not fill whole rounds: the 128 x 128 kernel with the work dealt by k-slabs (every unit busy for
-    // the same time) where that beats what was found above by more than the model's error.  Its time is that of
-    // the tiles spread evenly over the units plus about 22 us per launch, whatever the shape: the parts of split
-    // tiles meet in memory and every work-group runs its epilogue at the same moment (this form reproduces the
-    // measured launches from 2200^3 to 4200^3 and 2048 x 4096 x 1024 to 3 %).  Measured against the choice without
-    // it, N,N, TFLOP/s: 2200^3 102 -> 113, 2300^3 115 -> 126, 2500^3 116 -> 122, 3000^3 125 -> 131, 3700^3 123 -> 133,
-    // 4000^3 129 -> 135, 3000 x 3000 x 8192 126 -> 135, 2500 x 3500 x 4096 121 -> 130, 5000 x 3000 x 2000 120 -> 128; no
-    // gain where whole rounds or split-off strips fit anyway (2816^3, 3200^3, 4200^3), a loss on 2048 x 4096 x 1024
-    // (121 against 134).  Beyond some 1100 tiles the work-groups of an XCD, each on its own run of tiles, no longer
-    // share their panels in the L2 (5000^3 131 against 135, 6500^3 120 against 142): not taken there.  The 256 x 128
-    // tile dealt the same way (mfma_f32_256x128k) wins nowhere by more than a percent.
-    if (p.dtype == WK_F32 && best >= 0 && p.K >= 1536 && g_test_options.stream_k) { // (k = 1024: 4200 x 4096 x 1024 128 against 131 in parts)
-        constexpr double SK_FIXED_US = 22.0, COST_PER_US = 3.05e5, SK_MAX_TILES = 1100.0;
-        const double tiles = (double)((p.M + 127) / 128) * (double)((p.N + 127) / 128);
-        if (tiles > cus && tiles <= SK_MAX_TILES && std::fmod(tiles, cus * 3.0) != 0.0 && gemm_f32_dma_stream_k_applies(p, 128, 128)) {
-            const double cost = tiles / cus * 128.0 * 128.0 / 0.922 + SK_FIXED_US * COST_PER_US / (double)p.K;
-            if (cost < 0.97 * best_cost)
+    // Tiles that do not come out even over the compute units: the whole rounds of tiles run whole and the k-slabs of
+    // the tiles that are left are dealt to one more work-group per unit (the "...k" kernels, wk_gemm_dma.hip), so
+    // that every unit has the same amount of matrix work, where that beats what was found above by more than the
+    // model's error.  Fitted on cubes from 2200 to 6000 and six other shapes (N,N): the time is that of tiles / units
+    // tile times at an efficiency of 0.90 (128 x 128) / 0.933 (256 x 128) plus 15 / 36 us per launch (the dealt
+    // work-groups are done early, and their parts are added while the whole tiles are still being multiplied;
+    // with every tile dealt, as at first, the exchange stood at the end of the launch and cost 22 us).
+    // Measured against the choice without it, N,N, TFLOP/s: 2200^3 100 -> 118, 2300^3 112 -> 130, 2500^3 113 -> 127,
+    // 2700^3 113 -> 126, 3000^3 122 -> 132, 3200^3 126 -> 140, 3500^3 124 -> 132, 3700^3 123 -> 138, 4000^3 130 -> 137,
+    // 4500^3 129 -> 135, 5000^3 133 -> 136, 6000^3 134 -> 141, 3000 x 3000 x 8192 124 -> 136, 2500 x 3500 x 4096 123 ->
+    // 133, 3333 x 3333 x 1111 105 -> 123; nothing to gain where the tiles are whole rounds (2048 x 4096 x 1024).
+    if (p.dtype == WK_F32 && best >= 0 && p.K >= 1024 && g_test_options.stream_k) {
+        constexpr double COST_PER_US = 3.05e5;
+        static const struct { const char *name; int bm, bn; double eff, fixed_us; } dealt[] = {
+            {"mfma_f32_128x128k", 128, 128, 0.90, 15.0}, {"mfma_f32_256x128k", 256, 128, 0.933, 36.0}};
+        const double plain_cost = best_cost;
+        for (const auto &d : dealt) {
+            const double tiles = (double)((p.M + d.bm - 1) / d.bm) * (double)((p.N + d.bn - 1) / d.bn);
+            if (tiles <= cus || std::fmod(tiles, cus) == 0.0 || !gemm_f32_dma_stream_k_applies(p, d.bm, d.bn)) continue;
+            const double cost = tiles / cus * d.bm * d.bn / d.eff + d.fixed_us * COST_PER_US / (double)p.K;
+            if (cost < 0.97 * plain_cost && cost < best_cost)
                 for (int w = 0; w < k_num_variants; ++w)
-                    if (!std::strcmp(k_variants[w].name, "mfma_f32_128x128k")) {
+                    if (!std::strcmp(k_variants[w].name, d.name)) {
                         best = w;
                         best_cost = cost;
                     }

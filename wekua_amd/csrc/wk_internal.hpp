@@ -44,7 +44,8 @@ struct TestOptions {
     int gemm_walk_rows = 0; // 1: the direct-to-LDS kernels walk the tiles in groups of rows, not XCD-local patches
     int tail_strict = 0;    // 1: forced k-split tail variants plan like the automatic choice
     int alloc_colours = 1;  // 0: wk_malloc hands out blocks as hipMalloc returns them
-    int stream_k = 1;       // 0: the automatic choice never deals work by k-slabs
+    int stream_k = 1;       // 0: the automatic choice never deals work by k-slabs; 2: every tile dealt, none run whole
+    int strips = 1;         // 0: products are never multiplied in parts; 2: thin strips split off whatever the model says
 };
 extern TestOptions g_test_options;
 
