@@ -1629,7 +1629,7 @@ int wk::gemm_mfma_pick(const GemmProblem &p, double *cost_out) {
             const double tiles = (double)((p.M + d.bm - 1) / d.bm) * (double)((p.N + d.bn - 1) / d.bn);
             if (tiles <= cus || std::fmod(tiles, cus) == 0.0 || !gemm_f32_dma_stream_k_applies(p, d.bm, d.bn)) continue;
             const double cost = tiles / cus * d.bm * d.bn / d.eff + d.fixed_us * COST_PER_US / (double)p.K;
-            if (cost < 0.97 * plain_cost && cost < best_cost)
+            if (cost < 0.98 * plain_cost && cost < best_cost)
                 for (int w = 0; w < k_num_variants; ++w)
                     if (!std::strcmp(k_variants[w].name, d.name)) {
                         best = w;
