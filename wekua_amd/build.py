@@ -79,15 +79,18 @@ def build_host(verbose: bool = False) -> str:
 
 
 def build_example(verbose: bool = False) -> str:
-    """The C++ usage example of the host mirror (benchmark/gemm.zig's flow); built to keep it compiling."""
-    src = os.path.join(HOST, "example_gemm.cpp")
-    if not os.path.exists(src):
-        return ""
-    exe = os.path.join(OBJ, "example_gemm")
-    out = _run(["g++", "-O2", "-std=c++20", "-Wall", "-Wextra", "-I" + INCLUDE, "-I" + HOST, src, "-o", exe,
-                "-L" + PKG, "-lwekua_hip", "-Wl,-rpath," + PKG])
-    if verbose and out.strip():
-        print(out)
+    """The C++ programs on the host mirror: the usage example (benchmark/gemm.zig's flow) and the reference
+    benchmark's size sweeps; built every time to keep them compiling."""
+    exe = ""
+    for name in ("example_gemm", "benchmark_sweep"):
+        src = os.path.join(HOST, name + ".cpp")
+        if not os.path.exists(src):
+            continue
+        exe = os.path.join(OBJ, name)
+        out = _run(["g++", "-O2", "-std=c++20", "-Wall", "-Wextra", "-I" + INCLUDE, "-I" + HOST, src, "-o", exe,
+                    "-L" + PKG, "-lwekua_hip", "-Wl,-rpath," + PKG])
+        if verbose and out.strip():
+            print(out)
     return exe
 
 
