@@ -79,7 +79,7 @@ def test_float_small_shapes(dev, dtype, op_a, op_b, alpha, beta):
 @pytest.mark.parametrize("variant", ["tile64", "mfma_f32_64x64", "mfma_f32_64x64s2", "mfma_f32_64x64s4", "mfma_f32_32x32s4",
                                      "mfma_f32_64x64z", "mfma_f32_128x128", "mfma_f32_128x128s2", "mfma_f32_256x128",
                                      "mfma_f32_128x128t", "mfma_f32_256x128t", "mfma_f32_256x128d", "mfma_f32_128x128d", "mfma_f32_64x64d",
-                                     "mfma_f32_128x128d2", "mfma_f32_64x64d2", "mfma_f32_256x128k", "mfma_f32_128x128k"])
+                                     "mfma_f32_128x128d2", "mfma_f32_64x64d2", "mfma_f32_256x128k", "mfma_f32_128x128k", "mfma_f32_64x64k"])
 @pytest.mark.parametrize("op_a,op_b", OPS)
 def test_f32_every_variant(dev, variant, op_a, op_b):
     import ctypes
@@ -491,7 +491,8 @@ def test_one_round_launches_take_the_k_split_tiles(dev):
     assert name("f32", 1000, 1000, 1000) == b"mfma_f32_64x64d2"    # ragged, rows of 4000 bytes
     assert name("f32", 2048, 1024, 1024) == b"mfma_f32_64x64d"     # two rounds
     assert name("f32", 1024, 1024, 128) == b"mfma_f32_64x64d"      # short k
-    assert name("f32", 1536, 1536, 1536) == b"mfma_f32_64x64d"
+    assert name("f32", 1536, 1536, 1536) == b"mfma_f32_64x64k"     # 2.25 tiles per compute unit: two rounds whole, the rest dealt by k-slabs
+    assert name("f32", 1408, 1408, 1408) == b"mfma_f32_64x64d"     # 1.89: nearly two whole rounds
     assert name("f32", 2048, 2048, 2048) == b"mfma_f32_128x128d2"  # one full round of 128x128 tiles
     assert name("f32", 2040, 2040, 2040) == b"mfma_f32_128x128d2"
     assert name("f32", 2048, 2048, 512) == b"mfma_f32_128x128d"
@@ -568,7 +569,11 @@ def test_work_dealt_by_k_slabs(dev, op_a, op_b):
     ("mfma_f32_256x128k", 1, 2300, 2500, 700, (1, 1)),    # 180 tiles, fewer than compute units: all dealt
     ("mfma_f32_128x128k", 1, 2048, 4096, 520, (0, 0)),    # 512 tiles, whole rounds: the last round dealt one tile each
     ("mfma_f32_128x128k", 1, 1000, 900, 2000, (1, 0)),    # 64 tiles over 768 work-groups: a dozen parts per tile
-    ("mfma_f32_256x128k", 2, 4100, 4200, 300, (0, 0))])
+    ("mfma_f32_256x128k", 2, 4100, 4200, 300, (0, 0)),
+    ("mfma_f32_64x64k", 1, 1100, 1300, 1500, (0, 0)),     # 378 tiles of 64 x 64: 256 whole, 122 dealt
+    ("mfma_f32_64x64k", 1, 1800, 1700, 600, (1, 0)),      # 783 tiles: three whole rounds (the last starts as slots free up), 15 dealt
+    ("mfma_f32_64x64k", 1, 900, 1000, 1100, (0, 1)),      # 240 tiles, fewer than compute units: all dealt
+    ("mfma_f32_64x64k", 2, 1100, 1300, 1500, (1, 1))])
 def test_work_dealt_by_k_slabs_in_every_form(dev, variant, mode, M, N, K, ops):
     """The kernels that deal k-slabs, forced, in both of their plans (whole rounds of tiles run whole and the rest
     dealt; every tile dealt) and on tile counts below, between and at whole rounds of the compute units: every

@@ -369,7 +369,7 @@ void gemm_f32_dma_kernel(DArgs g) {
     // The one-block-per-wavefront tile fetches C_old ahead of everything else (16 registers): its launches
     // are short and the latency of that read at the end of a tile is a visible share of them.  These loads
     // are older than every slab load, so the counted waits below cover them as well.
-    constexpr bool PRELOAD_C = FM * FN == 1;
+    constexpr bool PRELOAD_C = FM * FN == 1 && !SK; // (a dealt work-group does not know yet whether it will run its tile's epilogue)
     float c_old[PRELOAD_C ? 16 : 1];
     if constexpr (PRELOAD_C) {
         if (g.epi == EPI_ALPHA_BETA && (KS == 1 || kg == 0)) {
@@ -1208,17 +1208,18 @@ int wk::gemm_f64_dma_launch(hipStream_t st, const GemmProblem &p, int bm, int bn
     return launch_tile_d<64, 64, 16, 3, 3>(st, p);
 }
 
-// work dealt by k-slabs (the 256 x 128 and 128 x 128 tiles, rows that start on 16-byte boundaries)
+// work dealt by k-slabs (rows that start on 16-byte boundaries)
 bool wk::gemm_f32_dma_stream_k_applies(const GemmProblem &p, int bm, int bn) {
-    if (!(bn == 128 && (bm == 256 || bm == 128)) || !gemm_f32_dma_applies(p, bm, bn) || !f32_rows_aligned(p)) return false;
+    if (!gemm_f32_dma_applies(p, bm, bn) || !f32_rows_aligned(p) || p.ext) return false;
     unsigned groups;
     uint32_t units, total, first;
-    return stream_k_plan(p, bm, bn, 16, bm == 256 ? 2 : 3, groups, units, total, first);
+    return stream_k_plan(p, bm, bn, bm == 64 ? 32 : 16, bm == 256 ? 2 : 3, groups, units, total, first);
 }
 
 int wk::gemm_f32_dma_stream_k_launch(hipStream_t st, const GemmProblem &p, int bm, int bn) {
     if (!gemm_f32_dma_stream_k_applies(p, bm, bn)) return WK_E_INVALID_VALUE;
     if (bm == 256) return launch_tile<256, 128, 16, 3, 2, 1, 16, true>(st, p, 0);
+    if (bm == 64) return launch_tile<64, 64, 32, 3, 3, 1, 16, true>(st, p, 0);
     return launch_tile<128, 128, 16, 3, 3, 1, 16, true>(st, p, 0);
 }
 

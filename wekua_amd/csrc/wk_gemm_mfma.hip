@@ -1392,7 +1392,8 @@ template <int BM, int BN> int launch_f32_dma2(hipStream_t st, const GemmProblem 
 // work dealt by k-slabs to as many work-groups as are resident at once; where that does not apply, by tiles
 template <int BM, int BN, int OCC> int launch_f32_stream_k(hipStream_t st, const GemmProblem &p, bool edge) {
     if (gemm_f32_dma_stream_k_applies(p, BM, BN)) return gemm_f32_dma_stream_k_launch(st, p, BM, BN);
-    return launch_f32_dma<BM, BN, 16, OCC>(st, p, edge);
+    if constexpr (BM == 64) return launch_f32_dma<64, 64, 32, 4>(st, p, edge);
+    else return launch_f32_dma<BM, BN, 16, OCC>(st, p, edge);
 }
 
 template <int BM, int BN, int BK, int OCC> int launch_f64_dma(hipStream_t st, const GemmProblem &p, bool edge) {
@@ -1450,6 +1451,7 @@ const VariantDesc k_variants[] = {
     // the same kernels with the work dealt by k-slabs (see gemm_f32_dma_kernel), for tiles that do not fill whole rounds
     {"mfma_f32_256x128k", WK_F32, 256, 128, 16, 0.0, 0.08, &launch_f32_stream_k<256, 128, 2>, nullptr, nullptr, nullptr, nullptr, nullptr, 2},
     {"mfma_f32_128x128k", WK_F32, 128, 128, 16, 0.0, 0.08, &launch_f32_stream_k<128, 128, 3>, nullptr, nullptr, nullptr, nullptr, nullptr, 3},
+    {"mfma_f32_64x64k", WK_F32, 64, 64, 32, 0.0, 0.10, &launch_f32_stream_k<64, 64, 3>, nullptr, nullptr, nullptr, nullptr, nullptr, 3},
     {"mfma_f32_256x128t", WK_F32, 256, 128, 16, 0.0, 0.25, &launch_f32_tail<256, 128, 16, 2, 2, 2>, nullptr, nullptr, nullptr, nullptr,
      nullptr, 2}, // whole rounds + a k-split tail
     {"mfma_f32_128x128", WK_F32, 128, 128, 16, 0.897, 0.19, &launch_f32<128, 128, 16, 2, 2, 3>, nullptr, nullptr, nullptr, nullptr,
@@ -1620,14 +1622,18 @@ int wk::gemm_mfma_pick(const GemmProblem &p, double *cost_out) {
     // 2700^3 113 -> 126, 3000^3 122 -> 132, 3200^3 126 -> 140, 3500^3 124 -> 132, 3700^3 123 -> 138, 4000^3 130 -> 137,
     // 4500^3 129 -> 135, 5000^3 133 -> 136, 6000^3 134 -> 141, 3000 x 3000 x 8192 124 -> 136, 2500 x 3500 x 4096 123 ->
     // 133, 3333 x 3333 x 1111 105 -> 123; nothing to gain where the tiles are whole rounds (2048 x 4096 x 1024).
-    if (p.dtype == WK_F32 && best >= 0 && p.K >= 1024 && g_test_options.stream_k) {
+    if (p.dtype == WK_F32 && best >= 0 && p.K >= 512 && g_test_options.stream_k) {
         constexpr double COST_PER_US = 3.05e5;
-        static const struct { const char *name; int bm, bn; double eff, fixed_us; } dealt[] = {
-            {"mfma_f32_128x128k", 128, 128, 0.90, 15.0}, {"mfma_f32_256x128k", 256, 128, 0.933, 36.0}};
+        // (the 64 x 64 tile, fitted on cubes from 1100 to 3000: 0.83 and 6 us; it is what fills the valley between one
+        // and a few rounds of that tile: 1100^3 69 -> 92 TFLOP/s, 1280^3 98 -> 113, 1536^3 100 -> 126, 1792^3 104 -> 129,
+        // 1800^3 100 -> 118, 1900^3 110 -> 121)
+        static const struct { const char *name; int bm, bn; double eff, fixed_us; uint64_t min_k; } dealt[] = {
+            {"mfma_f32_128x128k", 128, 128, 0.90, 15.0, 1024}, {"mfma_f32_256x128k", 256, 128, 0.933, 36.0, 1024},
+            {"mfma_f32_64x64k", 64, 64, 0.83, 6.0, 512}};
         const double plain_cost = best_cost;
         for (const auto &d : dealt) {
             const double tiles = (double)((p.M + d.bm - 1) / d.bm) * (double)((p.N + d.bn - 1) / d.bn);
-            if (tiles <= cus || std::fmod(tiles, cus) == 0.0 || !gemm_f32_dma_stream_k_applies(p, d.bm, d.bn)) continue;
+            if (p.K < d.min_k || tiles <= cus || std::fmod(tiles, cus) == 0.0 || !gemm_f32_dma_stream_k_applies(p, d.bm, d.bn)) continue;
             const double cost = tiles / cus * d.bm * d.bn / d.eff + d.fixed_us * COST_PER_US / (double)p.K;
             if (cost < 0.98 * plain_cost && cost < best_cost)
                 for (int w = 0; w < k_num_variants; ++w)
@@ -1642,9 +1648,12 @@ int wk::gemm_mfma_pick(const GemmProblem &p, double *cost_out) {
     // wavefronts per CU) beats the four rounds of 64x64 the cost model would take -- 2048^3 126 / 132 /
     // 120 / 126 -> 130 / 136 / 126 / 131 TFLOP/s (NN / NT / TN / TT), 2048x2048x4096 128 -> 134.  With
     // fewer tiles (1536^3) or more than one round (3072^3) the 64x64 tile wins.
+    const bool best_dealt = best >= 0 && k_variants[best].name[std::strlen(k_variants[best].name) - 1] == 'k';
     if (p.dtype == WK_F32 && p.K >= 512) {
         const double tiles128 = (double)((p.M + 127) / 128) * (double)((p.N + 127) / 128);
-        if (tiles128 <= cus && tiles128 >= 0.85 * cus) {
+        // (where the small tile dealt by k-slabs was found cheaper, it is, unless the round is all but full:
+        // 1800^3 118 against 100 TFLOP/s, 1900^3 121 against 110, 2000^3 126 / 124, 2048^3 134 / 134.5)
+        if (tiles128 <= cus && tiles128 >= (best_dealt ? 0.97 : 0.85) * cus) {
             // (the direct-to-LDS kernel of that tile where it applies: 2048^3 N,N 131 against 128.5)
             const char *want = !gemm_f32_dma_applies(p, 128, 128) ? "mfma_f32_128x128s2"
                                : (p.K >= 1024 && !p.ext && gemm_dma_rows_aligned(p)) ? "mfma_f32_128x128d2"
