@@ -58,7 +58,7 @@ int wk_gemm_force_variant(const char *name);
  *                       blocks of 1 MiB and more start 0 / 3 / 6 / 9 KiB into their allocation in turn);
  *   "stream_k"       0: the automatic choice never takes the kernels that deal their work by k-slabs
  *                       ("...k") (default 1); 2: those kernels deal every tile's k-slabs instead of running the
- *                       whole rounds of tiles whole;
+ *                       whole rounds of tiles whole; 3: they run the whole rounds whole also where the default would not;
  *   "strips"         0: a product is never multiplied in parts (body of whole tiles + strips); 2: thin strips are
  *                       split off whatever the cost model says (default 1: where the model puts the parts below
  *                       the whole). */

@@ -140,7 +140,8 @@ def test_direct_to_lds_with_rows_that_start_anywhere(dev, variant, op_a, op_b):
 
 
 @pytest.mark.parametrize("variant", ["tile64", "mfma_f64_64x64", "mfma_f64_64x64s2", "mfma_f64_32x32s4", "mfma_f64_64x64z",
-                                     "mfma_f64_128x64", "mfma_f64_128x128", "mfma_f64_128x128d", "mfma_f64_64x64d"])
+                                     "mfma_f64_128x64", "mfma_f64_128x128", "mfma_f64_128x128d", "mfma_f64_64x64d",
+                                     "mfma_f64_128x128k", "mfma_f64_64x64k"])
 @pytest.mark.parametrize("op_a,op_b", OPS)
 def test_f64_every_variant(dev, variant, op_a, op_b):
     assert dev.lib.wk_gemm_force_variant(variant.encode()) == 0
@@ -573,16 +574,25 @@ def test_work_dealt_by_k_slabs(dev, op_a, op_b):
     ("mfma_f32_64x64k", 1, 1100, 1300, 1500, (0, 0)),     # 378 tiles of 64 x 64: 256 whole, 122 dealt
     ("mfma_f32_64x64k", 1, 1800, 1700, 600, (1, 0)),      # 783 tiles: three whole rounds (the last starts as slots free up), 15 dealt
     ("mfma_f32_64x64k", 1, 900, 1000, 1100, (0, 1)),      # 240 tiles, fewer than compute units: all dealt
-    ("mfma_f32_64x64k", 2, 1100, 1300, 1500, (1, 1))])
+    ("mfma_f32_64x64k", 2, 1100, 1300, 1500, (1, 1)),
+    ("mfma_f64_128x128k", 1, 2300, 2500, 360, (0, 0)),    # f64: 360 tiles, 256 whole, 104 dealt
+    ("mfma_f64_128x128k", 1, 1000, 900, 1001, (1, 0)),    # 64 tiles over 512 work-groups, a k tail
+    ("mfma_f64_128x128k", 2, 2300, 2500, 360, (0, 1)),
+    ("mfma_f64_64x64k", 1, 1100, 1300, 750, (1, 1)),      # 378 tiles of 64 x 64
+    ("mfma_f64_64x64k", 1, 1800, 1700, 300, (0, 0)),      # 783 tiles: three whole rounds, 15 dealt
+    ("mfma_f64_64x64k", 2, 900, 1000, 550, (1, 0))])
 def test_work_dealt_by_k_slabs_in_every_form(dev, variant, mode, M, N, K, ops):
     """The kernels that deal k-slabs, forced, in both of their plans (whole rounds of tiles run whole and the rest
     dealt; every tile dealt) and on tile counts below, between and at whole rounds of the compute units: every
     entry against the oracle and the same bits on three runs."""
     op_a, op_b = ops
-    a, b, c = gemm_operands("f32", M, N, K, op_a, op_b, 131 + mode)
+    dtype = variant[5:8]
+    rd = np.float32 if dtype == "f32" else np.float64
+    per = 16 // np.dtype(rd).itemsize
+    a, b, c = gemm_operands(dtype, M, N, K, op_a, op_b, 131 + mode)
     lda, ldb = a.shape[1], b.shape[1]
-    assert lda % 4 == 0 and ldb % 4 == 0, "these kernels take rows that start on 16-byte boundaries"
-    want = oracle.gemm("f32", 1.5, a, op_a, b, op_b, 0.5, c, threads=0)
+    assert lda % per == 0 and ldb % per == 0, "these kernels take rows that start on 16-byte boundaries"
+    want = oracle.gemm(dtype, 1.5, a, op_a, b, op_b, 0.5, c, threads=0)
     dA, dB = dev.upload(a), dev.upload(b)
     assert dev.lib.wk_gemm_force_variant(variant.encode()) == 0
     assert dev.lib.wk_test_option(b"stream_k", mode) == 0
@@ -590,13 +600,13 @@ def test_work_dealt_by_k_slabs_in_every_form(dev, variant, mode, M, N, K, ops):
         first = None
         for _ in range(3):
             dC = dev.upload(c)
-            dev.gemm("f32", op_a, op_b, M, N, K, 1.5, dA, lda, dB, ldb, 0.5, dC, N)
+            dev.gemm(dtype, op_a, op_b, M, N, K, 1.5, dA, lda, dB, ldb, 0.5, dC, N)
             dev.sync()
-            got = dC.download(np.float32, c.shape)
+            got = dC.download(rd, c.shape)
             dC.free()
             if first is None:
                 first = got
-                assert_gemm_close("f32", got, want, 1.5, a, op_a, b, op_b, 0.5, c, K, what=f"{variant}, plan {mode}")
+                assert_gemm_close(dtype, got, want, 1.5, a, op_a, b, op_b, 0.5, c, K, what=f"{variant}, plan {mode}")
             else:
                 assert np.array_equal(got, first), "the bits depend on the run"
     finally:
@@ -773,7 +783,8 @@ def test_direct_to_lds_on_seeded_random_shapes(dev, variant):
                                                 ("f32", 4200, 4096, 1024, True),    # 104 rows beyond: split off because the cost model says so
                                                 ("f32", 3000, 3000, 1024, False),   # ... and here it does not: the body would fill half a round
                                                 ("f32", 2049, 2047, 1024, False),   # the body is too small to carry a strip's launch
-                                                ("f64", 2049, 2050, 1024, True)])
+                                                ("f64", 3073, 3072, 1024, True),    # f64: one row beyond 24 tiles of 128
+                                                ("f64", 2049, 2050, 1024, False)])  # the whole, with its left-over tiles dealt by k-slabs, is cheaper
 def test_thin_strips_beyond_whole_tiles_are_products_of_their_own(dev, dtype, M, N, K, split):
     """A matrix a few rows or columns larger than whole large tiles is multiplied in parts (the body of whole
     tiles, then the thin strips beyond it, each with its own kernel) when k is long and the body large enough

@@ -660,17 +660,24 @@ struct DArgsD {
     const double *bias;
     int act;
     uint32_t patch_m, patch_n; // as in DArgs
+    // kernels instantiated with SK (work dealt by k-slabs), as in DArgs
+    uint32_t sk_units, sk_total, sk_first, sk_groups;
+    double *partials;
+    uint32_t *counters;
 };
 
 
 // VB as in the f32 kernel: 16 bytes per lane and load for rows that start on 16-byte boundaries, 4 (half a
-// double) for any other.
-template <int BM, int BN, int BK, int NS, int OCC, bool A_K, bool B_K, bool EXT, int VB = 16>
+// double) for any other.  SK as in the f32 kernel: the whole rounds of tiles run whole, the k-slabs of the tiles
+// that are left are dealt to the first work-groups of the launch, and the parts of a split tile meet in memory.
+template <int BM, int BN, int BK, int NS, int OCC, bool A_K, bool B_K, bool EXT, int VB = 16, bool SK = false>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(OCC)))
 void gemm_f64_dma_kernel(DArgsD g) {
     static_assert(NS == 2 || NS == 3, "stages");
     static_assert(VB == 16 || VB == 4, "bytes per lane");
     constexpr int SUB = 16 / VB;
+    __shared__ uint32_t s_last;
+    auto run = [&](const uint32_t pid, const uint32_t kb, const uint32_t ke, const uint32_t bq) __attribute__((always_inline)) {
     constexpr int WM = BM / 2, WN = BN / 2, FM = WM / 16, FN = WN / 16;
     constexpr int S = BK / 8;     // fragment steps per slab (8 values of k each, two matrix instructions per block)
     constexpr int CPR = BK / 2;   // 16-byte chunks per row of a k-contiguous slab
@@ -689,7 +696,6 @@ void gemm_f64_dma_kernel(DArgsD g) {
 
     uint32_t tile_m, tile_n;
     if (g.patch_m) { // XCD-local patches, as in the f32 kernel
-        const uint32_t pid = blockIdx.x;
         const uint32_t x = pid & 7u, j = pid >> 3;
         const uint32_t per_patch = g.patch_m * g.patch_n;
         const uint32_t patch = (j / per_patch) * 8u + x, q = j % per_patch;
@@ -697,7 +703,6 @@ void gemm_f64_dma_kernel(DArgsD g) {
         tile_m = (patch / patches_n) * g.patch_m + q % g.patch_m;
         tile_n = (patch % patches_n) * g.patch_n + q / g.patch_m;
     } else {
-        const uint32_t pid = blockIdx.x;
         const uint32_t group_size = GROUP_M * g.tiles_n;
         const uint32_t group = pid / group_size;
         const uint32_t first_m = group * GROUP_M;
@@ -715,6 +720,10 @@ void gemm_f64_dma_kernel(DArgsD g) {
     const double *b_base = B_K ? g.B + (size_t)n0 * g.ldb : g.B + n0;
     const size_t a_step = A_K ? (size_t)BK : (size_t)BK * g.lda;
     const size_t b_step = B_K ? (size_t)BK : (size_t)BK * g.ldb;
+    if constexpr (SK) { // this range starts at slab kb of the tile
+        a_base += kb * a_step;
+        b_base += kb * b_step;
+    }
     uint32_t a_off[A_LOADS * SUB], b_off[B_LOADS * SUB];
     // (k, row or column) of the double that lane `lane` of load q of group grp fetches half of with four bytes
     // per lane: the double that belongs at double 32 q + lane / 2 of the group
@@ -784,7 +793,7 @@ void gemm_f64_dma_kernel(DArgsD g) {
     // ---- the last slab when K is not a multiple of 16 (krem = K % 16 of its k values exist): chunks or rows
     // of k wholly beyond K are fetched from the last existing one, and the wavefront that loaded a share of
     // that slab writes zeros over its doubles whose k does not exist once the loads have landed ----
-    const uint32_t krem = g.K % BK;
+    const uint32_t krem = !SK || ke * BK >= g.K ? g.K % BK : 0u; // (a range that ends inside the tile has whole slabs only)
     auto tail_offset = [&](uint32_t off, int grp, int q, uint32_t ld, auto kc_tag, auto rows_tag) -> uint32_t {
         constexpr bool KC = decltype(kc_tag)::value;
         constexpr int ROWS = decltype(rows_tag)::value;
@@ -898,7 +907,7 @@ void gemm_f64_dma_kernel(DArgsD g) {
 
     // The stages rotate and the slabs are requested, waited for and handed over exactly as in the f32 kernel
     // (see there): st[0] holds the slab being multiplied, slab kt + NS - 1 goes into st[NS - 1].
-    const uint32_t ktiles = (g.K + BK - 1) / BK;
+    const uint32_t ktiles = SK ? ke - kb : (g.K + BK - 1) / BK;
     constexpr uint32_t STAGE_BYTES = STAGE * 8u;
     constexpr int LOADS = (A_LOADS + B_LOADS) * SUB;
     uint32_t st[NS];
@@ -964,6 +973,87 @@ void gemm_f64_dma_kernel(DArgsD g) {
     });
     iteration(F_{}, integral_constant<int, -1>{}, F_{}); // the last
 
+    if constexpr (SK) {
+        const uint32_t slabs_per_tile = (g.K + BK - 1) / BK;
+        if (!(kb == 0 && ke == slabs_per_tile)) {
+            // A part of the tile, exchanged as in the f32 kernel: to memory in accumulator-register order, 16 bytes
+            // (two doubles) per lane and store, slot 2 b' for the part that starts inside the tile and 2 b' + 1 for
+            // the one that starts it; device-scope accesses; the last to arrive adds the parts in the order of k.
+            constexpr size_t TILE = (size_t)BM * BN;
+            constexpr int SC1 = 16;
+            const uint32_t U = g.sk_units, t0 = (pid - g.sk_first) * slabs_per_tile;
+            const uint32_t b_first = t0 / U, b_last = (t0 + slabs_per_tile - 1) / U;
+            const uint32_t nparts = b_last - b_first + 1;
+            uint32_t first_part = 0;
+            if (kb == 0) { // the part that starts the tile stays in the registers when all the others have arrived
+                if (tid == 0) {
+                    const uint32_t arrived = __hip_atomic_load(&g.counters[pid], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    if (arrived == nparts - 1) __hip_atomic_store(&g.counters[pid], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    s_last = arrived == nparts - 1 ? 1u : 0u;
+                }
+                __syncthreads();
+                first_part = s_last;
+                __syncthreads(); // (s_last is written again below)
+            }
+            if (first_part == 0) {
+                __amdgpu_buffer_rsrc_t mine = __builtin_amdgcn_make_buffer_rsrc(
+                    g.partials + (size_t)(2 * bq + (kb == 0 ? 1u : 0u)) * TILE, 0, (int)(TILE * sizeof(double)), 0x00020000);
+#pragma unroll
+                for (int i = 0; i < FM; ++i)
+#pragma unroll
+                    for (int j = 0; j < FN; ++j)
+#pragma unroll
+                        for (int h = 0; h < 2; ++h) {
+                            const f64x2 v = {acc[i][j][2 * h], acc[i][j][2 * h + 1]};
+                            __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4_t, v), mine, tid * 16, ((i * FN + j) * 2 + h) * 4096, SC1);
+                        }
+                asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+                __syncthreads();
+                if (tid == 0) {
+                    const uint32_t before = __hip_atomic_fetch_add(&g.counters[pid], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    const uint32_t last = before == nparts - 1 ? 1u : 0u;
+                    if (last) __hip_atomic_store(&g.counters[pid], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    s_last = last;
+                }
+                __syncthreads();
+                if (!s_last) return;
+#pragma unroll
+                for (int i = 0; i < FM; ++i)
+#pragma unroll
+                    for (int j = 0; j < FN; ++j)
+#pragma unroll
+                        for (int r = 0; r < 4; ++r) acc[i][j][r] = 0.0;
+            }
+            constexpr int NB = FM * FN < 8 ? FM * FN : 8; // blocks per batch of loads (two loads per block)
+            static_assert((FM * FN) % NB == 0, "blocks divide into batches");
+            for (uint32_t pp = first_part; pp < nparts; ++pp) {
+                const uint32_t b2 = b_first + pp;
+                __amdgpu_buffer_rsrc_t part = __builtin_amdgcn_make_buffer_rsrc(
+                    g.partials + (size_t)(2 * b2 + (pp == 0 ? 1u : 0u)) * TILE, 0, (int)(TILE * sizeof(double)), 0x00020000);
+#pragma unroll
+                for (int batch = 0; batch < FM * FN / NB; ++batch) {
+                    u32x4_t v[NB][2];
+#pragma unroll
+                    for (int n = 0; n < NB; ++n)
+#pragma unroll
+                        for (int h = 0; h < 2; ++h)
+                            v[n][h] = __builtin_amdgcn_raw_buffer_load_b128(part, tid * 16, ((batch * NB + n) * 2 + h) * 4096, SC1);
+#pragma unroll
+                    for (int n = 0; n < NB; ++n) {
+                        const int blk = batch * NB + n, i = blk / FN, j = blk % FN;
+#pragma unroll
+                        for (int h = 0; h < 2; ++h) {
+                            const f64x2 f = __builtin_bit_cast(f64x2, v[n][h]);
+                            acc[i][j][2 * h] += f[0];
+                            acc[i][j][2 * h + 1] += f[1];
+                        }
+                    }
+                    __builtin_amdgcn_sched_barrier(0); // (one batch of loads at a time)
+                }
+            }
+        }
+    }
+
     // Tiles that reach beyond C clamp the addresses of C_old and the bias and skip the stores there.
     const double alpha = g.alpha, beta = g.beta;
     auto epilogue = [&](auto checked_tag) {
@@ -1002,11 +1092,35 @@ void gemm_f64_dma_kernel(DArgsD g) {
     };
     if (m0 + BM <= g.M && n0 + BN <= g.N) epilogue(std::false_type{});
     else epilogue(std::true_type{});
+    }; // run
+    if constexpr (!SK) {
+        run(blockIdx.x, 0u, 0u, 0u);
+    } else { // as in the f32 kernel
+        const uint32_t slabs_per_tile = (g.K + BK - 1) / BK;
+        if (blockIdx.x >= g.sk_groups) { // a whole tile
+            run(blockIdx.x - g.sk_groups, 0u, slabs_per_tile, 0u);
+            return;
+        }
+        const uint32_t bq = (blockIdx.x & 7u) * (g.sk_groups >> 3) + (blockIdx.x >> 3);
+        uint32_t u = bq * g.sk_units;
+        const uint32_t u_end = min(u + g.sk_units, g.sk_total);
+        bool first = true;
+        while (u < u_end) {
+            const uint32_t t = u / slabs_per_tile, kb = u - t * slabs_per_tile;
+            const uint32_t ke = min(slabs_per_tile, kb + (u_end - u));
+            if (!first) __syncthreads(); // every wavefront is done with the stages of the range before
+            run(g.sk_first + t, kb, ke, bq);
+            first = false;
+            u += ke - kb;
+        }
+    }
 }
 
-template <int BM, int BN, int BK, int NS, int OCC, bool A_K, bool B_K, bool EXT, int VB = 16> int launch_one_d(hipStream_t st, const DArgsD &g) {
+// sk_grid: work dealt by k-slabs: the work-groups of the launch (0: one work-group per tile)
+template <int BM, int BN, int BK, int NS, int OCC, bool A_K, bool B_K, bool EXT, int VB = 16, bool SK = false>
+int launch_one_d(hipStream_t st, const DArgsD &g, unsigned sk_grid = 0) {
     constexpr size_t lds_bytes = NS * (BM * BK + BN * BK) * sizeof(double);
-    auto kern = gemm_f64_dma_kernel<BM, BN, BK, NS, OCC, A_K, B_K, EXT, VB>;
+    auto kern = gemm_f64_dma_kernel<BM, BN, BK, NS, OCC, A_K, B_K, EXT, VB, SK>;
     static const int attr_rc = [&] {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
                                            (int)lds_bytes);
@@ -1017,11 +1131,44 @@ template <int BM, int BN, int BK, int NS, int OCC, bool A_K, bool B_K, bool EXT,
         return (int)WK_OK;
     }();
     if (attr_rc) return attr_rc;
-    hipLaunchKernelGGL(kern, dim3(g.tiles_m * g.tiles_n), dim3(256), lds_bytes, st, g);
+    hipLaunchKernelGGL(kern, dim3(SK ? sk_grid : g.tiles_m * g.tiles_n), dim3(256), lds_bytes, st, g);
     return launch_status();
 }
 
-template <int BM, int BN, int BK, int NS, int OCC, int VB = 16> int launch_tile_d(hipStream_t st, const GemmProblem &p) {
+// How the work-groups of a launch that deals its work by k-slabs share it.  With at least as many tiles as
+// compute units, the whole rounds of tiles (one tile per unit and round) are run whole, one work-group each, and
+// only the k-slabs of the tiles that are left are dealt, to one work-group per unit: every unit then has the same
+// amount of matrix work, few tiles are split, and the dealt work-groups -- the first of the launch, so the first to
+// start -- are done and their parts added up while the whole tiles are still being multiplied.  With fewer tiles
+// than units (or with the test option "stream_k" at 2) all tiles are dealt, to as many work-groups as are
+// resident at once (units x occ).  groups: the work-groups that take dealt k-slabs (a multiple of eight), units
+// = ceil(dealt tiles x slabs per tile / groups) slabs each, first: the number of tiles run whole.  false: the
+// problem does not fit (no scratch for two partial tiles per dealt work-group, more tiles than counters,
+// 32-bit slab numbers).
+bool stream_k_plan(const GemmProblem &p, int bm, int bn, int bk, int occ, unsigned &groups, uint32_t &units, uint32_t &total,
+                   uint32_t &first) {
+    const size_t elem = p.dtype == WK_F64 ? sizeof(double) : sizeof(float);
+    const uint64_t tiles = ((p.M + bm - 1) / bm) * ((p.N + bn - 1) / bn), slabs = (p.K + bk - 1) / bk;
+    const uint64_t cus = p.num_cus ? p.num_cus : 256;
+    uint64_t whole = g_test_options.stream_k == 2 || tiles < cus ? 0 : tiles / cus * cus;
+    // The f64 128 x 128 tile (two work-groups per unit) deals every tile once the launch would be more work-groups
+    // than are resident at once: which unit a late whole tile lands on is then up to the dispatcher, and with two
+    // slots per unit that both come free at about the same time it doubles them up on some units and leaves others
+    // idle (3456^3: 55 TFLOP/s against 70 with every tile dealt, 3500^3 52 / 67; where it went well the two plans
+    // were within 1.5 %: 3584^3 69 / 70, 3840^3 71 / 71, 4300^3 69 / 68).  The other kernels measured better with
+    // the whole rounds run whole at every size (f32 256 x 128, also two per unit: 4300^3 138 / 133, 8000^3 142 / 128).
+    if (p.dtype == WK_F64 && bm == 128 && g_test_options.stream_k != 3 && whole / cus >= (uint64_t)occ) whole = 0;
+    if (whole == tiles) whole -= cus; // (a launch of whole rounds has no use for this: deal the last round)
+    groups = (unsigned)(whole ? cus : cus * occ);
+    if (groups % 8 || !p.scratch || !p.counters || tiles > p.num_counters || tiles * slabs > 0x7fffffffull) return false;
+    if ((uint64_t)2 * groups * bm * bn * elem > p.scratch_bytes) return false;
+    first = (uint32_t)whole;
+    total = (uint32_t)((tiles - whole) * slabs);
+    units = (uint32_t)(((tiles - whole) * slabs + groups - 1) / groups);
+    return units >= 1;
+}
+
+template <int BM, int BN, int BK, int NS, int OCC, int VB = 16, bool SK = false> int launch_tile_d(hipStream_t st, const GemmProblem &p) {
     DArgsD g{};
     g.A = static_cast<const double *>(p.A);
     g.B = static_cast<const double *>(p.B);
@@ -1046,15 +1193,25 @@ template <int BM, int BN, int BK, int NS, int OCC, int VB = 16> int launch_tile_
             }
     }
     const int sel = (p.op_a ? 0 : 2) | (p.op_b ? 1 : 0);
+    unsigned sk_grid = 0;
+    if constexpr (SK) {
+        unsigned groups = 0;
+        if (p.ext || !stream_k_plan(p, BM, BN, BK, OCC, groups, g.sk_units, g.sk_total, g.sk_first)) return WK_E_INVALID_VALUE;
+        g.sk_groups = groups;
+        sk_grid = groups + g.sk_first; // the dealt work-groups, then one per whole tile
+        g.partials = static_cast<double *>(p.scratch);
+        g.counters = p.counters;
+        g.patch_m = g.patch_n = 0; // consecutive tile numbers are neighbours in the row-group walk
+    }
     if (p.ext) {
-        if constexpr (VB == 16) return sel == 3 ? launch_one_d<BM, BN, BK, NS, OCC, true, true, true>(st, g) : (int)WK_E_INVALID_VALUE;
+        if constexpr (VB == 16 && !SK) return sel == 3 ? launch_one_d<BM, BN, BK, NS, OCC, true, true, true>(st, g) : (int)WK_E_INVALID_VALUE;
         else return WK_E_INVALID_VALUE;
     }
     switch (sel) {
-    case 0: return launch_one_d<BM, BN, BK, NS, OCC, false, false, false, VB>(st, g);
-    case 1: return launch_one_d<BM, BN, BK, NS, OCC, false, true, false, VB>(st, g);
-    case 2: return launch_one_d<BM, BN, BK, NS, OCC, true, false, false, VB>(st, g);
-    default: return launch_one_d<BM, BN, BK, NS, OCC, true, true, false, VB>(st, g);
+    case 0: return launch_one_d<BM, BN, BK, NS, OCC, false, false, false, VB, SK>(st, g, sk_grid);
+    case 1: return launch_one_d<BM, BN, BK, NS, OCC, false, true, false, VB, SK>(st, g, sk_grid);
+    case 2: return launch_one_d<BM, BN, BK, NS, OCC, true, false, false, VB, SK>(st, g, sk_grid);
+    default: return launch_one_d<BM, BN, BK, NS, OCC, true, true, false, VB, SK>(st, g, sk_grid);
     }
 }
 
@@ -1081,31 +1238,6 @@ int launch_one(hipStream_t st, const DArgs &g, uint64_t first_tiles, unsigned sk
     const unsigned grid = SK ? sk_groups : first_tiles ? (unsigned)first_tiles : g.tiles_m * g.tiles_n;
     hipLaunchKernelGGL(kern, dim3(grid), dim3(256 * KS), lds_bytes, st, g);
     return launch_status();
-}
-
-// How the work-groups of a launch that deals its work by k-slabs share it.  With at least as many tiles as
-// compute units, the whole rounds of tiles (one tile per unit and round) are run whole, one work-group each, and
-// only the k-slabs of the tiles that are left are dealt, to one work-group per unit: every unit then has the same
-// amount of matrix work, few tiles are split, and the dealt work-groups -- the first of the launch, so the first to
-// start -- are done and their parts added up while the whole tiles are still being multiplied.  With fewer tiles
-// than units (or with the test option "stream_k" at 2) all tiles are dealt, to as many work-groups as are
-// resident at once (units x occ).  groups: the work-groups that take dealt k-slabs (a multiple of eight), units
-// = ceil(dealt tiles x slabs per tile / groups) slabs each, first: the number of tiles run whole.  false: the
-// problem does not fit (no scratch for two partial tiles per dealt work-group, more tiles than counters,
-// 32-bit slab numbers).
-bool stream_k_plan(const GemmProblem &p, int bm, int bn, int bk, int occ, unsigned &groups, uint32_t &units, uint32_t &total,
-                   uint32_t &first) {
-    const uint64_t tiles = ((p.M + bm - 1) / bm) * ((p.N + bn - 1) / bn), slabs = (p.K + bk - 1) / bk;
-    const uint64_t cus = p.num_cus ? p.num_cus : 256;
-    uint64_t whole = g_test_options.stream_k == 2 || tiles < cus ? 0 : tiles / cus * cus;
-    if (whole == tiles) whole -= cus; // (a launch of whole rounds has no use for this: deal the last round)
-    groups = (unsigned)(whole ? cus : cus * occ);
-    if (groups % 8 || !p.scratch || !p.counters || tiles > p.num_counters || tiles * slabs > 0x7fffffffull) return false;
-    if ((uint64_t)2 * groups * bm * bn * sizeof(float) > p.scratch_bytes) return false;
-    first = (uint32_t)whole;
-    total = (uint32_t)((tiles - whole) * slabs);
-    units = (uint32_t)(((tiles - whole) * slabs + groups - 1) / groups);
-    return units >= 1;
 }
 
 template <int BM, int BN, int BK, int NS, int OCC, int KS = 1, int VB = 16, bool SK = false> int launch_tile(hipStream_t st, const GemmProblem &p, uint64_t first_tiles) {
@@ -1221,6 +1353,19 @@ int wk::gemm_f32_dma_stream_k_launch(hipStream_t st, const GemmProblem &p, int b
     if (bm == 256) return launch_tile<256, 128, 16, 3, 2, 1, 16, true>(st, p, 0);
     if (bm == 64) return launch_tile<64, 64, 32, 3, 3, 1, 16, true>(st, p, 0);
     return launch_tile<128, 128, 16, 3, 3, 1, 16, true>(st, p, 0);
+}
+
+bool wk::gemm_f64_dma_stream_k_applies(const GemmProblem &p, int bm, int bn) {
+    if (!gemm_f64_dma_applies(p, bm, bn) || !f64_rows_aligned(p) || p.ext) return false;
+    unsigned groups;
+    uint32_t units, total, first;
+    return stream_k_plan(p, bm, bn, 16, bm == 128 ? 2 : 3, groups, units, total, first);
+}
+
+int wk::gemm_f64_dma_stream_k_launch(hipStream_t st, const GemmProblem &p, int bm, int bn) {
+    if (!gemm_f64_dma_stream_k_applies(p, bm, bn)) return WK_E_INVALID_VALUE;
+    if (bm == 128) return launch_tile_d<128, 128, 16, 2, 2, 16, true>(st, p);
+    return launch_tile_d<64, 64, 16, 3, 3, 16, true>(st, p);
 }
 
 int wk::gemm_f32_dma_launch(hipStream_t st, const GemmProblem &p, int bm, int bn, uint64_t first_tiles, int k_groups) {

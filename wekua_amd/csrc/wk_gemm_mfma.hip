@@ -1401,6 +1401,12 @@ template <int BM, int BN, int BK, int OCC> int launch_f64_dma(hipStream_t st, co
     return launch_f64<BM, BN, BK, 2, 2, OCC>(st, p, edge);
 }
 
+// f64 with the left-over tiles dealt by k-slabs; where that does not apply, by tiles
+template <int BM, int BN, int BK, int OCC> int launch_f64_stream_k(hipStream_t st, const GemmProblem &p, bool edge) {
+    if (gemm_f64_dma_stream_k_applies(p, BM, BN)) return gemm_f64_dma_stream_k_launch(st, p, BM, BN);
+    return launch_f64_dma<BM, BN, BK, OCC>(st, p, edge);
+}
+
 struct VariantDesc {
     const char *name;
     int dtype, bm, bn, bk; // bk: k values per LDS slab
@@ -1473,6 +1479,9 @@ const VariantDesc k_variants[] = {
     // 8192 x 256 x 8192 69.6 (staged 62.2), 2048^3 68 (61.7), 4096^3 69-70.5
     {"mfma_f64_64x64d", WK_F64, 64, 64, 32, 0.89, 0.05, &launch_f64_dma<64, 64, 32, 2>, nullptr, nullptr, "mfma_f64_32x32s4", "mfma_f64_64x64z"},
     {"mfma_f64_64x64z", WK_F64, 64, 64, 32, 0.0, 0.05, &launch_f64_split64}, // k split over work-groups
+    // the direct-to-LDS kernels with the left-over tiles dealt by k-slabs (see gemm_f64_dma_kernel)
+    {"mfma_f64_128x128k", WK_F64, 128, 128, 16, 0.0, 0.10, &launch_f64_stream_k<128, 128, 16, 2>, nullptr, nullptr, nullptr, nullptr, nullptr, 2},
+    {"mfma_f64_64x64k", WK_F64, 64, 64, 32, 0.0, 0.05, &launch_f64_stream_k<64, 64, 32, 2>, nullptr, nullptr, nullptr, nullptr, nullptr, 3},
     {"mfma_f64_64x64s2", WK_F64, 64, 64, 64, 0.0, 0.05, &launch_f64<64, 64, 32, 2, 2, 2, 2>}, // 2 groups x 32 k
     // (two wavefronts per SIMD: with a 128-register budget its staging sets and fragments spill and it
     // runs several times slower than the 64x64 tile)
@@ -1622,19 +1631,21 @@ int wk::gemm_mfma_pick(const GemmProblem &p, double *cost_out) {
     // 2700^3 113 -> 126, 3000^3 122 -> 132, 3200^3 126 -> 140, 3500^3 124 -> 132, 3700^3 123 -> 138, 4000^3 130 -> 137,
     // 4500^3 129 -> 135, 5000^3 133 -> 136, 6000^3 134 -> 141, 3000 x 3000 x 8192 124 -> 136, 2500 x 3500 x 4096 123 ->
     // 133, 3333 x 3333 x 1111 105 -> 123; nothing to gain where the tiles are whole rounds (2048 x 4096 x 1024).
-    if (p.dtype == WK_F32 && best >= 0 && p.K >= 512 && g_test_options.stream_k) {
-        constexpr double COST_PER_US = 3.05e5;
-        // (the 64 x 64 tile, fitted on cubes from 1100 to 3000: 0.83 and 6 us; it is what fills the valley between one
-        // and a few rounds of that tile: 1100^3 69 -> 92 TFLOP/s, 1280^3 98 -> 113, 1536^3 100 -> 126, 1792^3 104 -> 129,
-        // 1800^3 100 -> 118, 1900^3 110 -> 121)
-        static const struct { const char *name; int bm, bn; double eff, fixed_us; uint64_t min_k; } dealt[] = {
-            {"mfma_f32_128x128k", 128, 128, 0.90, 15.0, 1024}, {"mfma_f32_256x128k", 256, 128, 0.933, 36.0, 1024},
-            {"mfma_f32_64x64k", 64, 64, 0.83, 6.0, 512}};
+    // (f64, fitted the same way on cubes from 1100 to 4300: 64 x 64 0.887 and 12 us, 128 x 128 0.897 and 20 us; 1100^3
+    // 37 -> 50 TFLOP/s, 1536^3 51 -> 66, 1792^3 52 -> 66, 2300^3 58 -> 68, 2500^3 59 -> 65, 3456^3 51 -> 70, 4300^3 63 -> 69)
+    if ((p.dtype == WK_F32 || p.dtype == WK_F64) && best >= 0 && p.K >= 512 && g_test_options.stream_k) {
+        const double cost_per_us = p.dtype == WK_F32 ? 3.05e5 : 1.525e5;
+        static const struct { const char *name; int dtype, bm, bn; double eff, fixed_us; uint64_t min_k; } dealt[] = {
+            {"mfma_f32_128x128k", WK_F32, 128, 128, 0.90, 15.0, 1024}, {"mfma_f32_256x128k", WK_F32, 256, 128, 0.933, 36.0, 1024},
+            {"mfma_f32_64x64k", WK_F32, 64, 64, 0.83, 6.0, 512},
+            {"mfma_f64_128x128k", WK_F64, 128, 128, 0.897, 20.0, 1024}, {"mfma_f64_64x64k", WK_F64, 64, 64, 0.887, 12.0, 512}};
         const double plain_cost = best_cost;
         for (const auto &d : dealt) {
+            if (d.dtype != p.dtype || p.K < d.min_k) continue;
             const double tiles = (double)((p.M + d.bm - 1) / d.bm) * (double)((p.N + d.bn - 1) / d.bn);
-            if (p.K < d.min_k || tiles <= cus || std::fmod(tiles, cus) == 0.0 || !gemm_f32_dma_stream_k_applies(p, d.bm, d.bn)) continue;
-            const double cost = tiles / cus * d.bm * d.bn / d.eff + d.fixed_us * COST_PER_US / (double)p.K;
+            const bool applies = p.dtype == WK_F32 ? gemm_f32_dma_stream_k_applies(p, d.bm, d.bn) : gemm_f64_dma_stream_k_applies(p, d.bm, d.bn);
+            if (tiles <= cus || std::fmod(tiles, cus) == 0.0 || !applies) continue;
+            const double cost = tiles / cus * d.bm * d.bn / d.eff + d.fixed_us * cost_per_us / (double)p.K;
             if (cost < 0.98 * plain_cost && cost < best_cost)
                 for (int w = 0; w < k_num_variants; ++w)
                     if (!std::strcmp(k_variants[w].name, d.name)) {

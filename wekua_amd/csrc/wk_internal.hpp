@@ -44,7 +44,7 @@ struct TestOptions {
     int gemm_walk_rows = 0; // 1: the direct-to-LDS kernels walk the tiles in groups of rows, not XCD-local patches
     int tail_strict = 0;    // 1: forced k-split tail variants plan like the automatic choice
     int alloc_colours = 1;  // 0: wk_malloc hands out blocks as hipMalloc returns them
-    int stream_k = 1;       // 0: the automatic choice never deals work by k-slabs; 2: every tile dealt, none run whole
+    int stream_k = 1;       // 0: the automatic choice never deals work by k-slabs; 2: every tile dealt, none run whole; 3: whole rounds always run whole
     int strips = 1;         // 0: products are never multiplied in parts; 2: thin strips split off whatever the model says
 };
 extern TestOptions g_test_options;
@@ -248,6 +248,8 @@ bool gemm_f32_dma_applies(const GemmProblem &p, int bm, int bn);
 // (parts of tiles meet in p.scratch, counted on p.counters): for products whose tiles do not fill whole rounds
 bool gemm_f32_dma_stream_k_applies(const GemmProblem &p, int bm, int bn);
 int gemm_f32_dma_stream_k_launch(hipStream_t st, const GemmProblem &p, int bm, int bn);
+bool gemm_f64_dma_stream_k_applies(const GemmProblem &p, int bm, int bn);
+int gemm_f64_dma_stream_k_launch(hipStream_t st, const GemmProblem &p, int bm, int bn);
 bool gemm_dma_rows_aligned(const GemmProblem &p); // 16-byte loads (else 4-byte ones: one group of wavefronts, no fused epilogue)
 int gemm_f32_dma_launch(hipStream_t st, const GemmProblem &p, int bm, int bn, uint64_t first_tiles = 0, int k_groups = 1);
 // the same for f64: macro tiles 128 x 128 (k-slabs of 8) and 64 x 64 (k-slabs of 16)
