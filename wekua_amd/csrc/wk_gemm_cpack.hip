@@ -170,6 +170,9 @@ int wk::gemm_complex_packed_prepare(hipStream_t st, const GemmProblem &p, void *
     real.C = p.C; real.ldc = 2 * p.ldc;
     real.num_cus = p.num_cus;
     real.reuse_b = p.reuse_b;
+    // the stream's scratch and tile counters, for the real kernels that split k over work-groups or deal k-slabs
+    real.scratch = p.scratch; real.scratch_bytes = p.scratch_bytes;
+    real.counters = p.counters; real.num_counters = p.num_counters;
     std::memset(real.alpha, 0, sizeof real.alpha);
     std::memset(real.beta, 0, sizeof real.beta);
     if (p.epi == EPI_ALPHA_BETA) { // C was scaled by beta already, alpha is inside B~: C = 1 * acc + 1 * C
