@@ -76,6 +76,8 @@ HOST_SIGNATURES = {
     "wkz_fill_constant": (ci, [vp, vp, vp]),
     "wkz_identity": (ci, [vp, vp]),
     "wkz_axpy": (ci, [vp, vp, vp, vp]),
+    "wkz_axpy_repeat": (ci, [vp, vp, vp, vp, ctypes.c_uint32]),
+    "wkz_gemm_repeat": (ci, [vp, vp, vp, ci, vp, ci, vp, vp, vp, ctypes.c_uint32]),
     "wkz_packed_init": (ci, [vp, vp, u64, ci, ctypes.POINTER(vp)]),
     "wkz_packed_init_with_dimensions": (ci, [vp, ci, u64, u64, u64, ci, ci, ctypes.POINTER(vp)]),
     "wkz_packed_deinit": (ci, [vp, vp]),
@@ -468,6 +470,22 @@ class blas:
         """blas.axpy(T, pipeline, x, alpha, y): y = alpha*x + y (alpha None: y += x)."""
         _keep, p = _scalar_ptr(x.dtype, alpha)
         _check(_lib().wkz_axpy(pipeline._h, x._h, p, y._h), "blas.axpy")
+
+    @staticmethod
+    def axpy_repeat(pipeline: Pipeline, x: Tensor, alpha, y: Tensor, count: int) -> None:
+        """blas.axpy `count` times from one loop inside the host library (benchmarks: a call from Python costs more
+        interpreter time than a short launch takes)."""
+        _keep, p = _scalar_ptr(x.dtype, alpha)
+        _check(_lib().wkz_axpy_repeat(pipeline._h, x._h, p, y._h, int(count)), "blas.axpy")
+
+    @staticmethod
+    def gemm_repeat(pipeline: Pipeline, alpha, a: Tensor, op_a: int, b: Tensor, op_b: int, beta, c: Tensor,
+                    packed_tensors: "GemmPackedTensors | None", count: int) -> None:
+        """blas.gemm `count` times from one loop inside the host library (benchmarks)."""
+        _ka, pa = _scalar_ptr(c.dtype, alpha)
+        _kb, pb = _scalar_ptr(c.dtype, beta)
+        _check(_lib().wkz_gemm_repeat(pipeline._h, pa, a._h, int(op_a), b._h, int(op_b), pb, c._h,
+                                      packed_tensors._h if packed_tensors is not None else None, int(count)), "blas.gemm")
 
     @staticmethod
     def gemm(pipeline: Pipeline, alpha, a: Tensor, op_a: int, b: Tensor, op_b: int, beta, c: Tensor,

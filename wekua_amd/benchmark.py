@@ -77,9 +77,10 @@ class Session:
             self.wk.random.uniform(self.pipeline, t, seed, -100, 100)
         return t
 
-    def time_ms(self, call, iters, warm_seconds=0.15):
+    def time_ms(self, call, iters, warm_seconds=0.15, repeat=None):
         """ms per call from events on the stream, after keeping the device busy for `warm_seconds`
-        (short kernels measured right after an upload see the clocks still ramping)."""
+        (short kernels measured right after an upload see the clocks still ramping).  repeat(n): the
+        same call n times from one loop inside the host library, used for the timed launches when given."""
         import time
         t0 = time.perf_counter()
         while True:
@@ -90,8 +91,11 @@ class Session:
                 break
         check = self.wk._capi.check
         check(self.lib.wk_event_record(self.e0, self.stream))
-        for _ in range(iters):
-            call()
+        if repeat is not None:
+            repeat(iters)
+        else:
+            for _ in range(iters):
+                call()
         check(self.lib.wk_event_record(self.e1, self.stream))
         self.pipeline.waitAndCleanup()
         ms = self.ct.c_float()
@@ -124,7 +128,8 @@ def time_gemm(ses, dtype, M, N, K, op_a, op_b, alpha, beta, iters=10, device_fil
     if keep_b:
         packed.keepB(True)
     ses.pipeline.waitAndCleanup()
-    ms = ses.time_ms(lambda: wk.blas.gemm(ses.pipeline, alpha, A, op_a, B, op_b, beta, C, packed), iters)
+    ms = ses.time_ms(lambda: wk.blas.gemm(ses.pipeline, alpha, A, op_a, B, op_b, beta, C, packed), iters,
+                     repeat=lambda n: wk.blas.gemm_repeat(ses.pipeline, alpha, A, op_a, B, op_b, beta, C, packed, n))
     variant = ses.lib.wk_gemm_variant_with_workspace(raw.dtype_id(dtype), op_a, op_b, M, N, K, A.row_pitch, B.row_pitch,
                                                      C.row_pitch, A.buffer, B.buffer, C.buffer,
                                                      packed.workspace_bytes).decode()
@@ -146,10 +151,12 @@ def time_axpy(ses, dtype, n, iters=50, device_fill=False, batches=0):
         x, y = ses.tensor(dtype, _operand(rd, shape, 1)), ses.tensor(dtype, _operand(rd, shape, 2))
     ses.pipeline.waitAndCleanup()
     alpha = 0.75 if rd.kind == "f" else 3
+    once = lambda: wk.blas.axpy(ses.pipeline, x, alpha, y)
+    many = lambda count: wk.blas.axpy_repeat(ses.pipeline, x, alpha, y, count)
     if batches:
-        ms = [ses.time_ms(lambda: wk.blas.axpy(ses.pipeline, x, alpha, y), iters) for _ in range(batches)]
+        ms = [ses.time_ms(once, iters, repeat=many) for _ in range(batches)]
     else:
-        ms = ses.time_ms(lambda: wk.blas.axpy(ses.pipeline, x, alpha, y), iters)
+        ms = ses.time_ms(once, iters, repeat=many)
     x.release(ses.pipeline)
     y.release(ses.pipeline)
     return ms

@@ -442,6 +442,20 @@ int wkz_gemm(void *pipeline, const void *host_alpha, void *a, int op_a, void *b,
     });
 }
 
+// The same two calls `count` times in a row from one loop in this library: what a C++ or Zig caller's loop does,
+// for the benchmarks (from Python a call costs 4-5 us of interpreter and ctypes time, more than a short launch).
+int wkz_axpy_repeat(void *pipeline, void *x, const void *host_alpha, void *y, uint32_t count) {
+    int rc = 0;
+    for (uint32_t i = 0; i < count && !rc; ++i) rc = wkz_axpy(pipeline, x, host_alpha, y);
+    return rc;
+}
+int wkz_gemm_repeat(void *pipeline, const void *host_alpha, void *a, int op_a, void *b, int op_b, const void *host_beta, void *c,
+                    void *packed, uint32_t count) {
+    int rc = 0;
+    for (uint32_t i = 0; i < count && !rc; ++i) rc = wkz_gemm(pipeline, host_alpha, a, op_a, b, op_b, host_beta, c, packed);
+    return rc;
+}
+
 // ---- math ------------------------------------------------------------------------------------------
 int wkz_math_dot(void *pipeline, void *x, void *y) {
     return guard([&] {
