@@ -249,6 +249,11 @@ bool gemm_f32_dma_applies(const GemmProblem &p, int bm, int bn);
 bool gemm_f32_dma_stream_k_applies(const GemmProblem &p, int bm, int bn);
 int gemm_f32_dma_stream_k_launch(hipStream_t st, const GemmProblem &p, int bm, int bn);
 bool gemm_f64_dma_stream_k_applies(const GemmProblem &p, int bm, int bn);
+// rows of both f64 operands start on 16-byte boundaries
+bool gemm_f64_rows_aligned(const GemmProblem &p);
+// how a launch that deals k-slabs shares its work (wk_gemm_dma.hip); false: the problem does not fit
+bool gemm_dma_stream_k_plan(const GemmProblem &p, int bm, int bn, int bk, int occ, unsigned &groups, uint32_t &units, uint32_t &total,
+                            uint32_t &first);
 int gemm_f64_dma_stream_k_launch(hipStream_t st, const GemmProblem &p, int bm, int bn);
 bool gemm_dma_rows_aligned(const GemmProblem &p); // 16-byte loads (else 4-byte ones: one group of wavefronts, no fused epilogue)
 int gemm_f32_dma_launch(hipStream_t st, const GemmProblem &p, int bm, int bn, uint64_t first_tiles = 0, int k_groups = 1);
