@@ -71,15 +71,18 @@ struct DArgs {
 // VB: bytes per lane and load.  16 for operands whose rows start on 16-byte boundaries; 4 for any other (every
 // lane then fetches one float into the same place of the same LDS layout: SUB = 4 loads per KiB instead of one,
 // nothing read beyond the end of a row).
-// SK: the launch is as many work-groups as are resident at once (compute units x OCC), and the work is dealt to
-// them by k-slabs instead of by tiles: work-group b takes slabs [b' U, (b' + 1) U) of the tiles x slabs-per-tile
-// of the product in tile-walk order (b' numbers the work-groups of one XCD consecutively), so every unit is busy
-// for the same time whatever the number of tiles.  A range that holds a whole tile runs it as ever; a part of a
-// tile (at most two per work-group: the end of one tile at the start of its range, the start of another at its
-// end) goes to memory as a partial tile, and the work-group that arrives last at the tile's counter adds the
-// parts up in the order of k -- its own read back like the others, so the bits do not depend on who that is --
-// and runs the epilogue.  The same hand-over as the k-split kernels of wk_gemm_mfma.hip (device-scope stores and
-// loads, a wait for the stores in front of the count).
+// SK: for products whose tiles do not come out even over the compute units.  The first sk_groups work-groups of
+// the launch are dealt k-slabs instead of tiles: the slabs of the tiles from sk_first on are numbered in tile-walk
+// order and work-group b takes [b' U, (b' + 1) U) of them (b' numbers the work-groups of one XCD consecutively); every
+// later work-group runs one whole tile, as ever.  With one dealt work-group per unit beside the whole tiles every
+// unit has the same amount of matrix work (gemm_dma_stream_k_plan below; with fewer tiles than units every tile
+// is dealt, to as many work-groups as are resident).  A dealt range that holds a whole tile runs it as ever; a
+// part of a tile (at most two per work-group: the end of one tile at the start of its range, the start of
+// another at its end) goes to memory as a partial tile, and the work-group that arrives last at the tile's
+// counter adds the parts up in the order of k, so the bits do not depend on who that is (the part that starts the
+// tile stays in its registers when it is the last to arrive: 0 + p0 + p1 ... and p0 + p1 ... are the same
+// bits), and runs the epilogue.  The same hand-over as the k-split kernels of wk_gemm_mfma.hip (device-scope stores
+// and loads, a wait for the stores in front of the count).
 template <int BM, int BN, int BK, int NS, int OCC, bool A_K, bool B_K, bool EXT, int KS = 1, int VB = 16, bool SK = false>
 __global__ __launch_bounds__(256 * KS) __attribute__((amdgpu_waves_per_eu(OCC)))
 void gemm_f32_dma_kernel(DArgs g) {

@@ -1389,7 +1389,8 @@ template <int BM, int BN> int launch_f32_dma2(hipStream_t st, const GemmProblem 
     return launch_f32<64, 64, 16, 2, 2, 4, 4>(st, p, edge);
 }
 
-// work dealt by k-slabs to as many work-groups as are resident at once; where that does not apply, by tiles
+// the direct-to-LDS kernel with its left-over tiles dealt by k-slabs (see gemm_f32_dma_kernel); where that does not
+// apply, by tiles
 template <int BM, int BN, int OCC> int launch_f32_stream_k(hipStream_t st, const GemmProblem &p, bool edge) {
     if (gemm_f32_dma_stream_k_applies(p, BM, BN)) return gemm_f32_dma_stream_k_launch(st, p, BM, BN);
     if constexpr (BM == 64) return launch_f32_dma<64, 64, 32, 4>(st, p, edge);
