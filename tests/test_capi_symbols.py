@@ -34,8 +34,41 @@ def test_test_knobs_are_not_in_the_product_header():
     from wekua_amd import _capi
     lib = _capi.load()
     assert lib.wk_test_option(b"no-such-switch", 1) == 1
-    for name, default in ((b"gemm_walk_rows", 0), (b"tail_strict", 0), (b"alloc_colours", 1), (b"stream_k", 1)):
+    for name, default in ((b"gemm_walk_rows", 0), (b"tail_strict", 0), (b"alloc_colours", 1), (b"stream_k", 1), (b"strips", 1)):
         assert lib.wk_test_option(name, default) == 0
+
+
+def test_kernel_choice_by_name_without_a_device():
+    """The name query runs the cost model on the host (256 compute units assumed): products whose tiles do not
+    come out even over the units take the kernels that deal their left-over tiles by k-slabs, whole rounds do
+    not, and the two switches of the test header take them, and the strips, away."""
+    from wekua_amd import _capi, raw
+    lib = _capi.load()
+
+    def name(dtype, M, N, K):
+        per = 4 if dtype == "f32" else 2
+        up = lambda n: -(-n // per) * per
+        return lib.wk_gemm_variant(raw.dtype_id(dtype), 0, 0, M, N, K, up(K), up(N), up(N), None, None, None).decode()
+    assert name("f32", 2500, 2500, 2500) == "mfma_f32_128x128k"
+    assert name("f32", 1536, 1536, 1536) == "mfma_f32_64x64k"
+    assert name("f32", 4300, 4300, 4300) == "mfma_f32_256x128k"
+    assert name("f64", 1536, 1536, 1536) == "mfma_f64_64x64k"
+    assert name("f64", 3456, 3456, 3456) == "mfma_f64_128x128k"
+    for whole_rounds in (("f32", 8192, 8192, 8192), ("f32", 4096, 4096, 4096), ("f32", 2048, 4096, 1024), ("f32", 1024, 1024, 1024),
+                         ("f64", 4096, 4096, 4096), ("f64", 8192, 256, 8192)):
+        assert not name(*whole_rounds).endswith("k"), whole_rounds
+    assert name("f32", 1536, 1536, 256).endswith("d")                    # short k: the exchange would not pay
+    assert name("f32", 4097, 4095, 4093) == "mfma_f32_256x128d+strips"   # one row beyond sixteen tiles: in parts
+    assert name("f32", 2200, 2200, 2200) == "mfma_f32_64x64d"            # strips of 24: three more launches would cost more
+    try:
+        assert lib.wk_test_option(b"stream_k", 0) == 0
+        assert not name("f32", 2500, 2500, 2500).endswith("k")
+        assert not name("f64", 1536, 1536, 1536).endswith("k")
+        assert lib.wk_test_option(b"strips", 0) == 0
+        assert "+strips" not in name("f32", 4097, 4095, 4093)
+    finally:
+        lib.wk_test_option(b"stream_k", 1)
+        lib.wk_test_option(b"strips", 1)
 
 
 def test_header_declares_the_hot_path():

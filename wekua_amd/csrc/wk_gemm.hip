@@ -183,12 +183,13 @@ bool plan_strips(const GemmProblem &p, StripPlan &out) {
     // a launch more: about 4 us in the model's unit (cost x k / 3.05e5 = microseconds in f32, half that rate in f64)
     const double launch = 4.0 * (p.dtype == WK_F32 ? 3.05e5 : 1.525e5) / (double)p.K;
     const uint64_t m_rem = p.M > big ? p.M % big : 0, n_rem = p.N > bn ? p.N % bn : 0;
-    // (a whole whose work is dealt by k-slabs was already chosen with a margin of its own, and the model prices the
-    // parts a few per cent too high: 4296 x 4096 x 4096 142 TFLOP/s in parts against 139 dealt, 4096 x 4160 x 4096 143 / 139)
+    // (a whole whose work is dealt by k-slabs was already chosen with a margin of its own; measured either side of
+    // the model by 2-3 %: 4296 x 4096 x 4096 142 TFLOP/s in parts against 139 dealt, 4096 x 4160 x 4096 143 / 139, but
+    // 4700^3 137 / 141 and 4300^3 136 / 138)
     const int whole_v = gemm_mfma_pick(p, nullptr);
     const char *whole_name = whole_v >= 0 ? gemm_mfma_variant_name(whole_v) : "";
     const bool whole_dealt = whole_name[0] && whole_name[std::strlen(whole_name) - 1] == 'k';
-    double best = (whole_dealt ? 1.03 : 0.95) * whole;
+    double best = (whole_dealt ? 1.0 : 0.95) * whole;
     bool found = false;
     for (int cand = 1; cand < 4; ++cand) {
         const bool sm = cand & 1, sn = cand & 2;
