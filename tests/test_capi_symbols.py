@@ -34,7 +34,7 @@ def test_test_knobs_are_not_in_the_product_header():
     from wekua_amd import _capi
     lib = _capi.load()
     assert lib.wk_test_option(b"no-such-switch", 1) == 1
-    for name, default in ((b"gemm_walk_rows", 0), (b"tail_strict", 0), (b"alloc_colours", 1), (b"stream_k", 1), (b"strips", 1)):
+    for name, default in ((b"gemm_walk_rows", 0), (b"tail_strict", 0), (b"alloc_colours", 1), (b"stream_k", 1), (b"strips", 1), (b"persistent", 1)):
         assert lib.wk_test_option(name, default) == 0
 
 

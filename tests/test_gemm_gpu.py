@@ -615,6 +615,41 @@ def test_work_dealt_by_k_slabs_in_every_form(dev, variant, mode, M, N, K, ops):
         dA.free(); dB.free()
 
 
+@pytest.mark.parametrize("variant,M,N,K,ops", [
+    ("mfma_f32_64x64d", 2048, 2048, 96, (1, 0)),      # 1024 tiles on 768 resident work-groups
+    ("mfma_f32_64x64d", 1990, 2050, 70, (0, 0)),      # the same count, ragged
+    ("mfma_f32_128x128d", 4000, 3900, 48, (0, 1)),    # 992 tiles on 768
+    ("mfma_f32_256x128d", 4100, 4200, 40, (1, 1)),    # 561 tiles on 512
+    ("mfma_f64_128x128d", 3400, 3400, 40, (0, 0)),    # 729 tiles on 512
+    ("mfma_f64_64x64d", 2048, 2000, 36, (1, 0))])     # 1024 tiles on 768
+def test_launches_between_one_and_two_rounds_take_their_tiles_in_turn(dev, variant, M, N, K, ops):
+    """A launch of more tiles than work-groups are resident at once, but fewer than two rounds of them, is as
+    many work-groups as are resident, each taking every n-th tile: every entry against the oracle, and the same
+    bits as the launch of one work-group per tile (the test switch)."""
+    op_a, op_b = ops
+    dtype = variant[5:8]
+    rd = np.float32 if dtype == "f32" else np.float64
+    a, b, c = gemm_operands(dtype, M, N, K, op_a, op_b, 171)
+    want = oracle.gemm(dtype, 1.5, a, op_a, b, op_b, 0.5, c, threads=0)
+    dA, dB = dev.upload(a), dev.upload(b)
+    assert dev.lib.wk_gemm_force_variant(variant.encode()) == 0
+    try:
+        got = {}
+        for mode in (1, 0):
+            assert dev.lib.wk_test_option(b"persistent", mode) == 0
+            dC = dev.upload(c)
+            dev.gemm(dtype, op_a, op_b, M, N, K, 1.5, dA, a.shape[1], dB, b.shape[1], 0.5, dC, N)
+            dev.sync()
+            got[mode] = dC.download(rd, c.shape)
+            dC.free()
+        assert_gemm_close(dtype, got[1], want, 1.5, a, op_a, b, op_b, 0.5, c, K, what=variant)
+        assert np.array_equal(got[0], got[1])
+    finally:
+        dev.lib.wk_test_option(b"persistent", 1)
+        dev.lib.wk_gemm_force_variant(b"auto")
+        dA.free(); dB.free()
+
+
 @pytest.mark.parametrize("dtype", ["f32", "f64"])
 def test_k_split_over_work_groups(dev, dtype):
     """Few tiles of C and a long k: every tile goes to several work-groups, whose partial tiles meet in

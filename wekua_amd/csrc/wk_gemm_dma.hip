@@ -60,6 +60,8 @@ struct DArgs {
     // sk_first: the tiles before that one are run whole, one work-group each (work-groups sk_groups ... of the
     // launch); the k-slabs of the tiles from it on are dealt to work-groups 0 ... sk_groups - 1
     uint32_t sk_units, sk_total, sk_first, sk_groups;
+    // tiles of this launch (one work-group each, or fewer work-groups that take every gridDim.x-th tile in turn)
+    uint32_t tiles_run;
     float *partials;
     uint32_t *counters;
 };
@@ -611,33 +613,52 @@ void gemm_f32_dma_kernel(DArgs g) {
     else epilogue(std::true_type{});
     }; // run
     if constexpr (!SK) {
-        run(blockIdx.x, 0u, 0u, 0u);
+        // One work-group per tile, or -- a launch of more tiles than are resident at once -- as many work-groups as
+        // are resident, each taking every gridDim.x-th tile in turn: which unit a late tile lands on is then fixed
+        // here (every unit's work-groups get the same share) instead of left to the order in which slots come free.
+        for (uint32_t pid = blockIdx.x; pid < g.tiles_run; pid += gridDim.x) {
+            if (pid != blockIdx.x) __syncthreads(); // every wavefront is done with the stages of the tile before
+            run(pid, 0u, 0u, 0u);
+        }
     } else {
         const uint32_t slabs_per_tile = (g.K + BK - 1) / BK;
-        if (blockIdx.x >= g.sk_groups) { // a whole tile
-            run(blockIdx.x - g.sk_groups, 0u, slabs_per_tile, 0u);
-            return;
-        }
-        // work-groups b, b + 8, ... share an XCD: they take consecutive ranges, and with them neighbouring tiles
-        const uint32_t bq = (blockIdx.x & 7u) * (g.sk_groups >> 3) + (blockIdx.x >> 3);
-        uint32_t u = bq * g.sk_units;
-        const uint32_t u_end = min(u + g.sk_units, g.sk_total);
         bool first = true;
-        while (u < u_end) {
-            const uint32_t t = u / slabs_per_tile, kb = u - t * slabs_per_tile;
-            const uint32_t ke = min(slabs_per_tile, kb + (u_end - u));
-            if (!first) __syncthreads(); // every wavefront is done with the stages of the range before
-            run(g.sk_first + t, kb, ke, bq);
-            first = false;
-            u += ke - kb;
+        // Every tile dealt: all work-groups take a run of k-slabs.  Whole rounds run whole: the launch is `slots`
+        // work-groups per unit (work-group b sits on unit b % units, slot b / units: they are placed breadth
+        // first); slot 0 takes the unit's run of k-slabs first, and the unit's whole tiles -- tile c + units * j for
+        // j = 0 ... rounds - 1 -- go to the slots in turn, starting with slot 1, so that every unit's slots end up
+        // with the same amount of work.
+        const uint32_t units = g.sk_groups;
+        const uint32_t slot = g.sk_first ? blockIdx.x / units : 0u;
+        if (slot == 0) {
+            // work-groups b, b + 8, ... share an XCD: they take consecutive ranges, and with them neighbouring tiles
+            const uint32_t bq = (blockIdx.x & 7u) * (g.sk_groups >> 3) + (blockIdx.x >> 3);
+            uint32_t u = bq * g.sk_units;
+            const uint32_t u_end = min(u + g.sk_units, g.sk_total);
+            while (u < u_end) {
+                const uint32_t t = u / slabs_per_tile, kb = u - t * slabs_per_tile;
+                const uint32_t ke = min(slabs_per_tile, kb + (u_end - u));
+                if (!first) __syncthreads(); // every wavefront is done with the stages of the range before
+                run(g.sk_first + t, kb, ke, bq);
+                first = false;
+                u += ke - kb;
+            }
+        }
+        if (g.sk_first) {
+            const uint32_t c = blockIdx.x - slot * units, slots = gridDim.x / units, rounds = g.sk_first / units;
+            for (uint32_t j = (slot + slots - 1) % slots; j < rounds; j += slots) {
+                if (!first) __syncthreads();
+                run(c + units * j, 0u, slabs_per_tile, 0u);
+                first = false;
+            }
         }
     }
 }
 
-// first_tiles: launch only that many tiles, in tile-walk order (0: all of them)
-// sk_groups: work dealt by k-slabs to that many work-groups (0: one work-group per tile)
+// grid: the work-groups of the launch (one per tile of g.tiles_run, or fewer: they then take the tiles in turn;
+// kernels that deal k-slabs: as their plan says)
 template <int BM, int BN, int BK, int NS, int OCC, bool A_K, bool B_K, bool EXT, int KS = 1, int VB = 16, bool SK = false>
-int launch_one(hipStream_t st, const DArgs &g, uint64_t first_tiles, unsigned sk_groups = 0) {
+int launch_one(hipStream_t st, const DArgs &g, unsigned grid) {
     constexpr size_t lds_bytes = NS * (BM * BK + BN * BK) * sizeof(float); // 3 x 24 KB / 3 x 16 KB / 3 x 32 KB
     auto kern = gemm_f32_dma_kernel<BM, BN, BK, NS, OCC, A_K, B_K, EXT, KS, VB, SK>;
     static const int attr_rc = [&] {
@@ -650,7 +671,6 @@ int launch_one(hipStream_t st, const DArgs &g, uint64_t first_tiles, unsigned sk
         return (int)WK_OK;
     }();
     if (attr_rc) return attr_rc;
-    const unsigned grid = SK ? sk_groups : first_tiles ? (unsigned)first_tiles : g.tiles_m * g.tiles_n;
     hipLaunchKernelGGL(kern, dim3(grid), dim3(256 * KS), lds_bytes, st, g);
     return launch_status();
 }
@@ -683,26 +703,37 @@ template <int BM, int BN, int BK, int NS, int OCC, int KS = 1, int VB = 16, bool
             }
     }
     const int sel = (p.op_a ? 0 : 2) | (p.op_b ? 1 : 0); // bit 1: A k-contiguous, bit 0: B k-contiguous
-    unsigned sk_groups = 0;
+    g.tiles_run = first_tiles ? (uint32_t)first_tiles : g.tiles_m * g.tiles_n;
+    // Between one and two rounds of what is resident at once (units x OCC work-groups): that many work-groups, each
+    // taking every grid-th tile in turn.  Left to the dispatcher, the tiles of the second round go where slots come
+    // free first, and when the work-groups of a unit finish close together it puts two or three of them on one unit
+    // and none on others: 64 x 64 T,N at 2048 x 2048 x 2048 (1024 tiles on 768 slots) 109 TFLOP/s against 133 this way,
+    // 1536 x 2560 x 2048 107 / 126, f64 128 x 128 at 3400^3 49 / 63.  Whole rounds and longer launches are left as they
+    // are (8192^3 147 against 146 this way, 64 x 64 at 3000^3 128 / 125).
+    const unsigned resident = g_test_options.persistent && KS == 1 ? p.num_cus * (unsigned)OCC : 0u;
+    unsigned grid = resident && g.tiles_run > resident && g.tiles_run < 2 * resident ? resident : g.tiles_run;
     if constexpr (SK) {
+        unsigned sk_groups = 0;
         if (first_tiles || !gemm_dma_stream_k_plan(p, BM, BN, BK, OCC, sk_groups, g.sk_units, g.sk_total, g.sk_first)) return WK_E_INVALID_VALUE;
         g.sk_groups = sk_groups;
-        sk_groups += g.sk_first; // the launch: the dealt work-groups, then one per whole tile
+        // whole rounds run whole: one dealt work-group per unit and up to OCC - 1 more for the whole tiles
+        const unsigned rounds = g.sk_first / sk_groups;
+        grid = g.sk_first ? sk_groups * std::min<unsigned>((unsigned)OCC, rounds + 1) : sk_groups;
         g.partials = static_cast<float *>(p.scratch);
         g.counters = p.counters;
         g.patch_m = g.patch_n = 0; // consecutive tile numbers are neighbours in the row-group walk
     }
     if (p.ext) { // instantiated for op N, T only (what Linear.forward runs), one group of wavefronts, aligned rows
         if constexpr (KS == 1 && VB == 16)
-            return sel == 3 ? launch_one<BM, BN, BK, NS, OCC, true, true, true, 1, 16, SK>(st, g, first_tiles, sk_groups) : (int)WK_E_INVALID_VALUE;
+            return sel == 3 ? launch_one<BM, BN, BK, NS, OCC, true, true, true, 1, 16, SK>(st, g, grid) : (int)WK_E_INVALID_VALUE;
         else
             return WK_E_INVALID_VALUE;
     }
     switch (sel) {
-    case 0: return launch_one<BM, BN, BK, NS, OCC, false, false, false, KS, VB, SK>(st, g, first_tiles, sk_groups);
-    case 1: return launch_one<BM, BN, BK, NS, OCC, false, true, false, KS, VB, SK>(st, g, first_tiles, sk_groups);
-    case 2: return launch_one<BM, BN, BK, NS, OCC, true, false, false, KS, VB, SK>(st, g, first_tiles, sk_groups);
-    default: return launch_one<BM, BN, BK, NS, OCC, true, true, false, KS, VB, SK>(st, g, first_tiles, sk_groups);
+    case 0: return launch_one<BM, BN, BK, NS, OCC, false, false, false, KS, VB, SK>(st, g, grid);
+    case 1: return launch_one<BM, BN, BK, NS, OCC, false, true, false, KS, VB, SK>(st, g, grid);
+    case 2: return launch_one<BM, BN, BK, NS, OCC, true, false, false, KS, VB, SK>(st, g, grid);
+    default: return launch_one<BM, BN, BK, NS, OCC, true, true, false, KS, VB, SK>(st, g, grid);
     }
 }
 
@@ -729,13 +760,6 @@ bool wk::gemm_dma_stream_k_plan(const GemmProblem &p, int bm, int bn, int bk, in
     const uint64_t tiles = ((p.M + bm - 1) / bm) * ((p.N + bn - 1) / bn), slabs = (p.K + bk - 1) / bk;
     const uint64_t cus = p.num_cus ? p.num_cus : 256;
     uint64_t whole = g_test_options.stream_k == 2 || tiles < cus ? 0 : tiles / cus * cus;
-    // The f64 128 x 128 tile (two work-groups per unit) deals every tile once the launch would be more work-groups
-    // than are resident at once: which unit a late whole tile lands on is then up to the dispatcher, and with two
-    // slots per unit that both come free at about the same time it doubles them up on some units and leaves others
-    // idle (3456^3: 55 TFLOP/s against 70 with every tile dealt, 3500^3 52 / 67; where it went well the two plans
-    // were within 1.5 %: 3584^3 69 / 70, 3840^3 71 / 71, 4300^3 69 / 68).  The other kernels measured better with
-    // the whole rounds run whole at every size (f32 256 x 128, also two per unit: 4300^3 138 / 133, 8000^3 142 / 128).
-    if (p.dtype == WK_F64 && bm == 128 && g_test_options.stream_k != 3 && whole / cus >= (uint64_t)occ) whole = 0;
     if (whole == tiles) whole -= cus; // (a launch of whole rounds has no use for this: deal the last round)
     groups = (unsigned)(whole ? cus : cus * occ);
     if (groups % 8 || !p.scratch || !p.counters || tiles > p.num_counters || tiles * slabs > 0x7fffffffull) return false;

@@ -47,6 +47,8 @@ struct DArgsD {
     uint32_t patch_m, patch_n; // as in DArgs
     // kernels instantiated with SK (work dealt by k-slabs), as in DArgs
     uint32_t sk_units, sk_total, sk_first, sk_groups;
+    // tiles of this launch (one work-group each, or fewer work-groups that take every gridDim.x-th tile in turn)
+    uint32_t tiles_run;
     double *partials;
     uint32_t *counters;
 };
@@ -479,31 +481,52 @@ void gemm_f64_dma_kernel(DArgsD g) {
     else epilogue(std::true_type{});
     }; // run
     if constexpr (!SK) {
-        run(blockIdx.x, 0u, 0u, 0u);
-    } else { // as in the f32 kernel
-        const uint32_t slabs_per_tile = (g.K + BK - 1) / BK;
-        if (blockIdx.x >= g.sk_groups) { // a whole tile
-            run(blockIdx.x - g.sk_groups, 0u, slabs_per_tile, 0u);
-            return;
+        // One work-group per tile, or -- a launch of more tiles than are resident at once -- as many work-groups as
+        // are resident, each taking every gridDim.x-th tile in turn: which unit a late tile lands on is then fixed
+        // here (every unit's work-groups get the same share) instead of left to the order in which slots come free.
+        for (uint32_t pid = blockIdx.x; pid < g.tiles_run; pid += gridDim.x) {
+            if (pid != blockIdx.x) __syncthreads(); // every wavefront is done with the stages of the tile before
+            run(pid, 0u, 0u, 0u);
         }
-        const uint32_t bq = (blockIdx.x & 7u) * (g.sk_groups >> 3) + (blockIdx.x >> 3);
-        uint32_t u = bq * g.sk_units;
-        const uint32_t u_end = min(u + g.sk_units, g.sk_total);
+    } else {
+        const uint32_t slabs_per_tile = (g.K + BK - 1) / BK;
         bool first = true;
-        while (u < u_end) {
-            const uint32_t t = u / slabs_per_tile, kb = u - t * slabs_per_tile;
-            const uint32_t ke = min(slabs_per_tile, kb + (u_end - u));
-            if (!first) __syncthreads(); // every wavefront is done with the stages of the range before
-            run(g.sk_first + t, kb, ke, bq);
-            first = false;
-            u += ke - kb;
+        // Every tile dealt: all work-groups take a run of k-slabs.  Whole rounds run whole: the launch is `slots`
+        // work-groups per unit (work-group b sits on unit b % units, slot b / units: they are placed breadth
+        // first); slot 0 takes the unit's run of k-slabs first, and the unit's whole tiles -- tile c + units * j for
+        // j = 0 ... rounds - 1 -- go to the slots in turn, starting with slot 1, so that every unit's slots end up
+        // with the same amount of work.
+        const uint32_t units = g.sk_groups;
+        const uint32_t slot = g.sk_first ? blockIdx.x / units : 0u;
+        if (slot == 0) {
+            // work-groups b, b + 8, ... share an XCD: they take consecutive ranges, and with them neighbouring tiles
+            const uint32_t bq = (blockIdx.x & 7u) * (g.sk_groups >> 3) + (blockIdx.x >> 3);
+            uint32_t u = bq * g.sk_units;
+            const uint32_t u_end = min(u + g.sk_units, g.sk_total);
+            while (u < u_end) {
+                const uint32_t t = u / slabs_per_tile, kb = u - t * slabs_per_tile;
+                const uint32_t ke = min(slabs_per_tile, kb + (u_end - u));
+                if (!first) __syncthreads(); // every wavefront is done with the stages of the range before
+                run(g.sk_first + t, kb, ke, bq);
+                first = false;
+                u += ke - kb;
+            }
+        }
+        if (g.sk_first) {
+            const uint32_t c = blockIdx.x - slot * units, slots = gridDim.x / units, rounds = g.sk_first / units;
+            for (uint32_t j = (slot + slots - 1) % slots; j < rounds; j += slots) {
+                if (!first) __syncthreads();
+                run(c + units * j, 0u, slabs_per_tile, 0u);
+                first = false;
+            }
         }
     }
 }
 
-// sk_grid: work dealt by k-slabs: the work-groups of the launch (0: one work-group per tile)
+// grid: the work-groups of the launch (one per tile, or fewer: they then take the tiles in turn; kernels that deal
+// k-slabs: as their plan says)
 template <int BM, int BN, int BK, int NS, int OCC, bool A_K, bool B_K, bool EXT, int VB = 16, bool SK = false>
-int launch_one_d(hipStream_t st, const DArgsD &g, unsigned sk_grid = 0) {
+int launch_one_d(hipStream_t st, const DArgsD &g, unsigned grid) {
     constexpr size_t lds_bytes = NS * (BM * BK + BN * BK) * sizeof(double);
     auto kern = gemm_f64_dma_kernel<BM, BN, BK, NS, OCC, A_K, B_K, EXT, VB, SK>;
     static const int attr_rc = [&] {
@@ -516,7 +539,7 @@ int launch_one_d(hipStream_t st, const DArgsD &g, unsigned sk_grid = 0) {
         return (int)WK_OK;
     }();
     if (attr_rc) return attr_rc;
-    hipLaunchKernelGGL(kern, dim3(SK ? sk_grid : g.tiles_m * g.tiles_n), dim3(256), lds_bytes, st, g);
+    hipLaunchKernelGGL(kern, dim3(grid), dim3(256), lds_bytes, st, g);
     return launch_status();
 }
 
@@ -545,25 +568,28 @@ template <int BM, int BN, int BK, int NS, int OCC, int VB = 16, bool SK = false>
             }
     }
     const int sel = (p.op_a ? 0 : 2) | (p.op_b ? 1 : 0);
-    unsigned sk_grid = 0;
+    g.tiles_run = g.tiles_m * g.tiles_n;
+    const unsigned resident = g_test_options.persistent ? p.num_cus * (unsigned)OCC : 0u; // as in the f32 launch
+    unsigned grid = resident && g.tiles_run > resident && g.tiles_run < 2 * resident ? resident : g.tiles_run;
     if constexpr (SK) {
         unsigned groups = 0;
         if (p.ext || !gemm_dma_stream_k_plan(p, BM, BN, BK, OCC, groups, g.sk_units, g.sk_total, g.sk_first)) return WK_E_INVALID_VALUE;
         g.sk_groups = groups;
-        sk_grid = groups + g.sk_first; // the dealt work-groups, then one per whole tile
+        const unsigned rounds = g.sk_first / groups;
+        grid = g.sk_first ? groups * std::min<unsigned>((unsigned)OCC, rounds + 1) : groups;
         g.partials = static_cast<double *>(p.scratch);
         g.counters = p.counters;
         g.patch_m = g.patch_n = 0; // consecutive tile numbers are neighbours in the row-group walk
     }
     if (p.ext) {
-        if constexpr (VB == 16 && !SK) return sel == 3 ? launch_one_d<BM, BN, BK, NS, OCC, true, true, true>(st, g) : (int)WK_E_INVALID_VALUE;
+        if constexpr (VB == 16 && !SK) return sel == 3 ? launch_one_d<BM, BN, BK, NS, OCC, true, true, true>(st, g, grid) : (int)WK_E_INVALID_VALUE;
         else return WK_E_INVALID_VALUE;
     }
     switch (sel) {
-    case 0: return launch_one_d<BM, BN, BK, NS, OCC, false, false, false, VB, SK>(st, g, sk_grid);
-    case 1: return launch_one_d<BM, BN, BK, NS, OCC, false, true, false, VB, SK>(st, g, sk_grid);
-    case 2: return launch_one_d<BM, BN, BK, NS, OCC, true, false, false, VB, SK>(st, g, sk_grid);
-    default: return launch_one_d<BM, BN, BK, NS, OCC, true, true, false, VB, SK>(st, g, sk_grid);
+    case 0: return launch_one_d<BM, BN, BK, NS, OCC, false, false, false, VB, SK>(st, g, grid);
+    case 1: return launch_one_d<BM, BN, BK, NS, OCC, false, true, false, VB, SK>(st, g, grid);
+    case 2: return launch_one_d<BM, BN, BK, NS, OCC, true, false, false, VB, SK>(st, g, grid);
+    default: return launch_one_d<BM, BN, BK, NS, OCC, true, true, false, VB, SK>(st, g, grid);
     }
 }
 
