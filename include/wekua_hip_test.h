@@ -61,7 +61,8 @@ int wk_gemm_force_variant(const char *name);
  *                       whole rounds of tiles whole; 3: they run the whole rounds whole also where the default would not;
  *   "persistent"     0: a launch of the direct-to-LDS GEMM kernels with between one and two rounds of the work-groups
  *                       that are resident at once is one work-group per tile, placed by the dispatcher as slots come
- *                       free (default 1: as many work-groups as are resident, each taking every n-th tile);
+ *                       free (default 1: as many work-groups as are resident, each taking every n-th tile; 2: the same for
+ *                       every launch of more tiles than are resident, which measures 0.5-2 % slower on long launches);
  *   "strips"         0: a product is never multiplied in parts (body of whole tiles + strips); 2: thin strips are
  *                       split off whatever the cost model says (default 1: where the model puts the parts below
  *                       the whole). */

@@ -723,7 +723,7 @@ template <int BM, int BN, int BK, int NS, int OCC, int KS = 1, int VB = 16, bool
     // 1536 x 2560 x 2048 107 / 126, f64 128 x 128 at 3400^3 49 / 63.  Whole rounds and longer launches are left as they
     // are (8192^3 147 against 146 this way, 64 x 64 at 3000^3 128 / 125).
     const unsigned resident = g_test_options.persistent && KS == 1 ? p.num_cus * (unsigned)OCC : 0u;
-    unsigned grid = resident && g.tiles_run > resident && g.tiles_run < 2 * resident ? resident : g.tiles_run;
+    unsigned grid = resident && g.tiles_run > resident && (g.tiles_run < 2 * resident || g_test_options.persistent == 2) ? resident : g.tiles_run;
     if constexpr (SK) {
         unsigned sk_groups = 0;
         if (first_tiles || !gemm_dma_stream_k_plan(p, BM, BN, BK, OCC, sk_groups, g.sk_units, g.sk_total, g.sk_first)) return WK_E_INVALID_VALUE;

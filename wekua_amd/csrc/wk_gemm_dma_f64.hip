@@ -582,7 +582,7 @@ template <int BM, int BN, int BK, int NS, int OCC, int VB = 16, bool SK = false>
     const int sel = (p.op_a ? 0 : 2) | (p.op_b ? 1 : 0);
     g.tiles_run = g.tiles_m * g.tiles_n;
     const unsigned resident = g_test_options.persistent ? p.num_cus * (unsigned)OCC : 0u; // as in the f32 launch
-    unsigned grid = resident && g.tiles_run > resident && g.tiles_run < 2 * resident ? resident : g.tiles_run;
+    unsigned grid = resident && g.tiles_run > resident && (g.tiles_run < 2 * resident || g_test_options.persistent == 2) ? resident : g.tiles_run;
     if constexpr (SK) {
         unsigned groups = 0;
         if (p.ext || !gemm_dma_stream_k_plan(p, BM, BN, BK, OCC, groups, g.sk_units, g.sk_total, g.sk_first)) return WK_E_INVALID_VALUE;

@@ -45,7 +45,7 @@ struct TestOptions {
     int tail_strict = 0;    // 1: forced k-split tail variants plan like the automatic choice
     int alloc_colours = 1;  // 0: wk_malloc hands out blocks as hipMalloc returns them
     int stream_k = 1;       // 0: the automatic choice never deals work by k-slabs; 2: every tile dealt, none run whole; 3: whole rounds always run whole
-    int persistent = 1;     // 0: a launch of more tiles than are resident is one work-group per tile, placed by the dispatcher
+    int persistent = 1;     // 0: a launch of more tiles than are resident is one work-group per tile, placed by the dispatcher; 2: never
     int strips = 1;         // 0: products are never multiplied in parts; 2: thin strips split off whatever the model says
 };
 extern TestOptions g_test_options;
