@@ -494,9 +494,13 @@ def test_one_round_launches_take_the_k_split_tiles(dev):
     assert name("f32", 1024, 1024, 128) == b"mfma_f32_64x64d"      # short k
     assert name("f32", 1536, 1536, 1536) == b"mfma_f32_64x64k"     # 2.25 tiles per compute unit: two rounds whole, the rest dealt by k-slabs
     assert name("f32", 1408, 1408, 1408) == b"mfma_f32_64x64d"     # 1.89: nearly two whole rounds
-    assert name("f32", 2048, 2048, 2048) == b"mfma_f32_128x128d2"  # one full round of 128x128 tiles
-    assert name("f32", 2040, 2040, 2040) == b"mfma_f32_128x128d2"
-    assert name("f32", 2048, 2048, 512) == b"mfma_f32_128x128d"
+    # one full round of 128x128 tiles is between one and two rounds of the 64x64 tile, which then takes its tiles in
+    # turn and is the faster one up to k = 2048, except for N,T
+    assert name("f32", 2048, 2048, 2048) == b"mfma_f32_64x64d"
+    assert name("f32", 2040, 2040, 2040) == b"mfma_f32_64x64d"
+    assert name("f32", 2048, 2048, 512) == b"mfma_f32_64x64d"
+    assert name("f32", 2048, 2048, 4096) == b"mfma_f32_128x128d2"  # long k: two groups of wavefronts per 128x128 tile
+    assert dev.lib.wk_gemm_variant(raw.dtype_id("f32"), 0, 1, 2048, 2048, 2048, 2048, 2048, 2048, None, None, None) == b"mfma_f32_128x128d2"  # N,T
     assert dev.lib.wk_gemm_variant(raw.dtype_id("f32"), 1, 0, 1024, 1024, 1024, 1024, 1024, 1024, None, None, None) == b"mfma_f32_64x64d"  # T,N
     # ... any other leading dimension the same kernels with four bytes per lane and load, one group of wavefronts
     assert name("f32", 1001, 1001, 1001) == b"mfma_f32_64x64d"

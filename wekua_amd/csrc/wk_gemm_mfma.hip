@@ -1670,6 +1670,17 @@ int wk::gemm_mfma_pick(const GemmProblem &p, double *cost_out) {
             const char *want = !gemm_f32_dma_applies(p, 128, 128) ? "mfma_f32_128x128s2"
                                : (p.K >= 1024 && !p.ext && gemm_dma_rows_aligned(p)) ? "mfma_f32_128x128d2"
                                                                    : "mfma_f32_128x128d";
+            // Since launches of between one and two rounds of the 64 x 64 tile take their tiles in turn (three
+            // work-groups per unit: more than 768 and fewer than 1536 tiles), that tile is the faster one here up to
+            // k = 2048, except with a k-contiguous B beside an A that is too (N,T), which the two-group kernel reads
+            // best.  NN / NT / TN / TT, TFLOP/s, two-group 128 x 128 against 64 x 64: 2048^3 130 / 136 / 128 / 129 against
+            // 134 / 131 / 132 / 131, 2048 x 2048 x 1024 121 / 125 / 119 / 120 against 127 / 125 / 126 / 126, 2048 x 2048 x 512
+            // 105 / 108 / 104 / 104 against 113 / 115 / 111 / 112, 4096 x 1024 x 2048 130 / 136 / 128 / 129 against 133 /
+            // 132 / 132 / 132; 2048 x 2048 x 4096 137 / 142 / 134 / 135 against 136 / 135 / 136 / 137: not from there on.
+            const double tiles64 = (double)((p.M + 63) / 64) * (double)((p.N + 63) / 64);
+            if (!p.ext && g_test_options.persistent && tiles64 > 3.0 * cus && tiles64 < 6.0 * cus && p.K <= 2048 &&
+                (p.K <= 512 || p.op_a || !p.op_b) && gemm_f32_dma_applies(p, 64, 64) && gemm_dma_rows_aligned(p))
+                want = "mfma_f32_64x64d";
             for (int v = 0; v < k_num_variants; ++v)
                 if (!std::strcmp(k_variants[v].name, want)) return v;
         }
