@@ -281,16 +281,57 @@ __global__ __launch_bounds__(EW_BLOCK) void adam_multi_kernel(AdamMultiArgs<T> a
 // passes so that the result does not depend on scheduling. ------------------------------------
 constexpr int SUM_PARTIALS = 1024;
 
-template <typename T>
+// VEC: every row starts on a 16-byte boundary (base, pitches): a thread takes 16-byte vectors, four of them in
+// flight, and the < 16 bytes at the end of a row element by element; one division per vector, none when the
+// region is one row (a 1-D tensor, or rows and slices that follow each other without gaps: the host then passes
+// it as one row).  Which thread adds which elements is fixed by the shape alone, so the result is the same bits
+// on every run.  2^28 f32: 725 us with one element and two divisions per step -> 198 us = 5.4 TB/s (f64 5.8, 8192 x 8192 pitched 5.7).
+typedef unsigned int sum_u32x4 __attribute__((ext_vector_type(4)));
+template <typename T, bool VEC>
 __global__ __launch_bounds__(256) void sum_pass1_kernel(const T *__restrict__ x, Region rg, uint64_t rp, uint64_t sp,
                                                         T *__restrict__ partials) {
     __shared__ T red[256];
-    const uint64_t total = rg.depth * rg.rows * rg.cols;
+    constexpr uint64_t THREADS = (uint64_t)SUM_PARTIALS * 256ull;
+    const uint64_t tid = blockIdx.x * 256ull + threadIdx.x;
     T acc = T(0);
-    for (uint64_t idx = blockIdx.x * 256ull + threadIdx.x; idx < total; idx += (uint64_t)SUM_PARTIALS * 256ull) {
-        const uint64_t k = idx % rg.cols;
-        const uint64_t ij = idx / rg.cols;
-        acc += x[(ij / rg.rows) * sp + (ij % rg.rows) * rp + k];
+    if constexpr (VEC) {
+        constexpr int VE = 16 / sizeof(T);
+        const uint64_t nrows = rg.depth * rg.rows, nv = rg.cols / VE, total_v = nrows * nv;
+        auto vector_at = [&](uint64_t v) -> const sum_u32x4 * {
+            uint64_t row = 0, c = v;
+            if (nrows > 1) {
+                row = v / nv;
+                c = v - row * nv;
+            }
+            const T *p = x + (row / rg.rows) * sp + (row % rg.rows) * rp + c * VE;
+            return reinterpret_cast<const sum_u32x4 *>(p);
+        };
+        for (uint64_t v = tid; v < total_v; v += 4 * THREADS) {
+            sum_u32x4 q[4];
+#pragma unroll
+            for (int u = 0; u < 4; ++u)
+                if (v + u * THREADS < total_v) q[u] = __builtin_nontemporal_load(vector_at(v + u * THREADS));
+#pragma unroll
+            for (int u = 0; u < 4; ++u)
+                if (v + u * THREADS < total_v) {
+                    T e[VE];
+                    __builtin_memcpy(e, &q[u], 16);
+#pragma unroll
+                    for (int i = 0; i < VE; ++i) acc += e[i];
+                }
+        }
+        const uint64_t tail = rg.cols - nv * VE, total_t = nrows * tail;
+        for (uint64_t t = tid; t < total_t; t += THREADS) {
+            const uint64_t row = t / tail, k = nv * VE + (t - row * tail);
+            acc += x[(row / rg.rows) * sp + (row % rg.rows) * rp + k];
+        }
+    } else {
+        const uint64_t total = rg.depth * rg.rows * rg.cols;
+        for (uint64_t idx = tid; idx < total; idx += THREADS) {
+            const uint64_t k = idx % rg.cols;
+            const uint64_t ij = idx / rg.cols;
+            acc += x[(ij / rg.rows) * sp + (ij % rg.rows) * rp + k];
+        }
     }
     red[threadIdx.x] = acc;
     __syncthreads();
@@ -594,8 +635,21 @@ int wk_sum(wk_stream *s, int dtype, const uint64_t shape3[3], const void *x, uin
     if (!workspace || !dev_result) return WK_E_INVALID_VALUE;
     return dispatch_float(dtype, [&]<typename T>() -> int {
         if (check_opnd<T>(rg, x, xrp, xsp)) return WK_E_INVALID_VALUE;
-        hipLaunchKernelGGL((sum_pass1_kernel<T>), dim3(SUM_PARTIALS), dim3(256), 0, s->stream, static_cast<const T *>(x), rg,
-                           xrp, xsp, static_cast<T *>(workspace));
+        // rows and slices that follow each other without gaps are one long row
+        Region flat = rg;
+        uint64_t rp = xrp, sp = xsp;
+        if (rg.cols == xrp && (rg.depth == 1 || xsp == rg.rows * xrp)) {
+            flat = Region{1, 1, rg.depth * rg.rows * rg.cols};
+            rp = sp = flat.cols;
+        }
+        const bool vec = reinterpret_cast<uintptr_t>(x) % 16 == 0 && flat.cols >= 16 / sizeof(T) &&
+                         (flat.depth * flat.rows == 1 || ((rp * sizeof(T)) % 16 == 0 && (sp * sizeof(T)) % 16 == 0));
+        if (vec)
+            hipLaunchKernelGGL((sum_pass1_kernel<T, true>), dim3(SUM_PARTIALS), dim3(256), 0, s->stream, static_cast<const T *>(x),
+                               flat, rp, sp, static_cast<T *>(workspace));
+        else
+            hipLaunchKernelGGL((sum_pass1_kernel<T, false>), dim3(SUM_PARTIALS), dim3(256), 0, s->stream, static_cast<const T *>(x),
+                               rg, xrp, xsp, static_cast<T *>(workspace));
         int lrc = launch_status();
         if (lrc) return lrc;
         hipLaunchKernelGGL((sum_pass2_kernel<T>), dim3(1), dim3(256), 0, s->stream, static_cast<const T *>(workspace),
