@@ -265,10 +265,12 @@ def main():
     # every benchmark configuration through the reference-shaped API (tensors from Tensor.alloc, so with
     # the library's own pitches and placement), operands drawn on the device
     configs = None
+    off_sizes = None
     if not args.no_configs:
         ses = benchmark.Session()
         try:
             configs = benchmark.run_baseline_configs(ses, log=lambda m: log("[bench] " + m))
+            off_sizes = benchmark.run_off_benchmark_sizes(ses, log=lambda m: log("[bench] " + m))
         finally:
             ses.close()
     ax_key = f"2_axpy_f32_2p{args.axpy_log2n}"
@@ -364,6 +366,7 @@ def main():
                  "cpu_baseline": (axpy_cpu or {}).get(f"2_axpy_f32_2p{args.axpy_log2n}")},
         "mlp_step": mlp,
         "configs": configs,
+        "off_benchmark_sizes": off_sizes,
         "cpu_baseline": cpu,
         "cpu_baselines": cpu_all,
         "perf_floor": floor,

@@ -269,6 +269,31 @@ def run_baseline_configs(ses, log=None, device_fill=True):
     return out
 
 
+def off_benchmark_gemm_cases():
+    """Square products whose sides are not among the benchmark configurations: sides between the powers of
+    two, where the tiles do not fill whole rounds of the device and the choice of a kernel is what counts."""
+    cases = [("f32", n, 0, 0) for n in (1100, 1536, 2300, 2500, 3200, 4300, 6000)]
+    cases += [("f32", 2300, 1, 0), ("f32", 2300, 0, 1)]
+    cases += [("f64", n, 0, 0) for n in (1100, 1536, 2300, 3456, 4300)]
+    return cases
+
+
+def run_off_benchmark_sizes(ses, log=None):
+    """The products of off_benchmark_gemm_cases, timed like the benchmark configurations.  Returns a dict
+    key -> {ms, value, unit, kernel, frac}."""
+    out = {}
+    names = {(a, b): name for a, b, name in OPS}
+    for dtype, n, op_a, op_b in off_benchmark_gemm_cases():
+        ms, variant = time_gemm(ses, dtype, n, n, n, op_a, op_b, 1.5, 0.5, device_fill=True)
+        peak, unit, _, _ = PEAK[dtype]
+        rate = 2.0 * n * n * n / ms / 1e9
+        key = f"{dtype}_gemm_{n}_{names[(op_a, op_b)]}"
+        out[key] = {"ms": ms, "value": rate, "unit": unit, "kernel": variant, "frac": rate / peak}
+        if log:
+            log(f"{key}: {ms:.4f} ms -> {rate:.1f} {unit} = {100 * rate / peak:.1f} % of peak [{variant}]")
+    return out
+
+
 def cmd_configs(ses, args):
     rows = run_baseline_configs(ses, device_fill=False)
     print(f"{'config':38s} {'ms':>9s} {'rate':>9s} unit     % peak  kernel")
