@@ -15,7 +15,8 @@ extern "C" {
 #endif
 
 /* Name of the kernel variant wk_gemm() would launch for these arguments ("mfma_f32_256x128",
- * "tile64", "thin" for a product of at most four rows or columns, ...).  A name that ends in "+strips" is the kernel of the body of whole tiles of a product
+ * "tile64", "thin" for a product of one row or column (up to four where the next does not apply), "skinny" for one of
+ * two to 32 rows or columns against a large other operand, ...).  A name that ends in "+strips" is the kernel of the body of whole tiles of a product
  * that wk_gemm launches in parts: the rows or columns beyond the body follow as products of their own.
  */
 const char *wk_gemm_variant(int dtype, int op_a, int op_b, uint64_t M, uint64_t N, uint64_t K,
@@ -63,6 +64,9 @@ int wk_gemm_force_variant(const char *name);
  *                       that are resident at once is one work-group per tile, placed by the dispatcher as slots come
  *                       free (default 1: as many work-groups as are resident, each taking every n-th tile; 2: the same for
  *                       every launch of more tiles than are resident, which measures 0.5-2 % slower on long launches);
+ *   "skinny"         0: products of at most 32 rows or columns of C never take the kernel that streams the large
+ *                       operand into registers (default 1); n >= 2: that kernel splits k over n work-groups per
+ *                       compute unit instead of what its registers allow to be resident;
  *   "strips"         0: a product is never multiplied in parts (body of whole tiles + strips); 2: thin strips are
  *                       split off whatever the cost model says (default 1: where the model puts the parts below
  *                       the whole). */

@@ -34,7 +34,7 @@ def test_test_knobs_are_not_in_the_product_header():
     from wekua_amd import _capi
     lib = _capi.load()
     assert lib.wk_test_option(b"no-such-switch", 1) == 1
-    for name, default in ((b"gemm_walk_rows", 0), (b"tail_strict", 0), (b"alloc_colours", 1), (b"stream_k", 1), (b"strips", 1), (b"persistent", 1)):
+    for name, default in ((b"gemm_walk_rows", 0), (b"tail_strict", 0), (b"alloc_colours", 1), (b"stream_k", 1), (b"strips", 1), (b"persistent", 1), (b"skinny", 1)):
         assert lib.wk_test_option(name, default) == 0
 
 
@@ -175,13 +175,23 @@ def test_thin_products_and_strips_by_name():
             assert name(dt, 1, 4096, 4096, op_a, op_b) == "thin" and name(dt, 4096, 4, 512, op_a, op_b) == "thin"
             assert name(dt, 5, 4096, 4096, op_a, op_b) != "thin" and name(dt, 1, 256, 4096, op_a, op_b) != "thin"
             assert name(dt, 4, 4, 4096, op_a, op_b) != "thin" and name(dt, 1, 4096, 64, op_a, op_b) != "thin"
-            # a row or a column beyond whole tiles: body + strips, whether the rows start on 16-byte boundaries or not
+            # two to 32 rows or columns against a large operand whose rows start on 16-byte boundaries: the kernel
+            # that streams that operand once
+            assert name(dt, 5, 4096, 4096, op_a, op_b) == "skinny" and name(dt, 4, 4096, 4096, op_a, op_b) == "skinny"
+            assert name(dt, 4096, 32, 4096, op_a, op_b) == "skinny" and name(dt, 33, 4096, 4096, op_a, op_b) != "skinny"
+            assert name(dt, 32, 4096, 512, op_a, op_b) != "skinny" and name(dt, 32, 200, 65536, op_a, op_b) != "skinny"
+            assert name(dt, 16, 4095, 4095, op_a, op_b, ldb=4095) != "skinny"
             lda, ldb = (4100 if op_a else 4096), (4096 if op_b else 4100)
             assert name(dt, 4097, 4097, 4096, op_a, op_b, lda, ldb).endswith("+strips")
             assert name(dt, 4097, 4097, 4095, op_a, op_b, 4097 if op_a else 4095, 4095 if op_b else 4097).endswith("+strips")
             assert not name(dt, 4096, 4096, 4096, op_a, op_b).endswith("+strips")              # nothing beyond
             assert not name(dt, 4097, 4096, 256, op_a, op_b, lda, 4096).endswith("+strips")     # short k
             assert not name(dt, 1025, 1024, 4096, op_a, op_b, 1028 if op_a else 4096, 4096 if op_b else 1024).endswith("+strips")  # small body
+    assert lib.wk_test_option(b"skinny", 0) == 0
+    try:
+        assert name(8, 5, 4096, 4096) != "skinny" and name(8, 4, 4096, 4096) == "thin"
+    finally:
+        lib.wk_test_option(b"skinny", 1)
     assert name(4, 4097, 4097, 4096) in ("mfma_i32_128x128", "mfma_i32_64x128")            # integers: never in parts
     assert name(8, 4200, 4096, 1024).endswith("+strips") and not name(8, 3000, 3000, 1024, lda=3000, ldb=3000).endswith("+strips")
 

@@ -71,6 +71,28 @@ def test_fused_equals_two_calls(dev, dtype, variant, kind):
         dev.lib.wk_gemm_force_variant(b"auto")
 
 
+@pytest.mark.parametrize("dtype", ["f32", "f64"])
+@pytest.mark.parametrize("op_a,op_b", [(0, 1), (0, 0), (1, 0), (1, 1)])
+@pytest.mark.parametrize("kind", ["none", "sigmoid", "tanh"])
+def test_fused_small_batches(dev, dtype, op_a, op_b, kind):
+    """A batch of at most 32 rows through a large weight matrix, and a large batch into at most 32 outputs: the
+    kernel for such products carries the bias and the activation in every layout (the bias goes by the column
+    of C whichever side is the short one).  Against the two calls to the bit and against float64."""
+    did = raw.dtype_id(dtype)
+    per = 16 // np.dtype(oracle.real_np_dtype(dtype)).itemsize
+    seed = 40
+    for (M, N, K) in [(32, 4096, 2048), (7, 4100, 1100), (4096, 24, 2052), (20, 1024, 4100)]:
+        assert dev.lib.wk_gemm_variant(did, op_a, op_b, M, N, K, M if op_a else K, K if op_b else N, N, None, None, None) == b"skinny"
+        for with_bias in (True, False):
+            seed += 1
+            fused, two, A, B, bias = both(dev, dtype, M, N, K, op_a, op_b, kind, with_bias, seed, per if with_bias else 0)
+            assert np.array_equal(fused, two), f"{M}x{N}x{K} bias={with_bias}"
+            z = A.astype(np.float64) @ B.astype(np.float64) + (bias.astype(np.float64) if bias is not None else 0.0)
+            want = {"none": z, "sigmoid": 1 / (1 + np.exp(-z)), "tanh": np.tanh(z)}[kind]
+            eps = np.finfo(oracle.real_np_dtype(dtype)).eps
+            assert np.abs(fused - want).max() <= 8 * eps * np.sqrt(K) * max(1.0, np.abs(z).max())
+
+
 @pytest.mark.parametrize("op_a,op_b", [(0, 0), (1, 0), (1, 1)])
 def test_other_layouts_run_the_two_calls(dev, op_a, op_b):
     fused, two, _A, _B, _bias = both(dev, "f32", 130, 70, 50, op_a, op_b, "tanh", True, 9)

@@ -868,6 +868,80 @@ def test_thin_products(dev, dtype, op_a, op_b):
         n += 1
 
 
+SKINNY_SHAPES = [(32, 4096, 2048), (17, 4100, 1100), (5, 8190, 600), (16, 3001, 1500), (9, 4096, 1030), (31, 260, 17000), (2, 4096, 2048),
+                 (4096, 32, 2048), (4100, 9, 1100), (8190, 24, 777), (3001, 16, 1500), (300, 7, 16001), (4099, 3, 1100), (4, 8190, 600),
+                 (17, 2100, 2090), (2100, 24, 2053)]
+
+
+@pytest.mark.parametrize("dtype", ["f32", "f64"])
+@pytest.mark.parametrize("op_a,op_b", OPS)
+def test_skinny_products(dev, dtype, op_a, op_b):
+    """Five to 32 rows or columns of C against a large other operand (a small batch through a weight matrix):
+    the kernel that streams the large operand once into registers.  One and two blocks of sixteen on the short
+    side, both storage orders of both operands, k with every kind of tail (a last group of k that is partial, a
+    last share that is short), ragged long sides, every epilogue, gaps between the rows of all three matrices
+    whose poison must survive; against the oracle.  The name query says which products take it, and the test
+    option takes it away."""
+    from wekua_amd import raw
+    per = 4 if dtype == "f32" else 2
+    up = lambda n: -(-n // per) * per
+    did = raw.dtype_id(dtype)
+
+    def name(M, N, K, lda=None, ldb=None):
+        return dev.lib.wk_gemm_variant(did, op_a, op_b, M, N, K, lda or up(M if op_a else K), ldb or up(K if op_b else N), N, None, None, None)
+    assert name(32, 4096, 2048) == b"skinny" and name(4096, 32, 2048) == b"skinny" and name(5, 8192, 512) == b"skinny"
+    assert name(33, 4096, 2048) != b"skinny" and name(32, 1024, 1024) != b"skinny"
+    # one row or column stays with the thin kernel (a matrix-vector product); two to four come here where the long
+    # operand is large and its rows start on 16-byte boundaries
+    assert name(1, 4096, 2048) == b"thin" and name(4, 4096, 2048) == b"skinny" and name(4096, 2, 2048) == b"skinny" and name(4, 512, 128) == b"thin"
+    assert name(32, 32, 1 << 20) != b"skinny" and name(32, 1 << 20, 128) != b"skinny"
+    # a leading dimension of the large operand that is no multiple of 16 bytes: the tile kernels' business
+    assert name(32, 4095, 2047, ldb=2047 if op_b else 4095) != b"skinny"
+    assert dev.lib.wk_test_option(b"skinny", 0) == 0
+    try:
+        assert name(32, 4096, 2048) != b"skinny"
+    finally:
+        dev.lib.wk_test_option(b"skinny", 1)
+    options = [(1.5, 0.5), (None, None), (2.0, None), (None, -0.25)]
+    for n, (M, N, K) in enumerate(SKINNY_SHAPES):
+        alpha, beta = options[n % 4]
+        cols_a, cols_b = (M if op_a else K), (K if op_b else N)
+        # (f32 with more than sixteen on the short side and k below 2048 stays with the tile kernels, which start faster)
+        assert (name(M, N, K) == b"skinny") == (not (dtype == "f32" and min(M, N) > 16 and K < 2048)), (M, N, K)
+        check(dev, dtype, M, N, K, op_a, op_b, alpha, beta, seed=700 + n, lda=up(cols_a), ldb=up(cols_b), ldc=N)
+        check(dev, dtype, M, N, K, op_a, op_b, alpha, beta, seed=720 + n, lda=up(cols_a) + per, ldb=up(cols_b) + 2 * per, ldc=N + 3)
+
+
+@pytest.mark.parametrize("dtype", ["f32", "f64"])
+def test_skinny_products_give_the_same_bits_on_every_run(dev, dtype):
+    """k is split over the wavefronts of a work-group and over work-groups; the sums are added in the order of
+    k whichever work-group arrives last.  Also with two to four work-groups per unit instead of the default
+    (other shares of k, so other bits between the settings, the same within one)."""
+    rd = np.float32 if dtype == "f32" else np.float64
+    for (M, N, K, op_a, op_b) in [(32, 4096, 8192, 0, 0), (8192, 12, 4096, 0, 1), (20, 8192, 4096, 1, 1)]:
+        a, b, c = gemm_operands(dtype, M, N, K, op_a, op_b, 333)
+        want = oracle.gemm(dtype, 1.5, a, op_a, b, op_b, 0.5, c, threads=0)
+        dA, dB = dev.upload(a), dev.upload(b)
+        for per_unit in (1, 2, 4):
+            assert dev.lib.wk_test_option(b"skinny", per_unit) == 0
+            try:
+                first = None
+                for _ in range(4):
+                    dC = dev.upload(c)
+                    dev.gemm(dtype, op_a, op_b, M, N, K, 1.5, dA, a.shape[1], dB, b.shape[1], 0.5, dC, N)
+                    dev.sync()
+                    got = dC.download(rd, c.shape)
+                    dC.free()
+                    if first is None:
+                        first = got
+                        assert_gemm_close(dtype, got, want, 1.5, a, op_a, b, op_b, 0.5, c, K, what=f"skinny {M}x{N}x{K}, {per_unit} per unit")
+                    else:
+                        assert np.array_equal(got, first), "the bits depend on the run"
+            finally:
+                dev.lib.wk_test_option(b"skinny", 1)
+        dA.free(); dB.free()
+
+
 def test_left_over_tiles_run_as_a_k_split_tail(dev):
     """A launch whose tiles do not fill whole rounds of the compute units: the whole rounds run as they
     are, the left-over tiles as a second launch with k split over work-groups.  Checked: the plan of the

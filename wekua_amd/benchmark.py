@@ -301,6 +301,34 @@ def cmd_configs(ses, args):
         print(f"{name:38s} {r['ms']:9.4f} {r['value']:9.2f} {r['unit']:8s} {100 * r['roofline']['frac']:6.1f}  {r['kernel']}")
 
 
+NARROW_SHAPES = [(1, 8192, 8192), (4, 8192, 8192), (8, 4096, 4096), (16, 8192, 8192), (32, 8192, 8192), (24, 4096, 16384),
+                 (32, 2048, 2048), (16, 16384, 1024), (8192, 32, 8192), (4096, 8, 4096), (8192, 4, 8192)]
+
+
+def cmd_narrow(ses, args):
+    """Products with at most 32 rows or columns of C against a large other operand (small batches through a
+    weight matrix): the automatic choice beside the same call with the skinny kernel switched off (the thin
+    kernel up to four rows or columns, the 64 x 64 tile kernels beyond), and the rate at which the large
+    operand is read."""
+    did = raw.dtype_id(args.dtype)
+    sz = raw.elem_size(args.dtype)
+    print(f"{'dtype':5s} {'shape':>16s} {'op':2s} {'us':>8s} {'TB/s':>6s}  {'kernel':8s} | {'us':>8s}  kernel without the skinny kernel")
+    for M, N, K in NARROW_SHAPES:
+        for op_a, op_b, name in OPS:
+            if args.ops and name not in args.ops:
+                continue
+            rows = []
+            for skinny in (1, 0):
+                raw.check(ses.lib.wk_test_option(b"skinny", skinny), "wk_test_option")
+                try:
+                    rows.append(time_gemm(ses, args.dtype, M, N, K, op_a, op_b, 1.5, 0.5, iters=20, device_fill=True))
+                finally:
+                    ses.lib.wk_test_option(b"skinny", 1)
+            (ms, kernel), (ms0, kernel0) = rows
+            print(f"{args.dtype:5s} {f'{M}x{N}x{K}':>16s} {name:2s} {ms * 1e3:8.1f} {max(M, N) * K * sz / ms / 1e9:6.2f}  {kernel:8s} | "
+                  f"{ms0 * 1e3:8.1f}  {kernel0}", flush=True)
+
+
 def cmd_tensor(ses, args):
     """Streaming rates of the tensor support operations (algorithmic bytes: one read and one write of
     every element, one write for random.uniform)."""
@@ -465,6 +493,9 @@ def main(argv=None):
     a = sub.add_parser("axpy")
     a.add_argument("--dtype", default="f32")
     sub.add_parser("tensor")
+    n = sub.add_parser("narrow")
+    n.add_argument("--dtype", default="f32", choices=["f32", "f64"])
+    n.add_argument("--ops", nargs="+", default=None, choices=["NN", "NT", "TN", "TT"], help="only these operand layouts")
     sub.add_parser("probe")
     c = sub.add_parser("configs")
     c.add_argument("--variant", default="auto")
@@ -484,7 +515,7 @@ def main(argv=None):
     try:
         if getattr(args, "variant", "auto") != "auto":
             raw.check(ses.lib.wk_gemm_force_variant(args.variant.encode()), "wk_gemm_force_variant")
-        {"gemm": cmd_gemm, "axpy": cmd_axpy, "configs": cmd_configs, "tensor": cmd_tensor, "probe": cmd_probe}[args.cmd](ses, args)
+        {"gemm": cmd_gemm, "axpy": cmd_axpy, "configs": cmd_configs, "tensor": cmd_tensor, "probe": cmd_probe, "narrow": cmd_narrow}[args.cmd](ses, args)
     finally:
         ses.close()
     return 0

@@ -27,7 +27,7 @@ HIP_FLAGS = [
     "-I" + INCLUDE, "-I" + CSRC,
 ]
 
-HIP_SOURCES = ["wk_runtime.hip", "wk_axpy.hip", "wk_gemm.hip", "wk_gemm_generic.hip", "wk_gemm_mfma.hip", "wk_gemm_dma.hip", "wk_gemm_dma_f64.hip", "wk_gemm_imfma.hip", "wk_gemm_ipack.hip", "wk_gemm_i64pack.hip", "wk_gemm_cpack.hip", "wk_gemm_thin.hip", "wk_nn.hip", "wk_tensor_ops.hip"]
+HIP_SOURCES = ["wk_runtime.hip", "wk_axpy.hip", "wk_gemm.hip", "wk_gemm_generic.hip", "wk_gemm_mfma.hip", "wk_gemm_dma.hip", "wk_gemm_dma_f64.hip", "wk_gemm_imfma.hip", "wk_gemm_ipack.hip", "wk_gemm_i64pack.hip", "wk_gemm_cpack.hip", "wk_gemm_thin.hip", "wk_gemm_skinny.hip", "wk_nn.hip", "wk_tensor_ops.hip"]
 
 
 def _run(cmd):

@@ -135,6 +135,19 @@ void make_parts(const GemmProblem &p, uint64_t Mb, uint64_t Nb, StripPlan &out) 
     }
 }
 
+// Products with a handful of rows or columns of C have kernels of their own, which read the long operand once:
+// a single row or column (a matrix-vector product) goes to the thin kernel, whose lanes walk k without matrix
+// instructions; two to 32 to the skinny kernel where it applies (4 x 8192 x 8192 f32: 45 us there against 72-114
+// in the thin kernel), else up to four to the thin one.  0: neither, 1: thin, 2: skinny.
+int narrow_kind(const GemmProblem &p) {
+    const bool vector = p.M == 1 || p.N == 1;
+    if (vector && gemm_thin_applies(p)) return 1;
+    if (gemm_skinny_applies(p)) return 2;
+    return gemm_thin_applies(p) ? 1 : 0;
+}
+
+int narrow_launch(hipStream_t st, const GemmProblem &p, int kind) { return kind == 1 ? gemm_thin_launch(st, p) : gemm_skinny_launch(st, p); }
+
 bool plan_strips(const GemmProblem &p, StripPlan &out) {
     if ((p.dtype != WK_F32 && p.dtype != WK_F64) || p.ext || p.K < 512 || !g_test_options.strips) return false;
     if (!(p.dtype == WK_F32 ? gemm_f32_dma_applies(p, 128, 128) : gemm_f64_dma_applies(p, 128, 128))) return false;
@@ -157,7 +170,8 @@ bool plan_strips(const GemmProblem &p, StripPlan &out) {
             // Wider strips are launches of tile kernels, 20 us and more each: the model decides (2200^3: 123 TFLOP/s
             // whole against 106 in parts, 4000^3 138 against 130, 2312 x 2304 x 2304 127 against 120).
             bool all_thin = true;
-            for (int i = 1; i < out.parts; ++i) all_thin = all_thin && gemm_thin_applies(out.part[i]);
+            for (int i = 1; i < out.parts; ++i)
+                all_thin = all_thin && (out.part[i].M <= 4 || out.part[i].N <= 4) && narrow_kind(out.part[i]) != 0;
             double whole = 0.0;
             const int wv = gemm_mfma_pick(p, &whole);
             if (wv < 0) return true;
@@ -168,7 +182,7 @@ bool plan_strips(const GemmProblem &p, StripPlan &out) {
             double sum = 0.0;
             for (int i = 0; i < out.parts; ++i) {
                 double c = 0.0;
-                if (gemm_thin_applies(out.part[i])) c = 5.0 * launch; // (a thin product reads the long operand once)
+                if (narrow_kind(out.part[i])) c = 5.0 * launch; // (a thin or skinny product reads the long operand once)
                 else if (gemm_mfma_pick(out.part[i], &c) < 0) return true;
                 sum += c + (i ? launch : 0.0);
             }
@@ -276,13 +290,15 @@ static int gemm_entry(wk_stream *s, int dtype, int op_a, int op_b, uint64_t M, u
         }
     }
     if (g_forced.load(std::memory_order_relaxed) == -2) {
-        if (gemm_thin_applies(p)) return gemm_thin_launch(s->stream, p);
+        const int narrow = narrow_kind(p);
+        if (narrow) return narrow_launch(s->stream, p, narrow);
         StripPlan sp;
         if (plan_strips(p, sp)) {
             for (int i = 0; i < sp.parts; ++i) {
                 const GemmProblem &q = sp.part[i];
-                if (gemm_thin_applies(q)) {
-                    rc = gemm_thin_launch(s->stream, q);
+                const int nq = narrow_kind(q);
+                if (nq) {
+                    rc = narrow_launch(s->stream, q, nq);
                 } else {
                     const int pv = gemm_mfma_pick(q);
                     rc = pv >= 0 ? gemm_mfma_launch(s->stream, q, pv) : gemm_generic_launch(s->stream, q);
@@ -331,6 +347,12 @@ int wk_gemm_bias_activation(wk_stream *s, int dtype, int op_a, int op_b, uint64_
     p.scratch_bytes = s->scratch_bytes;
     p.counters = s->gemm_counters;
     p.num_counters = WK_GEMM_COUNTERS;
+    if (g_forced.load(std::memory_order_relaxed) == -2 && gemm_skinny_applies(p)) {
+        p.ext = bias || kind != WK_ACT_NONE; // (every layout: the kernel's epilogue is one for all)
+        p.ext_bias = bias;
+        p.ext_act = kind;
+        return gemm_skinny_launch(s->stream, p);
+    }
     const int v = choose(p);
     if (v >= 0 && gemm_mfma_fuses(p, v) && (bias || kind != WK_ACT_NONE)) {
         p.ext = true;
@@ -360,7 +382,7 @@ const char *wk_gemm_variant(int dtype, int op_a, int op_b, uint64_t M, uint64_t 
     p.counters = &dummy_counter;
     p.num_counters = WK_GEMM_COUNTERS;
     if (g_forced.load(std::memory_order_relaxed) == -2) {
-        if (gemm_thin_applies(p)) return "thin";
+        if (const int narrow = narrow_kind(p)) return narrow == 1 ? "thin" : "skinny";
         StripPlan sp;
         if (plan_strips(p, sp)) { // the body's kernel, marked: the strips beyond it are launches of their own
             const int bv = gemm_mfma_pick(sp.part[0]);

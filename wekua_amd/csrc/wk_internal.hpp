@@ -46,6 +46,7 @@ struct TestOptions {
     int alloc_colours = 1;  // 0: wk_malloc hands out blocks as hipMalloc returns them
     int stream_k = 1;       // 0: the automatic choice never deals work by k-slabs; 2: every tile dealt, none run whole; 3: whole rounds always run whole
     int persistent = 1;     // 0: a launch of more tiles than are resident is one work-group per tile, placed by the dispatcher; 2: never
+    int skinny = 1;         // 0: products of at most 32 rows or columns go to the tile kernels; n >= 2: n work-groups per unit
     int strips = 1;         // 0: products are never multiplied in parts; 2: thin strips split off whatever the model says
 };
 extern TestOptions g_test_options;
@@ -265,6 +266,10 @@ bool gemm_mfma_fuses(const GemmProblem &p, int variant); // variant can run p wi
 // f32 / f64 products with at most four rows or columns of C (wk_gemm_thin.hip)
 bool gemm_thin_applies(const GemmProblem &p);
 int gemm_thin_launch(hipStream_t st, const GemmProblem &p);
+// f32 / f64 products with at most 32 rows or columns of C and a large other operand (wk_gemm_skinny.hip);
+// every layout, and the fused bias + activation epilogue of Linear.forward in every layout
+bool gemm_skinny_applies(const GemmProblem &p);
+int gemm_skinny_launch(hipStream_t st, const GemmProblem &p);
 int gemm_mfma_pick(const GemmProblem &p, double *cost = nullptr); // -1: not applicable; cost: the model's figure for
                                                               // the chosen tile (rounds x tile area / efficiency; times k
                                                               // proportional to the launch's time: 3.05e5 per us in f32)

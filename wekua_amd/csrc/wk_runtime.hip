@@ -21,6 +21,7 @@ int wk_test_option(const char *name, int value) {
     else if (std::strcmp(name, "alloc_colours") == 0) g_test_options.alloc_colours = value;
     else if (std::strcmp(name, "stream_k") == 0) g_test_options.stream_k = value;
     else if (std::strcmp(name, "strips") == 0) g_test_options.strips = value;
+    else if (std::strcmp(name, "skinny") == 0) g_test_options.skinny = value;
     else if (std::strcmp(name, "persistent") == 0) g_test_options.persistent = value;
     else return WK_E_INVALID_VALUE;
     return WK_OK;
