@@ -194,7 +194,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(RB == 2 ? 2
 #pragma unroll
                 for (int i = 0; i < 4; ++i) {
                     const uint32_t kk = k + 4 * q + i;
-                    load_t v = *reinterpret_cast<const load_t *>(big_base + big_off[j] + (uint64_t)(kk < g.K ? k + i : g.K - 1 - 4 * q) * big_step);
+                    const int64_t row = kk < g.K ? (int64_t)(k + i) : (int64_t)g.K - 1 - 4 * (int64_t)q; // (big_off holds row 4 q)
+                    load_t v = *reinterpret_cast<const load_t *>(big_base + big_off[j] + row * (int64_t)big_step);
                     if (kk >= g.K) v = load_t{};
                     f.big[j * 4 + i] = v;
                 }
@@ -489,6 +490,7 @@ bool wk::gemm_skinny_applies(const GemmProblem &p) {
     const void *big = sh.rows_short ? p.B : p.A;
     const uint64_t ld = sh.rows_short ? p.ldb : p.lda;
     if (ld % epl || (reinterpret_cast<uintptr_t>(big) & 15u)) return false;
+    if (p.lda > (1ull << 21) || p.ldb > (1ull << 21)) return false; // (the lanes' offsets from the moving base are 32 bits)
     uint32_t tiles, shares, klen;
     plan_shares(p, sh, tiles, shares, klen);
     if (shares > 65535) return false;
