@@ -270,27 +270,38 @@ def run_baseline_configs(ses, log=None, device_fill=True):
 
 
 def off_benchmark_gemm_cases():
-    """Square products whose sides are not among the benchmark configurations: sides between the powers of
-    two, where the tiles do not fill whole rounds of the device and the choice of a kernel is what counts."""
-    cases = [("f32", n, 0, 0) for n in (1100, 1536, 2300, 2500, 3200, 4300, 6000)]
-    cases += [("f32", 2300, 1, 0), ("f32", 2300, 0, 1)]
-    cases += [("f64", n, 0, 0) for n in (1100, 1536, 2300, 3456, 4300)]
+    """(dtype, M, N, K, op_a, op_b) of products that are not among the benchmark configurations: squares with
+    sides between the powers of two, where the tiles do not fill whole rounds of the device and the choice of a
+    kernel is what counts, and small batches against a large matrix (Linear.forward at batch sizes up to 32)."""
+    cases = [("f32", n, n, n, 0, 0) for n in (1100, 1536, 2300, 2500, 3200, 4300, 6000)]
+    cases += [("f32", 2300, 2300, 2300, 1, 0), ("f32", 2300, 2300, 2300, 0, 1)]
+    cases += [("f64", n, n, n, 0, 0) for n in (1100, 1536, 2300, 3456, 4300)]
+    cases += [("f32", 32, 8192, 8192, 0, 1), ("f32", 16, 8192, 8192, 0, 1), ("f32", 8, 4096, 4096, 0, 1), ("f32", 1, 8192, 8192, 0, 1),
+              ("f64", 32, 8192, 8192, 0, 1), ("f64", 8, 4096, 4096, 0, 1)]
     return cases
 
 
 def run_off_benchmark_sizes(ses, log=None):
     """The products of off_benchmark_gemm_cases, timed like the benchmark configurations.  Returns a dict
-    key -> {ms, value, unit, kernel, frac}."""
+    key -> {ms, value, unit, kernel, frac}; products of at most 32 rows, which wait for memory, also carry the
+    rate at which their large operand is read (`operand_GBs`)."""
     out = {}
     names = {(a, b): name for a, b, name in OPS}
-    for dtype, n, op_a, op_b in off_benchmark_gemm_cases():
-        ms, variant = time_gemm(ses, dtype, n, n, n, op_a, op_b, 1.5, 0.5, device_fill=True)
+    for dtype, M, N, K, op_a, op_b in off_benchmark_gemm_cases():
+        ms, variant = time_gemm(ses, dtype, M, N, K, op_a, op_b, 1.5, 0.5, device_fill=True)
         peak, unit, _, _ = PEAK[dtype]
-        rate = 2.0 * n * n * n / ms / 1e9
-        key = f"{dtype}_gemm_{n}_{names[(op_a, op_b)]}"
+        rate = 2.0 * M * N * K / ms / 1e9
+        shape = str(M) if M == N == K else f"{M}x{N}x{K}"
+        key = f"{dtype}_gemm_{shape}_{names[(op_a, op_b)]}"
         out[key] = {"ms": ms, "value": rate, "unit": unit, "kernel": variant, "frac": rate / peak}
+        note = f"{100 * rate / peak:.1f} % of peak"
+        if min(M, N) <= 32:
+            gbs = max(M, N) * K * raw.elem_size(dtype) / ms / 1e6
+            out[key]["operand_GBs"] = gbs
+            out[key]["operand_frac_of_hbm_peak"] = gbs / HBM_PEAK_GBS
+            note = f"large operand read at {gbs:.0f} GB/s = {100 * gbs / HBM_PEAK_GBS:.1f} % of HBM peak"
         if log:
-            log(f"{key}: {ms:.4f} ms -> {rate:.1f} {unit} = {100 * rate / peak:.1f} % of peak [{variant}]")
+            log(f"{key}: {ms:.4f} ms -> {rate:.1f} {unit}, {note} [{variant}]")
     return out
 
 
