@@ -66,7 +66,8 @@ int wk_gemm_force_variant(const char *name);
  *                       every launch of more tiles than are resident, which measures 0.5-2 % slower on long launches);
  *   "skinny"         0: products of at most 32 rows or columns of C never take the kernel that streams the large
  *                       operand into registers (default 1); n >= 2: that kernel splits k over n work-groups per
- *                       compute unit instead of what its registers allow to be resident;
+ *                       compute unit instead of what its registers allow to be resident (7: the default number, and
+ *                       every tile walks k from the start of its share instead of from a place of its own);
  *   "strips"         0: a product is never multiplied in parts (body of whole tiles + strips); 2: thin strips are
  *                       split off whatever the cost model says (default 1: where the model puts the parts below
  *                       the whole). */

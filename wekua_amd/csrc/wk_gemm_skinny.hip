@@ -70,6 +70,7 @@ template <typename T> struct SkinnyArgs {
     int ext;             // fused epilogue: + bias, activation
     int act;             // WK_ACT_*
     int bias_by_b;       // the column of C is b (rows short) rather than s
+    int rotate;          // tiles of b start their walk along k at different places (k-contiguous Big)
     T *partials;         // [share][tile][16-byte piece][thread]
     uint32_t *counters;  // one per tile of b
 };
@@ -239,27 +240,37 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(RB == 2 ? 2
     // between the loads of a group and the matrix instructions of the one before: at a branch the wait-count pass
     // would wait for everything that may be in flight, the loads just issued included ----
     const uint32_t groups = (k_hi - k_lo) / KG; // whole groups inside [k_lo, k_hi)
+    // The work-groups of a share all walk the same k at the same time, each along its own rows of a k-contiguous
+    // Big: with a leading dimension that is a multiple of the memory channels' period those rows' pieces sit in
+    // the same channels.  Each tile of b therefore starts its groups at another place and wraps around (a fixed
+    // place per tile: the sums are still the same bits on every run).
+    const uint32_t rot = BIG_K && g.rotate ? (uint32_t)((uint64_t)(blockIdx.x % 16u) * groups / 16u) : 0u;
+    auto big_of = [&](uint32_t i) { // bases of the i-th group in walking order
+        const uint32_t at = i + rot < groups ? i + rot : i + rot - groups;
+        return big_base + ((uint64_t)k_lo + (uint64_t)at * KG) * big_step;
+    };
+    auto s_of = [&](uint32_t i) {
+        const uint32_t at = i + rot < groups ? i + rot : i + rot - groups;
+        return s_base + ((uint64_t)k_lo + (uint64_t)at * KG) * s_step;
+    };
     Frag f0, f1;
     if (groups) {
-        const char *bigp = big_base + (uint64_t)k_lo * big_step, *sp = s_base + (uint64_t)k_lo * s_step;
-        load(f0, bigp, sp);
+        load(f0, big_of(0), s_of(0));
         uint32_t i = 1; // f0 holds group i - 1
         // (the scheduler is kept from moving a group's loads down among the matrix instructions that come after
         // them in the source, which is where it puts them to save registers: next to their use)
         for (; i + 1 < groups; i += 2) {
-            bigp += KG * big_step; sp += KG * s_step;
-            load(f1, bigp, sp);
+            load(f1, big_of(i), s_of(i));
             __builtin_amdgcn_sched_barrier(0);
             multiply(f0);
             __builtin_amdgcn_sched_barrier(0);
-            bigp += KG * big_step; sp += KG * s_step;
-            load(f0, bigp, sp);
+            load(f0, big_of(i + 1), s_of(i + 1));
             __builtin_amdgcn_sched_barrier(0);
             multiply(f1);
             __builtin_amdgcn_sched_barrier(0);
         }
         if (i < groups) {
-            load(f1, bigp + KG * big_step, sp + KG * s_step);
+            load(f1, big_of(i), s_of(i));
             __builtin_amdgcn_sched_barrier(0);
             multiply(f0);
             multiply(f1);
@@ -410,22 +421,36 @@ Shape shape_of(const GemmProblem &p) {
 
 uint32_t tile_width(const GemmProblem &p, const Shape &sh) { return sh.big_k || p.dtype == WK_F64 ? 64 : 128; }
 
-// k shares: as many work-groups as are resident at once (by the registers of the instantiation: two to four
-// per unit), every wavefront with at least four groups of k; klen a multiple of 4 wavefronts x one group
+// k shares.  Two (two blocks of rows) or four work-groups are resident per unit; a launch takes
+// ceil(work-groups / resident) turns, each as long as a share of k plus what a work-group costs whatever its
+// share (start, the sums: about 128 values of k), and every share adds a part per tile to write and read back.
+// The number of shares with the smallest such time, every wavefront with at least four groups of k; klen a
+// multiple of 4 wavefronts x one group.  (32 x 8200 x 8200: 129 tiles; three shares leave a quarter of the
+// slots empty, seven fill two turns.)
 void plan_shares(const GemmProblem &p, const Shape &sh, uint32_t &tiles, uint32_t &shares, uint32_t &klen) {
     const bool f64 = p.dtype == WK_F64, two = sh.R > 16;
     const uint32_t cw = tile_width(p, sh);
     const uint32_t step = 4 * (sh.big_k && !f64 ? 32 : 16);
     tiles = (uint32_t)((sh.L + cw - 1) / cw);
-    const uint64_t per_unit = g_test_options.skinny >= 2 ? (uint64_t)g_test_options.skinny : two ? 2 : 4;
+    const uint64_t per_unit = g_test_options.skinny >= 2 && g_test_options.skinny != 7 ? (uint64_t)g_test_options.skinny : two ? 2 : 4;
     const uint64_t resident = per_unit * (p.num_cus ? p.num_cus : 256);
-    uint64_t want = resident / tiles;
-    if (want < 1) want = 1;
-    uint64_t len = (p.K + want - 1) / want;
-    if (len < 4 * step) len = 4 * step;
-    len = (len + step - 1) / step * step;
-    klen = (uint32_t)len;
-    shares = (uint32_t)((p.K + len - 1) / len);
+    const uint64_t most = p.K / (4 * step) ? p.K / (4 * step) : 1; // shares of at least four groups per wavefront
+    double best = 0.0;
+    uint64_t best_len = 0;
+    for (uint64_t want = 1; want <= most && want <= 64; ++want) {
+        uint64_t len = (p.K + want - 1) / want;
+        len = (len + step - 1) / step * step;
+        const uint64_t n = (p.K + len - 1) / len; // shares this length gives
+        const double turns = (double)((tiles * n + resident - 1) / resident);
+        const double parts = n > 1 ? 1.0 + (double)n * 2.0 * (two ? 32.0 : 16.0) / (double)p.K : 1.0;
+        const double t = turns * ((double)len + 128.0) * parts;
+        if (!best_len || t < best) {
+            best = t;
+            best_len = len;
+        }
+    }
+    klen = (uint32_t)best_len;
+    shares = (uint32_t)((p.K + best_len - 1) / best_len);
 }
 
 template <typename T, int RB, bool BIG_K> int launch_s(hipStream_t st, const SkinnyArgs<T> &g, dim3 grid, bool s_vec) {
@@ -456,6 +481,7 @@ template <typename T> int launch_t(hipStream_t st, const GemmProblem &p) {
     g.act = p.ext_act;
     g.bias = p.ext ? static_cast<const T *>(p.ext_bias) : nullptr;
     g.bias_by_b = sh.rows_short ? 1 : 0;
+    g.rotate = g_test_options.skinny == 7 ? 0 : 1;
     uint32_t tiles, shares;
     plan_shares(p, sh, tiles, shares, g.klen);
     if (shares > 1) {
