@@ -16,7 +16,7 @@ extern "C" {
 
 /* Name of the kernel variant wk_gemm() would launch for these arguments ("mfma_f32_256x128",
  * "tile64", "thin" for a product of one row or column (up to four where the next does not apply), "skinny" for one of
- * two to 32 rows or columns against a large other operand, ...).  A name that ends in "+strips" is the kernel of the body of whole tiles of a product
+ * two to 32 (in one layout of the large operand: 64) rows or columns against a large other operand, ...).  A name that ends in "+strips" is the kernel of the body of whole tiles of a product
  * that wk_gemm launches in parts: the rows or columns beyond the body follow as products of their own.
  */
 const char *wk_gemm_variant(int dtype, int op_a, int op_b, uint64_t M, uint64_t N, uint64_t K,

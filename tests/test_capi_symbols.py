@@ -178,9 +178,12 @@ def test_thin_products_and_strips_by_name():
             # two to 32 rows or columns against a large operand whose rows start on 16-byte boundaries: the kernel
             # that streams that operand once
             assert name(dt, 5, 4096, 4096, op_a, op_b) == "skinny" and name(dt, 4, 4096, 4096, op_a, op_b) == "skinny"
-            assert name(dt, 4096, 32, 4096, op_a, op_b) == "skinny" and name(dt, 33, 4096, 4096, op_a, op_b) != "skinny"
+            assert name(dt, 4096, 32, 4096, op_a, op_b) == "skinny" and name(dt, 65, 4096, 4096, op_a, op_b) != "skinny"
             assert name(dt, 32, 4096, 512, op_a, op_b) != "skinny" and name(dt, 32, 200, 65536, op_a, op_b) != "skinny"
             assert name(dt, 16, 4095, 4095, op_a, op_b, ldb=4095) != "skinny"
+            # 33 to 64: only with a large operand that is contiguous along the long side (f32: and a short one along k)
+            assert (name(dt, 64, 4096, 4096, op_a, op_b) == "skinny") == (op_b == 0 and (op_a == 0 or dt == 9))
+            assert (name(dt, 4096, 48, 4096, op_a, op_b) == "skinny") == (op_a == 1 and (op_b == 1 or dt == 9))
             lda, ldb = (4100 if op_a else 4096), (4096 if op_b else 4100)
             assert name(dt, 4097, 4097, 4096, op_a, op_b, lda, ldb).endswith("+strips")
             assert name(dt, 4097, 4097, 4095, op_a, op_b, 4097 if op_a else 4095, 4095 if op_b else 4097).endswith("+strips")

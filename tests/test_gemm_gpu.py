@@ -870,7 +870,7 @@ def test_thin_products(dev, dtype, op_a, op_b):
 
 SKINNY_SHAPES = [(32, 4096, 2048), (17, 4100, 1100), (5, 8190, 600), (16, 3001, 1500), (9, 4096, 1030), (31, 260, 17000), (2, 4096, 2048),
                  (4096, 32, 2048), (4100, 9, 1100), (8190, 24, 777), (3001, 16, 1500), (300, 7, 16001), (4099, 3, 1100), (4, 8190, 600),
-                 (17, 2100, 2090), (2100, 24, 2053)]
+                 (17, 2100, 2090), (2100, 24, 2053), (64, 4096, 2048), (33, 4100, 2100), (4100, 48, 2090), (8190, 64, 600)]
 
 
 @pytest.mark.parametrize("dtype", ["f32", "f64"])
@@ -890,7 +890,7 @@ def test_skinny_products(dev, dtype, op_a, op_b):
     def name(M, N, K, lda=None, ldb=None):
         return dev.lib.wk_gemm_variant(did, op_a, op_b, M, N, K, lda or up(M if op_a else K), ldb or up(K if op_b else N), N, None, None, None)
     assert name(32, 4096, 2048) == b"skinny" and name(4096, 32, 2048) == b"skinny" and name(5, 8192, 512) == b"skinny"
-    assert name(33, 4096, 2048) != b"skinny" and name(32, 1024, 1024) != b"skinny"
+    assert name(65, 4096, 2048) != b"skinny" and name(32, 1024, 1024) != b"skinny"
     # one row or column stays with the thin kernel (a matrix-vector product); two to four come here where the long
     # operand is large and its rows start on 16-byte boundaries
     assert name(1, 4096, 2048) == b"thin" and name(4, 4096, 2048) == b"skinny" and name(4096, 2, 2048) == b"skinny" and name(4, 512, 128) == b"thin"
@@ -906,8 +906,14 @@ def test_skinny_products(dev, dtype, op_a, op_b):
     for n, (M, N, K) in enumerate(SKINNY_SHAPES):
         alpha, beta = options[n % 4]
         cols_a, cols_b = (M if op_a else K), (K if op_b else N)
-        # (f32 with more than sixteen on the short side and k below 2048 stays with the tile kernels, which start faster)
-        assert (name(M, N, K) == b"skinny") == (not (dtype == "f32" and min(M, N) > 16 and K < 2048)), (M, N, K)
+        # (f32 with more than sixteen on the short side and k below 2048 stays with the tile kernels, which start
+        # faster; 33 to 64 on the short side come here with a large operand that is contiguous along the long side,
+        # in f32 only with a short operand that allows 16-byte loads along k)
+        expect = not (dtype == "f32" and min(M, N) > 16 and K < 2048)
+        if min(M, N) > 32:
+            big_k, s_kc = (op_b != 0, op_a == 0) if M <= N else (op_a == 0, op_b != 0)
+            expect = expect and not big_k and (s_kc or dtype == "f64")
+        assert (name(M, N, K) == b"skinny") == expect, (M, N, K)
         check(dev, dtype, M, N, K, op_a, op_b, alpha, beta, seed=700 + n, lda=up(cols_a), ldb=up(cols_b), ldc=N)
         check(dev, dtype, M, N, K, op_a, op_b, alpha, beta, seed=720 + n, lda=up(cols_a) + per, ldb=up(cols_b) + 2 * per, ldc=N + 3)
 

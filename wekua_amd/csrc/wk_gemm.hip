@@ -137,7 +137,7 @@ void make_parts(const GemmProblem &p, uint64_t Mb, uint64_t Nb, StripPlan &out) 
 
 // Products with a handful of rows or columns of C have kernels of their own, which read the long operand once:
 // a single row or column (a matrix-vector product) goes to the thin kernel, whose lanes walk k without matrix
-// instructions; two to 32 to the skinny kernel where it applies (4 x 8192 x 8192 f32: 45 us there against 72-114
+// instructions; two to 32 (64 in one layout) to the skinny kernel where it applies (4 x 8192 x 8192 f32: 45 us there against 72-114
 // in the thin kernel), else up to four to the thin one.  0: neither, 1: thin, 2: skinny.
 int narrow_kind(const GemmProblem &p) {
     const bool vector = p.M == 1 || p.N == 1;
@@ -182,7 +182,9 @@ bool plan_strips(const GemmProblem &p, StripPlan &out) {
             double sum = 0.0;
             for (int i = 0; i < out.parts; ++i) {
                 double c = 0.0;
-                if (narrow_kind(out.part[i])) c = 5.0 * launch; // (a thin or skinny product reads the long operand once)
+                // (a thin or skinny product reads the long operand once; beyond 32 rows or columns the tile kernels'
+                // figure stands for it)
+                if (narrow_kind(out.part[i]) && (out.part[i].M <= 32 || out.part[i].N <= 32)) c = 5.0 * launch;
                 else if (gemm_mfma_pick(out.part[i], &c) < 0) return true;
                 sum += c + (i ? launch : 0.0);
             }

@@ -1,14 +1,14 @@
-// f32 / f64 products whose C has at most 32 rows or at most 32 columns and whose other operand is large: a
+// f32 / f64 products whose C has at most 32 (one layout of the large operand: 64) rows or columns and whose other operand is large: a
 // batch of a few rows through a weight matrix (Linear.forward and its sensitivities at small batch sizes are
 // blas.gemm calls of this shape).  A 64 x 64 tile kernel pads the short side to 64 and spends two to eight
 // times the matrix work the product needs, which makes a product that should wait for memory wait for the
 // matrix pipes instead.  Here the large operand is read once, straight into registers along its storage order,
-// and multiplied with v_mfma_*_16x16x4 (one or two blocks of sixteen on the short side), so that the launch is
+// and multiplied with v_mfma_*_16x16x4 (one, two or four blocks of sixteen on the short side), so that the launch is
 // bound by the memory that operand streams from.
 //
-//   out(s, b) = sum_k S(s, k) * Big(k, b),   s < R <= 32 (the short index), b < L
+//   out(s, b) = sum_k S(s, k) * Big(k, b),   s < R <= 64 (the short index), b < L
 //
-// Rows short (M <= 32): s = row of C, b = column; S = op(A), Big = op(B).  Columns short (N <= 32): s = column of
+// Rows short (M <= 64): s = row of C, b = column; S = op(A), Big = op(B).  Columns short (N <= 64): s = column of
 // C, b = row; S(s, k) = op(B)(k, s), Big(k, b) = op(A)(b, k).
 //
 // A work-group of four wavefronts owns CW values of b (128 floats of a b-contiguous Big, 64 values otherwise) and one
@@ -75,10 +75,12 @@ template <typename T> struct SkinnyArgs {
     uint32_t *counters;  // one per tile of b
 };
 
-template <typename T, bool BIG_K> struct Geometry {
+template <typename T, bool BIG_K, int RB> struct Geometry {
     static constexpr int EPL = 16 / (int)sizeof(T);          // elements per 16-byte load
-    static constexpr int NB = BIG_K ? 4 : 2;                 // blocks of b: sixteen columns each (k-contiguous) or 16 EPL
-    static constexpr int CW = BIG_K ? 64 : 32 * EPL;         // values of b per work-group
+    // blocks of b: sixteen columns each (k-contiguous) or 16 EPL; half as many under four blocks of rows, which
+    // keeps the accumulators at 64 registers
+    static constexpr int NB = (BIG_K ? 4 : 2) / (RB == 4 ? 2 : 1);
+    static constexpr int CW = NB * (BIG_K ? 16 : 16 * EPL);  // values of b per work-group
     static constexpr int KQ = BIG_K ? 2 * EPL : 4;           // consecutive k values per lane and group
     static constexpr int KG = 4 * KQ;                        // k values per group
     static constexpr int BIG_LOADS = BIG_K ? NB * 2 : NB * 4; // 16-byte loads of Big per lane and group
@@ -86,8 +88,9 @@ template <typename T, bool BIG_K> struct Geometry {
 };
 
 template <typename T, int RB, bool BIG_K, bool S_VEC>
-__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(RB == 2 ? 2 : 4))) void gemm_skinny_kernel(SkinnyArgs<T> g) {
-    using G = Geometry<T, BIG_K>;
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(RB >= 2 ? 2 : 4))) void gemm_skinny_kernel(SkinnyArgs<T> g) {
+    static_assert(RB == 1 || RB == 2 || RB == 4, "one, two or four blocks of sixteen rows");
+    using G = Geometry<T, BIG_K, RB>;
     using load_t = typename Vec<T>::load_t;
     using acc_t = typename Vec<T>::acc_t;
     constexpr int EPL = G::EPL, CW = G::CW, KQ = G::KQ, KG = G::KG, NB = G::NB;
@@ -108,7 +111,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(RB == 2 ? 2
     // ---- addresses: a scalar base that moves along k, and per-lane byte offsets of 32 bits that do not ----
     // Big: the base is the work-group's first column (row of storage) at k = 0
     const char *big_base = reinterpret_cast<const char *>(BIG_K ? g.Big + (uint64_t)b0 * g.ld : g.Big + b0);
-    uint32_t big_off[BIG_K ? NB : 2]; // first piece of the lane: the others lie EPL values (k-contiguous) or rows of k further
+    uint32_t big_off[NB]; // first piece of the lane: the others lie EPL values (k-contiguous) or rows of k further
     if constexpr (BIG_K) {
 #pragma unroll
         for (int gb = 0; gb < NB; ++gb) big_off[gb] = ((min(b0 + 16 * gb + c, g.L - 1) - b0) * (uint32_t)g.ld + KQ * q) * (uint32_t)sizeof(T);
@@ -117,7 +120,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(RB == 2 ? 2
         // of 16 bytes: it cannot leave that value's page); pieces wholly beyond L are read from the last one
         const uint32_t last_piece = (g.L - 1) / EPL * EPL;
 #pragma unroll
-        for (int j = 0; j < 2; ++j)
+        for (int j = 0; j < NB; ++j)
             big_off[j] = (min(b0 + j * 16 * EPL + EPL * c, last_piece) - b0 + 4 * q * (uint32_t)g.ld) * (uint32_t)sizeof(T);
     }
     const uint32_t ld_bytes = (uint32_t)g.ld * (uint32_t)sizeof(T);
@@ -134,11 +137,16 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(RB == 2 ? 2
     uint32_t big_lane[G::BIG_LOADS];
 #pragma unroll
     for (int n = 0; n < G::BIG_LOADS; ++n) big_lane[n] = BIG_K ? big_off[n / 2] + 16u * (n % 2) : big_off[n / 4] + (n % 4) * ld_bytes;
-    uint32_t s_lane[RB][KQ]; // single elements of S (used when its rows do not allow 16-byte loads along k)
+    // single elements of S (used when its rows do not allow 16-byte loads along k): their offsets in registers,
+    // except under four blocks of rows, where the registers are not there and the offsets are added up per load
+    auto s_lane_of = [&](int rb, int i) -> uint32_t { return s_off[rb] + i * s_ks_bytes; };
+    uint32_t s_lane[RB == 4 ? 1 : RB][RB == 4 ? 1 : KQ];
+    if constexpr (RB != 4) {
 #pragma unroll
-    for (int rb = 0; rb < RB; ++rb)
+        for (int rb = 0; rb < RB; ++rb)
 #pragma unroll
-        for (int i = 0; i < KQ; ++i) s_lane[rb][i] = s_off[rb] + i * s_ks_bytes;
+            for (int i = 0; i < KQ; ++i) s_lane[rb][i] = s_lane_of(rb, i);
+    }
 
     struct Frag {
         load_t big[G::BIG_LOADS];
@@ -166,8 +174,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(RB == 2 ? 2
             } else {
 #pragma unroll
                 for (int i = 0; i < KQ; ++i) {
-                    if constexpr (sizeof(T) == 4) f.s[rb][i] = __builtin_bit_cast(T, __builtin_amdgcn_raw_buffer_load_b32(s_rsrc, s_lane[rb][i], 0, 0));
-                    else f.s[rb][i] = __builtin_bit_cast(T, __builtin_amdgcn_raw_buffer_load_b64(s_rsrc, s_lane[rb][i], 0, 0));
+                    if constexpr (sizeof(T) == 4) f.s[rb][i] = __builtin_bit_cast(T, __builtin_amdgcn_raw_buffer_load_b32(s_rsrc, RB == 4 ? s_lane_of(rb, i) : s_lane[RB == 4 ? 0 : rb][RB == 4 ? 0 : i], 0, 0));
+                    else f.s[rb][i] = __builtin_bit_cast(T, __builtin_amdgcn_raw_buffer_load_b64(s_rsrc, RB == 4 ? s_lane_of(rb, i) : s_lane[RB == 4 ? 0 : rb][RB == 4 ? 0 : i], 0, 0));
                 }
             }
         }
@@ -191,7 +199,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(RB == 2 ? 2
                 }
         } else {
 #pragma unroll
-            for (int j = 0; j < 2; ++j)
+            for (int j = 0; j < NB; ++j)
 #pragma unroll
                 for (int i = 0; i < 4; ++i) {
                     const uint32_t kk = k + 4 * q + i;
@@ -226,7 +234,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(RB == 2 ? 2
                     for (int rb = 0; rb < RB; ++rb) acc[gb][rb] = mfma16(f.s[rb][i], f.big[gb * 2 + i / EPL][i % EPL], acc[gb][rb]);
             } else {
 #pragma unroll
-                for (int j = 0; j < 2; ++j)
+                for (int j = 0; j < NB; ++j)
 #pragma unroll
                     for (int e = 0; e < EPL; ++e)
 #pragma unroll
@@ -404,7 +412,7 @@ struct Shape {
 
 Shape shape_of(const GemmProblem &p) {
     Shape sh;
-    sh.rows_short = p.M <= 32 && p.M <= p.N;
+    sh.rows_short = p.M <= 64 && p.M <= p.N;
     if (sh.rows_short) {
         sh.R = p.M;
         sh.L = p.N;
@@ -419,7 +427,9 @@ Shape shape_of(const GemmProblem &p) {
     return sh;
 }
 
-uint32_t tile_width(const GemmProblem &p, const Shape &sh) { return sh.big_k || p.dtype == WK_F64 ? 64 : 128; }
+// blocks of sixteen rows the short side is padded to: 1, 2 or 4
+uint32_t row_blocks(const Shape &sh) { return sh.R <= 16 ? 1 : sh.R <= 32 ? 2 : 4; }
+uint32_t tile_width(const GemmProblem &p, const Shape &sh) { return (sh.big_k || p.dtype == WK_F64 ? 64u : 128u) / (row_blocks(sh) == 4 ? 2u : 1u); }
 
 // k shares.  Two (two blocks of rows) or four work-groups are resident per unit; a launch takes
 // ceil(work-groups / resident) turns, each as long as a share of k plus what a work-group costs whatever its
@@ -428,11 +438,12 @@ uint32_t tile_width(const GemmProblem &p, const Shape &sh) { return sh.big_k || 
 // multiple of 4 wavefronts x one group.  (32 x 8200 x 8200: 129 tiles; three shares leave a quarter of the
 // slots empty, seven fill two turns.)
 void plan_shares(const GemmProblem &p, const Shape &sh, uint32_t &tiles, uint32_t &shares, uint32_t &klen) {
-    const bool f64 = p.dtype == WK_F64, two = sh.R > 16;
+    const bool f64 = p.dtype == WK_F64;
+    const uint32_t rb = row_blocks(sh);
     const uint32_t cw = tile_width(p, sh);
     const uint32_t step = 4 * (sh.big_k && !f64 ? 32 : 16);
     tiles = (uint32_t)((sh.L + cw - 1) / cw);
-    const uint64_t per_unit = g_test_options.skinny >= 2 && g_test_options.skinny != 7 ? (uint64_t)g_test_options.skinny : two ? 2 : 4;
+    const uint64_t per_unit = g_test_options.skinny >= 2 && g_test_options.skinny != 7 ? (uint64_t)g_test_options.skinny : rb >= 2 ? 2 : 4;
     const uint64_t resident = per_unit * (p.num_cus ? p.num_cus : 256);
     const uint64_t most = p.K / (4 * step) ? p.K / (4 * step) : 1; // shares of at least four groups per wavefront
     double best = 0.0;
@@ -442,7 +453,7 @@ void plan_shares(const GemmProblem &p, const Shape &sh, uint32_t &tiles, uint32_
         len = (len + step - 1) / step * step;
         const uint64_t n = (p.K + len - 1) / len; // shares this length gives
         const double turns = (double)((tiles * n + resident - 1) / resident);
-        const double parts = n > 1 ? 1.0 + (double)n * 2.0 * (two ? 32.0 : 16.0) / (double)p.K : 1.0;
+        const double parts = n > 1 ? 1.0 + (double)n * 2.0 * 16.0 * rb / (double)p.K : 1.0;
         const double t = turns * ((double)len + 128.0) * parts;
         if (!best_len || t < best) {
             best = t;
@@ -485,7 +496,7 @@ template <typename T> int launch_t(hipStream_t st, const GemmProblem &p) {
     uint32_t tiles, shares;
     plan_shares(p, sh, tiles, shares, g.klen);
     if (shares > 1) {
-        const size_t need = (size_t)shares * tiles * 16 * (sh.R > 16 ? 2 : 1) * tile_width(p, sh) * sizeof(T);
+        const size_t need = (size_t)shares * tiles * 16 * row_blocks(sh) * tile_width(p, sh) * sizeof(T);
         if (!p.scratch || !p.counters || need > p.scratch_bytes || tiles > p.num_counters) return WK_E_SCRATCH_TOO_SMALL;
         g.partials = static_cast<T *>(p.scratch);
         g.counters = p.counters;
@@ -493,6 +504,7 @@ template <typename T> int launch_t(hipStream_t st, const GemmProblem &p) {
     constexpr uint64_t EPL = 16 / sizeof(T);
     const bool s_vec = sh.s_kc && g.s_rs % EPL == 0 && (reinterpret_cast<uintptr_t>(g.S) & 15u) == 0;
     const dim3 grid(tiles, shares);
+    if (sh.R > 32) return sh.big_k ? launch_s<T, 4, true>(st, g, grid, s_vec) : launch_s<T, 4, false>(st, g, grid, s_vec);
     if (sh.R > 16) return sh.big_k ? launch_s<T, 2, true>(st, g, grid, s_vec) : launch_s<T, 2, false>(st, g, grid, s_vec);
     return sh.big_k ? launch_s<T, 1, true>(st, g, grid, s_vec) : launch_s<T, 1, false>(st, g, grid, s_vec);
 }
@@ -505,14 +517,25 @@ template <typename T> int launch_t(hipStream_t st, const GemmProblem &p) {
 bool wk::gemm_skinny_applies(const GemmProblem &p) {
     if ((p.dtype != WK_F32 && p.dtype != WK_F64) || !g_test_options.skinny) return false;
     if (!p.M || !p.N || !p.K) return false;
-    if (p.M > 32 && p.N > 32) return false;
+    if (p.M > 64 && p.N > 64) return false;
     const Shape sh = shape_of(p);
     if (sh.L < 256 || sh.L > 0x7fffffffull || p.K < 256 || p.K > 0x7fffffffull) return false;
     if (sh.L * p.K < (1ull << 22)) return false;
+    const uint64_t epl = 16 / wk_dtype_size(p.dtype);
     // (f32 with two blocks of rows and a short k: the 64 x 64 tiles pad it to twice the work only, and start faster;
     // 32 x 4096 x 1024: 9 us there, 13 here)
     if (p.dtype == WK_F32 && sh.R > 16 && p.K < 2048) return false;
-    const uint64_t epl = 16 / wk_dtype_size(p.dtype);
+    // 33 to 64 rows or columns (four blocks, tiles of half the width): where the large operand is b-contiguous; a
+    // k-contiguous one is then read 128 bytes at a time from 32 rows per wavefront and loses to the 64 x 64 tiles
+    // (f32 64 x 8192 x 8192 N,N 80 -> 71 us, 48 rows 85 -> 69, N,T 79 -> 93; f64 48 rows N,N 165 -> 141, N,T 163 -> 165)
+    if (sh.R > 32 && sh.big_k) return false;
+    if (p.dtype == WK_F32 && sh.R > 32) {
+        // (four blocks of rows, a b-contiguous large operand and single-element loads of the short one do not fit
+        // the registers of a wavefront in f32: the short operand must allow 16-byte loads along k)
+        const void *sp = sh.rows_short ? p.A : p.B;
+        const uint64_t s_rs = sh.rows_short ? p.lda : p.ldb;
+        if (!sh.s_kc || s_rs % epl || (reinterpret_cast<uintptr_t>(sp) & 15u)) return false;
+    }
     const void *big = sh.rows_short ? p.B : p.A;
     const uint64_t ld = sh.rows_short ? p.ldb : p.lda;
     if (ld % epl || (reinterpret_cast<uintptr_t>(big) & 15u)) return false;
@@ -521,7 +544,7 @@ bool wk::gemm_skinny_applies(const GemmProblem &p) {
     plan_shares(p, sh, tiles, shares, klen);
     if (shares > 65535) return false;
     if (shares > 1) {
-        const size_t need = (size_t)shares * tiles * 16 * (sh.R > 16 ? 2 : 1) * tile_width(p, sh) * wk_dtype_size(p.dtype);
+        const size_t need = (size_t)shares * tiles * 16 * row_blocks(sh) * tile_width(p, sh) * wk_dtype_size(p.dtype);
         if (!p.scratch || !p.counters || need > p.scratch_bytes || tiles > p.num_counters) return false;
     }
     return true;
