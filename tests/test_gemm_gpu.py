@@ -666,11 +666,14 @@ def test_k_split_over_work_groups(dev, dtype):
     lib = dev.lib
     did = raw.dtype_id(dtype)
     z = f"mfma_{dtype}_64x64z".encode()
-    assert lib.wk_gemm_variant(did, 0, 0, 512, 512, 8192, 8192, 512, 512, None, None, None) == z
+    assert lib.wk_gemm_variant(did, 0, 0, 256, 256, 8192, 8192, 256, 256, None, None, None) == z
+    # (64 tiles: in f32 the small tile with all its k-slabs dealt over the resident work-groups measures faster; in
+    # f64, whose shares come out even over the units, the split stays)
+    assert lib.wk_gemm_variant(did, 0, 0, 512, 512, 8192, 8192, 512, 512, None, None, None) == (b"mfma_f32_64x64k" if dtype == "f32" else z)
     assert lib.wk_gemm_variant(did, 0, 0, 512, 512, 512, 512, 512, 512, None, None, None) != z      # k too short to split
     assert lib.wk_gemm_variant(did, 0, 0, 2048, 2048, 8192, 8192, 2048, 2048, None, None, None) != z  # enough tiles
     shares, klen, first, tiles, nbytes = ctypes.c_uint32(), ctypes.c_uint32(), ctypes.c_uint64(), ctypes.c_uint64(), ctypes.c_size_t()
-    assert lib.wk_gemm_split_plan(did, 0, 0, 512, 512, 8192, None, shares, klen, first, tiles, nbytes) == 0
+    assert lib.wk_gemm_split_plan(did, 0, 0, 512, 512, 8192, z, shares, klen, first, tiles, nbytes) == 0
     # 64 tiles on 256 compute units: shares until four (f32) / two (f64) work-groups sit on every unit
     assert (shares.value, klen.value, tiles.value) == ((16, 512, 64) if dtype == "f32" else (8, 1024, 64))
     for op_a, op_b in OPS:

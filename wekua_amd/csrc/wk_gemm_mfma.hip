@@ -1645,9 +1645,32 @@ int wk::gemm_mfma_pick(const GemmProblem &p, double *cost_out) {
             if (d.dtype != p.dtype || p.K < d.min_k) continue;
             const double tiles = (double)((p.M + d.bm - 1) / d.bm) * (double)((p.N + d.bn - 1) / d.bn);
             const bool applies = p.dtype == WK_F32 ? gemm_f32_dma_stream_k_applies(p, d.bm, d.bn) : gemm_f64_dma_stream_k_applies(p, d.bm, d.bn);
-            if (tiles <= cus || std::fmod(tiles, cus) == 0.0 || !applies) continue;
+            if (!applies) continue;
+            bool by_rule = false;
+            if (tiles <= cus) {
+                // At most one tile per unit: the small tile with every tile's k-slabs dealt over all the work-groups
+                // that are resident, where k is long and the tiles (or the shares the k-split kernels would cut
+                // them into) do not come out even over the units.  Measured against the choice without it, N,N /
+                // T,N, TFLOP/s: f64 768 x 768 x 4096 36 / 35 -> 57 / 57, 832^2 x 4096 42 / 41 -> 58 / 57, 640^2 x 4096 44 / 42 ->
+                // 51 / 52, 384^2 x 16384 32 -> 44, 960^2 x 2048 49 / 47 -> 53 / 54, 1024^2 x 8192 59 / 56 -> 66 / 66 (x 1024: 52 -> 48,
+                // not taken); 512^2 and 512 x 1024 (64 and 128 tiles: whole shares per unit) and 256^2 x 65536 within
+                // +-5 % or worse, not taken.  f32 768^2 x 4096 80 / 77 -> 107 / 99, x 2048 75 / 72 -> 86 / 83, 832^2 x 4096 93 / 90 -> 107 /
+                // 103, 640^2 x 4096 75 -> 91 (x 2048: 72 -> 68, not taken), 512^2 x 8192 90 -> 96, 384^2 x 16384 75 -> 85, 512 x
+                // 1024 x 8192 111 / 106 -> 117 / 119; a full round (1024^2) is the two-group kernel's: 130 against 121-125.
+                if (d.bm != 64 || p.K < 2048) continue;
+                const uint64_t t = (uint64_t)tiles, units = (uint64_t)cus;
+                // (N,T is the layout the plain kernels read best: a nearly full round of it stays theirs in f64, 0.91-0.96
+                // of their rate dealt, and so does k < 4096 in f32; f32 below 42 tiles loses: 256 x 384 x 4096 20 -> 32 us)
+                const bool nt = !p.op_a && p.op_b;
+                const bool take = p.dtype == WK_F64 ? t >= 32 && (t == units || units % t != 0) && !(nt && 10 * t > 8 * units)
+                                                    : 10 * t <= 9 * units && t >= 42 && (p.K >= 4096 || (2 * t > units && !nt));
+                if (!take) continue;
+                by_rule = true; // (the model above has no figure for a single round that these measurements bear out)
+            } else if (std::fmod(tiles, cus) == 0.0) {
+                continue;
+            }
             const double cost = tiles / cus * d.bm * d.bn / d.eff + d.fixed_us * cost_per_us / (double)p.K;
-            if (cost < 0.98 * plain_cost && cost < best_cost)
+            if (by_rule || (cost < 0.98 * plain_cost && cost < best_cost))
                 for (int w = 0; w < k_num_variants; ++w)
                     if (!std::strcmp(k_variants[w].name, d.name)) {
                         best = w;
