@@ -1637,7 +1637,7 @@ int wk::gemm_mfma_pick(const GemmProblem &p, double *cost_out) {
     if ((p.dtype == WK_F32 || p.dtype == WK_F64) && best >= 0 && p.K >= 256 && g_test_options.stream_k) {
         const double cost_per_us = p.dtype == WK_F32 ? 3.05e5 : 1.525e5;
         static const struct { const char *name; int dtype, bm, bn; double eff, fixed_us; uint64_t min_k; } dealt[] = {
-            {"mfma_f32_128x128k", WK_F32, 128, 128, 0.90, 15.0, 1024}, {"mfma_f32_256x128k", WK_F32, 256, 128, 0.933, 36.0, 1024},
+            {"mfma_f32_128x128k", WK_F32, 128, 128, 0.90, 15.0, 256}, {"mfma_f32_256x128k", WK_F32, 256, 128, 0.933, 36.0, 1024},
             {"mfma_f32_64x64k", WK_F32, 64, 64, 0.83, 6.0, 256},
             {"mfma_f64_128x128k", WK_F64, 128, 128, 0.897, 20.0, 1024}, {"mfma_f64_64x64k", WK_F64, 64, 64, 0.887, 12.0, 256}};
         // Below k = 1024 the figure found above leaves out what a tile costs whatever its k (filling the stages, the
@@ -1685,6 +1685,14 @@ int wk::gemm_mfma_pick(const GemmProblem &p, double *cost_out) {
                     }
         }
     }
+    // f64 with a short k: the small tile, whose epilogue and stage fill are a quarter of the large one's per work-group
+    // and overlap three to a unit (4096 x 2048 x 256 82 -> 74 us, 2048 x 6144 x 256 122 -> 109, 8192 x 1024 x 384 111 -> 103,
+    // 2048 x 6144 x 640 258 -> 238; from k = 1000 on the large tile is level or ahead
+    // -- up to four rounds of the large tile; beyond, it is the better one again: 7000 x 7000 x 512 T,N 798 us against 888)
+    if (p.dtype == WK_F64 && p.K < 768 && best >= 0 && !std::strcmp(k_variants[best].name, "mfma_f64_128x128d") &&
+        (double)((p.M + 127) / 128) * (double)((p.N + 127) / 128) <= 4.0 * cus && gemm_f64_dma_applies(p, 64, 64))
+        for (int w = 0; w < k_num_variants; ++w)
+            if (!std::strcmp(k_variants[w].name, "mfma_f64_64x64d")) best = w;
     if (cost_out) *cost_out = best_cost;
     // f32 problems that are one nearly full round of 128x128 tiles: that tile with two k-groups (eight
     // wavefronts per CU) beats the four rounds of 64x64 the cost model would take -- 2048^3 126 / 132 /
