@@ -340,6 +340,47 @@ def cmd_narrow(ses, args):
                   f"{ms0 * 1e3:8.1f}  {kernel0}", flush=True)
 
 
+REGRET_SHAPES = [(512, 2048), (1000, 3000), (1536, 1536), (2048, 1024), (3000, 1000), (1280, 5000), (4096, 2048), (6000, 1500), (2500, 2500),
+                 (3072, 5120), (700, 9000), (5000, 5000), (1792, 3584), (1100, 1100), (8192, 1024), (3333, 2222)]
+REGRET_VARIANTS = {"f32": ["256x128d", "128x128d", "64x64d", "128x128d2", "64x64d2", "32x32s4", "64x64z", "256x128k", "128x128k", "64x64k"],
+                   "f64": ["128x128d", "64x64d", "32x32s4", "64x64z", "128x128k", "64x64k", "64x64s2"]}
+
+
+def cmd_regret(ses, args):
+    """How far the automatic choice of a kernel is behind the best forced one: M x N of REGRET_SHAPES x the given
+    values of k x N,N / T,N, six launches per point.  Prints the points above the threshold and the mean."""
+    def timed(M, N, K, op_a, op_b, variant):
+        ses.lib.wk_gemm_force_variant(f"mfma_{args.dtype}_{variant}".encode() if variant else b"auto")
+        try:
+            return time_gemm(ses, args.dtype, M, N, K, op_a, op_b, 1.5, 0.5, iters=6, device_fill=True)
+        except Exception:   # a variant that does not take the shape
+            return float("inf"), "-"
+        finally:
+            ses.lib.wk_gemm_force_variant(b"auto")
+    total, points, above = 0.0, 0, 0
+    for M, N in REGRET_SHAPES:
+        for K in args.ks:
+            for op_a, op_b, name in OPS:
+                if name not in ("NN", "TN"):
+                    continue
+                auto_ms, auto_name = timed(M, N, K, op_a, op_b, None)
+                best_ms, best_name = auto_ms, "auto"
+                for v in REGRET_VARIANTS[args.dtype]:
+                    if M * N * K > 4e10 and v in ("32x32s4", "64x64z", "64x64s2"):   # (minutes per launch, never the best there)
+                        continue
+                    ms, _ = timed(M, N, K, op_a, op_b, v)
+                    if ms < best_ms:
+                        best_ms, best_name = ms, v
+                behind = auto_ms / best_ms - 1.0
+                total += behind
+                points += 1
+                if behind > args.threshold:
+                    above += 1
+                    print(f"{args.dtype} {M}x{N}x{K} {name}: automatic {auto_name} {auto_ms * 1e3:.1f} us, best {best_name} {best_ms * 1e3:.1f} us, "
+                          f"{100 * behind:.1f} % behind", flush=True)
+    print(f"{args.dtype}: {points} points, {100 * total / points:.2f} % behind on average, {above} above {100 * args.threshold:.0f} %", flush=True)
+
+
 def cmd_tensor(ses, args):
     """Streaming rates of the tensor support operations (algorithmic bytes: one read and one write of
     every element, one write for random.uniform)."""
@@ -504,6 +545,10 @@ def main(argv=None):
     a = sub.add_parser("axpy")
     a.add_argument("--dtype", default="f32")
     sub.add_parser("tensor")
+    r = sub.add_parser("regret")
+    r.add_argument("--dtype", default="f32", choices=["f32", "f64"])
+    r.add_argument("--ks", type=int, nargs="+", default=[384, 1024, 2500, 6000])
+    r.add_argument("--threshold", type=float, default=0.04)
     n = sub.add_parser("narrow")
     n.add_argument("--dtype", default="f32", choices=["f32", "f64"])
     n.add_argument("--ops", nargs="+", default=None, choices=["NN", "NT", "TN", "TT"], help="only these operand layouts")
@@ -526,7 +571,7 @@ def main(argv=None):
     try:
         if getattr(args, "variant", "auto") != "auto":
             raw.check(ses.lib.wk_gemm_force_variant(args.variant.encode()), "wk_gemm_force_variant")
-        {"gemm": cmd_gemm, "axpy": cmd_axpy, "configs": cmd_configs, "tensor": cmd_tensor, "probe": cmd_probe, "narrow": cmd_narrow}[args.cmd](ses, args)
+        {"gemm": cmd_gemm, "axpy": cmd_axpy, "configs": cmd_configs, "tensor": cmd_tensor, "probe": cmd_probe, "narrow": cmd_narrow, "regret": cmd_regret}[args.cmd](ses, args)
     finally:
         ses.close()
     return 0
